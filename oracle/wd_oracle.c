@@ -1,0 +1,775 @@
+/*
+ * CPU oracle for the batch=1 MoE decode path.  TEST INFRASTRUCTURE ONLY: the
+ * shipped library never links or calls this file.
+ *
+ * What each function follows and how it is pinned (tests/test_oracle_*.py):
+ *
+ *   f16 conversions        src/qwen38_cpu_moe.cuh:77-137     all 65536 halves vs numpy float16, RNE
+ *                                                            vs numpy on random + boundary floats, and
+ *                                                            vs the compiled reference header
+ *   quantize_q8_0 / q8_K   :220-263                          compiled reference header (bit-exact) +
+ *                                                            invariants (|q|<=127, bsums, sign rule)
+ *   row_iq3_s/iq2_s/q8_0/  :298-440, :565-758                compiled reference header, AVX2 and scalar
+ *   iq4_nl                                                   twins (bit-exact) + closed forms of
+ *                                                            tests/lowbit_cuda_test.cu:50-98 + brute
+ *                                                            force through an independent dequantiser
+ *   exp/silu/sigmoid       :816-842                          compiled reference header (bit-exact) +
+ *                                                            libm exp to 2 ulp
+ *   dot_f32                :847-871                          compiled reference header (bit-exact)
+ *   expert chain / layer   :1169-1291                        compiled reference run_layer (bit-exact)
+ *   softmax_row / select   src/qwen38_moe.cuh:711-818        known answer of tests/qwen38_moe_cuda_test.cu
+ *                                                            :237-254, numpy softmax/top-k away from
+ *                                                            ties, tie / -inf / underflow rows by
+ *                                                            hand.  The per-8 summation order is
+ *                                                            PARITY UNPINNED at bit level: that block
+ *                                                            of the reference only builds with CUDA
+ *                                                            headers, which this image lacks.
+ *   row_q4_0_q8_0          src/warodecode.cu:1534-1562       int32 block sums vs brute force; the
+ *                                                            reference fixes no float order there
+ *
+ * Build: see oracle/Makefile (gcc -O2 -ffp-contract=off, no fast-math).
+ */
+#include "wd_oracle.h"
+
+#include <math.h>
+#include <pthread.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "../warpdecode_amd/csrc/wd_codebooks.inc"
+
+/* ------------------------------------------------------------------------- */
+/* Codebooks                                                                 */
+/* ------------------------------------------------------------------------- */
+static uint32_t g_iq3s[512];
+static uint64_t g_iq2s[1024];
+static pthread_once_t g_grid_once = PTHREAD_ONCE_INIT;
+
+static void expand_grids(void) {
+    const char *s3 = WD_IQ3S_GRID_DIGITS;
+    for (int e = 0; e < 512; ++e) {
+        uint32_t v = 0;
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t t = (uint32_t)(s3[e * 4 + j] - '0');
+            v |= (2u * t + 1u) << (8 * j);
+        }
+        g_iq3s[e] = v;
+    }
+    const char *s2 = WD_IQ2S_GRID_DIGITS;
+    for (int e = 0; e < 1024; ++e) {
+        uint64_t v = 0;
+        for (int j = 0; j < 8; ++j) {
+            const uint64_t t = (uint64_t)(s2[e * 8 + j] - '0');
+            v |= (8u + 17u * t + (t == 2)) << (8 * j);
+        }
+        g_iq2s[e] = v;
+    }
+}
+
+const uint32_t *wdo_iq3s_grid(void) {
+    pthread_once(&g_grid_once, expand_grids);
+    return g_iq3s;
+}
+
+const uint64_t *wdo_iq2s_grid(void) {
+    pthread_once(&g_grid_once, expand_grids);
+    return g_iq2s;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Geometry                                                                  */
+/* ------------------------------------------------------------------------- */
+int wdo_block_elems(int type) {
+    switch (type) {
+        case WDO_IQ3_S:
+        case WDO_IQ2_S: return 256;
+        case WDO_Q8_0:
+        case WDO_Q4_0:
+        case WDO_IQ4_NL: return 32;
+        case WDO_F32: return 1;
+        default: return 0;
+    }
+}
+
+size_t wdo_block_bytes(int type) {
+    switch (type) {
+        case WDO_IQ3_S: return 110;
+        case WDO_IQ2_S: return 82;
+        case WDO_Q8_0: return 34;
+        case WDO_Q4_0:
+        case WDO_IQ4_NL: return 18;
+        case WDO_F32: return 4;
+        default: return 0;
+    }
+}
+
+size_t wdo_row_bytes(int type, int cols) {
+    const int be = wdo_block_elems(type);
+    if (be == 0 || cols <= 0 || cols % be != 0) return 0;
+    return (size_t)(cols / be) * wdo_block_bytes(type);
+}
+
+/* ------------------------------------------------------------------------- */
+/* Half precision                                                            */
+/* ------------------------------------------------------------------------- */
+static inline uint32_t f32_bits(float v) {
+    uint32_t b;
+    memcpy(&b, &v, 4);
+    return b;
+}
+
+static inline float bits_f32(uint32_t b) {
+    float v;
+    memcpy(&v, &b, 4);
+    return v;
+}
+
+float wdo_f16_to_f32(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    const uint32_t ex = (h >> 10) & 31u;
+    uint32_t man = h & 0x3ffu;
+    if (ex == 31u) return bits_f32(sign | 0x7f800000u | (man << 13));
+    if (ex != 0u) return bits_f32(sign | ((ex + 112u) << 23) | (man << 13));
+    if (man == 0u) return bits_f32(sign);
+    /* subnormal half: value = man * 2^-24, renormalise */
+    int e = 113; /* exponent field of 2^-14 */
+    while ((man & 0x400u) == 0u) {
+        man <<= 1;
+        --e;
+    }
+    return bits_f32(sign | ((uint32_t)e << 23) | ((man & 0x3ffu) << 13));
+}
+
+uint16_t wdo_f32_to_f16(float value) {
+    const uint32_t b = f32_bits(value);
+    const uint16_t sign = (uint16_t)((b >> 16) & 0x8000u);
+    const int e = (int)((b >> 23) & 0xffu) - 127;
+    const uint32_t man = b & 0x7fffffu;
+    /* The reference maps every exponent above 15 (NaN included) to infinity and
+     * everything below 2^-25 to signed zero. */
+    if (e > 15) return (uint16_t)(sign | 0x7c00u);
+    if (e < -24) return sign;
+    if (e < -14) {
+        const uint32_t full = man | 0x800000u;
+        const int shift = 13 + (-14 - e); /* 14..23 */
+        uint32_t q = full >> shift;
+        const uint32_t rest = full & ((1u << shift) - 1u);
+        const uint32_t half = 1u << (shift - 1);
+        if (rest > half || (rest == half && (q & 1u))) ++q;
+        return (uint16_t)(sign | q); /* q == 0x400 is the smallest normal: correct encoding */
+    }
+    uint32_t q = man >> 13;
+    const uint32_t rest = man & 0x1fffu;
+    uint32_t ef = (uint32_t)(e + 15);
+    if (rest > 0x1000u || (rest == 0x1000u && (q & 1u))) {
+        ++q;
+        if (q == 0x400u) {
+            q = 0;
+            ++ef; /* may reach 31 = infinity, as IEEE rounding demands */
+        }
+    }
+    return (uint16_t)(sign | (ef << 10) | q);
+}
+
+static inline float half_at(const uint8_t *p) {
+    uint16_t h;
+    memcpy(&h, p, 2);
+    return wdo_f16_to_f32(h);
+}
+
+/* ------------------------------------------------------------------------- */
+/* Activation quantisers                                                     */
+/* ------------------------------------------------------------------------- */
+void wdo_quantize_q8_0(const float *x, int n, int8_t *qs, uint16_t *d) {
+    for (int b = 0; b < n / 32; ++b) {
+        const float *src = x + (size_t)b * 32;
+        int8_t *dst = qs + (size_t)b * 32;
+        float amax = 0.0f;
+        for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(src[i]));
+        d[b] = wdo_f32_to_f16(amax / 127.0f);
+        if (amax == 0.0f) {
+            memset(dst, 0, 32);
+            continue;
+        }
+        const float inv = 127.0f / amax;
+        for (int i = 0; i < 32; ++i) {
+            int q = (int)nearbyintf(src[i] * inv);
+            if (q > 127) q = 127;
+            if (q < -128) q = -128;
+            dst[i] = (int8_t)q;
+        }
+    }
+}
+
+void wdo_quantize_q8_K(const float *x, int n, int8_t *qs, float *d, int16_t *bsums) {
+    for (int b = 0; b < n / 256; ++b) {
+        const float *src = x + (size_t)b * 256;
+        int8_t *dst = qs + (size_t)b * 256;
+        int16_t *bs = bsums + (size_t)b * 16;
+        float amax = 0.0f;
+        for (int i = 0; i < 256; ++i) amax = fmaxf(amax, fabsf(src[i]));
+        if (amax == 0.0f) {
+            d[b] = 0.0f;
+            memset(dst, 0, 256);
+            memset(bs, 0, 32);
+            continue;
+        }
+        /* Always-negative inverse scale: the quants carry the opposite sign of x
+         * and d is negative, so d*q has the sign of x. */
+        const float iscale = -127.0f / amax;
+        for (int i = 0; i < 256; ++i) {
+            int q = (int)nearbyintf(src[i] * iscale);
+            if (q > 127) q = 127;
+            dst[i] = (int8_t)q;
+        }
+        for (int j = 0; j < 16; ++j) {
+            int s = 0;
+            for (int i = 0; i < 16; ++i) s += dst[16 * j + i];
+            bs[j] = (int16_t)s;
+        }
+        d[b] = 1.0f / iscale;
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Row dots                                                                  */
+/* ------------------------------------------------------------------------- */
+/* Closing tree of the eight chunk lanes: ((l0+l4)+(l2+l6)) + ((l1+l5)+(l3+l7)). */
+static inline float close_lanes(const float l[8]) {
+    const float a = l[0] + l[4];
+    const float b = l[1] + l[5];
+    const float c = l[2] + l[6];
+    const float e = l[3] + l[7];
+    return (a + c) + (b + e);
+}
+
+/* Signed dot of four codebook magnitudes (bytes of `mags`) against four activations. */
+static inline int32_t dot4_signed(uint32_t mags, unsigned sign_bits, const int8_t *a) {
+    int32_t s = 0;
+    for (int j = 0; j < 4; ++j) {
+        const int m = (int)((mags >> (8 * j)) & 0xffu);
+        s += (int)a[j] * (((sign_bits >> j) & 1u) ? -m : m);
+    }
+    return s;
+}
+
+float wdo_row_iq3_s_q8_K(const uint8_t *w, const int8_t *qs_a, const float *d_a, int cols, int32_t *partials) {
+    const uint32_t *grid = wdo_iq3s_grid();
+    float lane[8] = {0};
+    for (int sb = 0; sb < cols / 256; ++sb) {
+        const uint8_t *blk = w + (size_t)sb * 110;
+        const uint8_t *qs = blk + 2, *qh = blk + 66, *signs = blk + 74, *scales = blk + 106;
+        const int8_t *a = qs_a + (size_t)sb * 256;
+        const float d = half_at(blk) * d_a[sb];
+        for (int c = 0; c < 8; ++c) {
+            const int g = c >> 1, h = c & 1;
+            int32_t p = 0;
+            for (int ib = 0; ib < 8; ++ib) {
+                const unsigned nib = (ib & 1) ? (scales[ib >> 1] >> 4) : (scales[ib >> 1] & 15u);
+                const int ls = 1 + 2 * (int)nib;
+                const unsigned idx = qs[ib * 8 + 2 * g + h] | (((unsigned)qh[ib] << (8 - 2 * g - h)) & 0x100u);
+                const unsigned sbits = (unsigned)signs[ib * 4 + g] >> (4 * h);
+                p += ls * dot4_signed(grid[idx], sbits, a + ib * 32 + c * 4);
+            }
+            if (partials) partials[sb * 8 + c] = p;
+            lane[c] = fmaf(d, (float)p, lane[c]);
+        }
+    }
+    return close_lanes(lane);
+}
+
+float wdo_row_iq2_s_q8_K(const uint8_t *w, const int8_t *qs_a, const float *d_a, int cols, int32_t *partials) {
+    const uint64_t *grid = wdo_iq2s_grid();
+    float lane[8] = {0};
+    for (int sb = 0; sb < cols / 256; ++sb) {
+        const uint8_t *blk = w + (size_t)sb * 82;
+        const uint8_t *qs = blk + 2, *signs = blk + 34, *qh = blk + 66, *scales = blk + 74;
+        const int8_t *a = qs_a + (size_t)sb * 256;
+        const float d = half_at(blk) * d_a[sb];
+        for (int c = 0; c < 8; ++c) {
+            const int g = c >> 1, h = c & 1;
+            int32_t p = 0;
+            for (int ib = 0; ib < 8; ++ib) {
+                const unsigned nib = (c < 4) ? (scales[ib] & 15u) : (scales[ib] >> 4);
+                const int ls = 1 + 2 * (int)nib;
+                const unsigned idx = qs[ib * 4 + g] | (((unsigned)qh[ib] << (8 - 2 * g)) & 0x300u);
+                const uint32_t mags = (uint32_t)(grid[idx] >> (32 * h));
+                const unsigned sbits = (unsigned)signs[ib * 4 + g] >> (4 * h);
+                p += ls * dot4_signed(mags, sbits, a + ib * 32 + c * 4);
+            }
+            if (partials) partials[sb * 8 + c] = p;
+            lane[c] = fmaf(d, (float)p, lane[c]);
+        }
+    }
+    return 0.125f * close_lanes(lane);
+}
+
+float wdo_row_q8_0_q8_0(const uint8_t *w, const int8_t *qs_a, const uint16_t *d_a, int cols, int32_t *partials) {
+    float lane[8] = {0};
+    for (int b = 0; b < cols / 32; ++b) {
+        const uint8_t *blk = w + (size_t)b * 34;
+        const int8_t *q = (const int8_t *)(blk + 2);
+        const int8_t *a = qs_a + (size_t)b * 32;
+        const float d = half_at(blk) * wdo_f16_to_f32(d_a[b]);
+        for (int c = 0; c < 8; ++c) {
+            int32_t p = 0;
+            for (int j = 0; j < 4; ++j) p += (int)q[4 * c + j] * (int)a[4 * c + j];
+            if (partials) partials[b * 8 + c] = p;
+            lane[c] = fmaf(d, (float)p, lane[c]);
+        }
+    }
+    return close_lanes(lane);
+}
+
+static const int8_t k_iq4nl[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+
+float wdo_row_iq4_nl_q8_0(const uint8_t *w, const int8_t *qs_a, const uint16_t *d_a, int cols, int32_t *partials) {
+    const int nb = cols / 32;
+    float acc[2][8];
+    memset(acc, 0, sizeof(acc));
+    int32_t p[8];
+    const int paired = nb & ~1;
+    for (int b = 0; b < nb; ++b) {
+        const uint8_t *blk = w + (size_t)b * 18;
+        const int8_t *a = qs_a + (size_t)b * 32;
+        for (int c = 0; c < 8; ++c) {
+            const int hi = c >> 2;
+            int32_t s = 0;
+            for (int j = 0; j < 4; ++j) {
+                const int i = 4 * (c & 3) + j;
+                const unsigned nib = hi ? (blk[2 + i] >> 4) : (blk[2 + i] & 15u);
+                s += (int)a[16 * hi + i] * (int)k_iq4nl[nib];
+            }
+            p[c] = s;
+            if (partials) partials[b * 8 + c] = s;
+        }
+        if (b < paired) {
+            const float d = half_at(blk) * wdo_f16_to_f32(d_a[b]);
+            for (int c = 0; c < 8; ++c) acc[b & 1][c] = fmaf(d, (float)p[c], acc[b & 1][c]);
+        }
+    }
+    float lane[8];
+    for (int c = 0; c < 8; ++c) lane[c] = acc[0][c] + acc[1][c];
+    float r = close_lanes(lane);
+    if (nb & 1) {
+        /* trailing unpaired block (p[] still holds its chunk sums): one rounded
+         * product with the whole-block integer sum, added after the tree */
+        const uint8_t *blk = w + (size_t)(nb - 1) * 18;
+        int total = 0;
+        for (int c = 0; c < 8; ++c) total += p[c];
+        r += (half_at(blk) * wdo_f16_to_f32(d_a[nb - 1])) * (float)total;
+    }
+    return r;
+}
+
+float wdo_row_q4_0_q8_0(const uint8_t *w, const int8_t *qs_a, const uint16_t *d_a, int cols, int32_t *partials) {
+    /* value i<16 = low nibble of byte i, value i>=16 = high nibble of byte i-16, minus 8. */
+    double acc = 0.0;
+    for (int b = 0; b < cols / 32; ++b) {
+        const uint8_t *blk = w + (size_t)b * 18;
+        const int8_t *a = qs_a + (size_t)b * 32;
+        int32_t s = 0;
+        for (int i = 0; i < 16; ++i) {
+            s += ((int)(blk[2 + i] & 15u) - 8) * (int)a[i];
+            s += ((int)(blk[2 + i] >> 4) - 8) * (int)a[16 + i];
+        }
+        if (partials) partials[b] = s;
+        acc += (double)(half_at(blk) * wdo_f16_to_f32(d_a[b]) * (float)s);
+    }
+    return (float)acc;
+}
+
+static int partials_per_row(int type, int cols) {
+    switch (type) {
+        case WDO_IQ3_S:
+        case WDO_IQ2_S: return cols / 256 * 8;
+        case WDO_Q8_0:
+        case WDO_IQ4_NL: return cols / 32 * 8;
+        case WDO_Q4_0: return cols / 32;
+        default: return 0;
+    }
+}
+
+static float row_dot(int type, const uint8_t *w, const int8_t *qs, const void *d, int cols, int32_t *partials) {
+    switch (type) {
+        case WDO_IQ3_S: return wdo_row_iq3_s_q8_K(w, qs, (const float *)d, cols, partials);
+        case WDO_IQ2_S: return wdo_row_iq2_s_q8_K(w, qs, (const float *)d, cols, partials);
+        case WDO_Q8_0: return wdo_row_q8_0_q8_0(w, qs, (const uint16_t *)d, cols, partials);
+        case WDO_IQ4_NL: return wdo_row_iq4_nl_q8_0(w, qs, (const uint16_t *)d, cols, partials);
+        case WDO_Q4_0: return wdo_row_q4_0_q8_0(w, qs, (const uint16_t *)d, cols, partials);
+        default: return NAN;
+    }
+}
+
+void wdo_gemv(int type, const uint8_t *w, int rows, int cols, const int8_t *act_qs, const void *act_d,
+              float *out, int32_t *partials) {
+    const size_t rb = wdo_row_bytes(type, cols);
+    const int pp = partials_per_row(type, cols);
+    for (int r = 0; r < rows; ++r) {
+        out[r] = row_dot(type, w + (size_t)r * rb, act_qs, act_d, cols, partials ? partials + (size_t)r * pp : NULL);
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Independent dequantiser (brute-force checks only)                          */
+/* ------------------------------------------------------------------------- */
+void wdo_dequant_row(int type, const uint8_t *w, int cols, float *out) {
+    if (type == WDO_Q8_0) {
+        for (int b = 0; b < cols / 32; ++b) {
+            const uint8_t *blk = w + (size_t)b * 34;
+            const float d = half_at(blk);
+            for (int i = 0; i < 32; ++i) out[b * 32 + i] = d * (float)(int8_t)blk[2 + i];
+        }
+    } else if (type == WDO_Q4_0 || type == WDO_IQ4_NL) {
+        for (int b = 0; b < cols / 32; ++b) {
+            const uint8_t *blk = w + (size_t)b * 18;
+            const float d = half_at(blk);
+            for (int i = 0; i < 32; ++i) {
+                const unsigned nib = (i < 16) ? (blk[2 + i] & 15u) : (blk[2 + i - 16] >> 4);
+                const int code = (type == WDO_Q4_0) ? (int)nib - 8 : (int)k_iq4nl[nib];
+                out[b * 32 + i] = d * (float)code;
+            }
+        }
+    } else if (type == WDO_IQ3_S) {
+        const uint32_t *grid = wdo_iq3s_grid();
+        for (int sb = 0; sb < cols / 256; ++sb) {
+            const uint8_t *blk = w + (size_t)sb * 110;
+            const float d = half_at(blk);
+            for (int i = 0; i < 256; ++i) {
+                /* value i: 32-block ib, quad q (0..7) inside it, element j */
+                const int ib = i >> 5, q = (i >> 2) & 7, j = i & 3;
+                const unsigned hb = ((unsigned)blk[66 + ib] >> q) & 1u;
+                const unsigned idx = blk[2 + ib * 8 + q] | (hb << 8);
+                const int mag = (int)((grid[idx] >> (8 * j)) & 0xffu);
+                const unsigned sb_bit = ((unsigned)blk[74 + ib * 4 + (q >> 1)] >> (4 * (q & 1) + j)) & 1u;
+                const unsigned sc = blk[106 + (ib >> 1)];
+                const int ls = 1 + 2 * (int)((ib & 1) ? (sc >> 4) : (sc & 15u));
+                out[sb * 256 + i] = d * (float)(ls * (sb_bit ? -mag : mag));
+            }
+        }
+    } else if (type == WDO_IQ2_S) {
+        const uint64_t *grid = wdo_iq2s_grid();
+        for (int sb = 0; sb < cols / 256; ++sb) {
+            const uint8_t *blk = w + (size_t)sb * 82;
+            const float d = half_at(blk);
+            for (int i = 0; i < 256; ++i) {
+                /* value i: 32-block ib, octet o (0..3) inside it, element j (0..7) */
+                const int ib = i >> 5, o = (i >> 3) & 3, j = i & 7;
+                const unsigned hb = ((unsigned)blk[66 + ib] >> (2 * o)) & 3u;
+                const unsigned idx = blk[2 + ib * 4 + o] | (hb << 8);
+                const int mag = (int)((grid[idx] >> (8 * j)) & 0xffu);
+                const unsigned sb_bit = ((unsigned)blk[34 + ib * 4 + o] >> j) & 1u;
+                const unsigned sc = blk[74 + ib];
+                const int ls = 1 + 2 * (int)((o < 2) ? (sc & 15u) : (sc >> 4));
+                out[sb * 256 + i] = (d * 0.125f) * (float)(ls * (sb_bit ? -mag : mag));
+            }
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Transcendentals                                                           */
+/* ------------------------------------------------------------------------- */
+float wdo_exp_ggml(float x) {
+    const float r = 0x1.8p23f;
+    const float z = fmaf(x, 0x1.715476p+0f, r);
+    const float n = z - r;
+    const float b = fmaf(-n, 0x1.7f7d1cp-20f, fmaf(-n, 0x1.62e4p-1f, x));
+    const uint32_t e = f32_bits(z) << 23;
+    const float k = bits_f32(e + 0x3f800000u);
+    const float u = b * b;
+    const float p2 = fmaf(0x1.0e4020p-7f, b, 0x1.573e2ep-5f);
+    const float p1 = fmaf(0x1.555e66p-3f, b, 0x1.fffdb6p-2f);
+    const float j = fmaf(fmaf(p2, u, p1), u, 0x1.ffffecp-1f * b);
+    if (fabsf(n) <= 126.0f) return fmaf(j, k, k);
+    const uint32_t g = (n <= 0.0f) ? 0x82000000u : 0u;
+    const float s1 = bits_f32(g + 0x7f000000u);
+    if (fabsf(n) > 192.0f) return s1 * s1;
+    const float s2 = bits_f32(e - g);
+    return fmaf(s2, j, s2) * s1;
+}
+
+float wdo_silu_ggml(float x) { return x / (1.0f + wdo_exp_ggml(-x)); }
+
+float wdo_sigmoid_ggml(float x) { return 1.0f / (1.0f + wdo_exp_ggml(-x)); }
+
+/* ------------------------------------------------------------------------- */
+/* F32 dot in the 4 x 8 accumulator order                                     */
+/* ------------------------------------------------------------------------- */
+float wdo_dot_f32(const float *a, const float *b, int n) {
+    float s[32];
+    for (int t = 0; t < 32; ++t) s[t] = 0.0f;
+    const int np = n & ~31;
+    for (int i = 0; i < np; i += 32) {
+        for (int t = 0; t < 32; ++t) s[t] = fmaf(a[i + t], b[i + t], s[t]);
+    }
+    /* fold accumulators 2->0, 3->1, then 1->0 (accumulator j holds s[8j..8j+7]) */
+    for (int l = 0; l < 8; ++l) {
+        s[l] = s[l] + s[16 + l];
+        s[8 + l] = s[8 + l] + s[24 + l];
+    }
+    for (int l = 0; l < 8; ++l) s[l] = s[l] + s[8 + l];
+    const float t0 = s[0] + s[4], t1 = s[1] + s[5], t2 = s[2] + s[6], t3 = s[3] + s[7];
+    float acc = (t0 + t1) + (t2 + t3);
+    for (int c = np; c < n; ++c) acc = acc + a[c] * b[c];
+    return acc;
+}
+
+void wdo_router_logits(const float *w, const float *x, int rows, int cols, float *logits) {
+    for (int r = 0; r < rows; ++r) logits[r] = wdo_dot_f32(w + (size_t)r * cols, x, cols);
+}
+
+/* ------------------------------------------------------------------------- */
+/* Router chain                                                              */
+/* ------------------------------------------------------------------------- */
+void wdo_softmax_row(const float *logits, int n, float *probs) {
+    float mx = -INFINITY;
+    for (int e = 0; e < n; ++e) mx = fmaxf(mx, logits[e]);
+    double sum = 0.0;
+    int i = 0;
+    for (; i + 8 <= n; i += 8) {
+        float v[8];
+        for (int j = 0; j < 8; ++j) {
+            v[j] = wdo_exp_ggml(logits[i + j] - mx);
+            probs[i + j] = v[j];
+        }
+        const float lo = v[0] + v[4], lh = v[2] + v[6], hi = v[1] + v[5], hh = v[3] + v[7];
+        sum += (double)((lo + lh) + (hi + hh));
+    }
+    for (; i < n; ++i) {
+        probs[i] = wdo_exp_ggml(logits[i] - mx);
+        sum += (double)probs[i];
+    }
+    if (sum == 0.0) {
+        for (int e = 0; e < n; ++e) probs[e] = -INFINITY;
+        return;
+    }
+    const float inv = (float)(1.0 / sum);
+    for (int e = 0; e < n; ++e) probs[e] = probs[e] * inv;
+}
+
+void wdo_router_select(const float *probs, int n, int k, float w_scale, int *ids, float *weights) {
+    float top[64];
+    if (k > 64) k = 64;
+    for (int j = 0; j < k; ++j) {
+        float best = -INFINITY;
+        int best_id = 0;
+        for (int e = 0; e < n; ++e) {
+            if (!(probs[e] > best)) continue;
+            int taken = 0;
+            for (int m = 0; m < j; ++m) taken |= (ids[m] == e);
+            if (!taken) {
+                best = probs[e];
+                best_id = e;
+            }
+        }
+        ids[j] = best_id;
+        top[j] = probs[best_id];
+    }
+    double wsum = 0.0;
+    for (int j = 0; j < k; ++j) wsum += (double)top[j];
+    const float denom = fmaxf((float)wsum, 6.103515625e-5f);
+    for (int j = 0; j < k; ++j) weights[j] = top[j] / denom;
+    if (w_scale != 0.0f && w_scale != 1.0f) {
+        for (int j = 0; j < k; ++j) weights[j] = weights[j] * w_scale;
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Expert chain and layer                                                    */
+/* ------------------------------------------------------------------------- */
+static int act_is_q8k(int type) { return type == WDO_IQ3_S || type == WDO_IQ2_S; }
+
+typedef struct {
+    /* quantised layer input, both flavours (filled on demand) */
+    int8_t *xk_qs;
+    float *xk_d;
+    int16_t *xk_bs;
+    int8_t *x0_qs;
+    uint16_t *x0_d;
+} xq_t;
+
+static void expert_ffn_q(int gate_type, int up_type, int down_type, const uint8_t *gate, const uint8_t *up,
+                         const uint8_t *down, int H, int F, const xq_t *xq, float *out, float *gate_up,
+                         float *act, int8_t *act_qs, uint16_t *act_d, int32_t *gup, int32_t *dp) {
+    float *gu = gate_up ? gate_up : (float *)malloc(sizeof(float) * 2 * (size_t)F);
+    float *ac = act ? act : (float *)malloc(sizeof(float) * (size_t)F);
+    int8_t *aq = act_qs ? act_qs : (int8_t *)malloc((size_t)F);
+    uint16_t *ad = act_d ? act_d : (uint16_t *)malloc(sizeof(uint16_t) * (size_t)(F / 32));
+    const int ppg = partials_per_row(gate_type, H);
+    wdo_gemv(gate_type, gate, F, H, act_is_q8k(gate_type) ? xq->xk_qs : xq->x0_qs,
+             act_is_q8k(gate_type) ? (const void *)xq->xk_d : (const void *)xq->x0_d, gu, gup);
+    wdo_gemv(up_type, up, F, H, act_is_q8k(up_type) ? xq->xk_qs : xq->x0_qs,
+             act_is_q8k(up_type) ? (const void *)xq->xk_d : (const void *)xq->x0_d, gu + F,
+             gup ? gup + (size_t)F * ppg : NULL);
+    for (int r = 0; r < F; ++r) ac[r] = wdo_silu_ggml(gu[r]) * gu[F + r];
+    wdo_quantize_q8_0(ac, F, aq, ad);
+    wdo_gemv(down_type, down, H, F, aq, ad, out, dp);
+    if (!gate_up) free(gu);
+    if (!act) free(ac);
+    if (!act_qs) free(aq);
+    if (!act_d) free(ad);
+}
+
+static void xq_make(xq_t *q, const float *x, int H, int need_k, int need_0) {
+    memset(q, 0, sizeof(*q));
+    if (need_k) {
+        q->xk_qs = (int8_t *)malloc((size_t)H);
+        q->xk_d = (float *)malloc(sizeof(float) * (size_t)(H / 256));
+        q->xk_bs = (int16_t *)malloc(sizeof(int16_t) * (size_t)(H / 16));
+        wdo_quantize_q8_K(x, H, q->xk_qs, q->xk_d, q->xk_bs);
+    }
+    if (need_0) {
+        q->x0_qs = (int8_t *)malloc((size_t)H);
+        q->x0_d = (uint16_t *)malloc(sizeof(uint16_t) * (size_t)(H / 32));
+        wdo_quantize_q8_0(x, H, q->x0_qs, q->x0_d);
+    }
+}
+
+static void xq_free(xq_t *q) {
+    free(q->xk_qs);
+    free(q->xk_d);
+    free(q->xk_bs);
+    free(q->x0_qs);
+    free(q->x0_d);
+}
+
+void wdo_expert_ffn(int gate_type, int up_type, int down_type, const uint8_t *gate, const uint8_t *up,
+                    const uint8_t *down, int hidden, int ffn, const float *x, float *out, float *gate_up,
+                    float *act, int8_t *act_qs, uint16_t *act_d, int32_t *gate_up_partials,
+                    int32_t *down_partials) {
+    xq_t xq;
+    const int need_k = act_is_q8k(gate_type) || act_is_q8k(up_type);
+    const int need_0 = !act_is_q8k(gate_type) || !act_is_q8k(up_type);
+    xq_make(&xq, x, hidden, need_k, need_0);
+    expert_ffn_q(gate_type, up_type, down_type, gate, up, down, hidden, ffn, &xq, out, gate_up, act, act_qs, act_d,
+                 gate_up_partials, down_partials);
+    xq_free(&xq);
+}
+
+typedef struct {
+    const wdo_layer *L;
+    const xq_t *xq;
+    wdo_dump *dump;
+    const int *ids;
+    float *expert_out; /* [k][H] */
+    float *shared_out; /* [H] */
+    int n_tasks;       /* k (+1 when a shared expert exists) */
+    int next;
+    pthread_mutex_t mu;
+} layer_job;
+
+static void run_task(layer_job *job, int t) {
+    const wdo_layer *L = job->L;
+    const int H = L->hidden, F = L->expert_ffn, k = L->top_k;
+    wdo_dump *dp = job->dump;
+    if (t < k) {
+        const int e = job->ids[t];
+        const size_t gs = (size_t)F * wdo_row_bytes(L->gate_type, H);
+        const size_t us = (size_t)F * wdo_row_bytes(L->up_type, H);
+        const size_t ds = (size_t)H * wdo_row_bytes(L->down_type, F);
+        const int ppg = partials_per_row(L->gate_type, H);
+        const int ppd = partials_per_row(L->down_type, F);
+        expert_ffn_q(L->gate_type, L->up_type, L->down_type, L->gate + gs * (size_t)e, L->up + us * (size_t)e,
+                     L->down + ds * (size_t)e, H, F, job->xq, job->expert_out + (size_t)t * H,
+                     dp && dp->gate_up ? dp->gate_up + (size_t)t * 2 * F : NULL,
+                     dp && dp->act ? dp->act + (size_t)t * F : NULL,
+                     dp && dp->act_qs ? dp->act_qs + (size_t)t * F : NULL,
+                     dp && dp->act_d ? dp->act_d + (size_t)t * (F / 32) : NULL,
+                     dp && dp->gate_up_partials ? dp->gate_up_partials + (size_t)t * 2 * F * ppg : NULL,
+                     dp && dp->down_partials ? dp->down_partials + (size_t)t * H * ppd : NULL);
+    } else {
+        expert_ffn_q(L->shared_type, L->shared_type, L->shared_type, L->shared_gate, L->shared_up, L->shared_down, H,
+                     F, job->xq, job->shared_out, NULL, NULL, NULL, NULL, NULL, NULL);
+    }
+}
+
+static void *worker(void *arg) {
+    layer_job *job = (layer_job *)arg;
+    for (;;) {
+        pthread_mutex_lock(&job->mu);
+        const int t = job->next++;
+        pthread_mutex_unlock(&job->mu);
+        if (t >= job->n_tasks) break;
+        run_task(job, t);
+    }
+    return NULL;
+}
+
+void wdo_moe_layer_mt(const wdo_layer *L, const float *x, float *out, wdo_dump *dump, int preselected,
+                      int threads) {
+    const int H = L->hidden, E = L->n_experts, k = L->top_k;
+    const int has_shared = L->shared_gate_inp != NULL;
+    int *ids = (int *)malloc(sizeof(int) * (size_t)k);
+    float *wts = (float *)malloc(sizeof(float) * (size_t)k);
+    if (preselected) {
+        memcpy(ids, dump->ids, sizeof(int) * (size_t)k);
+        memcpy(wts, dump->weights, sizeof(float) * (size_t)k);
+    } else {
+        float *logits = (float *)malloc(sizeof(float) * (size_t)E);
+        float *probs = (float *)malloc(sizeof(float) * (size_t)E);
+        wdo_router_logits(L->router, x, E, H, logits);
+        wdo_softmax_row(logits, E, probs);
+        wdo_router_select(probs, E, k, L->w_scale, ids, wts);
+        if (dump && dump->logits) memcpy(dump->logits, logits, sizeof(float) * (size_t)E);
+        if (dump && dump->ids) memcpy(dump->ids, ids, sizeof(int) * (size_t)k);
+        if (dump && dump->weights) memcpy(dump->weights, wts, sizeof(float) * (size_t)k);
+        free(logits);
+        free(probs);
+    }
+
+    xq_t xq;
+    const int any_k = act_is_q8k(L->gate_type) || act_is_q8k(L->up_type);
+    const int any_0 = !act_is_q8k(L->gate_type) || !act_is_q8k(L->up_type) || has_shared;
+    xq_make(&xq, x, H, any_k, any_0);
+
+    layer_job job;
+    job.L = L;
+    job.xq = &xq;
+    job.dump = dump;
+    job.ids = ids;
+    job.expert_out = (dump && dump->expert_out) ? dump->expert_out : (float *)malloc(sizeof(float) * (size_t)k * H);
+    job.shared_out = (dump && dump->shared_out) ? dump->shared_out : (float *)malloc(sizeof(float) * (size_t)H);
+    job.n_tasks = k + (has_shared ? 1 : 0);
+    job.next = 0;
+    pthread_mutex_init(&job.mu, NULL);
+    if (threads <= 1) {
+        for (int t = 0; t < job.n_tasks; ++t) run_task(&job, t);
+    } else {
+        if (threads > 64) threads = 64;
+        pthread_t th[64];
+        for (int i = 1; i < threads; ++i) pthread_create(&th[i], NULL, worker, &job);
+        worker(&job);
+        for (int i = 1; i < threads; ++i) pthread_join(th[i], NULL);
+    }
+    pthread_mutex_destroy(&job.mu);
+
+    /* ordered combine: product rounded, then sum rounded, top-k order */
+    for (int i = 0; i < H; ++i) out[i] = 0.0f;
+    for (int j = 0; j < k; ++j) {
+        const float *src = job.expert_out + (size_t)j * H;
+        const float wj = wts[j];
+        for (int i = 0; i < H; ++i) {
+            const float prod = src[i] * wj;
+            out[i] = out[i] + prod;
+        }
+    }
+    if (dump && dump->routed) memcpy(dump->routed, out, sizeof(float) * (size_t)H);
+    if (has_shared) {
+        const float g = wdo_sigmoid_ggml(wdo_dot_f32(L->shared_gate_inp, x, H));
+        if (dump && dump->shared_gate) *dump->shared_gate = g;
+        for (int i = 0; i < H; ++i) {
+            const float prod = job.shared_out[i] * g;
+            out[i] = out[i] + prod;
+        }
+    }
+    if (!(dump && dump->expert_out)) free(job.expert_out);
+    if (!(dump && dump->shared_out)) free(job.shared_out);
+    xq_free(&xq);
+    free(ids);
+    free(wts);
+}
+
+void wdo_moe_layer(const wdo_layer *L, const float *x, float *out, wdo_dump *dump, int preselected) {
+    wdo_moe_layer_mt(L, x, out, dump, preselected, 1);
+}

@@ -1,0 +1,27 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def oracle():
+    from oracle import pyoracle
+    pyoracle.lib()
+    return pyoracle
+
+
+@pytest.fixture(scope="session")
+def refcpu(oracle):
+    """The reference's own CPU header behind oracle/ref_shim.cpp; skips when it was not built."""
+    if oracle.ref() is None:
+        pytest.skip("oracle/_ref/libwdref.so not built (reference tree absent)")
+    return oracle
