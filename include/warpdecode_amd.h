@@ -1,0 +1,221 @@
+/*
+ * warpdecode_amd — C ABI of the MI355X (gfx950) batch=1 MoE decode path.
+ *
+ * Plain C: pointers and sizes only.  Every pointer named `d_*` or documented as
+ * "device" is HBM memory of the current HIP device; `stream` is a hipStream_t
+ * passed as void* (NULL = the default stream).  Every function returns 0 on
+ * success and a negative wd_status otherwise; wd_last_error() gives the text.
+ * Nothing here allocates device memory except the functions that say so.
+ *
+ * The reference engine has no C ABI of its own: its operator surface is a set of
+ * inline C++ launchers and RAII classes (namespace wd).  Each entry point below
+ * cites the reference launcher it replaces; host/wd_ops.hpp in this repository
+ * re-creates those C++ names on top of this ABI.
+ */
+#ifndef WARPDECODE_AMD_H
+#define WARPDECODE_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    WD_OK = 0,
+    WD_ERR_ARG = -1,      /* geometry / type / null-pointer error (reference: std::runtime_error) */
+    WD_ERR_HIP = -2,      /* a HIP runtime call failed */
+    WD_ERR_STATE = -3,    /* object used before initialisation / after destruction */
+    WD_ERR_UNSUPPORTED = -4
+} wd_status;
+
+/* GGML tensor type ids (reference: src/gguf.hpp:26-44). */
+typedef enum {
+    WD_TYPE_F32 = 0,
+    WD_TYPE_F16 = 1,
+    WD_TYPE_Q4_0 = 2,
+    WD_TYPE_Q8_0 = 8,
+    WD_TYPE_IQ4_NL = 20,
+    WD_TYPE_IQ3_S = 21,
+    WD_TYPE_IQ2_S = 22
+} wd_type;
+
+/* ---- library ------------------------------------------------------------- */
+const char *wd_last_error(void);
+/* Selects the device, checks it is gfx950-class and uploads the codebooks. */
+int wd_init(int device);
+/* Bytes of one row / of a whole [rows][cols] tensor of `type` (reference: TensorInfo::byte_size,
+ * src/gguf.hpp:276-310).  0 for an unsupported type or a column count that is not whole blocks. */
+size_t wd_row_bytes(int type, int cols);
+size_t wd_tensor_bytes(int type, int rows, int cols);
+
+/* ---- thin runtime helpers (reference: cudaMalloc / cudaMallocHost / cudaMemcpyAsync /
+ *      stream and event calls made inline by src/lowbit.cuh, src/expert_cache.cuh) ---------- */
+int wd_malloc(void **d_ptr, size_t bytes);
+int wd_free(void *d_ptr);
+int wd_malloc_host(void **h_ptr, size_t bytes);   /* pinned */
+int wd_free_host(void *h_ptr);
+int wd_memcpy_h2d(void *d_dst, const void *h_src, size_t bytes, void *stream); /* async when stream != NULL */
+int wd_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream);
+int wd_memset(void *d_dst, int value, size_t bytes, void *stream);
+int wd_stream_create(void **stream);
+int wd_stream_destroy(void *stream);
+int wd_stream_sync(void *stream);
+int wd_device_sync(void);
+
+/* ---- activation quantisers -------------------------------------------------
+ * Q8_K: 256-value blocks, int8 quants, f32 scale (always negative), int16 sums of 16.
+ *   reference: launch_q8_k_quantize_f32, src/lowbit.cuh:873-891; CPU quantize_q8_K,
+ *   src/qwen38_cpu_moe.cuh:239-263.  elements % 256 == 0.
+ * Q8_0: 32-value blocks, int8 quants, fp16 scale.
+ *   reference: q38_moe_quantize_activation_q8_0, src/qwen38_moe.cuh:1470-1481 and
+ *   q38_hc_q8_0_quantize_f32_exact_kernel, src/qwen38_hc.cuh:368-392; CPU quantize_q8_0,
+ *   src/qwen38_cpu_moe.cuh:220-237.  elements % 32 == 0.  Also the activation format of the dense
+ *   Q4_0 path (reference: q8_0_quantize_half_kernel, src/warodecode.cu:1504-1520). */
+int wd_q8_k_quantize_f32(const float *d_x, int elements, int8_t *d_qs, float *d_scales, int16_t *d_bsums,
+                         void *stream);
+int wd_q8_0_quantize_f32(const float *d_x, int elements, int8_t *d_qs, uint16_t *d_scales, void *stream);
+
+/* ---- router ----------------------------------------------------------------
+ * logits[r] = dot(w[r,:], x) in the 4x8-accumulator order of ggml_vec_dot_f32.
+ *   reference: launch_q38_router_gemv_f32, src/qwen38_moe.cuh:247-263.  w is f32 [rows][cols]. */
+int wd_router_gemv_f32(const float *d_w, const float *d_x, float *d_logits, int rows, int cols, void *stream);
+/* softmax over all experts, top-k by probability (ties to the lower id), renormalise, optional scale.
+ *   reference: q38_launch_topk_softmax, src/qwen38_moe.cuh:1065-1090.
+ *   n_experts % 8 == 0, n_experts <= 1024, 0 < k <= 16.  ids int32[k], weights f32[k] (device). */
+int wd_topk_softmax(const float *d_logits, int n_experts, int k, float expert_scale, int32_t *d_ids,
+                    float *d_weights, void *stream);
+
+/* ---- low-bit GEMV, one matrix ------------------------------------------------
+ * out[r] = row_dot(w[r], activation).  w: raw GGUF block bytes, rows packed back to back.
+ * `d_partials` (may be NULL) receives the exact int32 chunk sums used for parity checks:
+ *   IQ3_S / IQ2_S : [rows][cols/256][8];  Q8_0 / IQ4_NL : [rows][cols/32][8];  Q4_0 : [rows][cols/32].
+ * reference: launch_iq3_s_gemv_q8_k_f32 (src/lowbit.cuh:1483), launch_iq2_s_gemv_q8_k_f32 (:1181),
+ *   q38_hc_launch_exact_q8_0_gemv_f32 (src/qwen38_hc.cuh:1020-1049),
+ *   q4_0_q8_0_gemv_kernel via launch_q4_float (src/warodecode.cu:1534-1562, :1746-1768; the planar
+ *   prepack of the reference is not needed: raw 18-byte blocks are read directly). */
+int wd_gemv_q8_k_f32(int type, const uint8_t *d_w, int rows, int cols, const int8_t *d_act_qs,
+                     const float *d_act_scales, float *d_out, int32_t *d_partials, void *stream);
+int wd_gemv_q8_0_f32(int type, const uint8_t *d_w, int rows, int cols, const int8_t *d_act_qs,
+                     const uint16_t *d_act_scales, float *d_out, int32_t *d_partials, void *stream);
+
+/* ---- low-bit GEMV, one dispatch over several expert matrices ------------------
+ * out[e][r] for e < experts; d_w_experts is a DEVICE array of `experts` device pointers
+ * (the reference's expert pointer table).  One shared activation.
+ * reference: launch_iq3_s_gemv_q8_k_experts_f32 (src/lowbit.cuh:2390-2418),
+ *            launch_iq2_s_gemv_q8_k_experts_f32 (:2352-2388).  experts <= 64. */
+int wd_gemv_q8_k_experts_f32(int type, const uint8_t *const *d_w_experts, int experts, int rows, int cols,
+                             const int8_t *d_act_qs, const float *d_act_scales, float *d_out,
+                             int32_t *d_partials, void *stream);
+/* Per-expert activations act[e][cols] (the down projection): reference down stage of
+ * q38_moe_run_batched_experts, src/qwen38_moe.cuh:3313-3388. */
+int wd_gemv_q8_0_experts_f32(int type, const uint8_t *const *d_w_experts, int experts, int rows, int cols,
+                             const int8_t *d_act_qs, const uint16_t *d_act_scales, float *d_out,
+                             int32_t *d_partials, void *stream);
+
+/* ---- elementwise stages ------------------------------------------------------
+ * act[e][i] = silu_ggml(gate_up[e][0][i]) * gate_up[e][1][i]
+ *   reference: q38_moe_silu_scale_mul_experts_kernel, src/qwen38_moe.cuh:1240-1254. */
+int wd_silu_mul_experts_f32(const float *d_gate_up, float *d_act, int ffn, int experts, void *stream);
+/* accum[i] = add_rn(accum[i], mul_rn(experts[j][i], weights[j])) for j ascending.
+ *   reference: q38_moe_weighted_accum_experts_f32_kernel, src/qwen38_moe.cuh:1291-1304. */
+int wd_weighted_accum_experts_f32(const float *d_experts, const float *d_weights, float *d_accum, int n, int k,
+                                  void *stream);
+/* routed[i] = add_rn(routed[i], mul_rn(shared[i], gate[0])).
+ *   reference: q38_add_shared_f32_kernel / q38_finish_moe_f32, src/qwen38_moe.cuh:1691-1699, :2442-2453. */
+int wd_add_shared_f32(float *d_routed, const float *d_shared, const float *d_gate, int n, void *stream);
+
+/* ---- whole layer ---------------------------------------------------------------
+ * Device-side description of one MoE layer.  Expert e of a routed tensor lives at
+ * base + e * stride (raw GGUF bytes, the layout of a 3-D GGUF expert tensor) unless
+ * `slot_of_expert` is set, in which case it lives in slot slot_of_expert[e] of an
+ * expert-slot pool: gate at pool + slot*slot_bytes, up at + gate_bytes, down at
+ * + gate_bytes + up_bytes (reference: GpuExpertCache::views, src/expert_cache.cuh:2495-2511).
+ */
+typedef struct {
+    int hidden, expert_ffn, n_experts, top_k;
+    float expert_scale;            /* 0 or 1 = none (reference: q38_moe_router_select w_scale) */
+    int gate_type, up_type, down_type;
+    const float *router;           /* device f32 [n_experts][hidden] */
+    const uint8_t *gate, *up, *down;          /* device bases (resident mode) */
+    size_t gate_stride, up_stride, down_stride; /* bytes per expert */
+    const int32_t *slot_of_expert; /* device int32 [n_experts] or NULL */
+    const uint8_t *slot_pool;      /* device */
+    size_t slot_bytes, slot_gate_bytes, slot_up_bytes;
+    /* shared expert (Q8_0); shared_gate_inp == NULL disables it */
+    const float *shared_gate_inp;  /* device f32 [hidden] */
+    const uint8_t *shared_gate, *shared_up, *shared_down; /* device Q8_0 */
+} wd_moe_layer;
+
+/* Scratch for a layer pass (device memory owned by the library object). */
+typedef struct wd_moe_scratch wd_moe_scratch;
+int wd_moe_scratch_create(wd_moe_scratch **out, int hidden, int expert_ffn, int n_experts, int max_k);
+int wd_moe_scratch_destroy(wd_moe_scratch *s);
+/* Device views, named after Qwen38MoeScratch accessors (src/qwen38_moe.cuh:1701-2150). */
+float *wd_moe_scratch_logits(wd_moe_scratch *s);      /* f32 [n_experts] */
+int32_t *wd_moe_scratch_ids(wd_moe_scratch *s);       /* i32 [k] */
+float *wd_moe_scratch_weights(wd_moe_scratch *s);     /* f32 [k] */
+float *wd_moe_scratch_gate_up(wd_moe_scratch *s);     /* f32 [k+1][2][ffn] (slot k = shared expert) */
+float *wd_moe_scratch_act(wd_moe_scratch *s);         /* f32 [k+1][ffn] */
+int8_t *wd_moe_scratch_act_qs(wd_moe_scratch *s);     /* i8  [k+1][ffn] */
+uint16_t *wd_moe_scratch_act_scales(wd_moe_scratch *s); /* f16 [k+1][ffn/32] */
+float *wd_moe_scratch_expert_out(wd_moe_scratch *s);  /* f32 [k+1][hidden] (only with keep_expert_out) */
+float *wd_moe_scratch_accum(wd_moe_scratch *s);       /* f32 [hidden] routed weighted sum (d_accum) */
+float *wd_moe_scratch_down_f32(wd_moe_scratch *s);    /* f32 [hidden] shared expert output (down_f32) */
+float *wd_moe_scratch_shared_gate(wd_moe_scratch *s); /* f32 [1] sigmoid gate (d_shared_gate) */
+int32_t *wd_moe_scratch_gate_up_partials(wd_moe_scratch *s); /* NULL until enabled */
+int32_t *wd_moe_scratch_down_partials(wd_moe_scratch *s);
+/* Allocates the int32 chunk-sum dumps ([k][2][ffn][P_gate] and [k][hidden][P_down]) and makes the
+ * layer pass fill them.  Parity harness only. */
+int wd_moe_scratch_enable_partials(wd_moe_scratch *s, int gate_type, int down_type);
+
+/* flags for wd_moe_layer_f32 */
+#define WD_MOE_PRESELECTED 1u      /* ids/weights already in scratch: skip the router (reference `preselected`) */
+#define WD_MOE_KEEP_EXPERT_OUT 2u  /* also store the per-expert down outputs in scratch */
+
+/* One decode step of one layer: router -> top-k -> grouped gate/up -> SwiGLU -> Q8_0 ->
+ * grouped down -> ordered weighted sum -> + shared * sigmoid gate.  d_out is f32 [hidden]
+ * = q38_moe_branch_f32(routed, shared, gate).  The routed sum, the shared expert output and the
+ * gate are left in the scratch views above, as the reference leaves them for its caller.
+ * reference: run_qwen38_routed_moe_separate_f32_x (src/qwen38_moe.cuh:3650-3779) +
+ *   run_qwen38_shared_expert_f32_x (:3963-3969) + q38_finish_moe_f32 (:2442-2453). */
+int wd_moe_layer_f32(const wd_moe_layer *layer, const float *d_x, float *d_out, wd_moe_scratch *scratch,
+                     unsigned flags, void *stream);
+
+/* M tokens through one layer; the weights of an expert selected by several tokens are read once.
+ * d_x f32 [tokens][hidden], d_out f32 [tokens][hidden].  Bit-identical to `tokens` calls of
+ * wd_moe_layer_f32.  tokens <= 8.  reference: Qwen38MoeTokenBatch, src/qwen38_moe.cuh:2743-3237
+ * (which re-reads the weights per (token, expert) pair). */
+int wd_moe_layer_tokens_f32(const wd_moe_layer *layer, const float *d_x, float *d_out, int tokens,
+                            wd_moe_scratch *const *scratch_per_token, unsigned flags, void *stream);
+
+/* ---- expert-slot cache -----------------------------------------------------------
+ * LRU pool of fixed-size slots in HBM, key (layer << 32 | expert); a miss copies the expert's
+ * gate|up|down slices from pinned host memory with hipMemcpyAsync on a private copy stream and
+ * makes `stream` wait for it.  reference: GpuExpertCache (src/expert_cache.cuh:2156-2536),
+ * ExpertStagePath (:858-1583), ExpertCacheMonitor (:1592-2105). */
+typedef struct wd_expert_cache wd_expert_cache;
+typedef struct {
+    uint64_t accesses, hits, misses, evictions, bytes_copied;
+    uint64_t slots, slot_bytes, resident;
+} wd_expert_cache_stats;
+int wd_expert_cache_create(wd_expert_cache **out, size_t capacity_bytes, size_t gate_bytes, size_t up_bytes,
+                           size_t down_bytes, int n_layers, int n_experts, int layer_partition);
+int wd_expert_cache_destroy(wd_expert_cache *c);
+/* Host (pinned) sources of one layer's 3-D expert tensors; strides are bytes per expert. */
+int wd_expert_cache_register_layer(wd_expert_cache *c, int layer, const uint8_t *h_gate, const uint8_t *h_up,
+                                   const uint8_t *h_down);
+/* Makes `k` experts of `layer` resident (LRU order of the ids given), updates the device slot table
+ * of that layer and returns, per id, whether it was a hit.  All k slots stay valid until the next
+ * acquire call on this cache.  hit_out may be NULL. */
+int wd_expert_cache_acquire(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uint8_t *hit_out,
+                            void *stream);
+const int32_t *wd_expert_cache_slot_table(wd_expert_cache *c, int layer); /* device int32 [n_experts] */
+const uint8_t *wd_expert_cache_pool(wd_expert_cache *c);
+int wd_expert_cache_get_stats(wd_expert_cache *c, wd_expert_cache_stats *out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,36 @@
+"""CPU-side checks of the drop-in boundary: the shared library loads without a GPU, exports every
+symbol the public header declares, and reports errors instead of computing without a device."""
+import ctypes as C
+
+import pytest
+
+from warpdecode_amd import capi, synth
+
+
+def test_exports_every_declared_symbol():
+    lib = capi.load()
+    declared = capi.declared_symbols()
+    assert len(declared) >= 40
+    missing = [s for s in declared if not hasattr(lib, s)]
+    assert not missing, missing
+
+
+@pytest.mark.parametrize("t", [synth.Q4_0, synth.Q8_0, synth.IQ4_NL, synth.IQ3_S, synth.IQ2_S])
+def test_block_geometry(t):
+    lib = capi.load()
+    assert lib.wd_row_bytes(t, 2048) == synth.row_bytes(t, 2048)
+    assert lib.wd_row_bytes(t, 2048 + 1) == 0
+    assert lib.wd_tensor_bytes(t, 512, 2048) == 512 * synth.row_bytes(t, 2048)
+    assert lib.wd_row_bytes(99, 2048) == 0
+
+
+def test_argument_errors_are_reported():
+    lib = capi.load()
+    # geometry is validated before any device work, so these fail the same way with or without a GPU
+    assert lib.wd_q8_k_quantize_f32(None, 100, None, None, None, None) == -1
+    assert b"multiple of 256" in lib.wd_last_error()
+    assert lib.wd_topk_softmax(None, 12, 2, 1.0, None, None, None) == -1
+    assert b"multiple of 8" in lib.wd_last_error()
+    assert lib.wd_gemv_q8_k_f32(synth.Q8_0, C.c_void_p(8), 4, 256, None, None, None, None, None) == -1
+    with pytest.raises(capi.WdError):
+        capi.call("wd_q8_0_quantize_f32", None, 33, None, None, None)

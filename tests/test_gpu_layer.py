@@ -1,0 +1,123 @@
+"""GPU parity of the whole MoE layer against the CPU oracle: routed ids, router weights, the int32
+chunk sums of every selected expert's gate/up/down projection, and the f32 layer output."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from warpdecode_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+SEED = 20261014
+
+
+@pytest.fixture(scope="module")
+def g():
+    import gpu_util
+    gpu_util.init()
+    return gpu_util
+
+
+def run_layer(g, L, x, partials=True, flags=0, ids=None, weights=None):
+    H, F, E, k = L["hidden"], L["expert_ffn"], L["n_experts"], L["top_k"]
+    dl = g.DeviceLayer(L)
+    sc = g.Scratch(H, F, E, k)
+    if partials:
+        capi.call("wd_moe_scratch_enable_partials", sc.h, L["gate_type"], L["down_type"])
+    if ids is not None:
+        capi.call("wd_memcpy_h2d", C.c_void_p(sc.raw("ids")), np.asarray(ids, np.int32).ctypes.data_as(C.c_void_p),
+                  4 * k, None)
+        capi.call("wd_memcpy_h2d", C.c_void_p(sc.raw("weights")),
+                  np.asarray(weights, np.float32).ctypes.data_as(C.c_void_p), 4 * k, None)
+    dx, out = g.dev(x), g.empty(H, np.float32)
+    capi.call("wd_moe_layer_f32", C.byref(dl.desc), g.ptr(dx), g.ptr(out), sc.h, flags, g.stream())
+    g.sync()
+    res = dict(out=g.host(out), ids=sc.get("ids", k, np.int32), weights=sc.get("weights", k, np.float32),
+               logits=sc.get("logits", E, np.float32), accum=sc.get("accum", H, np.float32),
+               act=sc.get("act", k * F, np.float32).reshape(k, F),
+               act_qs=sc.get("act_qs", k * F, np.int8).reshape(k, F),
+               act_d=sc.get("act_scales", k * (F // 32), np.uint16).reshape(k, F // 32))
+    if L.get("shared_gate_inp") is not None:
+        res["shared_gate"] = sc.get("shared_gate", 1, np.float32)
+        res["down_f32"] = sc.get("down_f32", H, np.float32)
+    if partials:
+        from oracle import pyoracle
+        pg, pd = pyoracle.partials_per_row(L["gate_type"], H), pyoracle.partials_per_row(L["down_type"], F)
+        res["gate_up_partials"] = sc.get("gate_up_partials", k * 2 * F * pg, np.int32).reshape(k, 2, F, pg)
+        res["down_partials"] = sc.get("down_partials", k * H * pd, np.int32).reshape(k, H, pd)
+    sc.close()
+    return res
+
+
+def check_layer(g, oracle, L, x, **kw):
+    want, d = oracle.moe_layer(L, x, ids=kw.get("ids"), weights=kw.get("weights"), want_partials=True)
+    got = run_layer(g, L, x, **kw)
+    assert np.array_equal(got["ids"], d["ids"])
+    assert g.same_bits(got["weights"], d["weights"])
+    if kw.get("ids") is None:
+        assert g.same_bits(got["logits"], d["logits"])
+    assert np.array_equal(got["gate_up_partials"], d["gate_up_partials"])
+    assert g.same_bits(got["act"], d["act"])
+    assert np.array_equal(got["act_qs"], d["act_qs"]) and np.array_equal(got["act_d"], d["act_d"])
+    assert np.array_equal(got["down_partials"], d["down_partials"])
+    assert g.same_bits(got["accum"], d["routed"])
+    if L.get("shared_gate_inp") is not None:
+        assert g.same_bits(got["shared_gate"], d["shared_gate"])
+        assert g.same_bits(got["down_f32"], d["shared_out"])
+    assert g.same_bits(got["out"], want)
+    rel = np.linalg.norm(got["out"] - want) / max(np.linalg.norm(want), 1e-30)
+    assert rel <= 1e-5
+    return got
+
+
+@pytest.mark.parametrize("gate_t,down_t,shared", [(synth.IQ3_S, synth.Q8_0, True), (synth.Q8_0, synth.Q8_0, False),
+                                                   (synth.IQ2_S, synth.IQ4_NL, True), (synth.IQ3_S, synth.IQ4_NL, False)])
+def test_small_layers(g, oracle, gate_t, down_t, shared):
+    for H, F, E, k in [(512, 64, 8, 2), (768, 96, 16, 4), (256, 32, 8, 8)]:
+        L = synth.make_layer(H, F, E, k, gate_t, down_t, shared, seed=SEED, layer=H + k,
+                             router_sigma=1.0 / np.sqrt(H))
+        x = synth.rms_normed(synth.rng_for(SEED, 41, H), H)
+        check_layer(g, oracle, L, x)
+
+
+def test_c0_layer(g, oracle):
+    """Workload C0: hidden 2048, 64 experts, top-8, ffn 512, all Q8_0."""
+    L = synth.make_c0()
+    for s in range(2):
+        x = synth.rms_normed(synth.rng_for(SEED, 42, s), 2048)
+        check_layer(g, oracle, L, x)
+
+
+def test_c2_layer(g, oracle):
+    """Workload C2: 512 experts, top-10, IQ3_S gate/up, Q8_0 down, shared expert."""
+    L = synth.make_c2()
+    for s in range(2):
+        x = synth.rms_normed(synth.rng_for(SEED, 43, s), 2048)
+        got = check_layer(g, oracle, L, x)
+        assert len(set(got["ids"].tolist())) == 10 and abs(float(got["weights"].sum()) - 1.0) < 1e-5
+
+
+def test_preselected(g, oracle):
+    L = synth.make_c2(n_experts=64)
+    x = synth.rms_normed(synth.rng_for(SEED, 44), 2048)
+    ids = np.array([5, 63, 0, 17, 9, 33, 2, 41, 60, 12], np.int32)
+    wts = np.full(10, 0.1, np.float32)
+    check_layer(g, oracle, L, x, flags=capi.MOE_PRESELECTED, ids=ids, weights=wts)
+
+
+def test_linearity_of_combine(g, oracle):
+    """Size-independent property at full C2 size: with preselected ids the routed sum is the ordered
+    weighted sum of single-expert passes (each run with weight 1)."""
+    L = synth.make_c2(n_experts=128)
+    x = synth.rms_normed(synth.rng_for(SEED, 45), 2048)
+    ids = np.arange(10, dtype=np.int32) * 7
+    wts = np.linspace(0.02, 0.18, 10).astype(np.float32)
+    full = run_layer(g, L, x, partials=False, flags=capi.MOE_PRESELECTED, ids=ids, weights=wts)
+    acc = np.zeros(2048, np.float32)
+    L1 = dict(L); L1["top_k"] = 1
+    for j in range(10):
+        one = run_layer(g, L1, x, partials=False, flags=capi.MOE_PRESELECTED, ids=ids[j:j + 1],
+                        weights=np.ones(1, np.float32))
+        acc = (acc + (one["accum"] * wts[j]).astype(np.float32)).astype(np.float32)
+    assert g.same_bits(acc, full["accum"])

@@ -1,0 +1,221 @@
+"""GPU parity of the stand-alone operators against the CPU oracle, through the C ABI.
+Integer outputs (quants, ids, int32 chunk sums) and the f32 results of every operator whose float
+order the reference fixes must match bit for bit; the dense Q4_0 GEMV (no canonical float order in
+the reference) is held to 1e-5 relative."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from warpdecode_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+SEED = 20261014
+
+
+@pytest.fixture(scope="module")
+def g():
+    import gpu_util
+    gpu_util.init()
+    return gpu_util
+
+
+def _act_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    xs = [rng.normal(0, 1, n), rng.normal(0, 1e-3, n), rng.normal(0, 1e-6, n), rng.uniform(-5, 5, n), np.zeros(n)]
+    x = rng.normal(0, 1, n); x[:256] = 0.0; xs.append(x)
+    x = rng.normal(0, 1, n); x[n // 2 + 3] = -37.5; xs.append(x)
+    xs.append(np.round(rng.normal(0, 20, n)) / 254.0 * 3.0)       # exact .5 products: half-to-even
+    xs.append(rng.normal(0, 3e-7, n))                              # fp16 scale below 2^-24 in some blocks
+    return [np.asarray(v, np.float32) for v in xs]
+
+
+@pytest.mark.parametrize("n", [256, 2048, 2560, 512 * 11])
+def test_quantize_q8_k(g, oracle, n):
+    for x in _act_cases(n, SEED + n):
+        dx = g.dev(x)
+        qs, d, bs = g.empty(n, np.int8), g.empty(n // 256, np.float32), g.empty(n // 16, np.int16)
+        capi.call("wd_q8_k_quantize_f32", g.ptr(dx), n, g.ptr(qs), g.ptr(d), g.ptr(bs), g.stream())
+        g.sync()
+        oq, od, ob = oracle.quantize_q8_K(x)
+        assert np.array_equal(g.host(qs), oq)
+        assert g.same_bits(g.host(d), od)
+        assert np.array_equal(g.host(bs), ob)
+
+
+@pytest.mark.parametrize("n", [32, 512, 2048, 512 * 11, 32 * 37])
+def test_quantize_q8_0(g, oracle, n):
+    for x in _act_cases(max(n, 256), SEED + 7 * n):
+        x = x[:n].copy()
+        dx = g.dev(x)
+        qs, d = g.empty(n, np.int8), g.empty(n // 32, np.uint16)
+        capi.call("wd_q8_0_quantize_f32", g.ptr(dx), n, g.ptr(qs), g.ptr(d), g.stream())
+        g.sync()
+        oq, od = oracle.quantize_q8_0(x)
+        assert np.array_equal(g.host(qs), oq)
+        assert np.array_equal(g.host(d, np.uint16), od)
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 2048), (512, 2048), (512, 2560), (5, 96), (9, 2048 + 17), (3, 7)])
+def test_router_gemv(g, oracle, rows, cols):
+    rng = synth.rng_for(SEED, 11, rows, cols)
+    w = rng.normal(0, 0.05, (rows, cols)).astype(np.float32)
+    x = rng.normal(0, 1, cols).astype(np.float32)
+    dw, dx, out = g.dev(w), g.dev(x), g.empty(rows, np.float32)
+    capi.call("wd_router_gemv_f32", g.ptr(dw), g.ptr(dx), g.ptr(out), rows, cols, g.stream())
+    g.sync()
+    assert g.same_bits(g.host(out), oracle.router_logits(w, x))
+
+
+def _logit_rows(n, seed):
+    rng = np.random.default_rng(seed)
+    rows = [rng.normal(0, s, n) for s in (0.5, 1.0, 3.0, 10.0, 40.0)]
+    rows.append(np.zeros(n))                                            # all equal
+    r = np.full(n, -5.0); r[[n - 1, 3, n // 2]] = 3.0; r[5] = 2.0; rows.append(r)   # exact ties
+    r = np.full(n, -np.inf); r[[1, 6]] = [1.0, 2.0]; rows.append(r)     # -inf cells
+    r = rng.normal(0, 1, n); r[2] = 300.0; rows.append(r)               # everything else underflows
+    r = np.round(rng.normal(0, 2, n)); rows.append(r)                   # many duplicate logits
+    r = rng.normal(0, 1, n); r[0] = 1e-40; r[1] = -1e-40; rows.append(r)  # denormal logits
+    return [np.asarray(v, np.float32) for v in rows]
+
+
+@pytest.mark.parametrize("n,k", [(8, 2), (64, 8), (512, 10), (1024, 16), (72, 8)])
+def test_topk_softmax(g, oracle, n, k):
+    for scale in (1.0, 2.5):
+        for logits in _logit_rows(n, SEED + n):
+            dl = g.dev(logits)
+            ids, wts = g.empty(k, np.int32), g.empty(k, np.float32)
+            capi.call("wd_topk_softmax", g.ptr(dl), n, k, scale, g.ptr(ids), g.ptr(wts), g.stream())
+            g.sync()
+            oi, ow = oracle.route(logits, k, scale)
+            assert np.array_equal(g.host(ids), oi), (logits[:8], g.host(ids), oi)
+            assert g.same_bits(g.host(wts), ow)
+
+
+def _quant_act(oracle, t, x):
+    if t in (synth.IQ3_S, synth.IQ2_S):
+        qs, d, _ = oracle.quantize_q8_K(x)
+    else:
+        qs, d = oracle.quantize_q8_0(x)
+    return qs, d
+
+
+GEMV_SHAPES = {
+    synth.IQ3_S: [(512, 2048), (64, 2560), (5, 256), (33, 4096)],
+    synth.IQ2_S: [(640, 2560), (512, 2048), (3, 256)],
+    synth.Q8_0: [(2048, 512), (512, 2048), (7, 96), (640, 2560), (18, 32)],
+    synth.IQ4_NL: [(2560, 640), (2048, 512), (5, 96), (9, 32 * 5)],
+    synth.Q4_0: [(2048, 2048), (2048, 8192), (8192, 2048), (1000, 2048), (6, 96)],
+}
+
+
+@pytest.mark.parametrize("t", list(GEMV_SHAPES))
+def test_gemv_single(g, oracle, t):
+    for rows, cols in GEMV_SHAPES[t]:
+        rng = synth.rng_for(SEED, 21, t, rows, cols)
+        w = synth.matrix(t, rng, rows, cols)
+        x = rng.normal(0, 1, cols).astype(np.float32)
+        qs, d = _quant_act(oracle, t, x)
+        ppr = oracle.partials_per_row(t, cols)
+        dw, dq, dd = g.dev(w), g.dev(qs), g.dev(d)
+        out, part = g.empty(rows, np.float32), g.empty((rows, ppr), np.int32)
+        fn = "wd_gemv_q8_k_f32" if t in (synth.IQ3_S, synth.IQ2_S) else "wd_gemv_q8_0_f32"
+        capi.call(fn, t, g.ptr(dw), rows, cols, g.ptr(dq), g.ptr(dd), g.ptr(out), g.ptr(part), g.stream())
+        out2 = g.empty(rows, np.float32)
+        capi.call(fn, t, g.ptr(dw), rows, cols, g.ptr(dq), g.ptr(dd), g.ptr(out2), None, g.stream())
+        g.sync()
+        want, wpart = oracle.gemv(t, w, rows, cols, qs, d, want_partials=True)
+        assert np.array_equal(g.host(part), wpart), (t, rows, cols)
+        if t == synth.Q4_0:
+            # tolerance 1e-5 relative to the magnitude of the terms (float order is free there)
+            rb = synth.row_bytes(t, cols)
+            mag = np.array([np.abs(oracle.dequant_row(t, w[r], cols)).sum() for r in range(min(rows, 64))]).mean()
+            assert np.allclose(g.host(out), want, rtol=1e-5, atol=1e-5 * mag), (rows, cols)
+            assert np.allclose(g.host(out2), want, rtol=1e-5, atol=1e-5 * mag)
+        else:
+            assert g.same_bits(g.host(out), want), (t, rows, cols)
+            assert g.same_bits(g.host(out2), want), (t, rows, cols)
+
+
+@pytest.mark.parametrize("t,rows,cols,experts", [(synth.IQ3_S, 512, 2048, 20), (synth.IQ2_S, 640, 2560, 20),
+                                                  (synth.IQ3_S, 37, 512, 3)])
+def test_gemv_experts_q8k(g, oracle, t, rows, cols, experts):
+    rng = synth.rng_for(SEED, 22, t, rows, cols)
+    ws = [synth.matrix(t, rng, rows, cols) for _ in range(experts)]
+    x = rng.normal(0, 1, cols).astype(np.float32)
+    qs, d = _quant_act(oracle, t, x)
+    dws = [g.dev(w) for w in ws]
+    table = g.dev(np.array([w.data_ptr() for w in dws], np.uint64))
+    dq, dd = g.dev(qs), g.dev(d)
+    ppr = oracle.partials_per_row(t, cols)
+    out, part = g.empty((experts, rows), np.float32), g.empty((experts, rows, ppr), np.int32)
+    capi.call("wd_gemv_q8_k_experts_f32", t, g.ptr(table), experts, rows, cols, g.ptr(dq), g.ptr(dd), g.ptr(out),
+              g.ptr(part), g.stream())
+    g.sync()
+    for e in range(experts):
+        want, wpart = oracle.gemv(t, ws[e], rows, cols, qs, d, want_partials=True)
+        assert np.array_equal(g.host(part)[e], wpart)
+        assert g.same_bits(g.host(out)[e], want)
+
+
+@pytest.mark.parametrize("t,rows,cols,experts", [(synth.Q8_0, 2048, 512, 10), (synth.IQ4_NL, 2560, 640, 10),
+                                                  (synth.Q8_0, 21, 96, 4)])
+def test_gemv_experts_q8_0(g, oracle, t, rows, cols, experts):
+    rng = synth.rng_for(SEED, 23, t, rows, cols)
+    ws = [synth.matrix(t, rng, rows, cols) for _ in range(experts)]
+    xs = rng.normal(0, 1, (experts, cols)).astype(np.float32)
+    qd = [oracle.quantize_q8_0(xs[e]) for e in range(experts)]
+    qs = np.stack([q for q, _ in qd]); d = np.stack([s for _, s in qd])
+    dws = [g.dev(w) for w in ws]
+    table = g.dev(np.array([w.data_ptr() for w in dws], np.uint64))
+    dq, dd = g.dev(qs), g.dev(d)
+    out = g.empty((experts, rows), np.float32)
+    capi.call("wd_gemv_q8_0_experts_f32", t, g.ptr(table), experts, rows, cols, g.ptr(dq), g.ptr(dd), g.ptr(out),
+              None, g.stream())
+    g.sync()
+    for e in range(experts):
+        assert g.same_bits(g.host(out)[e], oracle.gemv(t, ws[e], rows, cols, qs[e], d[e]))
+
+
+def test_elementwise(g, oracle):
+    rng = np.random.default_rng(SEED + 31)
+    F, k, H = 512, 10, 2048
+    gu = np.concatenate([rng.normal(0, 2, (k, 2, F - 8)), rng.normal(0, 30, (k, 2, 8))], axis=2).astype(np.float32)
+    dgu, act = g.dev(gu), g.empty((k, F), np.float32)
+    capi.call("wd_silu_mul_experts_f32", g.ptr(dgu), g.ptr(act), F, k, g.stream())
+    g.sync()
+    want = (oracle.silu_ggml(gu[:, 0, :]) * gu[:, 1, :]).astype(np.float32)
+    assert g.same_bits(g.host(act), want)
+
+    ex = rng.normal(0, 1, (k, H)).astype(np.float32)
+    w = rng.uniform(0, 0.3, k).astype(np.float32)
+    acc0 = rng.normal(0, 1, H).astype(np.float32)
+    dex, dw, dacc = g.dev(ex), g.dev(w), g.dev(acc0)
+    capi.call("wd_weighted_accum_experts_f32", g.ptr(dex), g.ptr(dw), g.ptr(dacc), H, k, g.stream())
+    g.sync()
+    want = acc0.copy()
+    for j in range(k):
+        want = (want + (ex[j] * w[j]).astype(np.float32)).astype(np.float32)
+    assert g.same_bits(g.host(dacc), want)
+    # negative control: a fused multiply-add accumulation is a different function
+    fused = acc0.astype(np.float64)
+    for j in range(k):
+        fused = np.float32(fused + ex[j].astype(np.float64) * np.float64(w[j])).astype(np.float64)
+    assert not g.same_bits(fused.astype(np.float32), want)
+
+    sh = rng.normal(0, 1, H).astype(np.float32)
+    gate = np.array([0.37], np.float32)
+    dsh, dg = g.dev(sh), g.dev(gate)
+    capi.call("wd_add_shared_f32", g.ptr(dacc), g.ptr(dsh), g.ptr(dg), H, g.stream())
+    g.sync()
+    assert g.same_bits(g.host(dacc), (want + (sh * gate[0]).astype(np.float32)).astype(np.float32))
+
+
+def test_error_paths(g):
+    x = g.empty(300, np.float32)
+    lib = capi.load()
+    assert lib.wd_q8_k_quantize_f32(g.ptr(x), 300, g.ptr(x), g.ptr(x), g.ptr(x), None) == -1
+    assert lib.wd_topk_softmax(g.ptr(x), 64, 17, 1.0, g.ptr(x), g.ptr(x), None) == -1
+    assert lib.wd_gemv_q8_0_f32(synth.IQ3_S, g.ptr(x), 4, 256, g.ptr(x), g.ptr(x), g.ptr(x), None, None) == -1
+    assert lib.wd_gemv_q8_k_f32(synth.IQ3_S, g.ptr(x), 4, 100, g.ptr(x), g.ptr(x), g.ptr(x), None, None) == -1

@@ -1,0 +1,317 @@
+// __global__ kernels of the stand-alone operators (64-wide wavefronts, 256-thread workgroups).
+#pragma once
+
+#include "wd_rows.cuh"
+
+namespace wd {
+
+// Where the weight matrices of a grouped dispatch live.
+//   table != null      matrix m = table[m]                       (expert pointer table)
+//   ids   != null      matrix m belongs to expert ids[m / per_expert], tensor m % per_expert:
+//                        resident:  base[t] + expert * stride[t]
+//                        slot pool: pool + slot_of_expert[expert] * slot_bytes + slot_off[t]
+//   otherwise          the single matrix `single`
+struct MatSrc {
+    const uint8_t *single;
+    const uint8_t *const *table;
+    const int32_t *ids;
+    int per_expert;
+    const uint8_t *base[2];
+    size_t stride[2];
+    const int32_t *slot_of_expert;
+    const uint8_t *pool;
+    size_t slot_bytes;
+    size_t slot_off[2];
+};
+
+WD_DEV const uint8_t *mat_ptr(const MatSrc &s, int m) {
+    if (s.table) return s.table[m];
+    if (s.ids) {
+        const int j = m / s.per_expert, t = m - j * s.per_expert;
+        const int e = s.ids[j];
+        if (s.slot_of_expert) return s.pool + static_cast<size_t>(s.slot_of_expert[e]) * s.slot_bytes + s.slot_off[t];
+        return s.base[t] + static_cast<size_t>(e) * s.stride[t];
+    }
+    return s.single;
+}
+
+__global__ void k_fill_u32(uint32_t *dst, uint32_t v, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = v;
+}
+
+// ---- Q8_K quantiser: one wave per 256-value block, four values per lane -------------------
+__global__ __launch_bounds__(256) void k_q8_k_quantize(const float *__restrict__ x, int blocks,
+                                                        int8_t *__restrict__ qs, float *__restrict__ scales,
+                                                        int16_t *__restrict__ bsums) {
+    const int lane = threadIdx.x & 63;
+    const int blk = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (blk >= blocks) return;
+    const float4 v = reinterpret_cast<const float4 *>(x + static_cast<size_t>(blk) * 256)[lane];
+    float amax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)),
+                                 __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
+    amax = wave_max(amax);
+    uint32_t packed = 0;
+    int part = 0;
+    float d = 0.0f;
+    if (amax != 0.0f) {
+        // always-negative inverse scale (reference convention): quants carry the sign of -x
+        const float iscale = -127.0f / amax;
+        const int q0 = min(127, static_cast<int>(__builtin_rintf(v.x * iscale)));
+        const int q1 = min(127, static_cast<int>(__builtin_rintf(v.y * iscale)));
+        const int q2 = min(127, static_cast<int>(__builtin_rintf(v.z * iscale)));
+        const int q3 = min(127, static_cast<int>(__builtin_rintf(v.w * iscale)));
+        packed = (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | (static_cast<uint32_t>(q3 & 0xff) << 24);
+        part = q0 + q1 + q2 + q3;
+        d = 1.0f / iscale;
+    }
+    reinterpret_cast<uint32_t *>(qs + static_cast<size_t>(blk) * 256)[lane] = packed;
+    part += lane_xor(part, 1);
+    part += lane_xor(part, 2);
+    if ((lane & 3) == 0) bsums[static_cast<size_t>(blk) * 16 + (lane >> 2)] = static_cast<int16_t>(part);
+    if (lane == 0) scales[blk] = d;
+}
+
+// ---- Q8_0 quantiser: eight lanes per 32-value block, four values per lane -----------------
+WD_DEV uint32_t q8_0_pack4(float4 v, float amax) {
+    if (amax == 0.0f) return 0u;
+    const float inv = 127.0f / amax;
+    const int q0 = max(-128, min(127, static_cast<int>(__builtin_rintf(v.x * inv))));
+    const int q1 = max(-128, min(127, static_cast<int>(__builtin_rintf(v.y * inv))));
+    const int q2 = max(-128, min(127, static_cast<int>(__builtin_rintf(v.z * inv))));
+    const int q3 = max(-128, min(127, static_cast<int>(__builtin_rintf(v.w * inv))));
+    return (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | (static_cast<uint32_t>(q3 & 0xff) << 24);
+}
+
+__global__ __launch_bounds__(256) void k_q8_0_quantize(const float *__restrict__ x, int blocks,
+                                                        int8_t *__restrict__ qs, uint16_t *__restrict__ scales) {
+    const int sub = threadIdx.x & 7;
+    const int blk = blockIdx.x * 32 + (threadIdx.x >> 3);
+    const bool on = blk < blocks;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (on) v = reinterpret_cast<const float4 *>(x + static_cast<size_t>(blk) * 32)[sub];
+    float amax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)),
+                                 __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
+    amax = __builtin_fmaxf(amax, lane_xor(amax, 1));
+    amax = __builtin_fmaxf(amax, lane_xor(amax, 2));
+    amax = __builtin_fmaxf(amax, lane_xor(amax, 4));
+    if (!on) return;
+    reinterpret_cast<uint32_t *>(qs + static_cast<size_t>(blk) * 32)[sub] = q8_0_pack4(v, amax);
+    if (sub == 0) scales[blk] = f2h_ref(amax / 127.0f);
+}
+
+// ---- router GEMV: 32 lanes per row, lane t owns accumulator t of the 4x8 scheme --------------
+// (src/qwen38_moe.cuh:198-245).  Optional extra row (the shared expert's gate vector).
+__global__ __launch_bounds__(256) void k_router_gemv(const float *__restrict__ w, const float *__restrict__ x,
+                                                      float *__restrict__ logits, int rows, int cols,
+                                                      const float *__restrict__ extra_w,
+                                                      float *__restrict__ extra_out) {
+    const int t = threadIdx.x & 31;
+    const int row = blockIdx.x * 8 + (threadIdx.x >> 5);
+    const int total = rows + (extra_w ? 1 : 0);
+    const bool on = row < total;
+    const float *wr = on ? (row < rows ? w + static_cast<size_t>(row) * cols : extra_w) : w;
+    const int np = cols & ~31;
+    float s = 0.0f;
+    if (on) {
+#pragma unroll 16
+        for (int i = 0; i < np; i += 32) s = __builtin_fmaf(wr[i + t], x[i + t], s);
+    }
+    float o = __shfl_down(s, 16, 32);
+    if (t < 16) s = s + o;
+    o = __shfl_down(s, 8, 32);
+    if (t < 8) s = s + o;
+    o = __shfl_down(s, 4, 32);
+    if (t < 4) s = s + o;
+    o = __shfl_down(s, 1, 32);
+    if (t == 0 || t == 2) s = s + o;
+    o = __shfl_down(s, 2, 32);
+    float acc = s + o;
+    if (on && t == 0) {
+        for (int c = np; c < cols; ++c) acc = acc + wr[c] * x[c];
+        if (row < rows)
+            logits[row] = acc;
+        else
+            extra_out[0] = acc;
+    }
+}
+
+// ---- softmax + top-k + renormalise: one wave (src/qwen38_moe.cuh:711-818) ---------------------
+// If gate_logit != null, gate_logit[0] is replaced by sigmoid_ggml(gate_logit[0]) (shared expert gate).
+__global__ __launch_bounds__(64) void k_topk_softmax(const float *__restrict__ logits, int n, int k, float w_scale,
+                                                      int32_t *__restrict__ ids, float *__restrict__ weights,
+                                                      float *__restrict__ gate_logit) {
+    __shared__ float probs[1024];
+    __shared__ double gsum[128];
+    __shared__ float top[16];
+    const int lane = threadIdx.x;
+    if (gate_logit && lane == 0) gate_logit[0] = sigmoid_ggml(gate_logit[0]);
+
+    float mx = -INFINITY;
+    for (int e = lane; e < n; e += 64) mx = __builtin_fmaxf(mx, logits[e]);
+    mx = wave_max(mx);
+    for (int e = lane; e < n; e += 64) probs[e] = exp_ggml(logits[e] - mx);
+    __syncthreads();
+    const int groups = n >> 3;
+    for (int g = lane; g < groups; g += 64) {
+        const float *v = probs + g * 8;
+        const float lo = v[0] + v[4], lh = v[2] + v[6], hi = v[1] + v[5], hh = v[3] + v[7];
+        gsum[g] = static_cast<double>((lo + lh) + (hi + hh));
+    }
+    __syncthreads();
+    double sum = 0.0;
+    for (int g = 0; g < groups; ++g) sum += gsum[g];  // every lane, same ascending order
+    float v[16];
+    if (sum == 0.0) {
+        for (int e = lane; e < n; e += 64) probs[e] = -INFINITY;
+    } else {
+        const float inv = static_cast<float>(1.0 / sum);
+        for (int e = lane; e < n; e += 64) probs[e] = probs[e] * inv;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int e = lane + 64 * i;
+        v[i] = (e < n) ? probs[e] : -INFINITY;
+    }
+    for (int j = 0; j < k; ++j) {
+        // lowest index among this lane's largest not-yet-taken probabilities
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            if (v[i] > bv) {
+                bv = v[i];
+                bi = lane + 64 * i;
+            }
+        }
+        const float m = wave_max(bv);
+        const int cand = (bv == m && m > -INFINITY) ? bi : 0x7fffffff;
+        int win = wave_min_i(cand);
+        if (win == 0x7fffffff) win = 0;  // nothing beats -inf: the reference keeps id 0
+        if (lane == 0) {
+            ids[j] = win;
+            top[j] = probs[win];
+        }
+        if ((win & 63) == lane) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                if ((win >> 6) == i) v[i] = -INFINITY;
+        }
+    }
+    __syncthreads();
+    if (lane == 0) {
+        double wsum = 0.0;
+        for (int j = 0; j < k; ++j) wsum += static_cast<double>(top[j]);
+        const float denom = __builtin_fmaxf(static_cast<float>(wsum), 6.103515625e-5f);
+        for (int j = 0; j < k; ++j) {
+            float wj = top[j] / denom;
+            if (w_scale != 0.0f && w_scale != 1.0f) wj = wj * w_scale;
+            weights[j] = wj;
+        }
+    }
+}
+
+// ---- IQ3_S / IQ2_S x Q8_K GEMV: 16 rows per workgroup, 4 per wave, grid.y = matrix -----------
+template <int TYPE, bool PART>
+__global__ __launch_bounds__(256) void k_gemv_iq(MatSrc src, int rows, int cols, const int8_t *__restrict__ act_qs,
+                                                  const float *__restrict__ act_d, float *__restrict__ out,
+                                                  int32_t *__restrict__ partials, int ppr) {
+    __shared__ IqTables tables;
+    stage_tables<TYPE == 21, TYPE == 22>(tables, threadIdx.x, 256);
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int m = blockIdx.y;
+    const uint8_t *w = mat_ptr(src, m);
+    const int nb = cols >> 8;
+    const size_t rb = static_cast<size_t>(nb) * (TYPE == 21 ? 110 : 82);
+    const int r0 = blockIdx.x * 16 + wave * 4;
+    for (int r = r0; r < min(rows, r0 + 4); ++r) {
+        int32_t *pp = PART ? partials + (static_cast<size_t>(m) * rows + r) * ppr : nullptr;
+        const float y = iq_row_q8k<TYPE, PART>(w + static_cast<size_t>(r) * rb, nb, tables, act_qs, act_d, lane, pp);
+        if (lane == 0) out[static_cast<size_t>(m) * rows + r] = y;
+    }
+}
+
+// ---- Q8_0 / IQ4_NL / Q4_0 x Q8_0 GEMV: 16 rows per workgroup, 4 per wave ----------------------
+// act_stride: elements between the activations of consecutive matrices (0 = one shared activation).
+template <int KIND, bool PART>
+__global__ __launch_bounds__(256) void k_gemv_q8(MatSrc src, int rows, int cols, const int8_t *__restrict__ act_qs,
+                                                  const uint16_t *__restrict__ act_d, int act_stride,
+                                                  float *__restrict__ out, int32_t *__restrict__ partials, int ppr) {
+    __shared__ Q8Tile tiles[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int m = blockIdx.y;
+    const uint8_t *w = mat_ptr(src, m);
+    const int nb = cols >> 5;
+    const int8_t *aq = act_qs + static_cast<size_t>(m) * act_stride;
+    const uint16_t *ad = act_d + static_cast<size_t>(m) * (act_stride >> 5);
+    const int r0 = blockIdx.x * 16 + wave * 4;
+    if (r0 >= rows) return;
+    const int nrows = min(4, rows - r0);
+    const size_t rb = static_cast<size_t>(nb) * (KIND == 0 ? 34 : 18);
+    int32_t *pp = PART ? partials + (static_cast<size_t>(m) * rows + r0) * ppr : nullptr;
+    float y;
+    if (KIND == 2)
+        y = q4_0_rows4<PART>(w + r0 * rb, nrows, nb, aq, ad, lane, pp);
+    else
+        y = q8_rows4<(KIND == 1 ? 1 : 0), PART>(w + r0 * rb, nrows, nb, aq, ad, tiles[wave], lane, pp);
+    const int r4 = lane >> 4;
+    if ((lane & 15) == 0 && r4 < nrows) out[static_cast<size_t>(m) * rows + r0 + r4] = y;
+}
+
+// ---- elementwise ---------------------------------------------------------------------------------
+__global__ void k_silu_mul_experts(const float *__restrict__ gate_up, float *__restrict__ act, int ffn) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= ffn) return;
+    const float *g = gate_up + static_cast<size_t>(2) * blockIdx.y * ffn;
+    act[static_cast<size_t>(blockIdx.y) * ffn + i] = silu_ggml(g[i]) * g[ffn + i];
+}
+
+__global__ void k_weighted_accum(const float *__restrict__ experts, const float *__restrict__ weights,
+                                 float *__restrict__ accum, int n, int k) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float a = accum[i];
+    for (int j = 0; j < k; ++j) {
+        const float prod = experts[static_cast<size_t>(j) * n + i] * weights[j];
+        a = a + prod;
+    }
+    accum[i] = a;
+}
+
+// out may alias routed
+__global__ void k_add_shared(const float *routed, const float *__restrict__ shared,
+                             const float *__restrict__ gate, float *out, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float prod = shared[i] * gate[0];
+    out[i] = routed[i] + prod;
+}
+
+// gate[0] = sigmoid_ggml(gate[0])
+__global__ void k_sigmoid1(float *gate) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) gate[0] = sigmoid_ggml(gate[0]);
+}
+
+// accum[i] = ordered weighted sum of the k expert outputs (product rounded, then sum rounded);
+// out[i] = accum[i] + shared[i] * gate[0] when a shared expert is present, else accum[i].
+__global__ void k_combine(const float *__restrict__ experts, const float *__restrict__ weights, int k,
+                          const float *__restrict__ shared, const float *__restrict__ gate,
+                          float *__restrict__ accum, float *__restrict__ out, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float a = 0.0f;
+    for (int j = 0; j < k; ++j) {
+        const float prod = experts[static_cast<size_t>(j) * n + i] * weights[j];
+        a = a + prod;
+    }
+    accum[i] = a;
+    if (shared) {
+        const float prod = shared[i] * gate[0];
+        a = a + prod;
+    }
+    out[i] = a;
+}
+
+}  // namespace wd

@@ -1,0 +1,293 @@
+// Whole-layer entry points: scratch object and the staged layer pass (one launch per stage,
+// every stage a stand-alone operator of wd_ops.hip resolved against the device-side ids).
+#include "wd_common.h"
+#include "wd_kernels.cuh"
+
+#include <new>
+
+using namespace wd;
+
+struct wd_moe_scratch {
+    int hidden = 0, ffn = 0, n_experts = 0, max_k = 0;
+    uint8_t *block = nullptr;
+    float *logits = nullptr;
+    int32_t *ids = nullptr;
+    float *weights = nullptr;
+    int8_t *xk_qs = nullptr;
+    float *xk_d = nullptr;
+    int16_t *xk_bs = nullptr;
+    int8_t *x0_qs = nullptr;
+    uint16_t *x0_d = nullptr;
+    float *gate_up = nullptr;
+    float *act = nullptr;
+    int8_t *act_qs = nullptr;
+    uint16_t *act_d = nullptr;
+    float *expert_out = nullptr;
+    float *accum = nullptr;
+    float *down_f32 = nullptr;
+    float *shared_gate = nullptr;
+    int32_t *gup = nullptr;
+    int32_t *dp = nullptr;
+    int gup_type = -1, dp_type = -1;
+};
+
+namespace {
+
+struct Carver {
+    size_t off = 0;
+    size_t take(size_t bytes) {
+        const size_t at = off;
+        off += (bytes + 255) & ~static_cast<size_t>(255);
+        return at;
+    }
+};
+
+}  // namespace
+
+extern "C" {
+
+int wd_moe_scratch_create(wd_moe_scratch **out, int hidden, int expert_ffn, int n_experts, int max_k) {
+    WD_REQUIRE(out != nullptr, "wd_moe_scratch_create: null output pointer");
+    WD_REQUIRE(hidden > 0 && hidden % 256 == 0, "MoE scratch: hidden must be a positive multiple of 256 (got %d)", hidden);
+    WD_REQUIRE(expert_ffn > 0 && expert_ffn % 32 == 0, "MoE scratch: expert_ffn must be a positive multiple of 32 (got %d)",
+               expert_ffn);
+    WD_REQUIRE(n_experts > 0 && max_k > 0 && max_k <= 16, "MoE scratch: invalid expert counts (%d experts, k=%d)",
+               n_experts, max_k);
+    wd_moe_scratch *s = new (std::nothrow) wd_moe_scratch;
+    WD_REQUIRE(s != nullptr, "MoE scratch: out of host memory");
+    s->hidden = hidden, s->ffn = expert_ffn, s->n_experts = n_experts, s->max_k = max_k;
+    const size_t H = hidden, F = expert_ffn, K1 = max_k + 1;
+    Carver c;
+    const size_t o_logits = c.take(sizeof(float) * n_experts), o_ids = c.take(sizeof(int32_t) * 16),
+                 o_w = c.take(sizeof(float) * 16), o_xkq = c.take(H), o_xkd = c.take(sizeof(float) * (H / 256)),
+                 o_xkb = c.take(sizeof(int16_t) * (H / 16)), o_x0q = c.take(H),
+                 o_x0d = c.take(sizeof(uint16_t) * (H / 32)), o_gu = c.take(sizeof(float) * K1 * 2 * F),
+                 o_act = c.take(sizeof(float) * K1 * F), o_aq = c.take(K1 * F),
+                 o_ad = c.take(sizeof(uint16_t) * K1 * (F / 32)), o_eo = c.take(sizeof(float) * K1 * H),
+                 o_acc = c.take(sizeof(float) * H), o_dn = c.take(sizeof(float) * H), o_sg = c.take(256);
+    const hipError_t e = hipMalloc(reinterpret_cast<void **>(&s->block), c.off);
+    if (e != hipSuccess) {
+        delete s;
+        return fail(WD_ERR_HIP, "hipMalloc MoE scratch (%zu bytes) failed: %s", c.off, hipGetErrorString(e));
+    }
+    uint8_t *b = s->block;
+    s->logits = reinterpret_cast<float *>(b + o_logits);
+    s->ids = reinterpret_cast<int32_t *>(b + o_ids);
+    s->weights = reinterpret_cast<float *>(b + o_w);
+    s->xk_qs = reinterpret_cast<int8_t *>(b + o_xkq);
+    s->xk_d = reinterpret_cast<float *>(b + o_xkd);
+    s->xk_bs = reinterpret_cast<int16_t *>(b + o_xkb);
+    s->x0_qs = reinterpret_cast<int8_t *>(b + o_x0q);
+    s->x0_d = reinterpret_cast<uint16_t *>(b + o_x0d);
+    s->gate_up = reinterpret_cast<float *>(b + o_gu);
+    s->act = reinterpret_cast<float *>(b + o_act);
+    s->act_qs = reinterpret_cast<int8_t *>(b + o_aq);
+    s->act_d = reinterpret_cast<uint16_t *>(b + o_ad);
+    s->expert_out = reinterpret_cast<float *>(b + o_eo);
+    s->accum = reinterpret_cast<float *>(b + o_acc);
+    s->down_f32 = reinterpret_cast<float *>(b + o_dn);
+    s->shared_gate = reinterpret_cast<float *>(b + o_sg);
+    (void)hipMemset(s->block, 0, c.off);
+    *out = s;
+    return WD_OK;
+}
+
+int wd_moe_scratch_destroy(wd_moe_scratch *s) {
+    if (!s) return WD_OK;
+    (void)hipFree(s->block);
+    (void)hipFree(s->gup);
+    (void)hipFree(s->dp);
+    delete s;
+    return WD_OK;
+}
+
+float *wd_moe_scratch_logits(wd_moe_scratch *s) { return s->logits; }
+int32_t *wd_moe_scratch_ids(wd_moe_scratch *s) { return s->ids; }
+float *wd_moe_scratch_weights(wd_moe_scratch *s) { return s->weights; }
+float *wd_moe_scratch_gate_up(wd_moe_scratch *s) { return s->gate_up; }
+float *wd_moe_scratch_act(wd_moe_scratch *s) { return s->act; }
+int8_t *wd_moe_scratch_act_qs(wd_moe_scratch *s) { return s->act_qs; }
+uint16_t *wd_moe_scratch_act_scales(wd_moe_scratch *s) { return s->act_d; }
+float *wd_moe_scratch_expert_out(wd_moe_scratch *s) { return s->expert_out; }
+float *wd_moe_scratch_accum(wd_moe_scratch *s) { return s->accum; }
+float *wd_moe_scratch_down_f32(wd_moe_scratch *s) { return s->down_f32; }
+float *wd_moe_scratch_shared_gate(wd_moe_scratch *s) { return s->shared_gate; }
+int32_t *wd_moe_scratch_gate_up_partials(wd_moe_scratch *s) { return s->gup; }
+int32_t *wd_moe_scratch_down_partials(wd_moe_scratch *s) { return s->dp; }
+
+int wd_moe_scratch_enable_partials(wd_moe_scratch *s, int gate_type, int down_type) {
+    WD_REQUIRE(s != nullptr, "enable partials: null scratch");
+    const int pg = partials_per_row(gate_type, s->hidden), pd = partials_per_row(down_type, s->ffn);
+    WD_REQUIRE(pg > 0 && pd > 0, "enable partials: unsupported tensor types %d / %d", gate_type, down_type);
+    (void)hipFree(s->gup);
+    (void)hipFree(s->dp);
+    s->gup = s->dp = nullptr;
+    WD_HIP(hipMalloc(reinterpret_cast<void **>(&s->gup), sizeof(int32_t) * s->max_k * 2 * s->ffn * pg));
+    WD_HIP(hipMalloc(reinterpret_cast<void **>(&s->dp), sizeof(int32_t) * s->max_k * s->hidden * pd));
+    s->gup_type = gate_type, s->dp_type = down_type;
+    return WD_OK;
+}
+
+}  // extern "C"
+
+namespace {
+
+int check_layer(const wd_moe_layer *L, const wd_moe_scratch *s) {
+    WD_REQUIRE(L && s, "MoE layer: null layer or scratch");
+    WD_REQUIRE(L->hidden == s->hidden && L->expert_ffn == s->ffn, "MoE layer geometry mismatch: layer %d/%d, scratch %d/%d",
+               L->hidden, L->expert_ffn, s->hidden, s->ffn);
+    WD_REQUIRE(L->n_experts > 0 && L->n_experts <= s->n_experts, "MoE layer: %d experts exceed the scratch (%d)",
+               L->n_experts, s->n_experts);
+    WD_REQUIRE(L->top_k > 0 && L->top_k <= s->max_k && L->top_k <= L->n_experts, "MoE layer: top_k %d out of range",
+               L->top_k);
+    WD_REQUIRE(L->gate_type == L->up_type, "MoE layer: gate and up tensors must share a type (%d vs %d)", L->gate_type,
+               L->up_type);
+    WD_REQUIRE(consumes_q8k(L->gate_type) || L->gate_type == WD_TYPE_Q8_0 || L->gate_type == WD_TYPE_IQ4_NL,
+               "MoE layer: unsupported gate/up type %d", L->gate_type);
+    WD_REQUIRE(L->down_type == WD_TYPE_Q8_0 || L->down_type == WD_TYPE_IQ4_NL, "MoE layer: unsupported down type %d",
+               L->down_type);
+    WD_REQUIRE(L->router != nullptr, "MoE layer: null router");
+    if (L->slot_of_expert) {
+        WD_REQUIRE(L->slot_pool != nullptr && L->slot_bytes > 0, "MoE layer: slot table without a slot pool");
+    } else {
+        WD_REQUIRE(L->gate && L->up && L->down, "MoE layer: null expert tensors");
+    }
+    if (L->shared_gate_inp) WD_REQUIRE(L->shared_gate && L->shared_up && L->shared_down, "MoE layer: incomplete shared expert");
+    return WD_OK;
+}
+
+MatSrc routed_src(const wd_moe_layer *L, const int32_t *ids, bool down) {
+    MatSrc m{};
+    m.ids = ids;
+    m.per_expert = down ? 1 : 2;
+    if (L->slot_of_expert) {
+        m.slot_of_expert = L->slot_of_expert;
+        m.pool = L->slot_pool;
+        m.slot_bytes = L->slot_bytes;
+        if (down) {
+            m.slot_off[0] = L->slot_gate_bytes + L->slot_up_bytes;
+        } else {
+            m.slot_off[0] = 0;
+            m.slot_off[1] = L->slot_gate_bytes;
+        }
+    } else if (down) {
+        m.base[0] = L->down;
+        m.stride[0] = L->down_stride;
+    } else {
+        m.base[0] = L->gate, m.base[1] = L->up;
+        m.stride[0] = L->gate_stride, m.stride[1] = L->up_stride;
+    }
+    return m;
+}
+
+template <int TYPE>
+void launch_iq(bool part, dim3 grid, hipStream_t st, MatSrc src, int rows, int cols, const int8_t *qs, const float *d,
+               float *out, int32_t *partials, int ppr) {
+    if (part)
+        k_gemv_iq<TYPE, true><<<grid, dim3(256), 0, st>>>(src, rows, cols, qs, d, out, partials, ppr);
+    else
+        k_gemv_iq<TYPE, false><<<grid, dim3(256), 0, st>>>(src, rows, cols, qs, d, out, nullptr, 0);
+}
+
+template <int KIND>
+void launch_q8(bool part, dim3 grid, hipStream_t st, MatSrc src, int rows, int cols, const int8_t *qs,
+               const uint16_t *d, int act_stride, float *out, int32_t *partials, int ppr) {
+    if (part)
+        k_gemv_q8<KIND, true><<<grid, dim3(256), 0, st>>>(src, rows, cols, qs, d, act_stride, out, partials, ppr);
+    else
+        k_gemv_q8<KIND, false><<<grid, dim3(256), 0, st>>>(src, rows, cols, qs, d, act_stride, out, nullptr, 0);
+}
+
+// One grouped GEMV of `mats` matrices of `type` ([rows][cols]) against the layer's quantised input
+// (shared activation) or against per-matrix Q8_0 activations (act_stride != 0).
+int grouped_gemv(int type, MatSrc src, int mats, int rows, int cols, const wd_moe_scratch *s, const int8_t *q0,
+                 const uint16_t *d0, int act_stride, float *out, int32_t *partials, hipStream_t st) {
+    const dim3 grid((rows + 15) / 16, mats);
+    const int ppr = partials_per_row(type, cols);
+    const bool part = partials != nullptr;
+    switch (type) {
+        case WD_TYPE_IQ3_S: launch_iq<21>(part, grid, st, src, rows, cols, s->xk_qs, s->xk_d, out, partials, ppr); break;
+        case WD_TYPE_IQ2_S: launch_iq<22>(part, grid, st, src, rows, cols, s->xk_qs, s->xk_d, out, partials, ppr); break;
+        case WD_TYPE_Q8_0: launch_q8<0>(part, grid, st, src, rows, cols, q0, d0, act_stride, out, partials, ppr); break;
+        case WD_TYPE_IQ4_NL: launch_q8<1>(part, grid, st, src, rows, cols, q0, d0, act_stride, out, partials, ppr); break;
+        default: return fail(WD_ERR_UNSUPPORTED, "grouped GEMV: unsupported type %d", type);
+    }
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+}  // namespace
+
+extern "C" int wd_moe_layer_f32(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s,
+                                unsigned flags, void *stream) {
+    if (const int rc = check_layer(L, s)) return rc;
+    WD_REQUIRE(d_x && d_out, "MoE layer: null activation or output pointer");
+    hipStream_t st = as_stream(stream);
+    const int H = L->hidden, F = L->expert_ffn, E = L->n_experts, k = L->top_k;
+    const bool shared = L->shared_gate_inp != nullptr;
+    const bool pre = (flags & WD_MOE_PRESELECTED) != 0;
+
+    // 1. router logits (+ the shared expert's gate logit as one more row), softmax/top-k, sigmoid
+    if (!pre) {
+        k_router_gemv<<<dim3((E + (shared ? 1 : 0) + 7) / 8), dim3(256), 0, st>>>(
+            L->router, d_x, s->logits, E, H, shared ? L->shared_gate_inp : nullptr, s->shared_gate);
+        WD_LAUNCH_CHECK();
+        if (E % 8 != 0 || E > 1024) return fail(WD_ERR_UNSUPPORTED, "router: n_experts %d must be a multiple of 8 <= 1024", E);
+        k_topk_softmax<<<dim3(1), dim3(64), 0, st>>>(s->logits, E, k, L->expert_scale, s->ids, s->weights,
+                                                     shared ? s->shared_gate : nullptr);
+        WD_LAUNCH_CHECK();
+    } else if (shared) {
+        k_router_gemv<<<dim3(1), dim3(256), 0, st>>>(L->router, d_x, s->logits, 0, H, L->shared_gate_inp, s->shared_gate);
+        WD_LAUNCH_CHECK();
+        k_sigmoid1<<<dim3(1), dim3(64), 0, st>>>(s->shared_gate);
+        WD_LAUNCH_CHECK();
+    }
+
+    // 2. quantise the layer input for the consumers that need it
+    if (consumes_q8k(L->gate_type)) {
+        k_q8_k_quantize<<<dim3((H / 256 + 3) / 4), dim3(256), 0, st>>>(d_x, H / 256, s->xk_qs, s->xk_d, s->xk_bs);
+        WD_LAUNCH_CHECK();
+    }
+    if (!consumes_q8k(L->gate_type) || shared) {
+        k_q8_0_quantize<<<dim3((H / 32 + 31) / 32), dim3(256), 0, st>>>(d_x, H / 32, s->x0_qs, s->x0_d);
+        WD_LAUNCH_CHECK();
+    }
+
+    // 3. gate/up of the k selected experts in one dispatch (2k matrices), then the shared expert's
+    const bool part = s->gup != nullptr && s->gup_type == L->gate_type && s->dp_type == L->down_type;
+    if (const int rc = grouped_gemv(L->gate_type, routed_src(L, s->ids, false), 2 * k, F, H, s, s->x0_qs, s->x0_d, 0,
+                                    s->gate_up, part ? s->gup : nullptr, st))
+        return rc;
+    if (shared) {
+        MatSrc g{}, u{};
+        g.single = L->shared_gate, u.single = L->shared_up;
+        float *gu = s->gate_up + static_cast<size_t>(2) * k * F;
+        if (const int rc = grouped_gemv(WD_TYPE_Q8_0, g, 1, F, H, s, s->x0_qs, s->x0_d, 0, gu, nullptr, st)) return rc;
+        if (const int rc = grouped_gemv(WD_TYPE_Q8_0, u, 1, F, H, s, s->x0_qs, s->x0_d, 0, gu + F, nullptr, st)) return rc;
+    }
+
+    // 4. SwiGLU in f32, 5. Q8_0 re-quantisation, for k (+1) experts at once
+    const int n_act = k + (shared ? 1 : 0);
+    k_silu_mul_experts<<<dim3((F + 255) / 256, n_act), dim3(256), 0, st>>>(s->gate_up, s->act, F);
+    WD_LAUNCH_CHECK();
+    k_q8_0_quantize<<<dim3((n_act * F / 32 + 31) / 32), dim3(256), 0, st>>>(s->act, n_act * F / 32, s->act_qs, s->act_d);
+    WD_LAUNCH_CHECK();
+
+    // 6. down projections: k routed matrices with their own activations, then the shared expert
+    if (const int rc = grouped_gemv(L->down_type, routed_src(L, s->ids, true), k, H, F, s, s->act_qs, s->act_d, F,
+                                    s->expert_out, part ? s->dp : nullptr, st))
+        return rc;
+    if (shared) {
+        MatSrc d{};
+        d.single = L->shared_down;
+        if (const int rc = grouped_gemv(WD_TYPE_Q8_0, d, 1, H, F, s, s->act_qs + static_cast<size_t>(k) * F,
+                                        s->act_d + static_cast<size_t>(k) * (F / 32), 0, s->down_f32, nullptr, st))
+            return rc;
+    }
+
+    // 7. ordered weighted sum and the shared branch
+    k_combine<<<dim3((H + 255) / 256), dim3(256), 0, st>>>(s->expert_out, s->weights, k, shared ? s->down_f32 : nullptr,
+                                                            s->shared_gate, s->accum, d_out, H);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}

@@ -1,0 +1,3 @@
+// Single translation unit of libwarpdecode_amd.so.
+#include "wd_ops.hip"
+#include "wd_layer.hip"

@@ -1,0 +1,268 @@
+// Stand-alone operators of the MoE decode path: activation quantisers, router GEMV,
+// softmax/top-k, low-bit GEMVs (one matrix or one dispatch over several expert matrices)
+// and the elementwise stages.  Each extern "C" entry point mirrors one launcher of the
+// reference operator surface (see include/warpdecode_amd.h for the citations).
+#include "wd_common.h"
+#include "wd_kernels.cuh"
+
+namespace wd {
+
+thread_local std::string g_last_error;
+std::string &last_error_slot() { return g_last_error; }
+
+int fail(int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+}  // namespace wd
+
+using namespace wd;
+
+extern "C" {
+
+const char *wd_last_error(void) { return last_error_slot().c_str(); }
+
+int wd_init(int device) {
+    int count = 0;
+    WD_HIP(hipGetDeviceCount(&count));
+    WD_REQUIRE(device >= 0 && device < count, "wd_init: device %d out of range (%d devices)", device, count);
+    WD_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    WD_HIP(hipGetDeviceProperties(&prop, device));
+    WD_REQUIRE(prop.warpSize == 64, "wd_init: device %s has %d-wide waves; this library is built for gfx950",
+               prop.name, prop.warpSize);
+    return WD_OK;
+}
+
+size_t wd_row_bytes(int type, int cols) { return row_bytes(type, cols); }
+size_t wd_tensor_bytes(int type, int rows, int cols) {
+    return rows > 0 ? static_cast<size_t>(rows) * row_bytes(type, cols) : 0;
+}
+
+// ---- runtime helpers ------------------------------------------------------------------
+int wd_malloc(void **d_ptr, size_t bytes) {
+    WD_REQUIRE(d_ptr != nullptr, "wd_malloc: null output pointer");
+    WD_HIP(hipMalloc(d_ptr, bytes));
+    return WD_OK;
+}
+int wd_free(void *d_ptr) {
+    WD_HIP(hipFree(d_ptr));
+    return WD_OK;
+}
+int wd_malloc_host(void **h_ptr, size_t bytes) {
+    WD_REQUIRE(h_ptr != nullptr, "wd_malloc_host: null output pointer");
+    WD_HIP(hipHostMalloc(h_ptr, bytes, hipHostMallocDefault));
+    return WD_OK;
+}
+int wd_free_host(void *h_ptr) {
+    WD_HIP(hipHostFree(h_ptr));
+    return WD_OK;
+}
+int wd_memcpy_h2d(void *d_dst, const void *h_src, size_t bytes, void *stream) {
+    if (stream)
+        WD_HIP(hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+    else
+        WD_HIP(hipMemcpy(d_dst, h_src, bytes, hipMemcpyHostToDevice));
+    return WD_OK;
+}
+int wd_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream) {
+    if (stream)
+        WD_HIP(hipMemcpyAsync(h_dst, d_src, bytes, hipMemcpyDeviceToHost, as_stream(stream)));
+    else
+        WD_HIP(hipMemcpy(h_dst, d_src, bytes, hipMemcpyDeviceToHost));
+    return WD_OK;
+}
+int wd_memset(void *d_dst, int value, size_t bytes, void *stream) {
+    WD_REQUIRE(bytes % 4 == 0, "wd_memset: size must be a multiple of 4 bytes");
+    const uint32_t b = static_cast<uint32_t>(value) & 0xffu;
+    const size_t n = bytes / 4;
+    if (n == 0) return WD_OK;
+    // a fill kernel rather than hipMemsetAsync, so the call may sit inside a captured graph
+    k_fill_u32<<<dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, as_stream(stream)>>>(
+        static_cast<uint32_t *>(d_dst), b * 0x01010101u, n);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+int wd_stream_create(void **stream) {
+    WD_REQUIRE(stream != nullptr, "wd_stream_create: null output pointer");
+    hipStream_t s;
+    WD_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream = s;
+    return WD_OK;
+}
+int wd_stream_destroy(void *stream) {
+    WD_HIP(hipStreamDestroy(as_stream(stream)));
+    return WD_OK;
+}
+int wd_stream_sync(void *stream) {
+    WD_HIP(hipStreamSynchronize(as_stream(stream)));
+    return WD_OK;
+}
+int wd_device_sync(void) {
+    WD_HIP(hipDeviceSynchronize());
+    return WD_OK;
+}
+
+// ---- quantisers -------------------------------------------------------------------------
+int wd_q8_k_quantize_f32(const float *d_x, int elements, int8_t *d_qs, float *d_scales, int16_t *d_bsums,
+                         void *stream) {
+    WD_REQUIRE(elements > 0 && elements % 256 == 0,
+               "Q8_K quantisation requires a positive multiple of 256 elements (got %d)", elements);
+    WD_REQUIRE(d_x && d_qs && d_scales && d_bsums, "wd_q8_k_quantize_f32: null pointer");
+    const int blocks = elements / 256;
+    k_q8_k_quantize<<<dim3((blocks + 3) / 4), dim3(256), 0, as_stream(stream)>>>(d_x, blocks, d_qs, d_scales, d_bsums);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+int wd_q8_0_quantize_f32(const float *d_x, int elements, int8_t *d_qs, uint16_t *d_scales, void *stream) {
+    WD_REQUIRE(elements > 0 && elements % 32 == 0,
+               "Q8_0 quantisation requires a positive multiple of 32 elements (got %d)", elements);
+    WD_REQUIRE(d_x && d_qs && d_scales, "wd_q8_0_quantize_f32: null pointer");
+    const int blocks = elements / 32;
+    k_q8_0_quantize<<<dim3((blocks + 31) / 32), dim3(256), 0, as_stream(stream)>>>(d_x, blocks, d_qs, d_scales);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+// ---- router -------------------------------------------------------------------------------
+int wd_router_gemv_f32(const float *d_w, const float *d_x, float *d_logits, int rows, int cols, void *stream) {
+    WD_REQUIRE(rows > 0 && cols > 0, "router GEMV: invalid shape %d x %d", rows, cols);
+    WD_REQUIRE(d_w && d_x && d_logits, "wd_router_gemv_f32: null pointer");
+    k_router_gemv<<<dim3((rows + 7) / 8), dim3(256), 0, as_stream(stream)>>>(d_w, d_x, d_logits, rows, cols, nullptr,
+                                                                             nullptr);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+int wd_topk_softmax(const float *d_logits, int n_experts, int k, float expert_scale, int32_t *d_ids,
+                    float *d_weights, void *stream) {
+    WD_REQUIRE(n_experts > 0 && n_experts <= 1024 && n_experts % 8 == 0,
+               "top-k softmax: n_experts must be a multiple of 8 in (0, 1024] (got %d)", n_experts);
+    WD_REQUIRE(k > 0 && k <= 16 && k <= n_experts, "top-k softmax: k must be in (0, 16] (got %d)", k);
+    WD_REQUIRE(d_logits && d_ids && d_weights, "wd_topk_softmax: null pointer");
+    k_topk_softmax<<<dim3(1), dim3(64), 0, as_stream(stream)>>>(d_logits, n_experts, k, expert_scale, d_ids, d_weights,
+                                                                nullptr);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+// ---- GEMVs --------------------------------------------------------------------------------
+static int launch_gemv_q8k(int type, MatSrc src, int mats, int rows, int cols, const int8_t *qs, const float *d,
+                           float *out, int32_t *partials, hipStream_t stream) {
+    WD_REQUIRE(type == WD_TYPE_IQ3_S || type == WD_TYPE_IQ2_S, "Q8_K-activation GEMV supports IQ3_S and IQ2_S (type %d)",
+               type);
+    WD_REQUIRE(rows > 0 && cols > 0 && cols % 256 == 0, "invalid low-bit matrix shape %d x %d", rows, cols);
+    WD_REQUIRE(mats > 0 && mats <= 64, "expert batch must be in (0, 64] (got %d)", mats);
+    WD_REQUIRE(qs && d && out, "low-bit GEMV: null pointer");
+    const dim3 grid((rows + 15) / 16, mats), block(256);
+    const int ppr = partials_per_row(type, cols);
+    if (type == WD_TYPE_IQ3_S) {
+        if (partials)
+            k_gemv_iq<21, true><<<grid, block, 0, stream>>>(src, rows, cols, qs, d, out, partials, ppr);
+        else
+            k_gemv_iq<21, false><<<grid, block, 0, stream>>>(src, rows, cols, qs, d, out, nullptr, 0);
+    } else {
+        if (partials)
+            k_gemv_iq<22, true><<<grid, block, 0, stream>>>(src, rows, cols, qs, d, out, partials, ppr);
+        else
+            k_gemv_iq<22, false><<<grid, block, 0, stream>>>(src, rows, cols, qs, d, out, nullptr, 0);
+    }
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+static int launch_gemv_q8_0(int type, MatSrc src, int mats, int rows, int cols, const int8_t *qs, const uint16_t *d,
+                            int act_per_mat, float *out, int32_t *partials, hipStream_t stream) {
+    WD_REQUIRE(type == WD_TYPE_Q8_0 || type == WD_TYPE_IQ4_NL || type == WD_TYPE_Q4_0,
+               "Q8_0-activation GEMV supports Q8_0, IQ4_NL and Q4_0 (type %d)", type);
+    WD_REQUIRE(rows > 0 && cols > 0 && cols % 32 == 0, "invalid low-bit matrix shape %d x %d", rows, cols);
+    WD_REQUIRE(mats > 0 && mats <= 64, "expert batch must be in (0, 64] (got %d)", mats);
+    WD_REQUIRE(qs && d && out, "low-bit GEMV: null pointer");
+    const dim3 grid((rows + 15) / 16, mats), block(256);
+    const int ppr = partials_per_row(type, cols);
+    const int act_stride = act_per_mat ? cols : 0;
+#define WD_Q8_LAUNCH(KIND)                                                                                          \
+    do {                                                                                                            \
+        if (partials)                                                                                               \
+            k_gemv_q8<KIND, true><<<grid, block, 0, stream>>>(src, rows, cols, qs, d, act_stride, out, partials, ppr); \
+        else                                                                                                        \
+            k_gemv_q8<KIND, false><<<grid, block, 0, stream>>>(src, rows, cols, qs, d, act_stride, out, nullptr, 0); \
+    } while (0)
+    if (type == WD_TYPE_Q8_0)
+        WD_Q8_LAUNCH(0);
+    else if (type == WD_TYPE_IQ4_NL)
+        WD_Q8_LAUNCH(1);
+    else
+        WD_Q8_LAUNCH(2);
+#undef WD_Q8_LAUNCH
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+int wd_gemv_q8_k_f32(int type, const uint8_t *d_w, int rows, int cols, const int8_t *d_act_qs,
+                     const float *d_act_scales, float *d_out, int32_t *d_partials, void *stream) {
+    WD_REQUIRE(d_w != nullptr, "low-bit GEMV: null weight pointer");
+    MatSrc src{};
+    src.single = d_w;
+    return launch_gemv_q8k(type, src, 1, rows, cols, d_act_qs, d_act_scales, d_out, d_partials, as_stream(stream));
+}
+
+int wd_gemv_q8_0_f32(int type, const uint8_t *d_w, int rows, int cols, const int8_t *d_act_qs,
+                     const uint16_t *d_act_scales, float *d_out, int32_t *d_partials, void *stream) {
+    WD_REQUIRE(d_w != nullptr, "low-bit GEMV: null weight pointer");
+    MatSrc src{};
+    src.single = d_w;
+    return launch_gemv_q8_0(type, src, 1, rows, cols, d_act_qs, d_act_scales, 0, d_out, d_partials, as_stream(stream));
+}
+
+int wd_gemv_q8_k_experts_f32(int type, const uint8_t *const *d_w_experts, int experts, int rows, int cols,
+                             const int8_t *d_act_qs, const float *d_act_scales, float *d_out,
+                             int32_t *d_partials, void *stream) {
+    WD_REQUIRE(d_w_experts != nullptr, "expert GEMV: null pointer table");
+    MatSrc src{};
+    src.table = d_w_experts;
+    return launch_gemv_q8k(type, src, experts, rows, cols, d_act_qs, d_act_scales, d_out, d_partials,
+                           as_stream(stream));
+}
+
+int wd_gemv_q8_0_experts_f32(int type, const uint8_t *const *d_w_experts, int experts, int rows, int cols,
+                             const int8_t *d_act_qs, const uint16_t *d_act_scales, float *d_out,
+                             int32_t *d_partials, void *stream) {
+    WD_REQUIRE(d_w_experts != nullptr, "expert GEMV: null pointer table");
+    MatSrc src{};
+    src.table = d_w_experts;
+    return launch_gemv_q8_0(type, src, experts, rows, cols, d_act_qs, d_act_scales, 1, d_out, d_partials,
+                            as_stream(stream));
+}
+
+// ---- elementwise ------------------------------------------------------------------------------
+int wd_silu_mul_experts_f32(const float *d_gate_up, float *d_act, int ffn, int experts, void *stream) {
+    WD_REQUIRE(ffn > 0 && experts > 0 && d_gate_up && d_act, "silu*up: invalid arguments");
+    k_silu_mul_experts<<<dim3((ffn + 255) / 256, experts), dim3(256), 0, as_stream(stream)>>>(d_gate_up, d_act, ffn);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+int wd_weighted_accum_experts_f32(const float *d_experts, const float *d_weights, float *d_accum, int n, int k,
+                                  void *stream) {
+    WD_REQUIRE(n > 0 && k > 0 && d_experts && d_weights && d_accum, "weighted accumulate: invalid arguments");
+    k_weighted_accum<<<dim3((n + 255) / 256), dim3(256), 0, as_stream(stream)>>>(d_experts, d_weights, d_accum, n, k);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+int wd_add_shared_f32(float *d_routed, const float *d_shared, const float *d_gate, int n, void *stream) {
+    WD_REQUIRE(n > 0 && d_routed && d_shared && d_gate, "add shared: invalid arguments");
+    k_add_shared<<<dim3((n + 255) / 256), dim3(256), 0, as_stream(stream)>>>(d_routed, d_shared, d_gate, d_routed, n);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+}  // extern "C"
