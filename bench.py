@@ -1,0 +1,259 @@
+#!/usr/bin/env python3
+"""Benchmark of the batch=1 MoE decode hot path on one MI355X.
+
+Workload (BASELINE.json configs[3], mode A): a stack of 48 MoE layers (hidden 2048, 512 experts,
+top-10, ffn 512, IQ3_S gate/up, Q8_0 down, Q8_0 shared expert gated by sigmoid(w.x), f32 router),
+all 24,576 experts resident in HBM, one token per step.  Per layer the router runs and its weights
+are used; the expert ids are replayed from a seeded Zipf(1.1) trace, as the workload prescribes.
+One "step" = one token through the 48 layers.  Weights are synthetic (random GGUF block bytes with
+the prescribed scale distributions) and are generated on the device before the timed region.
+
+Prints ONE JSON line (see the keys at the bottom).  `value` is tokens/s with everything resident
+in HBM; `roofline` prices the dominant kernel against the 8 TB/s HBM peak; `cpu_baseline` times the
+reference's CPU MoE path (oracle/_ref when built, else the C port) on a bounded sample.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+STACK_FLAGS = int(os.environ.get("WD_BENCH_FLAGS", "0"))   # experiments only (e.g. 4 = staged dispatches)
+RESIDUAL_SCALE = 2.0 ** -12   # glue between layers: x += scale * layer(x), keeps the chain finite
+
+
+def note(msg):
+    print("[bench %.1fs] %s" % (time.perf_counter() - T0, msg), file=sys.stderr, flush=True)
+
+
+T0 = time.perf_counter()
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=48)
+    ap.add_argument("--experts", type=int, default=512)
+    ap.add_argument("--routing", choices=["zipf", "router"], default="zipf",
+                    help="zipf: ids replayed from the Zipf(1.1) trace; router: ids chosen by the router itself")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a captured HIP graph")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--check", action="store_true", help="verify one layer pass against the CPU oracle first")
+    return ap.parse_args()
+
+
+def build_stack(torch, synth, capi, n_layers, n_experts, seed):
+    """Random GGUF-layout weights for n_layers C2 layers, generated on the device."""
+    H, F, k = 2048, 512, 10
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    rb_iq3, rb_q8h, rb_q8f = synth.row_bytes(synth.IQ3_S, H), synth.row_bytes(synth.Q8_0, H), synth.row_bytes(synth.Q8_0, F)
+
+    def iq3(rows):
+        t = torch.randint(0, 256, (rows * rb_iq3,), dtype=torch.uint8, device="cuda", generator=g)
+        d = (torch.randn(rows * (H // 256), device="cuda", generator=g).abs() * 0.01).half()
+        t.view(-1, 110)[:, 0:2] = d.view(torch.uint8).view(-1, 2)
+        return t
+
+    def q8(rows, cols):
+        nb = rows * (cols // 32)
+        t = torch.randint(-127, 128, (nb * 34,), dtype=torch.int8, device="cuda", generator=g).view(torch.uint8)
+        d = (torch.randn(nb, device="cuda", generator=g).abs() * (0.02 / 127.0)).half()
+        t.view(-1, 34)[:, 0:2] = d.view(torch.uint8).view(-1, 2)
+        return t
+
+    layers, keep = (capi.MoeLayer * n_layers)(), []
+    for l in range(n_layers):
+        t = dict(router=torch.randn(n_experts, H, device="cuda", generator=g) * (1.0 / np.sqrt(H)),
+                 gate=iq3(n_experts * F), up=iq3(n_experts * F), down=q8(n_experts * H, F),
+                 shared_gate_inp=torch.randn(H, device="cuda", generator=g) * 0.02,
+                 shared_gate=q8(F, H), shared_up=q8(F, H), shared_down=q8(H, F))
+        keep.append(t)
+        d = layers[l]
+        d.hidden, d.expert_ffn, d.n_experts, d.top_k, d.expert_scale = H, F, n_experts, k, 1.0
+        d.gate_type = d.up_type = synth.IQ3_S
+        d.down_type = synth.Q8_0
+        for name, tensor in t.items():
+            setattr(d, name, tensor.data_ptr())
+        d.gate_stride = d.up_stride = F * rb_iq3
+        d.down_stride = H * rb_q8f
+    return layers, keep
+
+
+def layer_dict(torch, synth, t, n_experts):
+    """Host copy of one device layer in the dict form the CPU checker takes."""
+    L = dict(hidden=2048, expert_ffn=512, n_experts=n_experts, top_k=10, w_scale=1.0, gate_type=synth.IQ3_S,
+             up_type=synth.IQ3_S, down_type=synth.Q8_0, shared_type=synth.Q8_0)
+    for name, tensor in t.items():
+        a = tensor.cpu().numpy()
+        L[name] = a.reshape(n_experts, -1) if name in ("gate", "up", "down") else a
+    return L
+
+
+def cpu_baseline(torch, synth, keep, n_experts, trace, xs, seconds):
+    """Times the reference CPU MoE path (routed experts through its own run_layer and thread pool, the
+    shared expert through its Q8_0 row kernels, router through the C port) on layer passes that rotate
+    over up to four layers' weights, until `seconds` have elapsed."""
+    from oracle import pyoracle
+    n_host = min(4, len(keep))
+    host_layers = [layer_dict(torch, synth, keep[l], n_experts) for l in range(n_host)]
+    note("cpu baseline: %d layers copied to the host" % n_host)
+    cores = os.cpu_count() or 1
+    threads = min(cores, 16)
+    use_ref = pyoracle.ref() is not None
+    passes, t0 = 0, time.perf_counter()
+    x = xs[0].copy()
+    while True:
+        L = host_layers[passes % n_host]
+        ids = trace[0, passes % trace.shape[1]]
+        if use_ref:
+            logits = pyoracle.router_logits(L["router"], x)
+            _, wts = pyoracle.route(logits, 10)
+            out = pyoracle.ref_run_layer(L, x, ids, wts, threads=threads)
+            sh = pyoracle.ref_q8_0_chain(L["shared_gate"], L["shared_up"], L["shared_down"], 2048, 512, x)
+            gate = pyoracle.sigmoid_ggml(pyoracle.dot_f32(L["shared_gate_inp"], x))
+            out = (out + (sh * gate).astype(np.float32)).astype(np.float32)
+        else:
+            logits = pyoracle.router_logits(L["router"], x)
+            _, wts = pyoracle.route(logits, 10)
+            out, _ = pyoracle.moe_layer(L, x, ids=ids, weights=wts, threads=threads)
+        passes += 1
+        dt = time.perf_counter() - t0
+        if dt >= seconds and passes >= 8:
+            break
+    per_layer = dt / passes
+    return dict(value=1.0 / (per_layer * 48), unit="tok/s", cores=threads,
+                kind="reference" if use_ref else "port",
+                sample="%d C2 layer passes in %.1f s rotating over %d layers' weights (%.2f ms/layer), "
+                       "x48 layers per token; host has %d logical cores" % (passes, dt, n_host, per_layer * 1e3, cores))
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the MoE decode hot path of the "
+              "reference is single-GPU); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from warpdecode_amd import capi, synth
+
+    torch.cuda.set_device(0)
+    capi.call("wd_init", 0)
+    H, F, k, E, NL = 2048, 512, 10, args.experts, args.layers
+    note("generating %d layers x %d experts on the device" % (NL, E))
+    layers, keep = build_stack(torch, synth, capi, NL, E, synth.BASE_SEED)
+    torch.cuda.synchronize()
+    note("weights ready (%.1f GB allocated)" % (torch.cuda.memory_allocated() / 1e9))
+    scratch = C.c_void_p()
+    capi.call("wd_moe_scratch_create", C.byref(scratch), H, F, E, k)
+
+    total_steps = args.warmup + args.steps
+    rng = synth.rng_for(synth.BASE_SEED, 9001)
+    perms = [rng.permutation(E) for _ in range(NL)]
+    trace = np.stack([np.stack([synth.zipf_ids(rng, E, k, 1.1, perms[l]) for l in range(NL)])
+                      for _ in range(total_steps)]).astype(np.int32)           # [steps][layers][k]
+    xs = np.stack([synth.rms_normed(rng, H) for _ in range(total_steps)])
+    d_trace_all, d_xs = torch.from_numpy(trace).cuda(), torch.from_numpy(xs).cuda()
+    d_trace = torch.zeros((NL, k), dtype=torch.int32, device="cuda")
+    d_x = torch.zeros(H, dtype=torch.float32, device="cuda")
+    d_out = torch.zeros(H, dtype=torch.float32, device="cuda")
+    trace_ptr = C.c_void_p(d_trace.data_ptr()) if args.routing == "zipf" else None
+
+    def launch_stack():
+        capi.call("wd_moe_stack_f32", layers, NL, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()), scratch,
+                  trace_ptr, RESIDUAL_SCALE, STACK_FLAGS, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+    if args.check:
+        from oracle import pyoracle
+        L0 = layer_dict(torch, synth, keep[0], E)
+        want, _ = pyoracle.moe_layer(L0, xs[0])
+        o = torch.zeros(H, dtype=torch.float32, device="cuda")
+        capi.call("wd_moe_layer_f32", C.byref(layers[0]), C.c_void_p(d_xs[0].data_ptr()), C.c_void_p(o.data_ptr()),
+                  scratch, 0, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        same = np.array_equal(o.cpu().numpy().view(np.uint32), want.view(np.uint32))
+        print("check: layer 0 output bit-identical to the CPU oracle: %s" % same, file=sys.stderr)
+        if not same:
+            sys.exit(1)
+
+    note("inputs and routing trace ready")
+    graph = None
+    if not args.no_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            launch_stack()                       # warm the launch path outside capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            launch_stack()
+
+    note("launch mode: %s" % ("eager" if graph is None else "hip-graph replay"))
+
+    def step(i):
+        d_x.copy_(d_xs[i], non_blocking=True)
+        d_trace.copy_(d_trace_all[i], non_blocking=True)
+        if graph is not None:
+            graph.replay()
+        else:
+            launch_stack()
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    note("warm-up done, timing %d steps" % args.steps)
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for i in range(args.steps):
+        step(args.warmup + i)
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = ev0.elapsed_time(ev1) / args.steps
+    tok_s = 1000.0 / ms_per_step
+    finite = bool(torch.isfinite(d_x).all().item())
+    note("timed region done: %.3f ms/step" % ms_per_step)
+
+    bytes_per_layer = 27697152 if E == 512 else None
+    if bytes_per_layer is None:
+        bytes_per_layer = E * H * 4 + k * (2 * F * synth.row_bytes(synth.IQ3_S, H) + H * synth.row_bytes(synth.Q8_0, F)) \
+            + 2 * F * synth.row_bytes(synth.Q8_0, H) + H * synth.row_bytes(synth.Q8_0, F) + H * 4
+    bytes_per_step = bytes_per_layer * NL
+    achieved = bytes_per_step / (ms_per_step * 1e-3) / 1e9
+    roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None,
+                    kernel="whole step (all launches of one token), %d B algorithmic per step" % bytes_per_step)
+
+    out = {
+        "metric": "MoE layer batch=1 decode: synthetic 48-layer tok/s (achieved HBM GB/s in roofline)",
+        "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 dot products (IQ3_S/Q8_0 weights x Q8_K/Q8_0 activations), f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "C3 mode A: %d-layer stack of the 512-expert top-10 IQ3_S/Q8_0 MoE layer "
+                               "(hidden 2048, ffn 512, Q8_0 shared expert), batch=1, all experts resident in HBM"
+                               % NL,
+                   "layers": NL, "experts": E, "top_k": k, "routing": args.routing,
+                   "launch": "eager" if graph is None else "hip-graph replay",
+                   "bytes_per_token": bytes_per_step, "wall_s": round(wall, 3), "finite": finite},
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch, synth, keep, E, trace, xs, args.cpu_seconds)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

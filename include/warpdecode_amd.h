@@ -170,9 +170,15 @@ int32_t *wd_moe_scratch_down_partials(wd_moe_scratch *s);
  * layer pass fill them.  Parity harness only. */
 int wd_moe_scratch_enable_partials(wd_moe_scratch *s, int gate_type, int down_type);
 
+/* Profiling aid: makes the fused layer dispatches record 100 MHz time stamps of workgroup `wg`
+ * ([dispatch A,B,C][wave 0..15][point 0..7], uint64) and returns the device buffer (NULL on failure).
+ * Counterpart of the reference's kernel profiler sites, src/qwen38_moe.cuh:296-535. */
+unsigned long long *wd_moe_scratch_trace(wd_moe_scratch *s, int wg);
+
 /* flags for wd_moe_layer_f32 */
 #define WD_MOE_PRESELECTED 1u      /* ids/weights already in scratch: skip the router (reference `preselected`) */
 #define WD_MOE_KEEP_EXPERT_OUT 2u  /* also store the per-expert down outputs in scratch */
+#define WD_MOE_STAGED 4u           /* one dispatch per stage (the operators above) instead of the fused kernels */
 
 /* One decode step of one layer: router -> top-k -> grouped gate/up -> SwiGLU -> Q8_0 ->
  * grouped down -> ordered weighted sum -> + shared * sigmoid gate.  d_out is f32 [hidden]
@@ -182,6 +188,16 @@ int wd_moe_scratch_enable_partials(wd_moe_scratch *s, int gate_type, int down_ty
  *   run_qwen38_shared_expert_f32_x (:3963-3969) + q38_finish_moe_f32 (:2442-2453). */
 int wd_moe_layer_f32(const wd_moe_layer *layer, const float *d_x, float *d_out, wd_moe_scratch *scratch,
                      unsigned flags, void *stream);
+
+/* One decode step through a stack of layers: for each layer, x += residual_scale * layer(x) (the scaled
+ * residual add stands in for the caller's own glue between two MoE blocks).  d_layer_out f32 [hidden] receives the last
+ * layer's output.  d_ids_trace (device int32 [n_layers][top_k], may be NULL) replays a routing trace:
+ * the router still runs and its weights are used, but the expert ids come from the trace.
+ * `layers` is a host array.  No counterpart in the reference, whose caller loops over layers
+ * (Qwen38Decoder::step, src/qwen38_forward.cuh:2923-3371). */
+int wd_moe_stack_f32(const wd_moe_layer *layers, int n_layers, float *d_x, float *d_layer_out,
+                     wd_moe_scratch *scratch, const int32_t *d_ids_trace, float residual_scale, unsigned flags,
+                     void *stream);
 
 /* M tokens through one layer; the weights of an expert selected by several tokens are read once.
  * d_x f32 [tokens][hidden], d_out f32 [tokens][hidden].  Bit-identical to `tokens` calls of

@@ -51,7 +51,20 @@ def run_layer(g, L, x, partials=True, flags=0, ids=None, weights=None):
 
 
 def check_layer(g, oracle, L, x, **kw):
+    """Staged pass (one dispatch per operator, int32 chunk sums exported) and fused pass (three
+    dispatches) against the oracle."""
     want, d = oracle.moe_layer(L, x, ids=kw.get("ids"), weights=kw.get("weights"), want_partials=True)
+    fused = run_layer(g, L, x, partials=False, **kw)
+    assert np.array_equal(fused["ids"], d["ids"])
+    assert g.same_bits(fused["weights"], d["weights"])
+    if kw.get("ids") is None:
+        assert g.same_bits(fused["logits"], d["logits"])
+    assert g.same_bits(fused["act"], d["act"])
+    assert g.same_bits(fused["accum"], d["routed"])
+    if L.get("shared_gate_inp") is not None:
+        assert g.same_bits(fused["shared_gate"], d["shared_gate"])
+        assert g.same_bits(fused["down_f32"], d["shared_out"])
+    assert g.same_bits(fused["out"], want)
     got = run_layer(g, L, x, **kw)
     assert np.array_equal(got["ids"], d["ids"])
     assert g.same_bits(got["weights"], d["weights"])

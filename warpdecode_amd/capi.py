@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(HERE, "libwarpdecode_amd.so")
 HEADER = os.path.join(os.path.dirname(HERE), "include", "warpdecode_amd.h")
 
 F32, F16, Q4_0, Q8_0, IQ4_NL, IQ3_S, IQ2_S = 0, 1, 2, 8, 20, 21, 22
-MOE_PRESELECTED, MOE_KEEP_EXPERT_OUT = 1, 2
+MOE_PRESELECTED, MOE_KEEP_EXPERT_OUT, MOE_STAGED = 1, 2, 4
 
 vp, i32, f32, sz, u32 = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint
 
@@ -71,7 +71,9 @@ _SIGS = {
     "wd_moe_scratch_create": (i32, [C.POINTER(vp), i32, i32, i32, i32]),
     "wd_moe_scratch_destroy": (i32, [vp]),
     "wd_moe_scratch_enable_partials": (i32, [vp, i32, i32]),
+    "wd_moe_scratch_trace": (vp, [vp, i32]),
     "wd_moe_layer_f32": (i32, [C.POINTER(MoeLayer), vp, vp, vp, u32, vp]),
+    "wd_moe_stack_f32": (i32, [C.POINTER(MoeLayer), i32, vp, vp, vp, vp, f32, u32, vp]),
 }
 for _n in ("logits", "ids", "weights", "gate_up", "act", "act_qs", "act_scales", "expert_out", "accum", "down_f32",
            "shared_gate", "gate_up_partials", "down_partials"):

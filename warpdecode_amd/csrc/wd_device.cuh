@@ -74,9 +74,63 @@ WD_DEV int sdot4(uint32_t a, uint32_t b, int acc) {
     return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), acc, false);
 }
 
-// ---- cross-lane -----------------------------------------------------------------
+// ---- cross-lane -----------------------------------------------------------------------
+// Data-parallel-primitive (DPP) moves work inside rows of 16 lanes without touching LDS:
+//   quad_perm 0xB1 / 0x4E   lane ^ 1 / lane ^ 2
+//   row_ror:8               lane ^ 8;     row_ror:4   lane i reads lane (i - 4) mod 16 of its row
+//   row_shr:n / row_shl:n   lane i reads lane i - n / i + n of its row (no source: keeps `old`,
+//                           or 0 with bound_ctrl)
+//   row_bcast15 / 31        rows 1,3 read lane 15 / 47; rows 2,3 read lane 31 (row_mask selects)
+// Halves and row pairs are exchanged with v_permlane32_swap / v_permlane16_swap (gfx950).
 WD_DEV int lane_id() { return static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u))); }
 
+template <int CTRL, int ROW_MASK = 0xf, int BANK_MASK = 0xf, bool BOUND = false>
+WD_DEV int dpp_i(int old, int v) {
+    return __builtin_amdgcn_update_dpp(old, v, CTRL, ROW_MASK, BANK_MASK, BOUND);
+}
+template <int CTRL, int ROW_MASK = 0xf, int BANK_MASK = 0xf, bool BOUND = false>
+WD_DEV float dpp_f(float old, float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, v),
+                                                                CTRL, ROW_MASK, BANK_MASK, BOUND));
+}
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppRor4 = 0x124, kDppRor8 = 0x128, kDppBcast15 = 0x142,
+              kDppBcast31 = 0x143;
+constexpr int kDppShr1 = 0x111, kDppShl1 = 0x101, kDppShl2 = 0x102, kDppShl4 = 0x104, kDppShl7 = 0x107;
+
+WD_DEV float readlane_f(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// Wave-wide reductions of order-free operations; the result is uniform.
+WD_DEV float wave_max(float v) {
+    v = __builtin_fmaxf(v, dpp_f<kDppXor1>(v, v));
+    v = __builtin_fmaxf(v, dpp_f<kDppXor2>(v, v));
+    v = __builtin_fmaxf(v, dpp_f<kDppRor4>(v, v));
+    v = __builtin_fmaxf(v, dpp_f<kDppRor8>(v, v));
+    v = __builtin_fmaxf(v, dpp_f<kDppBcast15, 0xa>(v, v));
+    v = __builtin_fmaxf(v, dpp_f<kDppBcast31, 0xc>(v, v));
+    return readlane_f(v, 63);
+}
+WD_DEV int wave_min_i(int v) {
+    v = min(v, dpp_i<kDppXor1>(v, v));
+    v = min(v, dpp_i<kDppXor2>(v, v));
+    v = min(v, dpp_i<kDppRor4>(v, v));
+    v = min(v, dpp_i<kDppRor8>(v, v));
+    v = min(v, dpp_i<kDppBcast15, 0xa>(v, v));
+    v = min(v, dpp_i<kDppBcast31, 0xc>(v, v));
+    return __builtin_amdgcn_readlane(v, 63);
+}
+// Maximum over aligned groups of four / eight lanes (every lane gets its group's value).
+WD_DEV float quad_max(float v) {
+    v = __builtin_fmaxf(v, dpp_f<kDppXor1>(v, v));
+    return __builtin_fmaxf(v, dpp_f<kDppXor2>(v, v));
+}
+WD_DEV int quad_sum_i(int v) {
+    v += dpp_i<kDppXor1>(0, v);
+    return v + dpp_i<kDppXor2>(0, v);
+}
+
+// General shuffles (LDS crossbar; slower than DPP, used off the hot paths).
 template <typename T>
 WD_DEV T lane_xor(T v, int mask) {
     return __shfl_xor(v, mask, kWave);
@@ -90,17 +144,6 @@ WD_DEV T lane_get(T v, int src) {
     return __shfl(v, src, kWave);
 }
 
-WD_DEV float wave_max(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v = __builtin_fmaxf(v, lane_xor(v, m));
-    return v;
-}
-WD_DEV int wave_min_i(int v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v = min(v, lane_xor(v, m));
-    return v;
-}
-
 // Orders this wave's LDS traffic for cross-lane hand-offs through LDS.  The hardware
 // executes a wave's LDS instructions in order; the fence keeps the compiler from moving
 // a lane's read above another lane's (earlier) write.
@@ -109,13 +152,40 @@ WD_DEV void wave_lds_fence() {
     __builtin_amdgcn_wave_barrier();
 }
 
-// Closing tree of eight chunk lanes held by eight consecutive lanes (lane & 7 = chunk):
-// ((l0+l4)+(l2+l6)) + ((l1+l5)+(l3+l7)); valid in the lane with (lane & 7) == 0.
+// Closing tree of eight chunk lanes held by lanes 0..7 of a 16-lane row (lane & 7 = chunk):
+// ((l0+l4)+(l2+l6)) + ((l1+l5)+(l3+l7)); valid in lane 0 of the row.
 WD_DEV float close_lanes8(float v) {
-    v = v + lane_down(v, 4);
-    v = v + lane_down(v, 2);
-    v = v + lane_down(v, 1);
+    v = v + dpp_f<kDppShl4>(0.0f, v);
+    v = v + dpp_f<kDppShl2>(0.0f, v);
+    v = v + dpp_f<kDppShl1>(0.0f, v);
     return v;
+}
+
+// The same tree over eight uniform-addressable values: chunk c is taken from lane 8*c + 7.
+// The result is uniform.
+WD_DEV float close_lanes8_strided(float v) {
+    const float l0 = readlane_f(v, 7), l1 = readlane_f(v, 15), l2 = readlane_f(v, 23), l3 = readlane_f(v, 31);
+    const float l4 = readlane_f(v, 39), l5 = readlane_f(v, 47), l6 = readlane_f(v, 55), l7 = readlane_f(v, 63);
+    const float a = l0 + l4, b = l1 + l5, c = l2 + l6, e = l3 + l7;
+    return (a + c) + (b + e);
+}
+
+// Unaligned loads from global memory (address space 1), so that no flat (generic) load is issued.
+typedef uint16_t __attribute__((aligned(2))) wd_u16a;
+typedef uint32_t __attribute__((aligned(2))) wd_u32a;
+typedef uint32_t wd_u64a __attribute__((ext_vector_type(2), aligned(2)));
+typedef uint32_t wd_u128a __attribute__((ext_vector_type(4), aligned(2)));
+#define WD_GLOBAL __attribute__((address_space(1)))
+WD_DEV uint32_t gld_u8(const uint8_t *p) { return *((const WD_GLOBAL uint8_t *)(p)); }
+WD_DEV uint16_t gld_u16(const uint8_t *p) { return *((const WD_GLOBAL wd_u16a *)(p)); }
+WD_DEV uint32_t gld_u32(const uint8_t *p) { return *((const WD_GLOBAL wd_u32a *)(p)); }
+WD_DEV uint2 gld_u64(const uint8_t *p) {
+    const wd_u64a v = *((const WD_GLOBAL wd_u64a *)(p));
+    return make_uint2(v.x, v.y);
+}
+WD_DEV uint4 gld_u128(const uint8_t *p) {
+    const wd_u128a v = *((const WD_GLOBAL wd_u128a *)(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
 }
 
 }  // namespace wd

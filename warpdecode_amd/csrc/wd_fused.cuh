@@ -1,0 +1,513 @@
+// Fused MoE layer: three dispatches per layer.
+//   A  router logits (+ shared-expert gate logit); the router workgroup that finishes last runs
+//      softmax/top-k, so the ids never leave the device and the selection overlaps the shared
+//      expert's gate/up + SwiGLU, which the remaining workgroups of the same dispatch compute
+//   B  gate/up + SwiGLU of the k selected experts
+//   C  Q8_0 re-quantisation of the k+1 activations, all down projections, the ordered weighted
+//      sum, the gated shared branch and the optional residual update
+// Activation quantisation is redone by every workgroup that needs it (8 KB of f32 from L2 and a
+// few dozen instructions per lane) instead of being a dispatch of its own, and it runs while the
+// workgroup's weight loads are already in flight.
+#pragma once
+
+#include "wd_kernels.cuh"
+
+namespace wd {
+
+struct LayerArgs {
+    int H, F, E, k;
+    float w_scale;
+    const float *x;
+    const float *router;
+    MatSrc gate_up, down;        // resolved through ids (global scratch)
+    const float *sh_inp;         // null = no shared expert
+    const uint8_t *sh_gate, *sh_up, *sh_down;
+    float *logits;               // [E]
+    int32_t *ids;                // [k]
+    float *weights;              // [k]
+    const int32_t *ids_override; // null or [k]
+    float *act;                  // [k+1][F]
+    float *shared_gate;          // [1]: logit after A, sigmoid after B
+    float *expert_out;           // null or [k][H]
+    float *accum, *down_f32, *out;
+    float *residual;             // null or [H]
+    float residual_scale;
+    int preselected;
+    int n_router_wgs;            // workgroups of dispatch A that take router rows
+    unsigned *arrive;            // device counter of finished router workgroups (zero between dispatches)
+    unsigned long long *trace;   // profiling aid: null, or [3][16][8] time stamps (100 MHz) of workgroup trace_wg
+    int trace_wg;
+};
+
+// Time stamp `i` of dispatch `d` (0 = A, 1 = B, 2 = C) for the traced workgroup; lane 0 of every wave.
+WD_DEV void mark(const LayerArgs &a, int d, int i) {
+    if (a.trace && static_cast<int>(blockIdx.x) == a.trace_wg && (threadIdx.x & 63) == 0 && (threadIdx.x >> 6) < 15)
+        a.trace[(d * 16 + (threadIdx.x >> 6)) * 8 + i] = wall_clock64();
+}
+// Row 15 of each dispatch: [0] earliest start, [1] latest end over all workgroups.
+WD_DEV void mark_span(const LayerArgs &a, int d, bool end) {
+    if (a.trace && threadIdx.x == 0) {
+        if (end)
+            atomicMax(&a.trace[(d * 16 + 15) * 8 + 1], wall_clock64());
+        else
+            atomicMin(&a.trace[(d * 16 + 15) * 8 + 0], wall_clock64());
+    }
+}
+
+// ---- in-workgroup quantisers (results in LDS) ------------------------------------------------
+// Q8_0 of n values (multiple of 32): four threads per block, eight values per thread.
+WD_DEV void lds_quantize_q8_0(const float *__restrict__ x, int n, int8_t *qs, uint16_t *d, int tid, int nthreads) {
+    const int per_pass = nthreads * 8;
+    for (int base0 = 0; base0 < n; base0 += per_pass) {
+        const int base = base0 + tid * 8;
+        const bool on = base < n;
+        float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
+        if (on) {
+            v0 = *reinterpret_cast<const float4 *>(x + base);
+            v1 = *reinterpret_cast<const float4 *>(x + base + 4);
+        }
+        float amax = __builtin_fmaxf(
+            __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v0.x), __builtin_fabsf(v0.y)),
+                            __builtin_fmaxf(__builtin_fabsf(v0.z), __builtin_fabsf(v0.w))),
+            __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v1.x), __builtin_fabsf(v1.y)),
+                            __builtin_fmaxf(__builtin_fabsf(v1.z), __builtin_fabsf(v1.w))));
+        amax = quad_max(amax);
+        if (on) {
+            uint2 packed;
+            packed.x = q8_0_pack4(v0, amax);
+            packed.y = q8_0_pack4(v1, amax);
+            *reinterpret_cast<uint2 *>(qs + base) = packed;
+            if ((tid & 3) == 0) d[base >> 5] = f2h_ref(amax / 127.0f);
+        }
+    }
+}
+
+// Q8_K of one 256-value block by one wave (four values per lane).
+WD_DEV void wave_quantize_q8_k_block(const float *__restrict__ x256, int8_t *qs256, float *d, int lane) {
+    const float4 v = reinterpret_cast<const float4 *>(x256)[lane];
+    float amax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)),
+                                 __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
+    amax = wave_max(amax);
+    uint32_t packed = 0;
+    float dv = 0.0f;
+    if (amax != 0.0f) {
+        const float iscale = -127.0f / amax;
+        const int q0 = min(127, static_cast<int>(__builtin_rintf(v.x * iscale)));
+        const int q1 = min(127, static_cast<int>(__builtin_rintf(v.y * iscale)));
+        const int q2 = min(127, static_cast<int>(__builtin_rintf(v.z * iscale)));
+        const int q3 = min(127, static_cast<int>(__builtin_rintf(v.w * iscale)));
+        packed = (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | (static_cast<uint32_t>(q3 & 0xff) << 24);
+        dv = 1.0f / iscale;
+    }
+    reinterpret_cast<uint32_t *>(qs256)[lane] = packed;
+    if (lane == 0) *d = dv;
+}
+
+// ---- softmax + top-k by one wave, probabilities kept in registers --------------------------------
+// Lane l owns the 8-expert groups l (and l + 64 when M == 2, i.e. more than 512 experts).
+// Lanes 0..k-1 write ids/weights through the given pointers (LDS or global).
+// src/qwen38_moe.cuh:711-818: softmax over all experts with the per-8 sums accumulated in a double in
+// ascending order, k rungs of "largest remaining probability, lowest index on ties", renormalise.
+// COHERENT: the logits were written by other workgroups of the same dispatch; they are read with
+// device-scope atomic loads so that no stale cached copy can be seen.
+template <int M, bool COHERENT>
+WD_DEV void topk_wave_m(const float *logits, int n, int k, float w_scale, int32_t *ids, float *weights,
+                        const int32_t *__restrict__ override_ids, int lane) {
+    const int groups = n >> 3;
+    float v[8 * M];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+        const int g = lane + 64 * m;
+        if (g < groups) {
+            if (COHERENT) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    v[8 * m + i] = __hip_atomic_load(logits + g * 8 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else {
+                const float4 a = *reinterpret_cast<const float4 *>(logits + g * 8);
+                const float4 b = *reinterpret_cast<const float4 *>(logits + g * 8 + 4);
+                v[8 * m + 0] = a.x, v[8 * m + 1] = a.y, v[8 * m + 2] = a.z, v[8 * m + 3] = a.w;
+                v[8 * m + 4] = b.x, v[8 * m + 5] = b.y, v[8 * m + 6] = b.z, v[8 * m + 7] = b.w;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[8 * m + i] = -INFINITY;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) mx = __builtin_fmaxf(mx, v[8 * m + i]);
+    }
+    mx = wave_max(mx);
+    float gs[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+        const bool on = lane + 64 * m < groups;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[8 * m + i] = on ? exp_ggml(v[8 * m + i] - mx) : 0.0f;
+        const float lo = v[8 * m + 0] + v[8 * m + 4], lh = v[8 * m + 2] + v[8 * m + 6];
+        const float hi = v[8 * m + 1] + v[8 * m + 5], hh = v[8 * m + 3] + v[8 * m + 7];
+        gs[m] = (lo + lh) + (hi + hh);
+    }
+    // group sums accumulated into a double in ascending group order (uniform arithmetic)
+    double sum = 0.0;
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+#pragma unroll
+        for (int l = 0; l < 64; ++l) {
+            const float gl = readlane_f(gs[m], l);
+            if (l + 64 * m < groups) sum += static_cast<double>(gl);
+        }
+    }
+    const bool dead = (sum == 0.0);
+    const float inv = dead ? 0.0f : static_cast<float>(1.0 / sum);
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+        const bool on = lane + 64 * m < groups;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[8 * m + i] = (on && !dead) ? v[8 * m + i] * inv : -INFINITY;
+    }
+    // For a row whose exponentials all vanished every probability is -inf, nothing ever beats the
+    // running best of -inf, and the reference keeps expert 0 with the value read back from the row.
+    float top_mine = 0.0f;  // lane j keeps the j-th selected probability
+    int id_mine = 0;
+    for (int j = 0; j < k; ++j) {
+        // this lane's largest remaining probability; lowest slot on ties
+        float bv = v[0];
+#pragma unroll
+        for (int i = 1; i < 8 * M; ++i) bv = __builtin_fmaxf(bv, v[i]);
+        int slot = 8 * M - 1;
+#pragma unroll
+        for (int i = 8 * M - 2; i >= 0; --i) slot = (v[i] == bv) ? i : slot;
+        const float best = wave_max(bv);
+        int win = 0;
+        if (best > -INFINITY) {
+            // lowest expert index among the lanes holding `best`: slots of group l come before the
+            // slots of group l + 64, and lower lanes before higher ones inside a group row
+            const bool mine = bv == best;
+            unsigned long long mask = __builtin_amdgcn_ballot_w64(mine && slot < 8);
+            if (M == 2 && mask == 0ull) mask = __builtin_amdgcn_ballot_w64(mine);
+            const int wl = __builtin_ctzll(mask);
+            const int ws = __builtin_amdgcn_readlane(slot, wl);
+            win = (wl + 64 * (ws >> 3)) * 8 + (ws & 7);
+#pragma unroll
+            for (int i = 0; i < 8 * M; ++i) v[i] = (lane == wl && ws == i) ? -INFINITY : v[i];
+        }
+        if (lane == j) {
+            top_mine = best;
+            id_mine = win;
+        }
+    }
+    // sum of the selected probabilities in selection order, in a double
+    double wsum = 0.0;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const float tj = readlane_f(top_mine, j);
+        if (j < k) wsum += static_cast<double>(tj);
+    }
+    const float denom = __builtin_fmaxf(static_cast<float>(wsum), 6.103515625e-5f);
+    if (lane < k) {
+        float wj = top_mine / denom;
+        if (w_scale != 0.0f && w_scale != 1.0f) wj = wj * w_scale;
+        weights[lane] = wj;
+        ids[lane] = override_ids ? override_ids[lane] : id_mine;
+    }
+}
+
+template <bool COHERENT>
+WD_DEV void topk_wave(const float *logits, int n, int k, float w_scale, int32_t *ids, float *weights,
+                      const int32_t *__restrict__ override_ids, int lane) {
+    if (n <= 512)
+        topk_wave_m<1, COHERENT>(logits, n, k, w_scale, ids, weights, override_ids, lane);
+    else
+        topk_wave_m<2, COHERENT>(logits, n, k, w_scale, ids, weights, override_ids, lane);
+}
+
+// Stand-alone softmax/top-k dispatch: one wave (src/qwen38_moe.cuh:711-818).
+// If gate_logit != null, gate_logit[0] is replaced by sigmoid_ggml(gate_logit[0]) (shared expert gate).
+// If override_ids != null the selected ids are replaced by override_ids[0..k) after the weights are formed.
+__global__ __launch_bounds__(64) void k_topk_softmax(const float *__restrict__ logits, int n, int k, float w_scale,
+                                                      int32_t *__restrict__ ids, float *__restrict__ weights,
+                                                      float *__restrict__ gate_logit,
+                                                      const int32_t *__restrict__ override_ids) {
+    const int lane = threadIdx.x;
+    if (gate_logit && lane == 0) gate_logit[0] = sigmoid_ggml(gate_logit[0]);
+    topk_wave<false>(logits, n, k, w_scale, ids, weights, override_ids, lane);
+}
+
+// ---- router rows: 32 lanes per row, 8 rows per 256-thread workgroup ---------------------------------
+// All loads of a 2048-column span are issued before the first multiply-add, so one HBM round trip
+// covers the span; the multiply-add chain of each accumulator still runs in ascending column order.
+// COHERENT: results are published with device-scope atomic stores (another workgroup of the same
+// dispatch reads them).
+template <bool COHERENT>
+WD_DEV void router_rows(const float *__restrict__ w, const float *__restrict__ x, float *logits, int rows, int cols,
+                        const float *__restrict__ extra_w, float *extra_out, int wg) {
+    const int t = threadIdx.x & 31;
+    const int row = wg * static_cast<int>(blockDim.x >> 5) + (threadIdx.x >> 5);
+    const int total = rows + (extra_w ? 1 : 0);
+    const bool on = row < total;
+    const float *wr = on ? (row < rows ? w + static_cast<size_t>(row) * cols : extra_w) : x;
+    const int np = cols & ~31;
+    float s = 0.0f;
+    if (on) {
+        for (int i0 = 0; i0 < np; i0 += 2048) {
+            float wv[64], xv[64];
+#pragma unroll
+            for (int u = 0; u < 64; ++u) {
+                const int i = i0 + 32 * u + t;
+                if (i0 + 32 * u < np) {
+                    wv[u] = wr[i];
+                    xv[u] = x[i];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 64; ++u)
+                if (i0 + 32 * u < np) s = __builtin_fmaf(wv[u], xv[u], s);
+        }
+    }
+    float o = __shfl_down(s, 16, 32);
+    if (t < 16) s = s + o;
+    o = __shfl_down(s, 8, 32);
+    if (t < 8) s = s + o;
+    o = __shfl_down(s, 4, 32);
+    if (t < 4) s = s + o;
+    o = __shfl_down(s, 1, 32);
+    if (t == 0 || t == 2) s = s + o;
+    o = __shfl_down(s, 2, 32);
+    float acc = s + o;
+    if (on && t == 0) {
+        for (int c = np; c < cols; ++c) acc = acc + wr[c] * x[c];
+        float *dst = (row < rows) ? logits + row : extra_out;
+        if (COHERENT)
+            __hip_atomic_store(dst, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else
+            *dst = acc;
+    }
+}
+
+// ---- dispatch A -----------------------------------------------------------------------------------------
+// grid = n_router_wgs + ceil(F / 8) (the second part only with a shared expert); 512 threads.
+// Router workgroups: 16 rows each.  Shared-expert workgroups: 8 (gate, up) row pairs, one per wave.
+// dynamic LDS: H bytes + H/32 halves for the Q8_0 copy of x.
+//
+// Hand-off to the selecting workgroup: logits are published with device-scope atomic stores, each
+// workgroup then waits for its stores to complete and bumps a counter with a relaxed device-scope
+// atomic; the workgroup that reads n_router_wgs - 1 knows every logit is complete and reads them
+// with device-scope atomic loads.  No cache-wide release/acquire is needed for 2 KB of data.
+__global__ __launch_bounds__(512) void k_layer_a(LayerArgs a) {
+    extern __shared__ __align__(16) uint8_t lds_a[];
+    __shared__ Q8RowTile tiles[8];
+    __shared__ int s_last;
+    const int wg = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    mark(a, 0, 0);
+    mark_span(a, 0, false);
+    if (wg < a.n_router_wgs) {
+        router_rows<true>(a.router, a.x, a.logits, a.preselected ? 0 : a.E, a.H, a.sh_inp, a.shared_gate, wg);
+        mark(a, 0, 1);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);  // this wave's stores have been acknowledged
+        __syncthreads();
+        if (threadIdx.x == 0)
+            s_last = (__hip_atomic_fetch_add(a.arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+                      static_cast<unsigned>(a.n_router_wgs - 1));
+        __syncthreads();
+        if (s_last && wave == 0) {
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+            if (a.trace && lane == 0) a.trace[(0 * 16 + 8) * 8 + 0] = wall_clock64();
+            if (!a.preselected) topk_wave<true>(a.logits, a.E, a.k, a.w_scale, a.ids, a.weights, a.ids_override, lane);
+            if (lane == 0) {
+                if (a.sh_inp) {
+                    const float g = __hip_atomic_load(a.shared_gate, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    a.shared_gate[0] = sigmoid_ggml(g);
+                }
+                a.arrive[0] = 0u;
+            }
+            if (a.trace && lane == 0) a.trace[(0 * 16 + 8) * 8 + 1] = wall_clock64();
+        }
+        mark(a, 0, 2);
+        mark_span(a, 0, true);
+        return;
+    }
+    int8_t *xq = reinterpret_cast<int8_t *>(lds_a);
+    uint16_t *xd = reinterpret_cast<uint16_t *>(lds_a + a.H);
+    const int r = (wg - a.n_router_wgs) * 8 + wave;
+    const int nb = a.H >> 5;
+    const size_t rb = static_cast<size_t>(nb) * 34;
+    const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
+    const uint8_t *const rows[2] = {a.sh_gate + off, a.sh_up + off};
+    float gu[2];
+    q8_row_wave<2>(rows, nb, xq, xd, tiles[wave], lane, gu, [&]() {
+        lds_quantize_q8_0(a.x, a.H, xq, xd, threadIdx.x, 512);
+        __syncthreads();
+        mark(a, 0, 2);
+    });
+    if (lane == 0 && r < a.F) a.act[static_cast<size_t>(a.k) * a.F + r] = silu_ggml(gu[0]) * gu[1];
+    mark(a, 0, 3);
+    mark_span(a, 0, true);
+}
+
+// ---- dispatch B -----------------------------------------------------------------------------------------
+// TYPE: gate/up tensor type (21 IQ3_S, 22 IQ2_S, 8 Q8_0, 20 IQ4_NL).
+// IQ types and Q8_0: 512-thread workgroups, one (gate,up) row pair per wave, grid = k * ceil(F / 8).
+// IQ4_NL: 256-thread workgroups, four row pairs per wave, grid = k * ceil(F / 16).
+// Every wave first requests its weight bytes; the workgroup then stages the codebooks and quantises x
+// while they are in flight.  dynamic LDS: quantised x (H bytes + scales).
+template <int TYPE>
+__global__ __launch_bounds__(TYPE == 20 ? 256 : 512) void k_layer_b(LayerArgs a) {
+    constexpr bool kIq = (TYPE == 21 || TYPE == 22);
+    constexpr int kThreads = (TYPE == 20) ? 256 : 512;
+    constexpr int kRowsPerWg = (TYPE == 20) ? 16 : 8;
+    extern __shared__ __align__(16) uint8_t lds_b[];
+    __shared__ IqTables tables;
+    __shared__ Q8TileN<4> tiles4[TYPE == 20 ? 4 : 1];
+    __shared__ Q8RowTile tiles1[TYPE == 8 ? 8 : 1];
+    int8_t *xq = reinterpret_cast<int8_t *>(lds_b);
+    uint8_t *xscale = lds_b + a.H;  // f32 [H/256] or f16 [H/32]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    mark(a, 1, 0);
+    mark_span(a, 1, false);
+
+    const int groups = (a.F + kRowsPerWg - 1) / kRowsPerWg;
+    const int j = blockIdx.x / groups;
+    const int rg = blockIdx.x - j * groups;
+    const int e = a.ids[j];
+    const uint8_t *gate = mat_ptr_ids(a.gate_up, 2 * j, e);
+    const uint8_t *up = mat_ptr_ids(a.gate_up, 2 * j + 1, e);
+    float *act = a.act + static_cast<size_t>(j) * a.F;
+    if (kIq) {
+        const int nb = a.H >> 8;
+        const size_t rb = static_cast<size_t>(nb) * (TYPE == 21 ? 110 : 82);
+        const int r = rg * 8 + wave;
+        const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
+        const uint8_t *const rows[2] = {gate + off, up + off};
+        float gu[2];
+        iq_rows_q8k<(kIq ? TYPE : 21), 2, false>(rows, nb, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
+                                                  nullptr, 0, [&]() {
+            stage_tables<TYPE == 21, TYPE == 22>(tables, threadIdx.x, kThreads);
+            for (int b = wave; b < (a.H >> 8); b += kThreads / 64)
+                wave_quantize_q8_k_block(a.x + b * 256, xq + b * 256, reinterpret_cast<float *>(xscale) + b, lane);
+            mark(a, 1, 1);
+            __syncthreads();
+            mark(a, 1, 2);
+        });
+        if (lane == 0 && r < a.F) act[r] = silu_ggml(gu[0]) * gu[1];
+        mark(a, 1, 3);
+    } else if (TYPE == 8) {
+        const int nb = a.H >> 5;
+        const size_t rb = static_cast<size_t>(nb) * 34;
+        const int r = rg * 8 + wave;
+        const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
+        const uint8_t *const rows[2] = {gate + off, up + off};
+        float gu[2];
+        q8_row_wave<2>(rows, nb, xq, reinterpret_cast<const uint16_t *>(xscale), tiles1[TYPE == 8 ? wave : 0], lane, gu,
+                       [&]() {
+                           lds_quantize_q8_0(a.x, a.H, xq, reinterpret_cast<uint16_t *>(xscale), threadIdx.x, kThreads);
+                           __syncthreads();
+                       });
+        if (lane == 0 && r < a.F) act[r] = silu_ggml(gu[0]) * gu[1];
+    } else {
+        const int nb = a.H >> 5;
+        const size_t rb = static_cast<size_t>(nb) * 18;
+        const int r0 = rg * 16 + wave * 4;
+        const int nrows = max(0, min(4, a.F - r0));
+        const size_t off = static_cast<size_t>(min(r0, a.F - 1)) * rb;
+        const uint8_t *const rows[2] = {gate + off, up + off};
+        float gu[2];
+        q8_rows4_multi<1, 2, 4, false>(rows, nrows, nb, xq, reinterpret_cast<const uint16_t *>(xscale),
+                                       tiles4[TYPE == 20 ? wave : 0], lane, gu, nullptr, 0, [&]() {
+                                           lds_quantize_q8_0(a.x, a.H, xq, reinterpret_cast<uint16_t *>(xscale),
+                                                             threadIdx.x, kThreads);
+                                           __syncthreads();
+                                       });
+        const int r4 = lane >> 4;
+        if ((lane & 15) == 0 && r4 < nrows) act[r0 + r4] = silu_ggml(gu[0]) * gu[1];
+    }
+    __syncthreads();
+    mark_span(a, 1, true);
+}
+
+// ---- dispatch C -----------------------------------------------------------------------------------------
+// KIND: down tensor kind (0 Q8_0, 1 IQ4_NL).  One workgroup per four output rows; wave m takes
+// matrix m (the k routed down tensors, then the shared one), so every weight byte of the four rows
+// is requested at once.  Each wave re-quantises the activation of its own matrix while its weights
+// are in flight.  The first four lanes of wave 0 then fold the k+1 results in the reference order.
+// grid = ceil(H / 4), block = 64 * min(k + 1, 16).
+// dynamic LDS per wave: F bytes + F/32 halves (+ pad), then [k+1][4] floats.
+template <int KIND>
+__global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
+    extern __shared__ __align__(16) uint8_t lds_c[];
+    __shared__ Q8Tile tiles[16];
+    const bool shared = a.sh_inp != nullptr;
+    const int n_act = a.k + (shared ? 1 : 0);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nwaves = blockDim.x >> 6;
+    const size_t per_wave = (static_cast<size_t>(a.F) + a.F / 16 + 15) & ~static_cast<size_t>(15);
+    int8_t *aq = reinterpret_cast<int8_t *>(lds_c + wave * per_wave);
+    uint16_t *ad = reinterpret_cast<uint16_t *>(lds_c + wave * per_wave + a.F);
+    float *ybuf = reinterpret_cast<float *>(lds_c + nwaves * per_wave);  // [n_act][4]
+    const int r0 = blockIdx.x * 4;
+    const int nrows = min(4, a.H - r0);
+    const int nb = a.F >> 5;
+    const int r4 = lane >> 4;
+    mark(a, 2, 0);
+    mark_span(a, 2, false);
+    // combine operands, requested early: lane m keeps router weight m, lane 16 the shared gate
+    float wreg = 0.0f;
+    if (wave == 0) {
+        if (lane < a.k) wreg = a.weights[lane];
+        if (lane == 16 && shared) wreg = a.shared_gate[0];
+    }
+    for (int m = wave; m < n_act; m += nwaves) {
+        const bool is_shared = m == a.k;
+        const uint8_t *w = is_shared ? a.sh_down : mat_ptr_ids(a.down, m, a.ids[m]);
+        const size_t rb = static_cast<size_t>(nb) * ((KIND == 0 || is_shared) ? 34 : 18);
+        const uint8_t *const rows[1] = {w + r0 * rb};
+        float y[1];
+        auto quantise = [&]() {
+            wave_lds_fence();
+            lds_quantize_q8_0(a.act + static_cast<size_t>(m) * a.F, a.F, aq, ad, lane, 64);
+            wave_lds_fence();
+            mark(a, 2, 1);
+        };
+        if (KIND == 0 || is_shared)
+            q8_rows4_multi<0, 1, 1, false>(rows, nrows, nb, aq, ad, tiles[wave], lane, y, nullptr, 0, quantise);
+        else
+            q8_rows4_multi<1, 1, 1, false>(rows, nrows, nb, aq, ad, tiles[wave], lane, y, nullptr, 0, quantise);
+        if ((lane & 15) == 0) ybuf[m * 4 + r4] = y[0];
+        mark(a, 2, 2);
+    }
+    __syncthreads();
+    mark(a, 2, 3);
+    if (wave == 0) {
+        const int row = r0 + lane;
+        const bool on = lane < nrows;
+        float acc = 0.0f;
+        for (int m = 0; m < a.k; ++m) {
+            const float wm = lane_get(wreg, m);
+            const float y = ybuf[m * 4 + (lane & 3)];
+            const float prod = y * wm;
+            acc = acc + prod;
+            if (a.expert_out && on) a.expert_out[static_cast<size_t>(m) * a.H + row] = y;
+        }
+        const float gate = lane_get(wreg, 16);
+        mark_span(a, 2, true);
+        if (!on) return;
+        float o = acc;
+        if (shared) {
+            const float y = ybuf[a.k * 4 + lane];
+            const float prod = y * gate;
+            o = acc + prod;
+            a.down_f32[row] = y;
+        }
+        a.accum[row] = acc;
+        a.out[row] = o;
+        if (a.residual) {
+            const float scaled = o * a.residual_scale;
+            a.residual[row] = a.residual[row] + scaled;
+        }
+    }
+    mark(a, 2, 4);
+}
+
+}  // namespace wd

@@ -35,6 +35,13 @@ WD_DEV const uint8_t *mat_ptr(const MatSrc &s, int m) {
     return s.single;
 }
 
+// Same, with the expert id already known to the caller (per_expert tensors per expert).
+WD_DEV const uint8_t *mat_ptr_ids(const MatSrc &s, int m, int e) {
+    const int t = m % s.per_expert;
+    if (s.slot_of_expert) return s.pool + static_cast<size_t>(s.slot_of_expert[e]) * s.slot_bytes + s.slot_off[t];
+    return s.base[t] + static_cast<size_t>(e) * s.stride[t];
+}
+
 __global__ void k_fill_u32(uint32_t *dst, uint32_t v, size_t n) {
     const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i < n) dst[i] = v;
@@ -66,8 +73,7 @@ __global__ __launch_bounds__(256) void k_q8_k_quantize(const float *__restrict__
         d = 1.0f / iscale;
     }
     reinterpret_cast<uint32_t *>(qs + static_cast<size_t>(blk) * 256)[lane] = packed;
-    part += lane_xor(part, 1);
-    part += lane_xor(part, 2);
+    part = quad_sum_i(part);
     if ((lane & 3) == 0) bsums[static_cast<size_t>(blk) * 16 + (lane >> 2)] = static_cast<int16_t>(part);
     if (lane == 0) scales[blk] = d;
 }
@@ -92,9 +98,8 @@ __global__ __launch_bounds__(256) void k_q8_0_quantize(const float *__restrict__
     if (on) v = reinterpret_cast<const float4 *>(x + static_cast<size_t>(blk) * 32)[sub];
     float amax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)),
                                  __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
-    amax = __builtin_fmaxf(amax, lane_xor(amax, 1));
-    amax = __builtin_fmaxf(amax, lane_xor(amax, 2));
-    amax = __builtin_fmaxf(amax, lane_xor(amax, 4));
+    amax = quad_max(amax);
+    amax = __builtin_fmaxf(amax, dpp_f<0x141>(amax, amax));  // row_half_mirror pairs the two quads of a block
     if (!on) return;
     reinterpret_cast<uint32_t *>(qs + static_cast<size_t>(blk) * 32)[sub] = q8_0_pack4(v, amax);
     if (sub == 0) scales[blk] = f2h_ref(amax / 127.0f);
@@ -133,82 +138,6 @@ __global__ __launch_bounds__(256) void k_router_gemv(const float *__restrict__ w
             logits[row] = acc;
         else
             extra_out[0] = acc;
-    }
-}
-
-// ---- softmax + top-k + renormalise: one wave (src/qwen38_moe.cuh:711-818) ---------------------
-// If gate_logit != null, gate_logit[0] is replaced by sigmoid_ggml(gate_logit[0]) (shared expert gate).
-__global__ __launch_bounds__(64) void k_topk_softmax(const float *__restrict__ logits, int n, int k, float w_scale,
-                                                      int32_t *__restrict__ ids, float *__restrict__ weights,
-                                                      float *__restrict__ gate_logit) {
-    __shared__ float probs[1024];
-    __shared__ double gsum[128];
-    __shared__ float top[16];
-    const int lane = threadIdx.x;
-    if (gate_logit && lane == 0) gate_logit[0] = sigmoid_ggml(gate_logit[0]);
-
-    float mx = -INFINITY;
-    for (int e = lane; e < n; e += 64) mx = __builtin_fmaxf(mx, logits[e]);
-    mx = wave_max(mx);
-    for (int e = lane; e < n; e += 64) probs[e] = exp_ggml(logits[e] - mx);
-    __syncthreads();
-    const int groups = n >> 3;
-    for (int g = lane; g < groups; g += 64) {
-        const float *v = probs + g * 8;
-        const float lo = v[0] + v[4], lh = v[2] + v[6], hi = v[1] + v[5], hh = v[3] + v[7];
-        gsum[g] = static_cast<double>((lo + lh) + (hi + hh));
-    }
-    __syncthreads();
-    double sum = 0.0;
-    for (int g = 0; g < groups; ++g) sum += gsum[g];  // every lane, same ascending order
-    float v[16];
-    if (sum == 0.0) {
-        for (int e = lane; e < n; e += 64) probs[e] = -INFINITY;
-    } else {
-        const float inv = static_cast<float>(1.0 / sum);
-        for (int e = lane; e < n; e += 64) probs[e] = probs[e] * inv;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const int e = lane + 64 * i;
-        v[i] = (e < n) ? probs[e] : -INFINITY;
-    }
-    for (int j = 0; j < k; ++j) {
-        // lowest index among this lane's largest not-yet-taken probabilities
-        float bv = -INFINITY;
-        int bi = 0x7fffffff;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            if (v[i] > bv) {
-                bv = v[i];
-                bi = lane + 64 * i;
-            }
-        }
-        const float m = wave_max(bv);
-        const int cand = (bv == m && m > -INFINITY) ? bi : 0x7fffffff;
-        int win = wave_min_i(cand);
-        if (win == 0x7fffffff) win = 0;  // nothing beats -inf: the reference keeps id 0
-        if (lane == 0) {
-            ids[j] = win;
-            top[j] = probs[win];
-        }
-        if ((win & 63) == lane) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i)
-                if ((win >> 6) == i) v[i] = -INFINITY;
-        }
-    }
-    __syncthreads();
-    if (lane == 0) {
-        double wsum = 0.0;
-        for (int j = 0; j < k; ++j) wsum += static_cast<double>(top[j]);
-        const float denom = __builtin_fmaxf(static_cast<float>(wsum), 6.103515625e-5f);
-        for (int j = 0; j < k; ++j) {
-            float wj = top[j] / denom;
-            if (w_scale != 0.0f && w_scale != 1.0f) wj = wj * w_scale;
-            weights[j] = wj;
-        }
     }
 }
 
@@ -296,9 +225,11 @@ __global__ void k_sigmoid1(float *gate) {
 
 // accum[i] = ordered weighted sum of the k expert outputs (product rounded, then sum rounded);
 // out[i] = accum[i] + shared[i] * gate[0] when a shared expert is present, else accum[i].
+// residual (optional): residual[i] += out[i] * residual_scale.
 __global__ void k_combine(const float *__restrict__ experts, const float *__restrict__ weights, int k,
                           const float *__restrict__ shared, const float *__restrict__ gate,
-                          float *__restrict__ accum, float *__restrict__ out, int n) {
+                          float *__restrict__ accum, float *__restrict__ out, float *__restrict__ residual,
+                          float residual_scale, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     float a = 0.0f;
@@ -312,6 +243,10 @@ __global__ void k_combine(const float *__restrict__ experts, const float *__rest
         a = a + prod;
     }
     out[i] = a;
+    if (residual) {  // next layer's input in a layer stack
+        const float scaled = a * residual_scale;
+        residual[i] = residual[i] + scaled;
+    }
 }
 
 }  // namespace wd

@@ -1,7 +1,7 @@
 // Whole-layer entry points: scratch object and the staged layer pass (one launch per stage,
 // every stage a stand-alone operator of wd_ops.hip resolved against the device-side ids).
 #include "wd_common.h"
-#include "wd_kernels.cuh"
+#include "wd_fused.cuh"
 
 #include <new>
 
@@ -29,6 +29,9 @@ struct wd_moe_scratch {
     int32_t *gup = nullptr;
     int32_t *dp = nullptr;
     int gup_type = -1, dp_type = -1;
+    unsigned *arrive = nullptr;           // device counter used inside the fused dispatch A
+    unsigned long long *trace = nullptr;  // device [3][16][8] time stamps, see wd_moe_scratch_trace
+    int trace_wg = 0;
 };
 
 namespace {
@@ -64,7 +67,8 @@ int wd_moe_scratch_create(wd_moe_scratch **out, int hidden, int expert_ffn, int 
                  o_x0d = c.take(sizeof(uint16_t) * (H / 32)), o_gu = c.take(sizeof(float) * K1 * 2 * F),
                  o_act = c.take(sizeof(float) * K1 * F), o_aq = c.take(K1 * F),
                  o_ad = c.take(sizeof(uint16_t) * K1 * (F / 32)), o_eo = c.take(sizeof(float) * K1 * H),
-                 o_acc = c.take(sizeof(float) * H), o_dn = c.take(sizeof(float) * H), o_sg = c.take(256);
+                 o_acc = c.take(sizeof(float) * H), o_dn = c.take(sizeof(float) * H), o_sg = c.take(256),
+                 o_arr = c.take(256);
     const hipError_t e = hipMalloc(reinterpret_cast<void **>(&s->block), c.off);
     if (e != hipSuccess) {
         delete s;
@@ -87,6 +91,7 @@ int wd_moe_scratch_create(wd_moe_scratch **out, int hidden, int expert_ffn, int 
     s->accum = reinterpret_cast<float *>(b + o_acc);
     s->down_f32 = reinterpret_cast<float *>(b + o_dn);
     s->shared_gate = reinterpret_cast<float *>(b + o_sg);
+    s->arrive = reinterpret_cast<unsigned *>(b + o_arr);
     (void)hipMemset(s->block, 0, c.off);
     *out = s;
     return WD_OK;
@@ -97,6 +102,7 @@ int wd_moe_scratch_destroy(wd_moe_scratch *s) {
     (void)hipFree(s->block);
     (void)hipFree(s->gup);
     (void)hipFree(s->dp);
+    (void)hipFree(s->trace);
     delete s;
     return WD_OK;
 }
@@ -114,6 +120,23 @@ float *wd_moe_scratch_down_f32(wd_moe_scratch *s) { return s->down_f32; }
 float *wd_moe_scratch_shared_gate(wd_moe_scratch *s) { return s->shared_gate; }
 int32_t *wd_moe_scratch_gate_up_partials(wd_moe_scratch *s) { return s->gup; }
 int32_t *wd_moe_scratch_down_partials(wd_moe_scratch *s) { return s->dp; }
+
+// Profiling aid: allocates (once) a buffer of 3 x 16 x 8 time stamps (100 MHz counter) that the fused
+// dispatches A, B, C fill for workgroup `wg` (per wave, per marked point); returns its device address.
+unsigned long long *wd_moe_scratch_trace(wd_moe_scratch *s, int wg) {
+    if (!s) return nullptr;
+    if (!s->trace) {
+        if (hipMalloc(reinterpret_cast<void **>(&s->trace), sizeof(unsigned long long) * 3 * 16 * 8) != hipSuccess) return nullptr;
+        (void)hipMemset(s->trace, 0, sizeof(unsigned long long) * 3 * 16 * 8);
+    }
+    for (int d = 0; d < 3; ++d) {  // earliest-start cells start at the maximum
+        const unsigned long long big = ~0ull;
+        (void)hipMemcpy(s->trace + (d * 16 + 15) * 8, &big, sizeof(big), hipMemcpyHostToDevice);
+        (void)hipMemset(s->trace + (d * 16 + 15) * 8 + 1, 0, sizeof(big));
+    }
+    s->trace_wg = wg;
+    return s->trace;
+}
 
 int wd_moe_scratch_enable_partials(wd_moe_scratch *s, int gate_type, int down_type) {
     WD_REQUIRE(s != nullptr, "enable partials: null scratch");
@@ -218,11 +241,12 @@ int grouped_gemv(int type, MatSrc src, int mats, int rows, int cols, const wd_mo
 
 }  // namespace
 
-extern "C" int wd_moe_layer_f32(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s,
-                                unsigned flags, void *stream) {
-    if (const int rc = check_layer(L, s)) return rc;
-    WD_REQUIRE(d_x && d_out, "MoE layer: null activation or output pointer");
-    hipStream_t st = as_stream(stream);
+namespace {
+
+// One layer, one launch per stage.  ids_override (device, k ids) replaces the router's ids while
+// keeping its weights; residual (device f32[hidden]) receives residual += layer output.
+int layer_staged(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s, unsigned flags,
+                 const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st) {
     const int H = L->hidden, F = L->expert_ffn, E = L->n_experts, k = L->top_k;
     const bool shared = L->shared_gate_inp != nullptr;
     const bool pre = (flags & WD_MOE_PRESELECTED) != 0;
@@ -234,7 +258,7 @@ extern "C" int wd_moe_layer_f32(const wd_moe_layer *L, const float *d_x, float *
         WD_LAUNCH_CHECK();
         if (E % 8 != 0 || E > 1024) return fail(WD_ERR_UNSUPPORTED, "router: n_experts %d must be a multiple of 8 <= 1024", E);
         k_topk_softmax<<<dim3(1), dim3(64), 0, st>>>(s->logits, E, k, L->expert_scale, s->ids, s->weights,
-                                                     shared ? s->shared_gate : nullptr);
+                                                     shared ? s->shared_gate : nullptr, ids_override);
         WD_LAUNCH_CHECK();
     } else if (shared) {
         k_router_gemv<<<dim3(1), dim3(256), 0, st>>>(L->router, d_x, s->logits, 0, H, L->shared_gate_inp, s->shared_gate);
@@ -287,7 +311,96 @@ extern "C" int wd_moe_layer_f32(const wd_moe_layer *L, const float *d_x, float *
 
     // 7. ordered weighted sum and the shared branch
     k_combine<<<dim3((H + 255) / 256), dim3(256), 0, st>>>(s->expert_out, s->weights, k, shared ? s->down_f32 : nullptr,
-                                                            s->shared_gate, s->accum, d_out, H);
+                                                            s->shared_gate, s->accum, d_out, residual, residual_scale, H);
     WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+// One layer in three dispatches (router+shared gate/up, top-k+routed gate/up, down+combine).
+int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s, unsigned flags,
+                const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st) {
+    const int H = L->hidden, F = L->expert_ffn, E = L->n_experts, k = L->top_k;
+    const bool shared = L->shared_gate_inp != nullptr;
+    LayerArgs a{};
+    a.H = H, a.F = F, a.E = E, a.k = k;
+    a.w_scale = L->expert_scale;
+    a.x = d_x;
+    a.router = L->router;
+    a.gate_up = routed_src(L, s->ids, false);
+    a.down = routed_src(L, s->ids, true);
+    a.sh_inp = L->shared_gate_inp;
+    a.sh_gate = L->shared_gate, a.sh_up = L->shared_up, a.sh_down = L->shared_down;
+    a.logits = s->logits, a.ids = s->ids, a.weights = s->weights;
+    a.ids_override = ids_override;
+    a.act = s->act;
+    a.shared_gate = s->shared_gate;
+    a.expert_out = (flags & WD_MOE_KEEP_EXPERT_OUT) ? s->expert_out : nullptr;
+    a.accum = s->accum, a.down_f32 = s->down_f32, a.out = d_out;
+    a.residual = residual, a.residual_scale = residual_scale;
+    a.preselected = (flags & WD_MOE_PRESELECTED) ? 1 : 0;
+    const int router_rows_n = (a.preselected ? 0 : E) + (shared ? 1 : 0);
+    a.n_router_wgs = (router_rows_n + 15) / 16;
+    a.trace = s->trace, a.trace_wg = s->trace_wg;
+    a.arrive = s->arrive;
+
+    const int grid_a = a.n_router_wgs + (shared ? (F + 7) / 8 : 0);
+    if (grid_a > 0) {
+        k_layer_a<<<dim3(grid_a), dim3(512), static_cast<size_t>(H) + H / 16, st>>>(a);
+        WD_LAUNCH_CHECK();
+    }
+    const bool iq = consumes_q8k(L->gate_type);
+    const size_t lds_b = H + (iq ? sizeof(float) * (H / 256) : sizeof(uint16_t) * (H / 32));
+    const int grid_b = k * (L->gate_type == WD_TYPE_IQ4_NL ? (F + 15) / 16 : (F + 7) / 8);
+    switch (L->gate_type) {
+        case WD_TYPE_IQ3_S: k_layer_b<21><<<dim3(grid_b), dim3(512), lds_b, st>>>(a); break;
+        case WD_TYPE_IQ2_S: k_layer_b<22><<<dim3(grid_b), dim3(512), lds_b, st>>>(a); break;
+        case WD_TYPE_Q8_0: k_layer_b<8><<<dim3(grid_b), dim3(512), lds_b, st>>>(a); break;
+        case WD_TYPE_IQ4_NL: k_layer_b<20><<<dim3(grid_b), dim3(256), lds_b, st>>>(a); break;
+        default: return fail(WD_ERR_UNSUPPORTED, "fused layer: unsupported gate/up type %d", L->gate_type);
+    }
+    WD_LAUNCH_CHECK();
+    const int n_act = k + (shared ? 1 : 0);
+    const int waves_c = n_act < 16 ? n_act : 16;
+    const size_t per_wave = (static_cast<size_t>(F) + F / 16 + 15) & ~static_cast<size_t>(15);
+    const size_t lds_c = waves_c * per_wave + sizeof(float) * 4 * n_act;
+    const int grid_c = (H + 3) / 4;
+    if (L->down_type == WD_TYPE_Q8_0)
+        k_layer_c<0><<<dim3(grid_c), dim3(64 * waves_c), lds_c, st>>>(a);
+    else
+        k_layer_c<1><<<dim3(grid_c), dim3(64 * waves_c), lds_c, st>>>(a);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+int layer_dispatch(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s, unsigned flags,
+                   const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st) {
+    const bool want_partials = s->gup != nullptr;
+    if ((flags & WD_MOE_STAGED) || want_partials)
+        return layer_staged(L, d_x, d_out, s, flags, ids_override, residual, residual_scale, st);
+    return layer_fused(L, d_x, d_out, s, flags, ids_override, residual, residual_scale, st);
+}
+
+}  // namespace
+
+extern "C" int wd_moe_layer_f32(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s,
+                                unsigned flags, void *stream) {
+    if (const int rc = check_layer(L, s)) return rc;
+    WD_REQUIRE(d_x && d_out, "MoE layer: null activation or output pointer");
+    return layer_dispatch(L, d_x, d_out, s, flags, nullptr, nullptr, 0.0f, as_stream(stream));
+}
+
+extern "C" int wd_moe_stack_f32(const wd_moe_layer *layers, int n_layers, float *d_x, float *d_layer_out,
+                                wd_moe_scratch *s, const int32_t *d_ids_trace, float residual_scale, unsigned flags,
+                                void *stream) {
+    WD_REQUIRE(layers && n_layers > 0, "MoE stack: no layers");
+    WD_REQUIRE(d_x && d_layer_out, "MoE stack: null activation or output pointer");
+    for (int l = 0; l < n_layers; ++l) {
+        if (const int rc = check_layer(&layers[l], s)) return rc;
+    }
+    for (int l = 0; l < n_layers; ++l) {
+        const int32_t *trace = d_ids_trace ? d_ids_trace + static_cast<size_t>(l) * layers[l].top_k : nullptr;
+        if (const int rc = layer_dispatch(&layers[l], d_x, d_layer_out, s, flags, trace, d_x, residual_scale, as_stream(stream)))
+            return rc;
+    }
     return WD_OK;
 }

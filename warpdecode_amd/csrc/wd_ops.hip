@@ -3,7 +3,7 @@
 // and the elementwise stages.  Each extern "C" entry point mirrors one launcher of the
 // reference operator surface (see include/warpdecode_amd.h for the citations).
 #include "wd_common.h"
-#include "wd_kernels.cuh"
+#include "wd_fused.cuh"
 
 namespace wd {
 
@@ -148,7 +148,7 @@ int wd_topk_softmax(const float *d_logits, int n_experts, int k, float expert_sc
     WD_REQUIRE(k > 0 && k <= 16 && k <= n_experts, "top-k softmax: k must be in (0, 16] (got %d)", k);
     WD_REQUIRE(d_logits && d_ids && d_weights, "wd_topk_softmax: null pointer");
     k_topk_softmax<<<dim3(1), dim3(64), 0, as_stream(stream)>>>(d_logits, n_experts, k, expert_scale, d_ids, d_weights,
-                                                                nullptr);
+                                                                nullptr, nullptr);
     WD_LAUNCH_CHECK();
     return WD_OK;
 }

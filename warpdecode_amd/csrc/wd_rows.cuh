@@ -79,143 +79,216 @@ WD_DEV void stage_tables(IqTables &t, int tid, int nthreads) {
 // Magnitudes are >= 1, so (m ^ 0xff) + 1 never carries out of its byte.
 WD_DEV uint32_t apply_signs(uint32_t mags, uint2 sm) { return (mags ^ sm.x) + sm.y; }
 
-// Sum over the eight lanes of a group of p[c], delivered to the lane with (lane & 7) == c.
-WD_DEV int reduce_scatter8(const int (&p)[8], int lane) {
-    const bool h4 = (lane & 4) != 0;
-    int r[4];
+typedef unsigned wd_uint2v __attribute__((ext_vector_type(2)));
+
+// Lane layout of the IQ decoders: lane = 8 * ib + sb (ib = 32-value block inside the super-block,
+// sb = super-block of the current pass).  The eight lanes that share sb are 8 apart, so their
+// chunk sums are folded with a half swap (ib bit 2), a row-pair swap (ib bit 1) and a rotate by 8
+// inside the row (ib bit 0).  Returns, in lane (ib, sb), the sum over the eight ib-lanes of p[ib].
+WD_DEV int reduce_scatter_ib(const int (&p)[8], int lane) {
+    int q[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const int keep = h4 ? p[j + 4] : p[j];
-        const int send = h4 ? p[j] : p[j + 4];
-        r[j] = keep + lane_xor(send, 4);
+        // .x = (own low half, partner-low's p[j+4]);  .y = (partner-high's p[j], own high half)
+        const wd_uint2v r = __builtin_amdgcn_permlane32_swap(static_cast<unsigned>(p[j]), static_cast<unsigned>(p[j + 4]),
+                                                            false, false);
+        q[j] = static_cast<int>(r.x + r.y);  // lanes < 32: chunk j, lanes >= 32: chunk j + 4
     }
-    const bool h2 = (lane & 2) != 0;
-    int s[2];
+    int s2[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        const int keep = h2 ? r[j + 2] : r[j];
-        const int send = h2 ? r[j] : r[j + 2];
-        s[j] = keep + lane_xor(send, 2);
+        const wd_uint2v r = __builtin_amdgcn_permlane16_swap(static_cast<unsigned>(q[j]), static_cast<unsigned>(q[j + 2]),
+                                                            false, false);
+        s2[j] = static_cast<int>(r.x + r.y);  // even rows: q[j] family, odd rows: q[j + 2] family
     }
-    const bool h1 = (lane & 1) != 0;
-    const int keep = h1 ? s[1] : s[0];
-    const int send = h1 ? s[0] : s[1];
-    return keep + lane_xor(send, 1);
+    const bool odd = (lane & 8) != 0;
+    const int keep = odd ? s2[1] : s2[0];
+    const int send = odd ? s2[0] : s2[1];
+    return keep + dpp_i<kDppRor8>(0, send);
 }
 
 // ---- IQ3_S / IQ2_S x Q8_K ------------------------------------------------------------
 // Lane (sb = lane >> 3, ib = lane & 7) decodes 32-value block ib of super-block 8*pass + sb.
 // chunk sums p[c] = ls * dot4(signed magnitudes of chunk c, activations 4c..4c+3 of the block).
-WD_DEV void iq3s_block_chunks(const uint8_t *blk, int ib, const IqTables &t, const uint32_t (&a)[8],
-                              int (&p)[8]) {
-    const uint2 qs = ldu<uint2>(blk + 2 + ib * 8);
-    const uint32_t qh = blk[66 + ib];
-    const uint32_t sg = ldu<uint32_t>(blk + 74 + ib * 4);
-    const uint32_t sc = blk[106 + (ib >> 1)];
-    const int ls = 1 + 2 * static_cast<int>((sc >> (4 * (ib & 1))) & 15u);
+// Loading and decoding are separate steps so that a wave can put the loads of several rows in
+// flight before it starts to decode the first one.
+struct IqFields {
+    uint2 qs;       // IQ3_S: 8 index bytes; IQ2_S: .x = 4 index bytes, .y = 4 sign bytes
+    uint32_t sg;    // IQ3_S: 4 sign bytes
+    uint32_t qh, sc;
+    uint16_t d;
+};
+
+template <int TYPE>
+WD_DEV IqFields iq_load(const uint8_t *blk, int ib) {
+    IqFields f;
+    if (TYPE == 21) {
+        f.qs = gld_u64(blk + 2 + ib * 8);
+        f.qh = gld_u8(blk + 66 + ib);
+        f.sg = gld_u32(blk + 74 + ib * 4);
+        f.sc = gld_u8(blk + 106 + (ib >> 1));
+    } else {
+        f.qs.x = gld_u32(blk + 2 + ib * 4);
+        f.qs.y = gld_u32(blk + 34 + ib * 4);
+        f.sg = 0;
+        f.qh = gld_u8(blk + 66 + ib);
+        f.sc = gld_u8(blk + 74 + ib);
+    }
+    f.d = gld_u16(blk);
+    return f;
+}
+
+template <int TYPE>
+WD_DEV void iq_chunks(const IqFields &f, int ib, const IqTables &t, const uint32_t (&a)[8], int (&p)[8]) {
+    if (TYPE == 21) {
+        const int ls = 1 + 2 * static_cast<int>((f.sc >> (4 * (ib & 1))) & 15u);
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-        const uint32_t q = ((c < 4 ? qs.x : qs.y) >> (8 * (c & 3))) & 0xffu;
-        const uint32_t idx = q | ((qh << (8 - c)) & 0x100u);
-        const uint32_t sbits = (sg >> (4 * c)) & 15u;  // byte c>>1, nibble c&1
-        const uint32_t w4 = apply_signs(t.grid3[idx], t.sign[sbits]);
-        p[c] = ls * sdot4(w4, a[c], 0);
+        for (int c = 0; c < 8; ++c) {
+            const uint32_t q = ((c < 4 ? f.qs.x : f.qs.y) >> (8 * (c & 3))) & 0xffu;
+            const uint32_t idx = q | ((f.qh << (8 - c)) & 0x100u);
+            const uint32_t sbits = (f.sg >> (4 * c)) & 15u;  // sign byte c>>1, nibble c&1
+            p[c] = __mul24(ls, sdot4(apply_signs(t.grid3[idx], t.sign[sbits]), a[c], 0));
+        }
+    } else {
+        const int ls_lo = 1 + 2 * static_cast<int>(f.sc & 15u);
+        const int ls_hi = 1 + 2 * static_cast<int>(f.sc >> 4);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const uint32_t idx = ((f.qs.x >> (8 * g)) & 0xffu) | ((f.qh << (8 - 2 * g)) & 0x300u);
+            const uint64_t mags = t.grid2[idx];
+            const uint32_t s8 = (f.qs.y >> (8 * g)) & 0xffu;
+            const int ls = (g < 2) ? ls_lo : ls_hi;  // chunks 0..3 low nibble, 4..7 high nibble
+            p[2 * g] = __mul24(ls, sdot4(apply_signs(static_cast<uint32_t>(mags), t.sign[s8 & 15u]), a[2 * g], 0));
+            p[2 * g + 1] = __mul24(ls, sdot4(apply_signs(static_cast<uint32_t>(mags >> 32), t.sign[s8 >> 4]), a[2 * g + 1], 0));
+        }
     }
 }
 
-WD_DEV void iq2s_block_chunks(const uint8_t *blk, int ib, const IqTables &t, const uint32_t (&a)[8],
-                              int (&p)[8]) {
-    const uint32_t qs = ldu<uint32_t>(blk + 2 + ib * 4);
-    const uint32_t sg = ldu<uint32_t>(blk + 34 + ib * 4);
-    const uint32_t qh = blk[66 + ib];
-    const uint32_t sc = blk[74 + ib];
-    const int ls_lo = 1 + 2 * static_cast<int>(sc & 15u);
-    const int ls_hi = 1 + 2 * static_cast<int>(sc >> 4);
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-        const uint32_t idx = ((qs >> (8 * g)) & 0xffu) | ((qh << (8 - 2 * g)) & 0x300u);
-        const uint64_t mags = t.grid2[idx];
-        const uint32_t s8 = (sg >> (8 * g)) & 0xffu;
-        const int ls = (g < 2) ? ls_lo : ls_hi;  // chunks 0..3 low nibble, 4..7 high nibble
-        p[2 * g] = ls * sdot4(apply_signs(static_cast<uint32_t>(mags), t.sign[s8 & 15u]), a[2 * g], 0);
-        p[2 * g + 1] = ls * sdot4(apply_signs(static_cast<uint32_t>(mags >> 32), t.sign[s8 >> 4]), a[2 * g + 1], 0);
-    }
-}
+// NR rows against one Q8_K activation (act_qs / act_d in global memory or LDS).  y[i] is uniform
+// across the wave.  `partials` (PART only): int32 [nb][8] per row, rows `pstride` ints apart.
+//
+// Float order: chunk lane c accumulates fma(d_w * d_x, (float)sum, acc) over ascending super-blocks.
+// After the integer fold, lane (c, sb) holds chunk c of super-block sb, so the eight lanes of one
+// group form the chain of chunk c: the accumulator moves one lane up per step (row_shr:1) and the
+// finished chain sits in the group's last lane.
+struct NoPre {
+    WD_DEV void operator()() const {}
+};
 
-// One row.  act_qs / act_d: Q8_K activation (global or LDS).  Result valid in lane 0.
-// `partials` (PART only): int32 [nb][8] for this row.
-template <int TYPE, bool PART>
-WD_DEV float iq_row_q8k(const uint8_t *row, int nb, const IqTables &t, const int8_t *act_qs, const float *act_d,
-                        int lane, int32_t *partials) {
+// `pre` runs once, after the weight loads of the first pass have been issued and before the
+// activation is read: the place to produce the activation (quantise into LDS, barrier) while the
+// weights are in flight.
+template <int TYPE, int NR, bool PART, typename Pre = NoPre>
+WD_DEV void iq_rows_q8k(const uint8_t *const (&rows)[NR], int nb, const IqTables &t, const int8_t *act_qs,
+                        const float *act_d, int lane, float (&y)[NR], int32_t *partials, size_t pstride,
+                        Pre pre = Pre()) {
     constexpr int kBlk = (TYPE == 21) ? 110 : 82;
-    const int sbl = lane >> 3, ib = lane & 7;
-    float acc = 0.0f;
+    const int ib = lane >> 3, sbl = lane & 7;
+    const bool first = sbl == 0;
+    float acc[NR];
+#pragma unroll
+    for (int i = 0; i < NR; ++i) acc[i] = 0.0f;
     for (int base = 0; base < nb; base += 8) {
         const int sb = base + sbl;
         const bool on = sb < nb;
-        int p[8];
-        float ds = 0.0f;
+        IqFields f[NR];
+        uint32_t a[8];
+        float dx = 0.0f;
         if (on) {
-            uint32_t a[8];
+#pragma unroll
+            for (int i = 0; i < NR; ++i) f[i] = iq_load<TYPE>(rows[i] + static_cast<size_t>(sb) * kBlk, ib);
+        }
+        if (base == 0) pre();
+        if (on) {
             const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32);
             const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32 + 16);
             a[0] = a0.x, a[1] = a0.y, a[2] = a0.z, a[3] = a0.w, a[4] = a1.x, a[5] = a1.y, a[6] = a1.z, a[7] = a1.w;
-            const uint8_t *blk = row + static_cast<size_t>(sb) * kBlk;
-            if (TYPE == 21)
-                iq3s_block_chunks(blk, ib, t, a, p);
-            else
-                iq2s_block_chunks(blk, ib, t, a, p);
-            ds = h2f(ldu<uint16_t>(blk)) * act_d[sb];
-        } else {
-#pragma unroll
-            for (int c = 0; c < 8; ++c) p[c] = 0;
+            dx = act_d[sb];
         }
-        const int P = reduce_scatter8(p, lane);  // lane (sbl, c): chunk c of super-block sb
-        if (PART && on) partials[sb * 8 + ib] = P;
-        const float pf = static_cast<float>(P);
-        const int cnt = min(8, nb - base);
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            if (s < cnt) {
-                const float pv = lane_get(pf, s * 8 + ib);
-                const float dv = lane_get(ds, s * 8 + ib);
-                acc = __builtin_fmaf(dv, pv, acc);
+        for (int i = 0; i < NR; ++i) {
+            int p[8];
+            float ds = 0.0f;
+            if (on) {
+                iq_chunks<TYPE>(f[i], ib, t, a, p);
+                ds = h2f(f[i].d) * dx;
+            } else {
+#pragma unroll
+                for (int c = 0; c < 8; ++c) p[c] = 0;
             }
+            const int P = reduce_scatter_ib(p, lane);  // lane (c = ib, sb): chunk c of super-block sb
+            if (PART && on) partials[i * pstride + sb * 8 + ib] = P;
+            const float pf = static_cast<float>(P);
+            // carry of the previous pass: last lane of the group -> first lane (lanes past the row's
+            // end pass the accumulator through unchanged, fma(0, 0, acc) == acc)
+            const float carry = dpp_f<kDppShl7>(0.0f, acc[i]);
+            float v = __builtin_fmaf(ds, pf, base == 0 ? 0.0f : carry);
+#pragma unroll
+            for (int s = 1; s < 8; ++s) {
+                const float up = dpp_f<kDppShr1>(0.0f, v);
+                const float nxt = __builtin_fmaf(ds, pf, up);
+                v = first ? v : nxt;
+            }
+            acc[i] = v;
         }
     }
-    float r = close_lanes8(acc);
-    if (TYPE == 22) r = 0.125f * r;
-    return r;
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+        const float r = close_lanes8_strided(acc[i]);
+        y[i] = (TYPE == 22) ? 0.125f * r : r;
+    }
+}
+
+template <int TYPE, bool PART>
+WD_DEV float iq_row_q8k(const uint8_t *row, int nb, const IqTables &t, const int8_t *act_qs, const float *act_d,
+                        int lane, int32_t *partials) {
+    const uint8_t *const rows[1] = {row};
+    float y[1];
+    iq_rows_q8k<TYPE, 1, PART, NoPre>(rows, nb, t, act_qs, act_d, lane, y, partials, 0);
+    return y[0];
 }
 
 // ---- Q8_0 (and Q4_0 / IQ4_NL codes) x Q8_0 ------------------------------------------------
 // Four rows per wave step: lane (r4 = lane >> 4, b = lane & 15) takes blocks b, b+16, ... of row r4.
 // The per-block chunk sums are handed to the chain lanes through a per-wave LDS tile so that every
 // chunk accumulator sees its blocks in ascending order.
-struct Q8Tile {
-    float pf[4 * 136];  // [r4][b][c], row stride padded to 136 floats (bank spread)
-    float ds[64];       // [r4][b]
+template <int CH>
+struct Q8TileN {
+    float pf[CH][4 * 136];  // [pass][r4][b][c], row stride padded to 136 floats (bank spread)
+    float ds[CH][64];       // [pass][r4][b]
 };
+using Q8Tile = Q8TileN<1>;
 
 // kind: 0 = Q8_0 (34-byte blocks), 1 = IQ4_NL (18-byte blocks, codebook values)
+struct Q8Block {
+    uint4 q0, q1;  // Q8_0: 32 quants; IQ4_NL: q0 = 16 nibble bytes
+    uint16_t d;
+};
+
 template <int KIND>
-WD_DEV void q8ish_block_chunks(const uint8_t *blk, const uint32_t (&a)[8], int (&p)[8]) {
+WD_DEV Q8Block q8_load(const uint8_t *blk) {
+    Q8Block w;
+    w.q0 = gld_u128(blk + 2);
+    if (KIND == 0) w.q1 = gld_u128(blk + 18);
+    w.d = gld_u16(blk);
+    return w;
+}
+
+template <int KIND>
+WD_DEV void q8_chunks(const Q8Block &w, const uint32_t (&a)[8], int (&p)[8]) {
     if (KIND == 0) {
-        const uint4 q0 = ldu<uint4>(blk + 2);
-        const uint4 q1 = ldu<uint4>(blk + 18);
-        p[0] = sdot4(q0.x, a[0], 0), p[1] = sdot4(q0.y, a[1], 0), p[2] = sdot4(q0.z, a[2], 0);
-        p[3] = sdot4(q0.w, a[3], 0), p[4] = sdot4(q1.x, a[4], 0), p[5] = sdot4(q1.y, a[5], 0);
-        p[6] = sdot4(q1.z, a[6], 0), p[7] = sdot4(q1.w, a[7], 0);
+        p[0] = sdot4(w.q0.x, a[0], 0), p[1] = sdot4(w.q0.y, a[1], 0), p[2] = sdot4(w.q0.z, a[2], 0);
+        p[3] = sdot4(w.q0.w, a[3], 0), p[4] = sdot4(w.q1.x, a[4], 0), p[5] = sdot4(w.q1.y, a[5], 0);
+        p[6] = sdot4(w.q1.z, a[6], 0), p[7] = sdot4(w.q1.w, a[7], 0);
     } else {
         // chunk l < 4: low nibbles of bytes 4l..4l+3; chunk l >= 4: high nibbles of bytes 4(l-4)..
-        const uint4 n = ldu<uint4>(blk + 2);
-        const uint32_t w[4] = {n.x, n.y, n.z, n.w};
+        const uint32_t n[4] = {w.q0.x, w.q0.y, w.q0.z, w.q0.w};
 #pragma unroll
         for (int l = 0; l < 4; ++l) {
             int lo = 0, hi = 0;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const uint32_t byte = (w[l] >> (8 * j)) & 0xffu;
+                const uint32_t byte = (n[l] >> (8 * j)) & 0xffu;
                 constexpr int8_t lut[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
                 lo += static_cast<int>(lut[byte & 15u]) * static_cast<int>(static_cast<int8_t>(a[l] >> (8 * j)));
                 hi += static_cast<int>(lut[byte >> 4]) * static_cast<int>(static_cast<int8_t>(a[l + 4] >> (8 * j)));
@@ -226,82 +299,189 @@ WD_DEV void q8ish_block_chunks(const uint8_t *blk, const uint32_t (&a)[8], int (
     }
 }
 
-// rows: pointer to the first of up to four consecutive rows (row stride = nb * block bytes);
-// nrows (1..4) rows are valid.  Result for row r4 valid in lane r4*16.
-// partials (PART): int32 [4][nb][8] starting at the first row.
-template <int KIND, bool PART>
-WD_DEV float q8_rows4(const uint8_t *rows, int nrows, int nb, const int8_t *act_qs, const uint16_t *act_d,
-                      Q8Tile &tile, int lane, int32_t *partials) {
+// NM matrices, the same four consecutive rows of each (row stride = nb * block bytes), against one
+// Q8_0 activation.  rows[i]: first of the (up to) four rows of matrix i; nrows (0..4) rows are valid.
+// y[i] for row r4 valid in lane r4*16.  CH passes (16 blocks per row each) of every matrix are
+// loaded before the first one is decoded, and their chunk sums go through the tile together, so a
+// row of up to 16*CH blocks needs one hand-off.
+// partials (PART): int32 [4][nb][8] per matrix, matrices `pstride` ints apart.
+template <int KIND, int NM, int CH, bool PART, typename Pre = NoPre>
+WD_DEV void q8_rows4_multi(const uint8_t *const (&rows)[NM], int nrows, int nb, const int8_t *act_qs,
+                           const uint16_t *act_d, Q8TileN<CH> &tile, int lane, float (&y)[NM], int32_t *partials,
+                           size_t pstride, Pre pre = Pre()) {
     constexpr int kBlk = (KIND == 0) ? 34 : 18;
     const int r4 = lane >> 4, b = lane & 15, c = lane & 7;
     const bool row_on = r4 < nrows;
-    const uint8_t *row = rows + static_cast<size_t>(r4) * nb * kBlk;
-    float acc = 0.0f;
+    const size_t row_off = static_cast<size_t>(r4) * nb * kBlk;
     // IQ4_NL pairs blocks into an even and an odd accumulator and treats a trailing unpaired block
     // apart (src/qwen38_cpu_moe.cuh:377-422).
-    float acc_odd = 0.0f;
+    float acc[NM], acc_odd[NM], tail[NM];
+#pragma unroll
+    for (int i = 0; i < NM; ++i) acc[i] = acc_odd[i] = tail[i] = 0.0f;
     const int paired = (KIND == 1) ? (nb & ~1) : nb;
-    for (int base = 0; base < nb; base += 16) {
-        const int bi = base + b;
-        const bool on = row_on && bi < nb;
-        int p[8];
-        float ds = 0.0f;
-        if (on) {
-            uint32_t a[8];
-            const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + bi * 32);
-            const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + bi * 32 + 16);
-            a[0] = a0.x, a[1] = a0.y, a[2] = a0.z, a[3] = a0.w, a[4] = a1.x, a[5] = a1.y, a[6] = a1.z, a[7] = a1.w;
-            const uint8_t *blk = row + static_cast<size_t>(bi) * kBlk;
-            q8ish_block_chunks<KIND>(blk, a, p);
-            ds = h2f(ldu<uint16_t>(blk)) * h2f(act_d[bi]);
-            if (PART) {
+    for (int base0 = 0; base0 < nb; base0 += 16 * CH) {
+        Q8Block wb[NM][CH];
+        uint4 a0[CH], a1[CH];
+        uint16_t dxh[CH];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) partials[(static_cast<size_t>(r4) * nb + bi) * 8 + j] = p[j];
+        for (int ch = 0; ch < CH; ++ch) {
+            const int bi = base0 + 16 * ch + b;
+            if (row_on && bi < nb) {
+#pragma unroll
+                for (int i = 0; i < NM; ++i) wb[i][ch] = q8_load<KIND>(rows[i] + row_off + static_cast<size_t>(bi) * kBlk);
             }
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) p[j] = 0;
         }
-        wave_lds_fence();  // previous pass's reads are done before the tile is overwritten
-        float4 *dst = reinterpret_cast<float4 *>(&tile.pf[r4 * 136 + b * 8]);
-        dst[0] = make_float4(static_cast<float>(p[0]), static_cast<float>(p[1]), static_cast<float>(p[2]),
-                             static_cast<float>(p[3]));
-        dst[1] = make_float4(static_cast<float>(p[4]), static_cast<float>(p[5]), static_cast<float>(p[6]),
-                             static_cast<float>(p[7]));
-        tile.ds[lane] = ds;
-        wave_lds_fence();
-        const int cnt = min(16, nb - base);
+        if (base0 == 0) pre();
 #pragma unroll
-        for (int s = 0; s < 16; ++s) {
-            if (s < cnt) {
-                const float pv = tile.pf[r4 * 136 + s * 8 + c];
-                const float dv = tile.ds[r4 * 16 + s];
-                if (KIND == 1) {
-                    const int blk_i = base + s;
-                    if (blk_i < paired) {
-                        if (blk_i & 1)
-                            acc_odd = __builtin_fmaf(dv, pv, acc_odd);
-                        else
-                            acc = __builtin_fmaf(dv, pv, acc);
+        for (int ch = 0; ch < CH; ++ch) {
+            const int bi = base0 + 16 * ch + b;
+            if (row_on && bi < nb) {
+                a0[ch] = *reinterpret_cast<const uint4 *>(act_qs + bi * 32);
+                a1[ch] = *reinterpret_cast<const uint4 *>(act_qs + bi * 32 + 16);
+                dxh[ch] = act_d[bi];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+            wave_lds_fence();  // earlier reads of the tile are done before it is overwritten
+#pragma unroll
+            for (int ch = 0; ch < CH; ++ch) {
+                const int bi = base0 + 16 * ch + b;
+                const bool on = row_on && bi < nb;
+                int p[8];
+                float ds = 0.0f;
+                if (on) {
+                    const uint32_t a[8] = {a0[ch].x, a0[ch].y, a0[ch].z, a0[ch].w, a1[ch].x, a1[ch].y, a1[ch].z, a1[ch].w};
+                    q8_chunks<KIND>(wb[i][ch], a, p);
+                    ds = h2f(wb[i][ch].d) * h2f(dxh[ch]);
+                    if (PART) {
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) partials[i * pstride + (static_cast<size_t>(r4) * nb + bi) * 8 + j] = p[j];
                     }
                 } else {
-                    acc = __builtin_fmaf(dv, pv, acc);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) p[j] = 0;
+                }
+                float4 *dst = reinterpret_cast<float4 *>(&tile.pf[ch][r4 * 136 + b * 8]);
+                dst[0] = make_float4(static_cast<float>(p[0]), static_cast<float>(p[1]), static_cast<float>(p[2]),
+                                     static_cast<float>(p[3]));
+                dst[1] = make_float4(static_cast<float>(p[4]), static_cast<float>(p[5]), static_cast<float>(p[6]),
+                                     static_cast<float>(p[7]));
+                tile.ds[ch][lane] = ds;
+            }
+            wave_lds_fence();
+#pragma unroll
+            for (int ch = 0; ch < CH; ++ch) {
+                const int base = base0 + 16 * ch;
+#pragma unroll
+                for (int s = 0; s < 16; ++s) {
+                    if (base + s < nb) {
+                        const float pv = tile.pf[ch][r4 * 136 + s * 8 + c];
+                        const float dv = tile.ds[ch][r4 * 16 + s];
+                        if (KIND == 1) {
+                            const int blk_i = base + s;
+                            if (blk_i < paired) {
+                                if (blk_i & 1)
+                                    acc_odd[i] = __builtin_fmaf(dv, pv, acc_odd[i]);
+                                else
+                                    acc[i] = __builtin_fmaf(dv, pv, acc[i]);
+                            }
+                        } else {
+                            acc[i] = __builtin_fmaf(dv, pv, acc[i]);
+                        }
+                    }
+                }
+                if (KIND == 1 && (nb & 1) && base < nb && base + 16 >= nb) {
+                    // trailing unpaired block: one rounded product with the whole-block integer sum
+                    // (every chunk value is an exact integer < 2^24), added after the closing tree
+                    const int s = (nb - 1) & 15;
+                    float tot = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) tot += tile.pf[ch][r4 * 136 + s * 8 + j];
+                    tail[i] = tile.ds[ch][r4 * 16 + s] * tot;
                 }
             }
         }
     }
-    if (KIND == 1) acc = acc + acc_odd;
-    float r = close_lanes8(acc);
-    if (KIND == 1 && (nb & 1)) {
-        // trailing block: one rounded product with the whole-block integer sum, added after the tree.
-        // The tile still holds the last pass; every chunk value is an exact integer < 2^24.
-        const int s = (nb - 1) & 15;
-        float tot = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) tot += tile.pf[r4 * 136 + s * 8 + j];
-        r = r + tile.ds[r4 * 16 + s] * tot;
+    for (int i = 0; i < NM; ++i) {
+        const float r = close_lanes8((KIND == 1) ? acc[i] + acc_odd[i] : acc[i]);
+        y[i] = (KIND == 1 && (nb & 1)) ? r + tail[i] : r;
     }
-    return r;
+}
+
+template <int KIND, bool PART>
+WD_DEV float q8_rows4(const uint8_t *rows, int nrows, int nb, const int8_t *act_qs, const uint16_t *act_d,
+                      Q8Tile &tile, int lane, int32_t *partials) {
+    const uint8_t *const rr[1] = {rows};
+    float y[1];
+    q8_rows4_multi<KIND, 1, 1, PART, NoPre>(rr, nrows, nb, act_qs, act_d, tile, lane, y, partials, 0);
+    return y[0];
+}
+
+// ---- Q8_0 x Q8_0, one row per wave ---------------------------------------------------------------------
+// For long rows (gate/up projections): lane b takes blocks b, b + 64, ...  The chunk sums of a pass
+// are handed over transposed ([chunk][block]) so that the chain lanes read them four at a time.
+struct Q8RowTile {
+    float pf[8][68];  // [c][block of the pass], rows padded to 68 floats (16-byte aligned, bank spread)
+    float ds[64];
+};
+
+// rows[i]: the row of matrix i.  y[i] valid in lane 0 (every aligned group of 8 lanes runs the same chain).
+template <int NM, typename Pre = NoPre>
+WD_DEV void q8_row_wave(const uint8_t *const (&rows)[NM], int nb, const int8_t *act_qs, const uint16_t *act_d,
+                        Q8RowTile &tile, int lane, float (&y)[NM], Pre pre = Pre()) {
+    const int c = lane & 7;
+    float acc[NM];
+#pragma unroll
+    for (int i = 0; i < NM; ++i) acc[i] = 0.0f;
+    for (int base = 0; base < nb; base += 64) {
+        const int bi = base + lane;
+        const bool on = bi < nb;
+        Q8Block wb[NM];
+        if (on) {
+#pragma unroll
+            for (int i = 0; i < NM; ++i) wb[i] = q8_load<0>(rows[i] + static_cast<size_t>(bi) * 34);
+        }
+        if (base == 0) pre();
+        uint32_t a[8];
+        float dx = 0.0f;
+        if (on) {
+            const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + bi * 32);
+            const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + bi * 32 + 16);
+            a[0] = a0.x, a[1] = a0.y, a[2] = a0.z, a[3] = a0.w, a[4] = a1.x, a[5] = a1.y, a[6] = a1.z, a[7] = a1.w;
+            dx = h2f(act_d[bi]);
+        }
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+            int p[8];
+            float ds = 0.0f;
+            if (on) {
+                q8_chunks<0>(wb[i], a, p);
+                ds = h2f(wb[i].d) * dx;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) p[j] = 0;
+            }
+            wave_lds_fence();  // earlier reads of the tile are done before it is overwritten
+#pragma unroll
+            for (int j = 0; j < 8; ++j) tile.pf[j][lane] = static_cast<float>(p[j]);
+            tile.ds[lane] = ds;
+            wave_lds_fence();
+            // blocks past the end of the row contribute fma(0, 0, acc) == acc
+#pragma unroll
+            for (int s4 = 0; s4 < 16; ++s4) {
+                const float4 pv = *reinterpret_cast<const float4 *>(&tile.pf[c][4 * s4]);
+                const float4 dv = *reinterpret_cast<const float4 *>(&tile.ds[4 * s4]);
+                acc[i] = __builtin_fmaf(dv.x, pv.x, acc[i]);
+                acc[i] = __builtin_fmaf(dv.y, pv.y, acc[i]);
+                acc[i] = __builtin_fmaf(dv.z, pv.z, acc[i]);
+                acc[i] = __builtin_fmaf(dv.w, pv.w, acc[i]);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NM; ++i) y[i] = close_lanes8(acc[i]);
 }
 
 // ---- dense Q4_0 x Q8_0 (src/warodecode.cu:1534-1562; no canonical float order) ------------
@@ -316,7 +496,7 @@ WD_DEV float q4_0_rows4(const uint8_t *rows, int nrows, int nb, const int8_t *ac
     if (r4 < nrows) {
         for (int bi = b; bi < nb; bi += 16) {
             const uint8_t *blk = row + static_cast<size_t>(bi) * 18;
-            const uint4 n = ldu<uint4>(blk + 2);
+            const uint4 n = gld_u128(blk + 2);
             const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + bi * 32);
             const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + bi * 32 + 16);
             const uint32_t w[4] = {n.x, n.y, n.z, n.w};
@@ -333,7 +513,7 @@ WD_DEV float q4_0_rows4(const uint8_t *rows, int nrows, int nb, const int8_t *ac
             }
             sumi -= 8 * asum;
             if (PART) partials[static_cast<size_t>(r4) * nb + bi] = sumi;
-            sumf += h2f(ldu<uint16_t>(blk)) * h2f(act_d[bi]) * static_cast<float>(sumi);
+            sumf += h2f(gld_u16(blk)) * h2f(act_d[bi]) * static_cast<float>(sumi);
         }
     }
 #pragma unroll
