@@ -1,0 +1,165 @@
+"""Expert-slot cache on the GPU: LRU semantics against a direct model of the reference rule
+(src/expert_cache.cuh:2252-2326, :2467-2493), device slot table contents, bytes in the slots, and a
+layer pass through the slot table that is bit-identical to the all-resident pass."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from warpdecode_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+SEED = 20261014
+
+
+@pytest.fixture(scope="module")
+def g():
+    import gpu_util
+    gpu_util.init()
+    return gpu_util
+
+
+class ModelCache:
+    """The reference rule, written the slow way: first empty slot, else smallest last_use."""
+
+    def __init__(self, n_slots, n_layers=1, partition=False):
+        self.slots = [None] * n_slots          # (key, last_use)
+        self.clock = 0
+        self.n_layers, self.partition = n_layers, partition and n_layers <= n_slots
+        self.hits = self.misses = self.evictions = 0
+
+    def bounds(self, layer):
+        n = len(self.slots)
+        if not self.partition:
+            return 0, n
+        per, rem = divmod(n, self.n_layers)
+        b = layer * per + min(layer, rem)
+        return b, b + per + (1 if layer < rem else 0)
+
+    def acquire(self, layer, expert):
+        key = (layer, expert)
+        self.clock += 1
+        for i, s in enumerate(self.slots):
+            if s is not None and s[0] == key:
+                self.slots[i] = (key, self.clock)
+                self.hits += 1
+                return i, True
+        self.misses += 1
+        b, e = self.bounds(layer)
+        empty = [i for i in range(b, e) if self.slots[i] is None]
+        if empty:
+            i = empty[0]
+        else:
+            i = min(range(b, e), key=lambda q: self.slots[q][1])
+            self.evictions += 1
+        self.slots[i] = (key, self.clock)
+        return i, False
+
+
+def _host_layers(n_layers, E, gb, ub, db, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(n_layers):
+        out.append([rng.integers(0, 256, E * gb, dtype=np.uint8), rng.integers(0, 256, E * ub, dtype=np.uint8),
+                    rng.integers(0, 256, E * db, dtype=np.uint8)])
+    return out
+
+
+@pytest.mark.parametrize("partition", [0, 1])
+def test_lru_semantics_and_contents(g, partition):
+    n_layers, E, k = 3, 24, 4
+    gb, ub, db = 256, 128, 64
+    n_slots = 17
+    host = _host_layers(n_layers, E, gb, ub, db, SEED)
+    cache = C.c_void_p()
+    capi.call("wd_expert_cache_create", C.byref(cache), n_slots * (gb + ub + db) + 5, gb, ub, db, n_layers, E, partition)
+    for l in range(n_layers):
+        capi.call("wd_expert_cache_register_layer", cache, l, *[h.ctypes.data_as(C.c_void_p) for h in host[l]])
+    model = ModelCache(n_slots, n_layers, bool(partition))
+    rng = np.random.default_rng(SEED + 1)
+    lib = capi.load()
+    pool = lib.wd_expert_cache_pool(cache)
+    for step in range(60):
+        layer = int(rng.integers(0, n_layers))
+        ids = rng.choice(E, size=k, replace=False, p=(lambda p: p / p.sum())(1.0 / np.arange(1, E + 1) ** 1.1)).astype(np.int32)
+        hits = np.zeros(k, np.uint8)
+        capi.call("wd_expert_cache_acquire", cache, layer, ids.ctypes.data_as(C.c_void_p), k,
+                  hits.ctypes.data_as(C.c_void_p), g.stream())
+        want = [model.acquire(layer, int(e)) for e in ids]
+        assert [bool(h) for h in hits] == [w[1] for w in want]
+        g.sync()
+        table = g.view(lib.wd_expert_cache_slot_table(cache, layer), E, np.int32)
+        for e, (slot, _) in zip(ids, want):
+            assert table[e] == slot
+            got = g.view(pool + slot * (gb + ub + db), gb + ub + db, np.uint8)
+            assert np.array_equal(got[:gb], host[layer][0][e * gb:(e + 1) * gb])
+            assert np.array_equal(got[gb:gb + ub], host[layer][1][e * ub:(e + 1) * ub])
+            assert np.array_equal(got[gb + ub:], host[layer][2][e * db:(e + 1) * db])
+        # every table entry agrees with the model, evicted experts read -1
+        for l in range(n_layers):
+            t = g.view(lib.wd_expert_cache_slot_table(cache, l), E, np.int32)
+            resident = {s[0][1]: i for i, s in enumerate(model.slots) if s is not None and s[0][0] == l}
+            for e in range(E):
+                assert t[e] == resident.get(e, -1)
+    st = capi.CacheStats()
+    capi.call("wd_expert_cache_get_stats", cache, C.byref(st))
+    assert (st.hits, st.misses, st.evictions) == (model.hits, model.misses, model.evictions)
+    assert st.accesses == 60 * k and st.bytes_copied == model.misses * (gb + ub + db)
+    assert st.slots == n_slots and st.resident == sum(s is not None for s in model.slots)
+    capi.call("wd_expert_cache_destroy", cache)
+
+
+def test_cache_errors(g):
+    cache = C.c_void_p()
+    lib = capi.load()
+    assert lib.wd_expert_cache_create(C.byref(cache), 100, 256, 128, 64, 1, 8, 0) == -1      # smaller than one slot
+    assert lib.wd_expert_cache_create(C.byref(cache), 0, 256, 128, 64, 1, 8, 0) == -1
+    capi.call("wd_expert_cache_create", C.byref(cache), 3 * 448, 256, 128, 64, 1, 8, 0)
+    ids = np.arange(4, dtype=np.int32)
+    assert lib.wd_expert_cache_acquire(cache, 0, ids.ctypes.data_as(C.c_void_p), 4, None, None) == -1   # unregistered
+    h = [np.zeros(8 * b, np.uint8) for b in (256, 128, 64)]
+    capi.call("wd_expert_cache_register_layer", cache, 0, *[x.ctypes.data_as(C.c_void_p) for x in h])
+    assert lib.wd_expert_cache_acquire(cache, 0, ids.ctypes.data_as(C.c_void_p), 4, None, None) == -1   # 3 slots < k
+    bad = np.array([0, 9], np.int32)
+    assert lib.wd_expert_cache_acquire(cache, 0, bad.ctypes.data_as(C.c_void_p), 2, None, None) == -1   # id range
+    capi.call("wd_expert_cache_destroy", cache)
+
+
+def test_layer_through_slot_table(g, oracle):
+    """A C2-shaped layer (fewer experts) whose routed tensors live only in the slot pool."""
+    L = synth.make_c2(n_experts=64)
+    H, F, E, k = 2048, 512, 64, 10
+    gb = F * synth.row_bytes(synth.IQ3_S, H)
+    db = H * synth.row_bytes(synth.Q8_0, F)
+    import torch
+    pinned = [torch.from_numpy(np.ascontiguousarray(L[n]).reshape(-1)).pin_memory() for n in ("gate", "up", "down")]
+    cache = C.c_void_p()
+    capi.call("wd_expert_cache_create", C.byref(cache), 24 * (2 * gb + db), gb, gb, db, 1, E, 0)
+    capi.call("wd_expert_cache_register_layer", cache, 0, *[C.c_void_p(t.data_ptr()) for t in pinned])
+    lib = capi.load()
+    dl = g.DeviceLayer(L)
+    d = dl.desc
+    d.gate = d.up = d.down = None
+    d.slot_of_expert = lib.wd_expert_cache_slot_table(cache, 0)
+    d.slot_pool = lib.wd_expert_cache_pool(cache)
+    d.slot_bytes, d.slot_gate_bytes, d.slot_up_bytes = 2 * gb + db, gb, gb
+    sc = g.Scratch(H, F, E, k)
+    rng = np.random.default_rng(SEED + 5)
+    for step in range(6):
+        x = synth.rms_normed(synth.rng_for(SEED, 61, step), H)
+        ids = rng.choice(E, size=k, replace=False).astype(np.int32)
+        wts = rng.uniform(0.05, 0.15, k).astype(np.float32)
+        capi.call("wd_expert_cache_acquire", cache, 0, ids.ctypes.data_as(C.c_void_p), k, None, g.stream())
+        capi.call("wd_memcpy_h2d", C.c_void_p(sc.raw("ids")), ids.ctypes.data_as(C.c_void_p), 4 * k, g.stream())
+        capi.call("wd_memcpy_h2d", C.c_void_p(sc.raw("weights")), wts.ctypes.data_as(C.c_void_p), 4 * k, g.stream())
+        dx, out = g.dev(x), g.empty(H, np.float32)
+        for flags in (capi.MOE_PRESELECTED, capi.MOE_PRESELECTED | capi.MOE_STAGED):
+            capi.call("wd_moe_layer_f32", C.byref(d), g.ptr(dx), g.ptr(out), sc.h, flags, g.stream())
+            g.sync()
+            want, _ = oracle.moe_layer(L, x, ids=ids, weights=wts)
+            assert g.same_bits(g.host(out), want), (step, flags)
+    st = capi.CacheStats()
+    capi.call("wd_expert_cache_get_stats", cache, C.byref(st))
+    assert st.misses > 24 and st.evictions > 0 and st.hits > 0
+    sc.close()
+    capi.call("wd_expert_cache_destroy", cache)

@@ -1,0 +1,123 @@
+"""M tokens through one layer (speculative-verify batch): every selected expert is read once for all
+tokens that routed to it, and each token's result is bit-identical to its own one-token pass and to
+the CPU oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from warpdecode_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+SEED = 20261014
+
+
+@pytest.fixture(scope="module")
+def g():
+    import gpu_util
+    gpu_util.init()
+    return gpu_util
+
+
+def correlated_tokens(H, T, seed, mix=0.6):
+    rng = synth.rng_for(SEED, 71, seed)
+    base = rng.normal(0, 1, H)
+    xs = []
+    for _ in range(T):
+        v = mix * base + (1 - mix) * rng.normal(0, 1, H)
+        xs.append((v / np.sqrt(np.mean(v ** 2))).astype(np.float32))
+    return np.stack(xs)
+
+
+def run_tokens(g, dl, L, xs, flags=0, ids=None, weights=None):
+    H, F, E, k = L["hidden"], L["expert_ffn"], L["n_experts"], L["top_k"]
+    T = xs.shape[0]
+    scs = [g.Scratch(H, F, E, k) for _ in range(T)]
+    if ids is not None:
+        for t in range(T):
+            capi.call("wd_memcpy_h2d", C.c_void_p(scs[t].raw("ids")), np.ascontiguousarray(ids[t], np.int32).ctypes.data_as(C.c_void_p), 4 * k, None)
+            capi.call("wd_memcpy_h2d", C.c_void_p(scs[t].raw("weights")), np.ascontiguousarray(weights[t], np.float32).ctypes.data_as(C.c_void_p), 4 * k, None)
+    arr = (C.c_void_p * T)(*[s.h for s in scs])
+    dx, out = g.dev(xs), g.empty((T, H), np.float32)
+    capi.call("wd_moe_layer_tokens_f32", C.byref(dl.desc), g.ptr(dx), g.ptr(out), T, arr, flags, g.stream())
+    g.sync()
+    res = dict(out=g.host(out), ids=np.stack([s.get("ids", k, np.int32) for s in scs]),
+               weights=np.stack([s.get("weights", k, np.float32) for s in scs]),
+               accum=np.stack([s.get("accum", H, np.float32) for s in scs]),
+               act=np.stack([s.get("act", (k + 1) * F, np.float32).reshape(k + 1, F) for s in scs]))
+    for s in scs:
+        s.close()
+    return res
+
+
+def run_single(g, dl, L, x, flags=0, ids=None, weights=None):
+    r = run_tokens(g, dl, L, x[None, :], flags, None if ids is None else ids[None], None if weights is None else weights[None])
+    return {n: v[0] for n, v in r.items()}
+
+
+@pytest.mark.parametrize("T", [1, 4, 8])
+def test_c4_tokens(g, oracle, T):
+    """Workload C4: T tokens through the 512-expert top-10 IQ3_S/Q8_0 layer with overlapping routing."""
+    L = synth.make_c2()
+    dl = g.DeviceLayer(L)
+    xs = correlated_tokens(2048, T, T)
+    got = run_tokens(g, dl, L, xs)
+    union = set(got["ids"].ravel().tolist())
+    if T == 4:
+        assert 10 < len(union) < 40        # the sets overlap but are not identical
+    for t in range(T):
+        want, d = oracle.moe_layer(L, xs[t])
+        assert np.array_equal(got["ids"][t], d["ids"])
+        assert g.same_bits(got["weights"][t], d["weights"])
+        assert g.same_bits(got["act"][t][:10], d["act"])
+        assert g.same_bits(got["accum"][t], d["routed"])
+        assert g.same_bits(got["out"][t], want)
+    one = run_tokens(g, dl, L, xs[:1])
+    assert g.same_bits(one["out"][0], got["out"][0])
+
+
+@pytest.mark.parametrize("gate_t,down_t,shared,H,F,E,k", [
+    (synth.IQ2_S, synth.Q8_0, True, 512, 64, 16, 4),
+    (synth.IQ3_S, synth.Q8_0, False, 768, 96, 8, 8),
+    (synth.Q8_0, synth.Q8_0, False, 512, 64, 8, 2),         # not on the union path: one pass per token
+    (synth.IQ3_S, synth.IQ4_NL, True, 512, 64, 8, 2),       # idem
+])
+def test_tokens_equal_single_passes(g, oracle, gate_t, down_t, shared, H, F, E, k):
+    L = synth.make_layer(H, F, E, k, gate_t, down_t, shared, seed=SEED, layer=7, router_sigma=1.0 / np.sqrt(H))
+    dl = g.DeviceLayer(L)
+    xs = correlated_tokens(H, 5, H)
+    got = run_tokens(g, dl, L, xs)
+    for t in range(5):
+        one = run_single(g, dl, L, xs[t])
+        assert np.array_equal(got["ids"][t], one["ids"])
+        assert g.same_bits(got["out"][t], one["out"]) and g.same_bits(got["accum"][t], one["accum"])
+        want, _ = oracle.moe_layer(L, xs[t])
+        assert g.same_bits(got["out"][t], want)
+
+
+def test_tokens_preselected_full_overlap(g, oracle):
+    """All tokens name the same experts in different orders: one union entry per expert."""
+    L = synth.make_c2(n_experts=32)
+    dl = g.DeviceLayer(L)
+    T, k = 4, 10
+    xs = correlated_tokens(2048, T, 3)
+    rng = np.random.default_rng(SEED)
+    base = rng.choice(32, size=k, replace=False)
+    ids = np.stack([rng.permutation(base) for _ in range(T)]).astype(np.int32)
+    wts = rng.uniform(0.05, 0.15, (T, k)).astype(np.float32)
+    got = run_tokens(g, dl, L, xs, flags=capi.MOE_PRESELECTED, ids=ids, weights=wts)
+    for t in range(T):
+        want, _ = oracle.moe_layer(L, xs[t], ids=ids[t], weights=wts[t])
+        assert g.same_bits(got["out"][t], want)
+
+
+def test_tokens_errors(g):
+    L = synth.make_layer(512, 64, 8, 2, synth.IQ3_S, synth.Q8_0, False)
+    dl = g.DeviceLayer(L)
+    sc = g.Scratch(512, 64, 8, 2)
+    arr = (C.c_void_p * 2)(sc.h, sc.h)
+    x = g.empty((2, 512), np.float32)
+    lib = capi.load()
+    assert lib.wd_moe_layer_tokens_f32(C.byref(dl.desc), g.ptr(x), g.ptr(x), 2, arr, 0, None) == -1   # shared scratch
+    assert lib.wd_moe_layer_tokens_f32(C.byref(dl.desc), g.ptr(x), g.ptr(x), 9, arr, 0, None) == -1
+    sc.close()

@@ -1,0 +1,273 @@
+// Expert-slot cache: an LRU pool of fixed-size slots in HBM fed from pinned host memory.
+//
+// Semantics follow the reference cache (src/expert_cache.cuh:2156-2536): key (layer << 32 | expert),
+// a hit refreshes last_use, a miss takes the lowest-numbered empty slot or else the slot with the
+// smallest last_use (inside the layer's partition when partitioning is on), the old key is dropped,
+// the slot is filled with gate | up | down at fixed offsets.  What differs is the machinery:
+//   * victim choice is O(1) (an intrusive list ordered by last_use and an ordered free list give
+//     the same victim as the reference's linear scan);
+//   * the kernels never see host pointers: every layer has a device table expert -> slot that the
+//     grouped GEMVs index with the routed ids, updated by a small kernel ordered on the caller's
+//     stream, so no pointer table is uploaded per layer;
+//   * fills are hipMemcpyAsync from pinned memory on a private copy stream: the copy stream waits
+//     for the work already queued on the caller's stream (which may still read the victim slot) and
+//     the caller's stream waits for the fills, so no host thread ever blocks.
+#include "wd_common.h"
+
+#include <list>
+#include <new>
+#include <unordered_map>
+#include <vector>
+
+using namespace wd;
+
+namespace {
+
+struct SlotUpdate {
+    int32_t index;  // position in the concatenated [layer][expert] table
+    int32_t value;  // slot number or -1
+};
+
+// One thread, in order: a batch may name the same table entry twice (evicted, then filled again).
+__global__ void k_apply_slot_updates(int32_t *table, const SlotUpdate *updates, int n) {
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+        for (int i = 0; i < n; ++i) table[updates[i].index] = updates[i].value;
+}
+
+__global__ void k_fill_i32(int32_t *dst, int32_t v, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = v;
+}
+
+struct Slot {
+    uint64_t key = 0;
+    uint64_t last_use = 0;
+    bool valid = false;
+    std::list<size_t>::iterator lru;  // position in its partition's list (valid slots only)
+};
+
+struct Partition {
+    size_t begin = 0, end = 0;
+    std::list<size_t> lru;       // front = least recently used
+    std::vector<size_t> free;    // empty slots, descending so that back() is the lowest index
+};
+
+constexpr int kUpdateRing = 32;
+constexpr int kMaxUpdates = 64;  // 2 per missed expert, k <= 16... one acquire call never needs more
+
+}  // namespace
+
+struct wd_expert_cache {
+    uint8_t *pool = nullptr;
+    size_t n_slots = 0, slot_bytes = 0, gate_bytes = 0, up_bytes = 0, down_bytes = 0;
+    int n_layers = 0, n_experts = 0;
+    bool partitioned = false;
+    std::vector<Slot> slots;
+    std::vector<Partition> parts;
+    std::unordered_map<uint64_t, size_t> index;
+    uint64_t clock = 0;
+    std::vector<const uint8_t *> h_gate, h_up, h_down;
+    int32_t *d_table = nullptr;  // [n_layers][n_experts]
+    hipStream_t copy_stream = nullptr;
+    hipEvent_t ev_retire = nullptr, ev_done = nullptr;
+    SlotUpdate *h_updates = nullptr;  // pinned ring [kUpdateRing][kMaxUpdates]
+    SlotUpdate *d_updates = nullptr;  // device ring of the same shape
+    hipEvent_t ring_free[kUpdateRing] = {};
+    bool ring_used[kUpdateRing] = {};
+    int ring_next = 0;
+    wd_expert_cache_stats stats{};
+};
+
+extern "C" {
+
+int wd_expert_cache_create(wd_expert_cache **out, size_t capacity_bytes, size_t gate_bytes, size_t up_bytes,
+                           size_t down_bytes, int n_layers, int n_experts, int layer_partition) {
+    WD_REQUIRE(out != nullptr, "expert cache: null output pointer");
+    WD_REQUIRE(capacity_bytes > 0, "expert cache capacity is zero");
+    WD_REQUIRE(gate_bytes > 0 && up_bytes > 0 && down_bytes > 0, "expert cache slot is empty");
+    WD_REQUIRE(n_layers > 0 && n_experts > 0, "expert cache: invalid layer/expert counts");
+    // every tensor of a slot starts 16-byte aligned so that rows keep the alignment they have in a GGUF file
+    WD_REQUIRE(gate_bytes % 16 == 0 && up_bytes % 16 == 0 && down_bytes % 16 == 0,
+               "expert cache: tensor slices must be multiples of 16 bytes");
+    const size_t slot_bytes = gate_bytes + up_bytes + down_bytes;
+    const size_t n_slots = capacity_bytes / slot_bytes;
+    WD_REQUIRE(n_slots > 0, "expert cache capacity is smaller than one expert slot");
+    wd_expert_cache *c = new (std::nothrow) wd_expert_cache;
+    WD_REQUIRE(c != nullptr, "expert cache: out of host memory");
+    c->n_slots = n_slots, c->slot_bytes = slot_bytes;
+    c->gate_bytes = gate_bytes, c->up_bytes = up_bytes, c->down_bytes = down_bytes;
+    c->n_layers = n_layers, c->n_experts = n_experts;
+    c->partitioned = layer_partition != 0 && static_cast<size_t>(n_layers) <= n_slots;
+    c->slots.resize(n_slots);
+    const int n_parts = c->partitioned ? n_layers : 1;
+    c->parts.resize(n_parts);
+    for (int p = 0; p < n_parts; ++p) {
+        // same split as the reference: n / layers slots each, the first n % layers partitions one more
+        const size_t per = n_slots / n_parts, rem = n_slots % n_parts;
+        Partition &P = c->parts[p];
+        P.begin = p * per + std::min<size_t>(p, rem);
+        P.end = P.begin + per + (static_cast<size_t>(p) < rem ? 1 : 0);
+        for (size_t s = P.end; s > P.begin; --s) P.free.push_back(s - 1);
+    }
+    c->h_gate.assign(n_layers, nullptr);
+    c->h_up.assign(n_layers, nullptr);
+    c->h_down.assign(n_layers, nullptr);
+    auto bail = [&](const char *what, hipError_t e) {
+        const int rc = fail(WD_ERR_HIP, "expert cache: %s failed: %s", what, hipGetErrorString(e));
+        wd_expert_cache_destroy(c);
+        return rc;
+    };
+    hipError_t e;
+    if ((e = hipMalloc(reinterpret_cast<void **>(&c->pool), n_slots * slot_bytes)) != hipSuccess) return bail("hipMalloc pool", e);
+    const size_t table_n = static_cast<size_t>(n_layers) * n_experts;
+    if ((e = hipMalloc(reinterpret_cast<void **>(&c->d_table), table_n * sizeof(int32_t))) != hipSuccess)
+        return bail("hipMalloc slot table", e);
+    k_fill_i32<<<dim3(static_cast<unsigned>((table_n + 255) / 256)), dim3(256)>>>(c->d_table, -1, table_n);
+    if ((e = hipDeviceSynchronize()) != hipSuccess) return bail("slot table fill", e);
+    if ((e = hipStreamCreateWithFlags(&c->copy_stream, hipStreamNonBlocking)) != hipSuccess) return bail("copy stream", e);
+    if ((e = hipEventCreateWithFlags(&c->ev_retire, hipEventDisableTiming)) != hipSuccess) return bail("event", e);
+    if ((e = hipEventCreateWithFlags(&c->ev_done, hipEventDisableTiming)) != hipSuccess) return bail("event", e);
+    if ((e = hipHostMalloc(reinterpret_cast<void **>(&c->h_updates), sizeof(SlotUpdate) * kUpdateRing * kMaxUpdates,
+                           hipHostMallocDefault)) != hipSuccess)
+        return bail("pinned update ring", e);
+    if ((e = hipMalloc(reinterpret_cast<void **>(&c->d_updates), sizeof(SlotUpdate) * kUpdateRing * kMaxUpdates)) != hipSuccess)
+        return bail("device update ring", e);
+    for (int i = 0; i < kUpdateRing; ++i)
+        if ((e = hipEventCreateWithFlags(&c->ring_free[i], hipEventDisableTiming)) != hipSuccess) return bail("ring event", e);
+    c->stats.slots = n_slots;
+    c->stats.slot_bytes = slot_bytes;
+    *out = c;
+    return WD_OK;
+}
+
+int wd_expert_cache_destroy(wd_expert_cache *c) {
+    if (!c) return WD_OK;
+    if (c->copy_stream) (void)hipStreamSynchronize(c->copy_stream);
+    (void)hipFree(c->pool);
+    (void)hipFree(c->d_table);
+    (void)hipFree(c->d_updates);
+    if (c->h_updates) (void)hipHostFree(c->h_updates);
+    if (c->ev_retire) (void)hipEventDestroy(c->ev_retire);
+    if (c->ev_done) (void)hipEventDestroy(c->ev_done);
+    for (int i = 0; i < kUpdateRing; ++i)
+        if (c->ring_free[i]) (void)hipEventDestroy(c->ring_free[i]);
+    if (c->copy_stream) (void)hipStreamDestroy(c->copy_stream);
+    delete c;
+    return WD_OK;
+}
+
+int wd_expert_cache_register_layer(wd_expert_cache *c, int layer, const uint8_t *h_gate, const uint8_t *h_up,
+                                   const uint8_t *h_down) {
+    WD_REQUIRE(c != nullptr, "expert cache is not initialized");
+    WD_REQUIRE(layer >= 0 && layer < c->n_layers, "expert cache: layer %d out of range", layer);
+    WD_REQUIRE(h_gate && h_up && h_down, "expert cache: null host tensor");
+    c->h_gate[layer] = h_gate, c->h_up[layer] = h_up, c->h_down[layer] = h_down;
+    return WD_OK;
+}
+
+int wd_expert_cache_acquire(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uint8_t *hit_out,
+                            void *stream) {
+    WD_REQUIRE(c != nullptr && c->pool != nullptr, "expert cache is not initialized");
+    WD_REQUIRE(layer >= 0 && layer < c->n_layers, "expert cache: layer %d out of range", layer);
+    WD_REQUIRE(h_ids != nullptr && k > 0 && 2 * k <= kMaxUpdates, "expert cache: invalid id list (k=%d)", k);
+    WD_REQUIRE(c->h_gate[layer] != nullptr, "expert cache: layer %d has no registered host tensors", layer);
+    Partition &P = c->parts[c->partitioned ? layer : 0];
+    WD_REQUIRE(P.end - P.begin >= static_cast<size_t>(k), "expert cache: %zu slots cannot hold %d experts at once",
+               P.end - P.begin, k);
+    hipStream_t st = as_stream(stream);
+    const uint64_t epoch_floor = c->clock;  // slots touched by this call carry last_use > epoch_floor
+    SlotUpdate updates[kMaxUpdates];
+    int n_updates = 0;
+    bool waited = false;
+
+    for (int j = 0; j < k; ++j) {
+        const int e = h_ids[j];
+        WD_REQUIRE(e >= 0 && e < c->n_experts, "expert index out of range: %d", e);
+        const uint64_t key = (static_cast<uint64_t>(static_cast<uint32_t>(layer)) << 32) | static_cast<uint32_t>(e);
+        ++c->clock;
+        ++c->stats.accesses;
+        auto it = c->index.find(key);
+        if (it != c->index.end()) {
+            Slot &s = c->slots[it->second];
+            s.last_use = c->clock;
+            Partition &Q = c->parts[c->partitioned ? static_cast<int>(s.key >> 32) : 0];
+            Q.lru.splice(Q.lru.end(), Q.lru, s.lru);  // most recently used goes to the back
+            ++c->stats.hits;
+            if (hit_out) hit_out[j] = 1;
+            continue;
+        }
+        ++c->stats.misses;
+        if (hit_out) hit_out[j] = 0;
+        size_t slot;
+        if (!P.free.empty()) {
+            slot = P.free.back();
+            P.free.pop_back();
+        } else {
+            slot = P.lru.front();
+            Slot &victim = c->slots[slot];
+            if (victim.last_use > epoch_floor)
+                return fail(WD_ERR_STATE, "expert cache: all slots are held by the current acquire call");
+            P.lru.pop_front();
+            c->index.erase(victim.key);
+            updates[n_updates++] = {static_cast<int32_t>((victim.key >> 32) * c->n_experts + (victim.key & 0xffffffffu)), -1};
+            ++c->stats.evictions;
+        }
+        Slot &s = c->slots[slot];
+        s.key = key, s.last_use = c->clock, s.valid = true;
+        P.lru.push_back(slot);
+        s.lru = std::prev(P.lru.end());
+        c->index[key] = slot;
+        updates[n_updates++] = {static_cast<int32_t>(layer * c->n_experts + e), static_cast<int32_t>(slot)};
+
+        if (!waited) {
+            // kernels already queued on the caller's stream may still read the victim slot
+            WD_HIP(hipEventRecord(c->ev_retire, st));
+            WD_HIP(hipStreamWaitEvent(c->copy_stream, c->ev_retire, 0));
+            waited = true;
+        }
+        uint8_t *dst = c->pool + slot * c->slot_bytes;
+        WD_HIP(hipMemcpyAsync(dst, c->h_gate[layer] + static_cast<size_t>(e) * c->gate_bytes, c->gate_bytes,
+                              hipMemcpyHostToDevice, c->copy_stream));
+        WD_HIP(hipMemcpyAsync(dst + c->gate_bytes, c->h_up[layer] + static_cast<size_t>(e) * c->up_bytes, c->up_bytes,
+                              hipMemcpyHostToDevice, c->copy_stream));
+        WD_HIP(hipMemcpyAsync(dst + c->gate_bytes + c->up_bytes, c->h_down[layer] + static_cast<size_t>(e) * c->down_bytes,
+                              c->down_bytes, hipMemcpyHostToDevice, c->copy_stream));
+        c->stats.bytes_copied += c->slot_bytes;
+    }
+    c->stats.resident = c->index.size();
+
+    if (n_updates > 0) {
+        const int r = c->ring_next;
+        c->ring_next = (r + 1) % kUpdateRing;
+        if (c->ring_used[r]) WD_HIP(hipEventSynchronize(c->ring_free[r]));  // the entry's last use has been consumed
+        SlotUpdate *h = c->h_updates + static_cast<size_t>(r) * kMaxUpdates;
+        SlotUpdate *d = c->d_updates + static_cast<size_t>(r) * kMaxUpdates;
+        for (int i = 0; i < n_updates; ++i) h[i] = updates[i];
+        WD_HIP(hipMemcpyAsync(d, h, sizeof(SlotUpdate) * n_updates, hipMemcpyHostToDevice, st));
+        k_apply_slot_updates<<<dim3(1), dim3(64), 0, st>>>(c->d_table, d, n_updates);
+        WD_LAUNCH_CHECK();
+        WD_HIP(hipEventRecord(c->ring_free[r], st));  // both copies of ring entry r are free after this point
+        c->ring_used[r] = true;
+    }
+    if (waited) {
+        WD_HIP(hipEventRecord(c->ev_done, c->copy_stream));
+        WD_HIP(hipStreamWaitEvent(st, c->ev_done, 0));
+    }
+    return WD_OK;
+}
+
+const int32_t *wd_expert_cache_slot_table(wd_expert_cache *c, int layer) {
+    if (!c || layer < 0 || layer >= c->n_layers) return nullptr;
+    return c->d_table + static_cast<size_t>(layer) * c->n_experts;
+}
+
+const uint8_t *wd_expert_cache_pool(wd_expert_cache *c) { return c ? c->pool : nullptr; }
+
+int wd_expert_cache_get_stats(wd_expert_cache *c, wd_expert_cache_stats *out) {
+    WD_REQUIRE(c != nullptr && out != nullptr, "expert cache stats: null pointer");
+    *out = c->stats;
+    out->resident = c->index.size();
+    return WD_OK;
+}
+
+}  // extern "C"

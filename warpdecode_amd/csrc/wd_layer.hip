@@ -1,7 +1,7 @@
 // Whole-layer entry points: scratch object and the staged layer pass (one launch per stage,
 // every stage a stand-alone operator of wd_ops.hip resolved against the device-side ids).
 #include "wd_common.h"
-#include "wd_fused.cuh"
+#include "wd_tokens.cuh"
 
 #include <new>
 
@@ -30,6 +30,7 @@ struct wd_moe_scratch {
     int32_t *dp = nullptr;
     int gup_type = -1, dp_type = -1;
     unsigned *arrive = nullptr;           // device counter used inside the fused dispatch A
+    int32_t *union_buf = nullptr;         // [1 + 128 + 128 * 8] expert union of a multi-token pass
     unsigned long long *trace = nullptr;  // device [3][16][8] time stamps, see wd_moe_scratch_trace
     int trace_wg = 0;
 };
@@ -68,7 +69,7 @@ int wd_moe_scratch_create(wd_moe_scratch **out, int hidden, int expert_ffn, int 
                  o_act = c.take(sizeof(float) * K1 * F), o_aq = c.take(K1 * F),
                  o_ad = c.take(sizeof(uint16_t) * K1 * (F / 32)), o_eo = c.take(sizeof(float) * K1 * H),
                  o_acc = c.take(sizeof(float) * H), o_dn = c.take(sizeof(float) * H), o_sg = c.take(256),
-                 o_arr = c.take(256);
+                 o_arr = c.take(256), o_uni = c.take(sizeof(int32_t) * (1 + 128 + 128 * kMaxTokens));
     const hipError_t e = hipMalloc(reinterpret_cast<void **>(&s->block), c.off);
     if (e != hipSuccess) {
         delete s;
@@ -92,6 +93,7 @@ int wd_moe_scratch_create(wd_moe_scratch **out, int hidden, int expert_ffn, int 
     s->down_f32 = reinterpret_cast<float *>(b + o_dn);
     s->shared_gate = reinterpret_cast<float *>(b + o_sg);
     s->arrive = reinterpret_cast<unsigned *>(b + o_arr);
+    s->union_buf = reinterpret_cast<int32_t *>(b + o_uni);
     (void)hipMemset(s->block, 0, c.off);
     *out = s;
     return WD_OK;
@@ -316,13 +318,11 @@ int layer_staged(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_s
     return WD_OK;
 }
 
-// One layer in three dispatches (router+shared gate/up, top-k+routed gate/up, down+combine).
-int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s, unsigned flags,
-                const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st) {
-    const int H = L->hidden, F = L->expert_ffn, E = L->n_experts, k = L->top_k;
+LayerArgs fused_args(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s, unsigned flags,
+                     const int32_t *ids_override, float *residual, float residual_scale) {
     const bool shared = L->shared_gate_inp != nullptr;
     LayerArgs a{};
-    a.H = H, a.F = F, a.E = E, a.k = k;
+    a.H = L->hidden, a.F = L->expert_ffn, a.E = L->n_experts, a.k = L->top_k;
     a.w_scale = L->expert_scale;
     a.x = d_x;
     a.router = L->router;
@@ -338,16 +338,30 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
     a.accum = s->accum, a.down_f32 = s->down_f32, a.out = d_out;
     a.residual = residual, a.residual_scale = residual_scale;
     a.preselected = (flags & WD_MOE_PRESELECTED) ? 1 : 0;
-    const int router_rows_n = (a.preselected ? 0 : E) + (shared ? 1 : 0);
+    const int router_rows_n = (a.preselected ? 0 : a.E) + (shared ? 1 : 0);
     a.n_router_wgs = (router_rows_n + 15) / 16;
     a.trace = s->trace, a.trace_wg = s->trace_wg;
     a.arrive = s->arrive;
+    return a;
+}
 
-    const int grid_a = a.n_router_wgs + (shared ? (F + 7) / 8 : 0);
+// Dispatch A: router logits (+ selection by the last router workgroup) and the shared expert's gate/up.
+int launch_a(const LayerArgs &a, hipStream_t st) {
+    const int grid_a = a.n_router_wgs + (a.sh_inp ? (a.F + 7) / 8 : 0);
     if (grid_a > 0) {
-        k_layer_a<<<dim3(grid_a), dim3(512), static_cast<size_t>(H) + H / 16, st>>>(a);
+        k_layer_a<<<dim3(grid_a), dim3(512), static_cast<size_t>(a.H) + a.H / 16, st>>>(a);
         WD_LAUNCH_CHECK();
     }
+    return WD_OK;
+}
+
+// One layer in three dispatches (router + shared gate/up, routed gate/up, down + combine).
+int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s, unsigned flags,
+                const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st) {
+    const int H = L->hidden, F = L->expert_ffn, k = L->top_k;
+    const bool shared = L->shared_gate_inp != nullptr;
+    const LayerArgs a = fused_args(L, d_x, d_out, s, flags, ids_override, residual, residual_scale);
+    if (const int rc = launch_a(a, st)) return rc;
     const bool iq = consumes_q8k(L->gate_type);
     const size_t lds_b = H + (iq ? sizeof(float) * (H / 256) : sizeof(uint16_t) * (H / 32));
     const int grid_b = k * (L->gate_type == WD_TYPE_IQ4_NL ? (F + 15) / 16 : (F + 7) / 8);
@@ -402,5 +416,61 @@ extern "C" int wd_moe_stack_f32(const wd_moe_layer *layers, int n_layers, float 
         if (const int rc = layer_dispatch(&layers[l], d_x, d_layer_out, s, flags, trace, d_x, residual_scale, as_stream(stream)))
             return rc;
     }
+    return WD_OK;
+}
+
+extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, float *d_out, int tokens,
+                                       wd_moe_scratch *const *scratch_per_token, unsigned flags, void *stream) {
+    WD_REQUIRE(tokens > 0 && tokens <= kMaxTokens, "multi-token pass: 1..%d tokens (got %d)", kMaxTokens, tokens);
+    WD_REQUIRE(scratch_per_token != nullptr && d_x && d_out, "multi-token pass: null pointer");
+    for (int t = 0; t < tokens; ++t) {
+        WD_REQUIRE(scratch_per_token[t] != nullptr, "multi-token pass: null scratch for token %d", t);
+        for (int q = 0; q < t; ++q)
+            WD_REQUIRE(scratch_per_token[q] != scratch_per_token[t], "multi-token pass: tokens %d and %d share a scratch", q, t);
+        if (const int rc = check_layer(L, scratch_per_token[t])) return rc;
+    }
+    hipStream_t st = as_stream(stream);
+    const int H = L->hidden, F = L->expert_ffn, k = L->top_k;
+    const bool union_path = !(flags & WD_MOE_STAGED) && consumes_q8k(L->gate_type) && L->down_type == WD_TYPE_Q8_0 &&
+                            F <= 512 && tokens * k <= 128 && scratch_per_token[0]->gup == nullptr;
+    if (!union_path) {
+        // same results, one pass per token (every pass reads its own experts)
+        for (int t = 0; t < tokens; ++t)
+            if (const int rc = layer_dispatch(L, d_x + static_cast<size_t>(t) * H, d_out + static_cast<size_t>(t) * H,
+                                              scratch_per_token[t], flags, nullptr, nullptr, 0.0f, st))
+                return rc;
+        return WD_OK;
+    }
+    TokenArgs ta{};
+    ta.T = tokens, ta.H = H, ta.F = F, ta.k = k;
+    for (int t = 0; t < tokens; ++t) {
+        wd_moe_scratch *s = scratch_per_token[t];
+        const LayerArgs a = fused_args(L, d_x + static_cast<size_t>(t) * H, d_out + static_cast<size_t>(t) * H, s, flags,
+                                       nullptr, nullptr, 0.0f);
+        if (const int rc = launch_a(a, st)) return rc;  // router, selection, shared gate/up of token t
+        ta.x[t] = a.x, ta.ids[t] = s->ids, ta.weights[t] = s->weights, ta.act[t] = s->act;
+        ta.shared_gate[t] = s->shared_gate;
+        ta.expert_out[t] = (flags & WD_MOE_KEEP_EXPERT_OUT) ? s->expert_out : nullptr;
+        ta.accum[t] = s->accum, ta.down_f32[t] = s->down_f32, ta.out[t] = a.out;
+    }
+    ta.gate_up = routed_src(L, nullptr, false);
+    ta.down = routed_src(L, nullptr, true);
+    ta.sh_down = L->shared_gate_inp ? L->shared_down : nullptr;
+    int32_t *ub = scratch_per_token[0]->union_buf;
+    ta.union_count = ub, ta.union_ids = ub + 1, ta.union_slot = ub + 1 + 128;
+    k_tokens_union<<<dim3(1), dim3(64), 0, st>>>(ta);
+    WD_LAUNCH_CHECK();
+    const size_t lds_b = static_cast<size_t>(tokens) * (H + sizeof(float) * (H / 256));
+    const int grid_b = tokens * k * ((F + 7) / 8);
+    if (L->gate_type == WD_TYPE_IQ3_S)
+        k_tokens_b<21><<<dim3(grid_b), dim3(512), lds_b, st>>>(ta);
+    else
+        k_tokens_b<22><<<dim3(grid_b), dim3(512), lds_b, st>>>(ta);
+    WD_LAUNCH_CHECK();
+    const int waves_c = 16;
+    const size_t per_wave = (static_cast<size_t>(F) + F / 16 + 15) & ~static_cast<size_t>(15);
+    const size_t lds_c = waves_c * per_wave + sizeof(float) * 4 * tokens * (k + 1);
+    k_tokens_c<<<dim3((H + 3) / 4), dim3(64 * waves_c), lds_c, st>>>(ta);
+    WD_LAUNCH_CHECK();
     return WD_OK;
 }

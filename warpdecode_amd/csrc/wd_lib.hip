@@ -1,3 +1,4 @@
 // Single translation unit of libwarpdecode_amd.so.
 #include "wd_ops.hip"
 #include "wd_layer.hip"
+#include "wd_cache.hip"
