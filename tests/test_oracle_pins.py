@@ -394,9 +394,10 @@ def test_layer_equals_reference_run_layer(refcpu, gate_t, down_t):
     L = _small_layer(gate_t, down_t, shared=False)
     x = synth.rms_normed(synth.rng_for(SEED, 5), L["hidden"])
     out, dump = refcpu.moe_layer(L, x)
-    for threads in (1, 4):
-        ref = refcpu.ref_run_layer(L, x, dump["ids"], dump["weights"], threads=threads)
-        assert np.array_equal(bits(out), bits(ref))
+    # one thread only: the reference's fork-join pool can hand a late worker a task of the next
+    # parallel_for (stale function pointer) and then never finishes; its arithmetic is what is pinned
+    ref = refcpu.ref_run_layer(L, x, dump["ids"], dump["weights"], threads=1)
+    assert np.array_equal(bits(out), bits(ref))
     out_mt, _ = refcpu.moe_layer(L, x, threads=4)
     assert np.array_equal(bits(out), bits(out_mt))
 
