@@ -143,7 +143,7 @@ def cpu_baseline(seconds):
     kinds = (["reference"] if pyoracle.ref() is not None else []) + ["port"]
     for kind in kinds:
         tot_passes, tot_time, stalls = 0, 0.0, 0
-        for attempt in range(8):
+        for attempt in range(40):
             remaining = seconds - tot_time
             if remaining <= 0.5:
                 break
@@ -181,6 +181,20 @@ def cpu_baseline(seconds):
                                   ("; the reference thread pool dead-locked %d times, each time the child was "
                                    "restarted and only completed passes are counted" % stalls) if stalls else ""))
     return dict(value=None, unit="tok/s", cores=threads, kind="port", sample="no CPU pass completed")
+
+
+def recorded_traffic(kernel):
+    """HBM bytes per launch of `kernel` as recorded from hardware-counter runs of this command (the file
+    says how they were taken and scaled); None when no record exists for this kernel."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_c3_mode_a.txt")
+    try:
+        for line in open(path):
+            f = line.split()
+            if len(f) >= 3 and f[0] == "traffic_bytes" and f[1] == kernel:
+                return int(f[2])
+    except OSError:
+        pass
+    return None
 
 
 def main():
@@ -274,15 +288,68 @@ def main():
     finite = bool(torch.isfinite(d_x).all().item())
     note("timed region done: %.3f ms/step" % ms_per_step)
 
-    bytes_per_layer = 27697152 if E == 512 else None
-    if bytes_per_layer is None:
-        bytes_per_layer = E * H * 4 + k * (2 * F * synth.row_bytes(synth.IQ3_S, H) + H * synth.row_bytes(synth.Q8_0, F)) \
-            + 2 * F * synth.row_bytes(synth.Q8_0, H) + H * synth.row_bytes(synth.Q8_0, F) + H * 4
+    # Algorithmic bytes of the three dispatches of one layer (weights only, as the workload prices them):
+    #   A  router f32 [E][H] + the shared expert's gate vector + its Q8_0 gate and up matrices
+    #   B  gate and up (IQ3_S) of the k selected experts
+    #   C  down (Q8_0) of the k selected experts and of the shared expert
+    q8h, q8f, iq3h = synth.row_bytes(synth.Q8_0, H), synth.row_bytes(synth.Q8_0, F), synth.row_bytes(synth.IQ3_S, H)
+    alg = {"k_layer_a": E * H * 4 + H * 4 + 2 * F * q8h, "k_layer_b": k * 2 * F * iq3h, "k_layer_c": (k + 1) * H * q8f}
+    bytes_per_layer = sum(alg.values())
+    assert E != 512 or bytes_per_layer == 27697152
     bytes_per_step = bytes_per_layer * NL
-    achieved = bytes_per_step / (ms_per_step * 1e-3) / 1e9
-    roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
-                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None,
-                    kernel="whole step (all launches of one token), %d B algorithmic per step" % bytes_per_step)
+
+    # Per-kernel launch time, live: the stack is replayed with one dispatch per layer only (the other two
+    # left out), so the timed region is a chain of NL launches of that one kernel over NL layers' weights.
+    # HIP events on the launch stream bracket `reps` replays; the period includes the gap between two
+    # dependent launches on a stream (about 1.5 us in a graph), which a profiler's begin-to-end time omits.
+    only = {"k_layer_a": 0x10, "k_layer_b": 0x20, "k_layer_c": 0x40}
+    per_kernel, reps = {}, 20
+    step(0)
+    for name, flag in only.items():
+        def chain():
+            capi.call("wd_moe_stack_f32", layers, NL, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()), scratch,
+                      trace_ptr, RESIDUAL_SCALE, flag, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            chain()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        runner = chain
+        if graph is not None:
+            g1 = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g1):
+                chain()
+            runner = g1.replay
+        for _ in range(3):
+            runner()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            runner()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (reps * NL)
+        per_kernel[name] = dict(us_per_launch=round(us, 3), bytes_per_launch=alg[name],
+                                achieved=round(alg[name] / (us * 1e-6) / 1e9, 1))
+    dominant = max(per_kernel, key=lambda n: per_kernel[n]["us_per_launch"])
+    note("per-kernel launch periods: %s; dominant: %s" % (per_kernel, dominant))
+    traffic = recorded_traffic(dominant)
+    dom = per_kernel[dominant]
+    whole = bytes_per_step / (ms_per_step * 1e-3) / 1e9
+    roofline = dict(bound="hbm", achieved=dom["achieved"], peak=HBM_PEAK_GBS, unit="GB/s",
+                    frac=round(dom["achieved"] / HBM_PEAK_GBS, 4), traffic=traffic,
+                    kernel=dominant, us_per_launch=dom["us_per_launch"], bytes_per_launch=dom["bytes_per_launch"],
+                    kernels=per_kernel,
+                    whole_step=dict(achieved=round(whole, 1), frac=round(whole / HBM_PEAK_GBS, 4),
+                                    bytes_per_step=bytes_per_step))
+
+    # A plain copy of known size, so that a counter run of this command can scale FETCH_SIZE / WRITE_SIZE.
+    cal_src = torch.empty(64 << 20, dtype=torch.float32, device="cuda").normal_()
+    cal_dst = torch.empty_like(cal_src)
+    cal_dst.copy_(cal_src)
+    torch.cuda.synchronize()
+    del cal_src, cal_dst
 
     out = {
         "metric": "MoE layer batch=1 decode: synthetic 48-layer tok/s (achieved HBM GB/s in roofline)",

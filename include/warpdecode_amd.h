@@ -179,6 +179,11 @@ unsigned long long *wd_moe_scratch_trace(wd_moe_scratch *s, int wg);
 #define WD_MOE_PRESELECTED 1u      /* ids/weights already in scratch: skip the router (reference `preselected`) */
 #define WD_MOE_KEEP_EXPERT_OUT 2u  /* also store the per-expert down outputs in scratch */
 #define WD_MOE_STAGED 4u           /* one dispatch per stage (the operators above) instead of the fused kernels */
+/* Measurement aids for the fused path: run only the named dispatch(es) of a layer.  The scratch must hold
+ * the results of the dispatches left out (run the whole layer once first). */
+#define WD_MOE_ONLY_A 0x10u /* router + selection + shared gate/up */
+#define WD_MOE_ONLY_B 0x20u /* routed gate/up + SwiGLU */
+#define WD_MOE_ONLY_C 0x40u /* down projections + combine */
 
 /* One decode step of one layer: router -> top-k -> grouped gate/up -> SwiGLU -> Q8_0 ->
  * grouped down -> ordered weighted sum -> + shared * sigmoid gate.  d_out is f32 [hidden]

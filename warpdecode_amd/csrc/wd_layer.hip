@@ -361,18 +361,24 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
     const int H = L->hidden, F = L->expert_ffn, k = L->top_k;
     const bool shared = L->shared_gate_inp != nullptr;
     const LayerArgs a = fused_args(L, d_x, d_out, s, flags, ids_override, residual, residual_scale);
-    if (const int rc = launch_a(a, st)) return rc;
+    const unsigned only = flags & (WD_MOE_ONLY_A | WD_MOE_ONLY_B | WD_MOE_ONLY_C);
+    if (!only || (only & WD_MOE_ONLY_A)) {
+        if (const int rc = launch_a(a, st)) return rc;
+    }
     const bool iq = consumes_q8k(L->gate_type);
     const size_t lds_b = H + (iq ? sizeof(float) * (H / 256) : sizeof(uint16_t) * (H / 32));
     const int grid_b = k * (L->gate_type == WD_TYPE_IQ4_NL ? (F + 15) / 16 : (F + 7) / 8);
-    switch (L->gate_type) {
-        case WD_TYPE_IQ3_S: k_layer_b<21><<<dim3(grid_b), dim3(512), lds_b, st>>>(a); break;
-        case WD_TYPE_IQ2_S: k_layer_b<22><<<dim3(grid_b), dim3(512), lds_b, st>>>(a); break;
-        case WD_TYPE_Q8_0: k_layer_b<8><<<dim3(grid_b), dim3(512), lds_b, st>>>(a); break;
-        case WD_TYPE_IQ4_NL: k_layer_b<20><<<dim3(grid_b), dim3(256), lds_b, st>>>(a); break;
-        default: return fail(WD_ERR_UNSUPPORTED, "fused layer: unsupported gate/up type %d", L->gate_type);
+    if (!only || (only & WD_MOE_ONLY_B)) {
+        switch (L->gate_type) {
+            case WD_TYPE_IQ3_S: k_layer_b<21><<<dim3(grid_b), dim3(512), lds_b, st>>>(a); break;
+            case WD_TYPE_IQ2_S: k_layer_b<22><<<dim3(grid_b), dim3(512), lds_b, st>>>(a); break;
+            case WD_TYPE_Q8_0: k_layer_b<8><<<dim3(grid_b), dim3(512), lds_b, st>>>(a); break;
+            case WD_TYPE_IQ4_NL: k_layer_b<20><<<dim3(grid_b), dim3(256), lds_b, st>>>(a); break;
+            default: return fail(WD_ERR_UNSUPPORTED, "fused layer: unsupported gate/up type %d", L->gate_type);
+        }
+        WD_LAUNCH_CHECK();
     }
-    WD_LAUNCH_CHECK();
+    if (only && !(only & WD_MOE_ONLY_C)) return WD_OK;
     const int n_act = k + (shared ? 1 : 0);
     const int waves_c = n_act < 16 ? n_act : 16;
     const size_t per_wave = (static_cast<size_t>(F) + F / 16 + 15) & ~static_cast<size_t>(15);
