@@ -58,6 +58,7 @@ int wd_malloc_host(void **h_ptr, size_t bytes);   /* pinned */
 int wd_free_host(void *h_ptr);
 int wd_memcpy_h2d(void *d_dst, const void *h_src, size_t bytes, void *stream); /* async when stream != NULL */
 int wd_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream);
+int wd_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes, void *stream);
 int wd_memset(void *d_dst, int value, size_t bytes, void *stream);
 int wd_stream_create(void **stream);
 int wd_stream_destroy(void *stream);
@@ -194,6 +195,14 @@ unsigned long long *wd_moe_scratch_trace(wd_moe_scratch *s, int wg);
 int wd_moe_layer_f32(const wd_moe_layer *layer, const float *d_x, float *d_out, wd_moe_scratch *scratch,
                      unsigned flags, void *stream);
 
+/* The shared expert alone: sigmoid(shared_gate_inp . x) into the scratch's shared_gate view and the Q8_0
+ * gate/up -> SwiGLU -> Q8_0 -> down chain into its down_f32 view; only the shared_* fields, hidden and
+ * expert_ffn of `layer` are read.  For callers that keep the reference's three calls (routed, shared,
+ * finish); wd_moe_layer_f32 does all three in its fused dispatches.
+ * reference: run_qwen38_shared_expert_f32_x (src/qwen38_moe.cuh:3963-3969),
+ *   q38_moe_run_shared_expert_f32_input (:3915-3948). */
+int wd_shared_expert_f32(const wd_moe_layer *layer, const float *d_x, wd_moe_scratch *scratch, void *stream);
+
 /* One decode step through a stack of layers: for each layer, x += residual_scale * layer(x) (the scaled
  * residual add stands in for the caller's own glue between two MoE blocks).  d_layer_out f32 [hidden] receives the last
  * layer's output.  d_ids_trace (device int32 [n_layers][top_k], may be NULL) replays a routing trace:
@@ -234,6 +243,9 @@ int wd_expert_cache_acquire(wd_expert_cache *c, int layer, const int32_t *h_ids,
                             void *stream);
 const int32_t *wd_expert_cache_slot_table(wd_expert_cache *c, int layer); /* device int32 [n_experts] */
 const uint8_t *wd_expert_cache_pool(wd_expert_cache *c);
+/* Host-side index: slot that holds (layer, expert) now, or -1 (reference: the `slot` of
+ * ExpertDeviceWeights, src/expert_cache.cuh:2148-2154). */
+long long wd_expert_cache_slot_of(wd_expert_cache *c, int layer, int expert);
 int wd_expert_cache_get_stats(wd_expert_cache *c, wd_expert_cache_stats *out);
 
 #ifdef __cplusplus

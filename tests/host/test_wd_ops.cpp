@@ -1,0 +1,276 @@
+// Host-side test of the C++ operator surface (warpdecode_amd/host/wd_ops.hpp): a caller written in the
+// style of the reference's own layer driver (routed experts, shared expert, finish;
+// src/qwen38_forward.cuh:3330-3371) runs against the library and every result is compared bit for
+// bit with the CPU oracle.  `--host-only` runs the checks that need no GPU (geometry errors, sizes).
+//
+// Built by warpdecode_amd/build.py (build_host_test) with g++ against libwarpdecode_amd.so and the oracle.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <functional>
+#include <random>
+
+#include "wd_ops.hpp"
+#include "wd_oracle.h"
+
+using namespace wd;
+
+static int g_checks = 0, g_fail = 0;
+#define CHECK(cond, ...)                          \
+    do {                                          \
+        ++g_checks;                               \
+        if (!(cond)) {                            \
+            ++g_fail;                             \
+            std::printf("FAIL %s:%d: ", __FILE__, __LINE__); \
+            std::printf(__VA_ARGS__);             \
+            std::printf("\n");                    \
+        }                                         \
+    } while (0)
+
+static bool throws(const std::function<void()> &f) {
+    try {
+        f();
+    } catch (const std::runtime_error &) {
+        return true;
+    }
+    return false;
+}
+
+static bool same_bits(const float *a, const float *b, size_t n) { return std::memcmp(a, b, n * sizeof(float)) == 0; }
+
+struct Rng {
+    std::mt19937_64 g;
+    explicit Rng(uint64_t s) : g(s) {}
+    uint32_t u32() { return static_cast<uint32_t>(g()); }
+    float normal() {
+        const double u1 = (static_cast<double>(g() >> 11) + 1.0) / 9007199254740993.0, u2 = static_cast<double>(g() >> 11) / 9007199254740992.0;
+        return static_cast<float>(std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586 * u2));
+    }
+};
+
+// Random GGUF block bytes with a sane fp16 scale at the head of every block.
+static std::vector<uint8_t> random_blocks(Rng &r, int type, size_t rows, int cols, float scale) {
+    const size_t bb = wdo_block_bytes(type), nb = rows * (cols / wdo_block_elems(type));
+    std::vector<uint8_t> w(nb * bb);
+    for (auto &b : w) b = static_cast<uint8_t>(r.u32());
+    for (size_t i = 0; i < nb; ++i) {
+        const uint16_t d = wdo_f32_to_f16(std::fabs(r.normal()) * scale);
+        std::memcpy(&w[i * bb], &d, 2);
+        if (type == WDO_Q8_0)
+            for (size_t j = 2; j < bb; ++j)
+                if (w[i * bb + j] == 0x80) w[i * bb + j] = 0x81;  // int8 quants in [-127, 127]
+    }
+    return w;
+}
+
+struct HostLayer {
+    int H, F, E, k;
+    std::vector<float> router, gate_inp;
+    std::vector<uint8_t> gate, up, down, sg, su, sd;
+    TensorInfo t_router, t_gate, t_up, t_down;
+    wdo_layer o{};
+};
+
+static HostLayer make_layer(uint64_t seed, int H, int F, int E, int k) {
+    HostLayer L;
+    L.H = H, L.F = F, L.E = E, L.k = k;
+    Rng r(seed);
+    L.router.resize(static_cast<size_t>(E) * H);
+    for (auto &v : L.router) v = r.normal() / std::sqrt(static_cast<float>(H));
+    L.gate_inp.resize(H);
+    for (auto &v : L.gate_inp) v = r.normal() * 0.02f;
+    L.gate = random_blocks(r, WDO_IQ3_S, static_cast<size_t>(E) * F, H, 0.01f);
+    L.up = random_blocks(r, WDO_IQ3_S, static_cast<size_t>(E) * F, H, 0.01f);
+    L.down = random_blocks(r, WDO_Q8_0, static_cast<size_t>(E) * H, F, 0.02f / 127.0f);
+    L.sg = random_blocks(r, WDO_Q8_0, F, H, 0.02f / 127.0f);
+    L.su = random_blocks(r, WDO_Q8_0, F, H, 0.02f / 127.0f);
+    L.sd = random_blocks(r, WDO_Q8_0, H, F, 0.02f / 127.0f);
+    L.t_router = {"ffn_gate_inp.weight", {static_cast<uint64_t>(H), static_cast<uint64_t>(E)}, GgmlType::F32, 0, reinterpret_cast<const uint8_t *>(L.router.data())};
+    L.t_gate = {"ffn_gate_exps.weight", {static_cast<uint64_t>(H), static_cast<uint64_t>(F), static_cast<uint64_t>(E)}, GgmlType::IQ3_S, 0, L.gate.data()};
+    L.t_up = {"ffn_up_exps.weight", {static_cast<uint64_t>(H), static_cast<uint64_t>(F), static_cast<uint64_t>(E)}, GgmlType::IQ3_S, 0, L.up.data()};
+    L.t_down = {"ffn_down_exps.weight", {static_cast<uint64_t>(F), static_cast<uint64_t>(H), static_cast<uint64_t>(E)}, GgmlType::Q8_0, 0, L.down.data()};
+    L.o.hidden = H, L.o.expert_ffn = F, L.o.n_experts = E, L.o.top_k = k, L.o.w_scale = 1.0f;
+    L.o.router = L.router.data();
+    L.o.gate_type = L.o.up_type = WDO_IQ3_S, L.o.down_type = WDO_Q8_0;
+    L.o.gate = L.gate.data(), L.o.up = L.up.data(), L.o.down = L.down.data();
+    L.o.shared_gate_inp = L.gate_inp.data(), L.o.shared_type = WDO_Q8_0;
+    L.o.shared_gate = L.sg.data(), L.o.shared_up = L.su.data(), L.o.shared_down = L.sd.data();
+    return L;
+}
+
+static std::vector<float> rms_normed(Rng &r, int n) {
+    std::vector<float> x(n);
+    double ss = 0;
+    for (auto &v : x) v = r.normal(), ss += static_cast<double>(v) * v;
+    const float inv = static_cast<float>(1.0 / std::sqrt(ss / n));
+    for (auto &v : x) v *= inv;
+    return x;
+}
+
+static void host_only_checks() {
+    TensorInfo t{"w", {256, 4}, GgmlType::IQ3_S, 0, nullptr};
+    CHECK(t.byte_size() == 4 * 110, "IQ3_S [4][256] is %zu bytes", t.byte_size());
+    t.type = GgmlType::Q8_0;
+    CHECK(t.byte_size() == 4 * 8 * 34, "Q8_0 [4][256] is %zu bytes", t.byte_size());
+    t.dims = {100, 4};
+    CHECK(throws([&] { t.byte_size(); }), "a ragged block count must throw");
+    TensorInfo one{"w", {256}, GgmlType::IQ3_S, 0, nullptr};
+    CHECK(throws([&] { upload_lowbit_matrix(one); }), "1-D tensor must be refused");
+    TensorInfo f32{"w", {256, 4}, GgmlType::F32, 0, nullptr};
+    CHECK(throws([&] { upload_lowbit_matrix(f32); }), "F32 tensor is not a low-bit matrix");
+    TensorInfo bad{"w", {288, 4}, GgmlType::IQ3_S, 0, nullptr};
+    CHECK(throws([&] { upload_lowbit_matrix(bad); }), "IQ3_S needs columns in multiples of 256");
+    TensorInfo two{"w", {256, 4}, GgmlType::IQ3_S, 0, nullptr};
+    CHECK(throws([&] { expert_slice(two, 0); }), "expert tensors are 3-D");
+    TensorInfo three{"w", {256, 4, 2}, GgmlType::IQ3_S, 0, nullptr};
+    CHECK(throws([&] { expert_slice(three, 2); }), "expert index out of range");
+    CHECK(expert_slice(three, 1).bytes == 440 && expert_slice(three, 1).data == static_cast<const uint8_t *>(nullptr) + 440, "slice offset");
+    Qwen38MoeScratch s;
+    CHECK(throws([&] { s.initialize(8, 17, 256, 32); }), "k > 16 must be refused");
+    CHECK(throws([&] { s.initialize(8, 9, 256, 32); }), "k > n_experts must be refused");
+    GpuExpertCache c;
+    CHECK(throws([&] { c.initialize(0, three, three, three); }), "zero capacity must be refused");
+    CHECK(throws([&] { c.acquire(0, 0, three, three, three, nullptr); }), "acquire before initialize must throw");
+    LowBitMatrix b = borrow_lowbit_matrix(reinterpret_cast<uint8_t *>(0x1000), 4, 256, GgmlType::IQ3_S, 440);
+    LowBitMatrix m = std::move(b);
+    CHECK(m.data == reinterpret_cast<uint8_t *>(0x1000) && !m.owns && b.data == nullptr, "move keeps the borrowed view");
+    GpuMatrix g;
+    CHECK(throws([&] { launch_q38_router_gemv_f32(g, nullptr, nullptr, nullptr); }), "router without F32 weights must throw");
+    LowBitMatrix q = borrow_lowbit_matrix(reinterpret_cast<uint8_t *>(0x1000), 4, 256, GgmlType::Q8_0, 4 * 8 * 34);
+    CHECK(throws([&] { launch_iq3_s_gemv_q8_k_f32(q, nullptr, nullptr, nullptr, nullptr); }), "type mismatch must throw");
+    CHECK(throws([&] { launch_q8_k_quantize_f32(nullptr, 100, nullptr, nullptr, nullptr, nullptr); }), "Q8_K needs multiples of 256");
+}
+
+// The reference's three calls, then the read-back a caller does.
+static std::vector<float> run_three_calls(int layer, const HostLayer &L, const GpuMatrix &router, GpuExpertCache &cache,
+                                          const Qwen38SharedExpertWeights &shared, Qwen38MoeScratch &scratch, const DeviceFloatArray &x,
+                                          DeviceFloatArray &out, Stream stream) {
+    run_qwen38_routed_moe_separate_f32_x(layer, x.data, router, L.t_gate, L.t_up, L.t_down, cache, scratch, nullptr, 1.0f, stream);
+    run_qwen38_shared_expert_f32_x(x.data, shared, scratch, stream);
+    q38_finish_moe_f32(scratch, out.data, stream);
+    check(wd_stream_sync(stream), "sync");
+    std::vector<float> h(L.H);
+    out.download(h.data());
+    return h;
+}
+
+static void gpu_checks() {
+    check(wd_init(0), "wd_init");
+    void *stream = nullptr;
+    check(wd_stream_create(&stream), "stream");
+    const int H = 512, F = 128, E = 32, k = 4, layers = 3;
+    std::vector<HostLayer> L;
+    for (int l = 0; l < layers; ++l) L.push_back(make_layer(1000 + l, H, F, E, k));
+
+    // operators: Q8_K quantiser + IQ3_S GEMV against the oracle
+    {
+        Rng r(7);
+        const std::vector<float> x = rms_normed(r, H);
+        DeviceFloatArray dx;
+        dx.upload(x.data(), H);
+        DeviceArray<int8_t> qs(H);
+        DeviceFloatArray sc(H / 256), y(F);
+        DeviceArray<int16_t> bs(H / 16);
+        launch_q8_k_quantize_f32(dx.data, H, qs.data, sc.data, bs.data, stream);
+        TensorInfo one{"gate0", {static_cast<uint64_t>(H), static_cast<uint64_t>(F)}, GgmlType::IQ3_S, 0, L[0].gate.data()};
+        LowBitMatrix w = upload_lowbit_matrix(one);
+        launch_iq3_s_gemv_q8_k_f32(w, qs.data, sc.data, y.data, stream);
+        check(wd_stream_sync(stream), "sync");
+        std::vector<int8_t> oq(H);
+        std::vector<float> od(H / 256), want(F), got(F);
+        std::vector<int16_t> ob(H / 16);
+        wdo_quantize_q8_K(x.data(), H, oq.data(), od.data(), ob.data());
+        wdo_gemv(WDO_IQ3_S, L[0].gate.data(), F, H, oq.data(), od.data(), want.data(), nullptr);
+        y.download(got.data());
+        CHECK(same_bits(got.data(), want.data(), F), "launch_iq3_s_gemv_q8_k_f32 differs from the oracle");
+    }
+
+    std::vector<GpuMatrix> routers;
+    std::vector<Qwen38SharedExpertWeights> shared(layers);
+    for (int l = 0; l < layers; ++l) {
+        routers.push_back(upload_matrix(L[l].t_router));
+        shared[l].gate_input_f32.upload(L[l].gate_inp.data(), H);
+        TensorInfo g{"sg", {static_cast<uint64_t>(H), static_cast<uint64_t>(F)}, GgmlType::Q8_0, 0, L[l].sg.data()};
+        TensorInfo u{"su", {static_cast<uint64_t>(H), static_cast<uint64_t>(F)}, GgmlType::Q8_0, 0, L[l].su.data()};
+        TensorInfo d{"sd", {static_cast<uint64_t>(F), static_cast<uint64_t>(H)}, GgmlType::Q8_0, 0, L[l].sd.data()};
+        shared[l].gate = upload_lowbit_matrix(g), shared[l].up = upload_lowbit_matrix(u), shared[l].down = upload_lowbit_matrix(d);
+    }
+    Qwen38MoeScratch scratch;
+    scratch.initialize(E, k, H, F);
+    CHECK(throws([&] { scratch.initialize(E, k, H, F); }), "double initialisation must throw");
+    CHECK(throws([&] { q38_finish_moe_f32(scratch, scratch.d_accum(), stream); }), "output aliasing the routed sum must throw");
+
+    ExpertCacheOptions opt;
+    opt.layer_count = layers;
+    const size_t slot = L[0].t_gate.byte_size() / E * 2 + L[0].t_down.byte_size() / E;
+
+    // (1) room for everything: preloaded, no host round trip; (2) 10 slots for 96 experts: LRU with misses
+    for (int mode = 0; mode < 2; ++mode) {
+        GpuExpertCache cache;
+        const size_t want_slots = mode == 0 ? static_cast<size_t>(layers) * E : 10;
+        cache.initialize((want_slots * slot + (1u << 20) - 1) >> 20, L[0].t_gate, L[0].t_up, L[0].t_down, 0, 0, 0, opt);
+        CHECK(cache.slot_bytes() == slot, "slot bytes %zu vs %zu", cache.slot_bytes(), slot);
+        CHECK(cache.slot_count() >= want_slots, "slot count %zu", cache.slot_count());
+        for (int l = 0; l < layers; ++l) cache.register_layer_experts(l, L[l].t_gate, L[l].t_up, L[l].t_down);
+        if (mode == 0)
+            for (int l = 0; l < layers; ++l) cache.preload_layer(l, stream);
+        CHECK(mode == 1 || cache.layer_resident(0), "layer 0 should be resident after the preload");
+        Rng r(99 + mode);
+        DeviceFloatArray dx(H), dout(H);
+        for (int token = 0; token < 4; ++token) {
+            for (int l = 0; l < layers; ++l) {
+                const std::vector<float> x = rms_normed(r, H);
+                dx.upload(x.data(), H);
+                const std::vector<float> got = run_three_calls(l, L[l], routers[l], cache, shared[l], scratch, dx, dout, stream);
+                std::vector<float> want(H), routed(H);
+                std::vector<int> ids(k);
+                wdo_dump dump{};
+                dump.ids = ids.data(), dump.routed = routed.data();
+                wdo_moe_layer(&L[l].o, x.data(), want.data(), &dump, 0);
+                CHECK(same_bits(got.data(), want.data(), H), "mode %d token %d layer %d: three-call output differs from the oracle", mode, token, l);
+                std::vector<int> gids(k);
+                check(wd_memcpy_d2h(gids.data(), scratch.d_ids(), sizeof(int) * k, nullptr), "ids");
+                CHECK(gids == ids, "mode %d token %d layer %d: routed ids differ", mode, token, l);
+                std::vector<float> acc(H);
+                check(wd_memcpy_d2h(acc.data(), scratch.d_accum(), sizeof(float) * H, nullptr), "accum");
+                CHECK(same_bits(acc.data(), routed.data(), H), "mode %d token %d layer %d: routed sum differs", mode, token, l);
+                if (mode == 0) {
+                    run_qwen38_moe_layer_f32_x(l, dx.data, routers[l], L[l].t_gate, L[l].t_up, L[l].t_down, cache, shared[l], scratch, dout.data, 1.0f, stream);
+                    check(wd_stream_sync(stream), "sync");
+                    std::vector<float> fused(H);
+                    dout.download(fused.data());
+                    CHECK(same_bits(fused.data(), want.data(), H), "token %d layer %d: fused call differs from the oracle", token, l);
+                }
+            }
+        }
+        const wd_expert_cache_stats st = cache.stats();
+        if (mode == 0) {
+            CHECK(st.evictions == 0 && st.resident == static_cast<uint64_t>(layers) * E, "resident mode evicted (%llu) or lost experts (%llu)",
+                  static_cast<unsigned long long>(st.evictions), static_cast<unsigned long long>(st.resident));
+        } else {
+            CHECK(st.misses > 0 && st.evictions > 0 && st.resident <= cache.slot_count() && cache.slot_count() < static_cast<size_t>(layers) * E, "LRU mode: misses %llu evictions %llu resident %llu",
+                  static_cast<unsigned long long>(st.misses), static_cast<unsigned long long>(st.evictions), static_cast<unsigned long long>(st.resident));
+            CHECK(st.bytes_copied == st.misses * slot, "bytes copied %llu vs misses x slot", static_cast<unsigned long long>(st.bytes_copied));
+            const ExpertDeviceWeights v = cache.acquire(0, 5, L[0].t_gate, L[0].t_up, L[0].t_down, stream);
+            check(wd_stream_sync(stream), "sync");
+            std::vector<uint8_t> back(v.gate.bytes);
+            check(wd_memcpy_d2h(back.data(), v.gate.data, v.gate.bytes, nullptr), "slot read-back");
+            CHECK(std::memcmp(back.data(), expert_slice(L[0].t_gate, 5).data, v.gate.bytes) == 0 && !v.gate.owns, "acquired view must hold the expert's gate bytes");
+        }
+    }
+    wd_stream_destroy(stream);
+}
+
+int main(int argc, char **argv) {
+    const bool host_only = argc > 1 && std::strcmp(argv[1], "--host-only") == 0;
+    try {
+        host_only_checks();
+        if (!host_only) gpu_checks();
+    } catch (const std::exception &e) {
+        std::printf("FAIL: unexpected exception: %s\n", e.what());
+        return 2;
+    }
+    std::printf("%d checks, %d failures\n", g_checks, g_fail);
+    return g_fail ? 1 : 0;
+}

@@ -1,0 +1,31 @@
+"""The C++ operator header (warpdecode_amd/host/wd_ops.hpp) exercised by tests/host/test_wd_ops.cpp:
+a caller in the reference's style (routed, shared, finish; resident and LRU cache) against the oracle."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EXE = os.path.join(ROOT, "tests", "host", "test_wd_ops")
+
+
+def _run(args):
+    p = subprocess.run([EXE] + args, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    assert p.returncode == 0, p.stdout
+    assert " 0 failures" in p.stdout, p.stdout
+    return p.stdout
+
+
+def test_header_compiles_and_host_checks_pass():
+    from warpdecode_amd import build
+    if not os.path.exists(build.LIB):
+        pytest.skip("HIP library not built")
+    build.build_host_test()
+    _run(["--host-only"])
+
+
+@pytest.mark.gpu
+def test_reference_style_caller_matches_oracle():
+    assert os.path.exists(EXE), "tests/host/test_wd_ops is built by __graft_entry__.build()"
+    out = _run([])
+    assert int(out.split(" checks")[0].split()[-1]) > 60, out

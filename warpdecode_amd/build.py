@@ -23,6 +23,21 @@ def build(verbose=False):
     return LIB
 
 
+def build_host_test(verbose=False):
+    """The C++ test of the operator header (tests/host/test_wd_ops.cpp): host compiler only, linked against
+    the HIP library and the oracle, both found again at run time relative to the binary."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "host", "test_wd_ops.cpp")
+    exe = os.path.join(root, "tests", "host", "test_wd_ops")
+    cmd = ["g++", "-std=c++17", "-O1", "-Wall", "-I" + os.path.join(root, "include"), "-I" + os.path.join(HERE, "host"),
+           "-I" + os.path.join(root, "oracle"), src, "-L" + HERE, "-lwarpdecode_amd", "-L" + os.path.join(root, "oracle"),
+           "-lwdoracle", "-Wl,-rpath,$ORIGIN/../../warpdecode_amd", "-Wl,-rpath,$ORIGIN/../../oracle", "-o", exe]
+    if verbose:
+        print(" ".join(cmd))
+    subprocess.check_call(cmd)
+    return exe
+
+
 if __name__ == "__main__":
     build(verbose=True)
     print("built", LIB)

@@ -52,6 +52,7 @@ _SIGS = {
     "wd_free_host": (i32, [vp]),
     "wd_memcpy_h2d": (i32, [vp, vp, sz, vp]),
     "wd_memcpy_d2h": (i32, [vp, vp, sz, vp]),
+    "wd_memcpy_d2d": (i32, [vp, vp, sz, vp]),
     "wd_memset": (i32, [vp, i32, sz, vp]),
     "wd_stream_create": (i32, [C.POINTER(vp)]),
     "wd_stream_destroy": (i32, [vp]),
@@ -73,6 +74,7 @@ _SIGS = {
     "wd_moe_scratch_enable_partials": (i32, [vp, i32, i32]),
     "wd_moe_scratch_trace": (vp, [vp, i32]),
     "wd_moe_layer_f32": (i32, [C.POINTER(MoeLayer), vp, vp, vp, u32, vp]),
+    "wd_shared_expert_f32": (i32, [C.POINTER(MoeLayer), vp, vp, vp]),
     "wd_moe_stack_f32": (i32, [C.POINTER(MoeLayer), i32, vp, vp, vp, vp, f32, u32, vp]),
 }
 for _n in ("logits", "ids", "weights", "gate_up", "act", "act_qs", "act_scales", "expert_out", "accum", "down_f32",
@@ -87,6 +89,7 @@ _OPTIONAL = {
     "wd_expert_cache_acquire": (i32, [vp, i32, vp, i32, vp, vp]),
     "wd_expert_cache_slot_table": (vp, [vp, i32]),
     "wd_expert_cache_pool": (vp, [vp]),
+    "wd_expert_cache_slot_of": (C.c_longlong, [vp, i32, i32]),
     "wd_expert_cache_get_stats": (i32, [vp, C.POINTER(CacheStats)]),
 }
 

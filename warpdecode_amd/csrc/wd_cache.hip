@@ -263,6 +263,12 @@ const int32_t *wd_expert_cache_slot_table(wd_expert_cache *c, int layer) {
 
 const uint8_t *wd_expert_cache_pool(wd_expert_cache *c) { return c ? c->pool : nullptr; }
 
+long long wd_expert_cache_slot_of(wd_expert_cache *c, int layer, int expert) {
+    if (!c || layer < 0 || expert < 0) return -1;
+    const auto it = c->index.find((static_cast<uint64_t>(layer) << 32) | static_cast<uint32_t>(expert));
+    return it == c->index.end() ? -1 : static_cast<long long>(it->second);
+}
+
 int wd_expert_cache_get_stats(wd_expert_cache *c, wd_expert_cache_stats *out) {
     WD_REQUIRE(c != nullptr && out != nullptr, "expert cache stats: null pointer");
     *out = c->stats;

@@ -409,6 +409,34 @@ extern "C" int wd_moe_layer_f32(const wd_moe_layer *L, const float *d_x, float *
     return layer_dispatch(L, d_x, d_out, s, flags, nullptr, nullptr, 0.0f, as_stream(stream));
 }
 
+extern "C" int wd_shared_expert_f32(const wd_moe_layer *L, const float *d_x, wd_moe_scratch *s, void *stream) {
+    WD_REQUIRE(L && s && d_x, "shared expert: null layer, scratch or activation");
+    WD_REQUIRE(L->hidden == s->hidden && L->expert_ffn == s->ffn, "shared expert geometry mismatch: layer %d/%d, scratch %d/%d",
+               L->hidden, L->expert_ffn, s->hidden, s->ffn);
+    WD_REQUIRE(L->shared_gate_inp && L->shared_gate && L->shared_up && L->shared_down, "shared expert: incomplete weights");
+    const int H = L->hidden, F = L->expert_ffn, slot = s->max_k;
+    const hipStream_t st = as_stream(stream);
+    k_router_gemv<<<dim3(1), dim3(256), 0, st>>>(L->router, d_x, s->logits, 0, H, L->shared_gate_inp, s->shared_gate);
+    WD_LAUNCH_CHECK();
+    k_sigmoid1<<<dim3(1), dim3(64), 0, st>>>(s->shared_gate);
+    WD_LAUNCH_CHECK();
+    k_q8_0_quantize<<<dim3((H / 32 + 31) / 32), dim3(256), 0, st>>>(d_x, H / 32, s->x0_qs, s->x0_d);
+    WD_LAUNCH_CHECK();
+    MatSrc g{}, u{}, d{};
+    g.single = L->shared_gate, u.single = L->shared_up, d.single = L->shared_down;
+    float *gu = s->gate_up + static_cast<size_t>(2) * slot * F;
+    float *act = s->act + static_cast<size_t>(slot) * F;
+    int8_t *aq = s->act_qs + static_cast<size_t>(slot) * F;
+    uint16_t *ad = s->act_d + static_cast<size_t>(slot) * (F / 32);
+    if (const int rc = grouped_gemv(WD_TYPE_Q8_0, g, 1, F, H, s, s->x0_qs, s->x0_d, 0, gu, nullptr, st)) return rc;
+    if (const int rc = grouped_gemv(WD_TYPE_Q8_0, u, 1, F, H, s, s->x0_qs, s->x0_d, 0, gu + F, nullptr, st)) return rc;
+    k_silu_mul_experts<<<dim3((F + 255) / 256, 1), dim3(256), 0, st>>>(gu, act, F);
+    WD_LAUNCH_CHECK();
+    k_q8_0_quantize<<<dim3((F / 32 + 31) / 32), dim3(256), 0, st>>>(act, F / 32, aq, ad);
+    WD_LAUNCH_CHECK();
+    return grouped_gemv(WD_TYPE_Q8_0, d, 1, H, F, s, aq, ad, 0, s->down_f32, nullptr, st);
+}
+
 extern "C" int wd_moe_stack_f32(const wd_moe_layer *layers, int n_layers, float *d_x, float *d_layer_out,
                                 wd_moe_scratch *s, const int32_t *d_ids_trace, float residual_scale, unsigned flags,
                                 void *stream) {

@@ -78,6 +78,10 @@ int wd_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream) {
         WD_HIP(hipMemcpy(h_dst, d_src, bytes, hipMemcpyDeviceToHost));
     return WD_OK;
 }
+int wd_memcpy_d2d(void *d_dst, const void *d_src, size_t bytes, void *stream) {
+    WD_HIP(hipMemcpyAsync(d_dst, d_src, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
+    return WD_OK;
+}
 int wd_memset(void *d_dst, int value, size_t bytes, void *stream) {
     WD_REQUIRE(bytes % 4 == 0, "wd_memset: size must be a multiple of 4 bytes");
     const uint32_t b = static_cast<uint32_t>(value) & 0xffu;

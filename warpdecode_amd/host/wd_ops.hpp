@@ -1,0 +1,580 @@
+// C++ operator surface of the MoE decode path, header-only, over the C ABI of
+// include/warpdecode_amd.h.  The names, argument order and error behaviour are those of the
+// reference's inline C++ API (namespace wd), so that a caller written against it compiles against
+// this header: owning objects are move-only and free device memory in their destructors, cache views
+// are borrowed, geometry/type mismatches and device errors throw std::runtime_error, the grouped
+// launchers return false when they launched nothing.  A stream is an opaque handle (hipStream_t
+// passed as void*), a half scale is 16-bit storage (uint16_t).
+//
+// Link with -lwarpdecode_amd.  No HIP header is needed to include this file.
+#pragma once
+
+#include <algorithm>
+#include <cstdint>
+#include <cstring>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "warpdecode_amd.h"
+
+namespace wd {
+
+using Stream = void *;
+using half_bits = uint16_t;
+
+// src/gguf.hpp:26-44
+enum class GgmlType : uint32_t {
+    F32 = 0,
+    F16 = 1,
+    Q4_0 = 2,
+    Q8_0 = 8,
+    IQ4_NL = 20,
+    IQ3_S = 21,
+    IQ2_S = 22,
+};
+
+inline void check(int rc, const char *what) {
+    if (rc != WD_OK) throw std::runtime_error(std::string(what) + ": " + wd_last_error());
+}
+
+// src/gguf.hpp:268-310
+struct TensorInfo {
+    std::string name;
+    std::vector<uint64_t> dims;  // GGUF order: dims[0] = columns, dims[1] = rows, dims[2] = experts
+    GgmlType type = GgmlType::F32;
+    uint64_t relative_offset = 0;
+    const uint8_t *data = nullptr;
+
+    uint64_t elements() const {
+        uint64_t n = 1;
+        for (uint64_t d : dims) n *= d;
+        return n;
+    }
+    size_t byte_size() const {
+        const uint64_t n = elements();
+        if (type == GgmlType::F32) return static_cast<size_t>(n * 4);
+        if (type == GgmlType::F16) return static_cast<size_t>(n * 2);
+        const uint64_t cols = dims.empty() ? 0 : dims[0];
+        const size_t row = wd_row_bytes(static_cast<int>(type), static_cast<int>(cols));
+        if (row == 0 || cols == 0) throw std::runtime_error("tensor size is not a whole number of blocks, or unsupported type: " + name);
+        return static_cast<size_t>(n / cols) * row;
+    }
+};
+
+// Owning device array (DeviceFloatArray of the reference, src/device_buffer.cuh).
+template <typename T>
+struct DeviceArray {
+    T *data = nullptr;
+    size_t count = 0;
+    DeviceArray() = default;
+    explicit DeviceArray(size_t n) { allocate(n); }
+    DeviceArray(const DeviceArray &) = delete;
+    DeviceArray &operator=(const DeviceArray &) = delete;
+    DeviceArray(DeviceArray &&o) noexcept : data(o.data), count(o.count) { o.data = nullptr, o.count = 0; }
+    DeviceArray &operator=(DeviceArray &&o) noexcept {
+        if (this != &o) {
+            reset();
+            data = o.data, count = o.count;
+            o.data = nullptr, o.count = 0;
+        }
+        return *this;
+    }
+    ~DeviceArray() { reset(); }
+    void allocate(size_t n) {
+        reset();
+        void *p = nullptr;
+        check(wd_malloc(&p, n * sizeof(T)), "device allocation failed");
+        data = static_cast<T *>(p), count = n;
+    }
+    void upload(const T *host, size_t n) {
+        if (n != count) allocate(n);
+        check(wd_memcpy_h2d(data, host, n * sizeof(T), nullptr), "host to device copy failed");
+    }
+    void download(T *host) const { check(wd_memcpy_d2h(host, data, count * sizeof(T), nullptr), "device to host copy failed"); }
+    void reset() {
+        if (data) wd_free(data);
+        data = nullptr, count = 0;
+    }
+    bool empty() const { return data == nullptr; }
+};
+using DeviceFloatArray = DeviceArray<float>;
+
+// src/lowbit.cuh:20-66
+struct LowBitMatrix {
+    int rows = 0;
+    int cols = 0;
+    GgmlType type = GgmlType::F32;
+    uint8_t *data = nullptr;
+    size_t bytes = 0;
+    bool owns = true;
+
+    LowBitMatrix() = default;
+    LowBitMatrix(const LowBitMatrix &) = delete;
+    LowBitMatrix &operator=(const LowBitMatrix &) = delete;
+    LowBitMatrix(LowBitMatrix &&o) noexcept { take(o); }
+    LowBitMatrix &operator=(LowBitMatrix &&o) noexcept {
+        if (this != &o) {
+            reset();
+            take(o);
+        }
+        return *this;
+    }
+    ~LowBitMatrix() { reset(); }
+    void reset() {
+        if (data && owns) wd_free(data);
+        data = nullptr, rows = cols = 0, bytes = 0, owns = true;
+    }
+
+private:
+    void take(LowBitMatrix &o) {
+        rows = o.rows, cols = o.cols, type = o.type, data = o.data, bytes = o.bytes, owns = o.owns;
+        o.data = nullptr, o.rows = o.cols = 0, o.bytes = 0, o.owns = true;
+    }
+};
+
+inline bool lowbit_gemv_supported(GgmlType t) {
+    return t == GgmlType::Q8_0 || t == GgmlType::IQ4_NL || t == GgmlType::IQ2_S || t == GgmlType::IQ3_S || t == GgmlType::Q4_0;
+}
+
+// src/lowbit.cuh:72-86
+inline LowBitMatrix borrow_lowbit_matrix(uint8_t *data, int rows, int cols, GgmlType type, size_t bytes) {
+    LowBitMatrix out;
+    out.data = data, out.rows = rows, out.cols = cols, out.type = type, out.bytes = bytes, out.owns = false;
+    return out;
+}
+
+// src/lowbit.cuh:88-117
+inline LowBitMatrix upload_lowbit_matrix(const TensorInfo &t) {
+    if (t.dims.size() != 2) throw std::runtime_error("low-bit GEMV requires a 2D tensor: " + t.name);
+    if (!lowbit_gemv_supported(t.type)) throw std::runtime_error("unsupported low-bit GEMV tensor type: " + t.name);
+    LowBitMatrix out;
+    out.cols = static_cast<int>(t.dims[0]);
+    out.rows = static_cast<int>(t.dims[1]);
+    out.type = t.type;
+    const int quantum = (t.type == GgmlType::IQ2_S || t.type == GgmlType::IQ3_S) ? 256 : 32;
+    if (out.cols <= 0 || out.rows <= 0 || out.cols % quantum != 0) throw std::runtime_error("invalid low-bit matrix shape: " + t.name);
+    out.bytes = t.byte_size();
+    void *p = nullptr;
+    check(wd_malloc(&p, out.bytes), "low-bit matrix allocation failed");
+    out.data = static_cast<uint8_t *>(p);
+    if (wd_memcpy_h2d(out.data, t.data, out.bytes, nullptr) != WD_OK) {
+        out.reset();
+        throw std::runtime_error(std::string("low-bit matrix upload failed: ") + wd_last_error());
+    }
+    return out;
+}
+
+// src/matrix.cuh:15-31 (the f16 mirror of the reference is not kept: F32 tensors stay F32)
+struct GpuMatrix {
+    int rows = 0;
+    int cols = 0;
+    GgmlType type = GgmlType::F32;
+    bool lowbit = false;
+    LowBitMatrix low;
+    DeviceFloatArray dense_f32;
+    GpuMatrix() = default;
+    GpuMatrix(const GpuMatrix &) = delete;
+    GpuMatrix &operator=(const GpuMatrix &) = delete;
+    GpuMatrix(GpuMatrix &&) noexcept = default;
+    GpuMatrix &operator=(GpuMatrix &&) noexcept = default;
+};
+
+inline bool matrix_has_f32_weights(const GpuMatrix &m) { return !m.lowbit && !m.dense_f32.empty(); }
+
+inline GpuMatrix upload_matrix(const TensorInfo &t) {
+    if (t.dims.size() != 2) throw std::runtime_error("matrix upload requires a 2D tensor: " + t.name);
+    GpuMatrix m;
+    m.cols = static_cast<int>(t.dims[0]), m.rows = static_cast<int>(t.dims[1]), m.type = t.type;
+    if (t.type == GgmlType::F32) {
+        m.dense_f32.upload(reinterpret_cast<const float *>(t.data), static_cast<size_t>(m.rows) * m.cols);
+    } else {
+        m.lowbit = true;
+        m.low = upload_lowbit_matrix(t);
+    }
+    return m;
+}
+
+// src/expert_cache.cuh:2107-2146
+struct ExpertHostSlice {
+    const uint8_t *data = nullptr;
+    size_t bytes = 0;
+    int rows = 0, cols = 0;
+    GgmlType type = GgmlType::F32;
+};
+inline ExpertHostSlice expert_slice(const TensorInfo &t, int expert) {
+    if (t.dims.size() != 3) throw std::runtime_error("expert tensor must be 3D: " + t.name);
+    const int n_expert = static_cast<int>(t.dims[2]);
+    if (expert < 0 || expert >= n_expert) throw std::runtime_error("expert index out of range: " + t.name);
+    if (!lowbit_gemv_supported(t.type)) throw std::runtime_error("expert tensor has unsupported low-bit type: " + t.name);
+    TensorInfo one;
+    one.name = t.name, one.dims = {t.dims[0], t.dims[1]}, one.type = t.type;
+    const size_t slice_bytes = one.byte_size();
+    if (slice_bytes * static_cast<size_t>(n_expert) != t.byte_size()) throw std::runtime_error("expert tensor is not slice-contiguous: " + t.name);
+    ExpertHostSlice out;
+    out.data = t.data + slice_bytes * static_cast<size_t>(expert);
+    out.bytes = slice_bytes, out.cols = static_cast<int>(t.dims[0]), out.rows = static_cast<int>(t.dims[1]), out.type = t.type;
+    return out;
+}
+
+// src/qwen38_moe.cuh:547-562
+struct Qwen38SharedExpertWeights {
+    DeviceFloatArray gate_input_f32;  // f32 [hidden]
+    LowBitMatrix gate, up, down;      // Q8_0
+};
+
+// src/qwen38_moe.cuh:1701-2150.  The device buffers belong to the library's scratch object; the accessors
+// keep the reference's names for the views a caller reads after a layer pass.
+class Qwen38MoeScratch {
+public:
+    Qwen38MoeScratch() = default;
+    Qwen38MoeScratch(const Qwen38MoeScratch &) = delete;
+    Qwen38MoeScratch &operator=(const Qwen38MoeScratch &) = delete;
+    ~Qwen38MoeScratch() { reset(); }
+
+    void initialize(int n_experts, int k, int hidden, int expert_ffn) {
+        if (s_) throw std::runtime_error("MoE scratch already initialized");
+        if (n_experts <= 0 || n_experts > 4096 || k <= 0 || k > 16 || k > n_experts || hidden <= 0 || expert_ffn <= 0)
+            throw std::runtime_error("invalid MoE scratch geometry");
+        check(wd_moe_scratch_create(&s_, hidden, expert_ffn, n_experts, k), "MoE scratch allocation failed");
+        n_experts_ = n_experts, k_ = k, hidden_ = hidden, expert_ffn_ = expert_ffn;
+        void *p = nullptr;
+        check(wd_malloc_host(&p, sizeof(int) * k), "pinned allocation failed");
+        h_ids_ = static_cast<int *>(p);
+        check(wd_malloc_host(&p, sizeof(float) * k), "pinned allocation failed");
+        h_weights_ = static_cast<float *>(p);
+    }
+    void reset() {
+        if (s_) wd_moe_scratch_destroy(s_);
+        if (h_ids_) wd_free_host(h_ids_);
+        if (h_weights_) wd_free_host(h_weights_);
+        s_ = nullptr, h_ids_ = nullptr, h_weights_ = nullptr;
+        moe_out_.reset();
+    }
+    float *moe_out_f32() {
+        if (moe_out_.empty()) moe_out_.allocate(static_cast<size_t>(hidden_));
+        return moe_out_.data;
+    }
+    int n_experts() const { return n_experts_; }
+    int k() const { return k_; }
+    int hidden() const { return hidden_; }
+    int expert_ffn() const { return expert_ffn_; }
+    float *d_logits() const { return wd_moe_scratch_logits(s_); }
+    int *d_ids() const { return wd_moe_scratch_ids(s_); }
+    float *d_weights() const { return wd_moe_scratch_weights(s_); }
+    float *d_accum() const { return wd_moe_scratch_accum(s_); }
+    float *d_shared_gate() const { return wd_moe_scratch_shared_gate(s_); }
+    float *down_f32() const { return wd_moe_scratch_down_f32(s_); }
+    float *rx_batch_gate_up() const { return wd_moe_scratch_gate_up(s_); }
+    float *rx_batch_act() const { return wd_moe_scratch_act(s_); }
+    int8_t *rx_batch_q8_0_values() const { return wd_moe_scratch_act_qs(s_); }
+    half_bits *rx_batch_q8_0_scales() const { return wd_moe_scratch_act_scales(s_); }
+    float *rx_batch_down() const { return wd_moe_scratch_expert_out(s_); }
+    int *h_ids() const { return h_ids_; }
+    float *h_weights() const { return h_weights_; }
+    wd_moe_scratch *handle() const { return s_; }
+
+private:
+    wd_moe_scratch *s_ = nullptr;
+    int n_experts_ = 0, k_ = 0, hidden_ = 0, expert_ffn_ = 0;
+    int *h_ids_ = nullptr;
+    float *h_weights_ = nullptr;
+    DeviceFloatArray moe_out_;
+};
+
+// src/expert_cache.cuh:76-115 (the file-backed staging knobs have no meaning here: sources are host memory)
+struct ExpertCacheOptions {
+    bool stats = false;
+    bool layer_evict = false;
+    int layer_count = 0;
+};
+
+// src/expert_cache.cuh:2148-2154
+struct ExpertDeviceWeights {
+    LowBitMatrix gate, up, down;  // borrowed views of one slot
+    bool cache_hit = false;
+    size_t slot = 0;
+};
+
+// src/expert_cache.cuh:2156-2536
+class GpuExpertCache {
+public:
+    GpuExpertCache() = default;
+    GpuExpertCache(const GpuExpertCache &) = delete;
+    GpuExpertCache &operator=(const GpuExpertCache &) = delete;
+    GpuExpertCache(GpuExpertCache &&o) noexcept { *this = std::move(o); }
+    GpuExpertCache &operator=(GpuExpertCache &&o) noexcept {
+        if (this != &o) {
+            release();
+            c_ = o.c_, n_slots_ = o.n_slots_, slot_bytes_ = o.slot_bytes_, gate_bytes_ = o.gate_bytes_, up_bytes_ = o.up_bytes_,
+            down_bytes_ = o.down_bytes_, n_experts_ = o.n_experts_, n_layers_ = o.n_layers_;
+            g_ = o.g_, u_ = o.u_, d_ = o.d_;
+            reg_ = std::move(o.reg_);
+            o.c_ = nullptr;
+        }
+        return *this;
+    }
+    ~GpuExpertCache() { release(); }
+
+    void initialize(size_t capacity_mib, const TensorInfo &sample_gate, const TensorInfo &sample_up, const TensorInfo &sample_down,
+                    size_t gate_capacity_bytes = 0, size_t up_capacity_bytes = 0, size_t down_capacity_bytes = 0,
+                    const ExpertCacheOptions &options = ExpertCacheOptions{}) {
+        if (c_) throw std::runtime_error("expert cache already initialized");
+        if (capacity_mib == 0) throw std::runtime_error("expert cache capacity is zero");
+        g_ = expert_slice(sample_gate, 0), u_ = expert_slice(sample_up, 0), d_ = expert_slice(sample_down, 0);
+        gate_bytes_ = gate_capacity_bytes ? gate_capacity_bytes : g_.bytes;
+        up_bytes_ = up_capacity_bytes ? up_capacity_bytes : u_.bytes;
+        down_bytes_ = down_capacity_bytes ? down_capacity_bytes : d_.bytes;
+        if (gate_bytes_ < g_.bytes || up_bytes_ < u_.bytes || down_bytes_ < d_.bytes)
+            throw std::runtime_error("expert cache slot capacity is smaller than sample tensors");
+        slot_bytes_ = gate_bytes_ + up_bytes_ + down_bytes_;
+        if (slot_bytes_ == 0) throw std::runtime_error("expert cache slot is empty");
+        const size_t capacity_bytes = capacity_mib * 1024ull * 1024ull;
+        if (capacity_bytes / slot_bytes_ == 0) throw std::runtime_error("expert cache capacity is smaller than one expert slot");
+        n_experts_ = static_cast<int>(sample_gate.dims[2]);
+        n_layers_ = options.layer_count > 0 ? options.layer_count : 128;
+        check(wd_expert_cache_create(&c_, capacity_bytes, gate_bytes_, up_bytes_, down_bytes_, n_layers_, n_experts_,
+                                     options.layer_evict ? 1 : 0),
+              "expert cache allocation failed");
+        wd_expert_cache_stats st{};
+        wd_expert_cache_get_stats(c_, &st);
+        n_slots_ = static_cast<size_t>(st.slots);
+    }
+
+    size_t slot_count() const { return n_slots_; }
+    size_t slot_bytes() const { return slot_bytes_; }
+    size_t resident_count() const {
+        wd_expert_cache_stats st{};
+        if (c_) wd_expert_cache_get_stats(c_, &st);
+        return static_cast<size_t>(st.resident);
+    }
+    wd_expert_cache_stats stats() const {
+        wd_expert_cache_stats st{};
+        if (c_) wd_expert_cache_get_stats(c_, &st);
+        return st;
+    }
+
+    // Host sources of a layer's 3-D expert tensors (pinned memory makes the fills asynchronous).
+    void register_layer_experts(int layer, const TensorInfo &gate, const TensorInfo &up, const TensorInfo &down) {
+        if (layer < 0) return;
+        if (!c_) throw std::runtime_error("expert cache is not initialized");
+        if (registered(layer)) return;
+        expert_slice(gate, 0), expert_slice(up, 0), expert_slice(down, 0);
+        check(wd_expert_cache_register_layer(c_, layer, gate.data, up.data, down.data), "expert cache layer registration failed");
+        if (reg_.size() <= static_cast<size_t>(layer)) reg_.resize(static_cast<size_t>(layer) + 1, 0);
+        reg_[static_cast<size_t>(layer)] = 1;
+    }
+
+    // Makes every expert of a registered layer resident.  With room for all experts of all layers (the
+    // normal case with 288 GB of HBM) nothing is ever evicted and layer passes need no host round trip.
+    void preload_layer(int layer, Stream stream) {
+        if (!registered(layer)) throw std::runtime_error("expert cache layer is not registered");
+        for (int e0 = 0; e0 < n_experts_; e0 += 16) {
+            int32_t ids[16];
+            const int n = std::min(16, n_experts_ - e0);
+            for (int i = 0; i < n; ++i) ids[i] = e0 + i;
+            check(wd_expert_cache_acquire(c_, layer, ids, n, nullptr, stream), "expert cache preload failed");
+        }
+        reg_[static_cast<size_t>(layer)] = 2;
+    }
+    // True when the layer was preloaded and no slot has been recycled since the cache was created.
+    bool layer_resident(int layer) const { return registered(layer) && reg_[static_cast<size_t>(layer)] == 2 && stats().evictions == 0; }
+
+    // One expert; the views stay valid until the slot is recycled by a later acquire.
+    ExpertDeviceWeights acquire(int layer, int expert, const TensorInfo &gate, const TensorInfo &up, const TensorInfo &down, Stream stream) {
+        if (!c_) throw std::runtime_error("expert cache is not initialized");
+        register_layer_experts(layer, gate, up, down);
+        const int32_t id = expert;
+        uint8_t hit = 0;
+        check(wd_expert_cache_acquire(c_, layer, &id, 1, &hit, stream), "expert cache acquire failed");
+        return view(layer, expert, hit != 0);
+    }
+
+    // The k experts of one layer pass at once (they are guaranteed to stay resident together).
+    void acquire_ids(int layer, const int *h_ids, int k, Stream stream, uint8_t *hit_out = nullptr) {
+        if (!c_) throw std::runtime_error("expert cache is not initialized");
+        check(wd_expert_cache_acquire(c_, layer, h_ids, k, hit_out, stream), "expert cache acquire failed");
+    }
+
+    ExpertDeviceWeights view(int layer, int expert, bool hit) const {
+        const long long slot = wd_expert_cache_slot_of(c_, layer, expert);
+        if (slot < 0) throw std::runtime_error("expert is not resident");
+        uint8_t *base = const_cast<uint8_t *>(wd_expert_cache_pool(c_)) + static_cast<size_t>(slot) * slot_bytes_;
+        ExpertDeviceWeights w;
+        w.gate = borrow_lowbit_matrix(base, g_.rows, g_.cols, g_.type, g_.bytes);
+        w.up = borrow_lowbit_matrix(base + gate_bytes_, u_.rows, u_.cols, u_.type, u_.bytes);
+        w.down = borrow_lowbit_matrix(base + gate_bytes_ + up_bytes_, d_.rows, d_.cols, d_.type, d_.bytes);
+        w.cache_hit = hit, w.slot = static_cast<size_t>(slot);
+        return w;
+    }
+
+    const int32_t *slot_table(int layer) const { return wd_expert_cache_slot_table(c_, layer); }
+    const uint8_t *pool() const { return wd_expert_cache_pool(c_); }
+    size_t gate_bytes() const { return gate_bytes_; }
+    size_t up_bytes() const { return up_bytes_; }
+    wd_expert_cache *handle() const { return c_; }
+
+private:
+    bool registered(int layer) const { return layer >= 0 && static_cast<size_t>(layer) < reg_.size() && reg_[static_cast<size_t>(layer)] != 0; }
+    void release() {
+        if (c_) wd_expert_cache_destroy(c_);
+        c_ = nullptr;
+    }
+    wd_expert_cache *c_ = nullptr;
+    size_t n_slots_ = 0, slot_bytes_ = 0, gate_bytes_ = 0, up_bytes_ = 0, down_bytes_ = 0;
+    int n_experts_ = 0, n_layers_ = 0;
+    ExpertHostSlice g_, u_, d_;
+    std::vector<char> reg_;
+};
+
+// ---- operators -----------------------------------------------------------------------------------
+
+// src/lowbit.cuh:873-891
+inline void launch_q8_k_quantize_f32(const float *x, int elements, int8_t *qs, float *scales, int16_t *bsums, Stream stream, int /*threads*/ = 256) {
+    if (elements <= 0 || elements % 256 != 0) throw std::runtime_error("Q8_K activation quantisation needs a multiple of 256 elements");
+    check(wd_q8_k_quantize_f32(x, elements, qs, scales, bsums, stream), "Q8_K quantisation failed");
+}
+
+// src/qwen38_moe.cuh:1470-1481
+inline void q38_moe_quantize_activation_q8_0(const float *input, int elements, int8_t *quantized, half_bits *scales, Stream stream) {
+    check(wd_q8_0_quantize_f32(input, elements, quantized, scales, stream), "Q8_0 quantisation failed");
+}
+
+// src/qwen38_moe.cuh:247-263
+inline void launch_q38_router_gemv_f32(const GpuMatrix &w, const float *x, float *y, Stream stream, int threads = 256) {
+    if (!matrix_has_f32_weights(w)) throw std::runtime_error("router F32 warp GEMV requires an F32 dense matrix");
+    if (threads < 32 || threads % 32 != 0) throw std::runtime_error("router F32 warp GEMV threads must be a multiple of 32");
+    check(wd_router_gemv_f32(w.dense_f32.data, x, y, w.rows, w.cols, stream), "router GEMV failed");
+}
+
+// src/qwen38_moe.cuh:1065-1090
+inline void q38_launch_topk_softmax(const float *logits, int n_experts, int k, float expert_scale, int *ids, float *weights, Stream stream) {
+    check(wd_topk_softmax(logits, n_experts, k, expert_scale, ids, weights, stream), "router top-k failed");
+}
+
+// src/lowbit.cuh:1483-1499, :1181-1197
+inline void launch_iq3_s_gemv_q8_k_f32(const LowBitMatrix &w, const int8_t *act, const float *act_scales, float *out, Stream stream, int /*threads*/ = 256) {
+    if (w.type != GgmlType::IQ3_S || w.rows <= 0 || w.cols <= 0 || w.cols % 256 != 0) throw std::runtime_error("IQ3_S x Q8_K GEMV geometry mismatch");
+    check(wd_gemv_q8_k_f32(WD_TYPE_IQ3_S, w.data, w.rows, w.cols, act, act_scales, out, nullptr, stream), "IQ3_S GEMV failed");
+}
+inline void launch_iq2_s_gemv_q8_k_f32(const LowBitMatrix &w, const int8_t *act, const float *act_scales, float *out, Stream stream, int /*threads*/ = 256) {
+    if (w.type != GgmlType::IQ2_S || w.rows <= 0 || w.cols <= 0 || w.cols % 256 != 0) throw std::runtime_error("IQ2_S x Q8_K GEMV geometry mismatch");
+    check(wd_gemv_q8_k_f32(WD_TYPE_IQ2_S, w.data, w.rows, w.cols, act, act_scales, out, nullptr, stream), "IQ2_S GEMV failed");
+}
+// src/lowbit.cuh:1787-1810
+inline void launch_iq4_nl_gemv_q8_0_f32(const LowBitMatrix &w, const int8_t *act, const half_bits *act_scales, float *out, Stream stream, int /*threads*/ = 256) {
+    if (w.type != GgmlType::IQ4_NL || w.rows <= 0 || w.cols <= 0 || w.cols % 64 != 0) throw std::runtime_error("IQ4_NL x Q8_0 GEMV geometry mismatch");
+    check(wd_gemv_q8_0_f32(WD_TYPE_IQ4_NL, w.data, w.rows, w.cols, act, act_scales, out, nullptr, stream), "IQ4_NL GEMV failed");
+}
+// src/qwen38_hc.cuh:1020-1049
+inline void q38_hc_launch_exact_q8_0_gemv_f32(const uint8_t *weight, const int8_t *act, const half_bits *act_scales, float *out, int rows, int cols, Stream stream) {
+    check(wd_gemv_q8_0_f32(WD_TYPE_Q8_0, weight, rows, cols, act, act_scales, out, nullptr, stream), "Q8_0 GEMV failed");
+}
+// src/warodecode.cu:1746-1768 (raw Q4_0 blocks; no planar prepack)
+inline void launch_q4_float(const LowBitMatrix &w, const int8_t *act, const half_bits *act_scales, float *out, Stream stream) {
+    if (w.type != GgmlType::Q4_0 || w.cols % 32 != 0) throw std::runtime_error("Q4_0 x Q8_0 GEMV geometry mismatch");
+    check(wd_gemv_q8_0_f32(WD_TYPE_Q4_0, w.data, w.rows, w.cols, act, act_scales, out, nullptr, stream), "Q4_0 GEMV failed");
+}
+
+// Grouped launchers over a DEVICE table of expert pointers; false = nothing launched
+// (src/lowbit.cuh:2352-2418, :2427-2460).
+inline bool launch_iq3_s_gemv_q8_k_experts_f32(const uint8_t *const *w_experts, int experts, int rows, int cols, const int8_t *act, const float *act_scales, float *out, Stream stream, int /*threads*/ = 256) {
+    return wd_gemv_q8_k_experts_f32(WD_TYPE_IQ3_S, w_experts, experts, rows, cols, act, act_scales, out, nullptr, stream) == WD_OK;
+}
+inline bool launch_iq2_s_gemv_q8_k_experts_f32(const uint8_t *const *w_experts, int experts, int rows, int cols, const int8_t *act, const float *act_scales, float *out, Stream stream, int /*threads*/ = 256) {
+    return wd_gemv_q8_k_experts_f32(WD_TYPE_IQ2_S, w_experts, experts, rows, cols, act, act_scales, out, nullptr, stream) == WD_OK;
+}
+inline bool launch_iq4_nl_gemv_q8_0_experts_f32(const uint8_t *const *w_experts, int experts, int rows, int cols, const int8_t *act, const half_bits *act_scales, float *out, Stream stream, int /*threads*/ = 256) {
+    return wd_gemv_q8_0_experts_f32(WD_TYPE_IQ4_NL, w_experts, experts, rows, cols, act, act_scales, out, nullptr, stream) == WD_OK;
+}
+inline bool launch_q8_0_gemv_q8_0_experts_f32(const uint8_t *const *w_experts, int experts, int rows, int cols, const int8_t *act, const half_bits *act_scales, float *out, Stream stream) {
+    return wd_gemv_q8_0_experts_f32(WD_TYPE_Q8_0, w_experts, experts, rows, cols, act, act_scales, out, nullptr, stream) == WD_OK;
+}
+
+// src/qwen38_moe.cuh:2425-2436
+inline void q38_moe_add_shared_f32(float *routed_in_out, const float *shared, const float *gate, int n, Stream stream) {
+    check(wd_add_shared_f32(routed_in_out, shared, gate, n, stream), "shared expert add failed");
+}
+
+// ---- layer -------------------------------------------------------------------------------------------
+
+namespace detail {
+inline void fill_routed(wd_moe_layer &L, int layer, const GpuMatrix &router, const TensorInfo &gate, const TensorInfo &up, const TensorInfo &down,
+                        const GpuExpertCache &cache, const Qwen38MoeScratch &scratch, float expert_scale) {
+    if (!matrix_has_f32_weights(router)) throw std::runtime_error("MoE router must be an F32 matrix");
+    const ExpertHostSlice g = expert_slice(gate, 0), u = expert_slice(up, 0), d = expert_slice(down, 0);
+    if (g.cols != router.cols || u.cols != g.cols || u.rows != g.rows || d.cols != g.rows || d.rows != g.cols)
+        throw std::runtime_error("MoE expert tensor geometry mismatch");
+    std::memset(&L, 0, sizeof(L));
+    L.hidden = g.cols, L.expert_ffn = g.rows, L.n_experts = router.rows, L.top_k = scratch.k();
+    L.expert_scale = expert_scale;
+    L.gate_type = static_cast<int>(g.type), L.up_type = static_cast<int>(u.type), L.down_type = static_cast<int>(d.type);
+    L.router = router.dense_f32.data;
+    L.slot_of_expert = cache.slot_table(layer);
+    L.slot_pool = cache.pool();
+    L.slot_bytes = cache.slot_bytes(), L.slot_gate_bytes = cache.gate_bytes(), L.slot_up_bytes = cache.up_bytes();
+    if (!L.slot_of_expert) throw std::runtime_error("MoE layer is outside the expert cache's layer range");
+}
+}  // namespace detail
+
+// Routed experts of one layer: router -> top-k -> (host ids, cache acquire) -> grouped gate/up -> SwiGLU ->
+// grouped down -> ordered weighted sum into scratch.d_accum() and `out`.
+// src/qwen38_moe.cuh:3650-3779.  When every expert of the layer is already resident the host never
+// waits: the selection stays on the device and the kernels index the slot table themselves.
+inline void run_qwen38_routed_moe_separate_f32_x(int layer, const float *x, const GpuMatrix &router, const TensorInfo &gate_exps,
+                                                 const TensorInfo &up_exps, const TensorInfo &down_exps, GpuExpertCache &cache,
+                                                 Qwen38MoeScratch &scratch, float *out, float expert_scale, Stream stream,
+                                                 bool preselected = false) {
+    wd_moe_layer L;
+    detail::fill_routed(L, layer, router, gate_exps, up_exps, down_exps, cache, scratch, expert_scale);
+    float *dst = out ? out : scratch.moe_out_f32();
+    if (cache.layer_resident(layer)) {
+        check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), preselected ? WD_MOE_PRESELECTED : 0u, stream), "MoE layer failed");
+        return;
+    }
+    if (!preselected) check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), WD_MOE_ONLY_A, stream), "MoE router failed");
+    check(wd_memcpy_d2h(scratch.h_ids(), scratch.d_ids(), sizeof(int) * L.top_k, stream), "routed ids copy failed");
+    check(wd_stream_sync(stream), "stream synchronisation failed");
+    cache.register_layer_experts(layer, gate_exps, up_exps, down_exps);
+    cache.acquire_ids(layer, scratch.h_ids(), L.top_k, stream);
+    check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), WD_MOE_PRESELECTED | WD_MOE_ONLY_B | WD_MOE_ONLY_C, stream), "MoE experts failed");
+}
+
+// src/qwen38_moe.cuh:3963-3969
+inline void run_qwen38_shared_expert_f32_x(const float *x, const Qwen38SharedExpertWeights &shared, Qwen38MoeScratch &scratch, Stream stream) {
+    if (shared.gate.type != GgmlType::Q8_0 || shared.up.type != GgmlType::Q8_0 || shared.down.type != GgmlType::Q8_0)
+        throw std::runtime_error("shared expert weights must be Q8_0");
+    if (shared.gate.cols != scratch.hidden() || shared.gate.rows != scratch.expert_ffn() || shared.down.rows != scratch.hidden() ||
+        shared.down.cols != scratch.expert_ffn() || shared.gate_input_f32.count != static_cast<size_t>(scratch.hidden()))
+        throw std::runtime_error("shared expert geometry mismatch");
+    wd_moe_layer L;
+    std::memset(&L, 0, sizeof(L));
+    L.hidden = scratch.hidden(), L.expert_ffn = scratch.expert_ffn();
+    L.shared_gate_inp = shared.gate_input_f32.data;
+    L.shared_gate = shared.gate.data, L.shared_up = shared.up.data, L.shared_down = shared.down.data;
+    check(wd_shared_expert_f32(&L, x, scratch.handle(), stream), "shared expert failed");
+}
+
+// out = routed weighted sum + shared expert * gate (src/qwen38_moe.cuh:2442-2453)
+inline void q38_finish_moe_f32(Qwen38MoeScratch &scratch, float *out, Stream stream) {
+    if (out == scratch.d_accum()) throw std::runtime_error("F32 MoE output must not alias the routed accumulation buffer");
+    check(wd_memcpy_d2d(out, scratch.d_accum(), sizeof(float) * scratch.hidden(), stream), "routed sum copy failed");
+    q38_moe_add_shared_f32(out, scratch.down_f32(), scratch.d_shared_gate(), scratch.hidden(), stream);
+}
+
+// The three calls above in the fused dispatches (router and shared expert overlap, the selection never
+// leaves the device): the fast path when the layer's experts are resident in `cache` or in plain device
+// tensors.  No single counterpart in the reference (its caller issues the three calls,
+// src/qwen38_forward.cuh:3330-3371).
+inline void run_qwen38_moe_layer_f32_x(int layer, const float *x, const GpuMatrix &router, const TensorInfo &gate_exps, const TensorInfo &up_exps,
+                                       const TensorInfo &down_exps, GpuExpertCache &cache, const Qwen38SharedExpertWeights &shared,
+                                       Qwen38MoeScratch &scratch, float *out, float expert_scale, Stream stream) {
+    wd_moe_layer L;
+    detail::fill_routed(L, layer, router, gate_exps, up_exps, down_exps, cache, scratch, expert_scale);
+    L.shared_gate_inp = shared.gate_input_f32.data;
+    L.shared_gate = shared.gate.data, L.shared_up = shared.up.data, L.shared_down = shared.down.data;
+    check(wd_moe_layer_f32(&L, x, out, scratch.handle(), 0u, stream), "MoE layer failed");
+}
+
+}  // namespace wd
