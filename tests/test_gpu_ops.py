@@ -106,7 +106,7 @@ GEMV_SHAPES = {
     synth.IQ2_S: [(640, 2560), (512, 2048), (3, 256)],
     synth.Q8_0: [(2048, 512), (512, 2048), (7, 96), (640, 2560), (18, 32)],
     synth.IQ4_NL: [(2560, 640), (2048, 512), (5, 96), (9, 32 * 5)],
-    synth.Q4_0: [(2048, 2048), (2048, 8192), (8192, 2048), (1000, 2048), (6, 96)],
+    synth.Q4_0: [(2048, 2048), (2048, 8192), (8192, 2048), (128256, 2048), (1000, 2048), (6, 96)],   # C1 incl. the lm_head
 }
 
 
