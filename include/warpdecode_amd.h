@@ -248,6 +248,17 @@ const uint8_t *wd_expert_cache_pool(wd_expert_cache *c);
 long long wd_expert_cache_slot_of(wd_expert_cache *c, int layer, int expert);
 int wd_expert_cache_get_stats(wd_expert_cache *c, wd_expert_cache_stats *out);
 
+
+/* One decode step through a stack of layers whose routed experts come from `cache` (layer l of the stack is
+ * layer l of the cache; the slot fields of `layers` are ignored and taken from the cache).  x is updated as in
+ * wd_moe_stack_f32.  With a routing trace (host and device copies of int32 [n_layers][top_k]) the fills of the
+ * next layer overlap the current layer's dispatches; without one each layer's ids go to the host first, as in
+ * the reference's loop (q38_moe_select_experts_f32_x + GpuExpertCache::acquire per selected expert,
+ * src/qwen38_moe.cuh:2323-2380, :3650-3779).  Counters: wd_expert_cache_get_stats. */
+int wd_moe_stack_cached_f32(const wd_moe_layer *layers, int n_layers, wd_expert_cache *cache, float *d_x,
+                            float *d_layer_out, wd_moe_scratch *scratch, const int32_t *h_ids_trace,
+                            const int32_t *d_ids_trace, float residual_scale, unsigned flags, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

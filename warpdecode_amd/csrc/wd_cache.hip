@@ -66,6 +66,8 @@ struct wd_expert_cache {
     std::vector<Partition> parts;
     std::unordered_map<uint64_t, size_t> index;
     uint64_t clock = 0;
+    uint64_t prev_floor = 0;     // clock value before the previous acquire call
+    bool fills_pending = false;  // a deferred acquire's fills have not been waited for yet
     std::vector<const uint8_t *> h_gate, h_up, h_down;
     int32_t *d_table = nullptr;  // [n_layers][n_experts]
     hipStream_t copy_stream = nullptr;
@@ -165,8 +167,15 @@ int wd_expert_cache_register_layer(wd_expert_cache *c, int layer, const uint8_t 
     return WD_OK;
 }
 
-int wd_expert_cache_acquire(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uint8_t *hit_out,
-                            void *stream) {
+}  // extern "C"
+
+namespace {
+
+// `defer_wait`: the fills are queued behind the work already on `stream`, but `stream` is not made to wait
+// for them; the caller does that later with wait_fills(), after it has queued work that does not depend on
+// the new experts (the previous layer).  A victim must then be older than the previous acquire call too.
+int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uint8_t *hit_out, void *stream,
+                 bool defer_wait) {
     WD_REQUIRE(c != nullptr && c->pool != nullptr, "expert cache is not initialized");
     WD_REQUIRE(layer >= 0 && layer < c->n_layers, "expert cache: layer %d out of range", layer);
     WD_REQUIRE(h_ids != nullptr && k > 0 && 2 * k <= kMaxUpdates, "expert cache: invalid id list (k=%d)", k);
@@ -176,6 +185,8 @@ int wd_expert_cache_acquire(wd_expert_cache *c, int layer, const int32_t *h_ids,
                P.end - P.begin, k);
     hipStream_t st = as_stream(stream);
     const uint64_t epoch_floor = c->clock;  // slots touched by this call carry last_use > epoch_floor
+    const uint64_t victim_floor = defer_wait ? c->prev_floor : epoch_floor;
+    c->prev_floor = epoch_floor;
     SlotUpdate updates[kMaxUpdates];
     int n_updates = 0;
     bool waited = false;
@@ -205,8 +216,8 @@ int wd_expert_cache_acquire(wd_expert_cache *c, int layer, const int32_t *h_ids,
         } else {
             slot = P.lru.front();
             Slot &victim = c->slots[slot];
-            if (victim.last_use > epoch_floor)
-                return fail(WD_ERR_STATE, "expert cache: all slots are held by the current acquire call");
+            if (victim.last_use > victim_floor)
+                return fail(WD_ERR_STATE, "expert cache: all slots are held by the experts being acquired");
             P.lru.pop_front();
             c->index.erase(victim.key);
             updates[n_updates++] = {static_cast<int32_t>((victim.key >> 32) * c->n_experts + (victim.key & 0xffffffffu)), -1};
@@ -251,9 +262,32 @@ int wd_expert_cache_acquire(wd_expert_cache *c, int layer, const int32_t *h_ids,
     }
     if (waited) {
         WD_HIP(hipEventRecord(c->ev_done, c->copy_stream));
-        WD_HIP(hipStreamWaitEvent(st, c->ev_done, 0));
+        if (defer_wait)
+            c->fills_pending = true;
+        else
+            WD_HIP(hipStreamWaitEvent(st, c->ev_done, 0));
     }
     return WD_OK;
+}
+
+int wait_fills(wd_expert_cache *c, hipStream_t st) {
+    if (c->fills_pending) {
+        WD_HIP(hipStreamWaitEvent(st, c->ev_done, 0));
+        c->fills_pending = false;
+    }
+    return WD_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int wd_expert_cache_acquire(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uint8_t *hit_out,
+                            void *stream) {
+    if (c && c->fills_pending) {
+        if (const int rc = wait_fills(c, as_stream(stream))) return rc;
+    }
+    return acquire_impl(c, layer, h_ids, k, hit_out, stream, false);
 }
 
 const int32_t *wd_expert_cache_slot_table(wd_expert_cache *c, int layer) {

@@ -33,6 +33,7 @@ struct wd_moe_scratch {
     int32_t *union_buf = nullptr;         // [1 + 128 + 128 * 8] expert union of a multi-token pass
     unsigned long long *trace = nullptr;  // device [3][16][8] time stamps, see wd_moe_scratch_trace
     int trace_wg = 0;
+    int32_t *h_ids = nullptr;             // pinned [16]: routed ids for callers that must see them on the host
 };
 
 namespace {
@@ -95,6 +96,11 @@ int wd_moe_scratch_create(wd_moe_scratch **out, int hidden, int expert_ffn, int 
     s->arrive = reinterpret_cast<unsigned *>(b + o_arr);
     s->union_buf = reinterpret_cast<int32_t *>(b + o_uni);
     (void)hipMemset(s->block, 0, c.off);
+    if (hipHostMalloc(reinterpret_cast<void **>(&s->h_ids), sizeof(int32_t) * 16, hipHostMallocDefault) != hipSuccess) {
+        (void)hipFree(s->block);
+        delete s;
+        return fail(WD_ERR_HIP, "hipHostMalloc MoE scratch ids failed");
+    }
     *out = s;
     return WD_OK;
 }
@@ -105,6 +111,7 @@ int wd_moe_scratch_destroy(wd_moe_scratch *s) {
     (void)hipFree(s->gup);
     (void)hipFree(s->dp);
     (void)hipFree(s->trace);
+    (void)hipHostFree(s->h_ids);
     delete s;
     return WD_OK;
 }

@@ -2,3 +2,4 @@
 #include "wd_ops.hip"
 #include "wd_layer.hip"
 #include "wd_cache.hip"
+#include "wd_stack.hip"

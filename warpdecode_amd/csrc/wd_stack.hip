@@ -1,0 +1,68 @@
+// A stack of MoE layers fed from the expert-slot cache: what a decode step does when the routed experts do
+// not all fit in HBM (or are kept in a bounded pool on purpose).  The cache's device slot tables stand in for
+// the reference's per-layer pointer-table upload (src/qwen38_moe.cuh:3288-3303).
+//
+// With a routing trace known to the host, the fills of layer l+1 are queued before layer l is launched and
+// waited for after it, so the host link works while the previous layer computes.  Without one, every layer
+// does what the reference does (src/qwen38_moe.cuh:2323-2380): router and selection, ids to pinned host
+// memory, stream synchronisation, acquire, expert dispatches.
+using namespace wd;
+
+extern "C" int wd_moe_stack_cached_f32(const wd_moe_layer *layers, int n_layers, wd_expert_cache *cache, float *d_x,
+                                       float *d_layer_out, wd_moe_scratch *s, const int32_t *h_ids_trace,
+                                       const int32_t *d_ids_trace, float residual_scale, unsigned flags, void *stream) {
+    WD_REQUIRE(layers && n_layers > 0 && cache && s, "cached MoE stack: null layers, cache or scratch");
+    WD_REQUIRE(d_x && d_layer_out, "cached MoE stack: null activation or output pointer");
+    WD_REQUIRE(n_layers <= cache->n_layers, "cached MoE stack: %d layers exceed the cache's %d", n_layers, cache->n_layers);
+    WD_REQUIRE((h_ids_trace == nullptr) == (d_ids_trace == nullptr), "cached MoE stack: the routing trace needs its host and device copy");
+    WD_REQUIRE(!(flags & (WD_MOE_ONLY_A | WD_MOE_ONLY_B | WD_MOE_ONLY_C | WD_MOE_STAGED)), "cached MoE stack: unsupported flags");
+    const hipStream_t st = as_stream(stream);
+    auto bind = [&](int l) {
+        wd_moe_layer L = layers[l];
+        L.slot_of_expert = cache->d_table + static_cast<size_t>(l) * cache->n_experts;
+        L.slot_pool = cache->pool;
+        L.slot_bytes = cache->slot_bytes, L.slot_gate_bytes = cache->gate_bytes, L.slot_up_bytes = cache->up_bytes;
+        return L;
+    };
+    for (int l = 0; l < n_layers; ++l) {
+        const wd_moe_layer L = bind(l);
+        if (const int rc = check_layer(&L, s)) return rc;
+        WD_REQUIRE(L.n_experts == cache->n_experts, "cached MoE stack: layer %d has %d experts, the cache %d", l, L.n_experts, cache->n_experts);
+    }
+    const int k = layers[0].top_k;
+    const size_t part_slots = cache->parts[0].end - cache->parts[0].begin;
+    const bool ahead = h_ids_trace != nullptr && part_slots >= static_cast<size_t>(4 * k);
+
+    if (h_ids_trace) {
+        if (const int rc = wd_expert_cache_acquire(cache, 0, h_ids_trace, k, nullptr, stream)) return rc;
+        for (int l = 0; l < n_layers; ++l) {
+            const wd_moe_layer L = bind(l);
+            if (ahead && l + 1 < n_layers) {
+                if (const int rc = acquire_impl(cache, l + 1, h_ids_trace + static_cast<size_t>(l + 1) * k, k, nullptr, stream, true)) return rc;
+            }
+            if (const int rc = layer_fused(&L, d_x, d_layer_out, s, flags, d_ids_trace + static_cast<size_t>(l) * k, d_x, residual_scale, st))
+                return rc;
+            if (l + 1 < n_layers) {
+                if (ahead) {
+                    if (const int rc = wait_fills(cache, st)) return rc;
+                } else if (const int rc = wd_expert_cache_acquire(cache, l + 1, h_ids_trace + static_cast<size_t>(l + 1) * k, k, nullptr, stream)) {
+                    return rc;
+                }
+            }
+        }
+        return WD_OK;
+    }
+
+    for (int l = 0; l < n_layers; ++l) {
+        const wd_moe_layer L = bind(l);
+        if (!(flags & WD_MOE_PRESELECTED)) {
+            if (const int rc = layer_fused(&L, d_x, d_layer_out, s, flags | WD_MOE_ONLY_A, nullptr, d_x, residual_scale, st)) return rc;
+        }
+        WD_HIP(hipMemcpyAsync(s->h_ids, s->ids, sizeof(int32_t) * L.top_k, hipMemcpyDeviceToHost, st));
+        WD_HIP(hipStreamSynchronize(st));
+        if (const int rc = wd_expert_cache_acquire(cache, l, s->h_ids, L.top_k, nullptr, stream)) return rc;
+        if (const int rc = layer_fused(&L, d_x, d_layer_out, s, flags | WD_MOE_ONLY_B | WD_MOE_ONLY_C, nullptr, d_x, residual_scale, st))
+            return rc;
+    }
+    return WD_OK;
+}
