@@ -26,6 +26,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 STACK_FLAGS = int(os.environ.get("WD_BENCH_FLAGS", "0"))   # experiments only (e.g. 4 = staged dispatches)
+CHAIN_FLAGS = int(os.environ.get("WD_BENCH_CHAIN_FLAGS", "0"))   # experiments only (0x80 = launch floor)
 RESIDUAL_SCALE = 2.0 ** -12   # glue between layers: x += scale * layer(x), keeps the chain finite
 
 
@@ -416,7 +417,7 @@ def main():
     for name, flag in only.items():
         def chain():
             capi.call("wd_moe_stack_f32", layers, NL, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()), scratch,
-                      trace_ptr, RESIDUAL_SCALE, flag, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+                      trace_ptr, RESIDUAL_SCALE, flag | CHAIN_FLAGS, C.c_void_p(torch.cuda.current_stream().cuda_stream))
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):

@@ -153,6 +153,9 @@ typedef struct {
 typedef struct wd_moe_scratch wd_moe_scratch;
 int wd_moe_scratch_create(wd_moe_scratch **out, int hidden, int expert_ffn, int n_experts, int max_k);
 int wd_moe_scratch_destroy(wd_moe_scratch *s);
+/* 0 when every bounded wait inside the fused dispatches was satisfied so far, 1 when one ran out (the layer's
+ * results are then invalid), -1 on error.  Synchronous read of one device word. */
+int wd_moe_scratch_status(wd_moe_scratch *s);
 /* Device views, named after Qwen38MoeScratch accessors (src/qwen38_moe.cuh:1701-2150). */
 float *wd_moe_scratch_logits(wd_moe_scratch *s);      /* f32 [n_experts] */
 int32_t *wd_moe_scratch_ids(wd_moe_scratch *s);       /* i32 [k] */
@@ -185,6 +188,8 @@ unsigned long long *wd_moe_scratch_trace(wd_moe_scratch *s, int wg);
 #define WD_MOE_ONLY_A 0x10u /* router + selection + shared gate/up */
 #define WD_MOE_ONLY_B 0x20u /* routed gate/up + SwiGLU */
 #define WD_MOE_ONLY_C 0x40u /* down projections + combine */
+#define WD_MOE_SPLIT_AB 0x100u /* router and routed gate/up as two launches instead of one with an in-dispatch hand-off */
+#define WD_MOE_DRY 0x80u    /* every workgroup of the fused dispatches returns at once: the launch floor */
 
 /* One decode step of one layer: router -> top-k -> grouped gate/up -> SwiGLU -> Q8_0 ->
  * grouped down -> ordered weighted sum -> + shared * sigmoid gate.  d_out is f32 [hidden]

@@ -32,26 +32,25 @@ struct LayerArgs {
     float *accum, *down_f32, *out;
     float *residual;             // null or [H]
     float residual_scale;
+    int dry;                     // measurement aid: every workgroup returns at once
     int preselected;
     int n_router_wgs;            // workgroups of dispatch A that take router rows
     unsigned *arrive;            // device counter of finished router workgroups (zero between dispatches)
+    uint32_t *ids_tagged;        // [kTagCopies][16] selected ids published inside the merged dispatch (kTagInvalid = not yet)
+    int clear_tagged;            // dispatch C resets ids_tagged when it is done with the layer
+    unsigned *status;            // [0] set to 1 when a bounded wait inside a dispatch ran out
     unsigned long long *trace;   // profiling aid: null, or [3][16][8] time stamps (100 MHz) of workgroup trace_wg
     int trace_wg;
 };
+
+constexpr int kTagCopies = 16;           // replicas of the published ids, 64 bytes apart, so that pollers spread over lines
+constexpr uint32_t kTagInvalid = 0xffffffffu;
+constexpr unsigned kSpinLimit = 1u << 21;  // polls (about a microsecond each) before a wait gives up
 
 // Time stamp `i` of dispatch `d` (0 = A, 1 = B, 2 = C) for the traced workgroup; lane 0 of every wave.
 WD_DEV void mark(const LayerArgs &a, int d, int i) {
     if (a.trace && static_cast<int>(blockIdx.x) == a.trace_wg && (threadIdx.x & 63) == 0 && (threadIdx.x >> 6) < 15)
         a.trace[(d * 16 + (threadIdx.x >> 6)) * 8 + i] = wall_clock64();
-}
-// Row 15 of each dispatch: [0] earliest start, [1] latest end over all workgroups.
-WD_DEV void mark_span(const LayerArgs &a, int d, bool end) {
-    if (a.trace && threadIdx.x == 0) {
-        if (end)
-            atomicMax(&a.trace[(d * 16 + 15) * 8 + 1], wall_clock64());
-        else
-            atomicMin(&a.trace[(d * 16 + 15) * 8 + 0], wall_clock64());
-    }
 }
 
 // ---- in-workgroup quantisers (results in LDS) ------------------------------------------------
@@ -285,6 +284,99 @@ WD_DEV void router_rows(const float *__restrict__ w, const float *__restrict__ x
     }
 }
 
+// Router rows for the merged dispatch: one row per wave, x staged once per workgroup in LDS (f32 [cols]).
+// Accumulator t (of ggml's 4 x 8) of the row lives in lanes t and t + 32: for every span of 2048 columns lane t
+// runs the multiply-adds of columns [span, span + 1024) and hands the value to lane t + 32, which continues with
+// [span + 1024, span + 2048) and hands it back for the next span, so each chain still sees its columns in
+// ascending order while a lane holds only 32 weights (half the registers of the 32-lanes-per-row version,
+// which lets three workgroups of the merged dispatch share a compute unit).
+// Every thread of the workgroup must call it (it contains a barrier).
+template <bool COHERENT>
+WD_DEV void router_rows_wave(const float *__restrict__ w, const float *__restrict__ x, float *xs, float *logits, int rows,
+                             int cols, const float *__restrict__ extra_w, float *extra_out, int wg) {
+    const int lane = threadIdx.x & 63, t = lane & 31;
+    const bool upper = lane >= 32;
+    const int row = wg * static_cast<int>(blockDim.x >> 6) + static_cast<int>(threadIdx.x >> 6);
+    const int total = rows + (extra_w ? 1 : 0);
+    const bool on = row < total;
+    const float *wr = on ? (row < rows ? w + static_cast<size_t>(row) * cols : extra_w) : x;
+    const int np = cols & ~31;
+    const int half_off = (upper ? 1024 : 0) + t;
+    float wv[32];
+    if (on) {
+#pragma unroll
+        for (int u = 0; u < 32; ++u) {
+            const int c = half_off + 32 * u;
+            wv[u] = (c < np) ? wr[c] : 0.0f;
+        }
+    }
+    for (int i = static_cast<int>(threadIdx.x) * 4; i < cols; i += static_cast<int>(blockDim.x) * 4) {
+        if (i + 4 <= cols) {
+            *reinterpret_cast<float4 *>(xs + i) = *reinterpret_cast<const float4 *>(x + i);
+        } else {
+            for (int c = i; c < cols; ++c) xs[c] = x[c];
+        }
+    }
+    __syncthreads();
+    float s = 0.0f;  // the chain value; valid in the half that ran last
+    if (on) {
+        for (int i0 = 0; i0 < np; i0 += 2048) {
+            if (i0 > 0) {
+#pragma unroll
+                for (int u = 0; u < 32; ++u) {
+                    const int c = i0 + half_off + 32 * u;
+                    wv[u] = (c < np) ? wr[c] : 0.0f;
+                }
+            }
+            // this lane's 32 multiply-adds of the span, continuing the chain from `start`
+            auto run_half = [&](float start) {
+                float v = start;
+#pragma unroll
+                for (int ub = 0; ub < 32; ub += 8) {
+                    float xv[8];
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) {
+                        const int c = i0 + half_off + 32 * (ub + q);
+                        xv[q] = xs[c < np ? c : 0];
+                    }
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) {
+                        const int c = i0 + half_off + 32 * (ub + q);
+                        const float nv = __builtin_fmaf(wv[ub + q], xv[q], v);
+                        v = (c < np) ? nv : v;
+                    }
+                }
+                return v;
+            };
+            // the lower half advances the chain (from the upper half's value of the previous span) ...
+            const wd_uint2v back = __builtin_amdgcn_permlane32_swap(f_bits(s), f_bits(s), false, false);
+            if (!upper) s = run_half(i0 == 0 ? 0.0f : bits_f(back.y));
+            // ... and the upper half continues from its result
+            const wd_uint2v fwd = __builtin_amdgcn_permlane32_swap(f_bits(s), f_bits(s), false, false);
+            if (upper) s = run_half(bits_f(fwd.x));
+        }
+    }
+    // the 32 accumulators are final in the upper half (lanes 32..63): ggml's closing tree
+    float o = __shfl_down(s, 16, 32);
+    if (t < 16) s = s + o;
+    o = __shfl_down(s, 8, 32);
+    if (t < 8) s = s + o;
+    o = __shfl_down(s, 4, 32);
+    if (t < 4) s = s + o;
+    o = __shfl_down(s, 1, 32);
+    if (t == 0 || t == 2) s = s + o;
+    o = __shfl_down(s, 2, 32);
+    float acc = s + o;
+    if (on && lane == 32) {
+        for (int c = np; c < cols; ++c) acc = acc + wr[c] * xs[c];
+        float *dst = (row < rows) ? logits + row : extra_out;
+        if (COHERENT)
+            __hip_atomic_store(dst, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else
+            *dst = acc;
+    }
+}
+
 // ---- dispatch A -----------------------------------------------------------------------------------------
 // grid = n_router_wgs + ceil(F / 8) (the second part only with a shared expert); 512 threads.
 // Router workgroups: 16 rows each.  Shared-expert workgroups: 8 (gate, up) row pairs, one per wave.
@@ -300,8 +392,8 @@ __global__ __launch_bounds__(512) void k_layer_a(LayerArgs a) {
     __shared__ int s_last;
     const int wg = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (a.dry) return;
     mark(a, 0, 0);
-    mark_span(a, 0, false);
     if (wg < a.n_router_wgs) {
         router_rows<true>(a.router, a.x, a.logits, a.preselected ? 0 : a.E, a.H, a.sh_inp, a.shared_gate, wg);
         mark(a, 0, 1);
@@ -326,7 +418,6 @@ __global__ __launch_bounds__(512) void k_layer_a(LayerArgs a) {
             if (a.trace && lane == 0) a.trace[(0 * 16 + 8) * 8 + 1] = wall_clock64();
         }
         mark(a, 0, 2);
-        mark_span(a, 0, true);
         return;
     }
     int8_t *xq = reinterpret_cast<int8_t *>(lds_a);
@@ -344,7 +435,144 @@ __global__ __launch_bounds__(512) void k_layer_a(LayerArgs a) {
     });
     if (lane == 0 && r < a.F) a.act[static_cast<size_t>(a.k) * a.F + r] = silu_ggml(gu[0]) * gu[1];
     mark(a, 0, 3);
-    mark_span(a, 0, true);
+}
+
+// ---- dispatches A and B in one launch ---------------------------------------------------------------------
+// Workgroups [0, n_router_wgs): router rows, the last one to finish selects the experts and publishes the ids;
+// then ceil(F / 8) workgroups for the shared expert's gate/up; then k * ceil(F / 8) workgroups for the routed
+// gate/up.  The routed workgroups are dispatched after the router ones (lower block index first), quantise x and
+// stage the codebooks while the router runs, then poll the published ids; as soon as these appear they request
+// their weights.  This removes a launch, a round trip for the ids and the serial activation set-up from the
+// critical path of the layer.
+//
+// Publication: id j goes, as one 32-bit word, to ids_tagged[c][j] of every replica c with a device-scope atomic
+// store; a word other than kTagInvalid is the id itself, so a reader needs no second flag.  The words are reset
+// to kTagInvalid by dispatch C (or by the caller) before the next layer pass uses them.  The wait is bounded:
+// when it runs out the workgroup sets status[0] and returns.
+template <int TYPE>
+__global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
+    constexpr bool kIq = (TYPE == 21 || TYPE == 22);
+    extern __shared__ __align__(16) uint8_t lds_ab[];
+    __shared__ __align__(16) uint8_t s_union[sizeof(Q8RowTile) * 8 > sizeof(IqTables) ? sizeof(Q8RowTile) * 8 : sizeof(IqTables)];
+    __shared__ int s_last;
+    const int wg = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (a.dry) return;
+    const int groups = (a.F + 7) / 8;
+    const int n_shared_wgs = a.sh_inp ? groups : 0;
+
+    mark(a, wg < a.n_router_wgs + n_shared_wgs ? 0 : 1, 0);
+    if (wg < a.n_router_wgs) {
+        router_rows_wave<true>(a.router, a.x, reinterpret_cast<float *>(lds_ab), a.logits, a.E, a.H, a.sh_inp,
+                               a.shared_gate, wg);
+        mark(a, 0, 1);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);  // this wave's stores have been acknowledged
+        __syncthreads();
+        if (threadIdx.x == 0)
+            s_last = (__hip_atomic_fetch_add(a.arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+                      static_cast<unsigned>(a.n_router_wgs - 1));
+        __syncthreads();
+        if (s_last && wave == 0) {
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+            if (a.trace && lane == 0) a.trace[(0 * 16 + 8) * 8 + 0] = wall_clock64();
+            int32_t *lds_ids = reinterpret_cast<int32_t *>(s_union);
+            float *lds_w = reinterpret_cast<float *>(s_union + 64);
+            topk_wave<true>(a.logits, a.E, a.k, a.w_scale, lds_ids, lds_w, a.ids_override, lane);
+            wave_lds_fence();
+            const int id = lds_ids[lane & 15];
+            // replicas first (the routed workgroups wait for them), then the plain copies for dispatch C
+#pragma unroll 4
+            for (int c = 0; c < kTagCopies; ++c)
+                if (lane < a.k)
+                    __hip_atomic_store(a.ids_tagged + c * 16 + lane, static_cast<uint32_t>(id), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+            if (lane < a.k) {
+                a.ids[lane] = id;
+                a.weights[lane] = lds_w[lane];
+            }
+            if (lane == 0) {
+                if (a.sh_inp) {
+                    const float g = __hip_atomic_load(a.shared_gate, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    a.shared_gate[0] = sigmoid_ggml(g);
+                }
+                a.arrive[0] = 0u;
+            }
+            if (a.trace && lane == 0) a.trace[(0 * 16 + 8) * 8 + 1] = wall_clock64();
+        }
+        mark(a, 0, 2);
+        return;
+    }
+
+    int8_t *xq = reinterpret_cast<int8_t *>(lds_ab);
+    uint8_t *xscale = lds_ab + a.H;  // Q8_K: f32 [H/256]; Q8_0: f16 [H/32]
+    if (wg < a.n_router_wgs + n_shared_wgs) {
+        Q8RowTile *tiles = reinterpret_cast<Q8RowTile *>(s_union);
+        const int r = (wg - a.n_router_wgs) * 8 + wave;
+        const int nb = a.H >> 5;
+        const size_t rb = static_cast<size_t>(nb) * 34;
+        const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
+        const uint8_t *const rows[2] = {a.sh_gate + off, a.sh_up + off};
+        float gu[2];
+        q8_row_wave<2>(rows, nb, xq, reinterpret_cast<const uint16_t *>(xscale), tiles[wave], lane, gu, [&]() {
+            lds_quantize_q8_0(a.x, a.H, xq, reinterpret_cast<uint16_t *>(xscale), threadIdx.x, 512);
+            __syncthreads();
+        });
+        if (lane == 0 && r < a.F) a.act[static_cast<size_t>(a.k) * a.F + r] = silu_ggml(gu[0]) * gu[1];
+        return;
+    }
+
+    // routed gate/up: set-up that does not need the ids
+    const int bw = wg - a.n_router_wgs - n_shared_wgs;
+    const int j = bw / groups;
+    const int rg = bw - j * groups;
+    IqTables &tables = *reinterpret_cast<IqTables *>(s_union);
+    if (kIq) {
+        stage_tables<TYPE == 21, TYPE == 22>(tables, threadIdx.x, 512);
+        for (int b = wave; b < (a.H >> 8); b += 8)
+            wave_quantize_q8_k_block(a.x + b * 256, xq + b * 256, reinterpret_cast<float *>(xscale) + b, lane);
+    } else {
+        lds_quantize_q8_0(a.x, a.H, xq, reinterpret_cast<uint16_t *>(xscale), threadIdx.x, 512);
+    }
+    mark(a, 1, 1);
+    __shared__ int s_expert;
+    if (threadIdx.x == 0) {
+        const uint32_t *src = a.ids_tagged + (bw & (kTagCopies - 1)) * 16 + j;
+        uint32_t e = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        unsigned polls = 0;
+        while (e == kTagInvalid && ++polls < kSpinLimit) {
+            __builtin_amdgcn_s_sleep(4);
+            e = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (e == kTagInvalid) __hip_atomic_store(a.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_expert = static_cast<int>(e);
+    }
+    __syncthreads();
+    mark(a, 1, 2);
+    const int e = s_expert;
+    if (e < 0 || e >= a.E) return;  // the wait ran out (status is set): leave without touching memory
+    const uint8_t *gate = mat_ptr_ids(a.gate_up, 2 * j, e);
+    const uint8_t *up = mat_ptr_ids(a.gate_up, 2 * j + 1, e);
+    float *act = a.act + static_cast<size_t>(j) * a.F;
+    const int r = rg * 8 + wave;
+    float gu[2];
+    if (kIq) {
+        const int nb = a.H >> 8;
+        const size_t rb = static_cast<size_t>(nb) * (TYPE == 21 ? 110 : 82);
+        const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
+        const uint8_t *const rows[2] = {gate + off, up + off};
+        iq_rows_q8k<(kIq ? TYPE : 21), 2, false>(rows, nb, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
+                                                  nullptr, 0);
+    } else {
+        Q8RowTile *tiles = reinterpret_cast<Q8RowTile *>(s_union);
+        const int nb = a.H >> 5;
+        const size_t rb = static_cast<size_t>(nb) * 34;
+        const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
+        const uint8_t *const rows[2] = {gate + off, up + off};
+        q8_row_wave<2>(rows, nb, xq, reinterpret_cast<const uint16_t *>(xscale), tiles[wave], lane, gu);
+    }
+    if (lane == 0 && r < a.F) act[r] = silu_ggml(gu[0]) * gu[1];
+    mark(a, 1, 3);
 }
 
 // ---- dispatch B -----------------------------------------------------------------------------------------
@@ -365,8 +593,8 @@ __global__ __launch_bounds__(TYPE == 20 ? 256 : 512) void k_layer_b(LayerArgs a)
     int8_t *xq = reinterpret_cast<int8_t *>(lds_b);
     uint8_t *xscale = lds_b + a.H;  // f32 [H/256] or f16 [H/32]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (a.dry) return;
     mark(a, 1, 0);
-    mark_span(a, 1, false);
 
     const int groups = (a.F + kRowsPerWg - 1) / kRowsPerWg;
     const int j = blockIdx.x / groups;
@@ -424,7 +652,6 @@ __global__ __launch_bounds__(TYPE == 20 ? 256 : 512) void k_layer_b(LayerArgs a)
         if ((lane & 15) == 0 && r4 < nrows) act[r0 + r4] = silu_ggml(gu[0]) * gu[1];
     }
     __syncthreads();
-    mark_span(a, 1, true);
 }
 
 // ---- dispatch C -----------------------------------------------------------------------------------------
@@ -450,8 +677,13 @@ __global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
     const int nrows = min(4, a.H - r0);
     const int nb = a.F >> 5;
     const int r4 = lane >> 4;
+    if (a.dry) return;
+    // every routed workgroup of this layer pass finished with the previous dispatch: make the ids published
+    // for them invalid again (this dispatch reads the plain copy)
+    if (a.clear_tagged && blockIdx.x == 0)
+        for (int i = threadIdx.x; i < kTagCopies * 16; i += blockDim.x)
+            __hip_atomic_store(a.ids_tagged + i, kTagInvalid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     mark(a, 2, 0);
-    mark_span(a, 2, false);
     // combine operands, requested early: lane m keeps router weight m, lane 16 the shared gate
     float wreg = 0.0f;
     if (wave == 0) {
@@ -491,7 +723,6 @@ __global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
             if (a.expert_out && on) a.expert_out[static_cast<size_t>(m) * a.H + row] = y;
         }
         const float gate = lane_get(wreg, 16);
-        mark_span(a, 2, true);
         if (!on) return;
         float o = acc;
         if (shared) {

@@ -34,7 +34,13 @@ struct wd_moe_scratch {
     unsigned long long *trace = nullptr;  // device [3][16][8] time stamps, see wd_moe_scratch_trace
     int trace_wg = 0;
     int32_t *h_ids = nullptr;             // pinned [16]: routed ids for callers that must see them on the host
+    uint32_t *tagged = nullptr;           // [kTagRecords][kTagCopies][16] ids published inside the merged dispatch
+    unsigned *status = nullptr;           // [0] != 0: a bounded wait inside a dispatch ran out
 };
+
+namespace {
+constexpr int kTagRecords = 64;  // one record per layer of a stack (modulo), so that a chain of layers needs no reset in between
+}
 
 namespace {
 
@@ -70,7 +76,8 @@ int wd_moe_scratch_create(wd_moe_scratch **out, int hidden, int expert_ffn, int 
                  o_act = c.take(sizeof(float) * K1 * F), o_aq = c.take(K1 * F),
                  o_ad = c.take(sizeof(uint16_t) * K1 * (F / 32)), o_eo = c.take(sizeof(float) * K1 * H),
                  o_acc = c.take(sizeof(float) * H), o_dn = c.take(sizeof(float) * H), o_sg = c.take(256),
-                 o_arr = c.take(256), o_uni = c.take(sizeof(int32_t) * (1 + 128 + 128 * kMaxTokens));
+                 o_arr = c.take(256), o_uni = c.take(sizeof(int32_t) * (1 + 128 + 128 * kMaxTokens)),
+                 o_tag = c.take(sizeof(uint32_t) * kTagRecords * kTagCopies * 16), o_status = c.take(256);
     const hipError_t e = hipMalloc(reinterpret_cast<void **>(&s->block), c.off);
     if (e != hipSuccess) {
         delete s;
@@ -95,7 +102,10 @@ int wd_moe_scratch_create(wd_moe_scratch **out, int hidden, int expert_ffn, int 
     s->shared_gate = reinterpret_cast<float *>(b + o_sg);
     s->arrive = reinterpret_cast<unsigned *>(b + o_arr);
     s->union_buf = reinterpret_cast<int32_t *>(b + o_uni);
+    s->tagged = reinterpret_cast<uint32_t *>(b + o_tag);
+    s->status = reinterpret_cast<unsigned *>(b + o_status);
     (void)hipMemset(s->block, 0, c.off);
+    (void)hipMemset(s->tagged, 0xff, sizeof(uint32_t) * kTagRecords * kTagCopies * 16);
     if (hipHostMalloc(reinterpret_cast<void **>(&s->h_ids), sizeof(int32_t) * 16, hipHostMallocDefault) != hipSuccess) {
         (void)hipFree(s->block);
         delete s;
@@ -116,6 +126,12 @@ int wd_moe_scratch_destroy(wd_moe_scratch *s) {
     return WD_OK;
 }
 
+int wd_moe_scratch_status(wd_moe_scratch *s) {
+    if (!s) return -1;
+    unsigned v = 0;
+    if (hipMemcpy(&v, s->status, sizeof(v), hipMemcpyDeviceToHost) != hipSuccess) return -1;
+    return static_cast<int>(v);
+}
 float *wd_moe_scratch_logits(wd_moe_scratch *s) { return s->logits; }
 int32_t *wd_moe_scratch_ids(wd_moe_scratch *s) { return s->ids; }
 float *wd_moe_scratch_weights(wd_moe_scratch *s) { return s->weights; }
@@ -326,7 +342,7 @@ int layer_staged(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_s
 }
 
 LayerArgs fused_args(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s, unsigned flags,
-                     const int32_t *ids_override, float *residual, float residual_scale) {
+                     const int32_t *ids_override, float *residual, float residual_scale, int rec = 0) {
     const bool shared = L->shared_gate_inp != nullptr;
     LayerArgs a{};
     a.H = L->hidden, a.F = L->expert_ffn, a.E = L->n_experts, a.k = L->top_k;
@@ -345,10 +361,14 @@ LayerArgs fused_args(const wd_moe_layer *L, const float *d_x, float *d_out, wd_m
     a.accum = s->accum, a.down_f32 = s->down_f32, a.out = d_out;
     a.residual = residual, a.residual_scale = residual_scale;
     a.preselected = (flags & WD_MOE_PRESELECTED) ? 1 : 0;
+    a.dry = (flags & WD_MOE_DRY) ? 1 : 0;
     const int router_rows_n = (a.preselected ? 0 : a.E) + (shared ? 1 : 0);
     a.n_router_wgs = (router_rows_n + 15) / 16;
     a.trace = s->trace, a.trace_wg = s->trace_wg;
     a.arrive = s->arrive;
+    a.ids_tagged = s->tagged + static_cast<size_t>(rec % kTagRecords) * kTagCopies * 16;
+    a.clear_tagged = 1;
+    a.status = s->status;
     return a;
 }
 
@@ -364,18 +384,35 @@ int launch_a(const LayerArgs &a, hipStream_t st) {
 
 // One layer in three dispatches (router + shared gate/up, routed gate/up, down + combine).
 int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s, unsigned flags,
-                const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st) {
+                const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st, int rec = 0) {
     const int H = L->hidden, F = L->expert_ffn, k = L->top_k;
     const bool shared = L->shared_gate_inp != nullptr;
-    const LayerArgs a = fused_args(L, d_x, d_out, s, flags, ids_override, residual, residual_scale);
+    const LayerArgs a = fused_args(L, d_x, d_out, s, flags, ids_override, residual, residual_scale, rec);
     const unsigned only = flags & (WD_MOE_ONLY_A | WD_MOE_ONLY_B | WD_MOE_ONLY_C);
-    if (!only || (only & WD_MOE_ONLY_A)) {
+    const bool run_a = !only || (only & WD_MOE_ONLY_A), run_b = !only || (only & WD_MOE_ONLY_B);
+    const bool iq = consumes_q8k(L->gate_type);
+    // router + selection + shared gate/up + routed gate/up in one launch (the routed workgroups wait for the ids
+    // inside the dispatch) unless the ids are given, the tensor type has no 512-thread kernel, or the caller
+    // asked for the two dispatches apart
+    const bool merged = run_a && run_b && !a.preselected && !(flags & WD_MOE_SPLIT_AB) &&
+                        (iq || L->gate_type == WD_TYPE_Q8_0);
+    if (merged) {
+        LayerArgs m = a;
+        m.n_router_wgs = (a.E + (shared ? 1 : 0) + 7) / 8;  // one router row per wave in the merged dispatch
+        const int grid_ab = m.n_router_wgs + (shared ? (F + 7) / 8 : 0) + k * ((F + 7) / 8);
+        const size_t lds_ab = sizeof(float) * static_cast<size_t>(H) + 16;  // f32 x of the router rows; the quantised x of the others fits inside
+        switch (L->gate_type) {
+            case WD_TYPE_IQ3_S: k_layer_ab<21><<<dim3(grid_ab), dim3(512), lds_ab, st>>>(m); break;
+            case WD_TYPE_IQ2_S: k_layer_ab<22><<<dim3(grid_ab), dim3(512), lds_ab, st>>>(m); break;
+            default: k_layer_ab<8><<<dim3(grid_ab), dim3(512), lds_ab, st>>>(m); break;
+        }
+        WD_LAUNCH_CHECK();
+    } else if (run_a) {
         if (const int rc = launch_a(a, st)) return rc;
     }
-    const bool iq = consumes_q8k(L->gate_type);
     const size_t lds_b = H + (iq ? sizeof(float) * (H / 256) : sizeof(uint16_t) * (H / 32));
     const int grid_b = k * (L->gate_type == WD_TYPE_IQ4_NL ? (F + 15) / 16 : (F + 7) / 8);
-    if (!only || (only & WD_MOE_ONLY_B)) {
+    if (run_b && !merged) {
         switch (L->gate_type) {
             case WD_TYPE_IQ3_S: k_layer_b<21><<<dim3(grid_b), dim3(512), lds_b, st>>>(a); break;
             case WD_TYPE_IQ2_S: k_layer_b<22><<<dim3(grid_b), dim3(512), lds_b, st>>>(a); break;
@@ -400,11 +437,11 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
 }
 
 int layer_dispatch(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s, unsigned flags,
-                   const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st) {
+                   const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st, int rec = 0) {
     const bool want_partials = s->gup != nullptr;
     if ((flags & WD_MOE_STAGED) || want_partials)
         return layer_staged(L, d_x, d_out, s, flags, ids_override, residual, residual_scale, st);
-    return layer_fused(L, d_x, d_out, s, flags, ids_override, residual, residual_scale, st);
+    return layer_fused(L, d_x, d_out, s, flags, ids_override, residual, residual_scale, st, rec);
 }
 
 }  // namespace
@@ -452,9 +489,16 @@ extern "C" int wd_moe_stack_f32(const wd_moe_layer *layers, int n_layers, float 
     for (int l = 0; l < n_layers; ++l) {
         if (const int rc = check_layer(&layers[l], s)) return rc;
     }
+    const unsigned only = flags & (WD_MOE_ONLY_A | WD_MOE_ONLY_B | WD_MOE_ONLY_C);
     for (int l = 0; l < n_layers; ++l) {
         const int32_t *trace = d_ids_trace ? d_ids_trace + static_cast<size_t>(l) * layers[l].top_k : nullptr;
-        if (const int rc = layer_dispatch(&layers[l], d_x, d_layer_out, s, flags, trace, d_x, residual_scale, as_stream(stream)))
+        if (only && !(only & WD_MOE_ONLY_C) && l % kTagRecords == 0) {
+            // no dispatch C to invalidate the published ids: reset all records before they are used again
+            const size_t n = static_cast<size_t>(kTagRecords) * kTagCopies * 16;
+            k_fill_u32<<<dim3((n + 255) / 256), dim3(256), 0, as_stream(stream)>>>(s->tagged, kTagInvalid, n);
+            WD_LAUNCH_CHECK();
+        }
+        if (const int rc = layer_dispatch(&layers[l], d_x, d_layer_out, s, flags, trace, d_x, residual_scale, as_stream(stream), l))
             return rc;
     }
     return WD_OK;

@@ -469,7 +469,8 @@ WD_DEV void q8_row_wave(const uint8_t *const (&rows)[NM], int nb, const int8_t *
             tile.ds[lane] = ds;
             wave_lds_fence();
             // blocks past the end of the row contribute fma(0, 0, acc) == acc
-#pragma unroll
+            // (partial unroll: a full one makes the compiler hold all 128 tile values in registers at once)
+#pragma unroll 4
             for (int s4 = 0; s4 < 16; ++s4) {
                 const float4 pv = *reinterpret_cast<const float4 *>(&tile.pf[c][4 * s4]);
                 const float4 dv = *reinterpret_cast<const float4 *>(&tile.ds[4 * s4]);
