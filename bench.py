@@ -397,21 +397,22 @@ def main():
     finite = bool(torch.isfinite(d_x).all().item())
     note("timed region done: %.3f ms/step" % ms_per_step)
 
-    # Algorithmic bytes of the three dispatches of one layer (weights only, as the workload prices them):
-    #   A  router f32 [E][H] + the shared expert's gate vector + its Q8_0 gate and up matrices
-    #   B  gate and up (IQ3_S) of the k selected experts
+    # Algorithmic bytes of the two dispatches of one layer (weights only, as the workload prices them):
+    #   AB router f32 [E][H] + the shared expert's gate vector + its Q8_0 gate and up matrices
+    #      + gate and up (IQ3_S) of the k selected experts
     #   C  down (Q8_0) of the k selected experts and of the shared expert
     q8h, q8f, iq3h = synth.row_bytes(synth.Q8_0, H), synth.row_bytes(synth.Q8_0, F), synth.row_bytes(synth.IQ3_S, H)
-    alg = {"k_layer_a": E * H * 4 + H * 4 + 2 * F * q8h, "k_layer_b": k * 2 * F * iq3h, "k_layer_c": (k + 1) * H * q8f}
+    alg = {"k_layer_ab": E * H * 4 + H * 4 + 2 * F * q8h + k * 2 * F * iq3h, "k_layer_c": (k + 1) * H * q8f}
     bytes_per_layer = sum(alg.values())
     assert E != 512 or bytes_per_layer == 27697152
     bytes_per_step = bytes_per_layer * NL
 
     # Per-kernel launch time, live: the stack is replayed with one dispatch per layer only (the other two
-    # left out), so the timed region is a chain of NL launches of that one kernel over NL layers' weights.
+    # left out), so the timed region is a chain of NL launches of that one kernel over NL layers' weights
+    # (plus, for k_layer_ab, one small fill launch per chain that resets the in-dispatch hand-off words).
     # HIP events on the launch stream bracket `reps` replays; the period includes the gap between two
     # dependent launches on a stream (about 1.5 us in a graph), which a profiler's begin-to-end time omits.
-    only = {"k_layer_a": 0x10, "k_layer_b": 0x20, "k_layer_c": 0x40}
+    only = {"k_layer_ab": 0x30, "k_layer_c": 0x40}
     per_kernel, reps = {}, 20
     step(0)
     for name, flag in only.items():

@@ -134,3 +134,59 @@ def test_linearity_of_combine(g, oracle):
                         weights=np.ones(1, np.float32))
         acc = (acc + (one["accum"] * wts[j]).astype(np.float32)).astype(np.float32)
     assert g.same_bits(acc, full["accum"])
+
+
+def _fused_vs_oracle(g, oracle, L, x, flags=0):
+    want, d = oracle.moe_layer(L, x)
+    got = run_layer(g, L, x, partials=False, flags=flags)
+    assert np.array_equal(got["ids"], d["ids"]), (got["ids"], d["ids"])
+    assert g.same_bits(got["weights"], d["weights"])
+    assert g.same_bits(got["logits"], d["logits"])
+    assert g.same_bits(got["out"], want)
+
+
+@pytest.mark.parametrize("flags", [0, 0x100], ids=["merged", "split"])
+def test_selection_edge_rows(g, oracle, flags):
+    """The selection inside the fused dispatches on rows that defeat its fast path: exact ties between
+    experts (duplicated router rows), all logits equal (zero router), a row dominated by one expert so that the
+    other exponentials underflow, and fewer experts than one wave holds."""
+    H, F, k = 512, 64, 4
+    for E in (8, 64, 512):
+        L = synth.make_layer(H, F, E, k, synth.IQ3_S, synth.Q8_0, True, seed=SEED, layer=900 + E,
+                             router_sigma=1.0 / np.sqrt(H))
+        x = synth.rms_normed(synth.rng_for(SEED, 46, E), H)
+        _fused_vs_oracle(g, oracle, L, x, flags)
+        dup = dict(L)
+        r = L["router"].copy()
+        r[1::2] = r[0::2]                       # every odd expert ties with its even neighbour
+        dup["router"] = r
+        _fused_vs_oracle(g, oracle, dup, x, flags)
+        zero = dict(L)
+        zero["router"] = np.zeros_like(L["router"])
+        _fused_vs_oracle(g, oracle, zero, x, flags)
+        spike = dict(L)
+        r = L["router"].copy()
+        r[E // 2] = x * np.float32(200.0 / H)    # logit 200: every other exponential underflows to zero
+        r[E // 2 + 1] = r[E // 2]
+        spike["router"] = r
+        _fused_vs_oracle(g, oracle, spike, x, flags)
+
+
+def test_selection_more_than_512_experts(g, oracle):
+    H, F, k = 256, 32, 10
+    for E in (520, 1024):
+        L = synth.make_layer(H, F, E, k, synth.IQ3_S, synth.Q8_0, False, seed=SEED, layer=950 + E,
+                             router_sigma=1.0 / np.sqrt(H))
+        x = synth.rms_normed(synth.rng_for(SEED, 47, E), H)
+        _fused_vs_oracle(g, oracle, L, x)
+        dup = dict(L)
+        r = L["router"].copy()
+        r[E // 2:] = r[:E - E // 2]
+        dup["router"] = r
+        _fused_vs_oracle(g, oracle, dup, x)
+
+
+def test_status_word_is_clear(g):
+    sc = g.Scratch(512, 64, 8, 2)
+    assert capi.load().wd_moe_scratch_status(sc.h) == 0
+    sc.close()

@@ -109,11 +109,11 @@ WD_DEV void wave_quantize_q8_k_block(const float *__restrict__ x256, int8_t *qs2
 // ascending order, k rungs of "largest remaining probability, lowest index on ties", renormalise.
 // COHERENT: the logits were written by other workgroups of the same dispatch; they are read with
 // device-scope atomic loads so that no stale cached copy can be seen.
+// Softmax of the row: lane l ends up with the probabilities of its 8-expert group(s) in v (or -inf everywhere
+// when every exponential vanished: `dead`).
 template <int M, bool COHERENT>
-WD_DEV void topk_wave_m(const float *logits, int n, int k, float w_scale, int32_t *ids, float *weights,
-                        const int32_t *__restrict__ override_ids, int lane) {
+WD_DEV void softmax_probs(const float *logits, int n, int lane, float (&v)[8 * M], bool &dead) {
     const int groups = n >> 3;
-    float v[8 * M];
     float mx = -INFINITY;
 #pragma unroll
     for (int m = 0; m < M; ++m) {
@@ -147,17 +147,37 @@ WD_DEV void topk_wave_m(const float *logits, int n, int k, float w_scale, int32_
         const float hi = v[8 * m + 1] + v[8 * m + 5], hh = v[8 * m + 3] + v[8 * m + 7];
         gs[m] = (lo + lh) + (hi + hh);
     }
-    // group sums accumulated into a double in ascending group order (uniform arithmetic)
-    double sum = 0.0;
+    // The reference accumulates the group sums into a double in ascending group order.  When every non-zero
+    // group sum is within a factor 2^20 of the largest, all of them are multiples of one power of two and every
+    // partial sum fits 53 bits, so the result is exact and the same in any order: a lane tree then replaces
+    // the chain of (up to 128) dependent double additions.
+    float gmax = 0.0f, gmin = INFINITY;
 #pragma unroll
     for (int m = 0; m < M; ++m) {
+        gmax = __builtin_fmaxf(gmax, gs[m]);
+        gmin = __builtin_fminf(gmin, gs[m] > 0.0f ? gs[m] : INFINITY);
+    }
+    gmax = wave_max(gmax);
+    gmin = -wave_max(-gmin);
+    double sum = 0.0;
+    if (gmin >= gmax * 0x1p-20f && gmax < INFINITY) {
+        double part = 0.0;
 #pragma unroll
-        for (int l = 0; l < 64; ++l) {
-            const float gl = readlane_f(gs[m], l);
-            if (l + 64 * m < groups) sum += static_cast<double>(gl);
+        for (int m = 0; m < M; ++m) part += static_cast<double>(gs[m]);
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) part += lane_xor(part, o);
+        sum = part;
+    } else {
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+#pragma unroll
+            for (int l = 0; l < 64; ++l) {
+                const float gl = readlane_f(gs[m], l);
+                if (l + 64 * m < groups) sum += static_cast<double>(gl);
+            }
         }
     }
-    const bool dead = (sum == 0.0);
+    dead = (sum == 0.0);
     const float inv = dead ? 0.0f : static_cast<float>(1.0 / sum);
 #pragma unroll
     for (int m = 0; m < M; ++m) {
@@ -165,10 +185,16 @@ WD_DEV void topk_wave_m(const float *logits, int n, int k, float w_scale, int32_
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[8 * m + i] = (on && !dead) ? v[8 * m + i] * inv : -INFINITY;
     }
-    // For a row whose exponentials all vanished every probability is -inf, nothing ever beats the
-    // running best of -inf, and the reference keeps expert 0 with the value read back from the row.
-    float top_mine = 0.0f;  // lane j keeps the j-th selected probability
-    int id_mine = 0;
+}
+
+// k rungs of "largest remaining probability, lowest index on ties" over the probabilities held as by
+// softmax_probs; lane j keeps the j-th selected probability and id.
+// For a row whose exponentials all vanished every probability is -inf, nothing ever beats the running best of
+// -inf, and the reference keeps expert 0 with the value read back from the row.
+template <int M>
+WD_DEV void rungs_on_probs(float (&v)[8 * M], int k, int lane, float &top_mine, int &id_mine) {
+    top_mine = 0.0f;
+    id_mine = 0;
     for (int j = 0; j < k; ++j) {
         // this lane's largest remaining probability; lowest slot on ties
         float bv = v[0];
@@ -196,13 +222,14 @@ WD_DEV void topk_wave_m(const float *logits, int n, int k, float w_scale, int32_
             id_mine = win;
         }
     }
-    // sum of the selected probabilities in selection order, in a double
+}
+
+// Renormalisation: the selected probabilities summed in selection order in a double, clamp, divide, optional
+// scale; lanes 0..k-1 write ids/weights through the given pointers (LDS or global).
+WD_DEV void finish_weights(float top_mine, int id_mine, int k, float w_scale, int32_t *ids, float *weights,
+                           const int32_t *__restrict__ override_ids, int lane) {
     double wsum = 0.0;
-#pragma unroll
-    for (int j = 0; j < 16; ++j) {
-        const float tj = readlane_f(top_mine, j);
-        if (j < k) wsum += static_cast<double>(tj);
-    }
+    for (int j = 0; j < k; ++j) wsum += static_cast<double>(readlane_f(top_mine, j));
     const float denom = __builtin_fmaxf(static_cast<float>(wsum), 6.103515625e-5f);
     if (lane < k) {
         float wj = top_mine / denom;
@@ -210,6 +237,158 @@ WD_DEV void topk_wave_m(const float *logits, int n, int k, float w_scale, int32_
         weights[lane] = wj;
         ids[lane] = override_ids ? override_ids[lane] : id_mine;
     }
+}
+
+template <int M, bool COHERENT>
+WD_DEV void topk_wave_m(const float *logits, int n, int k, float w_scale, int32_t *ids, float *weights,
+                        const int32_t *__restrict__ override_ids, int lane) {
+    float v[8 * M];
+    bool dead;
+    softmax_probs<M, COHERENT>(logits, n, lane, v, dead);
+    float top_mine;
+    int id_mine;
+    rungs_on_probs<M>(v, k, lane, top_mine, id_mine);
+    finish_weights(top_mine, id_mine, k, w_scale, ids, weights, override_ids, lane);
+}
+
+// The same selection by a whole workgroup (at least five waves; every wave must call it).  Wave 0 computes
+// the probabilities; meanwhile waves 1..4 each find the k largest LOGITS of a quarter of the row and wave 1
+// merges them into k candidates.  exp is monotone only up to rounding, so the candidates are then checked
+// against the probabilities: they are the reference's selection exactly when their probabilities are strictly
+// decreasing and the last one is strictly above every probability left.  If not (ties, rounding inversions,
+// rows with -inf or NaN) wave 0 falls back to the rungs over the probabilities it still holds.
+// lds: scratch of 4 * (512 * M + 160) bytes whose three `ready` words (see topk_ready_flags) the caller zeroes before
+// the barrier that precedes the call.  The results are written by wave 0 (lanes 0..k-1).
+WD_DEV int *topk_ready_flags(uint8_t *lds, int n) {
+    return reinterpret_cast<int *>(lds) + 512 * (n <= 512 ? 1 : 2) + 64 + 64 + 16;
+}
+
+template <int M>
+WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32_t *ids, float *weights,
+                         const int32_t *__restrict__ override_ids, uint8_t *lds, int lane, int wave,
+                         unsigned long long *stamps = nullptr) {
+#define WD_STAMP(i) do { if (stamps && wave == 0 && lane == 0) stamps[i] = wall_clock64(); } while (0)
+    float *p = reinterpret_cast<float *>(lds);          // [512 * M] probabilities
+    float *cv = p + 512 * M;                            // [4][16] candidate logits of the quarters
+    int *ci = reinterpret_cast<int *>(cv + 64);         // [4][16] their expert ids
+    int *sel = ci + 64;                                 // [16] merged candidates
+    int *ready = sel + 16;                              // [3] quarters 1..3 are in LDS; zeroed by the caller before its barrier
+    constexpr int NL = 2 * M;                           // logits per lane in a quarter
+    float v[8 * M];
+    bool dead = false;
+    if (wave == 0) {
+        WD_STAMP(0);
+        softmax_probs<M, true>(logits, n, lane, v, dead);
+        WD_STAMP(1);
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) p[(lane + 64 * m) * 8 + i] = v[8 * m + i];
+        WD_STAMP(2);
+    } else if (wave <= 4) {
+        const int base = (wave - 1) * 64 * NL + lane * NL;
+        float lv[NL];
+#pragma unroll
+        for (int i = 0; i < NL; ++i)
+            lv[i] = (base + i < n) ? __hip_atomic_load(logits + base + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
+        float cand = -INFINITY;
+        int cand_id = -1;
+        for (int j = 0; j < k; ++j) {
+            float bv = lv[0];
+#pragma unroll
+            for (int i = 1; i < NL; ++i) bv = __builtin_fmaxf(bv, lv[i]);
+            int slot = NL - 1;
+#pragma unroll
+            for (int i = NL - 2; i >= 0; --i) slot = (lv[i] == bv) ? i : slot;
+            const float best = wave_max(bv);
+            int win = -1;
+            if (best > -INFINITY) {
+                const unsigned long long mask = __builtin_amdgcn_ballot_w64(bv == best);
+                const int wl = __builtin_ctzll(mask);
+                const int ws = __builtin_amdgcn_readlane(slot, wl);
+                win = (wave - 1) * 64 * NL + wl * NL + ws;
+#pragma unroll
+                for (int i = 0; i < NL; ++i) lv[i] = (lane == wl && ws == i) ? -INFINITY : lv[i];
+            }
+            if (lane == j) {
+                cand = best;
+                cand_id = win;
+            }
+        }
+        if (lane < 16) {
+            cv[(wave - 1) * 16 + lane] = (lane < k) ? cand : -INFINITY;
+            ci[(wave - 1) * 16 + lane] = (lane < k) ? cand_id : -1;
+        }
+        wave_lds_fence();
+        if (wave > 1) {
+            if (lane == 0) __hip_atomic_store(&ready[wave - 2], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        } else {
+            // wave 1 merges as soon as the three other quarters are in LDS (flags instead of a workgroup
+            // barrier, which would also wait for wave 0).  The wait is bounded: candidates that are wrong or
+            // missing only send wave 0 down its own complete path.
+            if (lane == 0) {
+                for (int spin = 0; spin < (1 << 16); ++spin) {
+                    if (__hip_atomic_load(&ready[0], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) &&
+                        __hip_atomic_load(&ready[1], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) &&
+                        __hip_atomic_load(&ready[2], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP))
+                        break;
+                    __builtin_amdgcn_s_sleep(1);
+                }
+            }
+            wave_lds_fence();
+            // lane = quarter * 16 + rung: equal logits appear in ascending expert order along the lanes
+            float c = cv[lane];
+            const int id = ci[lane];
+            int sel_mine = -1;
+            for (int j = 0; j < k; ++j) {
+                const float best = wave_max(c);
+                int wid = -1;
+                if (best > -INFINITY) {
+                    const unsigned long long mask = __builtin_amdgcn_ballot_w64(c == best);
+                    const int wl = __builtin_ctzll(mask);
+                    wid = __builtin_amdgcn_readlane(id, wl);
+                    c = (lane == wl) ? -INFINITY : c;
+                }
+                if (lane == j) sel_mine = wid;
+            }
+            if (lane < 16) sel[lane] = sel_mine;
+        }
+    }
+    __syncthreads();
+    WD_STAMP(4);
+    if (wave == 0) {
+        const int id = (lane < k) ? sel[lane] : -1;
+        const bool have = id >= 0 && id < n;
+        const float top = have ? p[id] : 0.0f;
+        wave_lds_fence();
+        if (have) p[id] = -INFINITY;
+        wave_lds_fence();
+        float rest = -INFINITY;
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) rest = __builtin_fmaxf(rest, p[(lane + 64 * m) * 8 + i]);
+        rest = wave_max(rest);
+        const float nxt = lane_get(top, (lane + 1) & 63);
+        const bool good = lane >= k || (have && (lane == k - 1 ? top > rest : top > nxt));
+        const bool all_good = !dead && __builtin_amdgcn_ballot_w64(good) == ~0ull;
+        float top_mine = top;
+        int id_mine = id;
+        WD_STAMP(5);
+        if (!all_good) rungs_on_probs<M>(v, k, lane, top_mine, id_mine);
+        finish_weights(top_mine, id_mine, k, w_scale, ids, weights, override_ids, lane);
+        WD_STAMP(6);
+    }
+#undef WD_STAMP
+}
+
+WD_DEV void topk_block(const float *logits, int n, int k, float w_scale, int32_t *ids, float *weights,
+                       const int32_t *__restrict__ override_ids, uint8_t *lds, int lane, int wave,
+                       unsigned long long *stamps = nullptr) {
+    if (n <= 512)
+        topk_block_m<1>(logits, n, k, w_scale, ids, weights, override_ids, lds, lane, wave, stamps);
+    else
+        topk_block_m<2>(logits, n, k, w_scale, ids, weights, override_ids, lds, lane, wave, stamps);
 }
 
 template <bool COHERENT>
@@ -472,33 +651,38 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
         if (threadIdx.x == 0)
             s_last = (__hip_atomic_fetch_add(a.arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
                       static_cast<unsigned>(a.n_router_wgs - 1));
+        if (threadIdx.x < 3) topk_ready_flags(s_union, a.E)[threadIdx.x] = 0;
         __syncthreads();
-        if (s_last && wave == 0) {
+        if (s_last) {
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-            if (a.trace && lane == 0) a.trace[(0 * 16 + 8) * 8 + 0] = wall_clock64();
-            int32_t *lds_ids = reinterpret_cast<int32_t *>(s_union);
-            float *lds_w = reinterpret_cast<float *>(s_union + 64);
-            topk_wave<true>(a.logits, a.E, a.k, a.w_scale, lds_ids, lds_w, a.ids_override, lane);
-            wave_lds_fence();
-            const int id = lds_ids[lane & 15];
-            // replicas first (the routed workgroups wait for them), then the plain copies for dispatch C
+            if (a.trace && threadIdx.x == 0) a.trace[(0 * 16 + 8) * 8 + 0] = wall_clock64();
+            // results land behind the selection's own scratch
+            int32_t *lds_ids = reinterpret_cast<int32_t *>(s_union + 4 * (1024 + 160));
+            float *lds_w = reinterpret_cast<float *>(s_union + 4 * (1024 + 160) + 64);
+            topk_block(a.logits, a.E, a.k, a.w_scale, lds_ids, lds_w, a.ids_override, s_union, lane, wave,
+                       a.trace ? a.trace + (0 * 16 + 9) * 8 : nullptr);
+            if (wave == 0) {
+                wave_lds_fence();
+                const int id = lds_ids[lane & 15];
+                // replicas first (the routed workgroups wait for them), then the plain copies for dispatch C
 #pragma unroll 4
-            for (int c = 0; c < kTagCopies; ++c)
-                if (lane < a.k)
-                    __hip_atomic_store(a.ids_tagged + c * 16 + lane, static_cast<uint32_t>(id), __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-            if (lane < a.k) {
-                a.ids[lane] = id;
-                a.weights[lane] = lds_w[lane];
-            }
-            if (lane == 0) {
+                for (int c = 0; c < kTagCopies; ++c)
+                    if (lane < a.k)
+                        __hip_atomic_store(a.ids_tagged + c * 16 + lane, static_cast<uint32_t>(id), __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                if (lane < a.k) {
+                    a.ids[lane] = id;
+                    a.weights[lane] = lds_w[lane];
+                }
+                if (a.trace && lane == 0) a.trace[(0 * 16 + 8) * 8 + 1] = wall_clock64();
+            } else if (wave == 5 && lane == 0) {
+                // off the selection's path: the shared expert's gate, and the counter for the next layer pass
                 if (a.sh_inp) {
                     const float g = __hip_atomic_load(a.shared_gate, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     a.shared_gate[0] = sigmoid_ggml(g);
                 }
                 a.arrive[0] = 0u;
             }
-            if (a.trace && lane == 0) a.trace[(0 * 16 + 8) * 8 + 1] = wall_clock64();
         }
         mark(a, 0, 2);
         return;
