@@ -109,6 +109,59 @@ WD_DEV void wave_quantize_q8_k_block(const float *__restrict__ x256, int8_t *qs2
 // ascending order, k rungs of "largest remaining probability, lowest index on ties", renormalise.
 // COHERENT: the logits were written by other workgroups of the same dispatch; they are read with
 // device-scope atomic loads so that no stale cached copy can be seen.
+// Wave-wide exact sum of doubles (any order gives the same bits when the caller has made sure that the sum is
+// exact); the result is uniform.
+WD_DEV double wave_sum_exact_f64(double v) {
+    auto step = [](double x, auto mover) {
+        const uint64_t b = __builtin_bit_cast(uint64_t, x);
+        const int lo = mover(static_cast<int>(b & 0xffffffffu)), hi = mover(static_cast<int>(b >> 32));
+        return x + __builtin_bit_cast(double, (static_cast<uint64_t>(static_cast<uint32_t>(hi)) << 32) | static_cast<uint32_t>(lo));
+    };
+    v = step(v, [](int w) { return dpp_i<kDppXor1>(0, w); });
+    v = step(v, [](int w) { return dpp_i<kDppXor2>(0, w); });
+    v = step(v, [](int w) { return dpp_i<0x141>(0, w); });                     // row_half_mirror: quads 0/1, 2/3 of a row
+    v = step(v, [](int w) { return dpp_i<0x140>(0, w); });                     // row_mirror: the two halves of a row
+    v = step(v, [](int w) { return dpp_i<kDppBcast15, 0xa, 0xf, true>(0, w); });  // rows 1, 3 += lane 15 of rows 0, 2
+    v = step(v, [](int w) { return dpp_i<kDppBcast31, 0xc, 0xf, true>(0, w); });  // rows 2, 3 += lane 31
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(b & 0xffffffffu), 63));
+    const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(b >> 32), 63));
+    return __builtin_bit_cast(double, (static_cast<uint64_t>(hi) << 32) | lo);
+}
+
+// Sum of the group sums as the reference takes it (a double accumulated in ascending group order); gs[m] of lane
+// l is the sum of group l + 64 m.  When every non-zero group sum is within a factor 2^20 of the largest, all of
+// them are multiples of one power of two and every partial sum fits 53 bits, so the result is exact and the same
+// in any order: a lane tree then replaces the chain of dependent double additions.
+template <int M>
+WD_DEV double sum_groups(const float (&gs)[M], int groups, int lane) {
+    float gmax = 0.0f, gmin = INFINITY;
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+        gmax = __builtin_fmaxf(gmax, gs[m]);
+        gmin = __builtin_fminf(gmin, gs[m] > 0.0f ? gs[m] : INFINITY);
+    }
+    gmax = wave_max(gmax);
+    gmin = -wave_max(-gmin);
+    double sum = 0.0;
+    if (gmin >= gmax * 0x1p-20f && gmax < INFINITY) {
+        double part = 0.0;
+#pragma unroll
+        for (int m = 0; m < M; ++m) part += static_cast<double>(gs[m]);
+        sum = wave_sum_exact_f64(part);
+    } else {
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+#pragma unroll
+            for (int l = 0; l < 64; ++l) {
+                const float gl = readlane_f(gs[m], l);
+                if (l + 64 * m < groups) sum += static_cast<double>(gl);
+            }
+        }
+    }
+    return sum;
+}
+
 // Softmax of the row: lane l ends up with the probabilities of its 8-expert group(s) in v (or -inf everywhere
 // when every exponential vanished: `dead`).
 template <int M, bool COHERENT>
@@ -147,36 +200,7 @@ WD_DEV void softmax_probs(const float *logits, int n, int lane, float (&v)[8 * M
         const float hi = v[8 * m + 1] + v[8 * m + 5], hh = v[8 * m + 3] + v[8 * m + 7];
         gs[m] = (lo + lh) + (hi + hh);
     }
-    // The reference accumulates the group sums into a double in ascending group order.  When every non-zero
-    // group sum is within a factor 2^20 of the largest, all of them are multiples of one power of two and every
-    // partial sum fits 53 bits, so the result is exact and the same in any order: a lane tree then replaces
-    // the chain of (up to 128) dependent double additions.
-    float gmax = 0.0f, gmin = INFINITY;
-#pragma unroll
-    for (int m = 0; m < M; ++m) {
-        gmax = __builtin_fmaxf(gmax, gs[m]);
-        gmin = __builtin_fminf(gmin, gs[m] > 0.0f ? gs[m] : INFINITY);
-    }
-    gmax = wave_max(gmax);
-    gmin = -wave_max(-gmin);
-    double sum = 0.0;
-    if (gmin >= gmax * 0x1p-20f && gmax < INFINITY) {
-        double part = 0.0;
-#pragma unroll
-        for (int m = 0; m < M; ++m) part += static_cast<double>(gs[m]);
-#pragma unroll
-        for (int o = 32; o >= 1; o >>= 1) part += lane_xor(part, o);
-        sum = part;
-    } else {
-#pragma unroll
-        for (int m = 0; m < M; ++m) {
-#pragma unroll
-            for (int l = 0; l < 64; ++l) {
-                const float gl = readlane_f(gs[m], l);
-                if (l + 64 * m < groups) sum += static_cast<double>(gl);
-            }
-        }
-    }
+    const double sum = sum_groups<M>(gs, groups, lane);
     dead = (sum == 0.0);
     const float inv = dead ? 0.0f : static_cast<float>(1.0 / sum);
 #pragma unroll
@@ -251,133 +275,197 @@ WD_DEV void topk_wave_m(const float *logits, int n, int k, float w_scale, int32_
     finish_weights(top_mine, id_mine, k, w_scale, ids, weights, override_ids, lane);
 }
 
-// The same selection by a whole workgroup (at least five waves; every wave must call it).  Wave 0 computes
-// the probabilities; meanwhile waves 1..4 each find the k largest LOGITS of a quarter of the row and wave 1
-// merges them into k candidates.  exp is monotone only up to rounding, so the candidates are then checked
-// against the probabilities: they are the reference's selection exactly when their probabilities are strictly
-// decreasing and the last one is strictly above every probability left.  If not (ties, rounding inversions,
-// rows with -inf or NaN) wave 0 falls back to the rungs over the probabilities it still holds.
-// lds: scratch of 4 * (512 * M + 160) bytes whose three `ready` words (see topk_ready_flags) the caller zeroes before
-// the barrier that precedes the call.  The results are written by wave 0 (lanes 0..k-1).
-WD_DEV int *topk_ready_flags(uint8_t *lds, int n) {
-    return reinterpret_cast<int *>(lds) + 512 * (n <= 512 ? 1 : 2) + 64 + 64 + 16;
-}
-
+// The same selection by a workgroup of eight waves (every thread must call it; it contains barriers).
+// Expert m * 512 + 64 * wave + lane belongs to (wave, lane): one or two logits per lane.  A wave instruction
+// takes four cycles and a chain of k dependent arg-max steps costs about 0.2 us each, so candidates are found by
+// counting instead:
+//   1. every lane counts how many LOGITS of its wave are larger than its own (one uniform read and a compare per
+//      value): its rank in the wave.  Ranks below k form the wave's sorted candidate list;
+//   2. the eight lists are merged the same way: the rank of a candidate is its rank in its own list plus, for
+//      every other list, the number of entries ahead of it (each wave counts its own list against all
+//      candidates and adds the counts in LDS); rank r < k makes it candidate r.  Meanwhile the exponentials and
+//      the per-8 sums (a group is eight consecutive lanes) are computed eight waves wide;
+//   3. exp is monotone only up to rounding and equal probabilities must go to the lower id, so the candidates
+//      are checked against the probabilities: they are the reference's selection exactly when their
+//      probabilities are strictly decreasing and the last one is strictly above every probability left.
+//      If not (ties - which also make the counted ranks collide -, rounding inversions, rows with -inf or NaN,
+//      a dead row) wave 0 runs the reference's rungs over the probabilities themselves.
+// lds: 4 * (512 * M + 600) bytes of scratch.  The results are written by wave 0 (lanes 0..k-1).
 template <int M>
 WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32_t *ids, float *weights,
                          const int32_t *__restrict__ override_ids, uint8_t *lds, int lane, int wave,
                          unsigned long long *stamps = nullptr) {
 #define WD_STAMP(i) do { if (stamps && wave == 0 && lane == 0) stamps[i] = wall_clock64(); } while (0)
-    float *p = reinterpret_cast<float *>(lds);          // [512 * M] probabilities
-    float *cv = p + 512 * M;                            // [4][16] candidate logits of the quarters
-    int *ci = reinterpret_cast<int *>(cv + 64);         // [4][16] their expert ids
-    int *sel = ci + 64;                                 // [16] merged candidates
-    int *ready = sel + 16;                              // [3] quarters 1..3 are in LDS; zeroed by the caller before its barrier
-    constexpr int NL = 2 * M;                           // logits per lane in a quarter
-    float v[8 * M];
-    bool dead = false;
-    if (wave == 0) {
-        WD_STAMP(0);
-        softmax_probs<M, true>(logits, n, lane, v, dead);
-        WD_STAMP(1);
+    float *p = reinterpret_cast<float *>(lds);        // [512 M] probabilities by expert id
+    float *wmax = p + 512 * M;                        // [8] largest logit of each wave
+    float *gsum = wmax + 8;                           // [64 M] per-8 sums by group
+    float *cv = gsum + 64 * M;                        // [8][16] sorted candidate logits of each wave
+    int *ci = reinterpret_cast<int *>(cv + 128);      // [8][16] their ids (-1: none)
+    int *rank = ci + 128;                             // [8][16] global ranks
+    int *sel = rank + 128;                            // [16] candidate r
+    float *selp = reinterpret_cast<float *>(sel + 16);  // [16] its probability
+    float *rest = selp + 16;                          // [8] largest unselected probability of each wave
+    float *bc = rest + 8;                             // [2] 1 / sum, dead flag
+    const int groups = n >> 3;
+    WD_STAMP(0);
+
+    // 1. logits, largest of the wave, rank of every value inside the wave
+    float l[M];
+    int id[M];
 #pragma unroll
-        for (int m = 0; m < M; ++m)
+    for (int m = 0; m < M; ++m) {
+        id[m] = m * 512 + wave * 64 + lane;
+        l[m] = (id[m] < n) ? __hip_atomic_load(logits + id[m], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
+    }
+    if (lane < 16) {
+        cv[wave * 16 + lane] = -INFINITY;
+        ci[wave * 16 + lane] = -1;
+        rank[wave * 16 + lane] = lane;
+        if (wave == 0) sel[lane] = -1;
+    }
+    float lm = l[0];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) p[(lane + 64 * m) * 8 + i] = v[8 * m + i];
-        WD_STAMP(2);
-    } else if (wave <= 4) {
-        const int base = (wave - 1) * 64 * NL + lane * NL;
-        float lv[NL];
+    for (int m = 1; m < M; ++m) lm = __builtin_fmaxf(lm, l[m]);
+    lm = wave_max(lm);
+    if (lane == 0) wmax[wave] = lm;
+    WD_STAMP(1);
+    {
+        int larger[M];
 #pragma unroll
-        for (int i = 0; i < NL; ++i)
-            lv[i] = (base + i < n) ? __hip_atomic_load(logits + base + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
-        float cand = -INFINITY;
-        int cand_id = -1;
-        for (int j = 0; j < k; ++j) {
-            float bv = lv[0];
+        for (int m = 0; m < M; ++m) larger[m] = 0;
 #pragma unroll
-            for (int i = 1; i < NL; ++i) bv = __builtin_fmaxf(bv, lv[i]);
-            int slot = NL - 1;
+        for (int m2 = 0; m2 < M; ++m2) {
 #pragma unroll
-            for (int i = NL - 2; i >= 0; --i) slot = (lv[i] == bv) ? i : slot;
-            const float best = wave_max(bv);
-            int win = -1;
-            if (best > -INFINITY) {
-                const unsigned long long mask = __builtin_amdgcn_ballot_w64(bv == best);
-                const int wl = __builtin_ctzll(mask);
-                const int ws = __builtin_amdgcn_readlane(slot, wl);
-                win = (wave - 1) * 64 * NL + wl * NL + ws;
+            for (int src = 0; src < 64; ++src) {
+                const float other = readlane_f(l[m2], src);
 #pragma unroll
-                for (int i = 0; i < NL; ++i) lv[i] = (lane == wl && ws == i) ? -INFINITY : lv[i];
+                for (int m = 0; m < M; ++m) larger[m] += (other > l[m]) ? 1 : 0;
             }
-            if (lane == j) {
-                cand = best;
-                cand_id = win;
-            }
-        }
-        if (lane < 16) {
-            cv[(wave - 1) * 16 + lane] = (lane < k) ? cand : -INFINITY;
-            ci[(wave - 1) * 16 + lane] = (lane < k) ? cand_id : -1;
         }
         wave_lds_fence();
-        if (wave > 1) {
-            if (lane == 0) __hip_atomic_store(&ready[wave - 2], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
-        } else {
-            // wave 1 merges as soon as the three other quarters are in LDS (flags instead of a workgroup
-            // barrier, which would also wait for wave 0).  The wait is bounded: candidates that are wrong or
-            // missing only send wave 0 down its own complete path.
-            if (lane == 0) {
-                for (int spin = 0; spin < (1 << 16); ++spin) {
-                    if (__hip_atomic_load(&ready[0], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) &&
-                        __hip_atomic_load(&ready[1], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) &&
-                        __hip_atomic_load(&ready[2], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP))
-                        break;
-                    __builtin_amdgcn_s_sleep(1);
-                }
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            if (larger[m] < k && l[m] > -INFINITY) {
+                cv[wave * 16 + larger[m]] = l[m];
+                ci[wave * 16 + larger[m]] = id[m];
             }
-            wave_lds_fence();
-            // lane = quarter * 16 + rung: equal logits appear in ascending expert order along the lanes
-            float c = cv[lane];
-            const int id = ci[lane];
-            int sel_mine = -1;
-            for (int j = 0; j < k; ++j) {
-                const float best = wave_max(c);
-                int wid = -1;
-                if (best > -INFINITY) {
-                    const unsigned long long mask = __builtin_amdgcn_ballot_w64(c == best);
-                    const int wl = __builtin_ctzll(mask);
-                    wid = __builtin_amdgcn_readlane(id, wl);
-                    c = (lane == wl) ? -INFINITY : c;
-                }
-                if (lane == j) sel_mine = wid;
-            }
-            if (lane < 16) sel[lane] = sel_mine;
         }
     }
     __syncthreads();
-    WD_STAMP(4);
+    WD_STAMP(2);
+
+    // 2. exponentials and per-8 sums; this wave's list counted against every candidate of the other lists
+    float mx = wmax[0];
+#pragma unroll
+    for (int w = 1; w < 8; ++w) mx = __builtin_fmaxf(mx, wmax[w]);
+    float e[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+        e[m] = (id[m] < n) ? exp_ggml(l[m] - mx) : 0.0f;
+        const float gs = close_lanes8(e[m]);
+        if ((lane & 7) == 0) gsum[m * 64 + wave * 8 + (lane >> 3)] = gs;
+    }
+    {
+        float4 own_v[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) own_v[t] = *reinterpret_cast<const float4 *>(cv + wave * 16 + 4 * t);
+        const float val0 = cv[lane], val1 = cv[64 + lane];
+        int ahead0 = 0, ahead1 = 0;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float vv[4] = {own_v[t].x, own_v[t].y, own_v[t].z, own_v[t].w};
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                // empty entries hold -inf and are ahead of nothing; equal values collide (and fail the check)
+                ahead0 += (vv[u] > val0) ? 1 : 0;
+                ahead1 += (vv[u] > val1) ? 1 : 0;
+            }
+        }
+        if ((lane >> 4) != wave && ahead0) atomicAdd(&rank[lane], ahead0);
+        if ((4 + (lane >> 4)) != wave && ahead1) atomicAdd(&rank[64 + lane], ahead1);
+    }
+    __syncthreads();
+    WD_STAMP(3);
+
+    // wave 0: the denominator.  Waves 1, 2: candidates with rank < k take their place.
     if (wave == 0) {
-        const int id = (lane < k) ? sel[lane] : -1;
-        const bool have = id >= 0 && id < n;
-        const float top = have ? p[id] : 0.0f;
-        wave_lds_fence();
-        if (have) p[id] = -INFINITY;
-        wave_lds_fence();
-        float rest = -INFINITY;
+        float gs[M];
 #pragma unroll
-        for (int m = 0; m < M; ++m)
+        for (int m = 0; m < M; ++m) gs[m] = (lane + 64 * m < groups) ? gsum[m * 64 + lane] : 0.0f;
+        const double sum = sum_groups<M>(gs, groups, lane);
+        if (lane == 0) {
+            bc[0] = (sum == 0.0) ? 0.0f : static_cast<float>(1.0 / sum);
+            bc[1] = (sum == 0.0) ? 1.0f : 0.0f;
+        }
+    } else if (wave <= 2) {
+        const int c = (wave - 1) * 64 + lane;
+        const int r = rank[c];
+        if (ci[c] >= 0 && r < k) sel[r] = ci[c];
+    }
+    __syncthreads();
+    WD_STAMP(4);
+
+    // 3. probabilities; the candidates' ones and the largest of the rest
+    const float inv = bc[0];
+    const bool dead = bc[1] != 0.0f;
+    float pv[M];
+    bool taken[M];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) rest = __builtin_fmaxf(rest, p[(lane + 64 * m) * 8 + i]);
-        rest = wave_max(rest);
-        const float nxt = lane_get(top, (lane + 1) & 63);
-        const bool good = lane >= k || (have && (lane == k - 1 ? top > rest : top > nxt));
+    for (int m = 0; m < M; ++m) {
+        pv[m] = (id[m] < n && !dead) ? e[m] * inv : -INFINITY;
+        p[id[m]] = pv[m];
+        taken[m] = false;
+    }
+    {
+        int4 sq[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) sq[t] = *reinterpret_cast<const int4 *>(sel + 4 * t);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int sj[4] = {sq[t].x, sq[t].y, sq[t].z, sq[t].w};
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    if (4 * t + u < k && id[m] == sj[u]) {
+                        taken[m] = true;
+                        selp[4 * t + u] = pv[m];
+                    }
+                }
+            }
+        }
+    }
+    float rm = -INFINITY;
+#pragma unroll
+    for (int m = 0; m < M; ++m) rm = __builtin_fmaxf(rm, taken[m] ? -INFINITY : pv[m]);
+    rm = wave_max(rm);
+    if (lane == 0) rest[wave] = rm;
+    __syncthreads();
+    WD_STAMP(5);
+
+    if (wave == 0) {
+        const int idc = (lane < k) ? sel[lane] : -1;
+        const bool have = idc >= 0 && idc < n;
+        const float top = have ? selp[lane] : 0.0f;
+        float rest_all = rest[0];
+#pragma unroll
+        for (int w = 1; w < 8; ++w) rest_all = __builtin_fmaxf(rest_all, rest[w]);
+        const float nxt = dpp_f<kDppShl1>(0.0f, top);  // k <= 16: the candidates sit in one row of lanes
+        const bool good = lane >= k || (have && (lane == k - 1 ? top > rest_all : top > nxt));
         const bool all_good = !dead && __builtin_amdgcn_ballot_w64(good) == ~0ull;
         float top_mine = top;
-        int id_mine = id;
-        WD_STAMP(5);
-        if (!all_good) rungs_on_probs<M>(v, k, lane, top_mine, id_mine);
-        finish_weights(top_mine, id_mine, k, w_scale, ids, weights, override_ids, lane);
+        int id_mine = idc;
+        if (!all_good) {
+            float v[8 * M];
+#pragma unroll
+            for (int m = 0; m < M; ++m)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[8 * m + i] = p[(lane + 64 * m) * 8 + i];
+            rungs_on_probs<M>(v, k, lane, top_mine, id_mine);
+        }
         WD_STAMP(6);
+        finish_weights(top_mine, id_mine, k, w_scale, ids, weights, override_ids, lane);
+        WD_STAMP(7);
     }
 #undef WD_STAMP
 }
@@ -651,14 +739,13 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
         if (threadIdx.x == 0)
             s_last = (__hip_atomic_fetch_add(a.arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
                       static_cast<unsigned>(a.n_router_wgs - 1));
-        if (threadIdx.x < 3) topk_ready_flags(s_union, a.E)[threadIdx.x] = 0;
         __syncthreads();
         if (s_last) {
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
             if (a.trace && threadIdx.x == 0) a.trace[(0 * 16 + 8) * 8 + 0] = wall_clock64();
             // results land behind the selection's own scratch
-            int32_t *lds_ids = reinterpret_cast<int32_t *>(s_union + 4 * (1024 + 160));
-            float *lds_w = reinterpret_cast<float *>(s_union + 4 * (1024 + 160) + 64);
+            int32_t *lds_ids = reinterpret_cast<int32_t *>(s_union + 4 * (1024 + 600));
+            float *lds_w = reinterpret_cast<float *>(s_union + 4 * (1024 + 600) + 64);
             topk_block(a.logits, a.E, a.k, a.w_scale, lds_ids, lds_w, a.ids_override, s_union, lane, wave,
                        a.trace ? a.trace + (0 * 16 + 9) * 8 : nullptr);
             if (wave == 0) {
