@@ -54,7 +54,8 @@ def parse():
                     help="lru mode: tokens run before the warm-up steps so that the slot pool is in steady state")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a captured HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--cpu-seconds", type=float, default=6.0,
+                    help="wall-clock seconds of CPU layer passes to accumulate for cpu_baseline (all host threads busy)")
     ap.add_argument("--check", action="store_true", help="verify one layer pass against the CPU oracle first")
     return ap.parse_args()
 
@@ -124,8 +125,8 @@ def cpu_child(seconds, threads, kind):
     expert; router through the C port) or of the C port alone, and prints one progress line per pass."""
     from oracle import pyoracle
     from warpdecode_amd import synth
-    n_exp = 128
-    layers = [synth.make_c2(layer=l, n_experts=n_exp) for l in range(2)]       # 2 x 258 MB of expert bytes
+    n_exp = 64
+    layers = [synth.make_c2(layer=l, n_experts=n_exp) for l in range(2)]       # 2 x 129 MB of expert bytes
     rng = synth.rng_for(synth.BASE_SEED, 9002)
     x = synth.rms_normed(rng, 2048)
     print("READY", flush=True)
@@ -181,7 +182,7 @@ def cpu_baseline(seconds):
             while proc.poll() is None:
                 time.sleep(0.25)
                 # a pass takes milliseconds; only the start-up (weight generation) is slow
-                if time.perf_counter() - last[2] > (60.0 if last[0] == 0 else 8.0):
+                if time.perf_counter() - last[2] > (60.0 if last[0] == 0 else 2.5):
                     stalls += 1
                     proc.kill()
                     break
@@ -192,7 +193,7 @@ def cpu_baseline(seconds):
         if tot_passes >= 8:
             per_layer = tot_time / tot_passes
             return dict(value=round(1.0 / (per_layer * 48), 3), unit="tok/s", cores=threads, kind=kind,
-                        sample="%d C2 layer passes (512-expert layer shape, ids Zipf(1.1) over 128 resident experts, "
+                        sample="%d C2 layer passes (512-expert layer shape, ids Zipf(1.1) over 64 resident experts, "
                                "2 layers' weights alternating) in %.1f s = %.2f ms/layer, x48 layers per token; "
                                "%d threads on %d host cores%s"
                                % (tot_passes, tot_time, per_layer * 1e3, threads, cpus,

@@ -335,7 +335,8 @@ WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32
         for (int m = 0; m < M; ++m) larger[m] = 0;
 #pragma unroll
         for (int m2 = 0; m2 < M; ++m2) {
-#pragma unroll
+            // (partial unroll: a full one keeps every broadcast value in a scalar register at once)
+#pragma unroll 16
             for (int src = 0; src < 64; ++src) {
                 const float other = readlane_f(l[m2], src);
 #pragma unroll
