@@ -1,13 +1,14 @@
-// Fused MoE layer: three dispatches per layer.
-//   A  router logits (+ shared-expert gate logit); the router workgroup that finishes last runs
-//      softmax/top-k, so the ids never leave the device and the selection overlaps the shared
-//      expert's gate/up + SwiGLU, which the remaining workgroups of the same dispatch compute
-//   B  gate/up + SwiGLU of the k selected experts
+// Fused MoE layer: two dispatches per layer (three when the caller asks for the split form).
+//   AB router logits (+ shared-expert gate logit), one row per wave; the router workgroup that finishes last
+//      runs softmax/top-k and publishes the ids inside the dispatch; the shared expert's gate/up + SwiGLU and
+//      the routed gate/up + SwiGLU run in the same launch: the routed workgroups quantise x and stage the
+//      codebooks while the router runs and pick the ids up as soon as they appear
+//      (k_layer_a + k_layer_b are the same work as two launches: ids given by the caller, IQ4_NL gate/up,
+//      or WD_MOE_SPLIT_AB)
 //   C  Q8_0 re-quantisation of the k+1 activations, all down projections, the ordered weighted
 //      sum, the gated shared branch and the optional residual update
 // Activation quantisation is redone by every workgroup that needs it (8 KB of f32 from L2 and a
-// few dozen instructions per lane) instead of being a dispatch of its own, and it runs while the
-// workgroup's weight loads are already in flight.
+// few dozen instructions per lane) instead of being a dispatch of its own.
 #pragma once
 
 #include "wd_kernels.cuh"
