@@ -396,7 +396,11 @@ def main():
     ms_per_step = ev0.elapsed_time(ev1) / args.steps
     tok_s = 1000.0 / ms_per_step
     finite = bool(torch.isfinite(d_x).all().item())
+    waits_ok = capi.load().wd_moe_scratch_status(scratch) == 0   # no bounded wait inside a dispatch ran out
     note("timed region done: %.3f ms/step" % ms_per_step)
+    if not (finite and waits_ok):
+        print("bench.py: invalid run (finite=%s, in-dispatch waits ok=%s)" % (finite, waits_ok), file=sys.stderr)
+        sys.exit(1)
 
     # Algorithmic bytes of the two dispatches of one layer (weights only, as the workload prices them):
     #   AB router f32 [E][H] + the shared expert's gate vector + its Q8_0 gate and up matrices
@@ -473,7 +477,8 @@ def main():
                                % NL,
                    "layers": NL, "experts": E, "top_k": k, "routing": args.routing,
                    "launch": "eager" if graph is None else "hip-graph replay",
-                   "bytes_per_token": bytes_per_step, "wall_s": round(wall, 3), "finite": finite},
+                   "bytes_per_token": bytes_per_step, "wall_s": round(wall, 3), "finite": finite,
+                   "in_dispatch_waits_ok": waits_ok},
         "roofline": roofline,
     }
     if not args.no_cpu_baseline:
