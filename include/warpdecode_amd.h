@@ -156,6 +156,10 @@ int wd_moe_scratch_destroy(wd_moe_scratch *s);
 /* 0 when every bounded wait inside the fused dispatches was satisfied so far, 1 when one ran out (the layer's
  * results are then invalid), -1 on error.  Synchronous read of one device word. */
 int wd_moe_scratch_status(wd_moe_scratch *s);
+/* Sets the number of polls after which such a wait gives up (0 = the default, seconds of waiting) and clears the
+ * status word.  For tests of the failure path: with a limit of 1 the waiting workgroups give up at once, set the
+ * status and leave without touching memory; every kernel still ends normally.  Synchronous. */
+int wd_moe_scratch_set_wait_limit(wd_moe_scratch *s, unsigned polls);
 /* Device views, named after Qwen38MoeScratch accessors (src/qwen38_moe.cuh:1701-2150). */
 float *wd_moe_scratch_logits(wd_moe_scratch *s);      /* f32 [n_experts] */
 int32_t *wd_moe_scratch_ids(wd_moe_scratch *s);       /* i32 [k] */

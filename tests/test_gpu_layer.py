@@ -94,6 +94,16 @@ def test_small_layers(g, oracle, gate_t, down_t, shared):
         check_layer(g, oracle, L, x)
 
 
+@pytest.mark.parametrize("gate_t,down_t", [(synth.IQ2_S, synth.IQ4_NL), (synth.IQ3_S, synth.Q8_0), (synth.Q8_0, synth.Q8_0)])
+def test_model_shape_layers(g, oracle, gate_t, down_t):
+    """Hidden 2560 / ffn 640 (the shapes of the reference's target model, src/qwen38_moe.cuh:3462-3514): rows
+    longer than one 2048-column span in the router and in the Q8_0 row kernels, ffn not a power of two."""
+    H, F, E, k = 2560, 640, 32, 6
+    L = synth.make_layer(H, F, E, k, gate_t, down_t, True, seed=SEED, layer=77, router_sigma=1.0 / np.sqrt(H))
+    x = synth.rms_normed(synth.rng_for(SEED, 49), H)
+    check_layer(g, oracle, L, x)
+
+
 def test_c0_layer(g, oracle):
     """Workload C0: hidden 2048, 64 experts, top-8, ffn 512, all Q8_0."""
     L = synth.make_c0()
@@ -189,4 +199,29 @@ def test_selection_more_than_512_experts(g, oracle):
 def test_status_word_is_clear(g):
     sc = g.Scratch(512, 64, 8, 2)
     assert capi.load().wd_moe_scratch_status(sc.h) == 0
+    sc.close()
+
+
+def test_bounded_wait_gives_up_and_recovers(g, oracle):
+    """Failure path of the in-dispatch hand-off, forced from the host: with a wait limit of one poll the routed
+    workgroups give up before the ids are published, the status word says so, every kernel still ends; with the
+    default limit restored the same scratch gives the oracle's result again."""
+    L = synth.make_c2(n_experts=64)
+    H, F, E, k = 2048, 512, 64, 10
+    x = synth.rms_normed(synth.rng_for(SEED, 48), H)
+    dl, sc = g.DeviceLayer(L), g.Scratch(H, F, E, k)
+    dx, out = g.dev(x), g.empty(H, np.float32)
+    lib = capi.load()
+    capi.call("wd_moe_scratch_set_wait_limit", sc.h, 1)
+    capi.call("wd_moe_layer_f32", C.byref(dl.desc), g.ptr(dx), g.ptr(out), sc.h, 0, g.stream())
+    g.sync()
+    assert lib.wd_moe_scratch_status(sc.h) == 1
+    capi.call("wd_moe_scratch_set_wait_limit", sc.h, 0)
+    assert lib.wd_moe_scratch_status(sc.h) == 0
+    capi.call("wd_moe_layer_f32", C.byref(dl.desc), g.ptr(dx), g.ptr(out), sc.h, 0, g.stream())
+    g.sync()
+    want, d = oracle.moe_layer(L, x)
+    assert lib.wd_moe_scratch_status(sc.h) == 0
+    assert np.array_equal(sc.get("ids", k, np.int32), d["ids"])
+    assert g.same_bits(g.host(out), want)
     sc.close()

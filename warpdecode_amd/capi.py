@@ -76,6 +76,7 @@ _SIGS = {
     "wd_moe_layer_f32": (i32, [C.POINTER(MoeLayer), vp, vp, vp, u32, vp]),
     "wd_moe_stack_cached_f32": (i32, [C.POINTER(MoeLayer), i32, vp, vp, vp, vp, vp, vp, f32, u32, vp]),
     "wd_moe_scratch_status": (i32, [vp]),
+    "wd_moe_scratch_set_wait_limit": (i32, [vp, u32]),
     "wd_shared_expert_f32": (i32, [C.POINTER(MoeLayer), vp, vp, vp]),
     "wd_moe_stack_f32": (i32, [C.POINTER(MoeLayer), i32, vp, vp, vp, vp, f32, u32, vp]),
 }

@@ -40,13 +40,14 @@ struct LayerArgs {
     uint32_t *ids_tagged;        // [kTagCopies][16] selected ids published inside the merged dispatch (kTagInvalid = not yet)
     int clear_tagged;            // dispatch C resets ids_tagged when it is done with the layer
     unsigned *status;            // [0] set to 1 when a bounded wait inside a dispatch ran out
+    unsigned spin_limit;         // polls (about a microsecond each) before such a wait gives up
     unsigned long long *trace;   // profiling aid: null, or [3][16][8] time stamps (100 MHz) of workgroup trace_wg
     int trace_wg;
 };
 
 constexpr int kTagCopies = 16;           // replicas of the published ids, 64 bytes apart, so that pollers spread over lines
 constexpr uint32_t kTagInvalid = 0xffffffffu;
-constexpr unsigned kSpinLimit = 1u << 21;  // polls (about a microsecond each) before a wait gives up
+constexpr unsigned kSpinLimit = 1u << 21;  // default number of polls before a wait gives up (seconds)
 
 // Time stamp `i` of dispatch `d` (0 = A, 1 = B, 2 = C) for the traced workgroup; lane 0 of every wave.
 WD_DEV void mark(const LayerArgs &a, int d, int i) {
@@ -813,7 +814,7 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
         const uint32_t *src = a.ids_tagged + (bw & (kTagCopies - 1)) * 16 + j;
         uint32_t e = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         unsigned polls = 0;
-        while (e == kTagInvalid && ++polls < kSpinLimit) {
+        while (e == kTagInvalid && ++polls < a.spin_limit) {
             __builtin_amdgcn_s_sleep(4);
             e = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }

@@ -36,6 +36,7 @@ struct wd_moe_scratch {
     int32_t *h_ids = nullptr;             // pinned [16]: routed ids for callers that must see them on the host
     uint32_t *tagged = nullptr;           // [kTagRecords][kTagCopies][16] ids published inside the merged dispatch
     unsigned *status = nullptr;           // [0] != 0: a bounded wait inside a dispatch ran out
+    unsigned spin_limit = kSpinLimit;
 };
 
 namespace {
@@ -131,6 +132,14 @@ int wd_moe_scratch_status(wd_moe_scratch *s) {
     unsigned v = 0;
     if (hipMemcpy(&v, s->status, sizeof(v), hipMemcpyDeviceToHost) != hipSuccess) return -1;
     return static_cast<int>(v);
+}
+int wd_moe_scratch_set_wait_limit(wd_moe_scratch *s, unsigned polls) {
+    WD_REQUIRE(s != nullptr, "wd_moe_scratch_set_wait_limit: null scratch");
+    s->spin_limit = polls ? polls : kSpinLimit;
+    // a fresh start: clear the status word and make the published ids invalid again
+    WD_HIP(hipMemset(s->status, 0, sizeof(unsigned)));
+    WD_HIP(hipMemset(s->tagged, 0xff, sizeof(uint32_t) * kTagRecords * kTagCopies * 16));
+    return WD_OK;
 }
 float *wd_moe_scratch_logits(wd_moe_scratch *s) { return s->logits; }
 int32_t *wd_moe_scratch_ids(wd_moe_scratch *s) { return s->ids; }
@@ -369,6 +378,7 @@ LayerArgs fused_args(const wd_moe_layer *L, const float *d_x, float *d_out, wd_m
     a.ids_tagged = s->tagged + static_cast<size_t>(rec % kTagRecords) * kTagCopies * 16;
     a.clear_tagged = 1;
     a.status = s->status;
+    a.spin_limit = s->spin_limit;
     return a;
 }
 
