@@ -230,6 +230,9 @@ def bench_lru(args, torch, capi, synth):
     capi.call("wd_expert_cache_create", C.byref(cache), int(args.cache_gib * (1 << 30)), gb, gb, db, NL, E, 0)
     for l in range(NL):
         capi.call("wd_expert_cache_register_layer", cache, l, *pinned[l])
+    st_slots = int(args.cache_gib * (1 << 30)) // slot_bytes
+    for policy, slots in ((0, st_slots // 2), (0, 2 * st_slots), (1, st_slots)):   # counterfactual pools, same accesses
+        capi.call("wd_expert_cache_add_shadow", cache, policy, slots)
     scratch = C.c_void_p()
     capi.call("wd_moe_scratch_create", C.byref(scratch), H, F, E, k)
     st0 = capi.CacheStats()
@@ -282,6 +285,13 @@ def bench_lru(args, torch, capi, synth):
     ms_per_step = ev0.elapsed_time(ev1) / args.steps
     acc, hits, miss = s1.accesses - s0.accesses, s1.hits - s0.hits, s1.misses - s0.misses
     moved = s1.bytes_copied - s0.bytes_copied
+    lib = capi.load()
+    need = lib.wd_expert_cache_dump_json(cache, None, 0)
+    buf = C.create_string_buffer(need + 1)
+    lib.wd_expert_cache_dump_json(cache, buf, need + 1)
+    monitor = json.loads(buf.value.decode())
+    for key in ("layer_access", "layer_misses"):
+        monitor.pop(key, None)
     bytes_per_step = 27697152 * NL if E == 512 else None
     whole = bytes_per_step / (ms_per_step * 1e-3) / 1e9 if bytes_per_step else None
     out = {
@@ -297,7 +307,8 @@ def bench_lru(args, torch, capi, synth):
                    "hit_rate": round(hits / max(1, acc), 4), "misses_per_token": round(miss / args.steps, 2),
                    "host_link_bytes_per_token": int(moved / args.steps),
                    "host_link_GBps": round(moved / (ms_per_step * 1e-3 * args.steps) / 1e9, 2),
-                   "wall_s": round(wall, 3), "finite": bool(torch.isfinite(d_x).all().item())},
+                   "wall_s": round(wall, 3), "finite": bool(torch.isfinite(d_x).all().item()),
+                   "monitor_whole_run": monitor},
         "roofline": {"bound": "hbm", "achieved": round(whole, 1) if whole else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(whole / HBM_PEAK_GBS, 4) if whole else None, "traffic": None,
                      "kernel": "whole step (kernel bytes only; the host-link bytes are in config)"},

@@ -256,6 +256,15 @@ const uint8_t *wd_expert_cache_pool(wd_expert_cache *c);
  * ExpertDeviceWeights, src/expert_cache.cuh:2148-2154). */
 long long wd_expert_cache_slot_of(wd_expert_cache *c, int layer, int expert);
 int wd_expert_cache_get_stats(wd_expert_cache *c, wd_expert_cache_stats *out);
+/* Counterfactual caches that see the same (layer, expert) accesses as the pool and hold keys only: what would a pool
+ * of `slots` have hit under LRU (policy 0) or exact LFU (policy 1)?  Add them before the first acquire.
+ * reference: ShadowLru / ShadowFreq, src/expert_cache.cuh:1592-1668. */
+int wd_expert_cache_add_shadow(wd_expert_cache *c, int policy, size_t slots);
+/* The monitor's counters as one JSON object (hit rate, bytes copied, per-layer accesses and misses, distinct pairs,
+ * reuse of the previous call's experts per layer, host time spent in acquire, shadow hit rates).  Returns the length
+ * needed; writes at most `cap` bytes including the terminator.  reference: ExpertCacheMonitor::dump,
+ * src/expert_cache.cuh:1879-1960. */
+size_t wd_expert_cache_dump_json(wd_expert_cache *c, char *buf, size_t cap);
 
 
 /* One decode step through a stack of layers whose routed experts come from `cache` (layer l of the stack is

@@ -163,3 +163,47 @@ def test_layer_through_slot_table(g, oracle):
     assert st.misses > 24 and st.evictions > 0 and st.hits > 0
     sc.close()
     capi.call("wd_expert_cache_destroy", cache)
+
+
+def test_monitor_and_shadow_caches(g):
+    """Counters and counterfactual caches against a direct model: an LRU shadow with the pool's own capacity must
+    hit exactly as often as the pool, a larger one at least as often, and the JSON dump must carry the counters."""
+    import json
+    E, NL, k = 16, 2, 4
+    gb, ub, db = 256, 256, 512
+    slots = 6
+    host = _host_layers(NL, E, gb, ub, db, SEED + 9)
+    cache = C.c_void_p()
+    capi.call("wd_expert_cache_create", C.byref(cache), slots * (gb + ub + db), gb, ub, db, NL, E, 0)
+    capi.call("wd_expert_cache_add_shadow", cache, 0, slots)
+    capi.call("wd_expert_cache_add_shadow", cache, 0, 3 * slots)
+    capi.call("wd_expert_cache_add_shadow", cache, 1, slots)
+    import torch
+    pinned = [[torch.from_numpy(a).pin_memory() for a in layer] for layer in host]
+    for l in range(NL):
+        capi.call("wd_expert_cache_register_layer", cache, l, *[C.c_void_p(t.data_ptr()) for t in pinned[l]])
+    rng = np.random.default_rng(SEED + 10)
+    model = ModelCache(slots, NL, False)
+    big = ModelCache(3 * slots, NL, False)
+    accesses = 0
+    for step in range(40):
+        for l in range(NL):
+            ids = rng.choice(E, size=k, replace=False, p=np.arange(E, 0, -1) / np.arange(E, 0, -1).sum()).astype(np.int32)
+            capi.call("wd_expert_cache_acquire", cache, l, ids.ctypes.data_as(C.c_void_p), k, None, g.stream())
+            for e in ids:
+                model.acquire(l, int(e)); big.acquire(l, int(e))
+            accesses += k
+    g.sync()
+    lib = capi.load()
+    need = lib.wd_expert_cache_dump_json(cache, None, 0)
+    buf = C.create_string_buffer(need + 1)
+    lib.wd_expert_cache_dump_json(cache, buf, need + 1)
+    d = json.loads(buf.value.decode())
+    assert d["accesses"] == accesses and d["hits"] == model.hits and d["misses"] == model.misses
+    assert d["evictions"] == model.evictions and d["bytes_copied"] == model.misses * (gb + ub + db)
+    assert sum(d["layer_access"]) == accesses and sum(d["layer_misses"]) == model.misses
+    assert d["shadows"][0] == dict(policy="lru", slots=slots, hits=model.hits, hit_rate=round(model.hits / accesses, 4))
+    assert d["shadows"][1]["hits"] == big.hits >= model.hits
+    assert d["shadows"][2]["policy"] == "lfu" and 0 < d["shadows"][2]["hits"] <= accesses
+    assert d["distinct_pairs"] <= NL * E and 0.0 < d["prev_token_reuse"] < 1.0
+    capi.call("wd_expert_cache_destroy", cache)

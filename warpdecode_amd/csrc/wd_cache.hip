@@ -14,9 +14,14 @@
 //     the caller's stream waits for the fills, so no host thread ever blocks.
 #include "wd_common.h"
 
+#include <chrono>
+#include <cstdio>
+#include <cstring>
 #include <list>
 #include <new>
+#include <string>
 #include <unordered_map>
+#include <unordered_set>
 #include <vector>
 
 using namespace wd;
@@ -52,6 +57,59 @@ struct Partition {
     std::vector<size_t> free;    // empty slots, descending so that back() is the lowest index
 };
 
+// Counterfactual caches fed with the same (layer, expert) access trace as the real pool; they hold keys only
+// and never touch device memory (reference: ShadowLru / ShadowFreq, src/expert_cache.cuh:1592-1668).
+struct Shadow {
+    int policy = 0;  // 0 = LRU, 1 = LFU with the least recently inserted among the least frequent leaving
+    size_t capacity = 1;
+    uint64_t hits = 0, accesses = 0;
+    std::list<uint64_t> order;  // LRU: front = most recent
+    std::unordered_map<uint64_t, std::list<uint64_t>::iterator> where;
+    struct Entry {
+        uint64_t key, freq;
+    };
+    std::vector<Entry> entries;                    // LFU residents
+    std::unordered_map<uint64_t, size_t> resident; // LFU: key -> entry
+    std::unordered_map<uint64_t, uint64_t> seen;   // LFU: lifetime count of every key
+
+    void access(uint64_t key) {
+        ++accesses;
+        if (policy == 0) {
+            auto it = where.find(key);
+            if (it != where.end()) {
+                ++hits;
+                order.splice(order.begin(), order, it->second);
+                return;
+            }
+            order.push_front(key);
+            where[key] = order.begin();
+            if (order.size() > capacity) {
+                where.erase(order.back());
+                order.pop_back();
+            }
+            return;
+        }
+        const uint64_t n = ++seen[key];
+        auto it = resident.find(key);
+        if (it != resident.end()) {
+            ++entries[it->second].freq;
+            ++hits;
+            return;
+        }
+        if (entries.size() < capacity) {
+            resident[key] = entries.size();
+            entries.push_back({key, n});
+            return;
+        }
+        size_t victim = 0;
+        for (size_t i = 1; i < entries.size(); ++i)
+            if (entries[i].freq < entries[victim].freq) victim = i;
+        resident.erase(entries[victim].key);
+        entries[victim] = {key, n};
+        resident[key] = victim;
+    }
+};
+
 constexpr int kUpdateRing = 32;
 constexpr int kMaxUpdates = 64;  // 2 per missed expert, k <= 16... one acquire call never needs more
 
@@ -78,6 +136,13 @@ struct wd_expert_cache {
     bool ring_used[kUpdateRing] = {};
     int ring_next = 0;
     wd_expert_cache_stats stats{};
+    // monitor (reference: ExpertCacheMonitor, src/expert_cache.cuh:1670-2105)
+    std::vector<Shadow> shadows;
+    std::vector<uint64_t> layer_access, layer_misses;
+    std::unordered_set<uint64_t> distinct;
+    std::vector<std::vector<int32_t>> prev_ids;   // per layer: the ids of the previous acquire call
+    uint64_t prev_ready = 0, prev_hit = 0, acquire_calls = 0;
+    double acquire_ms = 0.0;
 };
 
 extern "C" {
@@ -184,6 +249,34 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
     WD_REQUIRE(P.end - P.begin >= static_cast<size_t>(k), "expert cache: %zu slots cannot hold %d experts at once",
                P.end - P.begin, k);
     hipStream_t st = as_stream(stream);
+    const auto t_begin = std::chrono::steady_clock::now();
+    struct Timer {
+        wd_expert_cache *c;
+        std::chrono::steady_clock::time_point t0;
+        ~Timer() {
+            c->acquire_ms += std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+            ++c->acquire_calls;
+        }
+    } timer{c, t_begin};
+    if (c->layer_access.size() < static_cast<size_t>(c->n_layers)) {
+        c->layer_access.assign(c->n_layers, 0);
+        c->layer_misses.assign(c->n_layers, 0);
+        c->prev_ids.assign(c->n_layers, {});
+    }
+    {   // reuse of the previous call's experts of this layer (the previous token in a decode loop)
+        std::vector<int32_t> &prev = c->prev_ids[layer];
+        if (!prev.empty()) {
+            for (int j = 0; j < k; ++j) {
+                ++c->prev_ready;
+                for (int32_t p : prev)
+                    if (p == h_ids[j]) {
+                        ++c->prev_hit;
+                        break;
+                    }
+            }
+        }
+        prev.assign(h_ids, h_ids + k);
+    }
     const uint64_t epoch_floor = c->clock;  // slots touched by this call carry last_use > epoch_floor
     const uint64_t victim_floor = defer_wait ? c->prev_floor : epoch_floor;
     c->prev_floor = epoch_floor;
@@ -197,6 +290,9 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
         const uint64_t key = (static_cast<uint64_t>(static_cast<uint32_t>(layer)) << 32) | static_cast<uint32_t>(e);
         ++c->clock;
         ++c->stats.accesses;
+        ++c->layer_access[layer];
+        c->distinct.insert(key);
+        for (Shadow &sh : c->shadows) sh.access(key);
         auto it = c->index.find(key);
         if (it != c->index.end()) {
             Slot &s = c->slots[it->second];
@@ -208,6 +304,7 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
             continue;
         }
         ++c->stats.misses;
+        ++c->layer_misses[layer];
         if (hit_out) hit_out[j] = 0;
         size_t slot;
         if (!P.free.empty()) {
@@ -301,6 +398,60 @@ long long wd_expert_cache_slot_of(wd_expert_cache *c, int layer, int expert) {
     if (!c || layer < 0 || expert < 0) return -1;
     const auto it = c->index.find((static_cast<uint64_t>(layer) << 32) | static_cast<uint32_t>(expert));
     return it == c->index.end() ? -1 : static_cast<long long>(it->second);
+}
+
+int wd_expert_cache_add_shadow(wd_expert_cache *c, int policy, size_t slots) {
+    WD_REQUIRE(c != nullptr, "expert cache is not initialized");
+    WD_REQUIRE(policy == 0 || policy == 1, "expert cache shadow: policy must be 0 (LRU) or 1 (LFU)");
+    WD_REQUIRE(c->stats.accesses == 0, "expert cache shadow: add shadows before the first acquire");
+    Shadow sh;
+    sh.policy = policy;
+    sh.capacity = slots ? slots : 1;
+    c->shadows.push_back(std::move(sh));
+    return WD_OK;
+}
+
+// JSON object with the counters; returns the length needed (without the terminator), writes at most cap bytes.
+size_t wd_expert_cache_dump_json(wd_expert_cache *c, char *buf, size_t cap) {
+    if (!c) return 0;
+    auto arr = [](const std::vector<uint64_t> &v) {
+        std::string s = "[";
+        for (size_t i = 0; i < v.size(); ++i) s += (i ? "," : "") + std::to_string(v[i]);
+        return s + "]";
+    };
+    char num[64];
+    auto fixed = [&](double v, int digits) {
+        std::snprintf(num, sizeof(num), "%.*f", digits, v);
+        return std::string(num);
+    };
+    const wd_expert_cache_stats &st = c->stats;
+    std::string s = "{";
+    s += "\"mode\":\"" + std::string(c->partitioned ? "layer-partitioned" : "shared") + "\"";
+    s += ",\"slots\":" + std::to_string(c->n_slots) + ",\"slot_bytes\":" + std::to_string(c->slot_bytes);
+    s += ",\"accesses\":" + std::to_string(st.accesses) + ",\"hits\":" + std::to_string(st.hits);
+    s += ",\"misses\":" + std::to_string(st.misses);
+    s += ",\"hit_rate\":" + fixed(st.accesses ? static_cast<double>(st.hits) / st.accesses : 0.0, 4);
+    s += ",\"evictions\":" + std::to_string(st.evictions) + ",\"bytes_copied\":" + std::to_string(st.bytes_copied);
+    s += ",\"gib_copied\":" + fixed(st.bytes_copied / (1024.0 * 1024.0 * 1024.0), 3);
+    s += ",\"resident\":" + std::to_string(c->index.size()) + ",\"distinct_pairs\":" + std::to_string(c->distinct.size());
+    s += ",\"acquire_calls\":" + std::to_string(c->acquire_calls) + ",\"acquire_ms\":" + fixed(c->acquire_ms, 1);
+    s += ",\"prev_token_ready\":" + std::to_string(c->prev_ready);
+    s += ",\"prev_token_reuse\":" + fixed(c->prev_ready ? static_cast<double>(c->prev_hit) / c->prev_ready : 0.0, 4);
+    s += ",\"layer_access\":" + arr(c->layer_access) + ",\"layer_misses\":" + arr(c->layer_misses);
+    s += ",\"shadows\":[";
+    for (size_t i = 0; i < c->shadows.size(); ++i) {
+        const Shadow &sh = c->shadows[i];
+        s += std::string(i ? "," : "") + "{\"policy\":\"" + (sh.policy ? "lfu" : "lru") + "\",\"slots\":" + std::to_string(sh.capacity) +
+             ",\"hits\":" + std::to_string(sh.hits) + ",\"hit_rate\":" +
+             fixed(sh.accesses ? static_cast<double>(sh.hits) / sh.accesses : 0.0, 4) + "}";
+    }
+    s += "]}";
+    if (buf && cap) {
+        const size_t n = s.size() < cap - 1 ? s.size() : cap - 1;
+        std::memcpy(buf, s.data(), n);
+        buf[n] = 0;
+    }
+    return s.size();
 }
 
 int wd_expert_cache_get_stats(wd_expert_cache *c, wd_expert_cache_stats *out) {
