@@ -245,6 +245,14 @@ int wd_expert_cache_destroy(wd_expert_cache *c);
 /* Host (pinned) sources of one layer's 3-D expert tensors; strides are bytes per expert. */
 int wd_expert_cache_register_layer(wd_expert_cache *c, int layer, const uint8_t *h_gate, const uint8_t *h_up,
                                    const uint8_t *h_down);
+/* The same for host tensors whose experts are further apart than their size, e.g. the fused gate_up tensor of the
+ * reference's target model (2 * ffn rows per expert, gate rows first: h_gate = base, h_up = base + ffn rows,
+ * gate_stride = up_stride = 2 * ffn rows; src/qwen38_moe.cuh:3462-3514, GpuFusedExpertCache,
+ * src/expert_cache.cuh:2546-2882).  In a wd_moe_layer the same tensor is gate = base, up = base + ffn rows with both
+ * strides 2 * ffn rows. */
+int wd_expert_cache_register_layer_strided(wd_expert_cache *c, int layer, const uint8_t *h_gate, const uint8_t *h_up,
+                                           const uint8_t *h_down, size_t gate_stride, size_t up_stride,
+                                           size_t down_stride);
 /* Makes `k` experts of `layer` resident (LRU order of the ids given), updates the device slot table
  * of that layer and returns, per id, whether it was a hit.  All k slots stay valid until the next
  * acquire call on this cache.  hit_out may be NULL. */

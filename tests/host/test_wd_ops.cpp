@@ -259,6 +259,33 @@ static void gpu_checks() {
             CHECK(std::memcmp(back.data(), expert_slice(L[0].t_gate, 5).data, v.gate.bytes) == 0 && !v.gate.owns, "acquired view must hold the expert's gate bytes");
         }
     }
+    // fused gate_up tensor (2 * ffn rows per expert) through the fused runner, LRU pool of 10+ slots
+    {
+        const size_t gb = L[0].t_gate.byte_size() / E;
+        std::vector<uint8_t> fused(2 * gb * E);
+        for (int e = 0; e < E; ++e) {
+            std::memcpy(&fused[2 * gb * e], &L[0].gate[gb * e], gb);
+            std::memcpy(&fused[2 * gb * e + gb], &L[0].up[gb * e], gb);
+        }
+        TensorInfo t_gu{"ffn_gate_up_exps.weight", {static_cast<uint64_t>(H), static_cast<uint64_t>(2 * F), static_cast<uint64_t>(E)}, GgmlType::IQ3_S, 0, fused.data()};
+        GpuExpertCache cache;
+        cache.initialize((10 * slot + (1u << 20) - 1) >> 20, L[0].t_gate, L[0].t_up, L[0].t_down, 0, 0, 0, opt);
+        Rng r(321);
+        DeviceFloatArray dx(H), dout(H);
+        for (int token = 0; token < 3; ++token) {
+            const std::vector<float> x = rms_normed(r, H);
+            dx.upload(x.data(), H);
+            run_qwen38_routed_moe_fused_f32_x(0, dx.data, routers[0], t_gu, L[0].t_down, cache, scratch, nullptr, 1.0f, stream);
+            run_qwen38_shared_expert_f32_x(dx.data, shared[0], scratch, stream);
+            q38_finish_moe_f32(scratch, dout.data, stream);
+            check(wd_stream_sync(stream), "sync");
+            std::vector<float> got(H), want(H);
+            dout.download(got.data());
+            wdo_moe_layer(&L[0].o, x.data(), want.data(), nullptr, 0);
+            CHECK(same_bits(got.data(), want.data(), H), "fused gate_up tensor, token %d: output differs from the oracle", token);
+        }
+        CHECK(wd_moe_scratch_status(scratch.handle()) == 0, "an in-dispatch wait ran out");
+    }
     wd_stream_destroy(stream);
 }
 

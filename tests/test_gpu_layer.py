@@ -225,3 +225,52 @@ def test_bounded_wait_gives_up_and_recovers(g, oracle):
     assert np.array_equal(sc.get("ids", k, np.int32), d["ids"])
     assert g.same_bits(g.host(out), want)
     sc.close()
+
+
+def test_fused_gate_up_tensor_layout(g, oracle):
+    """One tensor with 2 * ffn rows per expert (gate rows, then up rows), as the reference's target model stores
+    them (src/qwen38_moe.cuh:3462-3514): the layer descriptor addresses it in place, resident and through the
+    slot pool."""
+    import torch
+    H, F, E, k = 512, 64, 16, 4
+    L = synth.make_layer(H, F, E, k, synth.IQ3_S, synth.Q8_0, True, seed=SEED, layer=60, router_sigma=1.0 / np.sqrt(H))
+    x = synth.rms_normed(synth.rng_for(SEED, 50), H)
+    want, d = oracle.moe_layer(L, x)
+    rb = synth.row_bytes(synth.IQ3_S, H)
+    gate = np.ascontiguousarray(L["gate"]).reshape(E, F * rb)
+    up = np.ascontiguousarray(L["up"]).reshape(E, F * rb)
+    fused = np.ascontiguousarray(np.concatenate([gate, up], axis=1))          # [E][2 F rows]
+    dl = g.DeviceLayer(L)
+    dfused = g.dev(fused.reshape(-1))
+    desc = dl.desc
+    desc.gate = dfused.data_ptr()
+    desc.up = dfused.data_ptr() + F * rb
+    desc.gate_stride = desc.up_stride = 2 * F * rb
+    sc = g.Scratch(H, F, E, k)
+    dx, out = g.dev(x), g.empty(H, np.float32)
+    for flags in (0, capi.MOE_STAGED):
+        capi.call("wd_moe_layer_f32", C.byref(desc), g.ptr(dx), g.ptr(out), sc.h, flags, g.stream())
+        g.sync()
+        assert np.array_equal(sc.get("ids", k, np.int32), d["ids"])
+        assert g.same_bits(g.host(out), want)
+    # the same tensor as the host source of a slot pool
+    db = H * synth.row_bytes(synth.Q8_0, F)
+    cache = C.c_void_p()
+    capi.call("wd_expert_cache_create", C.byref(cache), 6 * (2 * F * rb + db), F * rb, F * rb, db, 1, E, 0)
+    hf = torch.from_numpy(fused.reshape(-1).copy()).pin_memory()
+    hd = torch.from_numpy(np.ascontiguousarray(L["down"]).reshape(-1)).pin_memory()
+    capi.call("wd_expert_cache_register_layer_strided", cache, 0, C.c_void_p(hf.data_ptr()),
+              C.c_void_p(hf.data_ptr() + F * rb), C.c_void_p(hd.data_ptr()), 2 * F * rb, 2 * F * rb, db)
+    lib = capi.load()
+    desc.gate = desc.up = desc.down = None
+    desc.slot_of_expert = lib.wd_expert_cache_slot_table(cache, 0)
+    desc.slot_pool = lib.wd_expert_cache_pool(cache)
+    desc.slot_bytes, desc.slot_gate_bytes, desc.slot_up_bytes = 2 * F * rb + db, F * rb, F * rb
+    arr = (capi.MoeLayer * 1)(desc)
+    out2 = g.empty(H, np.float32)
+    dx2 = g.dev(x)
+    capi.call("wd_moe_stack_cached_f32", arr, 1, cache, g.ptr(dx2), g.ptr(out2), sc.h, None, None, 0.0, 0, g.stream())
+    g.sync()
+    assert g.same_bits(g.host(out2), want)
+    sc.close()
+    capi.call("wd_expert_cache_destroy", cache)

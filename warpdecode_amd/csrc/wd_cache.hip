@@ -127,6 +127,7 @@ struct wd_expert_cache {
     uint64_t prev_floor = 0;     // clock value before the previous acquire call
     bool fills_pending = false;  // a deferred acquire's fills have not been waited for yet
     std::vector<const uint8_t *> h_gate, h_up, h_down;
+    std::vector<size_t> s_gate, s_up, s_down;  // bytes from one expert to the next in the host tensors
     int32_t *d_table = nullptr;  // [n_layers][n_experts]
     hipStream_t copy_stream = nullptr;
     hipEvent_t ev_retire = nullptr, ev_done = nullptr;
@@ -179,6 +180,7 @@ int wd_expert_cache_create(wd_expert_cache **out, size_t capacity_bytes, size_t 
     c->h_gate.assign(n_layers, nullptr);
     c->h_up.assign(n_layers, nullptr);
     c->h_down.assign(n_layers, nullptr);
+    c->s_gate.assign(n_layers, gate_bytes), c->s_up.assign(n_layers, up_bytes), c->s_down.assign(n_layers, down_bytes);
     auto bail = [&](const char *what, hipError_t e) {
         const int rc = fail(WD_ERR_HIP, "expert cache: %s failed: %s", what, hipGetErrorString(e));
         wd_expert_cache_destroy(c);
@@ -229,6 +231,17 @@ int wd_expert_cache_register_layer(wd_expert_cache *c, int layer, const uint8_t 
     WD_REQUIRE(layer >= 0 && layer < c->n_layers, "expert cache: layer %d out of range", layer);
     WD_REQUIRE(h_gate && h_up && h_down, "expert cache: null host tensor");
     c->h_gate[layer] = h_gate, c->h_up[layer] = h_up, c->h_down[layer] = h_down;
+    c->s_gate[layer] = c->gate_bytes, c->s_up[layer] = c->up_bytes, c->s_down[layer] = c->down_bytes;
+    return WD_OK;
+}
+
+int wd_expert_cache_register_layer_strided(wd_expert_cache *c, int layer, const uint8_t *h_gate, const uint8_t *h_up,
+                                           const uint8_t *h_down, size_t gate_stride, size_t up_stride,
+                                           size_t down_stride) {
+    if (const int rc = wd_expert_cache_register_layer(c, layer, h_gate, h_up, h_down)) return rc;
+    WD_REQUIRE(gate_stride >= c->gate_bytes && up_stride >= c->up_bytes && down_stride >= c->down_bytes,
+               "expert cache: an expert stride is smaller than the expert");
+    c->s_gate[layer] = gate_stride, c->s_up[layer] = up_stride, c->s_down[layer] = down_stride;
     return WD_OK;
 }
 
@@ -334,11 +347,11 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
             waited = true;
         }
         uint8_t *dst = c->pool + slot * c->slot_bytes;
-        WD_HIP(hipMemcpyAsync(dst, c->h_gate[layer] + static_cast<size_t>(e) * c->gate_bytes, c->gate_bytes,
+        WD_HIP(hipMemcpyAsync(dst, c->h_gate[layer] + static_cast<size_t>(e) * c->s_gate[layer], c->gate_bytes,
                               hipMemcpyHostToDevice, c->copy_stream));
-        WD_HIP(hipMemcpyAsync(dst + c->gate_bytes, c->h_up[layer] + static_cast<size_t>(e) * c->up_bytes, c->up_bytes,
+        WD_HIP(hipMemcpyAsync(dst + c->gate_bytes, c->h_up[layer] + static_cast<size_t>(e) * c->s_up[layer], c->up_bytes,
                               hipMemcpyHostToDevice, c->copy_stream));
-        WD_HIP(hipMemcpyAsync(dst + c->gate_bytes + c->up_bytes, c->h_down[layer] + static_cast<size_t>(e) * c->down_bytes,
+        WD_HIP(hipMemcpyAsync(dst + c->gate_bytes + c->up_bytes, c->h_down[layer] + static_cast<size_t>(e) * c->s_down[layer],
                               c->down_bytes, hipMemcpyHostToDevice, c->copy_stream));
         c->stats.bytes_copied += c->slot_bytes;
     }

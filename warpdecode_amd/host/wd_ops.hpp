@@ -366,6 +366,21 @@ public:
         reg_[static_cast<size_t>(layer)] = 1;
     }
 
+    // Fused gate_up tensor (dims {hidden, 2 * ffn, experts}: gate rows, then up rows, per expert) as the source of
+    // a layer (reference: GpuFusedExpertCache, src/expert_cache.cuh:2546-2882).  The slot keeps gate | up | down.
+    void register_layer_fused(int layer, const TensorInfo &gate_up, const TensorInfo &down) {
+        if (layer < 0) return;
+        if (!c_) throw std::runtime_error("expert cache is not initialized");
+        if (registered(layer)) return;
+        const ExpertHostSlice gu = expert_slice(gate_up, 0);
+        expert_slice(down, 0);
+        if (gu.rows % 2 != 0 || gu.bytes != gate_bytes_ + up_bytes_) throw std::runtime_error("fused gate_up tensor does not match the cache's slot layout: " + gate_up.name);
+        check(wd_expert_cache_register_layer_strided(c_, layer, gate_up.data, gate_up.data + gate_bytes_, down.data, gu.bytes, gu.bytes, down_bytes_),
+              "expert cache layer registration failed");
+        if (reg_.size() <= static_cast<size_t>(layer)) reg_.resize(static_cast<size_t>(layer) + 1, 0);
+        reg_[static_cast<size_t>(layer)] = 1;
+    }
+
     // Makes every expert of a registered layer resident.  With room for all experts of all layers (the
     // normal case with 288 GB of HBM) nothing is ever evicted and layer passes need no host round trip.
     void preload_layer(int layer, Stream stream) {
@@ -539,6 +554,24 @@ inline void run_qwen38_routed_moe_separate_f32_x(int layer, const float *x, cons
     cache.register_layer_experts(layer, gate_exps, up_exps, down_exps);
     cache.acquire_ids(layer, scratch.h_ids(), L.top_k, stream);
     check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), WD_MOE_PRESELECTED | WD_MOE_ONLY_B | WD_MOE_ONLY_C, stream), "MoE experts failed");
+}
+
+// The same with the gate and up projections stored as one tensor of 2 * ffn rows per expert
+// (run_qwen38_routed_moe_fused, src/qwen38_moe.cuh:3522-3647).
+inline void run_qwen38_routed_moe_fused_f32_x(int layer, const float *x, const GpuMatrix &router, const TensorInfo &gate_up_exps,
+                                              const TensorInfo &down_exps, GpuExpertCache &cache, Qwen38MoeScratch &scratch, float *out,
+                                              float expert_scale, Stream stream, bool preselected = false) {
+    if (gate_up_exps.dims.size() != 3 || gate_up_exps.dims[1] % 2 != 0) throw std::runtime_error("fused gate_up tensor must be 3D with an even row count: " + gate_up_exps.name);
+    TensorInfo half = gate_up_exps;   // geometry of one projection; the data pointer is only used for registration
+    half.dims[1] = gate_up_exps.dims[1] / 2;
+    cache.register_layer_fused(layer, gate_up_exps, down_exps);
+    // the slot pool holds gate | up | down per expert, so from here on the separate runner applies unchanged
+    // (its own registration call is a no-op for a layer that is registered already)
+    half.dims[2] = gate_up_exps.dims[2];
+    TensorInfo g = half, u = half;
+    g.data = gate_up_exps.data, u.data = gate_up_exps.data;
+    // expert_slice() checks contiguity against byte_size(): give it tensors of the half geometry
+    run_qwen38_routed_moe_separate_f32_x(layer, x, router, g, u, down_exps, cache, scratch, out, expert_scale, stream, preselected);
 }
 
 // src/qwen38_moe.cuh:3963-3969
