@@ -178,8 +178,10 @@ int32_t *wd_moe_scratch_down_partials(wd_moe_scratch *s);
  * layer pass fill them.  Parity harness only. */
 int wd_moe_scratch_enable_partials(wd_moe_scratch *s, int gate_type, int down_type);
 
-/* Profiling aid: makes the fused layer dispatches record 100 MHz time stamps of workgroup `wg`
- * ([dispatch A,B,C][wave 0..15][point 0..7], uint64) and returns the device buffer (NULL on failure).
+/* Profiling aid: makes the fused layer dispatches record 100 MHz time stamps of workgroup `wg` and returns the
+ * device buffer (NULL on failure): uint64 [3][16][8] = [dispatch][wave][point]; dispatch 0 = router and shared
+ * workgroups of the merged launch (wave rows 8 and 9: begin/end and the phases of the selection), 1 = routed gate/up
+ * workgroups, 2 = dispatch C.  Only the traced workgroup pays for it.
  * Counterpart of the reference's kernel profiler sites, src/qwen38_moe.cuh:296-535. */
 unsigned long long *wd_moe_scratch_trace(wd_moe_scratch *s, int wg);
 
