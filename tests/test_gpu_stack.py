@@ -111,3 +111,56 @@ def test_cached_stack(g, oracle, layers, slots, use_trace):
         assert st.evictions == 0
     sc.close()
     capi.call("wd_expert_cache_destroy", cache)
+
+
+def test_graph_replayed_c2_stack(g, oracle):
+    """The benchmark's own mechanics at reduced size: an 8-layer stack of C2-shaped layers (64 experts) captured
+    into a HIP graph and replayed for several tokens with fresh inputs and routing traces in between, every
+    replay checked against the oracle applied layer by layer (and against an eager run of the same token)."""
+    import torch
+    NLc, Ec, Kc, Hc, Fc = 8, 64, 10, 2048, 512
+    Ls = [synth.make_c2(layer=100 + l, n_experts=Ec) for l in range(NLc)]
+    dls, arr = _descs(g, Ls)
+    sc = g.Scratch(Hc, Fc, Ec, Kc)
+    scale = np.float32(2.0 ** -12)
+    d_x = torch.zeros(Hc, dtype=torch.float32, device="cuda")
+    d_out = torch.zeros(Hc, dtype=torch.float32, device="cuda")
+    d_tr = torch.zeros((NLc, Kc), dtype=torch.int32, device="cuda")
+
+    def launch():
+        capi.call("wd_moe_stack_f32", arr, NLc, g.ptr(d_x), g.ptr(d_out), sc.h, g.ptr(d_tr), float(scale), 0,
+                  C.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        launch()
+    rng = np.random.default_rng(SEED + 300)
+    for token in range(4):
+        x = synth.rms_normed(synth.rng_for(SEED, 83, token), Hc)
+        tr = np.stack([rng.choice(Ec, size=Kc, replace=False) for _ in range(NLc)]).astype(np.int32)
+        d_x.copy_(torch.from_numpy(x).cuda())
+        d_tr.copy_(torch.from_numpy(tr).cuda())
+        graph.replay()
+        torch.cuda.synchronize()
+        got_x, got_out = d_x.cpu().numpy(), d_out.cpu().numpy()
+        # oracle, layer by layer (router weights, ids from the trace)
+        wx = x.copy()
+        for l, L in enumerate(Ls):
+            _, wts = oracle.route(oracle.router_logits(L["router"], wx), Kc)
+            wout, _ = oracle.moe_layer(L, wx, ids=tr[l], weights=wts)
+            wx = (wx + (wout * scale).astype(np.float32)).astype(np.float32)
+        assert g.same_bits(got_x, wx), token
+        assert g.same_bits(got_out, wout), token
+        # the same token eagerly, between two replays
+        d_x.copy_(torch.from_numpy(x).cuda())
+        launch()
+        torch.cuda.synchronize()
+        assert g.same_bits(d_x.cpu().numpy(), wx), token
+    assert capi.load().wd_moe_scratch_status(sc.h) == 0
+    sc.close()
