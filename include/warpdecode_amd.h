@@ -287,6 +287,34 @@ int wd_moe_stack_cached_f32(const wd_moe_layer *layers, int n_layers, wd_expert_
                             float *d_layer_out, wd_moe_scratch *scratch, const int32_t *h_ids_trace,
                             const int32_t *d_ids_trace, float residual_scale, unsigned flags, void *stream);
 
+
+/* ---- GGUF container ---------------------------------------------------------------------------
+ * Read-only memory map of a GGUF file (versions 2 and 3) with its metadata and tensor directory parsed; tensor
+ * views point into the mapping (raw block bytes, as the expert cache, wd_memcpy_h2d and the layer descriptors
+ * take them).  reference: GgufFile / MappedFile / TensorInfo, src/gguf.hpp:71-491. */
+typedef struct wd_gguf wd_gguf;
+typedef struct {
+    const char *name;          /* owned by the wd_gguf object */
+    uint32_t n_dims;
+    uint64_t dims[4];          /* GGUF order: dims[0] = columns; unused ones are 1 */
+    uint32_t type;             /* ggml type id (WD_TYPE_* for the ones this library computes with) */
+    uint64_t relative_offset;  /* from the start of the data section */
+    uint64_t bytes;            /* size of the tensor data; 0 when the type's block size is unknown here */
+    const uint8_t *data;       /* inside the mapping, valid until wd_gguf_close */
+} wd_gguf_tensor_info;
+int wd_gguf_open(wd_gguf **out, const char *path);
+int wd_gguf_close(wd_gguf *g);
+uint32_t wd_gguf_version(const wd_gguf *g);
+size_t wd_gguf_data_offset(const wd_gguf *g);              /* file offset of the data section (for pread users) */
+long long wd_gguf_tensor_count(const wd_gguf *g);
+long long wd_gguf_find(const wd_gguf *g, const char *name); /* index or -1 */
+int wd_gguf_tensor(const wd_gguf *g, long long index, wd_gguf_tensor_info *out);
+/* Metadata: numbers of any scalar type as a double (WD_OK, or WD_ERR_ARG when absent or not a number), strings
+ * (NULL when absent), arrays of fixed-size elements (length, or -1; *data points into the mapping). */
+int wd_gguf_meta_number(const wd_gguf *g, const char *key, double *out);
+const char *wd_gguf_meta_string(const wd_gguf *g, const char *key);
+long long wd_gguf_meta_array(const wd_gguf *g, const char *key, uint32_t *elem_type, const void **data);
+
 #ifdef __cplusplus
 }
 #endif

@@ -11,6 +11,9 @@
 #include <functional>
 #include <random>
 
+#include <unistd.h>
+
+#include "wd_gguf.hpp"
 #include "wd_ops.hpp"
 #include "wd_oracle.h"
 
@@ -99,6 +102,70 @@ static HostLayer make_layer(uint64_t seed, int H, int F, int E, int k) {
     return L;
 }
 
+// Minimal GGUF v3 writer for the layers above (the names a model file uses for one MoE block).
+struct GgufOut {
+    std::vector<uint8_t> head, data;
+    uint64_t n_tensors = 0, n_kv = 0;
+    template <typename T>
+    void put(T v) {
+        const uint8_t *p = reinterpret_cast<const uint8_t *>(&v);
+        head.insert(head.end(), p, p + sizeof(T));
+    }
+    void str(const std::string &s) {
+        put<uint64_t>(s.size());
+        head.insert(head.end(), s.begin(), s.end());
+    }
+    void kv_u32(const std::string &k, uint32_t v) { str(k), put<uint32_t>(4), put<uint32_t>(v), ++n_kv; }
+    void kv_f32(const std::string &k, float v) { str(k), put<uint32_t>(6), put<float>(v), ++n_kv; }
+    void kv_str(const std::string &k, const std::string &v) { str(k), put<uint32_t>(8), str(v), ++n_kv; }
+    void tensor(const std::string &name, std::vector<uint64_t> dims, GgmlType type, const void *bytes, size_t n) {
+        str(name), put<uint32_t>(static_cast<uint32_t>(dims.size()));
+        for (uint64_t d : dims) put<uint64_t>(d);
+        put<uint32_t>(static_cast<uint32_t>(type)), put<uint64_t>(data.size());
+        const uint8_t *b = static_cast<const uint8_t *>(bytes);
+        data.insert(data.end(), b, b + n);
+        data.resize((data.size() + 31) & ~size_t(31));
+        ++n_tensors;
+    }
+    std::string write() {
+        char path[] = "/tmp/wd_gguf_test_XXXXXX";
+        const int fd = mkstemp(path);
+        if (fd < 0) throw std::runtime_error("mkstemp failed");
+        FILE *f = fdopen(fd, "wb");
+        const uint32_t magic = 0x46554747u, version = 3;
+        fwrite(&magic, 4, 1, f), fwrite(&version, 4, 1, f), fwrite(&n_tensors, 8, 1, f), fwrite(&n_kv, 8, 1, f);
+        fwrite(head.data(), 1, head.size(), f);
+        const std::vector<uint8_t> pad((32 - (24 + head.size()) % 32) % 32, 0);
+        fwrite(pad.data(), 1, pad.size(), f);
+        fwrite(data.data(), 1, data.size(), f);
+        fclose(f);
+        return path;
+    }
+};
+
+static std::string write_model_file(const std::vector<HostLayer> &L) {
+    GgufOut o;  // every key/value goes in before the first tensor: the directory follows the metadata in the file
+    o.kv_str("general.architecture", "qwen38");
+    o.kv_u32("qwen38.block_count", static_cast<uint32_t>(L.size()));
+    o.kv_u32("qwen38.expert_count", static_cast<uint32_t>(L[0].E));
+    o.kv_u32("qwen38.expert_used_count", static_cast<uint32_t>(L[0].k));
+    o.kv_f32("qwen38.expert_weights_scale", 1.0f);
+    for (size_t l = 0; l < L.size(); ++l) {
+        const HostLayer &h = L[l];
+        const std::string blk = "blk." + std::to_string(l) + ".";
+        const uint64_t H = h.H, F = h.F, E = h.E;
+        o.tensor(blk + "ffn_gate_inp.weight", {H, E}, GgmlType::F32, h.router.data(), h.router.size() * 4);
+        o.tensor(blk + "ffn_gate_exps.weight", {H, F, E}, GgmlType::IQ3_S, h.gate.data(), h.gate.size());
+        o.tensor(blk + "ffn_up_exps.weight", {H, F, E}, GgmlType::IQ3_S, h.up.data(), h.up.size());
+        o.tensor(blk + "ffn_down_exps.weight", {F, H, E}, GgmlType::Q8_0, h.down.data(), h.down.size());
+        o.tensor(blk + "ffn_gate_inp_shexp.weight", {H}, GgmlType::F32, h.gate_inp.data(), h.gate_inp.size() * 4);
+        o.tensor(blk + "ffn_gate_shexp.weight", {H, F}, GgmlType::Q8_0, h.sg.data(), h.sg.size());
+        o.tensor(blk + "ffn_up_shexp.weight", {H, F}, GgmlType::Q8_0, h.su.data(), h.su.size());
+        o.tensor(blk + "ffn_down_shexp.weight", {F, H}, GgmlType::Q8_0, h.sd.data(), h.sd.size());
+    }
+    return o.write();
+}
+
 static std::vector<float> rms_normed(Rng &r, int n) {
     std::vector<float> x(n);
     double ss = 0;
@@ -140,6 +207,26 @@ static void host_only_checks() {
     LowBitMatrix q = borrow_lowbit_matrix(reinterpret_cast<uint8_t *>(0x1000), 4, 256, GgmlType::Q8_0, 4 * 8 * 34);
     CHECK(throws([&] { launch_iq3_s_gemv_q8_k_f32(q, nullptr, nullptr, nullptr, nullptr); }), "type mismatch must throw");
     CHECK(throws([&] { launch_q8_k_quantize_f32(nullptr, 100, nullptr, nullptr, nullptr, nullptr); }), "Q8_K needs multiples of 256");
+
+    // model file: directory, metadata and tensor bytes through GgufFile
+    std::vector<HostLayer> L;
+    for (int l = 0; l < 2; ++l) L.push_back(make_layer(500 + l, 256, 32, 8, 2));
+    const std::string path = write_model_file(L);
+    {
+        GgufFile g(path);
+        CHECK(g.version() == 3 && g.tensors().size() == 16 && g.data_offset() % 32 == 0, "header: version %u, %zu tensors", g.version(), g.tensors().size());
+        CHECK(g.string_meta("general.architecture") == "qwen38" && g.string_meta("absent", "dflt") == "dflt", "string metadata");
+        CHECK(g.number_meta("qwen38.expert_count") == 8.0 && g.number_meta("absent", -1.0) == -1.0 && g.has_number_meta("qwen38.expert_weights_scale"), "number metadata");
+        CHECK(throws([&] { g.tensor("blk.9.ffn_gate_inp.weight"); }) && g.optional_tensor("blk.0.ffn_gate_up_exps.weight") == nullptr, "absent tensors");
+        const Qwen38MoeLayerTensors t = qwen38_moe_tensors(g, 1);
+        CHECK(!t.fused_gate_up() && t.gate->dims == std::vector<uint64_t>({256, 32, 8}) && t.gate->type == GgmlType::IQ3_S && t.down->type == GgmlType::Q8_0, "layer tensor set");
+        CHECK(t.gate->byte_size() == L[1].gate.size() && std::memcmp(t.gate->data, L[1].gate.data(), L[1].gate.size()) == 0, "gate bytes come back from the mapping");
+        CHECK(std::memcmp(t.router->data, L[1].router.data(), L[1].router.size() * 4) == 0, "router floats come back from the mapping");
+        CHECK(g.tensor_file_offset(*t.up) == g.data_offset() + t.up->relative_offset && t.up->relative_offset % 32 == 0, "file offsets");
+        CHECK(throws([&] { qwen38_moe_tensors(g, 2); }), "a layer the file does not hold must throw");
+    }
+    CHECK(throws([&] { GgufFile missing(path + ".nope"); }), "opening an absent file must throw");
+    unlink(path.c_str());
 }
 
 // The reference's three calls, then the read-back a caller does.
@@ -258,6 +345,44 @@ static void gpu_checks() {
             check(wd_memcpy_d2h(back.data(), v.gate.data, v.gate.bytes, nullptr), "slot read-back");
             CHECK(std::memcmp(back.data(), expert_slice(L[0].t_gate, 5).data, v.gate.bytes) == 0 && !v.gate.owns, "acquired view must hold the expert's gate bytes");
         }
+    }
+    // the same stack driven from a model file: tensors found by name, router / shared expert uploaded from the mapping,
+    // the mapping itself as the cache's host source (LRU pool, so experts stream from the file's pages)
+    {
+        const std::string path = write_model_file(L);
+        {
+            GgufFile g(path);
+            std::vector<Qwen38MoeLayerTensors> T;
+            std::vector<GpuMatrix> frouters;
+            std::vector<Qwen38SharedExpertWeights> fshared;
+            for (int l = 0; l < layers; ++l) {
+                T.push_back(qwen38_moe_tensors(g, l));
+                frouters.push_back(upload_matrix(*T[l].router));
+                fshared.push_back(load_qwen38_shared_expert(g, l, H, F));
+            }
+            CHECK(throws([&] { load_qwen38_shared_expert(g, 0, H, F + 32); }), "shared expert shape mismatch must throw");
+            GpuExpertCache cache;
+            cache.initialize((12 * slot + (1u << 20) - 1) >> 20, *T[0].gate, *T[0].up, *T[0].down, 0, 0, 0, opt);
+            for (int l = 0; l < layers; ++l) cache.register_layer_experts(l, *T[l].gate, *T[l].up, *T[l].down);
+            Rng r(321);
+            DeviceFloatArray dx(H), dout(H);
+            for (int token = 0; token < 3; ++token)
+                for (int l = 0; l < layers; ++l) {
+                    const std::vector<float> x = rms_normed(r, H);
+                    dx.upload(x.data(), H);
+                    run_qwen38_routed_moe_separate_f32_x(l, dx.data, frouters[l], *T[l].gate, *T[l].up, *T[l].down, cache, scratch, nullptr,
+                                                         static_cast<float>(g.number_meta("qwen38.expert_weights_scale", 1.0)), stream);
+                    run_qwen38_shared_expert_f32_x(dx.data, fshared[l], scratch, stream);
+                    q38_finish_moe_f32(scratch, dout.data, stream);
+                    check(wd_stream_sync(stream), "sync");
+                    std::vector<float> got(H), want(H);
+                    dout.download(got.data());
+                    wdo_moe_layer(&L[l].o, x.data(), want.data(), nullptr, 0);
+                    CHECK(same_bits(got.data(), want.data(), H), "model file, token %d layer %d: output differs from the oracle", token, l);
+                }
+            CHECK(cache.stats().misses > 0, "the file-backed pool should have taken misses");
+        }
+        unlink(path.c_str());
     }
     // fused gate_up tensor (2 * ffn rows per expert) through the fused runner, LRU pool of 10+ slots
     {

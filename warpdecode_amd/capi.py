@@ -37,6 +37,11 @@ class MoeLayer(C.Structure):
     ]
 
 
+class GgufTensorInfo(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("n_dims", C.c_uint32), ("dims", C.c_uint64 * 4), ("type", C.c_uint32),
+                ("relative_offset", C.c_uint64), ("bytes", C.c_uint64), ("data", vp)]
+
+
 class CacheStats(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in ("accesses", "hits", "misses", "evictions", "bytes_copied", "slots",
                                           "slot_bytes", "resident")]
@@ -96,6 +101,16 @@ _OPTIONAL = {
     "wd_expert_cache_slot_of": (C.c_longlong, [vp, i32, i32]),
     "wd_expert_cache_add_shadow": (i32, [vp, i32, sz]),
     "wd_expert_cache_dump_json": (sz, [vp, C.c_char_p, sz]),
+    "wd_gguf_open": (i32, [C.POINTER(vp), C.c_char_p]),
+    "wd_gguf_close": (i32, [vp]),
+    "wd_gguf_version": (C.c_uint32, [vp]),
+    "wd_gguf_data_offset": (sz, [vp]),
+    "wd_gguf_tensor_count": (C.c_longlong, [vp]),
+    "wd_gguf_find": (C.c_longlong, [vp, C.c_char_p]),
+    "wd_gguf_tensor": (i32, [vp, C.c_longlong, C.POINTER(GgufTensorInfo)]),
+    "wd_gguf_meta_number": (i32, [vp, C.c_char_p, C.POINTER(C.c_double)]),
+    "wd_gguf_meta_string": (C.c_char_p, [vp, C.c_char_p]),
+    "wd_gguf_meta_array": (C.c_longlong, [vp, C.c_char_p, C.POINTER(C.c_uint32), C.POINTER(vp)]),
     "wd_expert_cache_get_stats": (i32, [vp, C.POINTER(CacheStats)]),
 }
 

@@ -3,3 +3,4 @@
 #include "wd_layer.hip"
 #include "wd_cache.hip"
 #include "wd_stack.hip"
+#include "wd_gguf.hip"
