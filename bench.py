@@ -46,9 +46,10 @@ def parse():
     ap.add_argument("--experts", type=int, default=512)
     ap.add_argument("--routing", choices=["zipf", "router"], default="zipf",
                     help="zipf: ids replayed from the Zipf(1.1) trace; router: ids chosen by the router itself")
-    ap.add_argument("--mode", choices=["resident", "lru"], default="resident",
+    ap.add_argument("--mode", choices=["resident", "lru", "q4-sweep"], default="resident",
                     help="resident: C3 mode A, every expert in HBM; lru: C3 mode B, experts in pinned host memory "
-                         "behind an LRU slot pool of --cache-gib in HBM")
+                         "behind an LRU slot pool of --cache-gib in HBM; q4-sweep: the dense Q4_0 GEMV shapes "
+                         "(secondary workload, own JSON line)")
     ap.add_argument("--cache-gib", type=float, default=32.0)
     ap.add_argument("--cache-warm-tokens", type=int, default=256,
                     help="lru mode: tokens run before the warm-up steps so that the slot pool is in steady state")
@@ -316,6 +317,78 @@ def bench_lru(args, torch, capi, synth):
     print(json.dumps(out))
 
 
+def graph_period_us(torch, launch, launches, reps):
+    """Average period of one launch of `launch(i)`, i in [0, launches), captured once and replayed `reps` times."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch(0)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(launches):
+            launch(i)
+    for _ in range(max(2, reps // 4)):
+        graph.replay()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (reps * launches)
+
+
+def bench_q4_sweep(args, torch, capi, synth):
+    """Dense Q4_0 x Q8_0 GEMV at batch=1 over the Llama-3.2-1B shapes (BASELINE.json configs[1]).  Every launch
+    of a chain reads another copy of the matrix, with enough copies (>= 1.5 GB) that nothing is served from the
+    256 MB last-level cache; the period is taken over a captured chain, so it includes the launch gap."""
+    shapes = [(2048, 2048), (8192, 2048), (2048, 8192), (128256, 2048)]     # rows x cols of the weight
+    results = []
+    for rows, cols in shapes:
+        nbytes = rows * synth.row_bytes(synth.Q4_0, cols)
+        copies = max(2, min(640, -(-int(1.5e9) // nbytes)))
+        one = torch.from_numpy(synth.matrix(synth.Q4_0, synth.rng_for(synth.BASE_SEED, 77, rows, cols), min(rows, 8192), cols))
+        one = one.reshape(-1).cuda()
+        w = one.repeat(-(-rows // min(rows, 8192)))[:nbytes].repeat(copies).reshape(copies, nbytes)
+        x = torch.from_numpy(synth.rng_for(synth.BASE_SEED, 78, cols).normal(0, 1, cols).astype(np.float32)).cuda()
+        qs = torch.empty(cols, dtype=torch.int8, device="cuda")
+        sc = torch.empty(cols // 32, dtype=torch.int16, device="cuda")
+        y = torch.empty(rows, dtype=torch.float32, device="cuda")
+        stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        vp = lambda t: C.c_void_p(t.data_ptr())
+
+        def gemv(i):
+            capi.call("wd_gemv_q8_0_f32", synth.Q4_0, C.c_void_p(w[i % copies].data_ptr()), rows, cols, vp(qs), vp(sc), vp(y),
+                      None, stream())
+
+        def call(i):
+            capi.call("wd_q8_0_quantize_f32", vp(x), cols, vp(qs), vp(sc), stream())
+            gemv(i)
+
+        call(0)
+        torch.cuda.synchronize()
+        launches = max(copies, 32)
+        reps = max(3, int(1e11 // (nbytes * launches)))    # about 20 ms of streaming per timed region at full rate
+        us = graph_period_us(torch, gemv, launches, reps)
+        us_call = graph_period_us(torch, call, launches, reps)
+        results.append(dict(rows=rows, cols=cols, bytes=nbytes, copies=copies, us_per_gemv=round(us, 3),
+                            gbs=round(nbytes / us / 1e3, 1), frac=round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                            us_per_call_with_quantise=round(us_call, 3), finite=bool(torch.isfinite(y).all().item())))
+        note("Q4_0 %dx%d: %.2f us, %.0f GB/s" % (rows, cols, us, nbytes / us / 1e3))
+        del w, one
+        torch.cuda.empty_cache()
+    head = results[-1]
+    print(json.dumps({
+        "metric": "dense Q4_0 GEMV batch=1: achieved HBM GB/s (lm_head 128256x2048)", "value": head["gbs"], "unit": "GB/s",
+        "n_gpus": 1, "higher_is_better": True, "vs_baseline": None, "dtype": "int8 dot products, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "C1: Q4_0 x Q8_0 GEMV sweep, Llama-3.2-1B shapes, raw GGUF 18-byte blocks", "shapes": results},
+        "roofline": dict(bound="hbm", achieved=head["gbs"], peak=HBM_PEAK_GBS, unit="GB/s", frac=head["frac"], traffic=None,
+                         kernel="k_gemv_q8<Q4_0>", us_per_launch=head["us_per_gemv"], bytes_per_launch=head["bytes"])}))
+
+
 def main():
     if len(sys.argv) >= 5 and sys.argv[1] == "--cpu-child":
         cpu_child(float(sys.argv[2]), int(sys.argv[3]), sys.argv[4])
@@ -331,6 +404,8 @@ def main():
     torch.cuda.set_device(0)
     capi.call("wd_init", 0)
     H, F, k, E, NL = 2048, 512, 10, args.experts, args.layers
+    if args.mode == "q4-sweep":
+        return bench_q4_sweep(args, torch, capi, synth)
     note("generating %d layers x %d experts on the device" % (NL, E))
     if args.mode == "lru":
         return bench_lru(args, torch, capi, synth)

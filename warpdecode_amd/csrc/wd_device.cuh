@@ -187,5 +187,11 @@ WD_DEV uint4 gld_u128(const uint8_t *p) {
     const wd_u128a v = *((const WD_GLOBAL wd_u128a *)(p));
     return make_uint4(v.x, v.y, v.z, v.w);
 }
+// 16-byte aligned form (one full-width request per lane)
+typedef uint32_t wd_u128 __attribute__((ext_vector_type(4), aligned(16)));
+WD_DEV uint4 gld_u128_aligned(const uint8_t *p) {
+    const wd_u128 v = *((const WD_GLOBAL wd_u128 *)(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
 
 }  // namespace wd

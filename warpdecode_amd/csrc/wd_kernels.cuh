@@ -189,6 +189,116 @@ __global__ __launch_bounds__(256) void k_gemv_q8(MatSrc src, int rows, int cols,
     if ((lane & 15) == 0 && r4 < nrows) out[static_cast<size_t>(m) * rows + r0 + r4] = y;
 }
 
+// ---- Q4_0 x Q8_0 GEMV, streaming form ---------------------------------------------------------------------
+// For matrices whose rows are a whole number of 8-block groups (144 bytes = nine 16-byte words) and whose group
+// count per row (lpr) divides 64.  A wave owns 64 consecutive groups per pass (64 * 144 = 9216 contiguous bytes,
+// 64 / lpr rows): nine fully coalesced 16-byte loads per lane bring them in, LDS turns the lane-interleaved words
+// into one group per lane (both sides conflict-free: stride 16 in, stride 144 out), and the 18-byte blocks are cut
+// out of the 36 dwords in registers (even blocks with four byte-align ops, odd blocks are dword aligned).  Lane l
+// always works on column group l % lpr.  The workgroup keeps the activation in LDS (each group's 256 bytes padded
+// to 272 so that the 16-byte reads of neighbouring groups fall on different banks), with the per-block scale as a
+// float and 8 * sum(a) beside it; few registers per lane keep many waves, i.e. many loads, in flight, and the next
+// pass's loads are issued before the current one is computed.  Block sums are exact; the float side adds a lane's
+// eight blocks in order and folds the row's lanes with an xor tree (Q4_0 has no canonical float order).
+// grid.x * 4 waves * passes_per_wave passes cover ceil(rows / (64 / lpr)) passes.
+// dynamic LDS: lpr * 272 bytes of quants, then nb floats, then nb ints.
+template <bool PART>
+__global__ __launch_bounds__(256) void k_gemv_q4_stream(const uint8_t *__restrict__ w, int rows, int nb, int passes_per_wave,
+                                                         const int8_t *__restrict__ act_qs,
+                                                         const uint16_t *__restrict__ act_d, float *__restrict__ out,
+                                                         int32_t *__restrict__ partials) {
+    __shared__ uint4 stage[4][9 * 64];
+    extern __shared__ __align__(16) uint8_t q4_act[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lpr = nb >> 3, lpr_shift = __builtin_ctz(lpr), rpp = 64 >> lpr_shift;
+    const int col = lane & (lpr - 1), rsub = lane >> lpr_shift;
+    float *ad = reinterpret_cast<float *>(q4_act + lpr * 272);
+    int *corr = reinterpret_cast<int *>(ad + nb);
+    const size_t rb = static_cast<size_t>(nb) * 18;
+    const long long pass0 = (static_cast<long long>(blockIdx.x) * 4 + wave) * passes_per_wave;
+    uint4 v[9];
+    auto fetch = [&](long long pass) {
+        const long long row0 = pass * rpp;
+        const long long left = static_cast<long long>(rows) - row0;
+        const size_t valid = left <= 0 ? 0 : static_cast<size_t>(left < rpp ? left : rpp) * rb;
+        const uint8_t *base = w + static_cast<size_t>(row0) * rb;
+#pragma unroll
+        for (int k = 0; k < 9; ++k) {
+            const size_t off = static_cast<size_t>(k) * 1024 + static_cast<size_t>(lane) * 16;
+            v[k] = off < valid ? gld_u128_aligned(base + off) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    // activation into LDS: thread t takes 16-byte pieces t, t + 256, ...; a block's two pieces give its sum.  The
+    // first piece is requested before the weights so that it can be consumed while they are still in flight.
+    const int n_pieces = nb * 2;
+    uint4 q0 = make_uint4(0, 0, 0, 0);
+    uint16_t d0 = 0;
+    if (static_cast<int>(threadIdx.x) < n_pieces) {
+        q0 = *reinterpret_cast<const uint4 *>(act_qs + threadIdx.x * 16);
+        d0 = act_d[threadIdx.x >> 1];
+    }
+    fetch(pass0);
+    for (int i = threadIdx.x; i < n_pieces; i += 256) {
+        const bool first = i == static_cast<int>(threadIdx.x);
+        const uint4 q = first ? q0 : *reinterpret_cast<const uint4 *>(act_qs + i * 16);
+        *reinterpret_cast<uint4 *>(q4_act + (i >> 4) * 272 + (i & 15) * 16) = q;
+        int s = sdot4(0x01010101u, q.x, 0);
+        s = sdot4(0x01010101u, q.y, s);
+        s = sdot4(0x01010101u, q.z, s);
+        s = sdot4(0x01010101u, q.w, s);
+        s += lane_xor(s, 1);
+        if ((i & 1) == 0) {
+            corr[i >> 1] = 8 * s;
+            ad[i >> 1] = h2f(first ? d0 : act_d[i >> 1]);
+        }
+    }
+    __syncthreads();
+    const uint8_t *my_act = q4_act + col * 272;
+    for (int p = 0; p < passes_per_wave; ++p) {
+        const long long row0 = (pass0 + p) * rpp;
+        if (row0 >= rows) break;  // wave-uniform
+#pragma unroll
+        for (int k = 0; k < 9; ++k) stage[wave][k * 64 + lane] = v[k];
+        wave_lds_fence();
+        uint32_t d[36];
+#pragma unroll
+        for (int k = 0; k < 9; ++k) {
+            const uint4 u = stage[wave][lane * 9 + k];
+            d[4 * k] = u.x, d[4 * k + 1] = u.y, d[4 * k + 2] = u.z, d[4 * k + 3] = u.w;
+        }
+        wave_lds_fence();
+        if (p + 1 < passes_per_wave) fetch(pass0 + p + 1);
+        const int row = static_cast<int>(row0) + rsub;
+        float sumf = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int m = j >> 1;
+            uint32_t n[4], dw;
+            if ((j & 1) == 0) {
+                dw = d[9 * m] & 0xffffu;
+#pragma unroll
+                for (int l = 0; l < 4; ++l) n[l] = __builtin_amdgcn_alignbyte(d[9 * m + l + 1], d[9 * m + l], 2);
+            } else {
+                dw = d[9 * m + 4] >> 16;
+#pragma unroll
+                for (int l = 0; l < 4; ++l) n[l] = d[9 * m + 5 + l];
+            }
+            const uint4 lo = *reinterpret_cast<const uint4 *>(my_act + j * 32), hi = *reinterpret_cast<const uint4 *>(my_act + j * 32 + 16);
+            const uint32_t al[4] = {lo.x, lo.y, lo.z, lo.w}, ah[4] = {hi.x, hi.y, hi.z, hi.w};
+            int sumi = -corr[col * 8 + j];  // sum (nibble - 8) * a = sum nibble * a - 8 * sum a
+#pragma unroll
+            for (int l = 0; l < 4; ++l) {
+                sumi = sdot4(n[l] & 0x0f0f0f0fu, al[l], sumi);
+                sumi = sdot4((n[l] >> 4) & 0x0f0f0f0fu, ah[l], sumi);
+            }
+            if (PART && row < rows) partials[static_cast<size_t>(row) * nb + col * 8 + j] = sumi;
+            sumf += h2f(static_cast<uint16_t>(dw)) * ad[col * 8 + j] * static_cast<float>(sumi);
+        }
+        for (int mask = lpr >> 1; mask >= 1; mask >>= 1) sumf += lane_xor(sumf, mask);
+        if (col == 0 && row < rows) out[row] = sumf;
+    }
+}
+
 // ---- elementwise ---------------------------------------------------------------------------------
 __global__ void k_silu_mul_experts(const float *__restrict__ gate_up, float *__restrict__ act, int ffn) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;

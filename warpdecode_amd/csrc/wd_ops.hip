@@ -192,6 +192,24 @@ static int launch_gemv_q8_0(int type, MatSrc src, int mats, int rows, int cols, 
     const dim3 grid((rows + 15) / 16, mats), block(256);
     const int ppr = partials_per_row(type, cols);
     const int act_stride = act_per_mat ? cols : 0;
+    const int nb = cols / 32;
+    if (type == WD_TYPE_Q4_0 && mats == 1 && src.single && nb % 8 == 0 && nb / 8 <= 64 && 64 % (nb / 8) == 0 &&
+        reinterpret_cast<uintptr_t>(src.single) % 16 == 0 && reinterpret_cast<uintptr_t>(qs) % 16 == 0) {
+        // whole 8-block groups per row and a 16-byte aligned base: the streaming kernel
+        const int rpp = 64 / (nb / 8);
+        const long long passes = (static_cast<long long>(rows) + rpp - 1) / rpp;
+        static const int forced = getenv("WD_Q4_PASSES") ? atoi(getenv("WD_Q4_PASSES")) : 0;
+        long long per_wave = forced > 0 ? forced : passes / 16384;
+        per_wave = per_wave < 1 ? 1 : (per_wave > 8 ? 8 : per_wave);
+        const unsigned wgs = static_cast<unsigned>((passes + per_wave * 4 - 1) / (per_wave * 4));
+        const size_t lds = static_cast<size_t>(nb / 8) * 272 + static_cast<size_t>(nb) * 8;
+        if (partials)
+            k_gemv_q4_stream<true><<<wgs, 256, lds, stream>>>(src.single, rows, nb, static_cast<int>(per_wave), qs, d, out, partials);
+        else
+            k_gemv_q4_stream<false><<<wgs, 256, lds, stream>>>(src.single, rows, nb, static_cast<int>(per_wave), qs, d, out, nullptr);
+        WD_LAUNCH_CHECK();
+        return WD_OK;
+    }
 #define WD_Q8_LAUNCH(KIND)                                                                                          \
     do {                                                                                                            \
         if (partials)                                                                                               \
