@@ -106,7 +106,10 @@ GEMV_SHAPES = {
     synth.IQ2_S: [(640, 2560), (512, 2048), (3, 256)],
     synth.Q8_0: [(2048, 512), (512, 2048), (7, 96), (640, 2560), (18, 32)],
     synth.IQ4_NL: [(2560, 640), (2048, 512), (5, 96), (9, 32 * 5)],
-    synth.Q4_0: [(2048, 2048), (2048, 8192), (8192, 2048), (128256, 2048), (1000, 2048), (6, 96)],   # C1 incl. the lm_head
+    # C1 incl. the lm_head; then ragged row counts for every lanes-per-row case of the streaming kernel (columns a
+    # multiple of 256 whose 8-block groups per row divide 64) and shapes that take the general kernel
+    synth.Q4_0: [(2048, 2048), (2048, 8192), (8192, 2048), (128256, 2048), (1003, 2048), (5, 256), (67, 512), (131, 8192),
+                 (7, 16384), (33, 1024), (6, 96), (40, 768), (9, 32768)],
 }
 
 
@@ -136,6 +139,28 @@ def test_gemv_single(g, oracle, t):
         else:
             assert g.same_bits(g.host(out), want), (t, rows, cols)
             assert g.same_bits(g.host(out2), want), (t, rows, cols)
+
+
+def test_q4_0_gemv_misaligned_base(g, oracle):
+    """A matrix that starts 2 bytes into an allocation (GGUF blocks are only 2-byte aligned) takes the general
+    kernel instead of the streaming one; both must give the same block sums."""
+    import torch
+    rows, cols = 300, 2048
+    rng = synth.rng_for(SEED, 23, rows, cols)
+    w = synth.matrix(synth.Q4_0, rng, rows, cols)
+    x = rng.normal(0, 1, cols).astype(np.float32)
+    qs, d = oracle.quantize_q8_0(x)
+    raw = torch.zeros(w.size + 64, dtype=torch.uint8, device="cuda")
+    want, wpart = oracle.gemv(synth.Q4_0, w, rows, cols, qs, d, want_partials=True)
+    dq, dd = g.dev(qs), g.dev(d)
+    for shift in (0, 2, 16, 18):
+        raw[shift:shift + w.size] = torch.from_numpy(w.reshape(-1)).cuda()
+        out, part = g.empty(rows, np.float32), g.empty((rows, cols // 32), np.int32)
+        capi.call("wd_gemv_q8_0_f32", synth.Q4_0, C.c_void_p(raw.data_ptr() + shift), rows, cols, g.ptr(dq), g.ptr(dd),
+                  g.ptr(out), g.ptr(part), g.stream())
+        g.sync()
+        assert np.array_equal(g.host(part), wpart), shift
+        assert np.allclose(g.host(out), want, rtol=1e-5, atol=1e-7), shift
 
 
 @pytest.mark.parametrize("t,rows,cols,experts", [(synth.IQ3_S, 512, 2048, 20), (synth.IQ2_S, 640, 2560, 20),

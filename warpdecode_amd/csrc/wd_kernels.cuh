@@ -197,17 +197,17 @@ __global__ __launch_bounds__(256) void k_gemv_q8(MatSrc src, int rows, int cols,
 // out of the 36 dwords in registers (even blocks with four byte-align ops, odd blocks are dword aligned).  Lane l
 // always works on column group l % lpr.  The workgroup keeps the activation in LDS (each group's 256 bytes padded
 // to 272 so that the 16-byte reads of neighbouring groups fall on different banks), with the per-block scale as a
-// float and 8 * sum(a) beside it; few registers per lane keep many waves, i.e. many loads, in flight, and the next
-// pass's loads are issued before the current one is computed.  Block sums are exact; the float side adds a lane's
+// float and 8 * sum(a) beside it; Block sums are exact; the float side adds a lane's
 // eight blocks in order and folds the row's lanes with an xor tree (Q4_0 has no canonical float order).
-// grid.x * 4 waves * passes_per_wave passes cover ceil(rows / (64 / lpr)) passes.
+// A wave takes NP consecutive passes and requests all of them before it touches the first.
+// grid.x * WPB waves * NP passes cover ceil(rows / (64 / lpr)) passes.
 // dynamic LDS: lpr * 272 bytes of quants, then nb floats, then nb ints.
-template <bool PART>
-__global__ __launch_bounds__(256) void k_gemv_q4_stream(const uint8_t *__restrict__ w, int rows, int nb, int passes_per_wave,
+template <bool PART, int NP, int WPB>
+__global__ __launch_bounds__(WPB * 64) void k_gemv_q4_stream(const uint8_t *__restrict__ w, int rows, int nb,
                                                          const int8_t *__restrict__ act_qs,
                                                          const uint16_t *__restrict__ act_d, float *__restrict__ out,
                                                          int32_t *__restrict__ partials) {
-    __shared__ uint4 stage[4][9 * 64];
+    __shared__ uint4 stage[WPB][9 * 64];
     extern __shared__ __align__(16) uint8_t q4_act[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lpr = nb >> 3, lpr_shift = __builtin_ctz(lpr), rpp = 64 >> lpr_shift;
@@ -215,9 +215,9 @@ __global__ __launch_bounds__(256) void k_gemv_q4_stream(const uint8_t *__restric
     float *ad = reinterpret_cast<float *>(q4_act + lpr * 272);
     int *corr = reinterpret_cast<int *>(ad + nb);
     const size_t rb = static_cast<size_t>(nb) * 18;
-    const long long pass0 = (static_cast<long long>(blockIdx.x) * 4 + wave) * passes_per_wave;
-    uint4 v[9];
-    auto fetch = [&](long long pass) {
+    const long long pass0 = (static_cast<long long>(blockIdx.x) * WPB + wave) * NP;
+    uint4 v[NP][9];
+    auto fetch = [&](long long pass, int slot) {
         const long long row0 = pass * rpp;
         const long long left = static_cast<long long>(rows) - row0;
         const size_t valid = left <= 0 ? 0 : static_cast<size_t>(left < rpp ? left : rpp) * rb;
@@ -225,10 +225,10 @@ __global__ __launch_bounds__(256) void k_gemv_q4_stream(const uint8_t *__restric
 #pragma unroll
         for (int k = 0; k < 9; ++k) {
             const size_t off = static_cast<size_t>(k) * 1024 + static_cast<size_t>(lane) * 16;
-            v[k] = off < valid ? gld_u128_aligned(base + off) : make_uint4(0, 0, 0, 0);
+            v[slot][k] = off < valid ? gld_u128_aligned(base + off) : make_uint4(0, 0, 0, 0);
         }
     };
-    // activation into LDS: thread t takes 16-byte pieces t, t + 256, ...; a block's two pieces give its sum.  The
+    // activation into LDS: thread t takes 16-byte pieces t, t + blockDim.x, ...; a block's two pieces give its sum.  The
     // first piece is requested before the weights so that it can be consumed while they are still in flight.
     const int n_pieces = nb * 2;
     uint4 q0 = make_uint4(0, 0, 0, 0);
@@ -237,8 +237,9 @@ __global__ __launch_bounds__(256) void k_gemv_q4_stream(const uint8_t *__restric
         q0 = *reinterpret_cast<const uint4 *>(act_qs + threadIdx.x * 16);
         d0 = act_d[threadIdx.x >> 1];
     }
-    fetch(pass0);
-    for (int i = threadIdx.x; i < n_pieces; i += 256) {
+#pragma unroll
+    for (int p = 0; p < NP; ++p) fetch(pass0 + p, p);
+    for (int i = threadIdx.x; i < n_pieces; i += WPB * 64) {
         const bool first = i == static_cast<int>(threadIdx.x);
         const uint4 q = first ? q0 : *reinterpret_cast<const uint4 *>(act_qs + i * 16);
         *reinterpret_cast<uint4 *>(q4_act + (i >> 4) * 272 + (i & 15) * 16) = q;
@@ -254,11 +255,12 @@ __global__ __launch_bounds__(256) void k_gemv_q4_stream(const uint8_t *__restric
     }
     __syncthreads();
     const uint8_t *my_act = q4_act + col * 272;
-    for (int p = 0; p < passes_per_wave; ++p) {
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
         const long long row0 = (pass0 + p) * rpp;
         if (row0 >= rows) break;  // wave-uniform
 #pragma unroll
-        for (int k = 0; k < 9; ++k) stage[wave][k * 64 + lane] = v[k];
+        for (int k = 0; k < 9; ++k) stage[wave][k * 64 + lane] = v[p][k];
         wave_lds_fence();
         uint32_t d[36];
 #pragma unroll
@@ -267,7 +269,6 @@ __global__ __launch_bounds__(256) void k_gemv_q4_stream(const uint8_t *__restric
             d[4 * k] = u.x, d[4 * k + 1] = u.y, d[4 * k + 2] = u.z, d[4 * k + 3] = u.w;
         }
         wave_lds_fence();
-        if (p + 1 < passes_per_wave) fetch(pass0 + p + 1);
         const int row = static_cast<int>(row0) + rsub;
         float sumf = 0.0f;
 #pragma unroll

@@ -198,15 +198,22 @@ static int launch_gemv_q8_0(int type, MatSrc src, int mats, int rows, int cols, 
         // whole 8-block groups per row and a 16-byte aligned base: the streaming kernel
         const int rpp = 64 / (nb / 8);
         const long long passes = (static_cast<long long>(rows) + rpp - 1) / rpp;
-        static const int forced = getenv("WD_Q4_PASSES") ? atoi(getenv("WD_Q4_PASSES")) : 0;
-        long long per_wave = forced > 0 ? forced : passes / 16384;
-        per_wave = per_wave < 1 ? 1 : (per_wave > 8 ? 8 : per_wave);
-        const unsigned wgs = static_cast<unsigned>((passes + per_wave * 4 - 1) / (per_wave * 4));
+        // four waves per workgroup stream best; two when the whole matrix is only a few hundred passes
+        const int wpb = passes <= 256 ? 2 : 4;
+        const unsigned wgs = static_cast<unsigned>((passes + wpb - 1) / wpb);
         const size_t lds = static_cast<size_t>(nb / 8) * 272 + static_cast<size_t>(nb) * 8;
-        if (partials)
-            k_gemv_q4_stream<true><<<wgs, 256, lds, stream>>>(src.single, rows, nb, static_cast<int>(per_wave), qs, d, out, partials);
+#define WD_Q4S_LAUNCH(WPB)                                                                                              \
+    do {                                                                                                                \
+        if (partials)                                                                                                   \
+            k_gemv_q4_stream<true, 1, WPB><<<wgs, WPB * 64, lds, stream>>>(src.single, rows, nb, qs, d, out, partials); \
+        else                                                                                                            \
+            k_gemv_q4_stream<false, 1, WPB><<<wgs, WPB * 64, lds, stream>>>(src.single, rows, nb, qs, d, out, nullptr); \
+    } while (0)
+        if (wpb == 2)
+            WD_Q4S_LAUNCH(2);
         else
-            k_gemv_q4_stream<false><<<wgs, 256, lds, stream>>>(src.single, rows, nb, static_cast<int>(per_wave), qs, d, out, nullptr);
+            WD_Q4S_LAUNCH(4);
+#undef WD_Q4S_LAUNCH
         WD_LAUNCH_CHECK();
         return WD_OK;
     }
