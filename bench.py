@@ -27,6 +27,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 STACK_FLAGS = int(os.environ.get("WD_BENCH_FLAGS", "0"))   # experiments only (e.g. 4 = staged dispatches)
 CHAIN_FLAGS = int(os.environ.get("WD_BENCH_CHAIN_FLAGS", "0"))   # experiments only (0x80 = launch floor)
+TOKEN_MIX = float(os.environ.get("WD_BENCH_TOKEN_MIX", "0.6"))   # tokens mode: share of the common direction in every token
 RESIDUAL_SCALE = 2.0 ** -12   # glue between layers: x += scale * layer(x), keeps the chain finite
 
 
@@ -46,10 +47,12 @@ def parse():
     ap.add_argument("--experts", type=int, default=512)
     ap.add_argument("--routing", choices=["zipf", "router"], default="zipf",
                     help="zipf: ids replayed from the Zipf(1.1) trace; router: ids chosen by the router itself")
-    ap.add_argument("--mode", choices=["resident", "lru", "q4-sweep"], default="resident",
+    ap.add_argument("--mode", choices=["resident", "lru", "q4-sweep", "tokens", "c0"], default="resident",
                     help="resident: C3 mode A, every expert in HBM; lru: C3 mode B, experts in pinned host memory "
-                         "behind an LRU slot pool of --cache-gib in HBM; q4-sweep: the dense Q4_0 GEMV shapes "
-                         "(secondary workload, own JSON line)")
+                         "behind an LRU slot pool of --cache-gib in HBM; q4-sweep: the dense Q4_0 GEMV shapes; "
+                         "tokens: the 4-token speculative-verify pass over the same layers; c0: the 64-expert top-8 "
+                         "all-Q8_0 layer (secondary workloads, own JSON lines)")
+    ap.add_argument("--tokens", type=int, default=4, help="tokens mode: tokens per pass (<= 8)")
     ap.add_argument("--cache-gib", type=float, default=32.0)
     ap.add_argument("--cache-warm-tokens", type=int, default=256,
                     help="lru mode: tokens run before the warm-up steps so that the slot pool is in steady state")
@@ -389,6 +392,77 @@ def bench_q4_sweep(args, torch, capi, synth):
                          kernel="k_gemv_q8<Q4_0>", us_per_launch=head["us_per_gemv"], bytes_per_launch=head["bytes"])}))
 
 
+def bench_tokens(args, torch, capi, synth):
+    """Speculative-verify batch (BASELINE.json configs[4]): T correlated tokens through each of the C2 layers in one
+    pass that reads every selected expert once, against T one-token passes over the same layers.  The router picks
+    the experts; the tokens are mixed from a common direction so that their top-10 sets overlap by about half."""
+    H, F, k, E, NL, T = 2048, 512, 10, args.experts, args.layers, args.tokens
+    layers, keep = build_stack(torch, synth, capi, NL, E, synth.BASE_SEED)
+    rng = synth.rng_for(synth.BASE_SEED, 9104)
+    base = rng.normal(0, 1, H)
+    xs = np.stack([TOKEN_MIX * base + (1.0 - TOKEN_MIX) * rng.normal(0, 1, H) for _ in range(T)])
+    xs = (xs / np.sqrt((xs ** 2).mean(axis=1, keepdims=True))).astype(np.float32)
+    d_x = torch.from_numpy(xs).cuda()
+    d_out = torch.zeros((T, H), dtype=torch.float32, device="cuda")
+    d_out1 = torch.zeros((T, H), dtype=torch.float32, device="cuda")
+    scr = []
+    for _ in range(T):
+        h = C.c_void_p()
+        capi.call("wd_moe_scratch_create", C.byref(h), H, F, E, k)
+        scr.append(h)
+    arr = (C.c_void_p * T)(*[h.value for h in scr])
+    stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    lib = capi.load()
+
+    def batch(l):
+        capi.call("wd_moe_layer_tokens_f32", C.byref(layers[l]), C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()), T, arr,
+                  0, stream())
+
+    def serial(l):
+        for t in range(T):
+            capi.call("wd_moe_layer_f32", C.byref(layers[l]), C.c_void_p(d_x[t].data_ptr()), C.c_void_p(d_out1[t].data_ptr()),
+                      scr[t], 0, stream())
+
+    unions, same = [], True
+    for l in range(NL):                       # untimed: union sizes, and the two ways must agree bit for bit
+        batch(l)
+        torch.cuda.synchronize()
+        ids = np.empty((T, k), np.int32)
+        for t in range(T):
+            capi.call("wd_memcpy_d2h", ids[t].ctypes.data_as(C.c_void_p), C.c_void_p(lib.wd_moe_scratch_ids(scr[t])), 4 * k, None)
+        unions.append(len(set(ids.reshape(-1).tolist())))
+        serial(l)
+        torch.cuda.synchronize()
+        same = same and bool(torch.equal(d_out.view(torch.int32), d_out1.view(torch.int32)))
+    note("union of the %d top-%d sets: mean %.1f experts (min %d, max %d); batch == serial bit for bit: %s"
+         % (T, k, np.mean(unions), min(unions), max(unions), same))
+    if not same:
+        print("bench.py: the token batch differs from the one-token passes", file=sys.stderr)
+        sys.exit(1)
+    reps = 10
+    us_batch = graph_period_us(torch, batch, NL, reps)
+    us_serial = graph_period_us(torch, serial, NL, reps)
+    q8h, q8f, iq3h = synth.row_bytes(synth.Q8_0, H), synth.row_bytes(synth.Q8_0, F), synth.row_bytes(synth.IQ3_S, H)
+    per_expert = 2 * F * iq3h + H * q8f
+    fixed = E * H * 4 + H * 4 + 2 * F * q8h + H * q8f
+    union_bytes = np.mean(unions) * per_expert + fixed
+    serial_bytes = T * (k * per_expert + fixed)
+    print(json.dumps({
+        "metric": "speculative-verify pass of %d tokens through one MoE layer: us per layer" % T,
+        "value": round(us_batch, 2), "unit": "us", "n_gpus": 1, "higher_is_better": False, "vs_baseline": None,
+        "dtype": "int8 dot products (IQ3_S/Q8_0 weights x Q8_K/Q8_0 activations), f32 accumulate", "data": "synthetic",
+        "config": {"workload": "C4: %d tokens (router-selected, correlated inputs) through each of %d C2 layers, "
+                               "each selected expert read once per pass" % (T, NL),
+                   "tokens": T, "layers": NL, "experts": E, "top_k": k, "union_mean": round(float(np.mean(unions)), 2),
+                   "union_min": min(unions), "union_max": max(unions), "batch_equals_serial_bitwise": same,
+                   "us_per_layer_batch": round(us_batch, 2), "us_per_layer_serial": round(us_serial, 2),
+                   "speedup_vs_serial": round(us_serial / us_batch, 3),
+                   "union_bytes_per_layer": int(union_bytes), "serial_bytes_per_layer": int(serial_bytes)},
+        "roofline": dict(bound="hbm", achieved=round(union_bytes / us_batch / 1e3, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                         frac=round(union_bytes / us_batch / 1e3 / HBM_PEAK_GBS, 4), traffic=None,
+                         kernel="whole pass (k_tokens_a, k_tokens_b, k_tokens_c)")}))
+
+
 def main():
     if len(sys.argv) >= 5 and sys.argv[1] == "--cpu-child":
         cpu_child(float(sys.argv[2]), int(sys.argv[3]), sys.argv[4])
@@ -407,6 +481,8 @@ def main():
     if args.mode == "q4-sweep":
         return bench_q4_sweep(args, torch, capi, synth)
     note("generating %d layers x %d experts on the device" % (NL, E))
+    if args.mode == "tokens":
+        return bench_tokens(args, torch, capi, synth)
     if args.mode == "lru":
         return bench_lru(args, torch, capi, synth)
     layers, keep = build_stack(torch, synth, capi, NL, E, synth.BASE_SEED)

@@ -57,6 +57,22 @@ WD_DEV void mark(const LayerArgs &a, int d, int i) {
 
 // ---- in-workgroup quantisers (results in LDS) ------------------------------------------------
 // Q8_0 of n values (multiple of 32): four threads per block, eight values per thread.
+// The step on eight loaded values (v0, v1 = x[base .. base + 8)); all four threads of a block must call it.
+WD_DEV void lds_quantize_q8_0_step(const float4 &v0, const float4 &v1, bool on, int base, int8_t *qs, uint16_t *d, int tid) {
+    float amax = __builtin_fmaxf(
+        __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v0.x), __builtin_fabsf(v0.y)),
+                        __builtin_fmaxf(__builtin_fabsf(v0.z), __builtin_fabsf(v0.w))),
+        __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v1.x), __builtin_fabsf(v1.y)),
+                        __builtin_fmaxf(__builtin_fabsf(v1.z), __builtin_fabsf(v1.w))));
+    amax = quad_max(amax);
+    if (on) {
+        uint2 packed;
+        packed.x = q8_0_pack4(v0, amax);
+        packed.y = q8_0_pack4(v1, amax);
+        *reinterpret_cast<uint2 *>(qs + base) = packed;
+        if ((tid & 3) == 0) d[base >> 5] = f2h_ref(amax / 127.0f);
+    }
+}
 WD_DEV void lds_quantize_q8_0(const float *__restrict__ x, int n, int8_t *qs, uint16_t *d, int tid, int nthreads) {
     const int per_pass = nthreads * 8;
     for (int base0 = 0; base0 < n; base0 += per_pass) {
@@ -67,25 +83,17 @@ WD_DEV void lds_quantize_q8_0(const float *__restrict__ x, int n, int8_t *qs, ui
             v0 = *reinterpret_cast<const float4 *>(x + base);
             v1 = *reinterpret_cast<const float4 *>(x + base + 4);
         }
-        float amax = __builtin_fmaxf(
-            __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v0.x), __builtin_fabsf(v0.y)),
-                            __builtin_fmaxf(__builtin_fabsf(v0.z), __builtin_fabsf(v0.w))),
-            __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v1.x), __builtin_fabsf(v1.y)),
-                            __builtin_fmaxf(__builtin_fabsf(v1.z), __builtin_fabsf(v1.w))));
-        amax = quad_max(amax);
-        if (on) {
-            uint2 packed;
-            packed.x = q8_0_pack4(v0, amax);
-            packed.y = q8_0_pack4(v1, amax);
-            *reinterpret_cast<uint2 *>(qs + base) = packed;
-            if ((tid & 3) == 0) d[base >> 5] = f2h_ref(amax / 127.0f);
-        }
+        lds_quantize_q8_0_step(v0, v1, on, base, qs, d, tid);
     }
 }
 
 // Q8_K of one 256-value block by one wave (four values per lane).
+WD_DEV void wave_quantize_q8_k_regs(const float4 &v, int8_t *qs256, float *d, int lane);
 WD_DEV void wave_quantize_q8_k_block(const float *__restrict__ x256, int8_t *qs256, float *d, int lane) {
-    const float4 v = reinterpret_cast<const float4 *>(x256)[lane];
+    wave_quantize_q8_k_regs(reinterpret_cast<const float4 *>(x256)[lane], qs256, d, lane);
+}
+// The same on four loaded values per lane (v = x256[4 * lane .. 4 * lane + 4)).
+WD_DEV void wave_quantize_q8_k_regs(const float4 &v, int8_t *qs256, float *d, int lane) {
     float amax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)),
                                  __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
     amax = wave_max(amax);
@@ -561,7 +569,8 @@ WD_DEV void router_rows(const float *__restrict__ w, const float *__restrict__ x
 // ascending order while a lane holds only 32 weights (half the registers of the 32-lanes-per-row version,
 // which lets three workgroups of the merged dispatch share a compute unit).
 // Every thread of the workgroup must call it (it contains a barrier).
-template <bool COHERENT>
+// SCALAR_ROW: keep the wave's row pointer in scalar registers (two vector registers fewer).
+template <bool COHERENT, bool SCALAR_ROW = false>
 WD_DEV void router_rows_wave(const float *__restrict__ w, const float *__restrict__ x, float *xs, float *logits, int rows,
                              int cols, const float *__restrict__ extra_w, float *extra_out, int wg) {
     const int lane = threadIdx.x & 63, t = lane & 31;
@@ -570,6 +579,12 @@ WD_DEV void router_rows_wave(const float *__restrict__ w, const float *__restric
     const int total = rows + (extra_w ? 1 : 0);
     const bool on = row < total;
     const float *wr = on ? (row < rows ? w + static_cast<size_t>(row) * cols : extra_w) : x;
+    if (SCALAR_ROW) {  // the row is the same for the whole wave
+        const uintptr_t v = reinterpret_cast<uintptr_t>(wr);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+        const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+        wr = reinterpret_cast<const float *>((static_cast<uintptr_t>(hi) << 32) | lo);
+    }
     const int np = cols & ~31;
     const int half_off = (upper ? 1024 : 0) + t;
     float wv[32];

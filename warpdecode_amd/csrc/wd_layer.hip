@@ -30,7 +30,6 @@ struct wd_moe_scratch {
     int32_t *dp = nullptr;
     int gup_type = -1, dp_type = -1;
     unsigned *arrive = nullptr;           // device counter used inside the fused dispatch A
-    int32_t *union_buf = nullptr;         // [1 + 128 + 128 * 8] expert union of a multi-token pass
     unsigned long long *trace = nullptr;  // device [3][16][8] time stamps, see wd_moe_scratch_trace
     int trace_wg = 0;
     int32_t *h_ids = nullptr;             // pinned [16]: routed ids for callers that must see them on the host
@@ -77,7 +76,7 @@ int wd_moe_scratch_create(wd_moe_scratch **out, int hidden, int expert_ffn, int 
                  o_act = c.take(sizeof(float) * K1 * F), o_aq = c.take(K1 * F),
                  o_ad = c.take(sizeof(uint16_t) * K1 * (F / 32)), o_eo = c.take(sizeof(float) * K1 * H),
                  o_acc = c.take(sizeof(float) * H), o_dn = c.take(sizeof(float) * H), o_sg = c.take(256),
-                 o_arr = c.take(256), o_uni = c.take(sizeof(int32_t) * (1 + 128 + 128 * kMaxTokens)),
+                 o_arr = c.take(256),
                  o_tag = c.take(sizeof(uint32_t) * kTagRecords * kTagCopies * 16), o_status = c.take(256);
     const hipError_t e = hipMalloc(reinterpret_cast<void **>(&s->block), c.off);
     if (e != hipSuccess) {
@@ -102,7 +101,6 @@ int wd_moe_scratch_create(wd_moe_scratch **out, int hidden, int expert_ffn, int 
     s->down_f32 = reinterpret_cast<float *>(b + o_dn);
     s->shared_gate = reinterpret_cast<float *>(b + o_sg);
     s->arrive = reinterpret_cast<unsigned *>(b + o_arr);
-    s->union_buf = reinterpret_cast<int32_t *>(b + o_uni);
     s->tagged = reinterpret_cast<uint32_t *>(b + o_tag);
     s->status = reinterpret_cast<unsigned *>(b + o_status);
     (void)hipMemset(s->block, 0, c.off);
@@ -537,35 +535,45 @@ extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, 
         return WD_OK;
     }
     TokenArgs ta{};
-    ta.T = tokens, ta.H = H, ta.F = F, ta.k = k;
+    ta.T = tokens;
+    ta.common = fused_args(L, d_x, d_out, scratch_per_token[0], flags, nullptr, nullptr, 0.0f);
+    ta.common.gate_up = routed_src(L, nullptr, false);  // the kernels pass the expert id themselves
+    ta.common.down = routed_src(L, nullptr, true);
     for (int t = 0; t < tokens; ++t) {
         wd_moe_scratch *s = scratch_per_token[t];
-        const LayerArgs a = fused_args(L, d_x + static_cast<size_t>(t) * H, d_out + static_cast<size_t>(t) * H, s, flags,
-                                       nullptr, nullptr, 0.0f);
-        if (const int rc = launch_a(a, st)) return rc;  // router, selection, shared gate/up of token t
-        ta.x[t] = a.x, ta.ids[t] = s->ids, ta.weights[t] = s->weights, ta.act[t] = s->act;
-        ta.shared_gate[t] = s->shared_gate;
-        ta.expert_out[t] = (flags & WD_MOE_KEEP_EXPERT_OUT) ? s->expert_out : nullptr;
-        ta.accum[t] = s->accum, ta.down_f32[t] = s->down_f32, ta.out[t] = a.out;
+        TokenSlots &k_ = ta.tok[t];
+        k_.x = d_x + static_cast<size_t>(t) * H, k_.out = d_out + static_cast<size_t>(t) * H;
+        k_.logits = s->logits, k_.ids = s->ids, k_.weights = s->weights, k_.act = s->act;
+        k_.shared_gate = s->shared_gate, k_.arrive = s->arrive;
+        k_.expert_out = (flags & WD_MOE_KEEP_EXPERT_OUT) ? s->expert_out : nullptr;
+        k_.accum = s->accum, k_.down_f32 = s->down_f32;
     }
-    ta.gate_up = routed_src(L, nullptr, false);
-    ta.down = routed_src(L, nullptr, true);
-    ta.sh_down = L->shared_gate_inp ? L->shared_down : nullptr;
-    int32_t *ub = scratch_per_token[0]->union_buf;
-    ta.union_count = ub, ta.union_ids = ub + 1, ta.union_slot = ub + 1 + 128;
-    k_tokens_union<<<dim3(1), dim3(64), 0, st>>>(ta);
-    WD_LAUNCH_CHECK();
+    LayerArgs &a = ta.common;
+    a.n_router_wgs = ((a.preselected ? 0 : a.E) + (a.sh_inp ? 1 : 0) + 7) / 8;  // one router row per wave
+    const int grid_a = a.n_router_wgs + (a.sh_inp ? (F + 7) / 8 : 0);
+    if (grid_a > 0) {  // router, selection and shared gate/up of every token
+        k_tokens_a<<<dim3(grid_a, tokens), dim3(512), static_cast<size_t>(H) * 4 + 16, st>>>(ta);
+        WD_LAUNCH_CHECK();
+    }
     const size_t lds_b = static_cast<size_t>(tokens) * (H + sizeof(float) * (H / 256));
-    const int grid_b = tokens * k * ((F + 7) / 8);
-    if (L->gate_type == WD_TYPE_IQ3_S)
-        k_tokens_b<21><<<dim3(grid_b), dim3(512), lds_b, st>>>(ta);
-    else
-        k_tokens_b<22><<<dim3(grid_b), dim3(512), lds_b, st>>>(ta);
+    const int items_b = tokens * k * ((F + 7) / 8);
+    const int grid_b = items_b < 512 ? items_b : 512;  // persistent: two workgroups per compute unit walk the items
+    if (L->gate_type == WD_TYPE_IQ3_S) {
+        if (tokens <= 4)
+            k_tokens_b<21, 4><<<dim3(grid_b), dim3(512), lds_b, st>>>(ta);
+        else
+            k_tokens_b<21, kMaxTokens><<<dim3(grid_b), dim3(512), lds_b, st>>>(ta);
+    } else {
+        if (tokens <= 4)
+            k_tokens_b<22, 4><<<dim3(grid_b), dim3(512), lds_b, st>>>(ta);
+        else
+            k_tokens_b<22, kMaxTokens><<<dim3(grid_b), dim3(512), lds_b, st>>>(ta);
+    }
     WD_LAUNCH_CHECK();
     const int waves_c = 16;
     const size_t per_wave = (static_cast<size_t>(F) + F / 16 + 15) & ~static_cast<size_t>(15);
-    const size_t lds_c = waves_c * per_wave + sizeof(float) * 4 * tokens * (k + 1);
-    k_tokens_c<<<dim3((H + 3) / 4), dim3(64 * waves_c), lds_c, st>>>(ta);
+    const size_t lds_c = waves_c * per_wave + sizeof(float) * 8 * tokens * (k + 1);
+    k_tokens_c<<<dim3((H + 7) / 8), dim3(64 * waves_c), lds_c, st>>>(ta);
     WD_LAUNCH_CHECK();
     return WD_OK;
 }

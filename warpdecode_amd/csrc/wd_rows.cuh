@@ -164,6 +164,37 @@ WD_DEV void iq_chunks(const IqFields &f, int ib, const IqTables &t, const uint32
     }
 }
 
+// The same in two steps, for callers that apply one decoded sub-block to several activations: the 32 signed
+// weights (eight packed dwords) and the odd sub-scale of every chunk first, the chunk sums per activation after.
+template <int TYPE>
+WD_DEV void iq_decode(const IqFields &f, int ib, const IqTables &t, uint32_t (&w)[8], int (&ls)[2]) {
+    if (TYPE == 21) {
+        ls[0] = ls[1] = 1 + 2 * static_cast<int>((f.sc >> (4 * (ib & 1))) & 15u);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const uint32_t q = ((c < 4 ? f.qs.x : f.qs.y) >> (8 * (c & 3))) & 0xffu;
+            const uint32_t idx = q | ((f.qh << (8 - c)) & 0x100u);
+            const uint32_t sbits = (f.sg >> (4 * c)) & 15u;
+            w[c] = apply_signs(t.grid3[idx], t.sign[sbits]);
+        }
+    } else {
+        ls[0] = 1 + 2 * static_cast<int>(f.sc & 15u);  // chunks 0..3
+        ls[1] = 1 + 2 * static_cast<int>(f.sc >> 4);   // chunks 4..7
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const uint32_t idx = ((f.qs.x >> (8 * g)) & 0xffu) | ((f.qh << (8 - 2 * g)) & 0x300u);
+            const uint64_t mags = t.grid2[idx];
+            const uint32_t s8 = (f.qs.y >> (8 * g)) & 0xffu;
+            w[2 * g] = apply_signs(static_cast<uint32_t>(mags), t.sign[s8 & 15u]);
+            w[2 * g + 1] = apply_signs(static_cast<uint32_t>(mags >> 32), t.sign[s8 >> 4]);
+        }
+    }
+}
+WD_DEV void iq_dot_decoded(const uint32_t (&w)[8], const int (&ls)[2], const uint32_t (&a)[8], int (&p)[8]) {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) p[c] = __mul24(ls[c >> 2], sdot4(w[c], a[c], 0));
+}
+
 // NR rows against one Q8_K activation (act_qs / act_d in global memory or LDS).  y[i] is uniform
 // across the wave.  `partials` (PART only): int32 [nb][8] per row, rows `pstride` ints apart.
 //
@@ -375,20 +406,22 @@ WD_DEV void q8_rows4_multi(const uint8_t *const (&rows)[NM], int nrows, int nb, 
                 const int base = base0 + 16 * ch;
 #pragma unroll
                 for (int s = 0; s < 16; ++s) {
-                    if (base + s < nb) {
+                    if (KIND == 1) {
+                        const int blk_i = base + s;
+                        if (blk_i < paired) {
+                            const float pv = tile.pf[ch][r4 * 136 + s * 8 + c];
+                            const float dv = tile.ds[ch][r4 * 16 + s];
+                            if (blk_i & 1)
+                                acc_odd[i] = __builtin_fmaf(dv, pv, acc_odd[i]);
+                            else
+                                acc[i] = __builtin_fmaf(dv, pv, acc[i]);
+                        }
+                    } else {
+                        // every slot of the tile was written this pass, zeros for the blocks past the end of the row:
+                        // those steps are fma(0, 0, acc) == acc (acc is never -0), so the chain needs no test
                         const float pv = tile.pf[ch][r4 * 136 + s * 8 + c];
                         const float dv = tile.ds[ch][r4 * 16 + s];
-                        if (KIND == 1) {
-                            const int blk_i = base + s;
-                            if (blk_i < paired) {
-                                if (blk_i & 1)
-                                    acc_odd[i] = __builtin_fmaf(dv, pv, acc_odd[i]);
-                                else
-                                    acc[i] = __builtin_fmaf(dv, pv, acc[i]);
-                            }
-                        } else {
-                            acc[i] = __builtin_fmaf(dv, pv, acc[i]);
-                        }
+                        acc[i] = __builtin_fmaf(dv, pv, acc[i]);
                     }
                 }
                 if (KIND == 1 && (nb & 1) && base < nb && base + 16 >= nb) {
