@@ -392,6 +392,61 @@ def bench_q4_sweep(args, torch, capi, synth):
                          kernel="k_gemv_q8<Q4_0>", us_per_launch=head["us_per_gemv"], bytes_per_launch=head["bytes"])}))
 
 
+def bench_c0(args, torch, capi, synth):
+    """BASELINE.json configs[0] at stack depth: the 64-expert top-8 layer with Q8_0 gate/up/down and no shared expert
+    (hidden 2048, ffn 512), `--layers` independent layers chained as in the headline workload, router-selected."""
+    H, F, k, E, NL = 2048, 512, 8, 64, args.layers
+    g = torch.Generator(device="cuda")
+    g.manual_seed(synth.BASE_SEED + 5)
+    rb_h, rb_f = synth.row_bytes(synth.Q8_0, H), synth.row_bytes(synth.Q8_0, F)
+
+    def q8(rows, cols):
+        nb = rows * (cols // 32)
+        t = torch.randint(-127, 128, (nb * 34,), dtype=torch.int8, device="cuda", generator=g).view(torch.uint8)
+        d = (torch.randn(nb, device="cuda", generator=g).abs() * (0.02 / 127.0)).half()
+        t.view(-1, 34)[:, 0:2] = d.view(torch.uint8).view(-1, 2)
+        return t
+
+    layers, keep = (capi.MoeLayer * NL)(), []
+    for l in range(NL):
+        t = dict(router=torch.randn(E, H, device="cuda", generator=g) * 0.02, gate=q8(E * F, H), up=q8(E * F, H),
+                 down=q8(E * H, F))
+        keep.append(t)
+        d = layers[l]
+        d.hidden, d.expert_ffn, d.n_experts, d.top_k, d.expert_scale = H, F, E, k, 1.0
+        d.gate_type = d.up_type = d.down_type = synth.Q8_0
+        for name, tensor in t.items():
+            setattr(d, name, tensor.data_ptr())
+        d.gate_stride = d.up_stride = F * rb_h
+        d.down_stride = H * rb_f
+    scratch = C.c_void_p()
+    capi.call("wd_moe_scratch_create", C.byref(scratch), H, F, E, k)
+    rng = synth.rng_for(synth.BASE_SEED, 9200)
+    d_x = torch.from_numpy(synth.rms_normed(rng, H)).cuda()
+    d_out = torch.zeros(H, dtype=torch.float32, device="cuda")
+
+    def launch(_i):
+        capi.call("wd_moe_stack_f32", layers, NL, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()), scratch, None,
+                  RESIDUAL_SCALE, 0, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+    us = graph_period_us(torch, launch, 1, 50) / NL
+    ok = bool(torch.isfinite(d_x).all().item()) and capi.load().wd_moe_scratch_status(scratch) == 0
+    nbytes = E * H * 4 + k * (2 * F * rb_h + H * rb_f)
+    assert nbytes == 27262976
+    print(json.dumps({
+        "metric": "MoE layer batch=1 decode, 64 experts top-8 all Q8_0: us per layer", "value": round(us, 2), "unit": "us",
+        "n_gpus": 1, "higher_is_better": False, "vs_baseline": None,
+        "dtype": "int8 dot products (Q8_0 weights x Q8_0 activations), f32 accumulate", "data": "synthetic",
+        "config": {"workload": "C0: %d chained layers of hidden 2048, 64 experts, top-8, ffn 512, Q8_0 gate/up/down, "
+                               "router-selected, batch=1, HIP-graph replay" % NL,
+                   "layers": NL, "bytes_per_layer": nbytes, "tok_s_at_%d_layers" % NL: round(1e6 / (us * NL), 1), "valid": ok},
+        "roofline": dict(bound="hbm", achieved=round(nbytes / us / 1e3, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                         frac=round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), traffic=None,
+                         kernel="whole layer (k_layer_ab<Q8_0>, k_layer_c)")}))
+    if not ok:
+        sys.exit(1)
+
+
 def bench_tokens(args, torch, capi, synth):
     """Speculative-verify batch (BASELINE.json configs[4]): T correlated tokens through each of the C2 layers in one
     pass that reads every selected expert once, against T one-token passes over the same layers.  The router picks
@@ -480,6 +535,8 @@ def main():
     H, F, k, E, NL = 2048, 512, 10, args.experts, args.layers
     if args.mode == "q4-sweep":
         return bench_q4_sweep(args, torch, capi, synth)
+    if args.mode == "c0":
+        return bench_c0(args, torch, capi, synth)
     note("generating %d layers x %d experts on the device" % (NL, E))
     if args.mode == "tokens":
         return bench_tokens(args, torch, capi, synth)

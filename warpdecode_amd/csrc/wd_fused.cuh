@@ -840,8 +840,8 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
     mark(a, 1, 2);
     const int e = s_expert;
     if (e < 0 || e >= a.E) return;  // the wait ran out (status is set): leave without touching memory
-    const uint8_t *gate = mat_ptr_ids(a.gate_up, 2 * j, e);
-    const uint8_t *up = mat_ptr_ids(a.gate_up, 2 * j + 1, e);
+    const uint8_t *gate = mat_ptr_expert<0>(a.gate_up, e);
+    const uint8_t *up = mat_ptr_expert<1>(a.gate_up, e);
     float *act = a.act + static_cast<size_t>(j) * a.F;
     const int r = rg * 8 + wave;
     float gu[2];
@@ -889,8 +889,8 @@ __global__ __launch_bounds__(TYPE == 20 ? 256 : 512) void k_layer_b(LayerArgs a)
     const int j = blockIdx.x / groups;
     const int rg = blockIdx.x - j * groups;
     const int e = a.ids[j];
-    const uint8_t *gate = mat_ptr_ids(a.gate_up, 2 * j, e);
-    const uint8_t *up = mat_ptr_ids(a.gate_up, 2 * j + 1, e);
+    const uint8_t *gate = mat_ptr_expert<0>(a.gate_up, e);
+    const uint8_t *up = mat_ptr_expert<1>(a.gate_up, e);
     float *act = a.act + static_cast<size_t>(j) * a.F;
     if (kIq) {
         const int nb = a.H >> 8;
@@ -981,7 +981,8 @@ __global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
     }
     for (int m = wave; m < n_act; m += nwaves) {
         const bool is_shared = m == a.k;
-        const uint8_t *w = is_shared ? a.sh_down : mat_ptr_ids(a.down, m, a.ids[m]);
+        // m is the same for the whole wave: the id comes through the scalar path
+        const uint8_t *w = is_shared ? a.sh_down : mat_ptr_expert<0>(a.down, sld_i32(a.ids + m));
         const size_t rb = static_cast<size_t>(nb) * ((KIND == 0 || is_shared) ? 34 : 18);
         const uint8_t *const rows[1] = {w + r0 * rb};
         float y[1];

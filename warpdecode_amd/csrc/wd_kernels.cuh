@@ -35,11 +35,13 @@ WD_DEV const uint8_t *mat_ptr(const MatSrc &s, int m) {
     return s.single;
 }
 
-// Same, with the expert id already known to the caller (per_expert tensors per expert).
-WD_DEV const uint8_t *mat_ptr_ids(const MatSrc &s, int m, int e) {
-    const int t = m % s.per_expert;
-    if (s.slot_of_expert) return s.pool + static_cast<size_t>(s.slot_of_expert[e]) * s.slot_bytes + s.slot_off[t];
-    return s.base[t] + static_cast<size_t>(e) * s.stride[t];
+// Tensor T (0 = the first, 1 = the second of an expert's tensors in this source) of expert e.  T is a template
+// argument so that base, stride and slot offset are fixed members of the argument block (scalar registers, loaded
+// without waiting for e) instead of a lookup by a computed index.
+template <int T>
+WD_DEV const uint8_t *mat_ptr_expert(const MatSrc &s, int e) {
+    if (s.slot_of_expert) return s.pool + static_cast<size_t>(s.slot_of_expert[e]) * s.slot_bytes + s.slot_off[T];
+    return s.base[T] + static_cast<size_t>(e) * s.stride[T];
 }
 
 __global__ void k_fill_u32(uint32_t *dst, uint32_t v, size_t n) {

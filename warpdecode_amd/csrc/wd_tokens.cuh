@@ -230,7 +230,7 @@ __global__ __launch_bounds__(512, 4) void k_tokens_b(TokenArgs ta) {
         for (int t = 0; t < MAXT; ++t) rank[t] = __builtin_amdgcn_readfirstlane(static_cast<int>(un.rank[u][t]));
         const int r = rg * 8 + wave;
         const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
-        const uint8_t *const rows[2] = {mat_ptr_ids(a.gate_up, 0, e) + off, mat_ptr_ids(a.gate_up, 1, e) + off};
+        const uint8_t *const rows[2] = {mat_ptr_expert<0>(a.gate_up, e) + off, mat_ptr_expert<1>(a.gate_up, e) + off};
         float acc[MAXT][2];
 #pragma unroll
         for (int t = 0; t < MAXT; ++t) acc[t][0] = acc[t][1] = 0.0f;
@@ -358,7 +358,7 @@ __global__ __launch_bounds__(1024) void k_tokens_c(TokenArgs ta) {
             const bool is_shared = it_j[i] == a.k;
             const int pair = it_t[i] * a.k + (is_shared ? 0 : it_j[i]);
             const int e = pair < 64 ? __builtin_amdgcn_readlane(id_lo, pair) : __builtin_amdgcn_readlane(id_hi, pair - 64);
-            const uint8_t *w = is_shared ? a.sh_down : mat_ptr_ids(a.down, 0, e);
+            const uint8_t *w = is_shared ? a.sh_down : mat_ptr_expert<0>(a.down, e);
 #pragma unroll
             for (int g = 0; g < 2; ++g) {
                 const int row = min(r0 + 4 * g + r4, a.H - 1);
