@@ -950,7 +950,9 @@ __global__ __launch_bounds__(TYPE == 20 ? 256 : 512) void k_layer_b(LayerArgs a)
 // are in flight.  The first four lanes of wave 0 then fold the k+1 results in the reference order.
 // grid = ceil(H / 4), block = 64 * min(k + 1, 16).
 // dynamic LDS per wave: F bytes + F/32 halves (+ pad), then [k+1][4] floats.
-template <int KIND>
+// COAL: the rows are 16 blocks long, H is a multiple of 4 and every down tensor starts on a 16-byte boundary: the
+// four rows of a wave are fetched as aligned 16-byte words (q8_rows4x16).
+template <int KIND, bool COAL>
 __global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
     extern __shared__ __align__(16) uint8_t lds_c[];
     __shared__ Q8Tile tiles[16];
@@ -992,7 +994,9 @@ __global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
             wave_lds_fence();
             mark(a, 2, 1);
         };
-        if (KIND == 0 || is_shared)
+        if (COAL)
+            q8_rows4x16<1>(rows, aq, ad, tiles[wave], lane, y, quantise);
+        else if (KIND == 0 || is_shared)
             q8_rows4_multi<0, 1, 1, false>(rows, nrows, nb, aq, ad, tiles[wave], lane, y, nullptr, 0, quantise);
         else
             q8_rows4_multi<1, 1, 1, false>(rows, nrows, nb, aq, ad, tiles[wave], lane, y, nullptr, 0, quantise);

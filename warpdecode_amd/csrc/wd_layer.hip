@@ -436,10 +436,16 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
     const size_t per_wave = (static_cast<size_t>(F) + F / 16 + 15) & ~static_cast<size_t>(15);
     const size_t lds_c = waves_c * per_wave + sizeof(float) * 4 * n_act;
     const int grid_c = (H + 3) / 4;
-    if (L->down_type == WD_TYPE_Q8_0)
-        k_layer_c<0><<<dim3(grid_c), dim3(64 * waves_c), lds_c, st>>>(a);
+    auto al16 = [](const void *p_, size_t v) { return reinterpret_cast<uintptr_t>(p_) % 16 == 0 && v % 16 == 0; };
+    const bool coal = L->down_type == WD_TYPE_Q8_0 && F == 512 && H % 4 == 0 && al16(L->shared_down, 0) &&
+                      (L->slot_of_expert ? al16(L->slot_pool, L->slot_bytes) && (L->slot_gate_bytes + L->slot_up_bytes) % 16 == 0
+                                         : al16(L->down, L->down_stride));
+    if (coal)
+        k_layer_c<0, true><<<dim3(grid_c), dim3(64 * waves_c), lds_c, st>>>(a);
+    else if (L->down_type == WD_TYPE_Q8_0)
+        k_layer_c<0, false><<<dim3(grid_c), dim3(64 * waves_c), lds_c, st>>>(a);
     else
-        k_layer_c<1><<<dim3(grid_c), dim3(64 * waves_c), lds_c, st>>>(a);
+        k_layer_c<1, false><<<dim3(grid_c), dim3(64 * waves_c), lds_c, st>>>(a);
     WD_LAUNCH_CHECK();
     return WD_OK;
 }
