@@ -734,7 +734,9 @@ __global__ __launch_bounds__(512) void k_layer_a(LayerArgs a) {
 // store; a word other than kTagInvalid is the id itself, so a reader needs no second flag.  The words are reset
 // to kTagInvalid by dispatch C (or by the caller) before the next layer pass uses them.  The wait is bounded:
 // when it runs out the workgroup sets status[0] and returns.
-template <int TYPE>
+// COAL (IQ types): rows of eight super-blocks on 16-byte boundaries are fetched with one aligned 16-byte load per
+// lane and parked in LDS (iq_rows8_coal); dynamic LDS then has 8 * 2 * kIqStageBytes more bytes behind the 4 * H + 16.
+template <int TYPE, bool COAL>
 __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
     constexpr bool kIq = (TYPE == 21 || TYPE == 22);
     extern __shared__ __align__(16) uint8_t lds_ab[];
@@ -850,8 +852,12 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
         const size_t rb = static_cast<size_t>(nb) * (TYPE == 21 ? 110 : 82);
         const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
         const uint8_t *const rows[2] = {gate + off, up + off};
-        iq_rows_q8k<(kIq ? TYPE : 21), 2, false>(rows, nb, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
-                                                  nullptr, 0);
+        if (COAL)
+            iq_rows8_coal<(kIq ? TYPE : 21), 2>(rows, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
+                                                lds_ab + ((4 * a.H + 16 + 15) & ~15) + wave * 2 * kIqStageBytes);
+        else
+            iq_rows_q8k<(kIq ? TYPE : 21), 2, false>(rows, nb, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
+                                                      nullptr, 0);
     } else {
         Q8RowTile *tiles = reinterpret_cast<Q8RowTile *>(s_union);
         const int nb = a.H >> 5;

@@ -270,6 +270,79 @@ WD_DEV void iq_rows_q8k(const uint8_t *const (&rows)[NR], int nb, const IqTables
     }
 }
 
+// ---- IQ3_S / IQ2_S rows of exactly eight super-blocks, coalesced ------------------------------------------
+// Such a row is 880 (IQ3_S) or 656 (IQ2_S) contiguous bytes, a whole number of 16-byte words.  When it starts on a
+// 16-byte boundary the wave fetches it with one aligned 16-byte load per lane (55 or 41 lanes) instead of five
+// narrow loads per lane, parks it in LDS and picks the fields of (super-block, 32-value block) from there.
+// Blocks are only 2-byte aligned: fields wider than two bytes are read as aligned dwords and shifted by two bytes in
+// the even super-blocks (block offset 110 sb or 82 sb is 0 mod 4 there, and every such field sits at 2 mod 4).
+constexpr int kIqStageBytes = 896;  // per row, 16-byte multiple >= 880
+
+template <int TYPE>
+WD_DEV IqFields iq_fields_lds(const uint8_t *blk, int ib, int sb) {
+    const uint32_t sh = (sb & 1) ? 0u : 2u;
+    IqFields f;
+    f.d = *reinterpret_cast<const uint16_t *>(blk);
+    if (TYPE == 21) {
+        const uint32_t *q = reinterpret_cast<const uint32_t *>(blk + 2 + ib * 8 - sh);
+        const uint32_t r0 = q[0], r1 = q[1], r2 = q[2];
+        f.qs.x = __builtin_amdgcn_alignbyte(r1, r0, sh);
+        f.qs.y = __builtin_amdgcn_alignbyte(r2, r1, sh);
+        const uint32_t *g = reinterpret_cast<const uint32_t *>(blk + 74 + ib * 4 - sh);
+        f.sg = __builtin_amdgcn_alignbyte(g[1], g[0], sh);
+        f.qh = blk[66 + ib];
+        f.sc = blk[106 + (ib >> 1)];
+    } else {
+        const uint32_t *q = reinterpret_cast<const uint32_t *>(blk + 2 + ib * 4 - sh);
+        f.qs.x = __builtin_amdgcn_alignbyte(q[1], q[0], sh);
+        const uint32_t *g = reinterpret_cast<const uint32_t *>(blk + 34 + ib * 4 - sh);
+        f.qs.y = __builtin_amdgcn_alignbyte(g[1], g[0], sh);
+        f.sg = 0;
+        f.qh = blk[66 + ib];
+        f.sc = blk[74 + ib];
+    }
+    return f;
+}
+
+// iq_rows_q8k<TYPE, NR, false> for nb == 8 and 16-byte aligned rows.  stage: NR * kIqStageBytes bytes of LDS owned by
+// the wave, 16-byte aligned.
+template <int TYPE, int NR>
+WD_DEV void iq_rows8_coal(const uint8_t *const (&rows)[NR], const IqTables &t, const int8_t *act_qs, const float *act_d,
+                          int lane, float (&y)[NR], uint8_t *stage) {
+    constexpr int kBlk = (TYPE == 21) ? 110 : 82;
+    constexpr int kWords = 8 * kBlk / 16;
+    const int ib = lane >> 3, sb = lane & 7;
+    const bool first = sb == 0;
+    uint4 raw[NR];
+#pragma unroll
+    for (int i = 0; i < NR; ++i) raw[i] = gld_u128_aligned(rows[i] + 16 * min(lane, kWords - 1));
+    const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32);
+    const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32 + 16);
+    const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+    const float dx = act_d[sb];
+#pragma unroll
+    for (int i = 0; i < NR; ++i)
+        if (lane < kWords) reinterpret_cast<uint4 *>(stage + i * kIqStageBytes)[lane] = raw[i];
+    wave_lds_fence();
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+        const IqFields f = iq_fields_lds<TYPE>(stage + i * kIqStageBytes + sb * kBlk, ib, sb);
+        int p[8];
+        iq_chunks<TYPE>(f, ib, t, a, p);
+        const float ds = h2f(f.d) * dx;
+        const float pf = static_cast<float>(reduce_scatter_ib(p, lane));  // lane (c = ib, sb): chunk c of super-block sb
+        float v = __builtin_fmaf(ds, pf, 0.0f);
+#pragma unroll
+        for (int s = 1; s < 8; ++s) {
+            const float up = dpp_f<kDppShr1>(0.0f, v);
+            const float nxt = __builtin_fmaf(ds, pf, up);
+            v = first ? v : nxt;
+        }
+        const float r = close_lanes8_strided(v);
+        y[i] = (TYPE == 22) ? 0.125f * r : r;
+    }
+}
+
 template <int TYPE, bool PART>
 WD_DEV float iq_row_q8k(const uint8_t *row, int nb, const IqTables &t, const int8_t *act_qs, const float *act_d,
                         int lane, int32_t *partials) {
