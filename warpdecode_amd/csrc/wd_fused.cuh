@@ -587,15 +587,25 @@ WD_DEV void router_rows_wave(const float *__restrict__ w, const float *__restric
     }
     const int np = cols & ~31;
     const int half_off = (upper ? 1024 : 0) + t;
+    // x is requested first (it is small and every workgroup reads it, so it arrives early), then the row; x goes to
+    // LDS as soon as it is in, while the weights are still on their way
+    const int i0 = static_cast<int>(threadIdx.x) * 4;
+    const bool x_quad = i0 + 4 <= cols;
+    float4 xq4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (x_quad) xq4 = *reinterpret_cast<const float4 *>(x + i0);
     float wv[32];
-    if (on) {
 #pragma unroll
-        for (int u = 0; u < 32; ++u) {
-            const int c = half_off + 32 * u;
-            wv[u] = (c < np) ? wr[c] : 0.0f;
-        }
+    for (int u = 0; u < 32; ++u) {  // unconditional loads (clamped column; waves past the last row read x instead)
+        const int c = half_off + 32 * u;
+        const float v = wr[min(c, cols - 1)];
+        wv[u] = (c < np) ? v : 0.0f;
     }
-    for (int i = static_cast<int>(threadIdx.x) * 4; i < cols; i += static_cast<int>(blockDim.x) * 4) {
+    if (x_quad) {
+        *reinterpret_cast<float4 *>(xs + i0) = xq4;
+    } else {
+        for (int c = i0; c < cols; ++c) xs[c] = x[c];
+    }
+    for (int i = i0 + static_cast<int>(blockDim.x) * 4; i < cols; i += static_cast<int>(blockDim.x) * 4) {
         if (i + 4 <= cols) {
             *reinterpret_cast<float4 *>(xs + i) = *reinterpret_cast<const float4 *>(x + i);
         } else {
