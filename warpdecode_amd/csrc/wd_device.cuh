@@ -187,6 +187,15 @@ WD_DEV uint4 gld_u128(const uint8_t *p) {
     const wd_u128a v = *((const WD_GLOBAL wd_u128a *)(p));
     return make_uint4(v.x, v.y, v.z, v.w);
 }
+// A pointer that is the same in every lane of the wave, moved to scalar registers (frees two vector registers and
+// lets loads use the scalar base + vector offset form).
+template <typename T>
+WD_DEV T *uniform_ptr(T *p) {
+    const uintptr_t v = reinterpret_cast<uintptr_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+    return reinterpret_cast<T *>((static_cast<uintptr_t>(hi) << 32) | lo);
+}
 // A 32-bit value at a wave-uniform address through the scalar path (lower latency than a vector load).  Only for
 // data written before the launch: the scalar cache is not coherent with stores of the running dispatch.
 WD_DEV int sld_i32(const int32_t *p) {

@@ -587,25 +587,15 @@ WD_DEV void router_rows_wave(const float *__restrict__ w, const float *__restric
     }
     const int np = cols & ~31;
     const int half_off = (upper ? 1024 : 0) + t;
-    // x is requested first (it is small and every workgroup reads it, so it arrives early), then the row; x goes to
-    // LDS as soon as it is in, while the weights are still on their way
-    const int i0 = static_cast<int>(threadIdx.x) * 4;
-    const bool x_quad = i0 + 4 <= cols;
-    float4 xq4 = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (x_quad) xq4 = *reinterpret_cast<const float4 *>(x + i0);
     float wv[32];
+    if (on) {
 #pragma unroll
-    for (int u = 0; u < 32; ++u) {  // unconditional loads (clamped column; waves past the last row read x instead)
-        const int c = half_off + 32 * u;
-        const float v = wr[min(c, cols - 1)];
-        wv[u] = (c < np) ? v : 0.0f;
+        for (int u = 0; u < 32; ++u) {
+            const int c = half_off + 32 * u;
+            wv[u] = (c < np) ? wr[c] : 0.0f;
+        }
     }
-    if (x_quad) {
-        *reinterpret_cast<float4 *>(xs + i0) = xq4;
-    } else {
-        for (int c = i0; c < cols; ++c) xs[c] = x[c];
-    }
-    for (int i = i0 + static_cast<int>(blockDim.x) * 4; i < cols; i += static_cast<int>(blockDim.x) * 4) {
+    for (int i = static_cast<int>(threadIdx.x) * 4; i < cols; i += static_cast<int>(blockDim.x) * 4) {
         if (i + 4 <= cols) {
             *reinterpret_cast<float4 *>(xs + i) = *reinterpret_cast<const float4 *>(x + i);
         } else {
@@ -813,7 +803,7 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
         const int nb = a.H >> 5;
         const size_t rb = static_cast<size_t>(nb) * 34;
         const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
-        const uint8_t *const rows[2] = {a.sh_gate + off, a.sh_up + off};
+        const uint8_t *const rows[2] = {uniform_ptr(a.sh_gate + off), uniform_ptr(a.sh_up + off)};  // one row pair per wave
         float gu[2];
         q8_row_wave<2>(rows, nb, xq, reinterpret_cast<const uint16_t *>(xscale), tiles[wave], lane, gu, [&]() {
             lds_quantize_q8_0(a.x, a.H, xq, reinterpret_cast<uint16_t *>(xscale), threadIdx.x, 512);
@@ -861,7 +851,7 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
         const int nb = a.H >> 8;
         const size_t rb = static_cast<size_t>(nb) * (TYPE == 21 ? 110 : 82);
         const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
-        const uint8_t *const rows[2] = {gate + off, up + off};
+        const uint8_t *const rows[2] = {uniform_ptr(gate + off), uniform_ptr(up + off)};  // one row pair per wave
         if (COAL)
             iq_rows8_coal<(kIq ? TYPE : 21), 2>(rows, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
                                                 lds_ab + ((4 * a.H + 16 + 15) & ~15) + wave * 2 * kIqStageBytes);

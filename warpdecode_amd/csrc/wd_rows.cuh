@@ -313,17 +313,19 @@ WD_DEV void iq_rows8_coal(const uint8_t *const (&rows)[NR], const IqTables &t, c
     constexpr int kWords = 8 * kBlk / 16;
     const int ib = lane >> 3, sb = lane & 7;
     const bool first = sb == 0;
-    uint4 raw[NR];
+    {
+        uint4 raw[NR];
 #pragma unroll
-    for (int i = 0; i < NR; ++i) raw[i] = gld_u128_aligned(rows[i] + 16 * min(lane, kWords - 1));
+        for (int i = 0; i < NR; ++i) raw[i] = gld_u128_aligned(rows[i] + 16 * min(lane, kWords - 1));
+#pragma unroll
+        for (int i = 0; i < NR; ++i)
+            if (lane < kWords) reinterpret_cast<uint4 *>(stage + i * kIqStageBytes)[lane] = raw[i];
+    }
+    wave_lds_fence();
     const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32);
     const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32 + 16);
     const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
     const float dx = act_d[sb];
-#pragma unroll
-    for (int i = 0; i < NR; ++i)
-        if (lane < kWords) reinterpret_cast<uint4 *>(stage + i * kIqStageBytes)[lane] = raw[i];
-    wave_lds_fence();
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
         const IqFields f = iq_fields_lds<TYPE>(stage + i * kIqStageBytes + sb * kBlk, ib, sb);

@@ -89,7 +89,7 @@ __global__ __launch_bounds__(512, 6) void k_tokens_a(TokenArgs ta) {
     const int nb = a.H >> 5;
     const size_t rb = static_cast<size_t>(nb) * 34;
     const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
-    const uint8_t *const rows[2] = {a.sh_gate + off, a.sh_up + off};
+    const uint8_t *const rows[2] = {uniform_ptr(a.sh_gate + off), uniform_ptr(a.sh_up + off)};  // one row pair per wave
     float gu[2];
     q8_row_wave<2>(rows, nb, xq, xd, tiles[wave], lane, gu, [&]() {
         lds_quantize_q8_0(s.x, a.H, xq, xd, threadIdx.x, 512);
@@ -230,7 +230,8 @@ __global__ __launch_bounds__(512, 4) void k_tokens_b(TokenArgs ta) {
         for (int t = 0; t < MAXT; ++t) rank[t] = __builtin_amdgcn_readfirstlane(static_cast<int>(un.rank[u][t]));
         const int r = rg * 8 + wave;
         const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
-        const uint8_t *const rows[2] = {mat_ptr_expert<0>(a.gate_up, e) + off, mat_ptr_expert<1>(a.gate_up, e) + off};
+        const uint8_t *const rows[2] = {uniform_ptr(mat_ptr_expert<0>(a.gate_up, e) + off),
+                                        uniform_ptr(mat_ptr_expert<1>(a.gate_up, e) + off)};  // one row pair per wave
         float acc[MAXT][2];
 #pragma unroll
         for (int t = 0; t < MAXT; ++t) acc[t][0] = acc[t][1] = 0.0f;
