@@ -274,3 +274,43 @@ def test_fused_gate_up_tensor_layout(g, oracle):
     assert g.same_bits(g.host(out2), want)
     sc.close()
     capi.call("wd_expert_cache_destroy", cache)
+
+
+def test_alignment_chooses_the_fetch_path(g, oracle):
+    """The C2 layer shape (hidden 2048, ffn 512) takes the coalesced fetch paths (aligned 16-byte words regrouped through
+    LDS) when every routed and shared tensor starts on a 16-byte boundary, and the per-block loads otherwise.  The same
+    layer with its tensors moved 2 bytes into their allocations (GGUF only promises 2-byte alignment of blocks) must
+    give the same bits; token batches through both placements too."""
+    import torch
+    H, F, E, k = 2048, 512, 16, 4
+    L = synth.make_layer(H, F, E, k, synth.IQ3_S, synth.Q8_0, True, seed=SEED, layer=61, router_sigma=1.0 / np.sqrt(H))
+    xs = np.stack([synth.rms_normed(synth.rng_for(SEED, 51, t), H) for t in range(2)])
+    want = [oracle.moe_layer(L, x) for x in xs]
+    for shift in (0, 2):
+        dl = g.DeviceLayer(L)
+        keep = {}
+        for name in ("gate", "up", "down", "shared_gate", "shared_up", "shared_down"):
+            raw = np.ascontiguousarray(L[name]).reshape(-1)
+            buf = torch.zeros(raw.size + 32, dtype=torch.uint8, device="cuda")
+            buf[shift:shift + raw.size] = torch.from_numpy(raw).cuda()
+            keep[name] = buf
+            setattr(dl.desc, name, buf.data_ptr() + shift)
+        sc = g.Scratch(H, F, E, k)
+        for x, (w_out, d) in zip(xs, want):
+            dx, out = g.dev(x), g.empty(H, np.float32)
+            for flags in (0, 0x100):     # merged and split dispatches
+                capi.call("wd_moe_layer_f32", C.byref(dl.desc), g.ptr(dx), g.ptr(out), sc.h, flags, g.stream())
+                g.sync()
+                assert np.array_equal(sc.get("ids", k, np.int32), d["ids"]), (shift, flags)
+                assert g.same_bits(g.host(out), w_out), (shift, flags)
+        scs = [sc, g.Scratch(H, F, E, k)]
+        arr = (C.c_void_p * 2)(*[s.h for s in scs])
+        dx, out = g.dev(xs), g.empty((2, H), np.float32)
+        capi.call("wd_moe_layer_tokens_f32", C.byref(dl.desc), g.ptr(dx), g.ptr(out), 2, arr, 0, g.stream())
+        g.sync()
+        got = g.host(out)
+        for t in range(2):
+            assert g.same_bits(got[t], want[t][0]), (shift, t)
+        assert capi.load().wd_moe_scratch_status(sc.h) == 0
+        for s in scs:
+            s.close()
