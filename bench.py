@@ -54,6 +54,8 @@ def parse():
                          "all-Q8_0 layer (secondary workloads, own JSON lines)")
     ap.add_argument("--tokens", type=int, default=4, help="tokens mode: tokens per pass (<= 8)")
     ap.add_argument("--cache-gib", type=float, default=32.0)
+    ap.add_argument("--fill", choices=["kernel", "memcpy"], default="kernel",
+                    help="lru mode: fill misses with the copy kernel that reads pinned host memory, or with hipMemcpyAsync")
     ap.add_argument("--cache-warm-tokens", type=int, default=256,
                     help="lru mode: tokens run before the warm-up steps so that the slot pool is in steady state")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a captured HIP graph")
@@ -232,6 +234,7 @@ def bench_lru(args, torch, capi, synth):
     slot_bytes = 2 * gb + db
     cache = C.c_void_p()
     capi.call("wd_expert_cache_create", C.byref(cache), int(args.cache_gib * (1 << 30)), gb, gb, db, NL, E, 0)
+    capi.call("wd_expert_cache_set_copy_kernel", cache, 1 if args.fill == "kernel" else 0)
     for l in range(NL):
         capi.call("wd_expert_cache_register_layer", cache, l, *pinned[l])
     st_slots = int(args.cache_gib * (1 << 30)) // slot_bytes

@@ -269,6 +269,10 @@ int wd_expert_cache_get_stats(wd_expert_cache *c, wd_expert_cache_stats *out);
 /* Counterfactual caches that see the same (layer, expert) accesses as the pool and hold keys only: what would a pool
  * of `slots` have hit under LRU (policy 0) or exact LFU (policy 1)?  Add them before the first acquire.
  * reference: ShadowLru / ShadowFreq, src/expert_cache.cuh:1592-1668. */
+/* Misses are filled by one copy kernel per acquire call that reads the host tensors directly when these are pinned
+ * and 16-byte aligned (default), else - or with enabled = 0 - by hipMemcpyAsync per piece.  No counterpart in the
+ * reference (its fills are cudaMemcpyAsync per contiguous run, src/expert_cache.cuh:1166-1254). */
+int wd_expert_cache_set_copy_kernel(wd_expert_cache *c, int enabled);
 int wd_expert_cache_add_shadow(wd_expert_cache *c, int policy, size_t slots);
 /* The monitor's counters as one JSON object (hit rate, bytes copied, per-layer accesses and misses, distinct pairs,
  * reuse of the previous call's experts per layer, host time spent in acquire, shadow hit rates).  Returns the length

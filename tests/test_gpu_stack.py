@@ -72,7 +72,8 @@ def test_resident_stack(g, oracle, layers, flags, use_trace):
     sc.close()
 
 
-@pytest.mark.parametrize("slots", [NL * E, 20], ids=["all-resident", "lru-20-slots"])
+# 20 slots: fills one layer ahead; 30 slots (at least two tokens' experts): the whole token is acquired ahead, with evictions
+@pytest.mark.parametrize("slots", [NL * E, 30, 20], ids=["all-resident", "lru-30-slots", "lru-20-slots"])
 @pytest.mark.parametrize("use_trace", [False, True], ids=["router", "trace"])
 def test_cached_stack(g, oracle, layers, slots, use_trace):
     import torch

@@ -9,9 +9,13 @@
 //   * the kernels never see host pointers: every layer has a device table expert -> slot that the
 //     grouped GEMVs index with the routed ids, updated by a small kernel ordered on the caller's
 //     stream, so no pointer table is uploaded per layer;
-//   * fills are hipMemcpyAsync from pinned memory on a private copy stream: the copy stream waits
-//     for the work already queued on the caller's stream (which may still read the victim slot) and
-//     the caller's stream waits for the fills, so no host thread ever blocks.
+//   * fills run on a private copy stream: the copy stream waits for the work already queued on the caller's
+//     stream (which may still read the victim slot) and the caller's stream waits for the fills, so no host
+//     thread ever blocks.  When a layer's host tensors are pinned (the GPU can read them) and 16-byte aligned,
+//     all misses of an acquire call are filled by ONE copy kernel that reads host memory directly (three
+//     segments per miss, many workgroups per segment): a miss is three sub-megabyte pieces, and per-copy set-up
+//     of the DMA path, not the link, was what bounded the fill rate.  Otherwise (pageable memory such as a file
+//     mapping, odd alignment) the three pieces go through hipMemcpyAsync.
 #include "wd_common.h"
 
 #include <chrono>
@@ -32,6 +36,27 @@ struct SlotUpdate {
     int32_t index;  // position in the concatenated [layer][expert] table
     int32_t value;  // slot number or -1
 };
+
+// Copy kernel of the fill path: segment blockIdx.y is copied by gridDim.x workgroups in 16-byte words.
+constexpr int kMaxFillSegments = 3 * (64 / 2);  // three per miss, at most kMaxUpdates / 2 misses per call
+struct FillSegments {
+    const uint8_t *src[kMaxFillSegments];  // pinned host memory, read over the host link
+    uint8_t *dst[kMaxFillSegments];
+    uint32_t words[kMaxFillSegments];      // 16-byte words
+};
+__global__ __launch_bounds__(256) void k_fill_slots(FillSegments f) {
+    const int seg = blockIdx.y;
+    const uint4 *src = reinterpret_cast<const uint4 *>(f.src[seg]);
+    uint4 *dst = reinterpret_cast<uint4 *>(f.dst[seg]);
+    const uint32_t n = f.words[seg];
+    const uint32_t stride = gridDim.x * 256;
+    uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    for (; i + 3 * stride < n; i += 4 * stride) {  // four requests in flight per thread
+        const uint4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
+        dst[i] = a, dst[i + stride] = b, dst[i + 2 * stride] = c, dst[i + 3 * stride] = d;
+    }
+    for (; i < n; i += stride) dst[i] = src[i];
+}
 
 // One thread, in order: a batch may name the same table entry twice (evicted, then filled again).
 __global__ void k_apply_slot_updates(int32_t *table, const SlotUpdate *updates, int n) {
@@ -126,8 +151,13 @@ struct wd_expert_cache {
     uint64_t clock = 0;
     uint64_t prev_floor = 0;     // clock value before the previous acquire call
     bool fills_pending = false;  // a deferred acquire's fills have not been waited for yet
+    std::vector<hipEvent_t> ev_layer;      // token-ahead acquires: the fills of layer l are complete
+    std::vector<uint8_t> layer_pending;    // ev_layer[l] has been recorded and not yet waited for
     std::vector<const uint8_t *> h_gate, h_up, h_down;
     std::vector<size_t> s_gate, s_up, s_down;  // bytes from one expert to the next in the host tensors
+    std::vector<uint8_t> gpu_readable;          // per layer: pinned and 16-byte aligned, the copy kernel can read it
+    bool use_copy_kernel = true;
+    uint64_t kernel_fills = 0, dma_fills = 0;   // misses filled by the copy kernel / by hipMemcpyAsync
     int32_t *d_table = nullptr;  // [n_layers][n_experts]
     hipStream_t copy_stream = nullptr;
     hipEvent_t ev_retire = nullptr, ev_done = nullptr;
@@ -145,6 +175,27 @@ struct wd_expert_cache {
     uint64_t prev_ready = 0, prev_hit = 0, acquire_calls = 0;
     double acquire_ms = 0.0;
 };
+
+namespace {
+// Can the copy kernel read this layer's host tensors?  They must be pinned (known to the runtime as host memory) and
+// every expert slice must start and end on 16-byte boundaries.
+void classify_layer(wd_expert_cache *c, int layer) {
+    if (c->gpu_readable.size() < static_cast<size_t>(c->n_layers)) c->gpu_readable.assign(c->n_layers, 0);
+    bool ok = c->gate_bytes % 16 == 0 && c->up_bytes % 16 == 0 && c->down_bytes % 16 == 0 && c->slot_bytes % 16 == 0 &&
+              c->s_gate[layer] % 16 == 0 && c->s_up[layer] % 16 == 0 && c->s_down[layer] % 16 == 0;
+    const uint8_t *ptrs[3] = {c->h_gate[layer], c->h_up[layer], c->h_down[layer]};
+    for (const uint8_t *p : ptrs) {
+        if (!ok) break;
+        hipPointerAttribute_t attr{};
+        if (reinterpret_cast<uintptr_t>(p) % 16 != 0 || hipPointerGetAttributes(&attr, p) != hipSuccess ||
+            attr.type != hipMemoryTypeHost) {
+            (void)hipGetLastError();  // a pointer the runtime does not know is an error there, not here
+            ok = false;
+        }
+    }
+    c->gpu_readable[layer] = ok ? 1 : 0;
+}
+}  // namespace
 
 extern "C" {
 
@@ -218,6 +269,8 @@ int wd_expert_cache_destroy(wd_expert_cache *c) {
     if (c->h_updates) (void)hipHostFree(c->h_updates);
     if (c->ev_retire) (void)hipEventDestroy(c->ev_retire);
     if (c->ev_done) (void)hipEventDestroy(c->ev_done);
+    for (hipEvent_t ev : c->ev_layer)
+        if (ev) (void)hipEventDestroy(ev);
     for (int i = 0; i < kUpdateRing; ++i)
         if (c->ring_free[i]) (void)hipEventDestroy(c->ring_free[i]);
     if (c->copy_stream) (void)hipStreamDestroy(c->copy_stream);
@@ -232,6 +285,7 @@ int wd_expert_cache_register_layer(wd_expert_cache *c, int layer, const uint8_t 
     WD_REQUIRE(h_gate && h_up && h_down, "expert cache: null host tensor");
     c->h_gate[layer] = h_gate, c->h_up[layer] = h_up, c->h_down[layer] = h_down;
     c->s_gate[layer] = c->gate_bytes, c->s_up[layer] = c->up_bytes, c->s_down[layer] = c->down_bytes;
+    classify_layer(c, layer);
     return WD_OK;
 }
 
@@ -242,6 +296,13 @@ int wd_expert_cache_register_layer_strided(wd_expert_cache *c, int layer, const 
     WD_REQUIRE(gate_stride >= c->gate_bytes && up_stride >= c->up_bytes && down_stride >= c->down_bytes,
                "expert cache: an expert stride is smaller than the expert");
     c->s_gate[layer] = gate_stride, c->s_up[layer] = up_stride, c->s_down[layer] = down_stride;
+    classify_layer(c, layer);
+    return WD_OK;
+}
+
+int wd_expert_cache_set_copy_kernel(wd_expert_cache *c, int enabled) {
+    WD_REQUIRE(c != nullptr, "expert cache is not initialized");
+    c->use_copy_kernel = enabled != 0;
     return WD_OK;
 }
 
@@ -252,8 +313,34 @@ namespace {
 // `defer_wait`: the fills are queued behind the work already on `stream`, but `stream` is not made to wait
 // for them; the caller does that later with wait_fills(), after it has queued work that does not depend on
 // the new experts (the previous layer).  A victim must then be older than the previous acquire call too.
+// `ahead` (token-ahead acquires, see acquire_token_ahead): victims must be older than ahead->floor, the fills'
+// completion is recorded in the layer's own event, and the wait for the slots' last readers is done once per token.
+struct AheadState {
+    uint64_t floor;
+    bool retired;
+    std::vector<SlotUpdate> updates;
+};
+
+// Uploads a batch of slot-table changes and applies them in order on the caller's stream.
+int flush_slot_updates(wd_expert_cache *c, const SlotUpdate *updates, int n_updates, hipStream_t st) {
+    for (int done = 0; done < n_updates; done += kMaxUpdates) {
+        const int n = n_updates - done < kMaxUpdates ? n_updates - done : kMaxUpdates;
+        const int r = c->ring_next;
+        c->ring_next = (r + 1) % kUpdateRing;
+        if (c->ring_used[r]) WD_HIP(hipEventSynchronize(c->ring_free[r]));  // the entry's last use has been consumed
+        SlotUpdate *h = c->h_updates + static_cast<size_t>(r) * kMaxUpdates;
+        SlotUpdate *d = c->d_updates + static_cast<size_t>(r) * kMaxUpdates;
+        for (int i = 0; i < n; ++i) h[i] = updates[done + i];
+        WD_HIP(hipMemcpyAsync(d, h, sizeof(SlotUpdate) * n, hipMemcpyHostToDevice, st));
+        k_apply_slot_updates<<<dim3(1), dim3(64), 0, st>>>(c->d_table, d, n);
+        WD_LAUNCH_CHECK();
+        WD_HIP(hipEventRecord(c->ring_free[r], st));  // both copies of ring entry r are free after this point
+        c->ring_used[r] = true;
+    }
+    return WD_OK;
+}
 int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uint8_t *hit_out, void *stream,
-                 bool defer_wait) {
+                 bool defer_wait, AheadState *ahead = nullptr) {
     WD_REQUIRE(c != nullptr && c->pool != nullptr, "expert cache is not initialized");
     WD_REQUIRE(layer >= 0 && layer < c->n_layers, "expert cache: layer %d out of range", layer);
     WD_REQUIRE(h_ids != nullptr && k > 0 && 2 * k <= kMaxUpdates, "expert cache: invalid id list (k=%d)", k);
@@ -291,11 +378,15 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
         prev.assign(h_ids, h_ids + k);
     }
     const uint64_t epoch_floor = c->clock;  // slots touched by this call carry last_use > epoch_floor
-    const uint64_t victim_floor = defer_wait ? c->prev_floor : epoch_floor;
+    const uint64_t victim_floor = ahead ? ahead->floor : (defer_wait ? c->prev_floor : epoch_floor);
     c->prev_floor = epoch_floor;
     SlotUpdate updates[kMaxUpdates];
     int n_updates = 0;
     bool waited = false;
+    const bool by_kernel = c->use_copy_kernel && static_cast<size_t>(layer) < c->gpu_readable.size() && c->gpu_readable[layer];
+    FillSegments fills;
+    int n_fill = 0;
+    uint32_t max_words = 0;
 
     for (int j = 0; j < k; ++j) {
         const int e = h_ids[j];
@@ -342,40 +433,85 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
 
         if (!waited) {
             // kernels already queued on the caller's stream may still read the victim slot
-            WD_HIP(hipEventRecord(c->ev_retire, st));
-            WD_HIP(hipStreamWaitEvent(c->copy_stream, c->ev_retire, 0));
+            if (!ahead || !ahead->retired) {
+                WD_HIP(hipEventRecord(c->ev_retire, st));
+                WD_HIP(hipStreamWaitEvent(c->copy_stream, c->ev_retire, 0));
+                if (ahead) ahead->retired = true;
+            }
             waited = true;
         }
         uint8_t *dst = c->pool + slot * c->slot_bytes;
-        WD_HIP(hipMemcpyAsync(dst, c->h_gate[layer] + static_cast<size_t>(e) * c->s_gate[layer], c->gate_bytes,
-                              hipMemcpyHostToDevice, c->copy_stream));
-        WD_HIP(hipMemcpyAsync(dst + c->gate_bytes, c->h_up[layer] + static_cast<size_t>(e) * c->s_up[layer], c->up_bytes,
-                              hipMemcpyHostToDevice, c->copy_stream));
-        WD_HIP(hipMemcpyAsync(dst + c->gate_bytes + c->up_bytes, c->h_down[layer] + static_cast<size_t>(e) * c->s_down[layer],
-                              c->down_bytes, hipMemcpyHostToDevice, c->copy_stream));
+        const uint8_t *src3[3] = {c->h_gate[layer] + static_cast<size_t>(e) * c->s_gate[layer],
+                                  c->h_up[layer] + static_cast<size_t>(e) * c->s_up[layer],
+                                  c->h_down[layer] + static_cast<size_t>(e) * c->s_down[layer]};
+        uint8_t *dst3[3] = {dst, dst + c->gate_bytes, dst + c->gate_bytes + c->up_bytes};
+        const size_t len3[3] = {c->gate_bytes, c->up_bytes, c->down_bytes};
+        if (by_kernel) {
+            for (int q = 0; q < 3; ++q) {
+                fills.src[n_fill] = src3[q], fills.dst[n_fill] = dst3[q];
+                fills.words[n_fill] = static_cast<uint32_t>(len3[q] / 16);
+                max_words = fills.words[n_fill] > max_words ? fills.words[n_fill] : max_words;
+                ++n_fill;
+            }
+            ++c->kernel_fills;
+        } else {
+            for (int q = 0; q < 3; ++q)
+                WD_HIP(hipMemcpyAsync(dst3[q], src3[q], len3[q], hipMemcpyHostToDevice, c->copy_stream));
+            ++c->dma_fills;
+        }
         c->stats.bytes_copied += c->slot_bytes;
     }
     c->stats.resident = c->index.size();
+    if (n_fill > 0) {
+        // enough workgroups per segment to keep the host link busy, few enough to leave the decode its compute units
+        const uint32_t per_seg = (max_words + 256 * 16 - 1) / (256 * 16);
+        k_fill_slots<<<dim3(per_seg < 32 ? (per_seg ? per_seg : 1) : 32, n_fill), dim3(256), 0, c->copy_stream>>>(fills);
+        WD_LAUNCH_CHECK();
+    }
 
     if (n_updates > 0) {
-        const int r = c->ring_next;
-        c->ring_next = (r + 1) % kUpdateRing;
-        if (c->ring_used[r]) WD_HIP(hipEventSynchronize(c->ring_free[r]));  // the entry's last use has been consumed
-        SlotUpdate *h = c->h_updates + static_cast<size_t>(r) * kMaxUpdates;
-        SlotUpdate *d = c->d_updates + static_cast<size_t>(r) * kMaxUpdates;
-        for (int i = 0; i < n_updates; ++i) h[i] = updates[i];
-        WD_HIP(hipMemcpyAsync(d, h, sizeof(SlotUpdate) * n_updates, hipMemcpyHostToDevice, st));
-        k_apply_slot_updates<<<dim3(1), dim3(64), 0, st>>>(c->d_table, d, n_updates);
-        WD_LAUNCH_CHECK();
-        WD_HIP(hipEventRecord(c->ring_free[r], st));  // both copies of ring entry r are free after this point
-        c->ring_used[r] = true;
+        if (ahead) {  // applied once for the whole token, before its first layer
+            ahead->updates.insert(ahead->updates.end(), updates, updates + n_updates);
+        } else if (const int rc = flush_slot_updates(c, updates, n_updates, st)) {
+            return rc;
+        }
     }
     if (waited) {
-        WD_HIP(hipEventRecord(c->ev_done, c->copy_stream));
-        if (defer_wait)
-            c->fills_pending = true;
-        else
-            WD_HIP(hipStreamWaitEvent(st, c->ev_done, 0));
+        if (ahead) {
+            WD_HIP(hipEventRecord(c->ev_layer[layer], c->copy_stream));
+            c->layer_pending[layer] = 1;
+        } else {
+            WD_HIP(hipEventRecord(c->ev_done, c->copy_stream));
+            if (defer_wait)
+                c->fills_pending = true;
+            else
+                WD_HIP(hipStreamWaitEvent(st, c->ev_done, 0));
+        }
+    }
+    return WD_OK;
+}
+
+// Acquires the experts of every layer of one token before any of the token's layers is launched, so that the host
+// link streams the token's misses back to back while the layers compute; wait_layer_fills(l) then makes the stream
+// wait for layer l's fills only.  Needs a pool that holds a whole token: the slots a token touches are not evicted
+// by its own later layers (victims must be older than the token).  h_ids: [n_layers][k].
+int acquire_token_ahead(wd_expert_cache *c, int n_layers, const int32_t *h_ids, int k, void *stream) {
+    if (c->ev_layer.size() < static_cast<size_t>(c->n_layers)) {
+        c->ev_layer.resize(c->n_layers, nullptr);
+        c->layer_pending.assign(c->n_layers, 0);
+        for (hipEvent_t &ev : c->ev_layer)
+            if (!ev) WD_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+    }
+    AheadState ahead{c->clock, false, {}};
+    for (int l = 0; l < n_layers; ++l)
+        if (const int rc = acquire_impl(c, l, h_ids + static_cast<size_t>(l) * k, k, nullptr, stream, true, &ahead)) return rc;
+    return flush_slot_updates(c, ahead.updates.data(), static_cast<int>(ahead.updates.size()), as_stream(stream));
+}
+
+int wait_layer_fills(wd_expert_cache *c, int layer, hipStream_t st) {
+    if (static_cast<size_t>(layer) < c->layer_pending.size() && c->layer_pending[layer]) {
+        WD_HIP(hipStreamWaitEvent(st, c->ev_layer[layer], 0));
+        c->layer_pending[layer] = 0;
     }
     return WD_OK;
 }
@@ -448,6 +584,7 @@ size_t wd_expert_cache_dump_json(wd_expert_cache *c, char *buf, size_t cap) {
     s += ",\"gib_copied\":" + fixed(st.bytes_copied / (1024.0 * 1024.0 * 1024.0), 3);
     s += ",\"resident\":" + std::to_string(c->index.size()) + ",\"distinct_pairs\":" + std::to_string(c->distinct.size());
     s += ",\"acquire_calls\":" + std::to_string(c->acquire_calls) + ",\"acquire_ms\":" + fixed(c->acquire_ms, 1);
+    s += ",\"fills_by_copy_kernel\":" + std::to_string(c->kernel_fills) + ",\"fills_by_memcpy\":" + std::to_string(c->dma_fills);
     s += ",\"prev_token_ready\":" + std::to_string(c->prev_ready);
     s += ",\"prev_token_reuse\":" + fixed(c->prev_ready ? static_cast<double>(c->prev_hit) / c->prev_ready : 0.0, 4);
     s += ",\"layer_access\":" + arr(c->layer_access) + ",\"layer_misses\":" + arr(c->layer_misses);

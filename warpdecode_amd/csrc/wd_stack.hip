@@ -2,8 +2,10 @@
 // not all fit in HBM (or are kept in a bounded pool on purpose).  The cache's device slot tables stand in for
 // the reference's per-layer pointer-table upload (src/qwen38_moe.cuh:3288-3303).
 //
-// With a routing trace known to the host, the fills of layer l+1 are queued before layer l is launched and
-// waited for after it, so the host link works while the previous layer computes.  Without one, every layer
+// With a routing trace known to the host and a pool that holds at least two tokens' experts, the experts of all
+// layers are acquired before the first layer is launched and every layer waits for its own fills only: the host
+// link streams the token's misses back to back under the layers' compute.  With a smaller pool the fills of layer
+// l+1 are queued before layer l is launched and waited for after it.  Without one, every layer
 // does what the reference does (src/qwen38_moe.cuh:2323-2380): router and selection, ids to pinned host
 // memory, stream synchronisation, acquire, expert dispatches.
 using namespace wd;
@@ -32,7 +34,21 @@ extern "C" int wd_moe_stack_cached_f32(const wd_moe_layer *layers, int n_layers,
     const int k = layers[0].top_k;
     const size_t part_slots = cache->parts[0].end - cache->parts[0].begin;
     const bool ahead = h_ids_trace != nullptr && part_slots >= static_cast<size_t>(4 * k);
+    const bool token_ahead = h_ids_trace != nullptr && !cache->partitioned &&
+                             part_slots >= 2 * static_cast<size_t>(n_layers) * k;
 
+    if (token_ahead) {
+        if (cache->fills_pending)
+            if (const int rc = wait_fills(cache, st)) return rc;
+        if (const int rc = acquire_token_ahead(cache, n_layers, h_ids_trace, k, stream)) return rc;
+        for (int l = 0; l < n_layers; ++l) {
+            const wd_moe_layer L = bind(l);
+            if (const int rc = wait_layer_fills(cache, l, st)) return rc;
+            if (const int rc = layer_fused(&L, d_x, d_layer_out, s, flags, d_ids_trace + static_cast<size_t>(l) * k, d_x, residual_scale, st))
+                return rc;
+        }
+        return WD_OK;
+    }
     if (h_ids_trace) {
         if (const int rc = wd_expert_cache_acquire(cache, 0, h_ids_trace, k, nullptr, stream)) return rc;
         for (int l = 0; l < n_layers; ++l) {
