@@ -273,6 +273,12 @@ int wd_expert_cache_get_stats(wd_expert_cache *c, wd_expert_cache_stats *out);
  * and 16-byte aligned (default), else - or with enabled = 0 - by hipMemcpyAsync per piece.  No counterpart in the
  * reference (its fills are cudaMemcpyAsync per contiguous run, src/expert_cache.cuh:1166-1254). */
 int wd_expert_cache_set_copy_kernel(wd_expert_cache *c, int enabled);
+/* File-backed fills: a read-only mapping [map_base, map_base + map_bytes) of the file behind `fd` (the cache keeps its
+ * own duplicate of the descriptor).  Layers whose registered host tensors lie inside the mapping and are not pinned are
+ * then filled by pread() of the expert's slices into a pinned ring (`threads` readers share every expert) and one DMA per
+ * miss, instead of a pageable copy from the mapping.  reference: ExpertFileMap, ExpertPreadPool and the pinned ring of
+ * ExpertStagePath (src/expert_cache.cuh:204-508, :1166-1254); there the file is found through /proc/self/maps. */
+int wd_expert_cache_attach_file(wd_expert_cache *c, const uint8_t *map_base, size_t map_bytes, int fd, int threads);
 int wd_expert_cache_add_shadow(wd_expert_cache *c, int policy, size_t slots);
 /* The monitor's counters as one JSON object (hit rate, bytes copied, per-layer accesses and misses, distinct pairs,
  * reuse of the previous call's experts per layer, host time spent in acquire, shadow hit rates).  Returns the length
@@ -310,6 +316,9 @@ int wd_gguf_open(wd_gguf **out, const char *path);
 int wd_gguf_close(wd_gguf *g);
 uint32_t wd_gguf_version(const wd_gguf *g);
 size_t wd_gguf_data_offset(const wd_gguf *g);              /* file offset of the data section (for pread users) */
+const uint8_t *wd_gguf_map_base(const wd_gguf *g);         /* the mapping of the whole file, its size, its descriptor */
+size_t wd_gguf_map_bytes(const wd_gguf *g);
+int wd_gguf_fd(const wd_gguf *g);
 long long wd_gguf_tensor_count(const wd_gguf *g);
 long long wd_gguf_find(const wd_gguf *g, const char *name); /* index or -1 */
 int wd_gguf_tensor(const wd_gguf *g, long long index, wd_gguf_tensor_info *out);

@@ -102,8 +102,12 @@ def test_resident_stack_from_file(g, oracle, layers, tmp_path, fused):
     sc.close()
 
 
+@pytest.mark.parametrize("attach", ["no", "before", "after"], ids=["pageable", "pread-attached-first", "pread-attached-late"])
 @pytest.mark.parametrize("fused", [False, True], ids=["separate", "gate_up"])
-def test_cached_stack_streams_experts_from_the_mapping(g, oracle, layers, tmp_path, fused):
+def test_cached_stack_streams_experts_from_the_mapping(g, oracle, layers, tmp_path, fused, attach):
+    """attach = no: the mapping is a pageable host source (hipMemcpyAsync per piece); otherwise the file is attached to
+    the cache and misses are read with pread() into the pinned ring (three reader threads), one DMA per miss."""
+    import json
     gb = F * synth.row_bytes(synth.IQ3_S, H)
     db = H * synth.row_bytes(synth.Q8_0, F)
     slots = 20
@@ -111,6 +115,8 @@ def test_cached_stack_streams_experts_from_the_mapping(g, oracle, layers, tmp_pa
         Ls = [_layer_from_file(gf, l) for l in range(NL)]
         cache = C.c_void_p()
         capi.call("wd_expert_cache_create", C.byref(cache), slots * (2 * gb + db), gb, gb, db, NL, E, 0)
+        if attach == "before":
+            capi.call("wd_expert_cache_attach_file", cache, C.c_void_p(gf.map_base), gf.map_bytes, gf.fd, 3)
         for l, L in enumerate(Ls):
             ptr = lambda a: C.c_void_p(a.ctypes.data)
             if fused:
@@ -118,6 +124,8 @@ def test_cached_stack_streams_experts_from_the_mapping(g, oracle, layers, tmp_pa
                           L["gate_up_stride"], L["gate_up_stride"], db)
             else:
                 capi.call("wd_expert_cache_register_layer", cache, l, ptr(L["gate"]), ptr(L["up"]), ptr(L["down"]))
+        if attach == "after":
+            capi.call("wd_expert_cache_attach_file", cache, C.c_void_p(gf.map_base), gf.map_bytes, gf.fd, 3)
         dls, arr = _descs(g, [dict(L, gate=L["gate"][:1], up=L["up"][:1], down=L["down"][:1]) for L in Ls])
         for i in range(NL):                  # routed tensors come from the cache only
             arr[i].gate = arr[i].up = arr[i].down = None
@@ -134,5 +142,12 @@ def test_cached_stack_streams_experts_from_the_mapping(g, oracle, layers, tmp_pa
         st = capi.CacheStats()
         capi.call("wd_expert_cache_get_stats", cache, C.byref(st))
         assert st.accesses == 4 * NL * K and st.misses > 0 and st.bytes_copied == st.misses * (2 * gb + db)
+        buf = C.create_string_buffer(1 << 16)
+        capi.load().wd_expert_cache_dump_json(cache, buf, len(buf))
+        mon = json.loads(buf.value.decode())
+        if attach == "no":
+            assert mon["fills_by_memcpy"] == st.misses and mon["fills_by_pread"] == 0
+        else:
+            assert mon["fills_by_pread"] == st.misses and mon["fills_by_memcpy"] == 0 and mon["fills_by_copy_kernel"] == 0
         sc.close()
         capi.call("wd_expert_cache_destroy", cache)

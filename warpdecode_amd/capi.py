@@ -101,11 +101,15 @@ _OPTIONAL = {
     "wd_expert_cache_slot_of": (C.c_longlong, [vp, i32, i32]),
     "wd_expert_cache_add_shadow": (i32, [vp, i32, sz]),
     "wd_expert_cache_set_copy_kernel": (i32, [vp, i32]),
+    "wd_expert_cache_attach_file": (i32, [vp, vp, sz, i32, i32]),
     "wd_expert_cache_dump_json": (sz, [vp, C.c_char_p, sz]),
     "wd_gguf_open": (i32, [C.POINTER(vp), C.c_char_p]),
     "wd_gguf_close": (i32, [vp]),
     "wd_gguf_version": (C.c_uint32, [vp]),
     "wd_gguf_data_offset": (sz, [vp]),
+    "wd_gguf_map_base": (vp, [vp]),
+    "wd_gguf_map_bytes": (sz, [vp]),
+    "wd_gguf_fd": (i32, [vp]),
     "wd_gguf_tensor_count": (C.c_longlong, [vp]),
     "wd_gguf_find": (C.c_longlong, [vp, C.c_char_p]),
     "wd_gguf_tensor": (i32, [vp, C.c_longlong, C.POINTER(GgufTensorInfo)]),

@@ -15,15 +15,27 @@
 //     all misses of an acquire call are filled by ONE copy kernel that reads host memory directly (three
 //     segments per miss, many workgroups per segment): a miss is three sub-megabyte pieces, and per-copy set-up
 //     of the DMA path, not the link, was what bounded the fill rate.  Otherwise (pageable memory such as a file
-//     mapping, odd alignment) the three pieces go through hipMemcpyAsync.
+//     mapping, odd alignment) the three pieces go through hipMemcpyAsync;
+//   * a file mapping attached to the cache (wd_expert_cache_attach_file) turns fills from pointers inside it into
+//     pread() of the expert's three slices into one entry of a pinned ring, shared out over a few worker threads
+//     (a single core does not reach the page cache's bandwidth), followed by ONE DMA of the whole slot from the
+//     ring entry; an entry is reused when the event recorded behind its DMA has completed.  Same role as the
+//     reference's ExpertFileMap / ExpertPreadPool / pinned ring (src/expert_cache.cuh:204-508, :858-1583), without
+//     the /proc/self/maps lookup: the file is named by the caller.
 #include "wd_common.h"
 
+#include <unistd.h>
+
+#include <atomic>
 #include <chrono>
+#include <condition_variable>
 #include <cstdio>
 #include <cstring>
 #include <list>
+#include <mutex>
 #include <new>
 #include <string>
+#include <thread>
 #include <unordered_map>
 #include <unordered_set>
 #include <vector>
@@ -140,6 +152,99 @@ constexpr int kMaxUpdates = 64;  // 2 per missed expert, k <= 16... one acquire 
 
 }  // namespace
 
+namespace {
+
+// Fork-join pool for pread(): the caller publishes a list of (fd, offset, length, destination) pieces, takes its
+// share and returns when every piece has landed.  threads == 1 keeps everything inline.
+struct PreadPiece {
+    int fd;
+    uint64_t off;
+    size_t len;
+    uint8_t *dst;
+};
+class PreadPool {
+public:
+    explicit PreadPool(int threads) {
+        for (int i = 1; i < threads; ++i) workers_.emplace_back([this] { loop(); });
+    }
+    ~PreadPool() {
+        {
+            std::lock_guard<std::mutex> g(m_);
+            stop_ = true;
+        }
+        cv_.notify_all();
+        for (std::thread &t : workers_) t.join();
+    }
+    // false when a read came up short or failed
+    bool run(const PreadPiece *pieces, int n) {
+        {
+            std::lock_guard<std::mutex> g(m_);
+            pieces_ = pieces, n_ = n, next_ = 0, pending_ = n, failed_ = false;
+            ++generation_;
+        }
+        cv_.notify_all();
+        work();
+        std::unique_lock<std::mutex> g(m_);
+        done_.wait(g, [this] { return pending_ == 0; });
+        pieces_ = nullptr, n_ = 0;
+        return !failed_;
+    }
+
+private:
+    static bool read_all(const PreadPiece &p) {
+        size_t got = 0;
+        while (got < p.len) {
+            const ssize_t r = ::pread(p.fd, p.dst + got, p.len - got, static_cast<off_t>(p.off + got));
+            if (r <= 0) return false;
+            got += static_cast<size_t>(r);
+        }
+        return true;
+    }
+    void work() {
+        for (;;) {
+            PreadPiece p;
+            {
+                std::lock_guard<std::mutex> g(m_);
+                if (next_ >= n_) return;
+                p = pieces_[next_++];
+            }
+            const bool ok = read_all(p);
+            std::lock_guard<std::mutex> g(m_);
+            if (!ok) failed_ = true;
+            if (--pending_ == 0) done_.notify_all();
+        }
+    }
+    void loop() {
+        uint64_t seen = 0;
+        for (;;) {
+            {
+                std::unique_lock<std::mutex> g(m_);
+                cv_.wait(g, [&] { return stop_ || generation_ != seen; });
+                if (stop_) return;
+                seen = generation_;
+            }
+            work();
+        }
+    }
+    std::vector<std::thread> workers_;
+    std::mutex m_;
+    std::condition_variable cv_, done_;
+    const PreadPiece *pieces_ = nullptr;
+    int n_ = 0, next_ = 0, pending_ = 0;
+    uint64_t generation_ = 0;
+    bool stop_ = false, failed_ = false;
+};
+
+struct FileSource {
+    const uint8_t *base = nullptr;  // start of the caller's read-only mapping of the file
+    size_t size = 0;
+    int fd = -1;                    // our own descriptor of the same file
+};
+
+constexpr int kStageRing = 16;  // pinned ring entries of one slot each
+
+}  // namespace
+
 struct wd_expert_cache {
     uint8_t *pool = nullptr;
     size_t n_slots = 0, slot_bytes = 0, gate_bytes = 0, up_bytes = 0, down_bytes = 0;
@@ -158,6 +263,15 @@ struct wd_expert_cache {
     std::vector<uint8_t> gpu_readable;          // per layer: pinned and 16-byte aligned, the copy kernel can read it
     bool use_copy_kernel = true;
     uint64_t kernel_fills = 0, dma_fills = 0;   // misses filled by the copy kernel / by hipMemcpyAsync
+    std::vector<FileSource> files;              // attached mappings: fills from pointers inside them go through pread
+    std::vector<int8_t> layer_file;             // per layer: index into files, or -1
+    uint8_t *stage = nullptr;                   // pinned ring [kStageRing][slot_bytes]
+    hipEvent_t stage_done[kStageRing] = {};
+    bool stage_used[kStageRing] = {};
+    int stage_next = 0;
+    PreadPool *pread_pool = nullptr;
+    uint64_t pread_fills = 0;
+    double pread_ms = 0.0;
     int32_t *d_table = nullptr;  // [n_layers][n_experts]
     hipStream_t copy_stream = nullptr;
     hipEvent_t ev_retire = nullptr, ev_done = nullptr;
@@ -194,6 +308,20 @@ void classify_layer(wd_expert_cache *c, int layer) {
         }
     }
     c->gpu_readable[layer] = ok ? 1 : 0;
+    // all three tensors inside one attached mapping: misses are read from the file
+    if (c->layer_file.size() < static_cast<size_t>(c->n_layers)) c->layer_file.assign(c->n_layers, -1);
+    c->layer_file[layer] = -1;
+    const size_t span[3] = {c->s_gate[layer] * (c->n_experts - 1) + c->gate_bytes, c->s_up[layer] * (c->n_experts - 1) + c->up_bytes,
+                            c->s_down[layer] * (c->n_experts - 1) + c->down_bytes};
+    for (size_t f = 0; f < c->files.size() && !ok; ++f) {
+        bool inside = true;
+        for (int q = 0; q < 3; ++q)
+            inside = inside && ptrs[q] >= c->files[f].base && ptrs[q] + span[q] <= c->files[f].base + c->files[f].size;
+        if (inside) {
+            c->layer_file[layer] = static_cast<int8_t>(f);
+            break;
+        }
+    }
 }
 }  // namespace
 
@@ -274,7 +402,38 @@ int wd_expert_cache_destroy(wd_expert_cache *c) {
     for (int i = 0; i < kUpdateRing; ++i)
         if (c->ring_free[i]) (void)hipEventDestroy(c->ring_free[i]);
     if (c->copy_stream) (void)hipStreamDestroy(c->copy_stream);
+    delete c->pread_pool;
+    if (c->stage) (void)hipHostFree(c->stage);
+    for (int i = 0; i < kStageRing; ++i)
+        if (c->stage_done[i]) (void)hipEventDestroy(c->stage_done[i]);
+    for (FileSource &f : c->files)
+        if (f.fd >= 0) ::close(f.fd);
     delete c;
+    return WD_OK;
+}
+
+int wd_expert_cache_attach_file(wd_expert_cache *c, const uint8_t *map_base, size_t map_bytes, int fd, int threads) {
+    WD_REQUIRE(c != nullptr, "expert cache is not initialized");
+    WD_REQUIRE(map_base != nullptr && map_bytes > 0 && fd >= 0, "expert cache: invalid file mapping");
+    WD_REQUIRE(threads >= 1 && threads <= 64, "expert cache: 1..64 pread threads (got %d)", threads);
+    WD_REQUIRE(c->files.size() < 100, "expert cache: too many attached files");
+    const int own = ::dup(fd);
+    WD_REQUIRE(own >= 0, "expert cache: cannot duplicate the file descriptor");
+    if (!c->stage) {
+        hipError_t e = hipHostMalloc(reinterpret_cast<void **>(&c->stage), static_cast<size_t>(kStageRing) * c->slot_bytes,
+                                     hipHostMallocDefault);
+        if (e != hipSuccess) {
+            ::close(own);
+            return fail(WD_ERR_HIP, "expert cache: pinned staging ring failed: %s", hipGetErrorString(e));
+        }
+        for (int i = 0; i < kStageRing; ++i) WD_HIP(hipEventCreateWithFlags(&c->stage_done[i], hipEventDisableTiming));
+    }
+    if (!c->pread_pool) c->pread_pool = new PreadPool(threads);
+    FileSource f;
+    f.base = map_base, f.size = map_bytes, f.fd = own;
+    c->files.push_back(f);
+    for (int l = 0; l < c->n_layers; ++l)  // layers registered before the file was attached
+        if (c->h_gate[l]) classify_layer(c, l);
     return WD_OK;
 }
 
@@ -384,6 +543,8 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
     int n_updates = 0;
     bool waited = false;
     const bool by_kernel = c->use_copy_kernel && static_cast<size_t>(layer) < c->gpu_readable.size() && c->gpu_readable[layer];
+    const bool by_file = !by_kernel && static_cast<size_t>(layer) < c->layer_file.size() && c->layer_file[layer] >= 0 &&
+                         !(static_cast<size_t>(layer) < c->gpu_readable.size() && c->gpu_readable[layer]);
     FillSegments fills;
     int n_fill = 0;
     uint32_t max_words = 0;
@@ -446,7 +607,34 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
                                   c->h_down[layer] + static_cast<size_t>(e) * c->s_down[layer]};
         uint8_t *dst3[3] = {dst, dst + c->gate_bytes, dst + c->gate_bytes + c->up_bytes};
         const size_t len3[3] = {c->gate_bytes, c->up_bytes, c->down_bytes};
-        if (by_kernel) {
+        if (by_file) {
+            // the three slices land in one ring entry in slot order, then the slot is filled with one DMA
+            const FileSource &fs = c->files[c->layer_file[layer]];
+            const int r = c->stage_next;
+            c->stage_next = (r + 1) % kStageRing;
+            if (c->stage_used[r]) WD_HIP(hipEventSynchronize(c->stage_done[r]));  // its last DMA has read it
+            uint8_t *entry = c->stage + static_cast<size_t>(r) * c->slot_bytes;
+            const auto t0 = std::chrono::steady_clock::now();
+            PreadPiece pieces[3 * 8];
+            int n_pieces = 0;
+            size_t at = 0;
+            for (int q = 0; q < 3; ++q) {  // pieces of about 256 KiB so that the workers share one expert
+                const uint64_t file_off = static_cast<uint64_t>(src3[q] - fs.base);
+                const size_t parts = len3[q] >= (512u << 10) ? 4 : (len3[q] >= (256u << 10) ? 2 : 1);
+                for (size_t pi = 0; pi < parts; ++pi) {
+                    const size_t lo = len3[q] * pi / parts, hi = len3[q] * (pi + 1) / parts;
+                    pieces[n_pieces++] = {fs.fd, file_off + lo, hi - lo, entry + at + lo};
+                }
+                at += len3[q];
+            }
+            if (!c->pread_pool->run(pieces, n_pieces))
+                return fail(WD_ERR_STATE, "expert cache: pread of layer %d expert %d failed or came up short", layer, e);
+            c->pread_ms += std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+            WD_HIP(hipMemcpyAsync(dst, entry, c->slot_bytes, hipMemcpyHostToDevice, c->copy_stream));
+            WD_HIP(hipEventRecord(c->stage_done[r], c->copy_stream));
+            c->stage_used[r] = true;
+            ++c->pread_fills;
+        } else if (by_kernel) {
             for (int q = 0; q < 3; ++q) {
                 fills.src[n_fill] = src3[q], fills.dst[n_fill] = dst3[q];
                 fills.words[n_fill] = static_cast<uint32_t>(len3[q] / 16);
@@ -585,6 +773,7 @@ size_t wd_expert_cache_dump_json(wd_expert_cache *c, char *buf, size_t cap) {
     s += ",\"resident\":" + std::to_string(c->index.size()) + ",\"distinct_pairs\":" + std::to_string(c->distinct.size());
     s += ",\"acquire_calls\":" + std::to_string(c->acquire_calls) + ",\"acquire_ms\":" + fixed(c->acquire_ms, 1);
     s += ",\"fills_by_copy_kernel\":" + std::to_string(c->kernel_fills) + ",\"fills_by_memcpy\":" + std::to_string(c->dma_fills);
+    s += ",\"fills_by_pread\":" + std::to_string(c->pread_fills) + ",\"pread_ms\":" + fixed(c->pread_ms, 1);
     s += ",\"prev_token_ready\":" + std::to_string(c->prev_ready);
     s += ",\"prev_token_reuse\":" + fixed(c->prev_ready ? static_cast<double>(c->prev_hit) / c->prev_ready : 0.0, 4);
     s += ",\"layer_access\":" + arr(c->layer_access) + ",\"layer_misses\":" + arr(c->layer_misses);

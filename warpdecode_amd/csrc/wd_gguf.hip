@@ -221,6 +221,9 @@ int wd_gguf_open(wd_gguf **out, const char *path) {
 
 uint32_t wd_gguf_version(const wd_gguf *g) { return g ? g->version : 0; }
 size_t wd_gguf_data_offset(const wd_gguf *g) { return g ? g->data_offset : 0; }
+const uint8_t *wd_gguf_map_base(const wd_gguf *g) { return g ? g->map : nullptr; }
+size_t wd_gguf_map_bytes(const wd_gguf *g) { return g ? g->size : 0; }
+int wd_gguf_fd(const wd_gguf *g) { return g ? g->fd : -1; }
 long long wd_gguf_tensor_count(const wd_gguf *g) { return g ? static_cast<long long>(g->tensors.size()) : 0; }
 
 long long wd_gguf_find(const wd_gguf *g, const char *name) {

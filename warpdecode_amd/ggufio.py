@@ -93,6 +93,7 @@ class GgufFile:
         lib = capi.load()
         self.version = lib.wd_gguf_version(self.h)
         self.data_offset = lib.wd_gguf_data_offset(self.h)
+        self.map_base, self.map_bytes, self.fd = lib.wd_gguf_map_base(self.h), lib.wd_gguf_map_bytes(self.h), lib.wd_gguf_fd(self.h)
         self.tensors = {}
         for i in range(lib.wd_gguf_tensor_count(self.h)):
             ti = capi.GgufTensorInfo()
