@@ -56,6 +56,11 @@ def parse():
     ap.add_argument("--cache-gib", type=float, default=32.0)
     ap.add_argument("--fill", choices=["kernel", "memcpy"], default="kernel",
                     help="lru mode: fill misses with the copy kernel that reads pinned host memory, or with hipMemcpyAsync")
+    ap.add_argument("--source", choices=["pinned", "file", "mapping"], default="pinned",
+                    help="lru mode: where the routed experts live - pinned host memory; a GGUF file written to --file-dir, "
+                         "misses read with pread into the cache's pinned ring; the same file as a plain (pageable) mapping")
+    ap.add_argument("--file-dir", default="/tmp", help="lru mode with --source file/mapping: directory of the model file")
+    ap.add_argument("--pread-threads", type=int, default=4)
     ap.add_argument("--cache-warm-tokens", type=int, default=256,
                     help="lru mode: tokens run before the warm-up steps so that the slot pool is in steady state")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a captured HIP graph")
@@ -227,16 +232,43 @@ def bench_lru(args, torch, capi, synth):
     recently used ones.  The routing trace is known to the host, so the fills of layer l+1 are queued while
     layer l computes.  Eager launches (the cache decides per token what to copy)."""
     H, F, k, E, NL = 2048, 512, 10, args.experts, args.layers
-    note("generating %d layers x %d experts, routed tensors to pinned host memory" % (NL, E))
-    layers, keep, pinned = build_stack(torch, synth, capi, NL, E, synth.BASE_SEED, offload=True)
-    torch.cuda.synchronize()
     gb, db = F * synth.row_bytes(synth.IQ3_S, H), H * synth.row_bytes(synth.Q8_0, F)
     slot_bytes = 2 * gb + db
     cache = C.c_void_p()
-    capi.call("wd_expert_cache_create", C.byref(cache), int(args.cache_gib * (1 << 30)), gb, gb, db, NL, E, 0)
-    capi.call("wd_expert_cache_set_copy_kernel", cache, 1 if args.fill == "kernel" else 0)
-    for l in range(NL):
-        capi.call("wd_expert_cache_register_layer", cache, l, *pinned[l])
+    model_file = None
+    if args.source == "pinned":
+        note("generating %d layers x %d experts, routed tensors to pinned host memory" % (NL, E))
+        layers, keep, pinned = build_stack(torch, synth, capi, NL, E, synth.BASE_SEED, offload=True)
+        torch.cuda.synchronize()
+        capi.call("wd_expert_cache_create", C.byref(cache), int(args.cache_gib * (1 << 30)), gb, gb, db, NL, E, 0)
+        capi.call("wd_expert_cache_set_copy_kernel", cache, 1 if args.fill == "kernel" else 0)
+        for l in range(NL):
+            capi.call("wd_expert_cache_register_layer", cache, l, *pinned[l])
+    else:
+        # the routed tensors go into a GGUF file (names of the model files), are dropped from the device, and come back
+        # through the library's reader: the cache's host sources are pointers into its mapping
+        from warpdecode_amd import ggufio
+        layers, keep = build_stack(torch, synth, capi, NL, E, synth.BASE_SEED)
+        path = os.path.join(args.file_dir, "wd_bench_%d_%dx%d.gguf" % (os.getpid(), NL, E))
+        note("writing %d layers x %d experts (%.1f GB) to %s" % (NL, E, NL * E * slot_bytes / 1e9, path))
+        tensors = []
+        for l in range(NL):
+            for name, dims, ttype in (("gate", [H, F, E], synth.IQ3_S), ("up", [H, F, E], synth.IQ3_S), ("down", [F, H, E], synth.Q8_0)):
+                tensors.append(("blk.%d.ffn_%s_exps.weight" % (l, name), dims, ttype, keep[l][name].cpu().numpy()))
+                keep[l][name] = None
+                setattr(layers[l], name, None)
+        torch.cuda.empty_cache()
+        ggufio.write_gguf(path, tensors, [("general.architecture", ggufio.STRING, "qwen38")])
+        del tensors
+        model_file = ggufio.GgufFile(path)
+        os.unlink(path)     # the open mapping and descriptor keep the file alive; nothing is left behind
+        capi.call("wd_expert_cache_create", C.byref(cache), int(args.cache_gib * (1 << 30)), gb, gb, db, NL, E, 0)
+        if args.source == "file":
+            capi.call("wd_expert_cache_attach_file", cache, C.c_void_p(model_file.map_base), model_file.map_bytes, model_file.fd,
+                      args.pread_threads)
+        for l in range(NL):
+            ptrs = [C.c_void_p(model_file.tensors["blk.%d.ffn_%s_exps.weight" % (l, n)]["ptr"]) for n in ("gate", "up", "down")]
+            capi.call("wd_expert_cache_register_layer", cache, l, *ptrs)
     st_slots = int(args.cache_gib * (1 << 30)) // slot_bytes
     for policy, slots in ((0, st_slots // 2), (0, 2 * st_slots), (1, st_slots)):   # counterfactual pools, same accesses
         capi.call("wd_expert_cache_add_shadow", cache, policy, slots)
@@ -244,8 +276,8 @@ def bench_lru(args, torch, capi, synth):
     capi.call("wd_moe_scratch_create", C.byref(scratch), H, F, E, k)
     st0 = capi.CacheStats()
     capi.call("wd_expert_cache_get_stats", cache, C.byref(st0))
-    note("pool: %d slots of %d B (%.1f GiB) for %d (layer, expert) pairs; host pinned %.1f GB"
-         % (st0.slots, slot_bytes, st0.slots * slot_bytes / 2 ** 30, NL * E, NL * E * slot_bytes / 1e9))
+    note("pool: %d slots of %d B (%.1f GiB) for %d (layer, expert) pairs; host side (%s) %.1f GB"
+         % (st0.slots, slot_bytes, st0.slots * slot_bytes / 2 ** 30, NL * E, args.source, NL * E * slot_bytes / 1e9))
 
     total = args.cache_warm_tokens + args.warmup + args.steps
     rng = synth.rng_for(synth.BASE_SEED, 9001)
@@ -309,7 +341,7 @@ def bench_lru(args, torch, capi, synth):
         "data": "synthetic",
         "config": {"workload": "C3 mode B: %d-layer stack of the 512-expert top-10 IQ3_S/Q8_0 MoE layer, batch=1, routed "
                                "experts in pinned host memory behind a %.0f GiB LRU slot pool in HBM, Zipf(1.1) trace" % (NL, args.cache_gib),
-                   "layers": NL, "experts": E, "top_k": k, "routing": "zipf", "launch": "eager",
+                   "layers": NL, "experts": E, "top_k": k, "routing": "zipf", "launch": "eager", "source": args.source,
                    "slots": int(s1.slots), "slot_bytes": int(slot_bytes), "cache_warm_tokens": args.cache_warm_tokens,
                    "hit_rate": round(hits / max(1, acc), 4), "misses_per_token": round(miss / args.steps, 2),
                    "host_link_bytes_per_token": int(moved / args.steps),

@@ -58,6 +58,10 @@ public:
         double v = 0.0;
         return wd_gguf_meta_number(g_, key.c_str(), &v) == WD_OK ? v : fallback;
     }
+    // The read-only mapping of the whole file and its descriptor, for readers that bypass the mapping.
+    const uint8_t *map_base() const { return wd_gguf_map_base(g_); }
+    size_t map_bytes() const { return wd_gguf_map_bytes(g_); }
+    int fd() const { return wd_gguf_fd(g_); }
     bool has_number_meta(const std::string &key) const {
         double v;
         return wd_gguf_meta_number(g_, key.c_str(), &v) == WD_OK;
@@ -68,6 +72,13 @@ private:
     std::vector<TensorInfo> tensors_;
     std::unordered_map<std::string, size_t> index_;
 };
+
+// Misses of experts that live in this file are read with pread() into the cache's pinned ring (`threads` readers per
+// expert) instead of a pageable copy from the mapping; call it once, before or after the layers are registered.
+// reference: ExpertFileMap / ExpertPreadPool, src/expert_cache.cuh:204-508.
+inline void attach_expert_file(GpuExpertCache &cache, const GgufFile &g, int threads = 4) {
+    check(wd_expert_cache_attach_file(cache.handle(), g.map_base(), g.map_bytes(), g.fd(), threads), "wd_expert_cache_attach_file");
+}
 
 struct Qwen38MoeLayerTensors {
     const TensorInfo *router = nullptr;
