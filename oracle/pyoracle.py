@@ -73,6 +73,7 @@ def _load():
     lib.wdo_quantize_q8_K.argtypes = [_f32p, C.c_int, _i8p, _f32p, _i16p]
     lib.wdo_gemv.argtypes = [C.c_int, _u8p, C.c_int, C.c_int, _i8p, C.c_void_p, _f32p, _i32p]
     lib.wdo_dequant_row.argtypes = [C.c_int, _u8p, C.c_int, _f32p]
+    lib.wdo_gemv_q6_K.argtypes = [_u8p, C.c_int, C.c_int, _i8p, _f32p, _i16p, _f32p, _i32p]
     for n in ("wdo_exp_ggml", "wdo_silu_ggml", "wdo_sigmoid_ggml"):
         getattr(lib, n).restype = C.c_float
         getattr(lib, n).argtypes = [C.c_float]
@@ -161,6 +162,18 @@ def gemv(t, w, rows, cols, act_qs, act_d, want_partials=False):
     act_d = np.ascontiguousarray(act_d, dtype=want_d)
     lib().wdo_gemv(t, _ptr(w, _u8p), rows, cols, _ptr(act_qs, _i8p), act_d.ctypes.data_as(C.c_void_p),
                    _ptr(out, _f32p), _ptr(part, _i32p))
+    return (out, part) if want_partials else out
+
+
+def gemv_q6_K(w, rows, cols, act_qs, act_d, act_bsums, want_partials=False):
+    """Q6_K x Q8_K rows (the output head): out f32 [rows], partials int32 [rows][cols/256][8]."""
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    assert w.size == rows * (cols // 256) * 210
+    out = np.empty(rows, np.float32)
+    part = np.empty((rows, cols // 256 * 8), np.int32) if want_partials else None
+    lib().wdo_gemv_q6_K(_ptr(w, _u8p), rows, cols, _ptr(np.ascontiguousarray(act_qs, np.int8), _i8p),
+                        _ptr(np.ascontiguousarray(act_d, np.float32), _f32p),
+                        _ptr(np.ascontiguousarray(act_bsums, np.int16), _i16p), _ptr(out, _f32p), _ptr(part, _i32p))
     return (out, part) if want_partials else out
 
 

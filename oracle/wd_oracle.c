@@ -26,6 +26,15 @@
  *                                                            headers, which this image lacks.
  *   row_q4_0_q8_0          src/warodecode.cu:1534-1562       int32 block sums vs brute force; the
  *                                                            reference fixes no float order there
+ *   row_q6_K_q8_K          src/lowbit.cuh:2510-2612          integer lane sums vs brute force through an
+ *                                                            independent dequantiser (value formula of
+ *                                                            src/ggml_dequant.hpp:102-140), the known
+ *                                                            answer of tests/lowbit_cuda_test.cu:60-68,
+ *                                                            float64 dot within 1e-5.  The float order
+ *                                                            (eight lanes, fma per super-block, hsum
+ *                                                            tree) is PARITY UNPINNED at bit level: the
+ *                                                            reference has it only as a CUDA kernel and
+ *                                                            ggml itself is not in the tree.
  *
  * Build: see oracle/Makefile (gcc -O2 -ffp-contract=off, no fast-math).
  */
@@ -82,7 +91,8 @@ const uint64_t *wdo_iq2s_grid(void) {
 int wdo_block_elems(int type) {
     switch (type) {
         case WDO_IQ3_S:
-        case WDO_IQ2_S: return 256;
+        case WDO_IQ2_S:
+        case WDO_Q6_K: return 256;
         case WDO_Q8_0:
         case WDO_Q4_0:
         case WDO_IQ4_NL: return 32;
@@ -95,6 +105,7 @@ size_t wdo_block_bytes(int type) {
     switch (type) {
         case WDO_IQ3_S: return 110;
         case WDO_IQ2_S: return 82;
+        case WDO_Q6_K: return 210;
         case WDO_Q8_0: return 34;
         case WDO_Q4_0:
         case WDO_IQ4_NL: return 18;
@@ -379,6 +390,48 @@ float wdo_row_q4_0_q8_0(const uint8_t *w, const int8_t *qs_a, const uint16_t *d_
     return (float)acc;
 }
 
+float wdo_row_q6_K_q8_K(const uint8_t *w, const int8_t *qs, const float *d, const int16_t *bsums, int cols, int32_t *partials) {
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int sb = 0; sb < cols / 256; ++sb) {
+        const uint8_t *blk = w + (size_t)sb * 210;
+        const uint8_t *ql = blk, *qh = blk + 128;
+        const int8_t *sc = (const int8_t *)(blk + 192);
+        const float dw = half_at(blk + 208);
+        const int8_t *a = qs + (size_t)sb * 256;
+        const int16_t *bs = bsums + (size_t)sb * 16;
+        const float ds = dw * d[sb];
+        for (int m = 0; m < 8; ++m) {
+            /* float lane m: byte positions 4m..4m+3 of each of the eight 32-value chunks */
+            int32_t sumi = 0;
+            for (int is = 0; is < 8; ++is) {
+                const int half = is >> 2, sub = is & 3;
+                const int scale = sc[2 * is + (m >> 2)];  /* low 16 bytes of the chunk: scale 2 is, high 16: 2 is + 1 */
+                for (int j = 0; j < 4; ++j) {
+                    const int l = 4 * m + j;
+                    const unsigned qlb = ql[64 * half + ((sub & 1) ? 32 : 0) + l];
+                    const unsigned qhb = qh[32 * half + l];
+                    const int v = (int)((sub < 2 ? (qlb & 15u) : (qlb >> 4)) | (((qhb >> (2 * sub)) & 3u) << 4));
+                    sumi += v * (int)a[32 * is + l] * scale;
+                }
+            }
+            /* the -32 offset of the codes, folded in through the 16-value sums of the activation */
+            const int32_t corr = (int32_t)((uint32_t)((int32_t)bs[2 * m] * sc[2 * m] + (int32_t)bs[2 * m + 1] * sc[2 * m + 1]) << 5);
+            const int32_t lane_sum = sumi - corr;
+            if (partials) partials[sb * 8 + m] = lane_sum;
+            acc[m] = fmaf(ds, (float)lane_sum, acc[m]);
+        }
+    }
+    const float r0 = acc[4] + acc[0], r1 = acc[5] + acc[1], r2 = acc[6] + acc[2], r3 = acc[7] + acc[3];
+    return (r0 + r2) + (r1 + r3);
+}
+
+void wdo_gemv_q6_K(const uint8_t *w, int rows, int cols, const int8_t *qs, const float *d, const int16_t *bsums, float *out,
+                   int32_t *partials) {
+    const size_t rb = (size_t)(cols / 256) * 210;
+    for (int r = 0; r < rows; ++r)
+        out[r] = wdo_row_q6_K_q8_K(w + (size_t)r * rb, qs, d, bsums, cols, partials ? partials + (size_t)r * (cols / 256) * 8 : NULL);
+}
+
 static int partials_per_row(int type, int cols) {
     switch (type) {
         case WDO_IQ3_S:
@@ -428,6 +481,21 @@ void wdo_dequant_row(int type, const uint8_t *w, int cols, float *out) {
                 const unsigned nib = (i < 16) ? (blk[2 + i] & 15u) : (blk[2 + i - 16] >> 4);
                 const int code = (type == WDO_Q4_0) ? (int)nib - 8 : (int)k_iq4nl[nib];
                 out[b * 32 + i] = d * (float)code;
+            }
+        }
+    } else if (type == WDO_Q6_K) {
+        /* value i of a super-block: half = i / 128, quarter q = (i % 128) / 32, l = i % 32; low four bits from
+         * ql[64 half + 32 (q & 1) + l] (low nibble for q < 2, high for q >= 2), two high bits from
+         * qh[32 half + l] >> 2q, scale sc[8 half + 2 q + l / 16]; value = d * sc * (code - 32). */
+        for (int sb = 0; sb < cols / 256; ++sb) {
+            const uint8_t *blk = w + (size_t)sb * 210;
+            const int8_t *sc = (const int8_t *)(blk + 192);
+            const float d = half_at(blk + 208);
+            for (int i = 0; i < 256; ++i) {
+                const int half = i >> 7, q = (i & 127) >> 5, l = i & 31;
+                const unsigned lo = blk[64 * half + 32 * (q & 1) + l];
+                const unsigned code = ((q < 2) ? (lo & 15u) : (lo >> 4)) | (((blk[128 + 32 * half + l] >> (2 * q)) & 3u) << 4);
+                out[sb * 256 + i] = d * (float)sc[8 * half + 2 * q + (l >> 4)] * (float)((int)code - 32);
             }
         }
     } else if (type == WDO_IQ3_S) {

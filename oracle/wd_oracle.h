@@ -28,6 +28,7 @@ enum {
     WDO_F32 = 0,
     WDO_Q4_0 = 2,
     WDO_Q8_0 = 8,
+    WDO_Q6_K = 14,
     WDO_IQ4_NL = 20,
     WDO_IQ3_S = 21,
     WDO_IQ2_S = 22,
@@ -63,6 +64,12 @@ float wdo_row_q8_0_q8_0(const uint8_t *w, const int8_t *qs, const uint16_t *d, i
 float wdo_row_iq4_nl_q8_0(const uint8_t *w, const int8_t *qs, const uint16_t *d, int cols, int32_t *partials);
 /* src/warodecode.cu:1534-1562 (dense Q4_0 x Q8 activation; float order is not canonical there). */
 float wdo_row_q4_0_q8_0(const uint8_t *w, const int8_t *qs, const uint16_t *d, int cols, int32_t *partials);
+/* Q6_K x Q8_K row of the output head, src/lowbit.cuh:2510-2612 (the warp form of ggml's AVX2
+ * ggml_vec_dot_q6_K_q8_K): eight float lanes, lane m = bytes 4m..4m+3 of every 32-value chunk; partials [cols/256][8] =
+ * integer lane sums after the -32 correction.  PARITY UNPINNED for the float order (see wd_oracle.c). */
+float wdo_row_q6_K_q8_K(const uint8_t *w, const int8_t *qs, const float *d, const int16_t *bsums, int cols, int32_t *partials);
+void wdo_gemv_q6_K(const uint8_t *w, int rows, int cols, const int8_t *qs, const float *d, const int16_t *bsums, float *out,
+                   int32_t *partials);
 
 /*
  * Matrix x quantised activation.  `act_d` is float* for Q8_K consumers

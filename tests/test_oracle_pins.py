@@ -466,3 +466,75 @@ def test_layer_against_float64_model(oracle):
                        deq(synth.Q8_0, L["shared_down"], H, F))
     err = np.linalg.norm(out - want) / np.linalg.norm(want)
     assert err < 0.02, err
+
+
+# ---- Q6_K x Q8_K (the output head) ------------------------------------------------------------------------
+def _q6k_codes(w_row, cols):
+    """Independent reading of the Q6_K layout by value index: (code - 32) and the sub-block scale of every value."""
+    nb = cols // 256
+    blk = np.asarray(w_row, np.uint8).reshape(nb, 210).astype(np.int64)
+    i = np.arange(256)
+    half, q, l = i >> 7, (i & 127) >> 5, i & 31
+    lo = blk[:, 64 * half + 32 * (q & 1) + l]
+    low4 = np.where(q < 2, lo & 15, lo >> 4)
+    high2 = (blk[:, 128 + 32 * half + l] >> (2 * q)) & 3
+    sc = blk[:, 192 + 8 * half + 2 * q + (l >> 4)]
+    sc = np.where(sc > 127, sc - 256, sc)
+    return (low4 | (high2 << 4)) - 32, sc
+
+
+def test_q6_k_known_answer(oracle):
+    """tests/lowbit_cuda_test.cu:60-68: every code 33 (value +1), scales 1, d = 1, against an activation of ones."""
+    raw = np.zeros(210, np.uint8)
+    raw[0:128], raw[128:192], raw[192:208] = 0x11, 0xAA, 1
+    raw[208:210] = np.array([1.0], np.float16).view(np.uint8)
+    qs, d, bs = oracle.quantize_q8_K(np.ones(256, np.float32))
+    y, part = oracle.gemv_q6_K(raw, 1, 256, qs, d, bs, want_partials=True)
+    assert abs(float(y[0]) - 256.0) < 0.02
+    assert np.array_equal(part[0], np.full(8, 32 * int(qs[0]), np.int32))   # 32 values of +1 per float lane
+
+
+@pytest.mark.parametrize("cols", [256, 768, 2048, 4096])
+def test_q6_k_brute_force(oracle, cols):
+    rng = synth.rng_for(SEED, 300, cols)
+    rows = 6
+    w = synth.q6_k_matrix(rng, rows, cols)
+    x = rng.normal(0, 1, cols).astype(np.float32)
+    x[256 * (cols // 512):256 * (cols // 512) + 256] *= 1e-3     # one quiet super-block
+    qs, d, bs = oracle.quantize_q8_K(x)
+    y, part = oracle.gemv_q6_K(w, rows, cols, qs, d, bs, want_partials=True)
+    a = qs.astype(np.int64).reshape(-1, 256)
+    for r in range(rows):
+        code, sc = _q6k_codes(w[r], cols)
+        # the eight lane sums of a super-block add up to the exact integer dot of that super-block
+        exact = (code * sc * a).sum(axis=1)
+        assert np.array_equal(part[r].reshape(-1, 8).astype(np.int64).sum(axis=1), exact), (cols, r)
+        # lane m holds bytes 4m..4m+3 of every 32-value chunk, before the -32 offset is moved to the 16-value sums
+        raw = ((code + 32) * sc * a).reshape(-1, 8, 8, 4).sum(axis=(1, 3))          # [sb][m]
+        sc16 = sc.reshape(-1, 16, 16)[:, :, 0]
+        corr = 32 * (bs.astype(np.int64).reshape(-1, 16) * sc16).reshape(-1, 8, 2).sum(axis=2)
+        assert np.array_equal(part[r].reshape(-1, 8).astype(np.int64), raw - corr), (cols, r)
+        dq = oracle.dequant_row(14, w[r], cols).astype(np.float64)
+        dw = np.asarray(w[r], np.uint8).reshape(-1, 210)[:, 208:210].copy().view(np.float16).astype(np.float64)[:, 0]
+        assert np.allclose(dq.reshape(-1, 256), dw[:, None] * sc * code, rtol=0, atol=0)  # the C dequantiser reads the same layout
+        act = (a * d.astype(np.float64)[:, None]).reshape(-1)
+        ref = float(dq @ act)
+        assert abs(float(y[r]) - ref) <= 1e-5 * np.abs(dq * act).sum(), (cols, r)
+
+
+def test_q6_k_float_lanes_are_not_a_plain_sum(oracle):
+    """Negative control: adding the super-block products in plain order gives other bits on some rows, so a check
+    of the eight-lane order would notice a kernel that sums differently."""
+    rng = synth.rng_for(SEED, 301)
+    cols, rows = 2048, 64
+    w = synth.q6_k_matrix(rng, rows, cols)
+    qs, d, bs = oracle.quantize_q8_K(rng.normal(0, 1, cols).astype(np.float32))
+    y, part = oracle.gemv_q6_K(w, rows, cols, qs, d, bs, want_partials=True)
+    differs = 0
+    for r in range(rows):
+        dw = np.asarray(w[r], np.uint8).reshape(-1, 210)[:, 208:210].copy().view(np.float16).astype(np.float32)[:, 0]
+        acc = np.float32(0)
+        for sb in range(cols // 256):
+            acc = np.float32(acc + np.float32(dw[sb] * d[sb]) * np.float32(part[r].reshape(-1, 8)[sb].sum()))
+        differs += int(acc.view(np.uint32) != y[r].view(np.uint32))
+    assert differs > 0

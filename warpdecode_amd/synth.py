@@ -13,8 +13,8 @@ import numpy as np
 
 F32, Q4_0, Q8_0, IQ4_NL, IQ3_S, IQ2_S = 0, 2, 8, 20, 21, 22
 
-BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, IQ4_NL: 32, IQ3_S: 256, IQ2_S: 256}
-BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, IQ4_NL: 18, IQ3_S: 110, IQ2_S: 82}
+BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, IQ4_NL: 32, IQ3_S: 256, IQ2_S: 256, 14: 256}
+BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, IQ4_NL: 18, IQ3_S: 110, IQ2_S: 82, 14: 210}
 
 BASE_SEED = 20261014
 
@@ -80,8 +80,22 @@ def iq2_s_matrix(rng, rows, cols, sigma=0.01):
     return blk.reshape(rows, nb * 82)
 
 
+Q6_K = 14
+
+
+def q6_k_matrix(rng, rows, cols, sigma=0.02):
+    """Q6_K super-blocks (210 bytes per 256 values: ql[128] qh[64] scales[16] d): uniform 6-bit codes, int8 sub-block scales
+    uniform in [-64, 63], fp16 d = |N(0, sigma)| / 2048 at the end of the block."""
+    nb = cols // 256
+    blk = rng.integers(0, 256, size=(rows, nb, 210), dtype=np.uint8)
+    blk[:, :, 192:208] = rng.integers(-64, 64, size=(rows, nb, 16), dtype=np.int8).view(np.uint8)
+    d = (np.abs(rng.normal(0.0, sigma, size=(rows, nb))) / 2048.0).astype(np.float16)
+    blk[:, :, 208:210] = d.view(np.uint8).reshape(rows, nb, 2)
+    return blk.reshape(rows, nb * 210)
+
+
 MATRIX_GEN = {Q8_0: q8_0_matrix, Q4_0: q4_0_matrix, IQ4_NL: iq4_nl_matrix, IQ3_S: iq3_s_matrix,
-              IQ2_S: iq2_s_matrix}
+              IQ2_S: iq2_s_matrix, Q6_K: q6_k_matrix}
 
 
 def matrix(t, rng, rows, cols):
