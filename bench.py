@@ -47,7 +47,7 @@ def parse():
     ap.add_argument("--experts", type=int, default=512)
     ap.add_argument("--routing", choices=["zipf", "router"], default="zipf",
                     help="zipf: ids replayed from the Zipf(1.1) trace; router: ids chosen by the router itself")
-    ap.add_argument("--mode", choices=["resident", "lru", "q4-sweep", "tokens", "c0"], default="resident",
+    ap.add_argument("--mode", choices=["resident", "lru", "q4-sweep", "q6k-head", "tokens", "c0"], default="resident",
                     help="resident: C3 mode A, every expert in HBM; lru: C3 mode B, experts in pinned host memory "
                          "behind an LRU slot pool of --cache-gib in HBM; q4-sweep: the dense Q4_0 GEMV shapes; "
                          "tokens: the 4-token speculative-verify pass over the same layers; c0: the 64-expert top-8 "
@@ -427,6 +427,48 @@ def bench_q4_sweep(args, torch, capi, synth):
                          kernel="k_gemv_q8<Q4_0>", us_per_launch=head["us_per_gemv"], bytes_per_launch=head["bytes"])}))
 
 
+def bench_q6k_head(args, torch, capi, synth):
+    """The output head of the Qwen3 MoE models: Q6_K 151936 x 2048 against the Q8_K image of the F32 activation, once
+    per decoded token.  Every launch of a chain reads another copy of the matrix (7 copies, 1.8 GB) so that nothing
+    comes from the 256 MB last-level cache; the period is taken over a captured chain and includes the launch gap."""
+    rows, cols = 151936, 2048
+    nbytes = rows * synth.row_bytes(synth.Q6_K, cols)
+    copies = 7
+    part = torch.from_numpy(synth.matrix(synth.Q6_K, synth.rng_for(synth.BASE_SEED, 81, rows, cols), 4748, cols)).reshape(-1).cuda()
+    w = part.repeat(rows // 4748)[:nbytes].repeat(copies).reshape(copies, nbytes)
+    x = torch.from_numpy(synth.rms_normed(synth.rng_for(synth.BASE_SEED, 82, cols), cols)).cuda()
+    qs = torch.empty(cols, dtype=torch.int8, device="cuda")
+    sc = torch.empty(cols // 256, dtype=torch.float32, device="cuda")
+    bs = torch.empty(cols // 16, dtype=torch.int16, device="cuda")
+    y = torch.empty(rows, dtype=torch.float32, device="cuda")
+    stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    vp = lambda t: C.c_void_p(t.data_ptr())
+
+    def gemv(i):
+        capi.call("wd_gemv_q6_k_q8_k_f32", C.c_void_p(w[i % copies].data_ptr()), rows, cols, vp(qs), vp(sc), vp(bs), vp(y), None, stream())
+
+    def call(i):
+        capi.call("wd_q8_k_quantize_f32", vp(x), cols, vp(qs), vp(sc), vp(bs), stream())
+        gemv(i)
+
+    call(0)
+    torch.cuda.synchronize()
+    launches = 28
+    reps = max(3, int(1e11 // (nbytes * launches)))
+    us = graph_period_us(torch, gemv, launches, reps)
+    us_call = graph_period_us(torch, call, launches, reps)
+    gbs = nbytes / us / 1e3
+    note("Q6_K head %dx%d: %.2f us, %.0f GB/s" % (rows, cols, us, gbs))
+    print(json.dumps({
+        "metric": "Q6_K x Q8_K output head batch=1: achieved HBM GB/s (151936x2048)", "value": round(gbs, 1), "unit": "GB/s",
+        "n_gpus": 1, "higher_is_better": True, "vs_baseline": None, "dtype": "int8 dot products, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "output head: Q6_K x Q8_K GEMV 151936x2048, raw GGUF 210-byte super-blocks", "bytes": nbytes,
+                   "copies": copies, "us_per_call_with_quantise": round(us_call, 3), "finite": bool(torch.isfinite(y).all().item())},
+        "roofline": dict(bound="hbm", achieved=round(gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(gbs / HBM_PEAK_GBS, 4),
+                         traffic=None, kernel="k_gemv_q6k", us_per_launch=round(us, 3), bytes_per_launch=nbytes)}))
+
+
 def bench_c0(args, torch, capi, synth):
     """BASELINE.json configs[0] at stack depth: the 64-expert top-8 layer with Q8_0 gate/up/down and no shared expert
     (hidden 2048, ffn 512), `--layers` independent layers chained as in the headline workload, router-selected."""
@@ -572,6 +614,8 @@ def main():
         return bench_q4_sweep(args, torch, capi, synth)
     if args.mode == "c0":
         return bench_c0(args, torch, capi, synth)
+    if args.mode == "q6k-head":
+        return bench_q6k_head(args, torch, capi, synth)
     note("generating %d layers x %d experts on the device" % (NL, E))
     if args.mode == "tokens":
         return bench_tokens(args, torch, capi, synth)

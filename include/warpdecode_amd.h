@@ -36,6 +36,7 @@ typedef enum {
     WD_TYPE_F16 = 1,
     WD_TYPE_Q4_0 = 2,
     WD_TYPE_Q8_0 = 8,
+    WD_TYPE_Q6_K = 14,
     WD_TYPE_IQ4_NL = 20,
     WD_TYPE_IQ3_S = 21,
     WD_TYPE_IQ2_S = 22
@@ -96,6 +97,13 @@ int wd_topk_softmax(const float *d_logits, int n_experts, int k, float expert_sc
  *   q38_hc_launch_exact_q8_0_gemv_f32 (src/qwen38_hc.cuh:1020-1049),
  *   q4_0_q8_0_gemv_kernel via launch_q4_float (src/warodecode.cu:1534-1562, :1746-1768; the planar
  *   prepack of the reference is not needed: raw 18-byte blocks are read directly). */
+/* Q6_K x Q8_K GEMV (the output head): 210-byte super-blocks of 256 six-bit codes with sixteen int8 sub-block scales;
+ * the -32 offset of the codes is taken out through the activation's 16-value sums.  Eight float lanes per row (lane m =
+ * bytes 4m..4m+3 of every 32-value chunk), one fma per super-block, ggml's closing tree.  d_partials (may be NULL):
+ * int32 [rows][cols/256][8], the integer lane sums after the correction.
+ * reference: launch_q6_k_gemv_q8_k_f32 / q6_k_q8_k_gemv_kernel, src/lowbit.cuh:2510-2636. */
+int wd_gemv_q6_k_q8_k_f32(const uint8_t *d_w, int rows, int cols, const int8_t *d_act_qs, const float *d_act_scales,
+                          const int16_t *d_act_bsums, float *d_out, int32_t *d_partials, void *stream);
 int wd_gemv_q8_k_f32(int type, const uint8_t *d_w, int rows, int cols, const int8_t *d_act_qs,
                      const float *d_act_scales, float *d_out, int32_t *d_partials, void *stream);
 int wd_gemv_q8_0_f32(int type, const uint8_t *d_w, int rows, int cols, const int8_t *d_act_qs,

@@ -273,6 +273,37 @@ static void gpu_checks() {
         CHECK(same_bits(got.data(), want.data(), F), "launch_iq3_s_gemv_q8_k_f32 differs from the oracle");
     }
 
+    // the output head: Q6_K x Q8_K from the caller's F32 activation, against the oracle
+    {
+        Rng r(11);
+        const int V = 1003;
+        const std::vector<float> x = rms_normed(r, H);
+        std::vector<uint8_t> head(static_cast<size_t>(V) * (H / 256) * 210);
+        for (auto &b : head) b = static_cast<uint8_t>(r.u32());
+        for (size_t i = 0; i < head.size() / 210; ++i) {
+            const uint16_t d = wdo_f32_to_f16(std::fabs(r.normal()) * 1e-5f);
+            std::memcpy(&head[i * 210 + 208], &d, 2);
+        }
+        TensorInfo info{"output.weight", {static_cast<uint64_t>(H), static_cast<uint64_t>(V)}, GgmlType::Q6_K, 0, head.data()};
+        LowBitMatrix w = upload_lowbit_matrix(info);
+        CHECK(lowbit_q6_k_head_q8_k_eligible(w), "a Q6_K matrix with 256-multiple columns is eligible");
+        DeviceFloatArray dx, y(V);
+        dx.upload(x.data(), H);
+        launch_q6_k_head_gemv_q8_k_from_f32(w, dx.data, y.data, stream);
+        launch_q6_k_head_gemv_q8_k_from_f32(w, dx.data, y.data, stream);  // the kept scratch is reused
+        check(wd_stream_sync(stream), "sync");
+        std::vector<int8_t> oq(H);
+        std::vector<float> od(H / 256), want(V), got(V);
+        std::vector<int16_t> ob(H / 16);
+        wdo_quantize_q8_K(x.data(), H, oq.data(), od.data(), ob.data());
+        wdo_gemv_q6_K(head.data(), V, H, oq.data(), od.data(), ob.data(), want.data(), nullptr);
+        y.download(got.data());
+        CHECK(same_bits(got.data(), want.data(), V), "launch_q6_k_head_gemv_q8_k_from_f32 differs from the oracle");
+        LowBitMatrix q8 = borrow_lowbit_matrix(w.data, V, H, GgmlType::Q8_0, w.bytes);
+        CHECK(throws([&] { launch_q6_k_head_gemv_q8_k_from_f32(q8, dx.data, y.data, stream); }), "the head path refuses other types");
+        CHECK(throws([&] { launch_q6_k_gemv_q8_k_f32(w, nullptr, nullptr, nullptr, y.data, stream, 48); }), "threads must be a multiple of 32");
+    }
+
     std::vector<GpuMatrix> routers;
     std::vector<Qwen38SharedExpertWeights> shared(layers);
     for (int l = 0; l < layers; ++l) {

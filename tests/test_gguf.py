@@ -111,8 +111,8 @@ def test_malformed_files_are_refused(tmp_path):
 
 def test_unknown_tensor_type_is_listed_without_size(tmp_path):
     path = tmp_path / "q6.gguf"
-    ggufio.write_gguf(path, [("output.weight", [256, 4], 14, np.zeros(4 * 210, np.uint8)),   # Q6_K: not computed here
+    ggufio.write_gguf(path, [("output.weight", [256, 4], 12, np.zeros(4 * 144, np.uint8)),   # Q4_K: not computed here
                              ("x", [32], capi.Q8_0, np.zeros(34, np.uint8))])
     with ggufio.GgufFile(path) as g:
-        assert g.tensors["output.weight"]["bytes"] == 0 and g.tensors["output.weight"]["type"] == 14
+        assert g.tensors["output.weight"]["bytes"] == 0 and g.tensors["output.weight"]["type"] == 12
         assert g.tensors["x"]["bytes"] == 34

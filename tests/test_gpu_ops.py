@@ -141,6 +141,57 @@ def test_gemv_single(g, oracle, t):
             assert g.same_bits(g.host(out2), want), (t, rows, cols)
 
 
+# the output head of the Qwen3 MoE models (151936 x 2048), then ragged super-block counts (partial last pass, rows that
+# do not start on 16-byte boundaries), one super-block, many passes
+Q6K_SHAPES = [(151936, 2048), (1000, 4096), (37, 256), (129, 768), (65, 1280), (33, 2304), (9, 8192), (3, 32768)]
+
+
+@pytest.mark.parametrize("rows,cols", Q6K_SHAPES)
+def test_gemv_q6_k(g, oracle, rows, cols):
+    rng = synth.rng_for(SEED, 27, rows, cols)
+    w = synth.matrix(synth.Q6_K, rng, rows, cols)
+    x = rng.normal(0, 1, cols).astype(np.float32)
+    qs, d, bs = oracle.quantize_q8_K(x)
+    dw, dq, dd, db = g.dev(w), g.dev(qs), g.dev(d), g.dev(bs)
+    out, out2, part = g.empty(rows, np.float32), g.empty(rows, np.float32), g.empty((rows, cols // 256 * 8), np.int32)
+    capi.call("wd_gemv_q6_k_q8_k_f32", g.ptr(dw), rows, cols, g.ptr(dq), g.ptr(dd), g.ptr(db), g.ptr(out), g.ptr(part), g.stream())
+    capi.call("wd_gemv_q6_k_q8_k_f32", g.ptr(dw), rows, cols, g.ptr(dq), g.ptr(dd), g.ptr(db), g.ptr(out2), None, g.stream())
+    g.sync()
+    want, wpart = oracle.gemv_q6_K(w, rows, cols, qs, d, bs, want_partials=True)
+    assert np.array_equal(g.host(part), wpart), (rows, cols)
+    assert g.same_bits(g.host(out), want), (rows, cols)
+    assert g.same_bits(g.host(out2), want), (rows, cols)
+
+
+def test_gemv_q6_k_head_from_f32_and_misaligned(g, oracle):
+    """The head as the caller runs it (quantise on the device, then the GEMV), and the same matrix 2 bytes into an
+    allocation (GGUF blocks are only 2-byte aligned): the unaligned fetch must give the same bits."""
+    import torch
+    rows, cols = 515, 2048
+    rng = synth.rng_for(SEED, 28, rows, cols)
+    w = synth.matrix(synth.Q6_K, rng, rows, cols)
+    x = synth.rms_normed(rng, cols)
+    dx = g.dev(x)
+    dq, dd, db = g.empty(cols, np.int8), g.empty(cols // 256, np.float32), g.empty(cols // 16, np.int16)
+    capi.call("wd_q8_k_quantize_f32", g.ptr(dx), cols, g.ptr(dq), g.ptr(dd), g.ptr(db), g.stream())
+    out = g.empty(rows, np.float32)
+    dw = g.dev(w)
+    capi.call("wd_gemv_q6_k_q8_k_f32", g.ptr(dw), rows, cols, g.ptr(dq), g.ptr(dd), g.ptr(db), g.ptr(out), None, g.stream())
+    shifted = torch.zeros(w.size + 16, dtype=torch.uint8, device="cuda")
+    shifted[2:2 + w.size] = dw.reshape(-1)
+    out_s = g.empty(rows, np.float32)
+    capi.call("wd_gemv_q6_k_q8_k_f32", shifted.data_ptr() + 2, rows, cols, g.ptr(dq), g.ptr(dd), g.ptr(db), g.ptr(out_s), None, g.stream())
+    g.sync()
+    qs, d, bs = oracle.quantize_q8_K(x)
+    want = oracle.gemv_q6_K(w, rows, cols, qs, d, bs)
+    assert g.same_bits(g.host(out), want)
+    assert g.same_bits(g.host(out_s), want)
+    # against the dequantised weights in float64: the integer path is the exact product of the quantised operands
+    xq = (qs.astype(np.float64).reshape(-1, 256) * d.astype(np.float64)[:, None]).reshape(-1)
+    ref = np.array([oracle.dequant_row(synth.Q6_K, w[r], cols).astype(np.float64) @ xq for r in range(64)])
+    assert np.allclose(g.host(out)[:64], ref, rtol=1e-4, atol=1e-6)
+
+
 def test_q4_0_gemv_misaligned_base(g, oracle):
     """A matrix that starts 2 bytes into an allocation (GGUF blocks are only 2-byte aligned) takes the general
     kernel instead of the streaming one; both must give the same block sums."""
@@ -244,3 +295,5 @@ def test_error_paths(g):
     assert lib.wd_topk_softmax(g.ptr(x), 64, 17, 1.0, g.ptr(x), g.ptr(x), None) == -1
     assert lib.wd_gemv_q8_0_f32(synth.IQ3_S, g.ptr(x), 4, 256, g.ptr(x), g.ptr(x), g.ptr(x), None, None) == -1
     assert lib.wd_gemv_q8_k_f32(synth.IQ3_S, g.ptr(x), 4, 100, g.ptr(x), g.ptr(x), g.ptr(x), None, None) == -1
+    assert lib.wd_gemv_q6_k_q8_k_f32(g.ptr(x), 4, 300, g.ptr(x), g.ptr(x), g.ptr(x), g.ptr(x), None, None) == -1
+    assert lib.wd_gemv_q6_k_q8_k_f32(g.ptr(x), 4, 65536, g.ptr(x), g.ptr(x), g.ptr(x), g.ptr(x), None, None) == -1

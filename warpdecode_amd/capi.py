@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(HERE, "libwarpdecode_amd.so")
 HEADER = os.path.join(os.path.dirname(HERE), "include", "warpdecode_amd.h")
 
 F32, F16, Q4_0, Q8_0, IQ4_NL, IQ3_S, IQ2_S = 0, 1, 2, 8, 20, 21, 22
+Q6_K = 14
 MOE_PRESELECTED, MOE_KEEP_EXPERT_OUT, MOE_STAGED = 1, 2, 4
 
 vp, i32, f32, sz, u32 = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint
@@ -50,6 +51,7 @@ class CacheStats(C.Structure):
 _SIGS = {
     "wd_init": (i32, [i32]),
     "wd_row_bytes": (sz, [i32, i32]),
+    "wd_gemv_q6_k_q8_k_f32": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp]),
     "wd_tensor_bytes": (sz, [i32, i32, i32]),
     "wd_malloc": (i32, [C.POINTER(vp), sz]),
     "wd_free": (i32, [vp]),

@@ -34,7 +34,8 @@ inline hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
 inline int block_elems(int type) {
     switch (type) {
         case WD_TYPE_IQ3_S:
-        case WD_TYPE_IQ2_S: return 256;
+        case WD_TYPE_IQ2_S:
+        case WD_TYPE_Q6_K: return 256;
         case WD_TYPE_Q8_0:
         case WD_TYPE_Q4_0:
         case WD_TYPE_IQ4_NL: return 32;
@@ -47,6 +48,7 @@ inline size_t block_bytes(int type) {
     switch (type) {
         case WD_TYPE_IQ3_S: return 110;
         case WD_TYPE_IQ2_S: return 82;
+        case WD_TYPE_Q6_K: return 210;
         case WD_TYPE_Q8_0: return 34;
         case WD_TYPE_Q4_0:
         case WD_TYPE_IQ4_NL: return 18;

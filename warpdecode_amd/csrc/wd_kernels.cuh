@@ -302,6 +302,36 @@ __global__ __launch_bounds__(WPB * 64) void k_gemv_q4_stream(const uint8_t *__re
     }
 }
 
+// ---- Q6_K x Q8_K GEMV: one row per wave and step, `rows_per_wave` steps ---------------------------------------
+// The activation (quants, scales, 16-value sums) is staged in LDS once per workgroup.
+// dynamic LDS: cols bytes, then cols/256 floats, then cols/16 int16 (each part 16-byte aligned), then 4 * 1696 bytes.
+template <bool PART, bool ALIGNED>
+__global__ __launch_bounds__(256) void k_gemv_q6k(const uint8_t *__restrict__ w, int rows, int cols, int rows_per_wave,
+                                                   const int8_t *__restrict__ act_qs, const float *__restrict__ act_d,
+                                                   const int16_t *__restrict__ act_bsums, float *__restrict__ out,
+                                                   int32_t *__restrict__ partials) {
+    extern __shared__ __align__(16) uint8_t q6_lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nb = cols >> 8;
+    int8_t *aq = reinterpret_cast<int8_t *>(q6_lds);
+    float *ad = reinterpret_cast<float *>(q6_lds + cols);
+    int16_t *ab = reinterpret_cast<int16_t *>(q6_lds + cols + ((nb * 4 + 15) & ~15));
+    uint8_t *stage = q6_lds + cols + ((nb * 4 + 15) & ~15) + nb * 32 + wave * 1696;
+    for (int i = threadIdx.x; i < cols / 16; i += 256) reinterpret_cast<uint4 *>(aq)[i] = reinterpret_cast<const uint4 *>(act_qs)[i];
+    for (int i = threadIdx.x; i < nb; i += 256) ad[i] = act_d[i];
+    for (int i = threadIdx.x; i < nb * 8; i += 256) reinterpret_cast<uint32_t *>(ab)[i] = reinterpret_cast<const uint32_t *>(act_bsums)[i];
+    __syncthreads();
+    const size_t rb = static_cast<size_t>(nb) * 210;
+    const long long r0 = (static_cast<long long>(blockIdx.x) * 4 + wave) * rows_per_wave;
+    for (int i = 0; i < rows_per_wave; ++i) {
+        const long long r = r0 + i;
+        if (r >= rows) break;  // wave-uniform
+        const float y = q6k_row<PART, ALIGNED>(w + static_cast<size_t>(r) * rb, nb, aq, ad, ab, lane, stage,
+                                               PART ? partials + static_cast<size_t>(r) * nb * 8 : nullptr);
+        if (lane == 0) out[r] = y;
+    }
+}
+
 // ---- elementwise ---------------------------------------------------------------------------------
 __global__ void k_silu_mul_experts(const float *__restrict__ gate_up, float *__restrict__ act, int ffn) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;

@@ -235,6 +235,37 @@ static int launch_gemv_q8_0(int type, MatSrc src, int mats, int rows, int cols, 
     return WD_OK;
 }
 
+int wd_gemv_q6_k_q8_k_f32(const uint8_t *d_w, int rows, int cols, const int8_t *d_act_qs, const float *d_act_scales,
+                          const int16_t *d_act_bsums, float *d_out, int32_t *d_partials, void *stream) {
+    WD_REQUIRE(d_w && d_act_qs && d_act_scales && d_act_bsums && d_out, "Q6_K GEMV: null pointer");
+    WD_REQUIRE(rows > 0 && cols > 0 && cols % 256 == 0, "Q6_K x Q8_K GEMV geometry mismatch (%d x %d)", rows, cols);
+    WD_REQUIRE(cols <= 32768, "Q6_K GEMV: at most 32768 columns (got %d)", cols);
+    WD_REQUIRE(reinterpret_cast<uintptr_t>(d_act_qs) % 16 == 0 && reinterpret_cast<uintptr_t>(d_act_bsums) % 4 == 0,
+               "Q6_K GEMV: the activation quants must be 16-byte aligned, the sums 4-byte aligned");
+    const int nb = cols / 256;
+    // rows are 210 * nb bytes: they all start on 16-byte boundaries when the matrix does and nb is a multiple of 8
+    const bool aligned = reinterpret_cast<uintptr_t>(d_w) % 16 == 0 && nb % 8 == 0;
+    // enough rows per wave to pay for staging the activation, few enough to keep every compute unit busy
+    int rpw = rows / (4 * 2048);
+    rpw = rpw < 1 ? 1 : (rpw > 16 ? 16 : rpw);
+    const unsigned wgs = static_cast<unsigned>((static_cast<long long>(rows) + 4LL * rpw - 1) / (4LL * rpw));
+    const size_t lds = static_cast<size_t>(cols) + ((nb * 4 + 15) & ~15) + static_cast<size_t>(nb) * 32 + 4 * 1696;
+    hipStream_t st = as_stream(stream);
+    if (d_partials) {
+        if (aligned)
+            k_gemv_q6k<true, true><<<wgs, 256, lds, st>>>(d_w, rows, cols, rpw, d_act_qs, d_act_scales, d_act_bsums, d_out, d_partials);
+        else
+            k_gemv_q6k<true, false><<<wgs, 256, lds, st>>>(d_w, rows, cols, rpw, d_act_qs, d_act_scales, d_act_bsums, d_out, d_partials);
+    } else {
+        if (aligned)
+            k_gemv_q6k<false, true><<<wgs, 256, lds, st>>>(d_w, rows, cols, rpw, d_act_qs, d_act_scales, d_act_bsums, d_out, nullptr);
+        else
+            k_gemv_q6k<false, false><<<wgs, 256, lds, st>>>(d_w, rows, cols, rpw, d_act_qs, d_act_scales, d_act_bsums, d_out, nullptr);
+    }
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
 int wd_gemv_q8_k_f32(int type, const uint8_t *d_w, int rows, int cols, const int8_t *d_act_qs,
                      const float *d_act_scales, float *d_out, int32_t *d_partials, void *stream) {
     WD_REQUIRE(d_w != nullptr, "low-bit GEMV: null weight pointer");

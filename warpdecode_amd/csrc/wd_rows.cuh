@@ -354,6 +354,95 @@ WD_DEV float iq_row_q8k(const uint8_t *row, int nb, const IqTables &t, const int
     return y[0];
 }
 
+// ---- Q6_K x Q8_K (the output head) --------------------------------------------------------------------
+// src/lowbit.cuh:2510-2612.  A super-block is 210 bytes: ql[128] (low four bits of the codes), qh[64] (high two bits),
+// sixteen int8 scales, fp16 d.  Lane (is = lane >> 3, sb = lane & 7) takes the 32-value chunk `is` of super-block
+// 8 * pass + sb: half = is >> 2, sub = is & 3; code byte l = (ql[64 half + 32 (sub & 1) + l] low or high nibble by
+// sub < 2) | ((qh[32 half + l] >> 2 sub) & 3) << 4; the chunk's low 16 bytes use scale 2 is, the high 16 scale
+// 2 is + 1.  Its eight dwords are the eight float lanes of the reference (lane m = bytes 4m..4m+3): p[m] =
+// scale * dot4.  After the fold over the eight chunk lanes, lane (m, sb) holds lane sum m of super-block sb, takes
+// the -32 correction ((bsums[2m] scale[2m] + bsums[2m+1] scale[2m+1]) << 5 - it has read exactly that scale pair
+// for its own chunk) and runs chain m along the super-blocks, as the IQ rows do.
+// A pass (eight super-blocks, 1680 bytes) is fetched with one or two 16-byte loads per lane into LDS and the fields
+// are picked from there; blocks are 2-byte aligned, so the 32-byte runs are read as nine aligned dwords and shifted
+// by two bytes in the odd super-blocks.  ALIGNED: the row starts on a 16-byte boundary.
+// stage: 1696 bytes of LDS owned by the wave, 16-byte aligned.
+template <bool PART, bool ALIGNED>
+WD_DEV float q6k_row(const uint8_t *row, int nb, const int8_t *act_qs, const float *act_d, const int16_t *act_bsums, int lane,
+                     uint8_t *stage, int32_t *partials) {
+    const int is = lane >> 3, sbl = lane & 7;
+    const bool first = sbl == 0;
+    const int half = is >> 2, sub = is & 3;
+    float acc = 0.0f;
+    for (int base = 0; base < nb; base += 8) {
+        const int n_here = min(8, nb - base);
+        const int bytes = n_here * 210, words = bytes >> 4, tail = (bytes & 15) >> 1;  // full 16-byte words, then 2-byte pieces
+        const uint8_t *src = row + static_cast<size_t>(base) * 210;
+        uint4 u0 = make_uint4(0, 0, 0, 0), u1 = u0;
+        uint16_t t16 = 0;
+        if (lane < words) u0 = ALIGNED ? gld_u128_aligned(src + 16 * lane) : gld_u128(src + 16 * lane);
+        if (lane + 64 < words) u1 = ALIGNED ? gld_u128_aligned(src + 16 * (lane + 64)) : gld_u128(src + 16 * (lane + 64));
+        if (lane < tail) t16 = gld_u16(src + 16 * words + 2 * lane);
+        wave_lds_fence();  // the previous pass has been read
+        if (lane < words) reinterpret_cast<uint4 *>(stage)[lane] = u0;
+        if (lane + 64 < words) reinterpret_cast<uint4 *>(stage)[lane + 64] = u1;
+        if (lane < tail) reinterpret_cast<uint16_t *>(stage + 16 * words)[lane] = t16;
+        wave_lds_fence();
+        const int sb = base + sbl;
+        const bool on = sb < nb;
+        int p[8];
+        int sc0 = 0, sc1 = 0;
+        float ds = 0.0f;
+        if (on) {
+            const uint8_t *blk = stage + 210 * sbl;
+            const uint32_t sh = (sbl & 1) ? 2u : 0u;  // 210 * sbl is 2 (mod 4) in the odd super-blocks of a pass
+            const uint32_t *lw = reinterpret_cast<const uint32_t *>(blk + 64 * half + 32 * (sub & 1) - sh);
+            const uint32_t *hw = reinterpret_cast<const uint32_t *>(blk + 128 + 32 * half - sh);
+            uint32_t lr[9], hr[9];
+#pragma unroll
+            for (int j = 0; j < 9; ++j) lr[j] = lw[j], hr[j] = hw[j];
+            const uint32_t pair = *reinterpret_cast<const uint16_t *>(blk + 192 + 2 * is);
+            sc0 = static_cast<int8_t>(pair & 0xffu), sc1 = static_cast<int8_t>(pair >> 8);
+            const float dw = h2f(*reinterpret_cast<const uint16_t *>(blk + 208));
+            const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + is * 32);
+            const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + is * 32 + 16);
+            const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+            const uint32_t low_shift = (sub < 2) ? 0u : 4u, high_shift = 2u * sub;
+#pragma unroll
+            for (int m = 0; m < 8; ++m) {
+                const uint32_t lo = __builtin_amdgcn_alignbyte(lr[m + 1], lr[m], sh);
+                const uint32_t hi = __builtin_amdgcn_alignbyte(hr[m + 1], hr[m], sh);
+                const uint32_t code = ((lo >> low_shift) & 0x0f0f0f0fu) | (((hi >> high_shift) & 0x03030303u) << 4);
+                p[m] = __mul24(m < 4 ? sc0 : sc1, sdot4(code, a[m], 0));
+            }
+            ds = dw * act_d[sb];
+        } else {
+#pragma unroll
+            for (int m = 0; m < 8; ++m) p[m] = 0;
+        }
+        int lane_sum = reduce_scatter_ib(p, lane);  // lane (m = is, sb): float lane m of super-block sb
+        if (on) {
+            const uint32_t bs = *reinterpret_cast<const uint32_t *>(act_bsums + sb * 16 + 2 * is);
+            const int b0 = static_cast<int16_t>(bs & 0xffffu), b1 = static_cast<int16_t>(bs >> 16);
+            lane_sum -= static_cast<int>(static_cast<uint32_t>(b0 * sc0 + b1 * sc1) << 5);
+            if (PART) partials[sb * 8 + is] = lane_sum;
+        }
+        const float pf = on ? static_cast<float>(lane_sum) : 0.0f;
+        // carry of the previous pass: last lane of the group -> first lane (lanes past the row's end pass the
+        // accumulator through unchanged, fma(0, 0, acc) == acc)
+        const float carry = dpp_f<kDppShl7>(0.0f, acc);
+        float v = __builtin_fmaf(ds, pf, base == 0 ? 0.0f : carry);
+#pragma unroll
+        for (int s = 1; s < 8; ++s) {
+            const float up = dpp_f<kDppShr1>(0.0f, v);
+            const float nxt = __builtin_fmaf(ds, pf, up);
+            v = first ? v : nxt;
+        }
+        acc = v;
+    }
+    return close_lanes8_strided(acc);
+}
+
 // ---- Q8_0 (and Q4_0 / IQ4_NL codes) x Q8_0 ------------------------------------------------
 // Four rows per wave step: lane (r4 = lane >> 4, b = lane & 15) takes blocks b, b+16, ... of row r4.
 // The per-block chunk sums are handed to the chain lanes through a per-wave LDS tile so that every

@@ -30,6 +30,7 @@ enum class GgmlType : uint32_t {
     F16 = 1,
     Q4_0 = 2,
     Q8_0 = 8,
+    Q6_K = 14,
     IQ4_NL = 20,
     IQ3_S = 21,
     IQ2_S = 22,
@@ -135,7 +136,8 @@ private:
 };
 
 inline bool lowbit_gemv_supported(GgmlType t) {
-    return t == GgmlType::Q8_0 || t == GgmlType::IQ4_NL || t == GgmlType::IQ2_S || t == GgmlType::IQ3_S || t == GgmlType::Q4_0;
+    return t == GgmlType::Q8_0 || t == GgmlType::IQ4_NL || t == GgmlType::IQ2_S || t == GgmlType::IQ3_S || t == GgmlType::Q4_0 ||
+           t == GgmlType::Q6_K;
 }
 
 // src/lowbit.cuh:72-86
@@ -153,7 +155,7 @@ inline LowBitMatrix upload_lowbit_matrix(const TensorInfo &t) {
     out.cols = static_cast<int>(t.dims[0]);
     out.rows = static_cast<int>(t.dims[1]);
     out.type = t.type;
-    const int quantum = (t.type == GgmlType::IQ2_S || t.type == GgmlType::IQ3_S) ? 256 : 32;
+    const int quantum = (t.type == GgmlType::IQ2_S || t.type == GgmlType::IQ3_S || t.type == GgmlType::Q6_K) ? 256 : 32;
     if (out.cols <= 0 || out.rows <= 0 || out.cols % quantum != 0) throw std::runtime_error("invalid low-bit matrix shape: " + t.name);
     out.bytes = t.byte_size();
     void *p = nullptr;
@@ -477,6 +479,54 @@ inline void launch_iq2_s_gemv_q8_k_f32(const LowBitMatrix &w, const int8_t *act,
     if (w.type != GgmlType::IQ2_S || w.rows <= 0 || w.cols <= 0 || w.cols % 256 != 0) throw std::runtime_error("IQ2_S x Q8_K GEMV geometry mismatch");
     check(wd_gemv_q8_k_f32(WD_TYPE_IQ2_S, w.data, w.rows, w.cols, act, act_scales, out, nullptr, stream), "IQ2_S GEMV failed");
 }
+// src/lowbit.cuh:2615-2636
+inline void launch_q6_k_gemv_q8_k_f32(const LowBitMatrix &w, const int8_t *act, const float *act_scales, const int16_t *act_sums, float *out, Stream stream, int threads = 256) {
+    if (w.type != GgmlType::Q6_K || w.rows <= 0 || w.cols <= 0 || w.cols % 256 != 0) throw std::runtime_error("Q6_K x Q8_K GEMV geometry mismatch");
+    if (threads < 32 || threads % 32 != 0) throw std::runtime_error("Q6_K x Q8_K GEMV threads must be a multiple of 32");
+    check(wd_gemv_q6_k_q8_k_f32(w.data, w.rows, w.cols, act, act_scales, act_sums, out, nullptr, stream), "Q6_K GEMV failed");
+}
+
+// Q8_K image of the head's activation; a few kilobytes kept for the life of the process and never shrunk or moved
+// while a launch may still read it (a larger request allocates a new one and leaves the old in place).
+// src/lowbit.cuh:2638-2710
+struct LowBitHeadQ8KScratch {
+    int cols = 0;
+    int8_t *quants = nullptr;
+    float *scales = nullptr;
+    int16_t *sums = nullptr;
+};
+inline LowBitHeadQ8KScratch &lowbit_head_q8_k_scratch() {
+    static LowBitHeadQ8KScratch scratch;
+    return scratch;
+}
+inline void lowbit_head_q8_k_reserve(int cols) {
+    LowBitHeadQ8KScratch &s = lowbit_head_q8_k_scratch();
+    if (cols <= s.cols) return;
+    LowBitHeadQ8KScratch n;
+    void *q = nullptr, *d = nullptr, *b = nullptr;
+    if (wd_malloc(&q, static_cast<size_t>(cols)) != WD_OK || wd_malloc(&d, sizeof(float) * (cols / 256)) != WD_OK ||
+        wd_malloc(&b, sizeof(int16_t) * (cols / 16)) != WD_OK) {
+        wd_free(q), wd_free(d), wd_free(b);
+        throw std::runtime_error(std::string("Q8_K head scratch allocation failed: ") + wd_last_error());
+    }
+    n.cols = cols, n.quants = static_cast<int8_t *>(q), n.scales = static_cast<float *>(d), n.sums = static_cast<int16_t *>(b);
+    s = n;  // the previous buffers stay allocated: a launch in flight may still read them
+}
+// src/lowbit.cuh:2712-2716
+inline bool lowbit_q6_k_head_q8_k_eligible(const LowBitMatrix &w) {
+    return w.type == GgmlType::Q6_K && w.rows > 0 && w.cols > 0 && w.cols % 256 == 0;
+}
+// The output head from the caller's F32 activation: Q8_K quantisation, then the Q6_K x Q8_K GEMV into F32 logits.
+// src/lowbit.cuh:2724-2744
+inline void launch_q6_k_head_gemv_q8_k_from_f32(const LowBitMatrix &w, const float *activation, float *out, Stream stream, int threads = 256) {
+    if (!lowbit_q6_k_head_q8_k_eligible(w)) throw std::runtime_error("Q6_K x Q8_K output head path is not available for this matrix");
+    if (threads < 32 || threads % 32 != 0) throw std::runtime_error("Q6_K x Q8_K GEMV threads must be a multiple of 32");
+    lowbit_head_q8_k_reserve(w.cols);
+    LowBitHeadQ8KScratch &s = lowbit_head_q8_k_scratch();
+    launch_q8_k_quantize_f32(activation, w.cols, s.quants, s.scales, s.sums, stream, threads);
+    launch_q6_k_gemv_q8_k_f32(w, s.quants, s.scales, s.sums, out, stream, threads);
+}
+
 // src/lowbit.cuh:1787-1810
 inline void launch_iq4_nl_gemv_q8_0_f32(const LowBitMatrix &w, const int8_t *act, const half_bits *act_scales, float *out, Stream stream, int /*threads*/ = 256) {
     if (w.type != GgmlType::IQ4_NL || w.rows <= 0 || w.cols <= 0 || w.cols % 64 != 0) throw std::runtime_error("IQ4_NL x Q8_0 GEMV geometry mismatch");
