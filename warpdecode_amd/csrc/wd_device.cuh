@@ -96,6 +96,7 @@ WD_DEV float dpp_f(float old, float v) {
 constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppRor4 = 0x124, kDppRor8 = 0x128, kDppBcast15 = 0x142,
               kDppBcast31 = 0x143;
 constexpr int kDppShr1 = 0x111, kDppShl1 = 0x101, kDppShl2 = 0x102, kDppShl4 = 0x104, kDppShl7 = 0x107;
+constexpr int kDppShr2 = 0x112, kDppShl14 = 0x10E;
 
 WD_DEV float readlane_f(float v, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));

@@ -302,33 +302,82 @@ __global__ __launch_bounds__(WPB * 64) void k_gemv_q4_stream(const uint8_t *__re
     }
 }
 
-// ---- Q6_K x Q8_K GEMV: one row per wave and step, `rows_per_wave` steps ---------------------------------------
+// ---- Q6_K x Q8_K GEMV: the waves of the grid take the rows in turn, pass by pass, one pass fetched ahead -------
 // The activation (quants, scales, 16-value sums) is staged in LDS once per workgroup.
-// dynamic LDS: cols bytes, then cols/256 floats, then cols/16 int16 (each part 16-byte aligned), then 4 * 1696 bytes.
-template <bool PART, bool ALIGNED>
-__global__ __launch_bounds__(256) void k_gemv_q6k(const uint8_t *__restrict__ w, int rows, int cols, int rows_per_wave,
+// dynamic LDS: kQ6ActStride bytes per super-block, then cols/256 floats, then cols/16 int16 (each part 16-byte
+// aligned), then four wave stages of kQ6StageBytes.
+// FULL: rows are a whole number of passes.
+template <bool FULL>
+struct Q6Walk {  // the passes of a wave's rows, in memory order
+    const uint8_t *src;
+    size_t row_skip;  // bytes from the end of one of the wave's rows to the start of its next
+    int pass, npass, last_bytes;
+    Q6Pieces full, last;
+    WD_DEV bool is_last() const { return pass == npass - 1; }
+    WD_DEV const Q6Pieces &pieces() const { return (FULL || !is_last()) ? full : last; }
+    WD_DEV void advance() {
+        src = uniform_ptr(src + ((FULL || !is_last()) ? 1680 : last_bytes) + (is_last() ? row_skip : 0));
+        pass = is_last() ? 0 : pass + 1;
+    }
+};
+
+template <bool PART, bool ALIGNED, bool FULL>
+__global__ __launch_bounds__(256) void k_gemv_q6k(const uint8_t *__restrict__ w, int rows, int cols,
                                                    const int8_t *__restrict__ act_qs, const float *__restrict__ act_d,
                                                    const int16_t *__restrict__ act_bsums, float *__restrict__ out,
                                                    int32_t *__restrict__ partials) {
     extern __shared__ __align__(16) uint8_t q6_lds[];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int nb = cols >> 8;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nb = cols >> 8, npass = (nb + 7) >> 3;
+    const int aq_bytes = nb * kQ6ActStride;
     int8_t *aq = reinterpret_cast<int8_t *>(q6_lds);
-    float *ad = reinterpret_cast<float *>(q6_lds + cols);
-    int16_t *ab = reinterpret_cast<int16_t *>(q6_lds + cols + ((nb * 4 + 15) & ~15));
-    uint8_t *stage = q6_lds + cols + ((nb * 4 + 15) & ~15) + nb * 32 + wave * 1696;
-    for (int i = threadIdx.x; i < cols / 16; i += 256) reinterpret_cast<uint4 *>(aq)[i] = reinterpret_cast<const uint4 *>(act_qs)[i];
+    float *ad = reinterpret_cast<float *>(q6_lds + aq_bytes);
+    int16_t *ab = reinterpret_cast<int16_t *>(q6_lds + aq_bytes + ((nb * 4 + 15) & ~15));
+    uint8_t *stage = q6_lds + aq_bytes + ((nb * 4 + 15) & ~15) + nb * 32 + wave * kQ6StageBytes;
+    const size_t rb = static_cast<size_t>(nb) * 210;
+    // the waves of the grid take the rows in turn, so that the waves running together read neighbouring rows
+    const int n_waves = gridDim.x * 4;
+    const int r0 = blockIdx.x * 4 + wave;
+    const int n_rows = r0 < rows ? (rows - r0 + n_waves - 1) / n_waves : 0;
+    Q6Walk<FULL> fetch;  // runs one pass ahead of `work`
+    fetch.src = uniform_ptr(w + static_cast<size_t>(min(r0, rows - 1)) * rb);  // a wave without rows asks for the last one
+    fetch.row_skip = static_cast<size_t>(n_waves - 1) * rb;
+    fetch.pass = 0, fetch.npass = npass, fetch.last_bytes = (nb - 8 * (npass - 1)) * 210;
+    fetch.full = q6k_pieces(1680, lane), fetch.last = q6k_pieces(fetch.last_bytes, lane);
+    Q6Walk<FULL> work = fetch;
+    Q6Fetch fa = q6k_fetch<ALIGNED>(fetch.src, fetch.pieces()), fb;
+    for (int i = threadIdx.x; i < cols / 16; i += 256)  // 16 words of 16 bytes per super-block
+        reinterpret_cast<uint4 *>(aq + (i >> 4) * kQ6ActStride)[i & 15] = reinterpret_cast<const uint4 *>(act_qs)[i];
     for (int i = threadIdx.x; i < nb; i += 256) ad[i] = act_d[i];
     for (int i = threadIdx.x; i < nb * 8; i += 256) reinterpret_cast<uint32_t *>(ab)[i] = reinterpret_cast<const uint32_t *>(act_bsums)[i];
     __syncthreads();
-    const size_t rb = static_cast<size_t>(nb) * 210;
-    const long long r0 = (static_cast<long long>(blockIdx.x) * 4 + wave) * rows_per_wave;
-    for (int i = 0; i < rows_per_wave; ++i) {
-        const long long r = r0 + i;
-        if (r >= rows) break;  // wave-uniform
-        const float y = q6k_row<PART, ALIGNED>(w + static_cast<size_t>(r) * rb, nb, aq, ad, ab, lane, stage,
-                                               PART ? partials + static_cast<size_t>(r) * nb * 8 : nullptr);
-        if (lane == 0) out[r] = y;
+    if (n_rows <= 0) return;  // wave-uniform
+    const int items = n_rows * npass;
+    long long r = r0;
+    float acc = 0.0f;
+    auto step = [&](const Q6Fetch &cur) {
+        wave_lds_fence();  // the previous pass has been read
+        q6k_stage(stage, cur, work.pieces());
+        wave_lds_fence();
+        acc = q6k_pass<PART, FULL>(stage, 8 * work.pass, nb, aq, ad, ab, lane, acc, PART ? partials + static_cast<size_t>(r) * nb * 8 : nullptr);
+        if (work.is_last()) {
+            const float y = q6k_close(acc);
+            if (lane == 15) out[r] = y;
+            r += n_waves;
+        }
+        work.advance();
+    };
+    // Two register sets take turns, so that the request for the next pass stays in flight while this one is worked on.
+    // Every turn issues its three requests (after the wave's last pass: the same pass again, not used), so that the
+    // count of requests in flight does not depend on the path taken.
+    for (int t = 0; t < items; t += 2) {
+        if (t + 1 < items) fetch.advance();
+        fb = q6k_fetch<ALIGNED>(fetch.src, fetch.pieces());
+        step(fa);
+        if (t + 1 >= items) break;
+        if (t + 2 < items) fetch.advance();
+        fa = q6k_fetch<ALIGNED>(fetch.src, fetch.pieces());
+        step(fb);
     }
 }
 

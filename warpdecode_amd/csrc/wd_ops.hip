@@ -247,20 +247,20 @@ int wd_gemv_q6_k_q8_k_f32(const uint8_t *d_w, int rows, int cols, const int8_t *
     const bool aligned = reinterpret_cast<uintptr_t>(d_w) % 16 == 0 && nb % 8 == 0;
     // enough rows per wave to pay for staging the activation, few enough to keep every compute unit busy
     int rpw = rows / (4 * 2048);
-    rpw = rpw < 1 ? 1 : (rpw > 16 ? 16 : rpw);
+    rpw = rpw < 1 ? 1 : (rpw > 10 ? 10 : rpw);
     const unsigned wgs = static_cast<unsigned>((static_cast<long long>(rows) + 4LL * rpw - 1) / (4LL * rpw));
-    const size_t lds = static_cast<size_t>(cols) + ((nb * 4 + 15) & ~15) + static_cast<size_t>(nb) * 32 + 4 * 1696;
+    const size_t lds = static_cast<size_t>(nb) * kQ6ActStride + ((nb * 4 + 15) & ~15) + static_cast<size_t>(nb) * 32 + 4 * kQ6StageBytes;
     hipStream_t st = as_stream(stream);
+    const bool full = nb % 8 == 0;
+    auto launch = [&](auto kernel) { kernel<<<wgs, 256, lds, st>>>(d_w, rows, cols, d_act_qs, d_act_scales, d_act_bsums, d_out, d_partials); };
     if (d_partials) {
-        if (aligned)
-            k_gemv_q6k<true, true><<<wgs, 256, lds, st>>>(d_w, rows, cols, rpw, d_act_qs, d_act_scales, d_act_bsums, d_out, d_partials);
-        else
-            k_gemv_q6k<true, false><<<wgs, 256, lds, st>>>(d_w, rows, cols, rpw, d_act_qs, d_act_scales, d_act_bsums, d_out, d_partials);
+        if (aligned) launch(k_gemv_q6k<true, true, true>);  // aligned implies whole passes
+        else if (full) launch(k_gemv_q6k<true, false, true>);
+        else launch(k_gemv_q6k<true, false, false>);
     } else {
-        if (aligned)
-            k_gemv_q6k<false, true><<<wgs, 256, lds, st>>>(d_w, rows, cols, rpw, d_act_qs, d_act_scales, d_act_bsums, d_out, nullptr);
-        else
-            k_gemv_q6k<false, false><<<wgs, 256, lds, st>>>(d_w, rows, cols, rpw, d_act_qs, d_act_scales, d_act_bsums, d_out, nullptr);
+        if (aligned) launch(k_gemv_q6k<false, true, true>);
+        else if (full) launch(k_gemv_q6k<false, false, true>);
+        else launch(k_gemv_q6k<false, false, false>);
     }
     WD_LAUNCH_CHECK();
     return WD_OK;

@@ -356,91 +356,135 @@ WD_DEV float iq_row_q8k(const uint8_t *row, int nb, const IqTables &t, const int
 
 // ---- Q6_K x Q8_K (the output head) --------------------------------------------------------------------
 // src/lowbit.cuh:2510-2612.  A super-block is 210 bytes: ql[128] (low four bits of the codes), qh[64] (high two bits),
-// sixteen int8 scales, fp16 d.  Lane (is = lane >> 3, sb = lane & 7) takes the 32-value chunk `is` of super-block
-// 8 * pass + sb: half = is >> 2, sub = is & 3; code byte l = (ql[64 half + 32 (sub & 1) + l] low or high nibble by
-// sub < 2) | ((qh[32 half + l] >> 2 sub) & 3) << 4; the chunk's low 16 bytes use scale 2 is, the high 16 scale
-// 2 is + 1.  Its eight dwords are the eight float lanes of the reference (lane m = bytes 4m..4m+3): p[m] =
-// scale * dot4.  After the fold over the eight chunk lanes, lane (m, sb) holds lane sum m of super-block sb, takes
-// the -32 correction ((bsums[2m] scale[2m] + bsums[2m+1] scale[2m+1]) << 5 - it has read exactly that scale pair
-// for its own chunk) and runs chain m along the super-blocks, as the IQ rows do.
-// A pass (eight super-blocks, 1680 bytes) is fetched with one or two 16-byte loads per lane into LDS and the fields
-// are picked from there; blocks are 2-byte aligned, so the 32-byte runs are read as nine aligned dwords and shifted
-// by two bytes in the odd super-blocks.  ALIGNED: the row starts on a 16-byte boundary.
-// stage: 1696 bytes of LDS owned by the wave, 16-byte aligned.
-template <bool PART, bool ALIGNED>
-WD_DEV float q6k_row(const uint8_t *row, int nb, const int8_t *act_qs, const float *act_d, const int16_t *act_bsums, int lane,
-                     uint8_t *stage, int32_t *partials) {
-    const int is = lane >> 3, sbl = lane & 7;
-    const bool first = sbl == 0;
-    const int half = is >> 2, sub = is & 3;
-    float acc = 0.0f;
-    for (int base = 0; base < nb; base += 8) {
-        const int n_here = min(8, nb - base);
-        const int bytes = n_here * 210, words = bytes >> 4, tail = (bytes & 15) >> 1;  // full 16-byte words, then 2-byte pieces
-        const uint8_t *src = row + static_cast<size_t>(base) * 210;
-        uint4 u0 = make_uint4(0, 0, 0, 0), u1 = u0;
-        uint16_t t16 = 0;
-        if (lane < words) u0 = ALIGNED ? gld_u128_aligned(src + 16 * lane) : gld_u128(src + 16 * lane);
-        if (lane + 64 < words) u1 = ALIGNED ? gld_u128_aligned(src + 16 * (lane + 64)) : gld_u128(src + 16 * (lane + 64));
-        if (lane < tail) t16 = gld_u16(src + 16 * words + 2 * lane);
-        wave_lds_fence();  // the previous pass has been read
-        if (lane < words) reinterpret_cast<uint4 *>(stage)[lane] = u0;
-        if (lane + 64 < words) reinterpret_cast<uint4 *>(stage)[lane + 64] = u1;
-        if (lane < tail) reinterpret_cast<uint16_t *>(stage + 16 * words)[lane] = t16;
-        wave_lds_fence();
-        const int sb = base + sbl;
-        const bool on = sb < nb;
-        int p[8];
-        int sc0 = 0, sc1 = 0;
-        float ds = 0.0f;
-        if (on) {
-            const uint8_t *blk = stage + 210 * sbl;
-            const uint32_t sh = (sbl & 1) ? 2u : 0u;  // 210 * sbl is 2 (mod 4) in the odd super-blocks of a pass
-            const uint32_t *lw = reinterpret_cast<const uint32_t *>(blk + 64 * half + 32 * (sub & 1) - sh);
-            const uint32_t *hw = reinterpret_cast<const uint32_t *>(blk + 128 + 32 * half - sh);
-            uint32_t lr[9], hr[9];
+// sixteen int8 scales, fp16 d.  Value 128 h + 32 s + l (h = half, s = 0..3, l = 0..31) has the code
+// (ql[64 h + 32 (s & 1) + l] low nibble for s < 2, high nibble otherwise) | ((qh[32 h + l] >> 2 s) & 3) << 4 and the scale
+// 2 (4 h + s) + (l >> 4).  The reference keeps eight float lanes per row (lane m = bytes 4m..4m+3 of every 32-value
+// chunk): the integer lane sum of a super-block is sum over chunks of scale * dot4, minus the -32 correction
+// (bsums[2m] scale[2m] + bsums[2m+1] scale[2m+1]) << 5, then one fma(d_w d_x, float(sum), acc_m) per super-block.
+//
+// Lane layout: lane = 16 (j >> 1) + 2 sb + (j & 1) with j = 4 h + q (q = 0..3) and sb = 0..7; the lane works on
+// super-block 8 * pass + sb and takes bytes 8q..8q+7 of the three 32-byte runs of half h (two of ql, one of qh): these
+// hold bytes 8q..8q+7 of all four chunks of the half, that is float lanes 2q and 2q+1, with compile-time shifts.
+// v_permlane32_swap joins the two halves (lane and lane + 32 differ in h only) so that lanes 0..31 hold lane sum 2q
+// and lanes 32..63 lane sum 2q+1: lane (j, sb) carries float lane m = 2q + h.  The eight super-blocks of a chain sit
+// two lanes apart inside one 16-lane row, so the fma chain is DPP row_shr:2, the two chains of a row start in its
+// lanes 0 and 1 (where row_shr:2 has no source and leaves the carry in place), and the carry between passes is
+// row_shl:14.
+// A pass (eight super-blocks, 1680 bytes) is fetched with two 16-byte loads per lane and copied to LDS as it lies in
+// memory; blocks are only 2-byte aligned there, so the 8-byte fields are read as three aligned dwords and shifted by two
+// bytes in the odd super-blocks.
+constexpr int kQ6StageBytes = 1696;
+// The activation's quants lie in LDS with 288 bytes per super-block: the eight super-blocks that the lanes of a wave
+// read together then fall into different banks (at 256 bytes they would all share one).
+constexpr int kQ6ActStride = 288;
+
+struct Q6Fetch {
+    uint4 u0, u1;
+    uint32_t t16;
+};
+// Where a lane's pieces of a pass of `bytes` (a multiple of 210, at most 1680) lie, relative to the pass: two 16-byte
+// words (at least 13 exist; lanes past the end repeat the last one) and a 2-byte piece of the tail.
+struct Q6Pieces {
+    uint32_t off0, off1, off_tail;
+    bool has_tail;  // false: the pass is a whole number of 16-byte words (off_tail is 0 then, and its piece is not kept)
+};
+WD_DEV Q6Pieces q6k_pieces(int bytes, int lane) {
+    const int words = bytes >> 4, tail = (bytes & 15) >> 1;
+    Q6Pieces p;
+    p.off0 = 16 * min(lane, words - 1), p.off1 = 16 * min(lane + 64, words - 1);
+    p.has_tail = tail != 0;
+    p.off_tail = tail ? 16 * words + 2 * min(lane, tail - 1) : 0;
+    return p;
+}
+template <bool ALIGNED>
+WD_DEV Q6Fetch q6k_fetch(const uint8_t *src, const Q6Pieces &p) {
+    Q6Fetch f;
+    f.u0 = ALIGNED ? gld_u128_aligned(src + p.off0) : gld_u128(src + p.off0);
+    f.u1 = ALIGNED ? gld_u128_aligned(src + p.off1) : gld_u128(src + p.off1);
+    f.t16 = gld_u16(src + p.off_tail);  // always three requests, so that the number in flight is known
+    return f;
+}
+WD_DEV void q6k_stage(uint8_t *stage, const Q6Fetch &f, const Q6Pieces &p) {
+    *reinterpret_cast<uint4 *>(stage + p.off0) = f.u0;
+    *reinterpret_cast<uint4 *>(stage + p.off1) = f.u1;
+    if (p.has_tail) *reinterpret_cast<uint16_t *>(stage + p.off_tail) = static_cast<uint16_t>(f.t16);
+}
+// Eight bytes of LDS at p = q + sh, q on a 4-byte boundary and sh = 0 or 2 (per lane).
+WD_DEV uint2 lds_u64_shifted(const uint8_t *q, uint32_t sh) {
+    const uint32_t *w = reinterpret_cast<const uint32_t *>(q);
+    const uint32_t w0 = w[0], w1 = w[1], w2 = w[2];
+    return make_uint2(__builtin_amdgcn_alignbyte(w1, w0, sh), __builtin_amdgcn_alignbyte(w2, w1, sh));
+}
+WD_DEV uint32_t lds_u16(const uint8_t *p) { return *reinterpret_cast<const uint16_t *>(p); }
+
+// One pass of a row from the staged bytes (act_qs: LDS, kQ6ActStride bytes per super-block): returns the running float
+// lane after super-blocks base .. base + 7.  acc: the lane's value after the previous pass (any value for base == 0).
+// FULL: the row is a whole number of passes (every lane has a super-block).
+template <bool PART, bool FULL>
+WD_DEV float q6k_pass(const uint8_t *stage, int base, int nb, const int8_t *act_qs, const float *act_d, const int16_t *act_bsums,
+                      int lane, float acc, int32_t *partials) {
+    const int j = ((lane >> 4) << 1) | (lane & 1), sbl = (lane >> 1) & 7, half = j >> 2, q = j & 3;
+    const int m = 2 * q + half;  // the float lane this lane carries once the halves are joined
+    const int sb = base + sbl;
+    const bool on = FULL || sb < nb;
+    const int sbc = FULL ? sb : min(sb, nb - 1);  // lanes past the row's end read in-bounds data and contribute zero
+    const uint8_t *blk = stage + 210 * sbl;
+    const uint32_t sh = (sbl & 1) ? 2u : 0u;  // 210 * sbl is 2 (mod 4) in the odd super-blocks of a pass
+    const uint8_t *fld = blk - sh + 64 * half + 8 * q;
+    const uint2 l0 = lds_u64_shifted(fld, sh), l1 = lds_u64_shifted(fld + 32, sh);
+    const uint2 hh = lds_u64_shifted(fld + 128 - 32 * half, sh);
+    const int8_t *scq = reinterpret_cast<const int8_t *>(blk + 192) + 8 * half + (q >> 1);
+    const int s0 = scq[0], s1 = scq[2], s2 = scq[4], s3 = scq[6];
+    const uint2 *ap = reinterpret_cast<const uint2 *>(act_qs + sbc * kQ6ActStride + half * 128 + 8 * q);
+    const uint2 a0 = ap[0], a1 = ap[4], a2 = ap[8], a3 = ap[12];
+    constexpr uint32_t kLo = 0x0f0f0f0fu, kHi = 0x30303030u;
+    int h0, h1;
+    h0 = __mul24(s0, sdot4((l0.x & kLo) | ((hh.x << 4) & kHi), a0.x, 0));
+    h1 = __mul24(s0, sdot4((l0.y & kLo) | ((hh.y << 4) & kHi), a0.y, 0));
+    h0 += __mul24(s1, sdot4((l1.x & kLo) | ((hh.x << 2) & kHi), a1.x, 0));
+    h1 += __mul24(s1, sdot4((l1.y & kLo) | ((hh.y << 2) & kHi), a1.y, 0));
+    h0 += __mul24(s2, sdot4(((l0.x >> 4) & kLo) | (hh.x & kHi), a2.x, 0));
+    h1 += __mul24(s2, sdot4(((l0.y >> 4) & kLo) | (hh.y & kHi), a2.y, 0));
+    h0 += __mul24(s3, sdot4(((l1.x >> 4) & kLo) | ((hh.x >> 2) & kHi), a3.x, 0));
+    h1 += __mul24(s3, sdot4(((l1.y >> 4) & kLo) | ((hh.y >> 2) & kHi), a3.y, 0));
+    // lanes 0..31 (half 0) take both halves' sum of float lane 2q, lanes 32..63 that of 2q + 1
+    const auto sw = __builtin_amdgcn_permlane32_swap(static_cast<uint32_t>(h0), static_cast<uint32_t>(h1), false, false);
+    int lane_sum = static_cast<int>(sw[0] + sw[1]);
+    const uint32_t pair = lds_u16(blk + 192 + 2 * m);
+    const uint32_t bs = *reinterpret_cast<const uint32_t *>(act_bsums + sbc * 16 + 2 * m);
+    const int c0 = static_cast<int8_t>(pair & 0xffu), c1 = static_cast<int8_t>(pair >> 8);
+    const int b0 = static_cast<int16_t>(bs & 0xffffu), b1 = static_cast<int16_t>(bs >> 16);
+    lane_sum -= static_cast<int>(static_cast<uint32_t>(b0 * c0 + b1 * c1) << 5);
+    if (PART && on) partials[sb * 8 + m] = lane_sum;
+    const float pf = on ? static_cast<float>(lane_sum) : 0.0f;
+    const float ds = on ? h2f(static_cast<uint16_t>(lds_u16(blk + 208))) * act_d[sbc] : 0.0f;
+    // `up` is the chain value of the super-block before the lane's own.  The chains start in lanes 0 and 1 of every row
+    // with the carry of the previous pass (row_shl:14 reaches their last lanes); row_shr:2 has no source there, so it
+    // leaves the carry in place while the other lanes converge one super-block per step.  Lanes past the row's end pass
+    // the value through unchanged, fma(0, 0, up) == up.
+    float up = dpp_f<kDppShl14>(0.0f, acc);
+    up = base == 0 ? 0.0f : up;
+    float v = __builtin_fmaf(ds, pf, up);
 #pragma unroll
-            for (int j = 0; j < 9; ++j) lr[j] = lw[j], hr[j] = hw[j];
-            const uint32_t pair = *reinterpret_cast<const uint16_t *>(blk + 192 + 2 * is);
-            sc0 = static_cast<int8_t>(pair & 0xffu), sc1 = static_cast<int8_t>(pair >> 8);
-            const float dw = h2f(*reinterpret_cast<const uint16_t *>(blk + 208));
-            const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + is * 32);
-            const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + is * 32 + 16);
-            const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
-            const uint32_t low_shift = (sub < 2) ? 0u : 4u, high_shift = 2u * sub;
-#pragma unroll
-            for (int m = 0; m < 8; ++m) {
-                const uint32_t lo = __builtin_amdgcn_alignbyte(lr[m + 1], lr[m], sh);
-                const uint32_t hi = __builtin_amdgcn_alignbyte(hr[m + 1], hr[m], sh);
-                const uint32_t code = ((lo >> low_shift) & 0x0f0f0f0fu) | (((hi >> high_shift) & 0x03030303u) << 4);
-                p[m] = __mul24(m < 4 ? sc0 : sc1, sdot4(code, a[m], 0));
-            }
-            ds = dw * act_d[sb];
-        } else {
-#pragma unroll
-            for (int m = 0; m < 8; ++m) p[m] = 0;
-        }
-        int lane_sum = reduce_scatter_ib(p, lane);  // lane (m = is, sb): float lane m of super-block sb
-        if (on) {
-            const uint32_t bs = *reinterpret_cast<const uint32_t *>(act_bsums + sb * 16 + 2 * is);
-            const int b0 = static_cast<int16_t>(bs & 0xffffu), b1 = static_cast<int16_t>(bs >> 16);
-            lane_sum -= static_cast<int>(static_cast<uint32_t>(b0 * sc0 + b1 * sc1) << 5);
-            if (PART) partials[sb * 8 + is] = lane_sum;
-        }
-        const float pf = on ? static_cast<float>(lane_sum) : 0.0f;
-        // carry of the previous pass: last lane of the group -> first lane (lanes past the row's end pass the
-        // accumulator through unchanged, fma(0, 0, acc) == acc)
-        const float carry = dpp_f<kDppShl7>(0.0f, acc);
-        float v = __builtin_fmaf(ds, pf, base == 0 ? 0.0f : carry);
-#pragma unroll
-        for (int s = 1; s < 8; ++s) {
-            const float up = dpp_f<kDppShr1>(0.0f, v);
-            const float nxt = __builtin_fmaf(ds, pf, up);
-            v = first ? v : nxt;
-        }
-        acc = v;
+    for (int s = 1; s < 8; ++s) {
+        up = dpp_f<kDppShr2>(up, v);
+        v = __builtin_fmaf(ds, pf, up);
     }
-    return close_lanes8_strided(acc);
+    return v;
+}
+
+// ggml's closing tree over the eight float lanes, ((m0+m4)+(m2+m6)) + ((m1+m5)+(m3+m7)); float lane m = 2q + h ends in
+// lane 16 (2 h + (q >> 1)) + 14 + (q & 1): m0 m2 in lanes 14 15, m4 m6 in 30 31, m1 m3 in 46 47, m5 m7 in 62 63.
+// Swapping 16-lane rows adds m0+m4 | m2+m6 (lanes 14 15) and m1+m5 | m3+m7 (lanes 46 47), row_shr:1 adds the
+// neighbours, swapping the wave's halves adds the two sides.  The result is valid in lane 15.
+WD_DEV float q6k_close(float v) {
+    const uint32_t x = __builtin_bit_cast(uint32_t, v);
+    const auto rows = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+    const float s = __builtin_bit_cast(float, static_cast<uint32_t>(rows[0])) + __builtin_bit_cast(float, static_cast<uint32_t>(rows[1]));
+    const float t = dpp_f<kDppShr1>(0.0f, s) + s;
+    const uint32_t y = __builtin_bit_cast(uint32_t, t);
+    const auto halves = __builtin_amdgcn_permlane32_swap(y, y, false, false);
+    return __builtin_bit_cast(float, static_cast<uint32_t>(halves[0])) + __builtin_bit_cast(float, static_cast<uint32_t>(halves[1]));
 }
 
 // ---- Q8_0 (and Q4_0 / IQ4_NL codes) x Q8_0 ------------------------------------------------
