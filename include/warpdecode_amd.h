@@ -214,6 +214,23 @@ unsigned long long *wd_moe_scratch_trace(wd_moe_scratch *s, int wg);
 int wd_moe_layer_f32(const wd_moe_layer *layer, const float *d_x, float *d_out, wd_moe_scratch *scratch,
                      unsigned flags, void *stream);
 
+/* The hyper-connection combine that consumes the layer's output: residual is [hc][hidden] and stream c receives
+ * branch * (2 * sigmoid(inject[c] * (1 / hc))), the sigmoid through glibc's expf, every step one rounded float operation;
+ * round_half stores the sums rounded through half (the reference's legacy residual lifetime).
+ * wd_hc_combine_f32: branch = block_out (the finished layer output).
+ * reference: run_qwen38_hc_combine_f32_block_f32_inject, src/qwen38_hc.cuh:2530-2570.
+ * wd_hc_combine_moe_f32: branch = routed + shared * shared_gate[0]; shared_is_half: d_shared holds half bits (as the
+ * reference's scratch does), else floats.  reference: run_qwen38_hc_combine_moe_f32_inject, src/qwen38_hc.cuh:2241-2263, :2587-2600.
+ * wd_moe_layer_hc_f32: wd_moe_layer_f32 followed by wd_hc_combine_f32 on its output, the combine folded into the layer's
+ * last dispatch (no further launch).  d_residual must not be written by other work while the call runs; the layer's
+ * input d_x may be computed from it beforehand.  reference sequence: src/qwen38_forward.cuh:3330-3371. */
+int wd_hc_combine_f32(float *d_residual, const float *d_block_out, const float *d_inject, int hidden, int hc, int round_half,
+                      void *stream);
+int wd_hc_combine_moe_f32(float *d_residual, const float *d_routed, const void *d_shared, int shared_is_half,
+                          const float *d_shared_gate, const float *d_inject, int hidden, int hc, int round_half, void *stream);
+int wd_moe_layer_hc_f32(const wd_moe_layer *layer, const float *d_x, float *d_out, float *d_residual, const float *d_inject,
+                        int hc, int round_half, wd_moe_scratch *scratch, unsigned flags, void *stream);
+
 /* The shared expert alone: sigmoid(shared_gate_inp . x) into the scratch's shared_gate view and the Q8_0
  * gate/up -> SwiGLU -> Q8_0 -> down chain into its down_f32 view; only the shared_* fields, hidden and
  * expert_ffn of `layer` are read.  For callers that keep the reference's three calls (routed, shared,

@@ -79,6 +79,19 @@ def _load():
         getattr(lib, n).argtypes = [C.c_float]
     lib.wdo_dot_f32.restype = C.c_float
     lib.wdo_dot_f32.argtypes = [_f32p, _f32p, C.c_int]
+    for n in ("wdo_expf_glibc", "wdo_sigmoid_exact", "wdo_round_half"):
+        getattr(lib, n).restype = C.c_float
+        getattr(lib, n).argtypes = [C.c_float]
+    for n in ("wdo_expf_glibc_n", "wdo_libm_expf_n", "wdo_round_half_n"):
+        getattr(lib, n).restype = None
+        getattr(lib, n).argtypes = [_f32p, C.c_int, _f32p]
+    for n in ("wdo_moe_branch_f32", "wdo_residual_add_f32"):
+        getattr(lib, n).restype = C.c_float
+        getattr(lib, n).argtypes = [C.c_float] * 3
+    lib.wdo_hc_combine_f32.restype = None
+    lib.wdo_hc_combine_f32.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+    lib.wdo_hc_combine_moe_f32.restype = None
+    lib.wdo_hc_combine_moe_f32.argtypes = [_f32p, _f32p, C.c_void_p, C.c_int, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
     lib.wdo_router_logits.argtypes = [_f32p, _f32p, C.c_int, C.c_int, _f32p]
     lib.wdo_softmax_row.argtypes = [_f32p, C.c_int, _f32p]
     lib.wdo_router_select.argtypes = [_f32p, C.c_int, C.c_int, C.c_float, C.POINTER(C.c_int), _f32p]
@@ -196,6 +209,51 @@ def silu_ggml(x):
 
 def sigmoid_ggml(x):
     return np.float32(lib().wdo_sigmoid_ggml(float(x)))
+
+
+def _map_f32(name, x):
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    out = np.empty_like(x)
+    getattr(lib(), name)(_ptr(x, _f32p), x.size, _ptr(out, _f32p))
+    return out
+
+
+def expf_glibc(x):
+    return _map_f32("wdo_expf_glibc_n", x)
+
+
+def libm_expf(x):
+    return _map_f32("wdo_libm_expf_n", x)
+
+
+def round_half(x):
+    return _map_f32("wdo_round_half_n", x)
+
+
+def sigmoid_exact(x):
+    return np.float32(lib().wdo_sigmoid_exact(float(x)))
+
+
+def hc_combine(residual, block_out, inject, round_half=False):
+    """residual [hc][hidden] (a copy is updated and returned), block_out [hidden], inject [hc]."""
+    res = np.array(residual, dtype=np.float32, order="C", copy=True)
+    hc, hidden = res.shape
+    lib().wdo_hc_combine_f32(_ptr(res, _f32p), _ptr(np.ascontiguousarray(block_out, np.float32), _f32p),
+                             _ptr(np.ascontiguousarray(inject, np.float32), _f32p), hidden, hc, int(round_half))
+    return res
+
+
+def hc_combine_moe(residual, routed, shared, shared_gate, inject, round_half=False):
+    """shared: float32 [hidden], or uint16 [hidden] holding half bits."""
+    res = np.array(residual, dtype=np.float32, order="C", copy=True)
+    hc, hidden = res.shape
+    shared = np.ascontiguousarray(shared)
+    assert shared.dtype in (np.float32, np.uint16)
+    lib().wdo_hc_combine_moe_f32(_ptr(res, _f32p), _ptr(np.ascontiguousarray(routed, np.float32), _f32p),
+                                 shared.ctypes.data_as(C.c_void_p), int(shared.dtype == np.uint16),
+                                 _ptr(np.ascontiguousarray(shared_gate, np.float32).reshape(1), _f32p),
+                                 _ptr(np.ascontiguousarray(inject, np.float32), _f32p), hidden, hc, int(round_half))
+    return res
 
 
 def dot_f32(a, b):
@@ -339,6 +397,12 @@ def ref():
             getattr(r, n).argtypes = [C.c_float]
         r.wdref_dot_f32.restype = C.c_float
         r.wdref_dot_f32.argtypes = [_f32p, _f32p, C.c_int]
+        if hasattr(r, "wdref_round_half"):
+            r.wdref_round_half.restype = C.c_float
+            r.wdref_round_half.argtypes = [C.c_float]
+            for n in ("wdref_moe_branch_f32", "wdref_residual_add_f32"):
+                getattr(r, n).restype = C.c_float
+                getattr(r, n).argtypes = [C.c_float] * 3
         r.wdref_quantize_q8_0.argtypes = [_f32p, C.c_int, _i8p, _u16p]
         r.wdref_quantize_q8_K.argtypes = [_f32p, C.c_int, _i8p, _f32p, _i16p]
         r.wdref_row.restype = C.c_float

@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "qwen38_cpu_moe.cuh"
+#include "qwen38_precision.hpp"
 
 using namespace wd::cpu_moe;
 
@@ -67,6 +68,10 @@ float wdref_exp(float x) { return ggml_avx2_exp_f32(x); }
 float wdref_silu(float x) { return silu_ggml(x); }
 float wdref_sigmoid(float x) { return sigmoid_ggml(x); }
 float wdref_dot_f32(const float *a, const float *b, int n) { return dot_f32_avx2(a, b, n); }
+// src/qwen38_precision.hpp:32-55 (the host branches)
+float wdref_moe_branch_f32(float routed, float shared, float gate) { return wd::q38_moe_branch_f32(routed, shared, gate); }
+float wdref_residual_add_f32(float residual, float branch, float weight) { return wd::q38_residual_add_f32(residual, branch, weight); }
+float wdref_round_half(float value) { return wd::q38_round_half(value); }
 
 void wdref_quantize_q8_0(const float *x, int n, int8_t *qs, uint16_t *d) {
     std::vector<q8_0> y(static_cast<size_t>(n / 32));

@@ -46,6 +46,7 @@
 #include <string.h>
 
 #include "../warpdecode_amd/csrc/wd_codebooks.inc"
+#include "../warpdecode_amd/csrc/wd_exp2f_table.inc"
 
 /* ------------------------------------------------------------------------- */
 /* Codebooks                                                                 */
@@ -560,6 +561,106 @@ float wdo_exp_ggml(float x) {
 float wdo_silu_ggml(float x) { return x / (1.0f + wdo_exp_ggml(-x)); }
 
 float wdo_sigmoid_ggml(float x) { return 1.0f / (1.0f + wdo_exp_ggml(-x)); }
+
+/* ------------------------------------------------------------------------- */
+/* Hyper-connection combine of the FFN branch (the consumer of the layer)     */
+/* ------------------------------------------------------------------------- */
+static const uint64_t k_exp2f_tab[32] = WD_EXP2F_TABLE;
+
+static inline uint64_t f64_bits(double v) {
+    uint64_t b;
+    memcpy(&b, &v, 8);
+    return b;
+}
+static inline double bits_f64(uint64_t b) {
+    double v;
+    memcpy(&v, &b, 8);
+    return v;
+}
+
+/* src/qwen38_exact_math.cuh:136-166.  Every step is one rounded double operation (this file is built with
+ * -ffp-contract=off). */
+float wdo_expf_glibc(float x) {
+    const double shift = 0x1.8p+52, invln2n = 0x1.71547652b82fep+0 * 32.0;
+    const double c0 = 0x1.c6af84b912394p-5 / 32.0 / 32.0 / 32.0, c1 = 0x1.ebfce50fac4f3p-3 / 32.0 / 32.0, c2 = 0x1.62e42ff0c52d6p-1 / 32.0;
+    const uint32_t ix = f32_bits(x), abstop = (ix >> 20) & 0x7ffu;
+    if (abstop >= (0x42b00000u >> 20)) { /* |x| >= 88, infinities, NaN */
+        if (ix == 0xff800000u) return 0.0f;
+        if (abstop >= 0x7f8u) return x + x;
+        if (x > 0x1.62e42ep6f) return 0x1p97f * 0x1p97f;
+        if (x < -0x1.9fe368p6f) return 0x1p-95f * 0x1p-95f;
+    }
+    const double z = invln2n * (double)x;
+    const double kd_shift = z + shift;
+    const uint64_t ki = f64_bits(kd_shift);
+    const double kd = kd_shift - shift;
+    const double r = z - kd;
+    const uint64_t t = k_exp2f_tab[ki % 32u] + (ki << 47);
+    const double s = bits_f64(t);
+    const double p = c0 * r + c1;
+    const double r2 = r * r;
+    double y = c2 * r + 1.0;
+    y = p * r2 + y;
+    y = y * s;
+    return (float)y;
+}
+
+void wdo_expf_glibc_n(const float *x, int n, float *out) {
+    for (int i = 0; i < n; ++i) out[i] = wdo_expf_glibc(x[i]);
+}
+void wdo_libm_expf_n(const float *x, int n, float *out) {
+    for (int i = 0; i < n; ++i) out[i] = expf(x[i]);
+}
+
+float wdo_sigmoid_exact(float x) { return 1.0f / (1.0f + wdo_expf_glibc(-x)); }
+
+/* src/qwen38_precision.hpp:40-55 (the host branch; the device branch is the hardware conversion) */
+float wdo_round_half(float value) {
+    if (!isfinite(value) || value == 0.0f) return value;
+    const float magnitude = fabsf(value);
+    if (magnitude >= 65520.0f) return copysignf(INFINITY, value);
+    if (magnitude < ldexpf(1.0f, -14)) return copysignf(ldexpf(nearbyintf(ldexpf(magnitude, 24)), -24), value);
+    const float quantum = ldexpf(1.0f, ilogbf(magnitude) - 10);
+    return copysignf(nearbyintf(magnitude / quantum) * quantum, value);
+}
+
+void wdo_round_half_n(const float *x, int n, float *out) {
+    for (int i = 0; i < n; ++i) out[i] = wdo_round_half(x[i]);
+}
+
+float wdo_moe_branch_f32(float routed, float shared, float gate) {
+    const float weighted = shared * gate;
+    return routed + weighted;
+}
+float wdo_residual_add_f32(float residual, float branch, float weight) {
+    const float weighted = branch * weight;
+    return residual + weighted;
+}
+
+static float hc_weight(float inject, int hc) { return 2.0f * wdo_sigmoid_exact(inject * (1.0f / (float)hc)); }
+
+void wdo_hc_combine_f32(float *residual, const float *block_out, const float *inject, int hidden, int hc, int round_half) {
+    for (int c = 0; c < hc; ++c) {
+        const float w = hc_weight(inject[c], hc);
+        for (int h = 0; h < hidden; ++h) {
+            const float v = wdo_residual_add_f32(residual[(size_t)c * hidden + h], block_out[h], w);
+            residual[(size_t)c * hidden + h] = round_half ? wdo_round_half(v) : v;
+        }
+    }
+}
+
+void wdo_hc_combine_moe_f32(float *residual, const float *routed, const void *shared, int shared_is_half, const float *shared_gate,
+                            const float *inject, int hidden, int hc, int round_half) {
+    for (int c = 0; c < hc; ++c) {
+        const float w = hc_weight(inject[c], hc);
+        for (int h = 0; h < hidden; ++h) {
+            const float sh = shared_is_half ? wdo_f16_to_f32(((const uint16_t *)shared)[h]) : ((const float *)shared)[h];
+            const float branch = wdo_moe_branch_f32(routed[h], sh, shared_gate[0]);
+            const float v = wdo_residual_add_f32(residual[(size_t)c * hidden + h], branch, w);
+            residual[(size_t)c * hidden + h] = round_half ? wdo_round_half(v) : v;
+        }
+    }
+}
 
 /* ------------------------------------------------------------------------- */
 /* F32 dot in the 4 x 8 accumulator order                                     */

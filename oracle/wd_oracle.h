@@ -88,6 +88,26 @@ float wdo_exp_ggml(float x);
 float wdo_silu_ggml(float x);
 float wdo_sigmoid_ggml(float x);
 
+/* The consumer of the layer's output: the hyper-connection combine of the FFN branch.
+ * wdo_expf_glibc: glibc's expf (table of 2^(i/32), cubic in double, no fused operations), the routine the reference
+ * ports to the device in src/qwen38_exact_math.cuh:136-166; wdo_sigmoid_exact: 1 / (1 + expf(-x)), :195-198.
+ * wdo_round_half: IEEE float -> half -> float, src/qwen38_precision.hpp:40-55.
+ * wdo_moe_branch_f32 / wdo_residual_add_f32: one rounded multiply and one rounded add each, src/qwen38_precision.hpp:32-38.
+ * wdo_hc_combine_f32: residual[c][h] += block_out[h] * (2 * sigmoid(inject[c] * (1 / hc))) for the hc residual streams,
+ * src/qwen38_hc.cuh:2530-2547; wdo_hc_combine_moe_f32 takes the branch apart as routed + shared * gate, :2241-2263
+ * (shared_is_half: the shared expert's output is given as half bits, as the reference holds it, else as float). */
+float wdo_expf_glibc(float x);
+void wdo_expf_glibc_n(const float *x, int n, float *out);  /* the same over an array */
+void wdo_libm_expf_n(const float *x, int n, float *out);   /* the host C library's expf, for the pin tests */
+float wdo_sigmoid_exact(float x);
+void wdo_round_half_n(const float *x, int n, float *out);
+float wdo_round_half(float value);
+float wdo_moe_branch_f32(float routed, float shared, float gate);
+float wdo_residual_add_f32(float residual, float branch, float weight);
+void wdo_hc_combine_f32(float *residual, const float *block_out, const float *inject, int hidden, int hc, int round_half);
+void wdo_hc_combine_moe_f32(float *residual, const float *routed, const void *shared, int shared_is_half, const float *shared_gate,
+                            const float *inject, int hidden, int hc, int round_half);
+
 /* src/qwen38_cpu_moe.cuh:847-871 */
 float wdo_dot_f32(const float *a, const float *b, int n);
 

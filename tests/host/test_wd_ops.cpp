@@ -359,6 +359,30 @@ static void gpu_checks() {
                     std::vector<float> fused(H);
                     dout.download(fused.data());
                     CHECK(same_bits(fused.data(), want.data(), H), "token %d layer %d: fused call differs from the oracle", token, l);
+                    // the layer with the hyper-connection combine folded in, and the combine as calls of its own
+                    const int hc = 4;
+                    Qwen38HcF32DebugScratch hcs;
+                    hcs.initialize(H, hc);
+                    std::vector<float> res0(static_cast<size_t>(hc) * H), inject(hc);
+                    for (auto &v : res0) v = r.normal();
+                    for (auto &v : inject) v = 2.0f * r.normal();
+                    check(wd_memcpy_h2d(hcs.inject(), inject.data(), sizeof(float) * hc, nullptr), "inject");
+                    std::vector<float> want_res = res0;
+                    wdo_hc_combine_f32(want_res.data(), want.data(), inject.data(), H, hc, 0);
+                    DeviceFloatArray dres, dres2, dres3;
+                    dres.upload(res0.data(), res0.size()), dres2.upload(res0.data(), res0.size()), dres3.upload(res0.data(), res0.size());
+                    run_qwen38_moe_layer_hc_f32_x(l, dx.data, routers[l], L[l].t_gate, L[l].t_up, L[l].t_down, cache, shared[l], scratch, dout.data,
+                                                  dres.data, hcs, 1.0f, stream);
+                    run_qwen38_hc_combine_f32_block_f32_inject(dres2.data, dout.data, hcs, stream);
+                    run_qwen38_hc_combine_moe_f32_inject(dres3.data, scratch.d_accum(), scratch.down_f32(), scratch.d_shared_gate(), hcs, stream);
+                    check(wd_stream_sync(stream), "sync");
+                    std::vector<float> got_res(res0.size());
+                    dres.download(got_res.data());
+                    CHECK(same_bits(got_res.data(), want_res.data(), got_res.size()), "token %d layer %d: folded combine differs from the oracle", token, l);
+                    dres2.download(got_res.data());
+                    CHECK(same_bits(got_res.data(), want_res.data(), got_res.size()), "token %d layer %d: combine differs from the oracle", token, l);
+                    dres3.download(got_res.data());
+                    CHECK(same_bits(got_res.data(), want_res.data(), got_res.size()), "token %d layer %d: combine from the parts differs from the oracle", token, l);
                 }
             }
         }

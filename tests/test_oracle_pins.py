@@ -538,3 +538,122 @@ def test_q6_k_float_lanes_are_not_a_plain_sum(oracle):
             acc = np.float32(acc + np.float32(dw[sb] * d[sb]) * np.float32(part[r].reshape(-1, 8)[sb].sum()))
         differs += int(acc.view(np.uint32) != y[r].view(np.uint32))
     assert differs > 0
+
+
+# ---- hyper-connection combine of the FFN branch (the consumer of the layer's output) ---------------------------
+def test_exp2f_table_from_decimal_arithmetic():
+    """Entry i is the double nearest to 2^(i/32), minus i << 47 (e_exp2f_data.c of glibc / the ARM optimized routines)."""
+    from decimal import Decimal, getcontext
+    getcontext().prec = 60
+    text = open(os.path.join(os.path.dirname(__file__), "..", "warpdecode_amd", "csrc", "wd_exp2f_table.inc")).read()
+    got = [int(v, 16) for v in re.findall(r"0x([0-9a-f]{16})ull", text)]
+    want = []
+    for i in range(32):
+        bits = np.array([float(Decimal(2) ** (Decimal(i) / Decimal(32)))], np.float64).view(np.uint64)[0]
+        want.append((int(bits) - (i << 47)) & (2 ** 64 - 1))
+    assert got == want
+
+
+def _exp_probe_inputs():
+    rng = synth.rng_for(SEED, 400)
+    edges = np.array([0.0, -0.0, 1.0, -1.0, 88.0, 88.7, 88.72283, 88.72284, 88.8, 89.0, 128.0, -87.0, -87.33655, -103.0,
+                      -103.97, -103.972, -103.98, -104.0, -150.0, 1e-8, -1e-8, 1e-40, np.inf, -np.inf, np.nan, 3.4e38, -3.4e38],
+                     np.float32)
+    near = np.concatenate([np.nextafter(np.float32(v), np.float32(s)).reshape(1) for v in (88.72283, -103.972, -87.33655)
+                           for s in (np.inf, -np.inf)]).astype(np.float32)
+    return np.concatenate([edges, near, rng.uniform(-105.0, 90.0, 2_000_000).astype(np.float32),
+                           rng.normal(0.0, 4.0, 1_000_000).astype(np.float32),
+                           (rng.integers(0, 2 ** 32, 1_000_000, dtype=np.uint64).astype(np.uint32)).view(np.float32)])
+
+
+def test_expf_glibc_equals_the_c_library(oracle):
+    """The restated routine against the host C library's expf (glibc on x86-64, the routine the reference ports,
+    src/qwen38_exact_math.cuh:20-30) over four million inputs: thresholds, random bit patterns, the working range."""
+    x = _exp_probe_inputs()
+    got, want = oracle.expf_glibc(x), oracle.libm_expf(x)
+    same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+    assert same.all(), (x[~same][:5], got[~same][:5], want[~same][:5])
+    # and the function is what it claims to be: within half a unit in the last place of the float64 exponential
+    xs = x[np.isfinite(x) & (np.abs(x) < 80)][:200000]
+    ref = np.exp(xs.astype(np.float64))
+    assert np.all(np.abs(oracle.expf_glibc(xs).astype(np.float64) - ref) <= 0.502 * np.spacing(ref.astype(np.float32)).astype(np.float64))
+
+
+def test_round_half_equals_numpy_and_reference(oracle, refcpu):
+    rng = synth.rng_for(SEED, 401)
+    x = np.concatenate([
+        (rng.integers(0, 2 ** 32, 1_000_000, dtype=np.uint64).astype(np.uint32)).view(np.float32),
+        rng.normal(0, 1, 200000).astype(np.float32), rng.normal(0, 1e-6, 200000).astype(np.float32),
+        np.array([0.0, -0.0, 65504.0, 65519.996, 65520.0, 70000.0, 2.0 ** -14, 2.0 ** -24, 2.0 ** -25, 1.5 * 2.0 ** -25,
+                  np.nextafter(np.float32(2.0 ** -25), np.float32(1)), 2.0 ** -26, np.inf, -np.inf, 1.0009765625, 1.00048828125],
+                 np.float32)])
+    x = x[~np.isnan(x)]
+    got = oracle.round_half(x)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    r = refcpu.ref()
+    assert hasattr(r, "wdref_round_half")
+    if True:
+        for v in x[:20000]:
+            assert np.float32(r.wdref_round_half(float(v))).view(np.uint32) == np.float32(oracle.lib().wdo_round_half(float(v))).view(np.uint32)
+
+
+def test_branch_and_residual_steps(oracle, refcpu):
+    """One rounded multiply then one rounded add (no fused multiply-add): against numpy float32 steps, the reference's
+    header compiled in place, and the known answer of tests/issue1_ffn_precision_test.cpp:14-37."""
+    rng = synth.rng_for(SEED, 402)
+    a, b, c = (rng.normal(0, 1, 50000).astype(np.float32) for _ in range(3))
+    lib = oracle.lib()
+    fused_differs = 0
+    for i in range(a.size):
+        want = np.float32(a[i] + np.float32(b[i] * c[i]))
+        got = np.float32(lib.wdo_moe_branch_f32(float(a[i]), float(b[i]), float(c[i])))
+        assert got.view(np.uint32) == want.view(np.uint32)
+        assert np.float32(lib.wdo_residual_add_f32(float(a[i]), float(b[i]), float(c[i]))).view(np.uint32) == want.view(np.uint32)
+        fused_differs += int(np.float32(np.float64(b[i]) * np.float64(c[i]) + np.float64(a[i])) != want)
+        if i < 5000:
+            r = refcpu.ref()
+            assert np.float32(r.wdref_moe_branch_f32(float(a[i]), float(b[i]), float(c[i]))).view(np.uint32) == want.view(np.uint32)
+            assert np.float32(r.wdref_residual_add_f32(float(a[i]), float(b[i]), float(c[i]))).view(np.uint32) == want.view(np.uint32)
+    assert fused_differs > 100          # the sample tells a fused multiply-add from the two-step form
+    routed = np.float32(0.0)
+    for e in range(10):
+        half = oracle.round_half(np.array([1.0 if e % 2 == 0 else 1.0009765625], np.float32))[0]
+        routed = np.float32(np.float64(np.float32(0.1)) * np.float64(half) + np.float64(routed))   # fmaf: exact product, one rounding
+    moe = np.float32(lib.wdo_moe_branch_f32(float(routed), -0.00048828125, 0.5))
+    out = np.float32(lib.wdo_residual_add_f32(0.333251953125, float(moe), 1.25))
+    assert moe == np.float32(routed + np.float32(np.float32(0.5) * np.float32(-0.00048828125)))
+    assert out == np.float32(np.float32(0.333251953125) + np.float32(np.float32(1.25) * moe))
+
+
+@pytest.mark.parametrize("hc,hidden,round_half", [(4, 2048, False), (4, 2048, True), (3, 96, False), (1, 32, True), (8, 2560, False)])
+def test_hc_combine_against_numpy(oracle, hc, hidden, round_half):
+    """src/qwen38_hc.cuh:2530-2547 and :2241-2263 step by step in numpy float32, the weight through the C library's expf."""
+    rng = synth.rng_for(SEED, 403, hc, hidden)
+    res = rng.normal(0, 1, (hc, hidden)).astype(np.float32)
+    routed = rng.normal(0, 0.3, hidden).astype(np.float32)
+    shared = rng.normal(0, 0.3, hidden).astype(np.float32)
+    gate = np.float32(rng.uniform(0, 1))
+    inject = rng.normal(0, 2, hc).astype(np.float32)
+    z = (inject * np.float32(1.0 / np.float32(hc))).astype(np.float32)
+    e = oracle.libm_expf(-z)
+    w = (np.float32(2.0) * (np.float32(1.0) / (np.float32(1.0) + e)).astype(np.float32)).astype(np.float32)
+
+    def finish(v):
+        with np.errstate(over="ignore"):
+            return v.astype(np.float16).astype(np.float32) if round_half else v
+
+    block = (routed + (shared * gate).astype(np.float32)).astype(np.float32)
+    want = finish((res + (block[None, :] * w[:, None]).astype(np.float32)).astype(np.float32))
+    got = oracle.hc_combine(res, block, inject, round_half)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    got = oracle.hc_combine_moe(res, routed, shared, gate, inject, round_half)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    sh16 = shared.astype(np.float16)
+    block16 = (routed + (sh16.astype(np.float32) * gate).astype(np.float32)).astype(np.float32)
+    want16 = finish((res + (block16[None, :] * w[:, None]).astype(np.float32)).astype(np.float32))
+    got = oracle.hc_combine_moe(res, routed, sh16.view(np.uint16), gate, inject, round_half)
+    assert np.array_equal(got.view(np.uint32), want16.view(np.uint32))
+    for c in range(hc):                 # the weight itself: 2 / (1 + exp(-inject / hc)) to float accuracy
+        assert abs(float(w[c]) - 2.0 / (1.0 + np.exp(-float(inject[c]) / hc))) < 1e-6

@@ -52,6 +52,9 @@ _SIGS = {
     "wd_init": (i32, [i32]),
     "wd_row_bytes": (sz, [i32, i32]),
     "wd_gemv_q6_k_q8_k_f32": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp]),
+    "wd_hc_combine_f32": (i32, [vp, vp, vp, i32, i32, i32, vp]),
+    "wd_hc_combine_moe_f32": (i32, [vp, vp, vp, i32, vp, vp, i32, i32, i32, vp]),
+    "wd_moe_layer_hc_f32": (i32, [C.POINTER(MoeLayer), vp, vp, vp, vp, i32, i32, vp, u32, vp]),
     "wd_tensor_bytes": (sz, [i32, i32, i32]),
     "wd_malloc": (i32, [C.POINTER(vp), sz]),
     "wd_free": (i32, [vp]),

@@ -11,6 +11,8 @@
 
 #define WD_DEV __device__ __forceinline__
 
+#include "wd_exp2f_table.inc"
+
 namespace wd {
 
 constexpr int kWave = 64;
@@ -67,6 +69,44 @@ WD_DEV float exp_ggml(float x) {
 }
 
 // IEEE division (hipcc's default for '/': correctly rounded).
+// expf as glibc computes it (sysdeps/ieee754/flt-32/e_expf.c: a table of 2^(i/32), a cubic in double, every step one
+// rounded double operation), which the reference uses for its exact sigmoid: src/qwen38_exact_math.cuh:136-166.
+WD_DEV float expf_glibc(float x) {
+    constexpr uint64_t tab[32] = WD_EXP2F_TABLE;
+    constexpr double shift = 0x1.8p+52, invln2n = 0x1.71547652b82fep+0 * 32.0;
+    constexpr double c0 = 0x1.c6af84b912394p-5 / 32.0 / 32.0 / 32.0, c1 = 0x1.ebfce50fac4f3p-3 / 32.0 / 32.0,
+                     c2 = 0x1.62e42ff0c52d6p-1 / 32.0;
+    const uint32_t ix = f_bits(x), abstop = (ix >> 20) & 0x7ffu;
+    if (abstop >= (0x42b00000u >> 20)) {  // |x| >= 88, infinities, NaN
+        if (ix == 0xff800000u) return 0.0f;
+        if (abstop >= 0x7f8u) return x + x;
+        if (x > 0x1.62e42ep6f) return bits_f(0x7f800000u);  // 2^97 * 2^97
+        if (x < -0x1.9fe368p6f) return 0.0f;               // 2^-95 * 2^-95
+    }
+    const double z = invln2n * static_cast<double>(x);
+    const double kd_shift = z + shift;
+    const uint64_t ki = __builtin_bit_cast(uint64_t, kd_shift);
+    const double kd = kd_shift - shift;
+    const double r = z - kd;
+    const double s = __builtin_bit_cast(double, tab[ki & 31u] + (ki << 47));
+    const double p = c0 * r + c1;
+    const double r2 = r * r;
+    double y = c2 * r + 1.0;
+    y = p * r2 + y;
+    y = y * s;
+    return static_cast<float>(y);
+}
+// src/qwen38_exact_math.cuh:195-198
+WD_DEV float sigmoid_exact(float x) { return 1.0f / (1.0f + expf_glibc(-x)); }
+// float -> half -> float, IEEE round to nearest even (src/qwen38_precision.hpp:40-55)
+WD_DEV float round_half(float v) { return static_cast<float>(static_cast<_Float16>(v)); }
+// The weight of one residual stream in the hyper-connection combine: 2 sigmoid(inject / hc), each step one rounded
+// float operation (src/qwen38_hc.cuh:2542-2544).
+WD_DEV float hc_weight(float inject, int hc) {
+    const float z = inject * (1.0f / static_cast<float>(hc));
+    return 2.0f * sigmoid_exact(z);
+}
+
 WD_DEV float silu_ggml(float v) { return v / (1.0f + exp_ggml(-v)); }
 WD_DEV float sigmoid_ggml(float v) { return 1.0f / (1.0f + exp_ggml(-v)); }
 

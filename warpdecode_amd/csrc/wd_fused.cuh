@@ -31,8 +31,10 @@ struct LayerArgs {
     float *shared_gate;          // [1]: logit after A, sigmoid after B
     float *expert_out;           // null or [k][H]
     float *accum, *down_f32, *out;
-    float *residual;             // null or [H]
+    float *residual;             // null, [H] (residual += out * residual_scale), or [hc][H] when hc > 0
     float residual_scale;
+    const float *hc_inject;      // hc > 0: [hc] inject projections; residual[c] += out * 2 sigmoid(inject[c] / hc)
+    int hc, hc_round_half;
     int dry;                     // measurement aid: every workgroup returns at once
     int preselected;
     int n_router_wgs;            // workgroups of dispatch A that take router rows
@@ -982,10 +984,17 @@ __global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
             __hip_atomic_store(a.ids_tagged + i, kTagInvalid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     mark(a, 2, 0);
     // combine operands, requested early: lane m keeps router weight m, lane 16 the shared gate
-    float wreg = 0.0f;
+    float wreg = 0.0f, res_pre = 0.0f, inject = 0.0f;
     if (wave == 0) {
         if (lane < a.k) wreg = a.weights[lane];
         if (lane == 16 && shared) wreg = a.shared_gate[0];
+        // the residual values this workgroup updates at its end (nothing else writes them meanwhile): lane 4c + r
+        // holds stream c of row r0 + r
+        if (a.residual) {
+            const int c = a.hc > 0 ? min(lane >> 2, a.hc - 1) : 0;
+            res_pre = a.residual[static_cast<size_t>(c) * a.H + r0 + min(lane & 3, nrows - 1)];
+            if (a.hc > 0) inject = a.hc_inject[c];
+        }
     }
     for (int m = wave; m < n_act; m += nwaves) {
         const bool is_shared = m == a.k;
@@ -1012,6 +1021,7 @@ __global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
     __syncthreads();
     mark(a, 2, 3);
     if (wave == 0) {
+        // every lane folds row r0 + (lane & 3); lanes 0..3 store it
         const int row = r0 + lane;
         const bool on = lane < nrows;
         float acc = 0.0f;
@@ -1023,19 +1033,29 @@ __global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
             if (a.expert_out && on) a.expert_out[static_cast<size_t>(m) * a.H + row] = y;
         }
         const float gate = lane_get(wreg, 16);
-        if (!on) return;
         float o = acc;
         if (shared) {
-            const float y = ybuf[a.k * 4 + lane];
+            const float y = ybuf[a.k * 4 + (lane & 3)];
             const float prod = y * gate;
             o = acc + prod;
-            a.down_f32[row] = y;
+            if (on) a.down_f32[row] = y;
         }
-        a.accum[row] = acc;
-        a.out[row] = o;
+        if (on) {
+            a.accum[row] = acc;
+            a.out[row] = o;
+        }
         if (a.residual) {
-            const float scaled = o * a.residual_scale;
-            a.residual[row] = a.residual[row] + scaled;
+            if (a.hc > 0) {
+                const int c = lane >> 2;
+                if (c < a.hc && (lane & 3) < nrows) {
+                    const float weighted = o * hc_weight(inject, a.hc);
+                    const float v = res_pre + weighted;
+                    a.residual[static_cast<size_t>(c) * a.H + r0 + (lane & 3)] = a.hc_round_half ? round_half(v) : v;
+                }
+            } else if (on) {
+                const float scaled = o * a.residual_scale;
+                a.residual[row] = res_pre + scaled;
+            }
         }
     }
     mark(a, 2, 4);

@@ -441,4 +441,24 @@ __global__ void k_combine(const float *__restrict__ experts, const float *__rest
     }
 }
 
+// Hyper-connection combine of the FFN branch: residual[c][h] += branch[h] * (2 sigmoid(inject[c] / hc)) for the hc
+// residual streams, product rounded, then sum rounded (src/qwen38_hc.cuh:2530-2547).  SHARED: 0 = branch is block_out,
+// 1 / 2 = branch = routed + shared * gate[0] with the shared expert's output as float / as half bits (:2241-2263).
+template <int SHARED>
+__global__ void k_hc_combine(float *__restrict__ residual, const float *__restrict__ block_out, const void *__restrict__ shared,
+                             const float *__restrict__ gate, const float *__restrict__ inject, int hidden, int hc, int round) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= hidden * hc) return;
+    const int c = i / hidden, h = i - c * hidden;
+    float branch = block_out[h];
+    if (SHARED != 0) {
+        const float sh = SHARED == 1 ? static_cast<const float *>(shared)[h] : h2f(static_cast<const uint16_t *>(shared)[h]);
+        const float weighted = sh * gate[0];
+        branch = branch + weighted;
+    }
+    const float weighted = branch * hc_weight(inject[c], hc);
+    const float v = residual[i] + weighted;
+    residual[i] = round ? round_half(v) : v;
+}
+
 }  // namespace wd

@@ -275,10 +275,18 @@ int grouped_gemv(int type, MatSrc src, int mats, int rows, int cols, const wd_mo
 
 namespace {
 
+// The hyper-connection form of the residual update: residual is [hc][hidden] and stream c receives
+// out * 2 sigmoid(inject[c] / hc) (src/qwen38_hc.cuh:2530-2547).
+struct HcSpec {
+    const float *inject;
+    int hc, round_half;
+};
+
 // One layer, one launch per stage.  ids_override (device, k ids) replaces the router's ids while
 // keeping its weights; residual (device f32[hidden]) receives residual += layer output.
 int layer_staged(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s, unsigned flags,
-                 const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st) {
+                 const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st,
+                 const HcSpec *hc = nullptr) {
     const int H = L->hidden, F = L->expert_ffn, E = L->n_experts, k = L->top_k;
     const bool shared = L->shared_gate_inp != nullptr;
     const bool pre = (flags & WD_MOE_PRESELECTED) != 0;
@@ -343,13 +351,20 @@ int layer_staged(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_s
 
     // 7. ordered weighted sum and the shared branch
     k_combine<<<dim3((H + 255) / 256), dim3(256), 0, st>>>(s->expert_out, s->weights, k, shared ? s->down_f32 : nullptr,
-                                                            s->shared_gate, s->accum, d_out, residual, residual_scale, H);
+                                                            s->shared_gate, s->accum, d_out, hc ? nullptr : residual,
+                                                            residual_scale, H);
     WD_LAUNCH_CHECK();
+    if (hc && residual) {
+        k_hc_combine<0><<<dim3((H * hc->hc + 255) / 256), dim3(256), 0, st>>>(residual, d_out, nullptr, nullptr, hc->inject, H,
+                                                                             hc->hc, hc->round_half);
+        WD_LAUNCH_CHECK();
+    }
     return WD_OK;
 }
 
 LayerArgs fused_args(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s, unsigned flags,
-                     const int32_t *ids_override, float *residual, float residual_scale, int rec = 0) {
+                     const int32_t *ids_override, float *residual, float residual_scale, int rec = 0,
+                     const HcSpec *hc = nullptr) {
     const bool shared = L->shared_gate_inp != nullptr;
     LayerArgs a{};
     a.H = L->hidden, a.F = L->expert_ffn, a.E = L->n_experts, a.k = L->top_k;
@@ -367,6 +382,7 @@ LayerArgs fused_args(const wd_moe_layer *L, const float *d_x, float *d_out, wd_m
     a.expert_out = (flags & WD_MOE_KEEP_EXPERT_OUT) ? s->expert_out : nullptr;
     a.accum = s->accum, a.down_f32 = s->down_f32, a.out = d_out;
     a.residual = residual, a.residual_scale = residual_scale;
+    if (hc) a.hc_inject = hc->inject, a.hc = hc->hc, a.hc_round_half = hc->round_half;
     a.preselected = (flags & WD_MOE_PRESELECTED) ? 1 : 0;
     a.dry = (flags & WD_MOE_DRY) ? 1 : 0;
     const int router_rows_n = (a.preselected ? 0 : a.E) + (shared ? 1 : 0);
@@ -392,10 +408,11 @@ int launch_a(const LayerArgs &a, hipStream_t st) {
 
 // One layer in three dispatches (router + shared gate/up, routed gate/up, down + combine).
 int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s, unsigned flags,
-                const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st, int rec = 0) {
+                const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st, int rec = 0,
+                const HcSpec *hc = nullptr) {
     const int H = L->hidden, F = L->expert_ffn, k = L->top_k;
     const bool shared = L->shared_gate_inp != nullptr;
-    const LayerArgs a = fused_args(L, d_x, d_out, s, flags, ids_override, residual, residual_scale, rec);
+    const LayerArgs a = fused_args(L, d_x, d_out, s, flags, ids_override, residual, residual_scale, rec, hc);
     const unsigned only = flags & (WD_MOE_ONLY_A | WD_MOE_ONLY_B | WD_MOE_ONLY_C);
     const bool run_a = !only || (only & WD_MOE_ONLY_A), run_b = !only || (only & WD_MOE_ONLY_B);
     const bool iq = consumes_q8k(L->gate_type);
@@ -467,11 +484,12 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
 }
 
 int layer_dispatch(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s, unsigned flags,
-                   const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st, int rec = 0) {
+                   const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st, int rec = 0,
+                   const HcSpec *hc = nullptr) {
     const bool want_partials = s->gup != nullptr;
     if ((flags & WD_MOE_STAGED) || want_partials)
-        return layer_staged(L, d_x, d_out, s, flags, ids_override, residual, residual_scale, st);
-    return layer_fused(L, d_x, d_out, s, flags, ids_override, residual, residual_scale, st, rec);
+        return layer_staged(L, d_x, d_out, s, flags, ids_override, residual, residual_scale, st, hc);
+    return layer_fused(L, d_x, d_out, s, flags, ids_override, residual, residual_scale, st, rec, hc);
 }
 
 }  // namespace
@@ -481,6 +499,41 @@ extern "C" int wd_moe_layer_f32(const wd_moe_layer *L, const float *d_x, float *
     if (const int rc = check_layer(L, s)) return rc;
     WD_REQUIRE(d_x && d_out, "MoE layer: null activation or output pointer");
     return layer_dispatch(L, d_x, d_out, s, flags, nullptr, nullptr, 0.0f, as_stream(stream));
+}
+
+extern "C" int wd_moe_layer_hc_f32(const wd_moe_layer *L, const float *d_x, float *d_out, float *d_residual,
+                                   const float *d_inject, int hc, int round_half, wd_moe_scratch *s, unsigned flags,
+                                   void *stream) {
+    if (const int rc = check_layer(L, s)) return rc;
+    WD_REQUIRE(d_x && d_out && d_residual && d_inject, "MoE layer with combine: null activation, output, residual or inject pointer");
+    WD_REQUIRE(hc >= 1 && hc <= 16, "MoE layer with combine: 1..16 residual streams (got %d)", hc);
+    WD_REQUIRE(!(flags & (WD_MOE_ONLY_A | WD_MOE_ONLY_B | WD_MOE_ONLY_C | WD_MOE_DRY)), "MoE layer with combine: measurement flags are not supported");
+    const HcSpec spec{d_inject, hc, round_half ? 1 : 0};
+    return layer_dispatch(L, d_x, d_out, s, flags, nullptr, d_residual, 0.0f, as_stream(stream), 0, &spec);
+}
+
+extern "C" int wd_hc_combine_f32(float *d_residual, const float *d_block_out, const float *d_inject, int hidden, int hc,
+                                 int round_half, void *stream) {
+    WD_REQUIRE(d_residual && d_block_out && d_inject, "combine: null pointer");
+    WD_REQUIRE(hidden > 0 && hc > 0 && static_cast<long long>(hidden) * hc < (1LL << 31), "combine: bad geometry %d x %d", hc, hidden);
+    k_hc_combine<0><<<dim3((hidden * hc + 255) / 256), dim3(256), 0, as_stream(stream)>>>(d_residual, d_block_out, nullptr, nullptr,
+                                                                                          d_inject, hidden, hc, round_half ? 1 : 0);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+extern "C" int wd_hc_combine_moe_f32(float *d_residual, const float *d_routed, const void *d_shared, int shared_is_half,
+                                     const float *d_shared_gate, const float *d_inject, int hidden, int hc, int round_half,
+                                     void *stream) {
+    WD_REQUIRE(d_residual && d_routed && d_shared && d_shared_gate && d_inject, "combine: null pointer");
+    WD_REQUIRE(hidden > 0 && hc > 0 && static_cast<long long>(hidden) * hc < (1LL << 31), "combine: bad geometry %d x %d", hc, hidden);
+    const dim3 grid((hidden * hc + 255) / 256), block(256);
+    if (shared_is_half)
+        k_hc_combine<2><<<grid, block, 0, as_stream(stream)>>>(d_residual, d_routed, d_shared, d_shared_gate, d_inject, hidden, hc, round_half ? 1 : 0);
+    else
+        k_hc_combine<1><<<grid, block, 0, as_stream(stream)>>>(d_residual, d_routed, d_shared, d_shared_gate, d_inject, hidden, hc, round_half ? 1 : 0);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
 }
 
 extern "C" int wd_shared_expert_f32(const wd_moe_layer *L, const float *d_x, wd_moe_scratch *s, void *stream) {

@@ -660,4 +660,59 @@ inline void run_qwen38_moe_layer_f32_x(int layer, const float *x, const GpuMatri
     check(wd_moe_layer_f32(&L, x, out, scratch.handle(), 0u, stream), "MoE layer failed");
 }
 
+// The F32 inject projections of the hyper-connection combine (the part of the reference's Qwen38HcF32DebugScratch that
+// the combine reads: hidden(), hc(), inject(); src/qwen38_hc.cuh:2263-2330).
+class Qwen38HcF32DebugScratch {
+public:
+    void initialize(int hidden, int hc) {
+        if (hidden <= 0 || hc <= 0) throw std::runtime_error("invalid hyper-connection scratch geometry");
+        hidden_ = hidden, hc_ = hc;
+        inject_.reset();
+        inject_.allocate(static_cast<size_t>(hc));
+    }
+    int hidden() const { return hidden_; }
+    int hc() const { return hc_; }
+    float *inject() const { return inject_.data; }
+
+private:
+    int hidden_ = 0, hc_ = 0;
+    DeviceFloatArray inject_;
+};
+
+// src/qwen38_hc.cuh:2561-2570
+inline void run_qwen38_hc_combine_f32_block_f32_inject(float *residual, const float *block_out, const Qwen38HcF32DebugScratch &scratch,
+                                                       Stream stream, bool round_half = false) {
+    check(wd_hc_combine_f32(residual, block_out, scratch.inject(), scratch.hidden(), scratch.hc(), round_half ? 1 : 0, stream),
+          "hyper-connection combine failed");
+}
+// src/qwen38_hc.cuh:2587-2600 (shared: the shared expert's output as half bits)
+inline void run_qwen38_hc_combine_moe_f32_inject(float *residual, const float *routed, const half_bits *shared, const float *shared_gate,
+                                                 const Qwen38HcF32DebugScratch &scratch, Stream stream, bool round_half = false) {
+    check(wd_hc_combine_moe_f32(residual, routed, shared, 1, shared_gate, scratch.inject(), scratch.hidden(), scratch.hc(),
+                                round_half ? 1 : 0, stream),
+          "hyper-connection combine failed");
+}
+// The same with the shared expert's output in F32, as run_qwen38_shared_expert_f32_x leaves it in the scratch.
+inline void run_qwen38_hc_combine_moe_f32_inject(float *residual, const float *routed, const float *shared, const float *shared_gate,
+                                                 const Qwen38HcF32DebugScratch &scratch, Stream stream, bool round_half = false) {
+    check(wd_hc_combine_moe_f32(residual, routed, shared, 0, shared_gate, scratch.inject(), scratch.hidden(), scratch.hc(),
+                                round_half ? 1 : 0, stream),
+          "hyper-connection combine failed");
+}
+
+// run_qwen38_moe_layer_f32_x followed by run_qwen38_hc_combine_f32_block_f32_inject on its output, the combine folded into
+// the layer's last dispatch (src/qwen38_forward.cuh:3330-3371 issues them one after the other).
+inline void run_qwen38_moe_layer_hc_f32_x(int layer, const float *x, const GpuMatrix &router, const TensorInfo &gate_exps,
+                                          const TensorInfo &up_exps, const TensorInfo &down_exps, GpuExpertCache &cache,
+                                          const Qwen38SharedExpertWeights &shared, Qwen38MoeScratch &scratch, float *out, float *residual,
+                                          const Qwen38HcF32DebugScratch &hc, float expert_scale, Stream stream, bool round_half = false) {
+    if (hc.hidden() != static_cast<int>(gate_exps.dims[0])) throw std::runtime_error("hyper-connection scratch does not match the layer's hidden size");
+    wd_moe_layer L;
+    detail::fill_routed(L, layer, router, gate_exps, up_exps, down_exps, cache, scratch, expert_scale);
+    L.shared_gate_inp = shared.gate_input_f32.data;
+    L.shared_gate = shared.gate.data, L.shared_up = shared.up.data, L.shared_down = shared.down.data;
+    check(wd_moe_layer_hc_f32(&L, x, out, residual, hc.inject(), hc.hc(), round_half ? 1 : 0, scratch.handle(), 0u, stream),
+          "MoE layer with combine failed");
+}
+
 }  // namespace wd
