@@ -47,7 +47,7 @@ def parse():
     ap.add_argument("--experts", type=int, default=512)
     ap.add_argument("--routing", choices=["zipf", "router"], default="zipf",
                     help="zipf: ids replayed from the Zipf(1.1) trace; router: ids chosen by the router itself")
-    ap.add_argument("--mode", choices=["resident", "lru", "q4-sweep", "q6k-head", "tokens", "c0"], default="resident",
+    ap.add_argument("--mode", choices=["resident", "lru", "q4-sweep", "q8-sweep", "q6k-head", "hc", "tokens", "c0"], default="resident",
                     help="resident: C3 mode A, every expert in HBM; lru: C3 mode B, experts in pinned host memory "
                          "behind an LRU slot pool of --cache-gib in HBM; q4-sweep: the dense Q4_0 GEMV shapes; "
                          "tokens: the 4-token speculative-verify pass over the same layers; c0: the 64-expert top-8 "
@@ -427,6 +427,51 @@ def bench_q4_sweep(args, torch, capi, synth):
                          kernel="k_gemv_q8<Q4_0>", us_per_launch=head["us_per_gemv"], bytes_per_launch=head["bytes"])}))
 
 
+def bench_q8_sweep(args, torch, capi, synth):
+    """Dense exact-order Q8_0 x Q8_0 GEMV at batch=1 (the projections around the MoE layer: hyper-connection mix, attention
+    and recurrent blocks, src/qwen38_hc.cuh:1020-1049) over square, wide, tall and head-sized shapes.  Every launch of a
+    chain reads another copy of the matrix (>= 1.5 GB of copies); the period is taken over a captured chain."""
+    shapes = [(2048, 2048), (8192, 2048), (2048, 8192), (512, 8192), (8192, 512), (8192, 8192), (32768, 2048), (151936, 2048)]
+    results = []
+    for rows, cols in shapes:
+        nbytes = rows * synth.row_bytes(synth.Q8_0, cols)
+        copies = max(2, min(640, -(-int(1.5e9) // nbytes)))
+        part = min(rows, 2048)
+        one = torch.from_numpy(synth.matrix(synth.Q8_0, synth.rng_for(synth.BASE_SEED, 79, rows, cols), part, cols)).reshape(-1).cuda()
+        w = one.repeat(-(-rows // part))[:nbytes].repeat(copies).reshape(copies, nbytes)
+        x = torch.from_numpy(synth.rng_for(synth.BASE_SEED, 80, cols).normal(0, 1, cols).astype(np.float32)).cuda()
+        qs = torch.empty(cols, dtype=torch.int8, device="cuda")
+        sc = torch.empty(cols // 32, dtype=torch.int16, device="cuda")
+        y = torch.empty(rows, dtype=torch.float32, device="cuda")
+        stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        vp = lambda t: C.c_void_p(t.data_ptr())
+        capi.call("wd_q8_0_quantize_f32", vp(x), cols, vp(qs), vp(sc), stream())
+
+        def gemv(i):
+            capi.call("wd_gemv_q8_0_f32", synth.Q8_0, C.c_void_p(w[i % copies].data_ptr()), rows, cols, vp(qs), vp(sc), vp(y),
+                      None, stream())
+
+        gemv(0)
+        torch.cuda.synchronize()
+        launches = max(copies, 32)
+        reps = max(3, int(1e11 // (nbytes * launches)))
+        us = graph_period_us(torch, gemv, launches, reps)
+        results.append(dict(rows=rows, cols=cols, bytes=nbytes, copies=copies, us_per_gemv=round(us, 3),
+                            gbs=round(nbytes / us / 1e3, 1), frac=round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                            finite=bool(torch.isfinite(y).all().item())))
+        note("Q8_0 %dx%d: %.2f us, %.0f GB/s" % (rows, cols, us, nbytes / us / 1e3))
+        del w, one
+        torch.cuda.empty_cache()
+    head = results[-1]
+    print(json.dumps({
+        "metric": "dense Q8_0 GEMV batch=1: achieved HBM GB/s (151936x2048)", "value": head["gbs"], "unit": "GB/s",
+        "n_gpus": 1, "higher_is_better": True, "vs_baseline": None, "dtype": "int8 dot products, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "exact-order Q8_0 x Q8_0 GEMV sweep, raw GGUF 34-byte blocks", "shapes": results},
+        "roofline": dict(bound="hbm", achieved=head["gbs"], peak=HBM_PEAK_GBS, unit="GB/s", frac=head["frac"], traffic=None,
+                         kernel="k_gemv_q8_rows8", us_per_launch=head["us_per_gemv"], bytes_per_launch=head["bytes"])}))
+
+
 def bench_q6k_head(args, torch, capi, synth):
     """The output head of the Qwen3 MoE models: Q6_K 151936 x 2048 against the Q8_K image of the F32 activation, once
     per decoded token.  Every launch of a chain reads another copy of the matrix (7 copies, 1.8 GB) so that nothing
@@ -467,6 +512,53 @@ def bench_q6k_head(args, torch, capi, synth):
                    "copies": copies, "us_per_call_with_quantise": round(us_call, 3), "finite": bool(torch.isfinite(y).all().item())},
         "roofline": dict(bound="hbm", achieved=round(gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(gbs / HBM_PEAK_GBS, 4),
                          traffic=None, kernel="k_gemv_q6k", us_per_launch=round(us, 3), bytes_per_launch=nbytes)}))
+
+
+def bench_hc(args, torch, capi, synth):
+    """The layer together with the hyper-connection combine that consumes its output (four residual streams): the
+    combine folded into the layer's last dispatch against the layer followed by the combine as a launch of its own.
+    `--layers` different C2 layers per captured chain, router-selected experts."""
+    H, F, k, E, NL, hc = 2048, 512, 10, args.experts, args.layers, 4
+    layers, keep = build_stack(torch, synth, capi, NL, E, synth.BASE_SEED)
+    scratch = C.c_void_p()
+    capi.call("wd_moe_scratch_create", C.byref(scratch), H, F, E, k)
+    rng = synth.rng_for(synth.BASE_SEED, 9300)
+    d_x = torch.from_numpy(synth.rms_normed(rng, H)).cuda()
+    d_out = torch.zeros(H, dtype=torch.float32, device="cuda")
+    d_inject = torch.from_numpy(rng.normal(0, 1, hc).astype(np.float32)).cuda()
+    res0 = torch.from_numpy(rng.normal(0, 1, (hc, H)).astype(np.float32)).cuda()
+    d_res = res0.clone()
+    stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    vp = lambda t: C.c_void_p(t.data_ptr())
+
+    def folded(i):
+        capi.call("wd_moe_layer_hc_f32", C.byref(layers[i % NL]), vp(d_x), vp(d_out), vp(d_res), vp(d_inject), hc, 0, scratch, 0, stream())
+
+    def apart(i):
+        capi.call("wd_moe_layer_f32", C.byref(layers[i % NL]), vp(d_x), vp(d_out), scratch, 0, stream())
+        capi.call("wd_hc_combine_f32", vp(d_res), vp(d_out), vp(d_inject), H, hc, 0, stream())
+
+    results = {}
+    for name, fn in (("folded", folded), ("apart", apart)):
+        d_res.copy_(res0)
+        for i in range(NL):
+            fn(i)
+        torch.cuda.synchronize()
+        results[name + "_residual"] = d_res.clone()
+        results[name] = graph_period_us(torch, fn, NL, 50)
+    same = bool(torch.equal(results["folded_residual"].view(torch.int32), results["apart_residual"].view(torch.int32)))
+    ok = same and bool(torch.isfinite(d_res).all().item()) and capi.load().wd_moe_scratch_status(scratch) == 0
+    note("layer + combine: folded %.2f us, apart %.2f us per layer" % (results["folded"], results["apart"]))
+    nbytes = 27697152 + 2 * hc * H * 4   # the C2 layer plus the residual streams read and written
+    print(json.dumps({
+        "metric": "MoE layer + hyper-connection combine, batch=1: microseconds per layer", "value": round(results["folded"], 3),
+        "unit": "us", "n_gpus": 1, "higher_is_better": False, "vs_baseline": None,
+        "dtype": "int8 dot products, f32 accumulate", "data": "synthetic",
+        "config": {"workload": "C2 layer (512 experts, top-10, IQ3_S/Q8_0, shared expert) + combine into 4 residual streams",
+                   "layers": NL, "combine_as_its_own_launch_us": round(results["apart"], 3), "same_bits": same, "ok": ok},
+        "roofline": dict(bound="hbm", achieved=round(nbytes / results["folded"] / 1e3, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                         frac=round(nbytes / results["folded"] / 1e3 / HBM_PEAK_GBS, 4), traffic=None,
+                         kernel="k_layer_ab + k_layer_c", us_per_launch=round(results["folded"], 3), bytes_per_launch=nbytes)}))
 
 
 def bench_c0(args, torch, capi, synth):
@@ -612,6 +704,8 @@ def main():
     H, F, k, E, NL = 2048, 512, 10, args.experts, args.layers
     if args.mode == "q4-sweep":
         return bench_q4_sweep(args, torch, capi, synth)
+    if args.mode == "q8-sweep":
+        return bench_q8_sweep(args, torch, capi, synth)
     if args.mode == "c0":
         return bench_c0(args, torch, capi, synth)
     if args.mode == "q6k-head":
@@ -621,6 +715,8 @@ def main():
         return bench_tokens(args, torch, capi, synth)
     if args.mode == "lru":
         return bench_lru(args, torch, capi, synth)
+    if args.mode == "hc":
+        return bench_hc(args, torch, capi, synth)
     layers, keep = build_stack(torch, synth, capi, NL, E, synth.BASE_SEED)
     torch.cuda.synchronize()
     note("weights ready (%.1f GB allocated)" % (torch.cuda.memory_allocated() / 1e9))

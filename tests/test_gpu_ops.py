@@ -104,7 +104,10 @@ def _quant_act(oracle, t, x):
 GEMV_SHAPES = {
     synth.IQ3_S: [(512, 2048), (64, 2560), (5, 256), (33, 4096)],
     synth.IQ2_S: [(640, 2560), (512, 2048), (3, 256)],
-    synth.Q8_0: [(2048, 512), (512, 2048), (7, 96), (640, 2560), (18, 32)],
+    # the streaming kernel (eight rows per wave, 16- or 32-block chunks, single waves or four per workgroup, ragged row
+    # counts), then shapes that take the general kernel
+    synth.Q8_0: [(2048, 512), (512, 2048), (640, 2560), (2048, 8192), (1003, 2048), (5, 1024), (8203, 2048), (9, 16384),
+                 (33, 512), (7, 96), (18, 32), (12, 32768), (40, 768)],
     synth.IQ4_NL: [(2560, 640), (2048, 512), (5, 96), (9, 32 * 5)],
     # C1 incl. the lm_head; then ragged row counts for every lanes-per-row case of the streaming kernel (columns a
     # multiple of 256 whose 8-block groups per row divide 64) and shapes that take the general kernel
@@ -190,6 +193,26 @@ def test_gemv_q6_k_head_from_f32_and_misaligned(g, oracle):
     xq = (qs.astype(np.float64).reshape(-1, 256) * d.astype(np.float64)[:, None]).reshape(-1)
     ref = np.array([oracle.dequant_row(synth.Q6_K, w[r], cols).astype(np.float64) @ xq for r in range(64)])
     assert np.allclose(g.host(out)[:64], ref, rtol=1e-4, atol=1e-6)
+
+
+def test_q8_0_gemv_misaligned_base(g, oracle):
+    """A Q8_0 matrix 2 bytes into an allocation takes the general kernel: same bits as the streaming one."""
+    import torch
+    rows, cols = 77, 2048
+    rng = synth.rng_for(SEED, 24, rows, cols)
+    w = synth.matrix(synth.Q8_0, rng, rows, cols)
+    x = rng.normal(0, 1, cols).astype(np.float32)
+    qs, d = oracle.quantize_q8_0(x)
+    dq, dd = g.dev(qs), g.dev(d)
+    dw = g.dev(w)
+    shifted = torch.zeros(w.size + 16, dtype=torch.uint8, device="cuda")
+    shifted[2:2 + w.size] = dw.reshape(-1)
+    out, out_s = g.empty(rows, np.float32), g.empty(rows, np.float32)
+    capi.call("wd_gemv_q8_0_f32", synth.Q8_0, g.ptr(dw), rows, cols, g.ptr(dq), g.ptr(dd), g.ptr(out), None, g.stream())
+    capi.call("wd_gemv_q8_0_f32", synth.Q8_0, shifted.data_ptr() + 2, rows, cols, g.ptr(dq), g.ptr(dd), g.ptr(out_s), None, g.stream())
+    g.sync()
+    want = oracle.gemv(synth.Q8_0, w, rows, cols, qs, d)
+    assert g.same_bits(g.host(out), want) and g.same_bits(g.host(out_s), want)
 
 
 def test_q4_0_gemv_misaligned_base(g, oracle):

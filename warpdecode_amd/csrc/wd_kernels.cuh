@@ -302,6 +302,155 @@ __global__ __launch_bounds__(WPB * 64) void k_gemv_q4_stream(const uint8_t *__re
     }
 }
 
+// ---- dense Q8_0 x Q8_0 GEMV, streaming: one lane per (row, chain) ----------------------------------------------
+// The reference order of a Q8_0 row (src/qwen38_cpu_moe.cuh:690-722) is eight chains, chain c over bytes 4c..4c+3 of
+// every block, each one fma(d_w d_a, float(dot4), acc) per block in block order: the chains of a row are as long as
+// the row, and nothing shortens them.  A wave therefore takes eight rows and gives every (row, chain) pair a lane
+// (lane = 8 row + chain): each fma instruction then advances 64 chains, no value crosses lanes until the closing tree,
+// and the cost per block and row is under one vector instruction.
+// The eight rows are fetched KB blocks at a time (34 KB bytes per row, whole 16-byte words because KB is a multiple of
+// 8 and rows start on 16-byte boundaries) with lane-contiguous 16-byte loads, one chunk ahead in a second register set,
+// and copied to LDS with a row stride that spreads the eight rows over the banks.  Blocks are 34 bytes, so the four
+// bytes of a lane are dword aligned in the odd blocks of a chunk and two bytes off in the even ones (two dwords and a
+// v_alignbyte); the parity is the same for every lane, so the unrolled loop knows it at compile time.
+// The activation's quants and its scales (as floats) are staged in LDS once per workgroup.
+// dynamic LDS: cols bytes, cols/32 floats, then one stage of 8 * kQ8sRowStride<KB> bytes per wave.
+template <int KB>
+constexpr int kQ8sRowStride = KB == 64 ? 2208 : (KB == 32 ? 1184 : 544);  // 34 KB + padding, 8 (mod 32) dwords
+
+template <int KB>
+struct Q8sFetch {
+    static constexpr int kWordsPerRow = 34 * KB / 16;                 // 16-byte words of a row's chunk
+    static constexpr int kWords = 8 * kWordsPerRow;                    // of the eight rows
+    static constexpr int kLoads = (kWords + 63) / 64;
+    uint4 u[kLoads];
+};
+
+// SETS: register sets of fetched chunks in flight per wave (2 for grids of single waves, which have nothing else to
+// hide the memory latency with).
+template <int KB, bool PART, int WAVES, int SETS>
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(WAVES == 1 ? 1 : 4))) void k_gemv_q8_rows8(const uint8_t *__restrict__ w, int rows, int nb,
+                                                              const int8_t *__restrict__ act_qs, const uint16_t *__restrict__ act_d,
+                                                              float *__restrict__ out, int32_t *__restrict__ partials) {
+    using Fetch = Q8sFetch<KB>;
+    constexpr int RS = kQ8sRowStride<KB>;
+    extern __shared__ __align__(16) uint8_t q8s_lds[];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int cols = nb * 32;
+    int8_t *aq = reinterpret_cast<int8_t *>(q8s_lds);
+    float *ad = reinterpret_cast<float *>(q8s_lds + cols);
+    uint8_t *stage = q8s_lds + cols + nb * 4 + wave * (8 * RS);
+    const size_t rb = static_cast<size_t>(nb) * 34;
+    // the waves of the grid take the groups of eight rows in turn (rows >= 8)
+    const int n_groups = (rows + 7) >> 3, n_waves = gridDim.x * WAVES, first = blockIdx.x * WAVES + wave;
+    const int my_groups = first < n_groups ? (n_groups - first + n_waves - 1) / n_waves : 0;
+    const int nchunks = nb / KB;
+    // where the lane's words of a chunk lie: in memory (relative to the chunk of the group's first row) and in the stage
+    const int row = lane >> 3, c = lane & 7;
+    uint32_t goff[Fetch::kLoads], loff[Fetch::kLoads];
+#pragma unroll
+    for (int i = 0; i < Fetch::kLoads; ++i) {
+        const int u = min(i * 64 + lane, Fetch::kWords - 1);
+        const int r = u / Fetch::kWordsPerRow, within = u - r * Fetch::kWordsPerRow;
+        goff[i] = static_cast<uint32_t>(r * rb + 16 * within);
+        loff[i] = static_cast<uint32_t>(r * RS + 16 * within);
+    }
+    // the fetch runs SETS chunks ahead of the arithmetic, over the group boundaries
+    int f_group = min(first, n_groups - 1), f_chunk = 0, fetched = 0;
+    const int items = my_groups * nchunks;
+    Fetch fs[SETS];
+    auto fetch = [&](Fetch &f) {
+        // a last group of fewer than eight rows is moved up to end with the matrix: it then repeats rows of the group
+        // before it, which come out the same
+        const uint8_t *p = uniform_ptr(w + static_cast<size_t>(min(8 * f_group, rows - 8)) * rb + static_cast<size_t>(f_chunk) * (34 * KB));
+#pragma unroll
+        for (int i = 0; i < Fetch::kLoads; ++i) f.u[i] = gld_u128_aligned(p + goff[i]);
+        // past the wave's last chunk the same chunk is requested again (and not used), so that every turn issues the
+        // same number of requests
+        if (++fetched < items) {
+            if (++f_chunk == nchunks) f_chunk = 0, f_group += n_waves;
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < SETS; ++i) fetch(fs[i]);
+    for (int i = threadIdx.x; i < cols / 16; i += 64 * WAVES) reinterpret_cast<uint4 *>(aq)[i] = reinterpret_cast<const uint4 *>(act_qs)[i];
+    for (int i = threadIdx.x; i < nb; i += 64 * WAVES) ad[i] = h2f(act_d[i]);
+    __syncthreads();
+    if (my_groups == 0) return;  // wave-uniform
+    const uint8_t *my = stage + row * RS + 4 * c;
+    const int8_t *my_a = aq + 4 * c;
+    // Eight blocks of the lane's row at a time: their LDS reads are issued as one group, the next group's before the
+    // arithmetic of this one, so that the reads' latency lies under it.
+    struct Batch {
+        uint32_t w[12];  // blocks 0 2 4 6 of the batch: two dwords each (w[3i], w[3i+1]); blocks 1 3 5 7: w[3i+2]
+        uint32_t dw[8], a[8];
+        float4 da[2];
+    };
+    auto load_batch = [&](Batch &t, int b0, int s) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint8_t *blk = my + 34 * (8 * s + 2 * i);
+            t.w[3 * i] = *reinterpret_cast<const uint32_t *>(blk);
+            t.w[3 * i + 1] = *reinterpret_cast<const uint32_t *>(blk + 4);
+            t.w[3 * i + 2] = *reinterpret_cast<const uint32_t *>(blk + 36);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            t.dw[i] = *reinterpret_cast<const uint16_t *>(stage + row * RS + 34 * (8 * s + i));
+            t.a[i] = *reinterpret_cast<const uint32_t *>(my_a + 32 * (b0 + 8 * s + i));
+        }
+        t.da[0] = *reinterpret_cast<const float4 *>(ad + b0 + 8 * s);
+        t.da[1] = *reinterpret_cast<const float4 *>(ad + b0 + 8 * s + 4);
+    };
+    float acc = 0.0f;
+    int group = first, chunk = 0;
+    auto turn = [&](Fetch &f) {
+        wave_lds_fence();  // the previous chunk has been read
+#pragma unroll
+        for (int i = 0; i < Fetch::kLoads; ++i) *reinterpret_cast<uint4 *>(stage + loff[i]) = f.u[i];
+        wave_lds_fence();
+        fetch(f);  // a later chunk, into the registers just written out
+        const int b0 = chunk * KB;
+        const int out_row = min(8 * group, rows - 8) + row;
+        int32_t *pp = PART ? partials + (static_cast<size_t>(out_row) * nb) * 8 + c : nullptr;
+        auto compute_batch = [&](const Batch &bt, int s) {
+            const float da[8] = {bt.da[0].x, bt.da[0].y, bt.da[0].z, bt.da[0].w, bt.da[1].x, bt.da[1].y, bt.da[1].z, bt.da[1].w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t q = (i & 1) ? bt.w[3 * (i >> 1) + 2]
+                                           : __builtin_amdgcn_alignbyte(bt.w[3 * (i >> 1) + 1], bt.w[3 * (i >> 1)], 2);
+                const int p = sdot4(q, bt.a[i], 0);
+                if (PART) pp[(b0 + 8 * s + i) * 8] = p;
+                const float d = h2f(static_cast<uint16_t>(bt.dw[i])) * da[i];
+                acc = __builtin_fmaf(d, static_cast<float>(p), acc);
+            }
+        };
+        Batch t0, t1;
+        load_batch(t0, b0, 0);
+#pragma unroll
+        for (int s = 0; s < KB / 8; s += 2) {
+            load_batch(t1, b0, s + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            compute_batch(t0, s);
+            if (s + 2 < KB / 8) load_batch(t0, b0, s + 2);
+            __builtin_amdgcn_sched_barrier(0);
+            compute_batch(t1, s + 1);
+        }
+        if (++chunk == nchunks) {
+            const float y = close_lanes8(acc);
+            if (c == 0) out[out_row] = y;
+            acc = 0.0f, chunk = 0, group += n_waves;
+        }
+    };
+    for (int t = 0; t < items; t += SETS) {
+#pragma unroll
+        for (int i = 0; i < SETS; ++i) {
+            if (t + i >= items) break;
+            turn(fs[i]);
+        }
+    }
+}
+
 // ---- Q6_K x Q8_K GEMV: the waves of the grid take the rows in turn, pass by pass, one pass fetched ahead -------
 // The activation (quants, scales, 16-value sums) is staged in LDS once per workgroup.
 // dynamic LDS: kQ6ActStride bytes per super-block, then cols/256 floats, then cols/16 int16 (each part 16-byte

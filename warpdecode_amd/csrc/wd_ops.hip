@@ -217,6 +217,27 @@ static int launch_gemv_q8_0(int type, MatSrc src, int mats, int rows, int cols, 
         WD_LAUNCH_CHECK();
         return WD_OK;
     }
+    if (type == WD_TYPE_Q8_0 && mats == 1 && src.single && nb % 16 == 0 && cols <= 16384 && rows >= 8 &&
+        reinterpret_cast<uintptr_t>(src.single) % 16 == 0 && reinterpret_cast<uintptr_t>(qs) % 16 == 0) {
+        // whole 16-byte words per row chunk and a 16-byte aligned base: the streaming kernel, eight rows per wave
+        const int groups = (rows + 7) / 8;
+        // Workgroups of four waves (taking several row groups each beyond 1024 workgroups) when there is a row group
+        // or more per SIMD; otherwise single waves, which keep two chunks in flight to cover the memory latency.
+        const int waves = groups >= 1024 ? 4 : 1;
+        int wgs_wanted = (groups + waves - 1) / waves;
+        wgs_wanted = std::min(wgs_wanted, waves == 4 ? 1024 : 2048);
+        const unsigned wgs = static_cast<unsigned>(wgs_wanted);
+        // single waves: 32-block chunks, two of them in flight; full workgroups: 16-block chunks, one ahead
+        const int kb = (waves == 1 && nb % 32 == 0) ? 32 : 16;
+        const size_t lds = static_cast<size_t>(cols) + static_cast<size_t>(nb) * 4 +
+                           static_cast<size_t>(waves) * 8 * (kb == 32 ? kQ8sRowStride<32> : kQ8sRowStride<16>);
+        auto launch = [&](auto kernel) { kernel<<<wgs, 64 * waves, lds, stream>>>(src.single, rows, nb, qs, d, out, partials); };
+        if (waves == 4) partials ? launch(k_gemv_q8_rows8<16, true, 4, 1>) : launch(k_gemv_q8_rows8<16, false, 4, 1>);
+        else if (kb == 32) partials ? launch(k_gemv_q8_rows8<32, true, 1, 2>) : launch(k_gemv_q8_rows8<32, false, 1, 2>);
+        else partials ? launch(k_gemv_q8_rows8<16, true, 1, 2>) : launch(k_gemv_q8_rows8<16, false, 1, 2>);
+        WD_LAUNCH_CHECK();
+        return WD_OK;
+    }
 #define WD_Q8_LAUNCH(KIND)                                                                                          \
     do {                                                                                                            \
         if (partials)                                                                                               \
