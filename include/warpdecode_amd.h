@@ -304,6 +304,18 @@ int wd_expert_cache_set_copy_kernel(wd_expert_cache *c, int enabled);
  * miss, instead of a pageable copy from the mapping.  reference: ExpertFileMap, ExpertPreadPool and the pinned ring of
  * ExpertStagePath (src/expert_cache.cuh:204-508, :1166-1254); there the file is found through /proc/self/maps. */
 int wd_expert_cache_attach_file(wd_expert_cache *c, const uint8_t *map_base, size_t map_bytes, int fd, int threads);
+/* The readable file mapping of this process that holds ptr, from /proc/self/maps: [start, end) in the address space,
+ * the file's path and the file offset of `start` (consecutive lines of one file that continue each other count as one).
+ * wd_expert_cache_attach_mappings looks every registered host tensor up that way, opens the files it finds and attaches
+ * them like wd_expert_cache_attach_file (tensors in anonymous or pinned memory are left to the other fill paths);
+ * n_attached (may be NULL) receives the number of mappings attached by the call.
+ * reference: ExpertFileMap::resolve, src/expert_cache.cuh:204-330. */
+typedef struct wd_file_mapping {
+    uint64_t start, end, file_offset;
+    char path[4096];
+} wd_file_mapping;
+int wd_file_mapping_of(const void *ptr, wd_file_mapping *out);
+int wd_expert_cache_attach_mappings(wd_expert_cache *cache, int threads, int *n_attached);
 int wd_expert_cache_add_shadow(wd_expert_cache *c, int policy, size_t slots);
 /* The monitor's counters as one JSON object (hit rate, bytes copied, per-layer accesses and misses, distinct pairs,
  * reuse of the previous call's experts per layer, host time spent in acquire, shadow hit rates).  Returns the length

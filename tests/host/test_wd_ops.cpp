@@ -419,7 +419,8 @@ static void gpu_checks() {
             GpuExpertCache cache;
             cache.initialize((12 * slot + (1u << 20) - 1) >> 20, *T[0].gate, *T[0].up, *T[0].down, 0, 0, 0, opt);
             for (int l = 0; l < layers; ++l) cache.register_layer_experts(l, *T[l].gate, *T[l].up, *T[l].down);
-            attach_expert_file(cache, g, 2);  // misses come through pread and the pinned ring
+            CHECK(attach_mapped_expert_files(cache, 2) == 1, "the model file's mapping is found through /proc/self/maps");
+            attach_expert_file(cache, g, 2);  // naming the file as well changes nothing: misses come through pread and the pinned ring
             Rng r(321);
             DeviceFloatArray dx(H), dout(H);
             for (int token = 0; token < 3; ++token)

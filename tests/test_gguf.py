@@ -2,6 +2,7 @@
 types, offsets, bytes and metadata must come back exactly, and malformed files must be refused with a message.
 The layout checked is the published GGUF one the reference's parser reads (src/gguf.hpp:394-470): v2/v3 header with
 u64 counts, typed key/values including arrays, tensor directory, data section at the next multiple of general.alignment."""
+import os
 import struct
 
 import numpy as np
@@ -116,3 +117,30 @@ def test_unknown_tensor_type_is_listed_without_size(tmp_path):
     with ggufio.GgufFile(path) as g:
         assert g.tensors["output.weight"]["bytes"] == 0 and g.tensors["output.weight"]["type"] == 12
         assert g.tensors["x"]["bytes"] == 34
+
+
+def test_file_mapping_lookup(tmp_path):
+    """wd_file_mapping_of finds a memory-mapped file (path, extent, file offset of the mapping's start) and refuses
+    anonymous memory; a mapping that starts inside the file reports its offset."""
+    import ctypes as C
+    import mmap
+    path = tmp_path / "blob.bin"
+    payload = np.arange(3 * 65536, dtype=np.uint8).tobytes()
+    path.write_bytes(payload)
+    lib = capi.load()
+    with open(path, "rb") as fh:
+        for offset in (0, 65536):
+            mm = mmap.mmap(fh.fileno(), len(payload) - offset, prot=mmap.PROT_READ, offset=offset)
+            view = np.frombuffer(mm, dtype=np.uint8)
+            addr = view.ctypes.data
+            m = capi.FileMapping()
+            assert lib.wd_file_mapping_of(C.c_void_p(addr + 1000), C.byref(m)) == 0
+            assert os.path.realpath(m.path.decode()) == os.path.realpath(str(path))
+            assert m.start <= addr and m.end >= addr + len(payload) - offset
+            assert m.file_offset + (addr - m.start) == offset
+            del view
+            mm.close()
+    anon = np.zeros(1 << 20, np.uint8)
+    m = capi.FileMapping()
+    assert lib.wd_file_mapping_of(C.c_void_p(anon.ctypes.data), C.byref(m)) == -1
+    assert b"no readable file mapping" in lib.wd_last_error()

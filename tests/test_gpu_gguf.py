@@ -102,11 +102,13 @@ def test_resident_stack_from_file(g, oracle, layers, tmp_path, fused):
     sc.close()
 
 
-@pytest.mark.parametrize("attach", ["no", "before", "after"], ids=["pageable", "pread-attached-first", "pread-attached-late"])
+@pytest.mark.parametrize("attach", ["no", "before", "after", "found"],
+                         ids=["pageable", "pread-attached-first", "pread-attached-late", "pread-found-in-proc-maps"])
 @pytest.mark.parametrize("fused", [False, True], ids=["separate", "gate_up"])
 def test_cached_stack_streams_experts_from_the_mapping(g, oracle, layers, tmp_path, fused, attach):
     """attach = no: the mapping is a pageable host source (hipMemcpyAsync per piece); otherwise the file is attached to
-    the cache and misses are read with pread() into the pinned ring (three reader threads), one DMA per miss."""
+    the cache (named by the caller, or found by the cache itself through /proc/self/maps) and misses are read with pread()
+    into the pinned ring (three reader threads), one DMA per miss."""
     import json
     gb = F * synth.row_bytes(synth.IQ3_S, H)
     db = H * synth.row_bytes(synth.Q8_0, F)
@@ -126,6 +128,12 @@ def test_cached_stack_streams_experts_from_the_mapping(g, oracle, layers, tmp_pa
                 capi.call("wd_expert_cache_register_layer", cache, l, ptr(L["gate"]), ptr(L["up"]), ptr(L["down"]))
         if attach == "after":
             capi.call("wd_expert_cache_attach_file", cache, C.c_void_p(gf.map_base), gf.map_bytes, gf.fd, 3)
+        if attach == "found":
+            n = C.c_int(0)
+            capi.call("wd_expert_cache_attach_mappings", cache, 3, C.byref(n))
+            assert n.value == 1          # one file holds every tensor
+            capi.call("wd_expert_cache_attach_mappings", cache, 3, C.byref(n))
+            assert n.value == 0          # nothing new the second time
         dls, arr = _descs(g, [dict(L, gate=L["gate"][:1], up=L["up"][:1], down=L["down"][:1]) for L in Ls])
         for i in range(NL):                  # routed tensors come from the cache only
             arr[i].gate = arr[i].up = arr[i].down = None

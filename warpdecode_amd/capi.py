@@ -38,6 +38,10 @@ class MoeLayer(C.Structure):
     ]
 
 
+class FileMapping(C.Structure):
+    _fields_ = [("start", C.c_uint64), ("end", C.c_uint64), ("file_offset", C.c_uint64), ("path", C.c_char * 4096)]
+
+
 class GgufTensorInfo(C.Structure):
     _fields_ = [("name", C.c_char_p), ("n_dims", C.c_uint32), ("dims", C.c_uint64 * 4), ("type", C.c_uint32),
                 ("relative_offset", C.c_uint64), ("bytes", C.c_uint64), ("data", vp)]
@@ -52,6 +56,8 @@ _SIGS = {
     "wd_init": (i32, [i32]),
     "wd_row_bytes": (sz, [i32, i32]),
     "wd_gemv_q6_k_q8_k_f32": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp]),
+    "wd_file_mapping_of": (i32, [vp, C.POINTER(FileMapping)]),
+    "wd_expert_cache_attach_mappings": (i32, [vp, i32, C.POINTER(i32)]),
     "wd_hc_combine_f32": (i32, [vp, vp, vp, i32, i32, i32, vp]),
     "wd_hc_combine_moe_f32": (i32, [vp, vp, vp, i32, vp, vp, i32, i32, i32, vp]),
     "wd_moe_layer_hc_f32": (i32, [C.POINTER(MoeLayer), vp, vp, vp, vp, i32, i32, vp, u32, vp]),

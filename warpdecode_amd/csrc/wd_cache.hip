@@ -20,10 +20,11 @@
 //     pread() of the expert's three slices into one entry of a pinned ring, shared out over a few worker threads
 //     (a single core does not reach the page cache's bandwidth), followed by ONE DMA of the whole slot from the
 //     ring entry; an entry is reused when the event recorded behind its DMA has completed.  Same role as the
-//     reference's ExpertFileMap / ExpertPreadPool / pinned ring (src/expert_cache.cuh:204-508, :858-1583), without
-//     the /proc/self/maps lookup: the file is named by the caller.
+//     reference's ExpertFileMap / ExpertPreadPool / pinned ring (src/expert_cache.cuh:204-508, :858-1583); the file
+//     is named by the caller or found through /proc/self/maps (wd_expert_cache_attach_mappings).
 #include "wd_common.h"
 
+#include <fcntl.h>
 #include <unistd.h>
 
 #include <atomic>
@@ -239,7 +240,49 @@ struct FileSource {
     const uint8_t *base = nullptr;  // start of the caller's read-only mapping of the file
     size_t size = 0;
     int fd = -1;                    // our own descriptor of the same file
+    uint64_t file_off = 0;          // offset in the file of the byte at `base`
 };
+
+// The file mapping that holds `ptr`, from /proc/self/maps ("start-end perms offset dev inode path"); consecutive lines
+// of one file whose addresses and offsets continue each other count as one mapping.  Same role as the reference's
+// ExpertFileMap (src/expert_cache.cuh:204-330).
+bool find_file_mapping(const void *ptr, wd_file_mapping *out) {
+    FILE *maps = std::fopen("/proc/self/maps", "r");
+    if (!maps) return false;
+    const uint64_t want = reinterpret_cast<uintptr_t>(ptr);
+    char line[4352];
+    uint64_t run_start = 0, run_end = 0, run_off = 0;
+    std::string run_path;
+    bool found = false;
+    auto flush = [&]() {
+        if (!run_path.empty() && want >= run_start && want < run_end) {
+            out->start = run_start, out->end = run_end, out->file_offset = run_off;
+            std::snprintf(out->path, sizeof(out->path), "%s", run_path.c_str());
+            found = run_path.size() < sizeof(out->path);
+        }
+    };
+    while (!found && std::fgets(line, sizeof(line), maps)) {
+        unsigned long long a = 0, b = 0, off = 0, inode = 0;
+        char perms[8] = {0}, dev[16] = {0};
+        int at = 0;
+        if (std::sscanf(line, "%llx-%llx %7s %llx %15s %llu %n", &a, &b, perms, &off, dev, &inode, &at) < 6) continue;
+        std::string path(line + at);
+        while (!path.empty() && (path.back() == '\n' || path.back() == ' ')) path.pop_back();
+        const bool file = inode != 0 && !path.empty() && path[0] == '/' && perms[0] == 'r';
+        if (file && path == run_path && a == run_end && off == run_off + (run_end - run_start)) {
+            run_end = b;  // the same file goes on
+            continue;
+        }
+        flush();
+        if (file)
+            run_start = a, run_end = b, run_off = off, run_path = path;
+        else
+            run_path.clear();
+    }
+    if (!found) flush();
+    std::fclose(maps);
+    return found;
+}
 
 constexpr int kStageRing = 16;  // pinned ring entries of one slot each
 
@@ -412,7 +455,45 @@ int wd_expert_cache_destroy(wd_expert_cache *c) {
     return WD_OK;
 }
 
+static int attach_file_at(wd_expert_cache *c, const uint8_t *map_base, size_t map_bytes, int fd, uint64_t file_off, int threads);
+
 int wd_expert_cache_attach_file(wd_expert_cache *c, const uint8_t *map_base, size_t map_bytes, int fd, int threads) {
+    return attach_file_at(c, map_base, map_bytes, fd, 0, threads);
+}
+
+int wd_file_mapping_of(const void *ptr, wd_file_mapping *out) {
+    WD_REQUIRE(ptr != nullptr && out != nullptr, "file mapping lookup: null pointer");
+    std::memset(out, 0, sizeof(*out));
+    if (!find_file_mapping(ptr, out)) return fail(WD_ERR_ARG, "no readable file mapping holds %p", ptr);
+    return WD_OK;
+}
+
+int wd_expert_cache_attach_mappings(wd_expert_cache *c, int threads, int *n_attached) {
+    WD_REQUIRE(c != nullptr, "expert cache is not initialized");
+    int attached = 0;
+    for (int l = 0; l < c->n_layers; ++l) {
+        if (!c->h_gate[l]) continue;
+        const uint8_t *ptrs[3] = {c->h_gate[l], c->h_up[l], c->h_down[l]};
+        for (const uint8_t *p : ptrs) {
+            bool known = false;
+            for (const FileSource &f : c->files) known = known || (p >= f.base && p < f.base + f.size);
+            if (known) continue;
+            wd_file_mapping m;
+            if (!find_file_mapping(p, &m)) continue;  // anonymous or pinned memory: the other fill paths take it
+            const int fd = ::open(m.path, O_RDONLY | O_CLOEXEC);
+            if (fd < 0) continue;
+            const int rc = attach_file_at(c, reinterpret_cast<const uint8_t *>(static_cast<uintptr_t>(m.start)),
+                                          static_cast<size_t>(m.end - m.start), fd, m.file_offset, threads);
+            ::close(fd);  // the cache keeps a duplicate
+            if (rc != WD_OK) return rc;
+            ++attached;
+        }
+    }
+    if (n_attached) *n_attached = attached;
+    return WD_OK;
+}
+
+static int attach_file_at(wd_expert_cache *c, const uint8_t *map_base, size_t map_bytes, int fd, uint64_t file_off, int threads) {
     WD_REQUIRE(c != nullptr, "expert cache is not initialized");
     WD_REQUIRE(map_base != nullptr && map_bytes > 0 && fd >= 0, "expert cache: invalid file mapping");
     WD_REQUIRE(threads >= 1 && threads <= 64, "expert cache: 1..64 pread threads (got %d)", threads);
@@ -430,7 +511,7 @@ int wd_expert_cache_attach_file(wd_expert_cache *c, const uint8_t *map_base, siz
     }
     if (!c->pread_pool) c->pread_pool = new PreadPool(threads);
     FileSource f;
-    f.base = map_base, f.size = map_bytes, f.fd = own;
+    f.base = map_base, f.size = map_bytes, f.fd = own, f.file_off = file_off;
     c->files.push_back(f);
     for (int l = 0; l < c->n_layers; ++l)  // layers registered before the file was attached
         if (c->h_gate[l]) classify_layer(c, l);
@@ -619,7 +700,7 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
             int n_pieces = 0;
             size_t at = 0;
             for (int q = 0; q < 3; ++q) {  // pieces of about 256 KiB so that the workers share one expert
-                const uint64_t file_off = static_cast<uint64_t>(src3[q] - fs.base);
+                const uint64_t file_off = fs.file_off + static_cast<uint64_t>(src3[q] - fs.base);
                 const size_t parts = len3[q] >= (512u << 10) ? 4 : (len3[q] >= (256u << 10) ? 2 : 1);
                 for (size_t pi = 0; pi < parts; ++pi) {
                     const size_t lo = len3[q] * pi / parts, hi = len3[q] * (pi + 1) / parts;

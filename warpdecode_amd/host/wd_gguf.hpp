@@ -80,6 +80,14 @@ inline void attach_expert_file(GpuExpertCache &cache, const GgufFile &g, int thr
     check(wd_expert_cache_attach_file(cache.handle(), g.map_base(), g.map_bytes(), g.fd(), threads), "wd_expert_cache_attach_file");
 }
 
+// The same without naming the file: every registered host tensor is looked up in /proc/self/maps and the files found
+// are attached (returns how many).  reference: ExpertFileMap::resolve, src/expert_cache.cuh:221-243.
+inline int attach_mapped_expert_files(GpuExpertCache &cache, int threads = 4) {
+    int n = 0;
+    check(wd_expert_cache_attach_mappings(cache.handle(), threads, &n), "wd_expert_cache_attach_mappings");
+    return n;
+}
+
 struct Qwen38MoeLayerTensors {
     const TensorInfo *router = nullptr;
     const TensorInfo *gate_up = nullptr;  // one tensor of 2*ffn rows per expert, when the file stores it so
