@@ -400,6 +400,32 @@ static void gpu_checks() {
             check(wd_memcpy_d2h(back.data(), v.gate.data, v.gate.bytes, nullptr), "slot read-back");
             CHECK(std::memcmp(back.data(), expert_slice(L[0].t_gate, 5).data, v.gate.bytes) == 0 && !v.gate.owns, "acquired view must hold the expert's gate bytes");
         }
+        // a batch of tokens through each layer (resident: on the device throughout; LRU pool of 10 slots: the union of
+        // two tokens' experts is acquired at once), every token against its own oracle pass
+        {
+            const int T = mode == 0 ? 3 : 2;
+            std::vector<Qwen38MoeScratch> ts(T);
+            std::vector<Qwen38MoeScratch *> tp;
+            for (auto &q : ts) q.initialize(E, k, H, F), tp.push_back(&q);
+            Rng rt(555 + mode);
+            DeviceFloatArray dxs(static_cast<size_t>(T) * H), douts(static_cast<size_t>(T) * H);
+            for (int l = 0; l < layers; ++l) {
+                std::vector<float> xs(static_cast<size_t>(T) * H);
+                for (int t = 0; t < T; ++t) {
+                    const std::vector<float> x = rms_normed(rt, H);
+                    std::copy(x.begin(), x.end(), xs.begin() + static_cast<size_t>(t) * H);
+                }
+                dxs.upload(xs.data(), xs.size());
+                run_qwen38_moe_tokens_f32_x(l, dxs.data, T, routers[l], L[l].t_gate, L[l].t_up, L[l].t_down, cache, shared[l], tp, douts.data, 1.0f, stream);
+                check(wd_stream_sync(stream), "sync");
+                std::vector<float> got(xs.size()), want(H);
+                douts.download(got.data());
+                for (int t = 0; t < T; ++t) {
+                    wdo_moe_layer(&L[l].o, xs.data() + static_cast<size_t>(t) * H, want.data(), nullptr, 0);
+                    CHECK(same_bits(got.data() + static_cast<size_t>(t) * H, want.data(), H), "mode %d layer %d token %d of the batch differs from the oracle", mode, l, t);
+                }
+            }
+        }
     }
     // the same stack driven from a model file: tensors found by name, router / shared expert uploaded from the mapping,
     // the mapping itself as the cache's host source (LRU pool, so experts stream from the file's pages)

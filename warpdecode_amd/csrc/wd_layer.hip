@@ -599,8 +599,12 @@ extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, 
     }
     hipStream_t st = as_stream(stream);
     const int H = L->hidden, F = L->expert_ffn, k = L->top_k;
-    const bool union_path = !(flags & WD_MOE_STAGED) && consumes_q8k(L->gate_type) && L->down_type == WD_TYPE_Q8_0 &&
-                            F <= 512 && tokens * k <= 128 && scratch_per_token[0]->gup == nullptr;
+    // the union pass over the gate/up tensors needs the IQ types; the multi-token down dispatch needs Q8_0 rows of at
+    // most 16 blocks (other down tensors take the one-token dispatch per token, on the activations the union pass left)
+    const bool union_path = !(flags & WD_MOE_STAGED) && consumes_q8k(L->gate_type) && tokens * k <= 128 &&
+                            scratch_per_token[0]->gup == nullptr &&
+                            !(flags & (WD_MOE_ONLY_A | WD_MOE_ONLY_B | WD_MOE_ONLY_C | WD_MOE_DRY));
+    const bool down_tokens = L->down_type == WD_TYPE_Q8_0 && F <= 512;
     if (!union_path) {
         // same results, one pass per token (every pass reads its own experts)
         for (int t = 0; t < tokens; ++t)
@@ -645,6 +649,13 @@ extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, 
             k_tokens_b<22, kMaxTokens><<<dim3(grid_b), dim3(512), lds_b, st>>>(ta);
     }
     WD_LAUNCH_CHECK();
+    if (!down_tokens) {
+        for (int t = 0; t < tokens; ++t)
+            if (const int rc = layer_fused(L, d_x + static_cast<size_t>(t) * H, d_out + static_cast<size_t>(t) * H, scratch_per_token[t],
+                                           flags | WD_MOE_ONLY_C, nullptr, nullptr, 0.0f, st))
+                return rc;
+        return WD_OK;
+    }
     const int waves_c = 16;
     const size_t per_wave = (static_cast<size_t>(F) + F / 16 + 15) & ~static_cast<size_t>(15);
     const size_t lds_c = waves_c * per_wave + sizeof(float) * 8 * tokens * (k + 1);

@@ -660,6 +660,49 @@ inline void run_qwen38_moe_layer_f32_x(int layer, const float *x, const GpuMatri
     check(wd_moe_layer_f32(&L, x, out, scratch.handle(), 0u, stream), "MoE layer failed");
 }
 
+// M tokens through one layer, every selected expert read once for all the tokens that chose it (the MTP block's
+// block_moe, src/qwen38_mtp.cuh:674-795, with Qwen38MoeTokenBatch, src/qwen38_moe.cuh:2743-3237: router and selection of
+// every token, the union of their experts acquired from the cache, one batch pass, then the shared expert and the
+// combine per token).  x and out are [tokens][hidden]; every token has a scratch of its own, which afterwards holds that
+// token's ids, weights, routed sum and shared-expert output exactly as after a one-token call.  When the layer's experts
+// are all resident nothing leaves the device; otherwise the ids of all tokens go to the host once, the union is acquired
+// (the cache must have room for it) and the pass runs on the given selection.
+inline void run_qwen38_moe_tokens_f32_x(int layer, const float *x, int tokens, const GpuMatrix &router, const TensorInfo &gate_exps,
+                                        const TensorInfo &up_exps, const TensorInfo &down_exps, GpuExpertCache &cache,
+                                        const Qwen38SharedExpertWeights &shared, const std::vector<Qwen38MoeScratch *> &scratch, float *out,
+                                        float expert_scale, Stream stream) {
+    if (tokens <= 0 || static_cast<size_t>(tokens) != scratch.size()) throw std::runtime_error("token batch: one scratch per token is required");
+    wd_moe_layer L;
+    detail::fill_routed(L, layer, router, gate_exps, up_exps, down_exps, cache, *scratch[0], expert_scale);
+    L.shared_gate_inp = shared.gate_input_f32.data;
+    L.shared_gate = shared.gate.data, L.shared_up = shared.up.data, L.shared_down = shared.down.data;
+    std::vector<wd_moe_scratch *> handles;
+    for (const Qwen38MoeScratch *s : scratch) handles.push_back(s->handle());
+    if (cache.layer_resident(layer)) {
+        check(wd_moe_layer_tokens_f32(&L, x, out, tokens, handles.data(), 0u, stream), "MoE token batch failed");
+        return;
+    }
+    const int k = L.top_k, H = L.hidden;
+    for (int t = 0; t < tokens; ++t) {
+        check(wd_moe_layer_f32(&L, x + static_cast<size_t>(t) * H, out + static_cast<size_t>(t) * H, handles[t], WD_MOE_ONLY_A, stream),
+              "MoE router failed");
+        check(wd_memcpy_d2h(scratch[t]->h_ids(), scratch[t]->d_ids(), sizeof(int) * k, stream), "routed ids copy failed");
+    }
+    check(wd_stream_sync(stream), "stream synchronisation failed");
+    std::vector<int> unique;
+    for (int t = 0; t < tokens; ++t)
+        for (int j = 0; j < k; ++j) {
+            const int e = scratch[t]->h_ids()[j];
+            if (std::find(unique.begin(), unique.end(), e) == unique.end()) unique.push_back(e);
+        }
+    cache.register_layer_experts(layer, gate_exps, up_exps, down_exps);
+    for (size_t at = 0; at < unique.size(); at += 16)  // most recently acquired experts are the last to be recycled
+        cache.acquire_ids(layer, unique.data() + at, static_cast<int>(std::min<size_t>(16, unique.size() - at)), stream);
+    for (int e : unique)
+        if (wd_expert_cache_slot_of(cache.handle(), layer, e) < 0) throw std::runtime_error("token batch: the expert cache is too small for the union of the tokens' experts");
+    check(wd_moe_layer_tokens_f32(&L, x, out, tokens, handles.data(), WD_MOE_PRESELECTED, stream), "MoE token batch failed");
+}
+
 // The F32 inject projections of the hyper-connection combine (the part of the reference's Qwen38HcF32DebugScratch that
 // the combine reads: hidden(), hc(), inject(); src/qwen38_hc.cuh:2263-2330).
 class Qwen38HcF32DebugScratch {
