@@ -431,7 +431,8 @@ def bench_q8_sweep(args, torch, capi, synth):
     """Dense exact-order Q8_0 x Q8_0 GEMV at batch=1 (the projections around the MoE layer: hyper-connection mix, attention
     and recurrent blocks, src/qwen38_hc.cuh:1020-1049) over square, wide, tall and head-sized shapes.  Every launch of a
     chain reads another copy of the matrix (>= 1.5 GB of copies); the period is taken over a captured chain."""
-    shapes = [(2048, 2048), (8192, 2048), (2048, 8192), (512, 8192), (8192, 512), (8192, 8192), (32768, 2048), (151936, 2048)]
+    shapes = [(2048, 2048), (8192, 2048), (2048, 8192), (512, 8192), (8192, 512), (1024, 4096), (4096, 8192), (8192, 8192),
+              (32768, 2048), (151936, 2048)]
     results = []
     for rows, cols in shapes:
         nbytes = rows * synth.row_bytes(synth.Q8_0, cols)

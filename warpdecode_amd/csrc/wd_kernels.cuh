@@ -451,6 +451,122 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(WAVE
     }
 }
 
+// ---- dense Q8_0 x Q8_0 GEMV, few rows: the waves of a workgroup share the eight rows of a group --------------------
+// With few row groups a group's wave runs alone on its SIMD and the time is the length of its chains (about 40 cycles
+// per block: one wave issues an instruction every four cycles and a block is ten of them).  Only the fma itself has to
+// run in block order.  So wave v of a workgroup takes blocks [v NCH*32, (v+1) NCH*32) of the eight rows, requests all
+// of them at once, turns them into (d_w d_a, float(dot4)) pairs in registers at its own pace, and then the waves run
+// their parts of the chains one after the other, handing the 64 accumulators on through LDS: NCH*32 dependent fma per
+// wave, nothing else.  Lane = 8 row + chain as in k_gemv_q8_rows8; nb = 32 NCH WAVES blocks per row.
+// dynamic LDS: cols bytes, cols/32 floats, 256 bytes of accumulators, then one stage of 8 * kQ8sRowStride<32> per wave.
+template <int NCH, int WAVES, bool PART>
+__global__ __launch_bounds__(64 * WAVES) void k_gemv_q8_rows8_split(const uint8_t *__restrict__ w, int rows, int nb,
+                                                              const int8_t *__restrict__ act_qs, const uint16_t *__restrict__ act_d,
+                                                              float *__restrict__ out, int32_t *__restrict__ partials) {
+    constexpr int KB = 32, SEG = NCH * KB;
+    using Fetch = Q8sFetch<KB>;
+    constexpr int RS = kQ8sRowStride<KB>;
+    extern __shared__ __align__(16) uint8_t q8p_lds[];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int cols = nb * 32;
+    int8_t *aq = reinterpret_cast<int8_t *>(q8p_lds);
+    float *ad = reinterpret_cast<float *>(q8p_lds + cols);
+    float *carry = reinterpret_cast<float *>(q8p_lds + cols + nb * 4);
+    uint8_t *stage = q8p_lds + cols + nb * 4 + 256 + wave * (8 * RS);
+    const size_t rb = static_cast<size_t>(nb) * 34;
+    const int row = lane >> 3, c = lane & 7;
+    // a last group of fewer than eight rows is moved up to end with the matrix (rows >= 8)
+    const int base_row = min(8 * static_cast<int>(blockIdx.x), rows - 8);
+    const uint8_t *src = uniform_ptr(w + static_cast<size_t>(base_row) * rb + static_cast<size_t>(wave) * (34 * SEG));
+    uint32_t loff[Fetch::kLoads];
+    Fetch f[NCH];
+#pragma unroll
+    for (int i = 0; i < Fetch::kLoads; ++i) {
+        const int u = min(i * 64 + lane, Fetch::kWords - 1);
+        const int r = u / Fetch::kWordsPerRow, within = u - r * Fetch::kWordsPerRow;
+        loff[i] = static_cast<uint32_t>(r * RS + 16 * within);
+        const uint32_t goff = static_cast<uint32_t>(r * rb + 16 * within);
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch) f[ch].u[i] = gld_u128_aligned(src + goff + ch * (34 * KB));
+    }
+    for (int i = threadIdx.x; i < cols / 16; i += 64 * WAVES) reinterpret_cast<uint4 *>(aq)[i] = reinterpret_cast<const uint4 *>(act_qs)[i];
+    for (int i = threadIdx.x; i < nb; i += 64 * WAVES) ad[i] = h2f(act_d[i]);
+    __syncthreads();
+    const uint8_t *my = stage + row * RS + 4 * c;
+    const int8_t *my_a = aq + 4 * c;
+    const int first_block = wave * SEG;
+    int32_t *pp = PART ? partials + (static_cast<size_t>(base_row + row) * nb) * 8 + c : nullptr;
+    float dv[SEG], pv[SEG];
+    struct Batch {
+        uint32_t w[12];  // blocks 0 2 4 6 of the batch: two dwords each (w[3i], w[3i+1]); blocks 1 3 5 7: w[3i+2]
+        uint32_t dw[8], a[8];
+        float4 da[2];
+    };
+    auto load_batch = [&](Batch &t, int b0, int s) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint8_t *blk = my + 34 * (8 * s + 2 * i);
+            t.w[3 * i] = *reinterpret_cast<const uint32_t *>(blk);
+            t.w[3 * i + 1] = *reinterpret_cast<const uint32_t *>(blk + 4);
+            t.w[3 * i + 2] = *reinterpret_cast<const uint32_t *>(blk + 36);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            t.dw[i] = *reinterpret_cast<const uint16_t *>(stage + row * RS + 34 * (8 * s + i));
+            t.a[i] = *reinterpret_cast<const uint32_t *>(my_a + 32 * (b0 + 8 * s + i));
+        }
+        t.da[0] = *reinterpret_cast<const float4 *>(ad + b0 + 8 * s);
+        t.da[1] = *reinterpret_cast<const float4 *>(ad + b0 + 8 * s + 4);
+    };
+#pragma unroll
+    for (int ch = 0; ch < NCH; ++ch) {
+        wave_lds_fence();  // the previous chunk has been read
+#pragma unroll
+        for (int i = 0; i < Fetch::kLoads; ++i) *reinterpret_cast<uint4 *>(stage + loff[i]) = f[ch].u[i];
+        wave_lds_fence();
+        const int b0 = first_block + ch * KB;
+        auto pairs = [&](const Batch &bt, int s) {
+            const float da[8] = {bt.da[0].x, bt.da[0].y, bt.da[0].z, bt.da[0].w, bt.da[1].x, bt.da[1].y, bt.da[1].z, bt.da[1].w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t q = (i & 1) ? bt.w[3 * (i >> 1) + 2]
+                                           : __builtin_amdgcn_alignbyte(bt.w[3 * (i >> 1) + 1], bt.w[3 * (i >> 1)], 2);
+                const int p = sdot4(q, bt.a[i], 0);
+                if (PART) pp[(b0 + 8 * s + i) * 8] = p;
+                dv[ch * KB + 8 * s + i] = h2f(static_cast<uint16_t>(bt.dw[i])) * da[i];
+                pv[ch * KB + 8 * s + i] = static_cast<float>(p);
+            }
+        };
+        Batch t0, t1;
+        load_batch(t0, b0, 0);
+#pragma unroll
+        for (int s = 0; s < KB / 8; s += 2) {
+            load_batch(t1, b0, s + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            pairs(t0, s);
+            if (s + 2 < KB / 8) load_batch(t0, b0, s + 2);
+            __builtin_amdgcn_sched_barrier(0);
+            pairs(t1, s + 1);
+        }
+    }
+    // the chains, one wave after the other in block order
+    float acc = 0.0f;
+#pragma unroll
+    for (int turn = 0; turn < WAVES; ++turn) {
+        if (wave == turn) {
+            if (turn > 0) acc = carry[lane];
+#pragma unroll
+            for (int i = 0; i < SEG; ++i) acc = __builtin_fmaf(dv[i], pv[i], acc);
+            if (turn < WAVES - 1) carry[lane] = acc;
+        }
+        if (turn < WAVES - 1) __syncthreads();
+    }
+    if (wave == WAVES - 1) {
+        const float y = close_lanes8(acc);
+        if (c == 0) out[base_row + row] = y;
+    }
+}
+
 // ---- Q6_K x Q8_K GEMV: the waves of the grid take the rows in turn, pass by pass, one pass fetched ahead -------
 // The activation (quants, scales, 16-value sums) is staged in LDS once per workgroup.
 // dynamic LDS: kQ6ActStride bytes per super-block, then cols/256 floats, then cols/16 int16 (each part 16-byte

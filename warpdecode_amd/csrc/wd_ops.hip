@@ -221,6 +221,20 @@ static int launch_gemv_q8_0(int type, MatSrc src, int mats, int rows, int cols, 
         reinterpret_cast<uintptr_t>(src.single) % 16 == 0 && reinterpret_cast<uintptr_t>(qs) % 16 == 0) {
         // whole 16-byte words per row chunk and a 16-byte aligned base: the streaming kernel, eight rows per wave
         const int groups = (rows + 7) / 8;
+        if (groups < 1024 && (nb == 64 || nb == 128 || nb == 256 || nb == 512)) {
+            // few row groups: the waves of a workgroup share a group, the chain runs over prepared pairs
+            int waves = nb == 64 ? 2 : (nb == 128 ? 4 : 8);
+            if (nb == 256 && groups > 256) waves = 4;  // more than one workgroup per compute unit: smaller ones
+            const size_t lds = static_cast<size_t>(cols) + static_cast<size_t>(nb) * 4 + 256 + static_cast<size_t>(waves) * 8 * kQ8sRowStride<32>;
+            auto launch = [&](auto kernel) { kernel<<<groups, 64 * waves, lds, stream>>>(src.single, rows, nb, qs, d, out, partials); };
+            if (nb == 64) partials ? launch(k_gemv_q8_rows8_split<1, 2, true>) : launch(k_gemv_q8_rows8_split<1, 2, false>);
+            else if (nb == 128) partials ? launch(k_gemv_q8_rows8_split<1, 4, true>) : launch(k_gemv_q8_rows8_split<1, 4, false>);
+            else if (nb == 256 && waves == 8) partials ? launch(k_gemv_q8_rows8_split<1, 8, true>) : launch(k_gemv_q8_rows8_split<1, 8, false>);
+            else if (nb == 256) partials ? launch(k_gemv_q8_rows8_split<2, 4, true>) : launch(k_gemv_q8_rows8_split<2, 4, false>);
+            else partials ? launch(k_gemv_q8_rows8_split<2, 8, true>) : launch(k_gemv_q8_rows8_split<2, 8, false>);
+            WD_LAUNCH_CHECK();
+            return WD_OK;
+        }
         // Workgroups of four waves (taking several row groups each beyond 1024 workgroups) when there is a row group
         // or more per SIMD; otherwise single waves, which keep two chunks in flight to cover the memory latency.
         const int waves = groups >= 1024 ? 4 : 1;
