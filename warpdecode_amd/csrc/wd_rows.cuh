@@ -513,6 +513,18 @@ WD_DEV Q8Block q8_load(const uint8_t *blk) {
     return w;
 }
 
+// The IQ4_NL codebook values of four 4-bit codes (one per byte of idx, each 0..15) as four int8: the 16 values are four
+// dwords, v_perm_b32 picks among eight bytes, so the codes' low three bits select in both halves of the table and
+// bit 3 chooses the half (src/lowbit.cuh:1648-1668 reads kvalues_iq4nl[code]).
+WD_DEV uint32_t iq4nl_values(uint32_t idx) {
+    // {-127, -104, -83, -65}, {-49, -35, -22, -10}, {1, 13, 25, 38}, {53, 69, 89, 113}
+    constexpr uint32_t t0 = 0xbfad9881u, t1 = 0xf6eaddcfu, t2 = 0x26190d01u, t3 = 0x71594535u;
+    const uint32_t sel = idx & 0x07070707u;
+    const uint32_t lo = __builtin_amdgcn_perm(t1, t0, sel), hi = __builtin_amdgcn_perm(t3, t2, sel);
+    const uint32_t upper = ((idx >> 3) & 0x01010101u) * 0xffu;  // 0xff in the bytes whose code is 8..15
+    return (hi & upper) | (lo & ~upper);
+}
+
 template <int KIND>
 WD_DEV void q8_chunks(const Q8Block &w, const uint32_t (&a)[8], int (&p)[8]) {
     if (KIND == 0) {
@@ -524,16 +536,8 @@ WD_DEV void q8_chunks(const Q8Block &w, const uint32_t (&a)[8], int (&p)[8]) {
         const uint32_t n[4] = {w.q0.x, w.q0.y, w.q0.z, w.q0.w};
 #pragma unroll
         for (int l = 0; l < 4; ++l) {
-            int lo = 0, hi = 0;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t byte = (n[l] >> (8 * j)) & 0xffu;
-                constexpr int8_t lut[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
-                lo += static_cast<int>(lut[byte & 15u]) * static_cast<int>(static_cast<int8_t>(a[l] >> (8 * j)));
-                hi += static_cast<int>(lut[byte >> 4]) * static_cast<int>(static_cast<int8_t>(a[l + 4] >> (8 * j)));
-            }
-            p[l] = lo;
-            p[l + 4] = hi;
+            p[l] = sdot4(iq4nl_values(n[l] & 0x0f0f0f0fu), a[l], 0);
+            p[l + 4] = sdot4(iq4nl_values((n[l] >> 4) & 0x0f0f0f0fu), a[l + 4], 0);
         }
     }
 }
