@@ -47,7 +47,7 @@ def parse():
     ap.add_argument("--experts", type=int, default=512)
     ap.add_argument("--routing", choices=["zipf", "router"], default="zipf",
                     help="zipf: ids replayed from the Zipf(1.1) trace; router: ids chosen by the router itself")
-    ap.add_argument("--mode", choices=["resident", "lru", "q4-sweep", "q8-sweep", "q6k-head", "hc", "tokens", "c0"], default="resident",
+    ap.add_argument("--mode", choices=["resident", "lru", "q4-sweep", "q8-sweep", "q6k-head", "hc", "tokens", "c0", "model-layer"], default="resident",
                     help="resident: C3 mode A, every expert in HBM; lru: C3 mode B, experts in pinned host memory "
                          "behind an LRU slot pool of --cache-gib in HBM; q4-sweep: the dense Q4_0 GEMV shapes; "
                          "tokens: the 4-token speculative-verify pass over the same layers; c0: the 64-expert top-8 "
@@ -427,6 +427,73 @@ def bench_q4_sweep(args, torch, capi, synth):
                          kernel="k_gemv_q8<Q4_0>", us_per_launch=head["us_per_gemv"], bytes_per_launch=head["bytes"])}))
 
 
+def bench_model_layer(args, torch, capi, synth):
+    """The layer at the model's own tensor types and shapes (hidden 2560, ffn 640, 512 experts, top-10, IQ2_S gate/up,
+    IQ4_NL down, Q8_0 shared expert): `--layers` independent layers chained as in the headline workload,
+    router-selected experts, one token per step."""
+    H, F, k, E, NL = 2560, 640, 10, args.experts, min(args.layers, 16)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(synth.BASE_SEED + 6)
+    rb_g, rb_d = synth.row_bytes(synth.IQ2_S, H), synth.row_bytes(synth.IQ4_NL, F)
+    rb_qh, rb_qf = synth.row_bytes(synth.Q8_0, H), synth.row_bytes(synth.Q8_0, F)
+
+    def blocks(rows, cols, block_bytes, block_elems, scale):
+        nb = rows * (cols // block_elems)
+        t = torch.randint(0, 256, (nb * block_bytes,), dtype=torch.uint8, device="cuda", generator=g)
+        d = (torch.randn(nb, device="cuda", generator=g).abs() * scale).half()
+        t.view(-1, block_bytes)[:, 0:2] = d.view(torch.uint8).view(-1, 2)
+        return t
+
+    def q8(rows, cols):
+        nb = rows * (cols // 32)
+        t = torch.randint(-127, 128, (nb * 34,), dtype=torch.int8, device="cuda", generator=g).view(torch.uint8)
+        d = (torch.randn(nb, device="cuda", generator=g).abs() * (0.02 / 127.0)).half()
+        t.view(-1, 34)[:, 0:2] = d.view(torch.uint8).view(-1, 2)
+        return t
+
+    layers, keep = (capi.MoeLayer * NL)(), []
+    for l in range(NL):
+        t = dict(router=torch.randn(E, H, device="cuda", generator=g) * (1.0 / np.sqrt(H)),
+                 gate=blocks(E * F, H, 82, 256, 0.0004), up=blocks(E * F, H, 82, 256, 0.0004), down=blocks(E * H, F, 18, 32, 0.0002),
+                 shared_gate_inp=torch.randn(H, device="cuda", generator=g) * 0.02,
+                 shared_gate=q8(F, H), shared_up=q8(F, H), shared_down=q8(H, F))
+        keep.append(t)
+        d = layers[l]
+        d.hidden, d.expert_ffn, d.n_experts, d.top_k, d.expert_scale = H, F, E, k, 1.0
+        d.gate_type = d.up_type = synth.IQ2_S
+        d.down_type = synth.IQ4_NL
+        for name, tensor in t.items():
+            setattr(d, name, tensor.data_ptr())
+        d.gate_stride = d.up_stride = F * rb_g
+        d.down_stride = H * rb_d
+    scratch = C.c_void_p()
+    capi.call("wd_moe_scratch_create", C.byref(scratch), H, F, E, k)
+    rng = synth.rng_for(synth.BASE_SEED, 9400)
+    d_x = torch.from_numpy(synth.rms_normed(rng, H)).cuda()
+    d_out = torch.zeros(H, dtype=torch.float32, device="cuda")
+
+    def launch(_i):
+        capi.call("wd_moe_stack_f32", layers, NL, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()), scratch, None,
+                  RESIDUAL_SCALE, 0, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+    us = graph_period_us(torch, launch, 1, 50) / NL
+    finite, waits_ok = bool(torch.isfinite(d_x).all().item()), capi.load().wd_moe_scratch_status(scratch) == 0
+    note("finite %s, |x| max %.3g, in-dispatch waits ok %s" % (finite, float(d_x.abs().max().item()), waits_ok))
+    ok = finite and waits_ok
+    nbytes = E * H * 4 + H * 4 + k * (2 * F * rb_g + H * rb_d) + 2 * F * rb_qh + H * rb_qf
+    note("model-shape layer: %.2f us per layer, %.0f GB/s" % (us, nbytes / us / 1e3))
+    print(json.dumps({
+        "metric": "MoE layer batch=1 decode at the model's own types and shapes: us per layer", "value": round(us, 2), "unit": "us",
+        "n_gpus": 1, "higher_is_better": False, "vs_baseline": None,
+        "dtype": "int8 dot products (IQ2_S/IQ4_NL/Q8_0 weights x Q8_K/Q8_0 activations), f32 accumulate", "data": "synthetic",
+        "config": {"workload": "%d chained layers of hidden 2560, %d experts, top-10, ffn 640, IQ2_S gate/up, IQ4_NL down, "
+                               "Q8_0 shared expert, router-selected, batch=1, HIP-graph replay" % (NL, E),
+                   "layers": NL, "bytes_per_layer": nbytes, "valid": ok},
+        "roofline": dict(bound="hbm", achieved=round(nbytes / us / 1e3, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                         frac=round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), traffic=None,
+                         kernel="whole layer (k_layer_ab<IQ2_S>, k_layer_c<IQ4_NL>)")}))
+
+
 def bench_q8_sweep(args, torch, capi, synth):
     """Dense exact-order Q8_0 x Q8_0 GEMV at batch=1 (the projections around the MoE layer: hyper-connection mix, attention
     and recurrent blocks, src/qwen38_hc.cuh:1020-1049) over square, wide, tall and head-sized shapes.  Every launch of a
@@ -709,6 +776,8 @@ def main():
         return bench_q8_sweep(args, torch, capi, synth)
     if args.mode == "c0":
         return bench_c0(args, torch, capi, synth)
+    if args.mode == "model-layer":
+        return bench_model_layer(args, torch, capi, synth)
     if args.mode == "q6k-head":
         return bench_q6k_head(args, torch, capi, synth)
     note("generating %d layers x %d experts on the device" % (NL, E))

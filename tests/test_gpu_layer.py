@@ -104,6 +104,16 @@ def test_model_shape_layers(g, oracle, gate_t, down_t):
     check_layer(g, oracle, L, x)
 
 
+@pytest.mark.parametrize("shared", [True, False])
+def test_iq4_nl_down_rows_of_16_blocks(g, oracle, shared):
+    """IQ4_NL down projection at ffn 512: the aligned fetch of four 16-block rows (with and without the Q8_0 shared
+    expert, which takes the same routine)."""
+    H, F, E, k = 2048, 512, 16, 5
+    L = synth.make_layer(H, F, E, k, synth.IQ3_S, synth.IQ4_NL, shared, seed=SEED, layer=78, router_sigma=1.0 / np.sqrt(H))
+    x = synth.rms_normed(synth.rng_for(SEED, 50), H)
+    check_layer(g, oracle, L, x)
+
+
 def test_c0_layer(g, oracle):
     """Workload C0: hidden 2048, 64 experts, top-8, ffn 512, all Q8_0."""
     L = synth.make_c0()

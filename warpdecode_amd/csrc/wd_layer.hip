@@ -465,20 +465,33 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
     }
     if (only && !(only & WD_MOE_ONLY_C)) return WD_OK;
     const int n_act = k + (shared ? 1 : 0);
-    const int waves_c = n_act < 16 ? n_act : 16;
+    const int grid_c = (H + 3) / 4;
+    // One wave per matrix (k routed and the shared one).  A compute unit holds two such workgroups; when the grid has
+    // more than the chip holds at once (hidden > 2048), waves take two matrices each instead, so that the smaller
+    // workgroups all run together rather than in two rounds.
+    int waves_c = n_act < 16 ? n_act : 16;
+    if (grid_c > 512) waves_c = (waves_c + 1) / 2;
     const size_t per_wave = (static_cast<size_t>(F) + F / 16 + 15) & ~static_cast<size_t>(15);
     const size_t lds_c = waves_c * per_wave + sizeof(float) * 4 * n_act;
-    const int grid_c = (H + 3) / 4;
     auto al16 = [](const void *p_, size_t v) { return reinterpret_cast<uintptr_t>(p_) % 16 == 0 && v % 16 == 0; };
-    const bool coal = L->down_type == WD_TYPE_Q8_0 && F == 512 && H % 4 == 0 && al16(L->shared_down, 0) &&
+    // rows of 16 or 20 blocks in 16-byte aligned groups of four: the coalesced fetch
+    const bool coal = (F == 512 || F == 640) && H % 4 == 0 && al16(L->shared_down, 0) &&
                       (L->slot_of_expert ? al16(L->slot_pool, L->slot_bytes) && (L->slot_gate_bytes + L->slot_up_bytes) % 16 == 0
                                          : al16(L->down, L->down_stride));
-    if (coal)
-        k_layer_c<0, true><<<dim3(grid_c), dim3(64 * waves_c), lds_c, st>>>(a);
-    else if (L->down_type == WD_TYPE_Q8_0)
-        k_layer_c<0, false><<<dim3(grid_c), dim3(64 * waves_c), lds_c, st>>>(a);
+    const dim3 grid(grid_c), block(64 * waves_c);
+    const bool q8 = L->down_type == WD_TYPE_Q8_0;
+    if (coal && F == 512 && q8)
+        k_layer_c<0, true><<<grid, block, lds_c, st>>>(a);
+    else if (coal && F == 512)
+        k_layer_c<1, true, 16><<<grid, block, lds_c, st>>>(a);
+    else if (coal && q8)
+        k_layer_c<0, true, 20><<<grid, block, lds_c, st>>>(a);
+    else if (coal)
+        k_layer_c<1, true, 20><<<grid, block, lds_c, st>>>(a);
+    else if (q8)
+        k_layer_c<0, false><<<grid, block, lds_c, st>>>(a);
     else
-        k_layer_c<1, false><<<dim3(grid_c), dim3(64 * waves_c), lds_c, st>>>(a);
+        k_layer_c<1, false><<<grid, block, lds_c, st>>>(a);
     WD_LAUNCH_CHECK();
     return WD_OK;
 }

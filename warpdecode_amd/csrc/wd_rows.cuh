@@ -727,6 +727,87 @@ WD_DEV void q8_rows4x16(const uint8_t *const (&rows)[NM], const int8_t *act_qs, 
     }
 }
 
+// Four consecutive rows of NB blocks (NB = 16 or 20; Q8_0 or IQ4_NL) that start on a 16-byte boundary: 4 NB blocks are a
+// whole number of 16-byte words (136 NB or 72 NB bytes), fetched as aligned words, copied to LDS and cut into blocks
+// there - lane t takes block t (row t / NB), lanes 0..15 also block 64 + t when NB is 20.  Unaligned 16-byte requests at
+// an 18- or 34-byte stride cost several times the address cycles of aligned ones, and with rows of 20 blocks the
+// general routine needs a second, mostly idle pass.  The tile's chunk-sum area doubles as the staging area.
+template <int NB>
+struct __attribute__((aligned(16))) Q8TileNB {
+    static constexpr int kRow = NB * 8 + 8;  // floats per row, padded (bank spread)
+    float pf[4 * kRow];
+    float ds[4 * NB];
+};
+template <int KIND>
+WD_DEV Q8Block q8_block_from_lds(const uint8_t *stage, int t) {
+    constexpr int kBlk = (KIND == 0) ? 34 : 18;
+    const int byte0 = kBlk * t;
+    Q8Block w;
+    w.d = *reinterpret_cast<const uint16_t *>(stage + byte0);
+    const uint32_t *sw = reinterpret_cast<const uint32_t *>(stage) + ((byte0 + 2) >> 2);
+    const uint32_t sh = (t & 1) ? 0u : 2u;  // kBlk t + 2 is 2 (mod 4) for even t, 0 for odd t (kBlk = 2 mod 4 for both kinds)
+    constexpr int kWords = (KIND == 0) ? 9 : 5;
+    uint32_t r[kWords];
+#pragma unroll
+    for (int j = 0; j < kWords; ++j) r[j] = sw[j];
+    w.q0.x = __builtin_amdgcn_alignbyte(r[1], r[0], sh), w.q0.y = __builtin_amdgcn_alignbyte(r[2], r[1], sh);
+    w.q0.z = __builtin_amdgcn_alignbyte(r[3], r[2], sh), w.q0.w = __builtin_amdgcn_alignbyte(r[4], r[3], sh);
+    if (KIND == 0) {
+        w.q1.x = __builtin_amdgcn_alignbyte(r[5], r[4], sh), w.q1.y = __builtin_amdgcn_alignbyte(r[6], r[5], sh);
+        w.q1.z = __builtin_amdgcn_alignbyte(r[7], r[6], sh), w.q1.w = __builtin_amdgcn_alignbyte(r[8], r[7], sh);
+    }
+    return w;
+}
+// rows: first of the four rows.  y of row r4 valid in lane 16 r4.  The float order is that of q8_rows4_multi.
+template <int KIND, int NB, typename Pre = NoPre>
+WD_DEV float q8_rows4_coal(const uint8_t *rows, const int8_t *act_qs, const uint16_t *act_d, Q8TileNB<NB> &tile, int lane,
+                           Pre pre = Pre()) {
+    static_assert(NB == 16 || NB == 20, "rows of 16 or 20 blocks");
+    constexpr int kBlk = (KIND == 0) ? 34 : 18;
+    constexpr int kWords = 4 * NB * kBlk / 16, kLoads = (kWords + 63) / 64, kSecond = 4 * NB - 64, kRow = Q8TileNB<NB>::kRow;
+    static_assert(4 * NB * kBlk % 16 == 0 && kWords * 16 + 8 <= static_cast<int>(sizeof(Q8TileNB<NB>)), "staging area");
+    uint4 raw[kLoads];
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) raw[i] = gld_u128_aligned(rows + 16 * min(i * 64 + lane, kWords - 1));
+    pre();
+    uint8_t *stage = reinterpret_cast<uint8_t *>(&tile);  // chunk sums and scales together are large enough
+    wave_lds_fence();  // earlier reads of the tile are done before it is overwritten
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) reinterpret_cast<uint4 *>(stage)[min(i * 64 + lane, kWords - 1)] = raw[i];
+    wave_lds_fence();
+    const int t1 = 64 + min(lane, max(kSecond, 1) - 1);
+    const Q8Block w0 = q8_block_from_lds<KIND>(stage, lane);
+    Q8Block w1 = w0;
+    if (kSecond > 0) w1 = q8_block_from_lds<KIND>(stage, t1);
+    wave_lds_fence();  // the staged bytes have been read; the area now takes the chunk sums
+    auto sums = [&](const Q8Block &w, int t) {
+        const int row = t / NB, bi = t - row * NB;
+        const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + bi * 32);
+        const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + bi * 32 + 16);
+        const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        int p[8];
+        q8_chunks<KIND>(w, a, p);
+        float4 *dst = reinterpret_cast<float4 *>(&tile.pf[row * kRow + bi * 8]);
+        dst[0] = make_float4(static_cast<float>(p[0]), static_cast<float>(p[1]), static_cast<float>(p[2]), static_cast<float>(p[3]));
+        dst[1] = make_float4(static_cast<float>(p[4]), static_cast<float>(p[5]), static_cast<float>(p[6]), static_cast<float>(p[7]));
+        tile.ds[row * NB + bi] = h2f(w.d) * h2f(act_d[bi]);
+    };
+    sums(w0, lane);
+    if (kSecond > 0 && lane < kSecond) sums(w1, t1);
+    wave_lds_fence();
+    const int r4 = lane >> 4, c = lane & 7;
+    float acc = 0.0f, acc_odd = 0.0f;
+#pragma unroll
+    for (int s = 0; s < NB; ++s) {
+        const float pv = tile.pf[r4 * kRow + s * 8 + c], dv = tile.ds[r4 * NB + s];
+        if (KIND == 1 && (s & 1))
+            acc_odd = __builtin_fmaf(dv, pv, acc_odd);  // IQ4_NL: even and odd blocks accumulate apart (NB is even: no tail)
+        else
+            acc = __builtin_fmaf(dv, pv, acc);
+    }
+    return close_lanes8(KIND == 1 ? acc + acc_odd : acc);
+}
+
 template <int KIND, bool PART>
 WD_DEV float q8_rows4(const uint8_t *rows, int nrows, int nb, const int8_t *act_qs, const uint16_t *act_d,
                       Q8Tile &tile, int lane, int32_t *partials) {
