@@ -739,7 +739,8 @@ __global__ __launch_bounds__(512) void k_layer_a(LayerArgs a) {
 // when it runs out the workgroup sets status[0] and returns.
 // COAL (IQ types): rows of eight super-blocks on 16-byte boundaries are fetched with one aligned 16-byte load per
 // lane and parked in LDS (iq_rows8_coal); dynamic LDS then has 8 * 2 * kIqStageBytes more bytes behind the 4 * H + 16.
-template <int TYPE, bool COAL>
+// NB (COAL only): super-blocks per row, 8 (hidden 2048) or 10 (hidden 2560).
+template <int TYPE, bool COAL, int NB = 8>
 __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
     constexpr bool kIq = (TYPE == 21 || TYPE == 22);
     extern __shared__ __align__(16) uint8_t lds_ab[];
@@ -855,7 +856,10 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
         const size_t rb = static_cast<size_t>(nb) * (TYPE == 21 ? 110 : 82);
         const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
         const uint8_t *const rows[2] = {uniform_ptr(gate + off), uniform_ptr(up + off)};  // one row pair per wave
-        if (COAL)
+        if (COAL && NB == 10)
+            iq_rows10_coal<(kIq ? TYPE : 21), 2>(rows, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
+                                                 lds_ab + ((4 * a.H + 16 + 15) & ~15) + wave * 2 * kIqStage10Bytes);
+        else if (COAL)
             iq_rows8_coal<(kIq ? TYPE : 21), 2>(rows, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
                                                 lds_ab + ((4 * a.H + 16 + 15) & ~15) + wave * 2 * kIqStageBytes);
         else

@@ -428,22 +428,28 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
         const size_t lds_ab = sizeof(float) * static_cast<size_t>(H) + 16;  // f32 x of the router rows; the quantised x of the others fits inside
         // rows of eight super-blocks on 16-byte boundaries: coalesced fetch with a per-wave staging area behind lds_ab
         auto al16_ = [](const void *p_, size_t v) { return reinterpret_cast<uintptr_t>(p_) % 16 == 0 && v % 16 == 0; };
-        const bool coal_ab = iq && H == 2048 &&
+        // (rows of ten super-blocks are 4-byte aligned then, and F rows end on a 16-byte boundary)
+        const bool coal_ab = iq && (H == 2048 || H == 2560) &&
                              (L->slot_of_expert ? al16_(L->slot_pool, L->slot_bytes) && L->slot_gate_bytes % 16 == 0
                                                 : al16_(L->gate, L->gate_stride) && al16_(L->up, L->up_stride));
-        const size_t lds_stage = 16 + 8 * 2 * static_cast<size_t>(kIqStageBytes);
+        const size_t lds_stage = 16 + 8 * 2 * static_cast<size_t>(H == 2048 ? kIqStageBytes : kIqStage10Bytes);
+        const dim3 grid(grid_ab), block(512);
         switch (L->gate_type) {
             case WD_TYPE_IQ3_S:
-                if (coal_ab)
-                    k_layer_ab<21, true><<<dim3(grid_ab), dim3(512), lds_ab + lds_stage, st>>>(m);
+                if (coal_ab && H == 2048)
+                    k_layer_ab<21, true><<<grid, block, lds_ab + lds_stage, st>>>(m);
+                else if (coal_ab)
+                    k_layer_ab<21, true, 10><<<grid, block, lds_ab + lds_stage, st>>>(m);
                 else
-                    k_layer_ab<21, false><<<dim3(grid_ab), dim3(512), lds_ab, st>>>(m);
+                    k_layer_ab<21, false><<<grid, block, lds_ab, st>>>(m);
                 break;
             case WD_TYPE_IQ2_S:
-                if (coal_ab)
-                    k_layer_ab<22, true><<<dim3(grid_ab), dim3(512), lds_ab + lds_stage, st>>>(m);
+                if (coal_ab && H == 2048)
+                    k_layer_ab<22, true><<<grid, block, lds_ab + lds_stage, st>>>(m);
+                else if (coal_ab)
+                    k_layer_ab<22, true, 10><<<grid, block, lds_ab + lds_stage, st>>>(m);
                 else
-                    k_layer_ab<22, false><<<dim3(grid_ab), dim3(512), lds_ab, st>>>(m);
+                    k_layer_ab<22, false><<<grid, block, lds_ab, st>>>(m);
                 break;
             default: k_layer_ab<8, false><<<dim3(grid_ab), dim3(512), lds_ab, st>>>(m); break;
         }

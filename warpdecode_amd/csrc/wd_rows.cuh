@@ -345,6 +345,76 @@ WD_DEV void iq_rows8_coal(const uint8_t *const (&rows)[NR], const IqTables &t, c
     }
 }
 
+// iq_rows_q8k<TYPE, NR, false> for nb == 10 (hidden 2560) with the aligned fetch.  A row of ten super-blocks is 1100
+// or 820 bytes: 4-byte but not 16-byte aligned, so the wave fetches the 16-byte words that cover it (at most 70) and
+// the fields are picked behind the row's offset in its first word.  Two passes: super-blocks 0..7, then 8 and 9 in the
+// first two lanes of every group of eight, the chain carried over as in iq_rows_q8k.
+// rows[i]: 4-byte aligned, inside a tensor whose end is 16-byte aligned.  stage: NR * kIqStage10Bytes bytes of LDS
+// owned by the wave, 16-byte aligned.
+constexpr int kIqStage10Bytes = 1120;
+template <int TYPE, int NR>
+WD_DEV void iq_rows10_coal(const uint8_t *const (&rows)[NR], const IqTables &t, const int8_t *act_qs, const float *act_d,
+                           int lane, float (&y)[NR], uint8_t *stage) {
+    constexpr int kBlk = (TYPE == 21) ? 110 : 82, kRow = 10 * kBlk;
+    constexpr bool kTwoLoads = 12 + kRow > 1024;
+    const int ib = lane >> 3, sbl = lane & 7;
+    uint32_t lead[NR];
+    {
+        uint4 raw0[NR], raw1[NR];
+        int words[NR];
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            lead[i] = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(rows[i])) & 15u;  // the same in every lane
+            words[i] = static_cast<int>((lead[i] + kRow + 15) >> 4);
+            const uint8_t *base = rows[i] - lead[i];
+            raw0[i] = gld_u128_aligned(base + 16 * min(lane, words[i] - 1));
+            if (kTwoLoads) raw1[i] = gld_u128_aligned(base + 16 * min(64 + lane, words[i] - 1));
+        }
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {  // lanes past the last word repeat it
+            uint4 *st = reinterpret_cast<uint4 *>(stage + i * kIqStage10Bytes);
+            st[min(lane, words[i] - 1)] = raw0[i];
+            if (kTwoLoads) st[min(64 + lane, words[i] - 1)] = raw1[i];
+        }
+    }
+    wave_lds_fence();
+    float acc[NR];
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const int sb = 8 * pass + sbl;
+        const bool on = sb < 10;
+        const int sbc = min(sb, 9);  // lanes without a super-block read the last one and contribute zero
+        const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + sbc * 256 + ib * 32);
+        const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + sbc * 256 + ib * 32 + 16);
+        const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        const float dx = act_d[sbc];
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            const IqFields f = iq_fields_lds<TYPE>(stage + i * kIqStage10Bytes + lead[i] + sbc * kBlk, ib, sbc);
+            int p[8];
+            iq_chunks<TYPE>(f, ib, t, a, p);
+            const float ds = on ? h2f(f.d) * dx : 0.0f;
+            const int P = reduce_scatter_ib(p, lane);  // lane (c = ib, sb): chunk c of super-block sb
+            const float pf = on ? static_cast<float>(P) : 0.0f;
+            // carry of the first pass: last lane of the group -> first lane (lanes past the row's end pass the
+            // accumulator through unchanged, fma(0, 0, acc) == acc)
+            float v = __builtin_fmaf(ds, pf, pass == 0 ? 0.0f : dpp_f<kDppShl7>(0.0f, acc[i]));
+#pragma unroll
+            for (int s = 1; s < 8; ++s) {
+                const float up = dpp_f<kDppShr1>(0.0f, v);
+                const float nxt = __builtin_fmaf(ds, pf, up);
+                v = (sbl == 0) ? v : nxt;
+            }
+            acc[i] = v;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+        const float r = close_lanes8_strided(acc[i]);
+        y[i] = (TYPE == 22) ? 0.125f * r : r;
+    }
+}
+
 template <int TYPE, bool PART>
 WD_DEV float iq_row_q8k(const uint8_t *row, int nb, const IqTables &t, const int8_t *act_qs, const float *act_d,
                         int lane, int32_t *partials) {
