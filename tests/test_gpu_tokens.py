@@ -81,8 +81,10 @@ def test_c4_tokens(g, oracle, T):
     (synth.IQ3_S, synth.Q8_0, False, 768, 96, 8, 8),
     (synth.Q8_0, synth.Q8_0, False, 512, 64, 8, 2),         # not on the union path: one pass per token
     (synth.IQ3_S, synth.IQ4_NL, True, 512, 64, 8, 2),       # union pass for gate/up, the one-token down dispatch per token
-    (synth.IQ2_S, synth.IQ4_NL, True, 2560, 640, 32, 10),   # the model's own types and shapes, idem
-    (synth.IQ3_S, synth.Q8_0, True, 2560, 640, 16, 4),      # 20-block down rows, idem
+    (synth.IQ2_S, synth.IQ4_NL, True, 2560, 640, 32, 10),   # the model's own types and shapes: the aligned multi-token down dispatch
+    (synth.IQ3_S, synth.Q8_0, True, 2560, 640, 16, 4),      # 20-block Q8_0 down rows: the aligned multi-token down dispatch
+    (synth.IQ3_S, synth.IQ4_NL, True, 2048, 512, 16, 4),    # 16-block IQ4_NL down rows, idem
+    (synth.IQ2_S, synth.IQ4_NL, False, 2560, 640, 16, 8),   # idem without a shared expert
 ])
 def test_tokens_equal_single_passes(g, oracle, gate_t, down_t, shared, H, F, E, k):
     L = synth.make_layer(H, F, E, k, gate_t, down_t, shared, seed=SEED, layer=7, router_sigma=1.0 / np.sqrt(H))

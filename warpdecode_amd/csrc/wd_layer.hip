@@ -668,6 +668,23 @@ extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, 
             k_tokens_b<22, kMaxTokens><<<dim3(grid_b), dim3(512), lds_b, st>>>(ta);
     }
     WD_LAUNCH_CHECK();
+    // other down tensors in aligned groups of four 16- or 20-block rows: the same dispatch with the aligned fetch
+    auto al16t = [](const void *p_, size_t v) { return reinterpret_cast<uintptr_t>(p_) % 16 == 0 && v % 16 == 0; };
+    const bool down_tokens_nb = !down_tokens && (F == 512 || F == 640) && H % 8 == 0 && tokens <= 16 &&
+                                (!L->shared_down || al16t(L->shared_down, 0)) &&
+                                (L->slot_of_expert ? al16t(L->slot_pool, L->slot_bytes) && (L->slot_gate_bytes + L->slot_up_bytes) % 16 == 0
+                                                   : al16t(L->down, L->down_stride));
+    if (down_tokens_nb) {
+        const size_t per_wave_n = (static_cast<size_t>(F) + F / 16 + 15) & ~static_cast<size_t>(15);
+        const size_t lds_n = 16 * per_wave_n + sizeof(float) * 8 * tokens * (k + 1);
+        const dim3 grid(H / 8), block(1024);
+        const bool q8 = L->down_type == WD_TYPE_Q8_0;
+        if (F == 512 && !q8) k_tokens_c_nb<1, 16><<<grid, block, lds_n, st>>>(ta);
+        else if (q8) k_tokens_c_nb<0, 20><<<grid, block, lds_n, st>>>(ta);
+        else k_tokens_c_nb<1, 20><<<grid, block, lds_n, st>>>(ta);
+        WD_LAUNCH_CHECK();
+        return WD_OK;
+    }
     if (!down_tokens) {
         for (int t = 0; t < tokens; ++t)
             if (const int rc = layer_fused(L, d_x + static_cast<size_t>(t) * H, d_out + static_cast<size_t>(t) * H, scratch_per_token[t],

@@ -828,22 +828,33 @@ WD_DEV Q8Block q8_block_from_lds(const uint8_t *stage, int t) {
     }
     return w;
 }
-// rows: first of the four rows.  y of row r4 valid in lane 16 r4.  The float order is that of q8_rows4_multi.
-template <int KIND, int NB, typename Pre = NoPre>
-WD_DEV float q8_rows4_coal(const uint8_t *rows, const int8_t *act_qs, const uint16_t *act_d, Q8TileNB<NB> &tile, int lane,
-                           Pre pre = Pre()) {
+// The request and the rest apart, so that a caller can have several row groups in flight.
+template <int KIND, int NB>
+struct Q8CoalRaw {
+    static constexpr int kBlk = (KIND == 0) ? 34 : 18;
+    static constexpr int kWords = 4 * NB * kBlk / 16, kLoads = (kWords + 63) / 64;
+    uint4 u[kLoads];
+};
+template <int KIND, int NB>
+WD_DEV Q8CoalRaw<KIND, NB> q8_rows4_coal_request(const uint8_t *rows, int lane) {
+    using Raw = Q8CoalRaw<KIND, NB>;
     static_assert(NB == 16 || NB == 20, "rows of 16 or 20 blocks");
-    constexpr int kBlk = (KIND == 0) ? 34 : 18;
-    constexpr int kWords = 4 * NB * kBlk / 16, kLoads = (kWords + 63) / 64, kSecond = 4 * NB - 64, kRow = Q8TileNB<NB>::kRow;
-    static_assert(4 * NB * kBlk % 16 == 0 && kWords * 16 + 8 <= static_cast<int>(sizeof(Q8TileNB<NB>)), "staging area");
-    uint4 raw[kLoads];
+    static_assert(4 * NB * Raw::kBlk % 16 == 0 && Raw::kWords * 16 + 8 <= static_cast<int>(sizeof(Q8TileNB<NB>)), "staging area");
+    Raw raw;
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) raw[i] = gld_u128_aligned(rows + 16 * min(i * 64 + lane, kWords - 1));
-    pre();
+    for (int i = 0; i < Raw::kLoads; ++i) raw.u[i] = gld_u128_aligned(rows + 16 * min(i * 64 + lane, Raw::kWords - 1));
+    return raw;
+}
+// y of row r4 valid in lane 16 r4.  The float order is that of q8_rows4_multi.
+template <int KIND, int NB>
+WD_DEV float q8_rows4_coal_finish(const Q8CoalRaw<KIND, NB> &raw, const int8_t *act_qs, const uint16_t *act_d, Q8TileNB<NB> &tile,
+                                  int lane) {
+    using Raw = Q8CoalRaw<KIND, NB>;
+    constexpr int kSecond = 4 * NB - 64, kRow = Q8TileNB<NB>::kRow;
     uint8_t *stage = reinterpret_cast<uint8_t *>(&tile);  // chunk sums and scales together are large enough
     wave_lds_fence();  // earlier reads of the tile are done before it is overwritten
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) reinterpret_cast<uint4 *>(stage)[min(i * 64 + lane, kWords - 1)] = raw[i];
+    for (int i = 0; i < Raw::kLoads; ++i) reinterpret_cast<uint4 *>(stage)[min(i * 64 + lane, Raw::kWords - 1)] = raw.u[i];
     wave_lds_fence();
     const int t1 = 64 + min(lane, max(kSecond, 1) - 1);
     const Q8Block w0 = q8_block_from_lds<KIND>(stage, lane);
@@ -876,6 +887,14 @@ WD_DEV float q8_rows4_coal(const uint8_t *rows, const int8_t *act_qs, const uint
             acc = __builtin_fmaf(dv, pv, acc);
     }
     return close_lanes8(KIND == 1 ? acc + acc_odd : acc);
+}
+// rows: first of the four rows.  `pre` runs between the request and the first read of the activation.
+template <int KIND, int NB, typename Pre = NoPre>
+WD_DEV float q8_rows4_coal(const uint8_t *rows, const int8_t *act_qs, const uint16_t *act_d, Q8TileNB<NB> &tile, int lane,
+                           Pre pre = Pre()) {
+    const Q8CoalRaw<KIND, NB> raw = q8_rows4_coal_request<KIND, NB>(rows, lane);
+    pre();
+    return q8_rows4_coal_finish<KIND, NB>(raw, act_qs, act_d, tile, lane);
 }
 
 template <int KIND, bool PART>

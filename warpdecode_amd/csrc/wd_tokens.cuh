@@ -442,4 +442,127 @@ __global__ __launch_bounds__(1024) void k_tokens_c(TokenArgs ta) {
     mark(a, 2, 6);
 }
 
+// The same for down tensors that k_tokens_c does not take: IQ4_NL (KIND 1) or Q8_0 (KIND 0) rows of NB = 16 or 20 blocks
+// in 16-byte aligned groups of four, fetched as aligned words (q8_rows4_coal).  Eight rows per workgroup, 16 waves, an
+// item is (token, matrix) with the shared expert (always Q8_0) as matrix k; a wave has the two row groups of two items
+// in flight.  dynamic LDS per wave: F bytes + F/32 halves (+ pad), then [T][k+1][8] floats.
+template <int KIND, int NB>
+__global__ __launch_bounds__(1024) void k_tokens_c_nb(TokenArgs ta) {
+    extern __shared__ __align__(16) uint8_t lds_tn[];
+    __shared__ Q8TileNB<NB> tiles[16];
+    const LayerArgs &a = ta.common;
+    const int lane = threadIdx.x & 63;
+    constexpr int kWaves = 16, kItems = 2, kF = NB * 32;
+    using RawQ8 = Q8CoalRaw<0, NB>;
+    using RawW = Q8CoalRaw<KIND, NB>;
+    const int tw = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+    const size_t per_wave = (static_cast<size_t>(kF) + kF / 16 + 15) & ~static_cast<size_t>(15);
+    int8_t *aq = reinterpret_cast<int8_t *>(lds_tn + tw * per_wave);
+    uint16_t *ad = reinterpret_cast<uint16_t *>(lds_tn + tw * per_wave + kF);
+    float *ybuf = reinterpret_cast<float *>(lds_tn + kWaves * per_wave);  // [T][k+1][8]
+    const bool shared = a.sh_down != nullptr;
+    const int per_token = a.k + (shared ? 1 : 0);
+    const int n_items = ta.T * per_token;
+    const int r0 = blockIdx.x * 8;  // hidden is a multiple of 8
+    const int r4 = lane >> 4;
+    const int id_lo = token_pair_id(ta, lane), id_hi = token_pair_id(ta, lane + 64);
+    float wreg;
+    {
+        const TokenSlots &s = ta.tok[min(tw, ta.T - 1)];
+        const float *src = (lane == 16 && shared) ? s.shared_gate : s.weights + min(lane, a.k - 1);
+        wreg = *src;
+    }
+    Q8TileNB<NB> &tile = tiles[tw];
+    for (int item0 = 0; item0 < n_items; item0 += kWaves * kItems) {
+        int it_t[kItems], it_j[kItems];
+        bool it_on[kItems];
+        float4 v0[kItems], v1[kItems], v2[kItems], v3[kItems];
+        uint4 raw[kItems][2][RawQ8::kLoads];
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) {  // unconditional loads: an item past the end repeats the last one
+            const int item = item0 + tw + kWaves * i;
+            it_on[i] = item < n_items;
+            const int ic = min(item, n_items - 1);
+            it_t[i] = ic / per_token, it_j[i] = ic - it_t[i] * per_token;
+            const float *act = ta.tok[it_t[i]].act + static_cast<size_t>(it_j[i]) * kF;
+            v0[i] = *reinterpret_cast<const float4 *>(act + lane * 8);
+            v1[i] = *reinterpret_cast<const float4 *>(act + lane * 8 + 4);
+            if (NB == 20) {  // values 512..639: lanes 0..15 (the others repeat them)
+                v2[i] = *reinterpret_cast<const float4 *>(act + 512 + (lane & 15) * 8);
+                v3[i] = *reinterpret_cast<const float4 *>(act + 512 + (lane & 15) * 8 + 4);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) {
+            const bool is_shared = it_j[i] == a.k;
+            const int pair = it_t[i] * a.k + (is_shared ? 0 : it_j[i]);
+            const int e = pair < 64 ? __builtin_amdgcn_readlane(id_lo, pair) : __builtin_amdgcn_readlane(id_hi, pair - 64);
+            const uint8_t *w = is_shared ? a.sh_down : mat_ptr_expert<0>(a.down, e);
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                if (KIND == 0 || is_shared) {  // wave-uniform
+                    const RawQ8 r = q8_rows4_coal_request<0, NB>(w + static_cast<size_t>(r0 + 4 * g) * NB * 34, lane);
+#pragma unroll
+                    for (int q = 0; q < RawQ8::kLoads; ++q) raw[i][g][q] = r.u[q];
+                } else {
+                    const RawW r = q8_rows4_coal_request<KIND, NB>(w + static_cast<size_t>(r0 + 4 * g) * NB * RawW::kBlk, lane);
+#pragma unroll
+                    for (int q = 0; q < RawW::kLoads; ++q) raw[i][g][q] = r.u[q];
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kItems; ++i) {
+            if (!it_on[i]) continue;  // uniform
+            const bool is_shared = it_j[i] == a.k;
+            wave_lds_fence();
+            lds_quantize_q8_0_step(v0[i], v1[i], true, lane * 8, aq, ad, lane);
+            if (NB == 20) lds_quantize_q8_0_step(v2[i], v3[i], lane < 16, 512 + (lane & 15) * 8, aq, ad, lane);
+            wave_lds_fence();
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                float y;
+                if (KIND == 0 || is_shared) {
+                    RawQ8 r;
+#pragma unroll
+                    for (int q = 0; q < RawQ8::kLoads; ++q) r.u[q] = raw[i][g][q];
+                    y = q8_rows4_coal_finish<0, NB>(r, aq, ad, tile, lane);
+                } else {
+                    RawW r;
+#pragma unroll
+                    for (int q = 0; q < RawW::kLoads; ++q) r.u[q] = raw[i][g][q];
+                    y = q8_rows4_coal_finish<KIND, NB>(r, aq, ad, tile, lane);
+                }
+                if ((lane & 15) == 0) ybuf[(it_t[i] * (a.k + 1) + it_j[i]) * 8 + 4 * g + r4] = y;
+            }
+        }
+    }
+    __syncthreads();
+    if (tw < ta.T) {
+        const TokenSlots &s = ta.tok[tw];
+        const int row = r0 + lane;
+        const bool row_on = lane < 8;
+        float acc = 0.0f;
+        for (int j = 0; j < a.k; ++j) {
+            const float wj = lane_get(wreg, j);
+            const float y = ybuf[(tw * (a.k + 1) + j) * 8 + (lane & 7)];
+            const float prod = y * wj;
+            acc = acc + prod;
+            if (s.expert_out && row_on) s.expert_out[static_cast<size_t>(j) * a.H + row] = y;
+        }
+        const float gate = lane_get(wreg, 16);
+        if (row_on) {
+            float o = acc;
+            if (shared) {
+                const float y = ybuf[(tw * (a.k + 1) + a.k) * 8 + lane];
+                const float prod = y * gate;
+                o = acc + prod;
+                s.down_f32[row] = y;
+            }
+            s.accum[row] = acc;
+            s.out[row] = o;
+        }
+    }
+}
+
 }  // namespace wd
