@@ -964,13 +964,12 @@ __global__ __launch_bounds__(TYPE == 20 ? 256 : 512) void k_layer_b(LayerArgs a)
 // grid = ceil(H / 4), block = 64 * min(k + 1, 16).
 // dynamic LDS per wave: F bytes + F/32 halves (+ pad), then [k+1][4] floats.
 // COAL: the rows are 16 blocks long, H is a multiple of 4 and every down tensor starts on a 16-byte boundary: the
-// four rows of a wave are fetched as aligned 16-byte words (q8_rows4x16).
-// NB (COAL only): blocks per row, 16 or 20; Q8_0 rows of 16 blocks keep q8_rows4x16, the others take q8_rows4_coal.
+// four rows of a wave are fetched as aligned 16-byte words (q8_rows4_coal).
+// NB (COAL only): blocks per row, 16 or 20.
 template <int KIND, bool COAL, int NB = 16>
 __global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
     extern __shared__ __align__(16) uint8_t lds_c[];
-    constexpr bool kGeneric = COAL && (KIND != 0 || NB != 16);
-    using Tile = typename std::conditional<kGeneric, Q8TileNB<NB>, Q8Tile>::type;
+    using Tile = typename std::conditional<COAL, Q8TileNB<NB>, Q8Tile>::type;
     __shared__ Tile tiles[16];
     const bool shared = a.sh_inp != nullptr;
     const int n_act = a.k + (shared ? 1 : 0);
@@ -1017,13 +1016,11 @@ __global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
             wave_lds_fence();
             mark(a, 2, 1);
         };
-        if constexpr (kGeneric) {
+        if constexpr (COAL) {
             if (KIND == 0 || is_shared)
                 y[0] = q8_rows4_coal<0, NB>(rows[0], aq, ad, tiles[wave], lane, quantise);
             else
                 y[0] = q8_rows4_coal<1, NB>(rows[0], aq, ad, tiles[wave], lane, quantise);
-        } else if constexpr (COAL) {
-            q8_rows4x16<1>(rows, aq, ad, tiles[wave], lane, y, quantise);
         } else {
             if (KIND == 0 || is_shared)
                 q8_rows4_multi<0, 1, 1, false>(rows, nrows, nb, aq, ad, tiles[wave], lane, y, nullptr, 0, quantise);

@@ -725,78 +725,7 @@ WD_DEV void q8_rows4_multi(const uint8_t *const (&rows)[NM], int nrows, int nb, 
     }
 }
 
-// ---- Q8_0 x Q8_0, four 16-block rows, coalesced -----------------------------------------------------------
-// Four consecutive rows of 16 blocks are 64 * 34 = 2176 contiguous bytes.  When they start on a 16-byte
-// boundary the wave fetches them as 136 aligned 16-byte words (two full loads and one of eight lanes) instead
-// of three requests per lane at a 34-byte stride, and regroups them through LDS: lane l wants block l, i.e. bytes
-// [34 l, 34 l + 34) - the scale as a 16-bit read, the 32 quants as nine aligned dwords shifted by two bytes in the
-// even lanes (34 l + 2 is 2 mod 4 there and 0 mod 4 in the odd ones).
-struct Q8Coal {
-    uint4 c0, c1, c2;
-};
-WD_DEV Q8Coal q8_rows4x16_request(const uint8_t *src, int lane) {
-    Q8Coal c;
-    c.c0 = gld_u128_aligned(src + 16 * lane);
-    c.c1 = gld_u128_aligned(src + 1024 + 16 * lane);
-    c.c2 = gld_u128_aligned(src + 2048 + 16 * (lane & 7));  // lanes 8.. repeat the first eight (their copy is not stored)
-    return c;
-}
-// stage: 2180 bytes of LDS owned by the wave, 16-byte aligned.
-WD_DEV Q8Block q8_rows4x16_regroup(const Q8Coal &c, uint8_t *stage, int lane) {
-    uint4 *st = reinterpret_cast<uint4 *>(stage);
-    st[lane] = c.c0;
-    st[64 + lane] = c.c1;
-    if (lane < 8) st[128 + lane] = c.c2;
-    wave_lds_fence();
-    const int byte0 = 34 * lane;
-    Q8Block w;
-    w.d = *reinterpret_cast<const uint16_t *>(stage + byte0);
-    const uint32_t *sw = reinterpret_cast<const uint32_t *>(stage) + ((byte0 + 2) >> 2);
-    uint32_t r[9];
-#pragma unroll
-    for (int j = 0; j < 9; ++j) r[j] = sw[j];
-    const uint32_t sh = (lane & 1) ? 0u : 2u;
-    w.q0.x = __builtin_amdgcn_alignbyte(r[1], r[0], sh), w.q0.y = __builtin_amdgcn_alignbyte(r[2], r[1], sh);
-    w.q0.z = __builtin_amdgcn_alignbyte(r[3], r[2], sh), w.q0.w = __builtin_amdgcn_alignbyte(r[4], r[3], sh);
-    w.q1.x = __builtin_amdgcn_alignbyte(r[5], r[4], sh), w.q1.y = __builtin_amdgcn_alignbyte(r[6], r[5], sh);
-    w.q1.z = __builtin_amdgcn_alignbyte(r[7], r[6], sh), w.q1.w = __builtin_amdgcn_alignbyte(r[8], r[7], sh);
-    wave_lds_fence();
-    return w;
-}
-
-// q8_rows4_multi<0, NM, 1, false> for rows of exactly 16 blocks, four valid rows and 16-byte aligned row groups,
-// with the coalesced fetch.  The tile's chunk-sum area doubles as the staging area (it is 2176 bytes).
-template <int NM, typename Pre = NoPre>
-WD_DEV void q8_rows4x16(const uint8_t *const (&rows)[NM], const int8_t *act_qs, const uint16_t *act_d, Q8Tile &tile,
-                        int lane, float (&y)[NM], Pre pre = Pre()) {
-    const int r4 = lane >> 4, b = lane & 15, c = lane & 7;
-    Q8Coal raw[NM];
-#pragma unroll
-    for (int i = 0; i < NM; ++i) raw[i] = q8_rows4x16_request(rows[i], lane);
-    pre();
-    const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + b * 32);
-    const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + b * 32 + 16);
-    const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
-    const float dx = h2f(act_d[b]);
-#pragma unroll
-    for (int i = 0; i < NM; ++i) {
-        wave_lds_fence();  // earlier reads of the tile are done before it is overwritten
-        const Q8Block wb = q8_rows4x16_regroup(raw[i], reinterpret_cast<uint8_t *>(&tile.pf[0][0]), lane);
-        int p[8];
-        q8_chunks<0>(wb, a, p);
-        const float ds = h2f(wb.d) * dx;
-        float4 *dst = reinterpret_cast<float4 *>(&tile.pf[0][r4 * 136 + b * 8]);
-        dst[0] = make_float4(static_cast<float>(p[0]), static_cast<float>(p[1]), static_cast<float>(p[2]), static_cast<float>(p[3]));
-        dst[1] = make_float4(static_cast<float>(p[4]), static_cast<float>(p[5]), static_cast<float>(p[6]), static_cast<float>(p[7]));
-        tile.ds[0][lane] = ds;
-        wave_lds_fence();
-        float acc = 0.0f;
-#pragma unroll
-        for (int s = 0; s < 16; ++s) acc = __builtin_fmaf(tile.ds[0][r4 * 16 + s], tile.pf[0][r4 * 136 + s * 8 + c], acc);
-        y[i] = close_lanes8(acc);
-    }
-}
-
+// ---- Q8_0 / IQ4_NL x Q8_0, four rows of 16 or 20 blocks, aligned fetch -----------------------------------------
 // Four consecutive rows of NB blocks (NB = 16 or 20; Q8_0 or IQ4_NL) that start on a 16-byte boundary: 4 NB blocks are a
 // whole number of 16-byte words (136 NB or 72 NB bytes), fetched as aligned words, copied to LDS and cut into blocks
 // there - lane t takes block t (row t / NB), lanes 0..15 also block 64 + t when NB is 20.  Unaligned 16-byte requests at
