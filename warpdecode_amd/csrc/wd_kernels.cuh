@@ -326,6 +326,42 @@ struct Q8sFetch {
     uint4 u[kLoads];
 };
 
+// Eight blocks of a lane's row (lane = 8 row + chain) out of a staged chunk: the lane's four bytes of every block, the
+// blocks' scales, the activation's four bytes and scales.  The LDS reads are issued as one group, so that a caller can put
+// the next group's before the arithmetic of this one.
+struct Q8sBatch {
+    uint32_t w[12];  // blocks 0 2 4 6 of the batch: two dwords each (w[3i], w[3i+1]); blocks 1 3 5 7: w[3i+2]
+    uint32_t dw[8], a[8];
+    float4 da[2];
+    // my: the lane's bytes of the chunk's first block; row_blocks: the row's first block in the stage; my_a / ad: the
+    // activation's quants at the lane's chain and its scales; b0: the chunk's first block in the row; s: batch in the chunk.
+    WD_DEV void load(const uint8_t *my, const uint8_t *row_blocks, const int8_t *my_a, const float *ad, int b0, int s) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint8_t *blk = my + 34 * (8 * s + 2 * i);
+            w[3 * i] = *reinterpret_cast<const uint32_t *>(blk);
+            w[3 * i + 1] = *reinterpret_cast<const uint32_t *>(blk + 4);
+            w[3 * i + 2] = *reinterpret_cast<const uint32_t *>(blk + 36);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            dw[i] = *reinterpret_cast<const uint16_t *>(row_blocks + 34 * (8 * s + i));
+            a[i] = *reinterpret_cast<const uint32_t *>(my_a + 32 * (b0 + 8 * s + i));
+        }
+        da[0] = *reinterpret_cast<const float4 *>(ad + b0 + 8 * s);
+        da[1] = *reinterpret_cast<const float4 *>(ad + b0 + 8 * s + 4);
+    }
+    // block i of the batch: its scale product and its chunk sum
+    WD_DEV float scale(int i) const {
+        const float d[8] = {da[0].x, da[0].y, da[0].z, da[0].w, da[1].x, da[1].y, da[1].z, da[1].w};
+        return h2f(static_cast<uint16_t>(dw[i])) * d[i];
+    }
+    WD_DEV int dot(int i) const {
+        const uint32_t q = (i & 1) ? w[3 * (i >> 1) + 2] : __builtin_amdgcn_alignbyte(w[3 * (i >> 1) + 1], w[3 * (i >> 1)], 2);
+        return sdot4(q, a[i], 0);
+    }
+};
+
 // SETS: register sets of fetched chunks in flight per wave (2 for grids of single waves, which have nothing else to
 // hide the memory latency with).
 template <int KB, bool PART, int WAVES, int SETS>
@@ -379,29 +415,6 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(WAVE
     if (my_groups == 0) return;  // wave-uniform
     const uint8_t *my = stage + row * RS + 4 * c;
     const int8_t *my_a = aq + 4 * c;
-    // Eight blocks of the lane's row at a time: their LDS reads are issued as one group, the next group's before the
-    // arithmetic of this one, so that the reads' latency lies under it.
-    struct Batch {
-        uint32_t w[12];  // blocks 0 2 4 6 of the batch: two dwords each (w[3i], w[3i+1]); blocks 1 3 5 7: w[3i+2]
-        uint32_t dw[8], a[8];
-        float4 da[2];
-    };
-    auto load_batch = [&](Batch &t, int b0, int s) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint8_t *blk = my + 34 * (8 * s + 2 * i);
-            t.w[3 * i] = *reinterpret_cast<const uint32_t *>(blk);
-            t.w[3 * i + 1] = *reinterpret_cast<const uint32_t *>(blk + 4);
-            t.w[3 * i + 2] = *reinterpret_cast<const uint32_t *>(blk + 36);
-        }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            t.dw[i] = *reinterpret_cast<const uint16_t *>(stage + row * RS + 34 * (8 * s + i));
-            t.a[i] = *reinterpret_cast<const uint32_t *>(my_a + 32 * (b0 + 8 * s + i));
-        }
-        t.da[0] = *reinterpret_cast<const float4 *>(ad + b0 + 8 * s);
-        t.da[1] = *reinterpret_cast<const float4 *>(ad + b0 + 8 * s + 4);
-    };
     float acc = 0.0f;
     int group = first, chunk = 0;
     auto turn = [&](Fetch &f) {
@@ -413,26 +426,24 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(WAVE
         const int b0 = chunk * KB;
         const int out_row = min(8 * group, rows - 8) + row;
         int32_t *pp = PART ? partials + (static_cast<size_t>(out_row) * nb) * 8 + c : nullptr;
-        auto compute_batch = [&](const Batch &bt, int s) {
-            const float da[8] = {bt.da[0].x, bt.da[0].y, bt.da[0].z, bt.da[0].w, bt.da[1].x, bt.da[1].y, bt.da[1].z, bt.da[1].w};
+        const uint8_t *row_blocks = stage + row * RS;
+        auto compute_batch = [&](const Q8sBatch &bt, int s) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const uint32_t q = (i & 1) ? bt.w[3 * (i >> 1) + 2]
-                                           : __builtin_amdgcn_alignbyte(bt.w[3 * (i >> 1) + 1], bt.w[3 * (i >> 1)], 2);
-                const int p = sdot4(q, bt.a[i], 0);
+                const int p = bt.dot(i);
                 if (PART) pp[(b0 + 8 * s + i) * 8] = p;
-                const float d = h2f(static_cast<uint16_t>(bt.dw[i])) * da[i];
-                acc = __builtin_fmaf(d, static_cast<float>(p), acc);
+                acc = __builtin_fmaf(bt.scale(i), static_cast<float>(p), acc);
             }
         };
-        Batch t0, t1;
-        load_batch(t0, b0, 0);
+        // eight blocks at a time, the next eight requested from LDS before the arithmetic of these
+        Q8sBatch t0, t1;
+        t0.load(my, row_blocks, my_a, ad, b0, 0);
 #pragma unroll
         for (int s = 0; s < KB / 8; s += 2) {
-            load_batch(t1, b0, s + 1);
+            t1.load(my, row_blocks, my_a, ad, b0, s + 1);
             __builtin_amdgcn_sched_barrier(0);
             compute_batch(t0, s);
-            if (s + 2 < KB / 8) load_batch(t0, b0, s + 2);
+            if (s + 2 < KB / 8) t0.load(my, row_blocks, my_a, ad, b0, s + 2);
             __builtin_amdgcn_sched_barrier(0);
             compute_batch(t1, s + 1);
         }
@@ -497,27 +508,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_gemv_q8_rows8_split(const uint8_
     const int first_block = wave * SEG;
     int32_t *pp = PART ? partials + (static_cast<size_t>(base_row + row) * nb) * 8 + c : nullptr;
     float dv[SEG], pv[SEG];
-    struct Batch {
-        uint32_t w[12];  // blocks 0 2 4 6 of the batch: two dwords each (w[3i], w[3i+1]); blocks 1 3 5 7: w[3i+2]
-        uint32_t dw[8], a[8];
-        float4 da[2];
-    };
-    auto load_batch = [&](Batch &t, int b0, int s) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint8_t *blk = my + 34 * (8 * s + 2 * i);
-            t.w[3 * i] = *reinterpret_cast<const uint32_t *>(blk);
-            t.w[3 * i + 1] = *reinterpret_cast<const uint32_t *>(blk + 4);
-            t.w[3 * i + 2] = *reinterpret_cast<const uint32_t *>(blk + 36);
-        }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            t.dw[i] = *reinterpret_cast<const uint16_t *>(stage + row * RS + 34 * (8 * s + i));
-            t.a[i] = *reinterpret_cast<const uint32_t *>(my_a + 32 * (b0 + 8 * s + i));
-        }
-        t.da[0] = *reinterpret_cast<const float4 *>(ad + b0 + 8 * s);
-        t.da[1] = *reinterpret_cast<const float4 *>(ad + b0 + 8 * s + 4);
-    };
+    const uint8_t *row_blocks = stage + row * RS;
 #pragma unroll
     for (int ch = 0; ch < NCH; ++ch) {
         wave_lds_fence();  // the previous chunk has been read
@@ -525,26 +516,23 @@ __global__ __launch_bounds__(64 * WAVES) void k_gemv_q8_rows8_split(const uint8_
         for (int i = 0; i < Fetch::kLoads; ++i) *reinterpret_cast<uint4 *>(stage + loff[i]) = f[ch].u[i];
         wave_lds_fence();
         const int b0 = first_block + ch * KB;
-        auto pairs = [&](const Batch &bt, int s) {
-            const float da[8] = {bt.da[0].x, bt.da[0].y, bt.da[0].z, bt.da[0].w, bt.da[1].x, bt.da[1].y, bt.da[1].z, bt.da[1].w};
+        auto pairs = [&](const Q8sBatch &bt, int s) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const uint32_t q = (i & 1) ? bt.w[3 * (i >> 1) + 2]
-                                           : __builtin_amdgcn_alignbyte(bt.w[3 * (i >> 1) + 1], bt.w[3 * (i >> 1)], 2);
-                const int p = sdot4(q, bt.a[i], 0);
+                const int p = bt.dot(i);
                 if (PART) pp[(b0 + 8 * s + i) * 8] = p;
-                dv[ch * KB + 8 * s + i] = h2f(static_cast<uint16_t>(bt.dw[i])) * da[i];
+                dv[ch * KB + 8 * s + i] = bt.scale(i);
                 pv[ch * KB + 8 * s + i] = static_cast<float>(p);
             }
         };
-        Batch t0, t1;
-        load_batch(t0, b0, 0);
+        Q8sBatch t0, t1;
+        t0.load(my, row_blocks, my_a, ad, b0, 0);
 #pragma unroll
         for (int s = 0; s < KB / 8; s += 2) {
-            load_batch(t1, b0, s + 1);
+            t1.load(my, row_blocks, my_a, ad, b0, s + 1);
             __builtin_amdgcn_sched_barrier(0);
             pairs(t0, s);
-            if (s + 2 < KB / 8) load_batch(t0, b0, s + 2);
+            if (s + 2 < KB / 8) t0.load(my, row_blocks, my_a, ad, b0, s + 2);
             __builtin_amdgcn_sched_barrier(0);
             pairs(t1, s + 1);
         }
