@@ -109,7 +109,8 @@ GEMV_SHAPES = {
     synth.Q8_0: [(2048, 512), (512, 2048), (640, 2560), (2048, 8192), (1003, 2048), (5, 1024), (8203, 2048), (9, 16384),
                  (33, 512), (7, 96), (18, 32), (12, 32768), (40, 768),
                  # long rows and few of them: four waves share a row group
-                 (100, 4096), (8, 8192), (515, 8192), (9, 4096), (8184, 4096), (4100, 8192), (21, 16384)],
+                 (100, 4096), (8, 8192), (515, 8192), (9, 4096), (8184, 4096), (4100, 8192), (21, 16384), (2563, 2560), (100, 5120),
+                 (24, 10240)],
     synth.IQ4_NL: [(2560, 640), (2048, 512), (5, 96), (9, 32 * 5)],
     # C1 incl. the lm_head; then ragged row counts for every lanes-per-row case of the streaming kernel (columns a
     # multiple of 256 whose 8-block groups per row divide 64) and shapes that take the general kernel

@@ -465,16 +465,16 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(WAVE
 // ---- dense Q8_0 x Q8_0 GEMV, few rows: the waves of a workgroup share the eight rows of a group --------------------
 // With few row groups a group's wave runs alone on its SIMD and the time is the length of its chains (about 40 cycles
 // per block: one wave issues an instruction every four cycles and a block is ten of them).  Only the fma itself has to
-// run in block order.  So wave v of a workgroup takes blocks [v NCH*32, (v+1) NCH*32) of the eight rows, requests all
+// run in block order.  So wave v of a workgroup takes blocks [v NCH*KB, (v+1) NCH*KB) of the eight rows, requests all
 // of them at once, turns them into (d_w d_a, float(dot4)) pairs in registers at its own pace, and then the waves run
-// their parts of the chains one after the other, handing the 64 accumulators on through LDS: NCH*32 dependent fma per
-// wave, nothing else.  Lane = 8 row + chain as in k_gemv_q8_rows8; nb = 32 NCH WAVES blocks per row.
-// dynamic LDS: cols bytes, cols/32 floats, 256 bytes of accumulators, then one stage of 8 * kQ8sRowStride<32> per wave.
-template <int NCH, int WAVES, bool PART>
+// their parts of the chains one after the other, handing the 64 accumulators on through LDS: NCH*KB dependent fma per
+// wave, nothing else.  Lane = 8 row + chain as in k_gemv_q8_rows8; nb = KB NCH WAVES blocks per row (KB = 16 or 32).
+// dynamic LDS: cols bytes, cols/32 floats, 256 bytes of accumulators, then one stage of 8 * kQ8sRowStride<KB> per wave.
+template <int KB, int NCH, int WAVES, bool PART>
 __global__ __launch_bounds__(64 * WAVES) void k_gemv_q8_rows8_split(const uint8_t *__restrict__ w, int rows, int nb,
                                                               const int8_t *__restrict__ act_qs, const uint16_t *__restrict__ act_d,
                                                               float *__restrict__ out, int32_t *__restrict__ partials) {
-    constexpr int KB = 32, SEG = NCH * KB;
+    constexpr int SEG = NCH * KB;
     using Fetch = Q8sFetch<KB>;
     constexpr int RS = kQ8sRowStride<KB>;
     extern __shared__ __align__(16) uint8_t q8p_lds[];

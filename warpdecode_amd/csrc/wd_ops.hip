@@ -221,17 +221,30 @@ static int launch_gemv_q8_0(int type, MatSrc src, int mats, int rows, int cols, 
         reinterpret_cast<uintptr_t>(src.single) % 16 == 0 && reinterpret_cast<uintptr_t>(qs) % 16 == 0) {
         // whole 16-byte words per row chunk and a 16-byte aligned base: the streaming kernel, eight rows per wave
         const int groups = (rows + 7) / 8;
-        if (groups < 1024 && (nb == 64 || nb == 128 || nb == 256 || nb == 512)) {
-            // few row groups: the waves of a workgroup share a group, the chain runs over prepared pairs
-            int waves = nb == 64 ? 2 : (nb == 128 ? 4 : 8);
-            if (nb == 256 && groups > 256) waves = 4;  // more than one workgroup per compute unit: smaller ones
-            const size_t lds = static_cast<size_t>(cols) + static_cast<size_t>(nb) * 4 + 256 + static_cast<size_t>(waves) * 8 * kQ8sRowStride<32>;
-            auto launch = [&](auto kernel) { kernel<<<groups, 64 * waves, lds, stream>>>(src.single, rows, nb, qs, d, out, partials); };
-            if (nb == 64) partials ? launch(k_gemv_q8_rows8_split<1, 2, true>) : launch(k_gemv_q8_rows8_split<1, 2, false>);
-            else if (nb == 128) partials ? launch(k_gemv_q8_rows8_split<1, 4, true>) : launch(k_gemv_q8_rows8_split<1, 4, false>);
-            else if (nb == 256 && waves == 8) partials ? launch(k_gemv_q8_rows8_split<1, 8, true>) : launch(k_gemv_q8_rows8_split<1, 8, false>);
-            else if (nb == 256) partials ? launch(k_gemv_q8_rows8_split<2, 4, true>) : launch(k_gemv_q8_rows8_split<2, 4, false>);
-            else partials ? launch(k_gemv_q8_rows8_split<2, 8, true>) : launch(k_gemv_q8_rows8_split<2, 8, false>);
+        // few row groups: the waves of a workgroup share a group, the chain runs over prepared pairs
+        struct Split { int nb, kb, nch, waves; };
+        static const Split kSplits[] = {{64, 32, 1, 2}, {80, 16, 1, 5}, {128, 32, 1, 4}, {160, 32, 1, 5}, {256, 32, 1, 8},
+                                        {256, 32, 2, 4}, {320, 32, 2, 5}, {512, 32, 2, 8}};
+        for (const Split &sp : kSplits) {
+            if (groups >= 1024 || sp.nb != nb) continue;
+            // 8192 columns: eight waves when a compute unit gets one workgroup, four (two chunks each) when it gets more
+            if (nb == 256 && (sp.waves == 8) != (groups <= 256)) continue;
+            const size_t lds = static_cast<size_t>(cols) + static_cast<size_t>(nb) * 4 + 256 +
+                               static_cast<size_t>(sp.waves) * 8 * (sp.kb == 32 ? kQ8sRowStride<32> : kQ8sRowStride<16>);
+            auto launch = [&](auto kernel) { kernel<<<groups, 64 * sp.waves, lds, stream>>>(src.single, rows, nb, qs, d, out, partials); };
+#define WD_Q8_SPLIT(KB_, NCH_, WAVES_)                                                                      \
+    if (sp.kb == KB_ && sp.nch == NCH_ && sp.waves == WAVES_) {                                               \
+        partials ? launch(k_gemv_q8_rows8_split<KB_, NCH_, WAVES_, true>) : launch(k_gemv_q8_rows8_split<KB_, NCH_, WAVES_, false>); \
+    }
+            WD_Q8_SPLIT(32, 1, 2)
+            WD_Q8_SPLIT(16, 1, 5)
+            WD_Q8_SPLIT(32, 1, 4)
+            WD_Q8_SPLIT(32, 1, 5)
+            WD_Q8_SPLIT(32, 1, 8)
+            WD_Q8_SPLIT(32, 2, 4)
+            WD_Q8_SPLIT(32, 2, 5)
+            WD_Q8_SPLIT(32, 2, 8)
+#undef WD_Q8_SPLIT
             WD_LAUNCH_CHECK();
             return WD_OK;
         }
