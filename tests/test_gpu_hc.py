@@ -94,6 +94,15 @@ def test_layer_with_combine(g, oracle, flags, shape):
 def test_hc_error_paths(g):
     x = g.empty(64, np.float32)
     lib = capi.load()
+    L = synth.make_layer(256, 64, 8, 2, synth.Q8_0, synth.Q8_0, False, seed=SEED, layer=3)
+    dl, sc = g.DeviceLayer(L), g.Scratch(256, 64, 8, 2)
+    big = g.empty(17 * 256, np.float32)
+    call = lambda hc, flags: lib.wd_moe_layer_hc_f32(C.byref(dl.desc), g.ptr(big), g.ptr(big), g.ptr(big), g.ptr(big), hc, 0, sc.h, flags, None)
+    assert call(17, 0) == -1 and b"1..16 residual streams" in lib.wd_last_error()
+    assert call(0, 0) == -1
+    assert call(4, 0x10) == -1 and b"measurement flags" in lib.wd_last_error()      # WD_MOE_ONLY_A
+    assert lib.wd_moe_layer_hc_f32(C.byref(dl.desc), g.ptr(big), g.ptr(big), None, g.ptr(big), 4, 0, sc.h, 0, None) == -1
+    sc.close()
     assert lib.wd_hc_combine_f32(None, g.ptr(x), g.ptr(x), 16, 4, 0, None) == -1
     assert lib.wd_hc_combine_f32(g.ptr(x), g.ptr(x), g.ptr(x), 0, 4, 0, None) == -1
     assert lib.wd_hc_combine_moe_f32(g.ptr(x), g.ptr(x), None, 0, g.ptr(x), g.ptr(x), 16, 4, 0, None) == -1
