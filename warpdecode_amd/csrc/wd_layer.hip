@@ -656,17 +656,31 @@ extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, 
     const size_t lds_b = static_cast<size_t>(tokens) * (H + sizeof(float) * (H / 256));
     const int items_b = tokens * k * ((F + 7) / 8);
     const int grid_b = items_b < 512 ? items_b : 512;  // persistent: two workgroups per compute unit walk the items
-    if (L->gate_type == WD_TYPE_IQ3_S) {
-        if (tokens <= 4)
-            k_tokens_b<21, 4><<<dim3(grid_b), dim3(512), lds_b, st>>>(ta);
-        else
-            k_tokens_b<21, kMaxTokens><<<dim3(grid_b), dim3(512), lds_b, st>>>(ta);
-    } else {
-        if (tokens <= 4)
-            k_tokens_b<22, 4><<<dim3(grid_b), dim3(512), lds_b, st>>>(ta);
-        else
-            k_tokens_b<22, kMaxTokens><<<dim3(grid_b), dim3(512), lds_b, st>>>(ta);
-    }
+    // rows of eight or ten super-blocks of aligned tensors: the aligned fetch, one item ahead
+    auto al16b = [](const void *p_, size_t v) { return reinterpret_cast<uintptr_t>(p_) % 16 == 0 && v % 16 == 0; };
+    const bool coal_b = (H == 2048 || H == 2560) &&
+                        (L->slot_of_expert ? al16b(L->slot_pool, L->slot_bytes) && L->slot_gate_bytes % 16 == 0
+                                           : al16b(L->gate, L->gate_stride) && al16b(L->up, L->up_stride));
+    const size_t lds_b_coal = ((lds_b + 15) & ~static_cast<size_t>(15)) + 8 * 2 * static_cast<size_t>(H == 2048 ? kIqStageBytes : kIqStage10Bytes);
+    const dim3 gb(grid_b), bb(512);
+#define WD_TOKENS_B(TYPE_)                                                                              \
+    do {                                                                                                \
+        if (coal_b && H == 2048) {                                                                      \
+            if (tokens <= 4) k_tokens_b<TYPE_, 4, 8><<<gb, bb, lds_b_coal, st>>>(ta);                   \
+            else k_tokens_b<TYPE_, kMaxTokens, 8><<<gb, bb, lds_b_coal, st>>>(ta);                      \
+        } else if (coal_b) {                                                                            \
+            if (tokens <= 4) k_tokens_b<TYPE_, 4, 10><<<gb, bb, lds_b_coal, st>>>(ta);                  \
+            else k_tokens_b<TYPE_, kMaxTokens, 10><<<gb, bb, lds_b_coal, st>>>(ta);                     \
+        } else {                                                                                        \
+            if (tokens <= 4) k_tokens_b<TYPE_, 4><<<gb, bb, lds_b, st>>>(ta);                           \
+            else k_tokens_b<TYPE_, kMaxTokens><<<gb, bb, lds_b, st>>>(ta);                              \
+        }                                                                                               \
+    } while (0)
+    if (L->gate_type == WD_TYPE_IQ3_S)
+        WD_TOKENS_B(21);
+    else
+        WD_TOKENS_B(22);
+#undef WD_TOKENS_B
     WD_LAUNCH_CHECK();
     // other down tensors in aligned groups of four 16- or 20-block rows: the same dispatch with the aligned fetch
     auto al16t = [](const void *p_, size_t v) { return reinterpret_cast<uintptr_t>(p_) % 16 == 0 && v % 16 == 0; };

@@ -345,13 +345,38 @@ WD_DEV void iq_rows8_coal(const uint8_t *const (&rows)[NR], const IqTables &t, c
     }
 }
 
+constexpr int kIqStage10Bytes = 1120;  // per row of ten super-blocks: the 70 words that cover 12 + 1100 bytes
+// The aligned fetch of one IQ row of NB = 8 or 10 super-blocks as a request and a store apart (for callers that keep a
+// row in flight while they work on another): the 16-byte words that cover the row (it is 16-byte aligned for NB = 8 and
+// 4-byte aligned for NB = 10), copied to a stage of kIqStageBytes / kIqStage10Bytes; the row then starts `lead` bytes
+// into the stage.
+template <int TYPE, int NB>
+struct IqRowFetch {
+    static constexpr int kBlk = (TYPE == 21) ? 110 : 82, kRow = NB * kBlk;
+    static constexpr bool kTwoLoads = 12 + kRow > 1024;
+    uint4 r0, r1;
+    uint32_t lead;
+    int words;
+    WD_DEV void request(const uint8_t *row, int lane) {
+        lead = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(row)) & 15u;  // the same in every lane
+        words = static_cast<int>((lead + kRow + 15) >> 4);
+        const uint8_t *base = row - lead;
+        r0 = gld_u128_aligned(base + 16 * min(lane, words - 1));
+        if (kTwoLoads) r1 = gld_u128_aligned(base + 16 * min(64 + lane, words - 1));
+    }
+    WD_DEV void store(uint8_t *stage, int lane) const {  // lanes past the last word repeat it
+        uint4 *st = reinterpret_cast<uint4 *>(stage);
+        st[min(lane, words - 1)] = r0;
+        if (kTwoLoads) st[min(64 + lane, words - 1)] = r1;
+    }
+};
+
 // iq_rows_q8k<TYPE, NR, false> for nb == 10 (hidden 2560) with the aligned fetch.  A row of ten super-blocks is 1100
 // or 820 bytes: 4-byte but not 16-byte aligned, so the wave fetches the 16-byte words that cover it (at most 70) and
 // the fields are picked behind the row's offset in its first word.  Two passes: super-blocks 0..7, then 8 and 9 in the
 // first two lanes of every group of eight, the chain carried over as in iq_rows_q8k.
 // rows[i]: 4-byte aligned, inside a tensor whose end is 16-byte aligned.  stage: NR * kIqStage10Bytes bytes of LDS
 // owned by the wave, 16-byte aligned.
-constexpr int kIqStage10Bytes = 1120;
 template <int TYPE, int NR>
 WD_DEV void iq_rows10_coal(const uint8_t *const (&rows)[NR], const IqTables &t, const int8_t *act_qs, const float *act_d,
                            int lane, float (&y)[NR], uint8_t *stage) {

@@ -172,7 +172,10 @@ WD_DEV void token_union_build(const TokenArgs &ta, TokenUnion &un, int lane) {
 // the item, decodes it once and applies it to every token that selected the expert.
 // MAXT: token capacity of the instantiation (4 or kMaxTokens).
 // dynamic LDS: T * (H bytes + H/256 floats): the Q8_K copies of the T inputs.
-template <int TYPE, int MAXT>
+// NB: 0, or the super-blocks per row (8 or 10) when the rows can be fetched as aligned words (IqRowFetch): the row pair of
+// the wave's next item is then requested before the current one is worked on.  dynamic LDS then has
+// 8 * 2 * (kIqStageBytes or kIqStage10Bytes) more bytes behind the activations (16-byte aligned).
+template <int TYPE, int MAXT, int NB = 0>
 __global__ __launch_bounds__(512, 4) void k_tokens_b(TokenArgs ta) {
     extern __shared__ __align__(16) uint8_t lds_tb[];
     __shared__ IqTables tables;
@@ -222,16 +225,41 @@ __global__ __launch_bounds__(512, 4) void k_tokens_b(TokenArgs ta) {
     const int n_items = un.count * groups;
     const int ib = lane >> 3, sbl = lane & 7;
     const bool first = sbl == 0;
-    for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
+    constexpr int kStage = (NB == 10) ? kIqStage10Bytes : kIqStageBytes;
+    uint8_t *stage = lds_tb + ((static_cast<size_t>(ta.T) * (a.H + sizeof(float) * nb) + 15) & ~static_cast<size_t>(15)) +
+                     static_cast<size_t>(wave) * 2 * kStage;
+    IqRowFetch<TYPE, NB == 0 ? 8 : NB> fetch[2];
+    auto row_pair = [&](int item, const uint8_t *(&rows)[2]) {
         const int u = item / groups, rg = item - u * groups;
         const int e = un.expert[u];
+        const size_t off = static_cast<size_t>(min(rg * 8 + wave, a.F - 1)) * rb;
+        rows[0] = uniform_ptr(mat_ptr_expert<0>(a.gate_up, e) + off), rows[1] = uniform_ptr(mat_ptr_expert<1>(a.gate_up, e) + off);
+    };
+    if (NB != 0 && static_cast<int>(blockIdx.x) < n_items) {
+        const uint8_t *rows[2];
+        row_pair(blockIdx.x, rows);
+        fetch[0].request(rows[0], lane), fetch[1].request(rows[1], lane);
+    }
+    for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
+        const int u = item / groups, rg = item - u * groups;
         int rank[MAXT];
 #pragma unroll
         for (int t = 0; t < MAXT; ++t) rank[t] = __builtin_amdgcn_readfirstlane(static_cast<int>(un.rank[u][t]));
         const int r = rg * 8 + wave;
-        const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
-        const uint8_t *const rows[2] = {uniform_ptr(mat_ptr_expert<0>(a.gate_up, e) + off),
-                                        uniform_ptr(mat_ptr_expert<1>(a.gate_up, e) + off)};  // one row pair per wave
+        const uint8_t *rows[2];  // one row pair per wave
+        row_pair(item, rows);
+        uint32_t lead[2] = {0, 0};
+        if (NB != 0) {
+            wave_lds_fence();  // the previous item's rows have been read
+            fetch[0].store(stage, lane), fetch[1].store(stage + kStage, lane);
+            lead[0] = fetch[0].lead, lead[1] = fetch[1].lead;
+            wave_lds_fence();
+            if (item + static_cast<int>(gridDim.x) < n_items) {  // the next item's rows, into the registers just written out
+                const uint8_t *next[2];
+                row_pair(item + gridDim.x, next);
+                fetch[0].request(next[0], lane), fetch[1].request(next[1], lane);
+            }
+        }
         float acc[MAXT][2];
 #pragma unroll
         for (int t = 0; t < MAXT; ++t) acc[t][0] = acc[t][1] = 0.0f;
@@ -243,8 +271,13 @@ __global__ __launch_bounds__(512, 4) void k_tokens_b(TokenArgs ta) {
             float dw[2] = {0.0f, 0.0f};
             if (on) {
                 IqFields f[2];
-                f[0] = iq_load<TYPE>(rows[0] + static_cast<size_t>(sb) * kBlk, ib);
-                f[1] = iq_load<TYPE>(rows[1] + static_cast<size_t>(sb) * kBlk, ib);
+                if (NB != 0) {
+                    f[0] = iq_fields_lds<TYPE>(stage + lead[0] + sb * kBlk, ib, sb);
+                    f[1] = iq_fields_lds<TYPE>(stage + kStage + lead[1] + sb * kBlk, ib, sb);
+                } else {
+                    f[0] = iq_load<TYPE>(rows[0] + static_cast<size_t>(sb) * kBlk, ib);
+                    f[1] = iq_load<TYPE>(rows[1] + static_cast<size_t>(sb) * kBlk, ib);
+                }
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
                     iq_decode<TYPE>(f[i], ib, tables, w[i], ls[i]);
