@@ -965,8 +965,9 @@ __global__ __launch_bounds__(TYPE == 20 ? 256 : 512) void k_layer_b(LayerArgs a)
 // dynamic LDS per wave: F bytes + F/32 halves (+ pad), then [k+1][4] floats.
 // COAL: the rows are 16 blocks long, H is a multiple of 4 and every down tensor starts on a 16-byte boundary: the
 // four rows of a wave are fetched as aligned 16-byte words (q8_rows4_coal).
-// NB (COAL only): blocks per row, 16 or 20.
-template <int KIND, bool COAL, int NB = 16>
+// NB (COAL only): blocks per row, 16 or 20.  TWO (COAL only): the workgroup has half as many waves as matrices; a wave
+// requests the rows and the activations of its two matrices together.
+template <int KIND, bool COAL, int NB = 16, bool TWO = false>
 __global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
     extern __shared__ __align__(16) uint8_t lds_c[];
     using Tile = typename std::conditional<COAL, Q8TileNB<NB>, Q8Tile>::type;
@@ -1003,6 +1004,58 @@ __global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
             if (a.hc > 0) inject = a.hc_inject[c];
         }
     }
+    if constexpr (COAL && TWO) {
+        using RawQ8 = Q8CoalRaw<0, NB>;
+        using RawW = Q8CoalRaw<KIND, NB>;
+        const int uw = __builtin_amdgcn_readfirstlane(wave);
+        uint4 raw[2][RawQ8::kLoads];
+        float4 v[2][NB == 20 ? 4 : 2];
+        int mm[2];
+        bool sh[2];
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {  // a wave without a second matrix repeats its first (not used)
+            mm[q] = (uw + q * nwaves < n_act) ? uw + q * nwaves : uw;
+            sh[q] = mm[q] == a.k;
+            const uint8_t *w = sh[q] ? a.sh_down : mat_ptr_expert<0>(a.down, sld_i32(a.ids + mm[q]));
+            if (KIND == 0 || sh[q]) {  // wave-uniform
+                const RawQ8 r = q8_rows4_coal_request<0, NB>(w + static_cast<size_t>(r0) * NB * 34, lane);
+#pragma unroll
+                for (int i = 0; i < RawQ8::kLoads; ++i) raw[q][i] = r.u[i];
+            } else {
+                const RawW r = q8_rows4_coal_request<KIND, NB>(w + static_cast<size_t>(r0) * NB * RawW::kBlk, lane);
+#pragma unroll
+                for (int i = 0; i < RawW::kLoads; ++i) raw[q][i] = r.u[i];
+            }
+            const float *act = a.act + static_cast<size_t>(mm[q]) * (NB * 32);
+            v[q][0] = *reinterpret_cast<const float4 *>(act + lane * 8);
+            v[q][1] = *reinterpret_cast<const float4 *>(act + lane * 8 + 4);
+            if (NB == 20) {  // values 512..639: lanes 0..15 (the others repeat them)
+                v[q][2] = *reinterpret_cast<const float4 *>(act + 512 + (lane & 15) * 8);
+                v[q][3] = *reinterpret_cast<const float4 *>(act + 512 + (lane & 15) * 8 + 4);
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            if (q == 1 && uw + nwaves >= n_act) break;  // wave-uniform
+            wave_lds_fence();
+            lds_quantize_q8_0_step(v[q][0], v[q][1], true, lane * 8, aq, ad, lane);
+            if (NB == 20) lds_quantize_q8_0_step(v[q][2], v[q][3], lane < 16, 512 + (lane & 15) * 8, aq, ad, lane);
+            wave_lds_fence();
+            float y;
+            if (KIND == 0 || sh[q]) {
+                RawQ8 r;
+#pragma unroll
+                for (int i = 0; i < RawQ8::kLoads; ++i) r.u[i] = raw[q][i];
+                y = q8_rows4_coal_finish<0, NB>(r, aq, ad, tiles[wave], lane);
+            } else {
+                RawW r;
+#pragma unroll
+                for (int i = 0; i < RawW::kLoads; ++i) r.u[i] = raw[q][i];
+                y = q8_rows4_coal_finish<KIND, NB>(r, aq, ad, tiles[wave], lane);
+            }
+            if ((lane & 15) == 0) ybuf[mm[q] * 4 + r4] = y;
+        }
+    } else
     for (int m = wave; m < n_act; m += nwaves) {
         const bool is_shared = m == a.k;
         // m is the same for the whole wave: the id comes through the scalar path

@@ -476,7 +476,7 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
     // more than the chip holds at once (hidden > 2048), waves take two matrices each instead, so that the smaller
     // workgroups all run together rather than in two rounds.
     int waves_c = n_act < 16 ? n_act : 16;
-    if (grid_c > 512) waves_c = (waves_c + 1) / 2;
+    if (grid_c > 512) waves_c = (n_act + 1) / 2;
     const size_t per_wave = (static_cast<size_t>(F) + F / 16 + 15) & ~static_cast<size_t>(15);
     const size_t lds_c = waves_c * per_wave + sizeof(float) * 4 * n_act;
     auto al16 = [](const void *p_, size_t v) { return reinterpret_cast<uintptr_t>(p_) % 16 == 0 && v % 16 == 0; };
@@ -486,7 +486,13 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
                                          : al16(L->down, L->down_stride));
     const dim3 grid(grid_c), block(64 * waves_c);
     const bool q8 = L->down_type == WD_TYPE_Q8_0;
-    if (coal && F == 512 && q8)
+    const bool two = waves_c < n_act;  // halved above: n_act <= 2 * waves_c
+    if (coal && two) {
+        if (F == 512 && q8) k_layer_c<0, true, 16, true><<<grid, block, lds_c, st>>>(a);
+        else if (F == 512) k_layer_c<1, true, 16, true><<<grid, block, lds_c, st>>>(a);
+        else if (q8) k_layer_c<0, true, 20, true><<<grid, block, lds_c, st>>>(a);
+        else k_layer_c<1, true, 20, true><<<grid, block, lds_c, st>>>(a);
+    } else if (coal && F == 512 && q8)
         k_layer_c<0, true><<<grid, block, lds_c, st>>>(a);
     else if (coal && F == 512)
         k_layer_c<1, true, 16><<<grid, block, lds_c, st>>>(a);
