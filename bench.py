@@ -424,7 +424,7 @@ def bench_q4_sweep(args, torch, capi, synth):
         "data": "synthetic",
         "config": {"workload": "C1: Q4_0 x Q8_0 GEMV sweep, Llama-3.2-1B shapes, raw GGUF 18-byte blocks", "shapes": results},
         "roofline": dict(bound="hbm", achieved=head["gbs"], peak=HBM_PEAK_GBS, unit="GB/s", frac=head["frac"], traffic=None,
-                         kernel="k_gemv_q8<Q4_0>", us_per_launch=head["us_per_gemv"], bytes_per_launch=head["bytes"])}))
+                         kernel="k_gemv_q4_stream", us_per_launch=head["us_per_gemv"], bytes_per_launch=head["bytes"])}))
 
 
 def bench_model_layer(args, torch, capi, synth):
