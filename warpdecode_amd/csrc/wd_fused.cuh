@@ -966,12 +966,16 @@ __global__ __launch_bounds__(TYPE == 20 ? 256 : 512) void k_layer_b(LayerArgs a)
 // COAL: the rows are 16 blocks long, H is a multiple of 4 and every down tensor starts on a 16-byte boundary: the
 // four rows of a wave are fetched as aligned 16-byte words (q8_rows4_coal).
 // NB (COAL only): blocks per row, 16 or 20.  TWO (COAL only): the workgroup has half as many waves as matrices; a wave
-// requests the rows and the activations of its two matrices together.
+// requests the rows and the activations of its two matrices together and parks all of it in LDS before the dot
+// products, which keeps it within 80 registers: the waves of a workgroup go to the four SIMDs in turn, so three
+// workgroups of six waves need six wave slots on two of them.  dynamic LDS per wave: two quantised activations and a
+// staging area of 4 * NB * 34 bytes.
 template <int KIND, bool COAL, int NB = 16, bool TWO = false>
-__global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
+__global__ __launch_bounds__(TWO ? 576 : 1024) __attribute__((amdgpu_waves_per_eu(TWO ? 6 : 4)))
+void k_layer_c(LayerArgs a) {
     extern __shared__ __align__(16) uint8_t lds_c[];
     using Tile = typename std::conditional<COAL, Q8TileNB<NB>, Q8Tile>::type;
-    __shared__ Tile tiles[16];
+    __shared__ Tile tiles[TWO ? 9 : 16];
     const bool shared = a.sh_inp != nullptr;
     const int n_act = a.k + (shared ? 1 : 0);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -979,7 +983,7 @@ __global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
     const size_t per_wave = (static_cast<size_t>(a.F) + a.F / 16 + 15) & ~static_cast<size_t>(15);
     int8_t *aq = reinterpret_cast<int8_t *>(lds_c + wave * per_wave);
     uint16_t *ad = reinterpret_cast<uint16_t *>(lds_c + wave * per_wave + a.F);
-    float *ybuf = reinterpret_cast<float *>(lds_c + nwaves * per_wave);  // [n_act][4]
+    float *ybuf = reinterpret_cast<float *>(lds_c + nwaves * per_wave);  // [n_act][4] (behind larger per-wave areas if TWO)
     const int r0 = blockIdx.x * 4;
     const int nrows = min(4, a.H - r0);
     const int nb = a.F >> 5;
@@ -1004,83 +1008,115 @@ __global__ __launch_bounds__(1024) void k_layer_c(LayerArgs a) {
             if (a.hc > 0) inject = a.hc_inject[c];
         }
     }
+    // COAL: the activation of one matrix in registers, values 8 lane .. 8 lane + 8 and, with 20 blocks, 512 .. 639 in
+    // lanes 0..15 (the others repeat them); its Q8_0 form into LDS
+    constexpr int kActRegs = (COAL && NB == 20) ? 4 : 2;
+    auto request_act = [&](int m, float4 (&v)[kActRegs]) {
+        const float *act = a.act + static_cast<size_t>(m) * (NB * 32);
+        v[0] = *reinterpret_cast<const float4 *>(act + lane * 8);
+        v[1] = *reinterpret_cast<const float4 *>(act + lane * 8 + 4);
+        if constexpr (kActRegs == 4) {
+            v[2] = *reinterpret_cast<const float4 *>(act + 512 + (lane & 15) * 8);
+            v[3] = *reinterpret_cast<const float4 *>(act + 512 + (lane & 15) * 8 + 4);
+        }
+    };
+    auto quantise_act = [&](const float4 (&v)[kActRegs], int8_t *qs, uint16_t *d) {
+        lds_quantize_q8_0_step(v[0], v[1], true, lane * 8, qs, d, lane);
+        if constexpr (kActRegs == 4) lds_quantize_q8_0_step(v[2], v[3], lane < 16, 512 + (lane & 15) * 8, qs, d, lane);
+    };
     if constexpr (COAL && TWO) {
+        // Everything is requested at once; both activations are quantised and both row groups parked in LDS as they
+        // arrive (loads return in order), so that no fetched word stays in a register while the dot products run.
         using RawQ8 = Q8CoalRaw<0, NB>;
         using RawW = Q8CoalRaw<KIND, NB>;
+        constexpr size_t kStage = 4 * NB * 34;  // the larger of the two kinds
         const int uw = __builtin_amdgcn_readfirstlane(wave);
-        uint4 raw[2][RawQ8::kLoads];
-        float4 v[2][NB == 20 ? 4 : 2];
-        int mm[2];
+        uint8_t *const wbase = lds_c + wave * (2 * per_wave + kStage);
+        int8_t *const aq2[2] = {reinterpret_cast<int8_t *>(wbase), reinterpret_cast<int8_t *>(wbase + per_wave)};
+        uint16_t *const ad2[2] = {reinterpret_cast<uint16_t *>(wbase + a.F), reinterpret_cast<uint16_t *>(wbase + per_wave + a.F)};
+        uint8_t *const stage2[2] = {reinterpret_cast<uint8_t *>(&tiles[wave]), wbase + 2 * per_wave};
+        ybuf = reinterpret_cast<float *>(lds_c + nwaves * (2 * per_wave + kStage));
+        const bool second = uw + nwaves < n_act;  // wave-uniform; a wave without a second matrix repeats its first (not used)
+        RawQ8 raw[2];  // (the request of either kind: as many loads as Q8_0 rows need)
+        float4 v[2][kActRegs];
+        int mm[2], words[2];
         bool sh[2];
-#pragma unroll
-        for (int q = 0; q < 2; ++q) {  // a wave without a second matrix repeats its first (not used)
-            mm[q] = (uw + q * nwaves < n_act) ? uw + q * nwaves : uw;
-            sh[q] = mm[q] == a.k;
-            const uint8_t *w = sh[q] ? a.sh_down : mat_ptr_expert<0>(a.down, sld_i32(a.ids + mm[q]));
-            if (KIND == 0 || sh[q]) {  // wave-uniform
-                const RawQ8 r = q8_rows4_coal_request<0, NB>(w + static_cast<size_t>(r0) * NB * 34, lane);
-#pragma unroll
-                for (int i = 0; i < RawQ8::kLoads; ++i) raw[q][i] = r.u[i];
-            } else {
-                const RawW r = q8_rows4_coal_request<KIND, NB>(w + static_cast<size_t>(r0) * NB * RawW::kBlk, lane);
-#pragma unroll
-                for (int i = 0; i < RawW::kLoads; ++i) raw[q][i] = r.u[i];
-            }
-            const float *act = a.act + static_cast<size_t>(mm[q]) * (NB * 32);
-            v[q][0] = *reinterpret_cast<const float4 *>(act + lane * 8);
-            v[q][1] = *reinterpret_cast<const float4 *>(act + lane * 8 + 4);
-            if (NB == 20) {  // values 512..639: lanes 0..15 (the others repeat them)
-                v[q][2] = *reinterpret_cast<const float4 *>(act + 512 + (lane & 15) * 8);
-                v[q][3] = *reinterpret_cast<const float4 *>(act + 512 + (lane & 15) * 8 + 4);
-            }
-        }
+        // the activations first: their addresses need no expert id, and loads return in order - the quantisation
+        // below then runs while the weights are still on their way
+        int e[2];
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
-            if (q == 1 && uw + nwaves >= n_act) break;  // wave-uniform
-            wave_lds_fence();
-            lds_quantize_q8_0_step(v[q][0], v[q][1], true, lane * 8, aq, ad, lane);
-            if (NB == 20) lds_quantize_q8_0_step(v[q][2], v[q][3], lane < 16, 512 + (lane & 15) * 8, aq, ad, lane);
-            wave_lds_fence();
-            float y;
-            if (KIND == 0 || sh[q]) {
-                RawQ8 r;
+            mm[q] = (q == 0 || second) ? uw + q * nwaves : uw;
+            sh[q] = mm[q] == a.k;
+            e[q] = sld_i32(a.ids + min(mm[q], a.k - 1));  // both ids asked for together (not used for the shared expert)
+        }
 #pragma unroll
-                for (int i = 0; i < RawQ8::kLoads; ++i) r.u[i] = raw[q][i];
-                y = q8_rows4_coal_finish<0, NB>(r, aq, ad, tiles[wave], lane);
-            } else {
-                RawW r;
+        for (int q = 0; q < 2; ++q) request_act(mm[q], v[q]);
 #pragma unroll
-                for (int i = 0; i < RawW::kLoads; ++i) r.u[i] = raw[q][i];
-                y = q8_rows4_coal_finish<KIND, NB>(r, aq, ad, tiles[wave], lane);
-            }
+        for (int q = 0; q < 2; ++q) {
+            const uint8_t *w = sh[q] ? a.sh_down : mat_ptr_expert_uniform<0>(a.down, e[q]);
+            const bool q8 = KIND == 0 || sh[q];  // wave-uniform
+            words[q] = q8 ? RawQ8::kWords : RawW::kWords;
+            raw[q] = q8_rows4_coal_request_any<NB>(w + static_cast<size_t>(r0) * NB * (q8 ? 34 : RawW::kBlk), words[q], lane);
+        }
+        mark(a, 2, 1);
+        wave_lds_fence();
+#pragma unroll
+        for (int q = 0; q < 2; ++q) quantise_act(v[q], aq2[q], ad2[q]);
+        mark(a, 2, 6);
+#pragma unroll
+        for (int q = 0; q < 2; ++q) q8_rows4_coal_stage_any<NB>(raw[q], stage2[q], words[q], lane);
+        wave_lds_fence();
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            if (q == 1 && !second) break;
+            const float y = (KIND == 0 || sh[q]) ? q8_rows4_coal_dots<0, NB>(stage2[q], aq2[q], ad2[q], tiles[wave], lane)
+                                                 : q8_rows4_coal_dots<KIND, NB>(stage2[q], aq2[q], ad2[q], tiles[wave], lane);
             if ((lane & 15) == 0) ybuf[mm[q] * 4 + r4] = y;
+            mark(a, 2, q == 0 ? 2 : 5);
         }
     } else
     for (int m = wave; m < n_act; m += nwaves) {
         const bool is_shared = m == a.k;
-        // m is the same for the whole wave: the id comes through the scalar path
-        const uint8_t *w = is_shared ? a.sh_down : mat_ptr_expert<0>(a.down, sld_i32(a.ids + m));
-        const size_t rb = static_cast<size_t>(nb) * ((KIND == 0 || is_shared) ? 34 : 18);
-        const uint8_t *const rows[1] = {w + r0 * rb};
-        float y[1];
-        auto quantise = [&]() {
-            wave_lds_fence();
-            lds_quantize_q8_0(a.act + static_cast<size_t>(m) * a.F, a.F, aq, ad, lane, 64);
-            wave_lds_fence();
-            mark(a, 2, 1);
-        };
         if constexpr (COAL) {
-            if (KIND == 0 || is_shared)
-                y[0] = q8_rows4_coal<0, NB>(rows[0], aq, ad, tiles[wave], lane, quantise);
-            else
-                y[0] = q8_rows4_coal<1, NB>(rows[0], aq, ad, tiles[wave], lane, quantise);
+            // the activation first: its address needs no expert id, and loads return in order - it is quantised while
+            // the weights are still on their way
+            float4 v[kActRegs];
+            request_act(m, v);
+            const uint8_t *w = is_shared ? a.sh_down : mat_ptr_expert_uniform<0>(a.down, sld_i32(a.ids + m));
+            float y;
+            if (KIND == 0 || is_shared) {
+                const auto raw = q8_rows4_coal_request<0, NB>(w + static_cast<size_t>(r0) * NB * 34, lane);
+                wave_lds_fence();
+                quantise_act(v, aq, ad);
+                mark(a, 2, 1);
+                y = q8_rows4_coal_finish<0, NB>(raw, aq, ad, tiles[wave], lane);
+            } else {
+                const auto raw = q8_rows4_coal_request<1, NB>(w + static_cast<size_t>(r0) * NB * 18, lane);
+                wave_lds_fence();
+                quantise_act(v, aq, ad);
+                mark(a, 2, 1);
+                y = q8_rows4_coal_finish<1, NB>(raw, aq, ad, tiles[wave], lane);
+            }
+            if ((lane & 15) == 0) ybuf[m * 4 + r4] = y;
         } else {
+            // m is the same for the whole wave: the id comes through the scalar path
+            const uint8_t *w = is_shared ? a.sh_down : mat_ptr_expert_uniform<0>(a.down, sld_i32(a.ids + m));
+            const size_t rb = static_cast<size_t>(nb) * ((KIND == 0 || is_shared) ? 34 : 18);
+            const uint8_t *const rows[1] = {w + r0 * rb};
+            float y[1];
+            auto quantise = [&]() {
+                wave_lds_fence();
+                lds_quantize_q8_0(a.act + static_cast<size_t>(m) * a.F, a.F, aq, ad, lane, 64);
+                wave_lds_fence();
+                mark(a, 2, 1);
+            };
             if (KIND == 0 || is_shared)
                 q8_rows4_multi<0, 1, 1, false>(rows, nrows, nb, aq, ad, tiles[wave], lane, y, nullptr, 0, quantise);
             else
                 q8_rows4_multi<1, 1, 1, false>(rows, nrows, nb, aq, ad, tiles[wave], lane, y, nullptr, 0, quantise);
+            if ((lane & 15) == 0) ybuf[m * 4 + r4] = y[0];
         }
-        if ((lane & 15) == 0) ybuf[m * 4 + r4] = y[0];
         mark(a, 2, 2);
     }
     __syncthreads();

@@ -44,6 +44,14 @@ WD_DEV const uint8_t *mat_ptr_expert(const MatSrc &s, int e) {
     return s.base[T] + static_cast<size_t>(e) * s.stride[T];
 }
 
+// The same for an e that is the same in every lane: the slot comes through the scalar path, so the lookup neither
+// waits for nor is counted among the wave's vector loads.
+template <int T>
+WD_DEV const uint8_t *mat_ptr_expert_uniform(const MatSrc &s, int e) {
+    if (s.slot_of_expert) return s.pool + static_cast<size_t>(sld_i32(s.slot_of_expert + e)) * s.slot_bytes + s.slot_off[T];
+    return s.base[T] + static_cast<size_t>(e) * s.stride[T];
+}
+
 __global__ void k_fill_u32(uint32_t *dst, uint32_t v, size_t n) {
     const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i < n) dst[i] = v;

@@ -478,7 +478,9 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
     int waves_c = n_act < 16 ? n_act : 16;
     if (grid_c > 512) waves_c = (n_act + 1) / 2;
     const size_t per_wave = (static_cast<size_t>(F) + F / 16 + 15) & ~static_cast<size_t>(15);
-    const size_t lds_c = waves_c * per_wave + sizeof(float) * 4 * n_act;
+    const bool two = waves_c < n_act;  // halved above: n_act <= 2 * waves_c
+    // such a wave keeps both quantised activations and the second row group (at most 4 rows of F / 32 34-byte blocks) in LDS
+    const size_t lds_c = waves_c * (two ? 2 * per_wave + static_cast<size_t>(4) * (F / 32) * 34 : per_wave) + sizeof(float) * 4 * n_act;
     auto al16 = [](const void *p_, size_t v) { return reinterpret_cast<uintptr_t>(p_) % 16 == 0 && v % 16 == 0; };
     // rows of 16 or 20 blocks in 16-byte aligned groups of four: the coalesced fetch
     const bool coal = (F == 512 || F == 640) && H % 4 == 0 && al16(L->shared_down, 0) &&
@@ -486,7 +488,6 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
                                          : al16(L->down, L->down_stride));
     const dim3 grid(grid_c), block(64 * waves_c);
     const bool q8 = L->down_type == WD_TYPE_Q8_0;
-    const bool two = waves_c < n_act;  // halved above: n_act <= 2 * waves_c
     if (coal && two) {
         if (F == 512 && q8) k_layer_c<0, true, 16, true><<<grid, block, lds_c, st>>>(a);
         else if (F == 512) k_layer_c<1, true, 16, true><<<grid, block, lds_c, st>>>(a);

@@ -799,22 +799,38 @@ WD_DEV Q8CoalRaw<KIND, NB> q8_rows4_coal_request(const uint8_t *rows, int lane) 
     for (int i = 0; i < Raw::kLoads; ++i) raw.u[i] = gld_u128_aligned(rows + 16 * min(i * 64 + lane, Raw::kWords - 1));
     return raw;
 }
-// y of row r4 valid in lane 16 r4.  The float order is that of q8_rows4_multi.
+// The fetched words into a staging area of Raw::kWords 16-byte words (the caller fences).
 template <int KIND, int NB>
-WD_DEV float q8_rows4_coal_finish(const Q8CoalRaw<KIND, NB> &raw, const int8_t *act_qs, const uint16_t *act_d, Q8TileNB<NB> &tile,
-                                  int lane) {
+WD_DEV void q8_rows4_coal_stage(const Q8CoalRaw<KIND, NB> &raw, uint8_t *stage, int lane) {
     using Raw = Q8CoalRaw<KIND, NB>;
-    constexpr int kSecond = 4 * NB - 64, kRow = Q8TileNB<NB>::kRow;
-    uint8_t *stage = reinterpret_cast<uint8_t *>(&tile);  // chunk sums and scales together are large enough
-    wave_lds_fence();  // earlier reads of the tile are done before it is overwritten
 #pragma unroll
     for (int i = 0; i < Raw::kLoads; ++i) reinterpret_cast<uint4 *>(stage)[min(i * 64 + lane, Raw::kWords - 1)] = raw.u[i];
-    wave_lds_fence();
+}
+// Request and staging for a kind only known at run time (words: Q8CoalRaw<kind, NB>::kWords, the same in every lane):
+// always as many loads as Q8_0 rows need, the surplus ones repeating the last word, so that the number of loads in
+// flight does not depend on the kind.
+template <int NB>
+WD_DEV Q8CoalRaw<0, NB> q8_rows4_coal_request_any(const uint8_t *rows, int words, int lane) {
+    Q8CoalRaw<0, NB> raw;
+#pragma unroll
+    for (int i = 0; i < Q8CoalRaw<0, NB>::kLoads; ++i) raw.u[i] = gld_u128_aligned(rows + 16 * min(i * 64 + lane, words - 1));
+    return raw;
+}
+template <int NB>
+WD_DEV void q8_rows4_coal_stage_any(const Q8CoalRaw<0, NB> &raw, uint8_t *stage, int words, int lane) {
+#pragma unroll
+    for (int i = 0; i < Q8CoalRaw<0, NB>::kLoads; ++i) reinterpret_cast<uint4 *>(stage)[min(i * 64 + lane, words - 1)] = raw.u[i];
+}
+// The dot products of the four staged rows; `stage` may be the tile itself (its chunk-sum area is overwritten only
+// after the staged bytes have been read).  y of row r4 valid in lane 16 r4.  The float order is that of q8_rows4_multi.
+template <int KIND, int NB>
+WD_DEV float q8_rows4_coal_dots(const uint8_t *stage, const int8_t *act_qs, const uint16_t *act_d, Q8TileNB<NB> &tile, int lane) {
+    constexpr int kSecond = 4 * NB - 64, kRow = Q8TileNB<NB>::kRow;
     const int t1 = 64 + min(lane, max(kSecond, 1) - 1);
     const Q8Block w0 = q8_block_from_lds<KIND>(stage, lane);
     Q8Block w1 = w0;
     if (kSecond > 0) w1 = q8_block_from_lds<KIND>(stage, t1);
-    wave_lds_fence();  // the staged bytes have been read; the area now takes the chunk sums
+    wave_lds_fence();  // the staged bytes (and, by an earlier call, the tile) have been read; the tile now takes the chunk sums
     auto sums = [&](const Q8Block &w, int t) {
         const int row = t / NB, bi = t - row * NB;
         const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + bi * 32);
@@ -841,6 +857,15 @@ WD_DEV float q8_rows4_coal_finish(const Q8CoalRaw<KIND, NB> &raw, const int8_t *
             acc = __builtin_fmaf(dv, pv, acc);
     }
     return close_lanes8(KIND == 1 ? acc + acc_odd : acc);
+}
+template <int KIND, int NB>
+WD_DEV float q8_rows4_coal_finish(const Q8CoalRaw<KIND, NB> &raw, const int8_t *act_qs, const uint16_t *act_d, Q8TileNB<NB> &tile,
+                                  int lane) {
+    uint8_t *stage = reinterpret_cast<uint8_t *>(&tile);  // chunk sums and scales together are large enough
+    wave_lds_fence();  // earlier reads of the tile are done before it is overwritten
+    q8_rows4_coal_stage<KIND, NB>(raw, stage, lane);
+    wave_lds_fence();
+    return q8_rows4_coal_dots<KIND, NB>(stage, act_qs, act_d, tile, lane);
 }
 // rows: first of the four rows.  `pre` runs between the request and the first read of the activation.
 template <int KIND, int NB, typename Pre = NoPre>
