@@ -39,6 +39,7 @@ struct LayerArgs {
     int dry;                     // measurement aid: every workgroup returns at once
     int preselected;
     int n_router_wgs;            // workgroups of dispatch A that take router rows
+    int n_routed_items;          // merged dispatch: (expert rung, group of eight rows) items shared by the routed workgroups
     unsigned *arrive;            // device counter of finished router workgroups (zero between dispatches)
     uint32_t *ids_tagged;        // [kTagCopies][16] selected ids published inside the merged dispatch (kTagInvalid = not yet)
     int clear_tagged;            // dispatch C resets ids_tagged when it is done with the layer
@@ -740,7 +741,9 @@ __global__ __launch_bounds__(512) void k_layer_a(LayerArgs a) {
 // COAL (IQ types): rows of eight super-blocks on 16-byte boundaries are fetched with one aligned 16-byte load per
 // lane and parked in LDS (iq_rows8_coal); dynamic LDS then has 8 * 2 * kIqStageBytes more bytes behind the 4 * H + 16.
 // NB (COAL only): super-blocks per row, 8 (hidden 2048) or 10 (hidden 2560).
-template <int TYPE, bool COAL, int NB = 8>
+// LOOP: the grid has fewer routed workgroups than there are (expert rung, group of eight rows) items; they walk them
+// with the stride of their number.
+template <int TYPE, bool COAL, int NB = 8, bool LOOP = false>
 __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
     constexpr bool kIq = (TYPE == 21 || TYPE == 22);
     extern __shared__ __align__(16) uint8_t lds_ab[];
@@ -819,8 +822,6 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
 
     // routed gate/up: set-up that does not need the ids
     const int bw = wg - a.n_router_wgs - n_shared_wgs;
-    const int j = bw / groups;
-    const int rg = bw - j * groups;
     IqTables &tables = *reinterpret_cast<IqTables *>(s_union);
     if (kIq) {
         stage_tables<TYPE == 21, TYPE == 22>(tables, threadIdx.x, 512);
@@ -831,50 +832,60 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
     }
     mark(a, 1, 1);
     __shared__ int s_expert;
-    if (threadIdx.x == 0) {
-        const uint32_t *src = a.ids_tagged + (bw & (kTagCopies - 1)) * 16 + j;
-        uint32_t e = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        unsigned polls = 0;
-        while (e == kTagInvalid && ++polls < a.spin_limit) {
-            __builtin_amdgcn_s_sleep(4);
-            e = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int n_routed_wgs = LOOP ? static_cast<int>(gridDim.x) - a.n_router_wgs - n_shared_wgs : 0;
+    int item = bw;
+    do {  // one item per workgroup unless the grid was capped (LOOP)
+        const int j = item / groups;
+        const int rg = item - j * groups;
+        if (threadIdx.x == 0) {
+            const uint32_t *src = a.ids_tagged + (bw & (kTagCopies - 1)) * 16 + j;
+            uint32_t e = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            unsigned polls = 0;
+            while (e == kTagInvalid && ++polls < a.spin_limit) {
+                __builtin_amdgcn_s_sleep(4);
+                e = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if (e == kTagInvalid) __hip_atomic_store(a.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_expert = static_cast<int>(e);
         }
-        if (e == kTagInvalid) __hip_atomic_store(a.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_expert = static_cast<int>(e);
-    }
-    __syncthreads();
-    mark(a, 1, 2);
-    const int e = s_expert;
-    if (e < 0 || e >= a.E) return;  // the wait ran out (status is set): leave without touching memory
-    const uint8_t *gate = mat_ptr_expert<0>(a.gate_up, e);
-    const uint8_t *up = mat_ptr_expert<1>(a.gate_up, e);
-    float *act = a.act + static_cast<size_t>(j) * a.F;
-    const int r = rg * 8 + wave;
-    float gu[2];
-    if (kIq) {
-        const int nb = a.H >> 8;
-        const size_t rb = static_cast<size_t>(nb) * (TYPE == 21 ? 110 : 82);
-        const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
-        const uint8_t *const rows[2] = {uniform_ptr(gate + off), uniform_ptr(up + off)};  // one row pair per wave
-        if (COAL && NB == 10)
-            iq_rows10_coal<(kIq ? TYPE : 21), 2>(rows, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
-                                                 lds_ab + ((4 * a.H + 16 + 15) & ~15) + wave * 2 * kIqStage10Bytes);
-        else if (COAL)
-            iq_rows8_coal<(kIq ? TYPE : 21), 2>(rows, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
-                                                lds_ab + ((4 * a.H + 16 + 15) & ~15) + wave * 2 * kIqStageBytes);
-        else
-            iq_rows_q8k<(kIq ? TYPE : 21), 2, false>(rows, nb, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
-                                                      nullptr, 0);
-    } else {
-        Q8RowTile *tiles = reinterpret_cast<Q8RowTile *>(s_union);
-        const int nb = a.H >> 5;
-        const size_t rb = static_cast<size_t>(nb) * 34;
-        const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
-        const uint8_t *const rows[2] = {gate + off, up + off};
-        q8_row_wave<2>(rows, nb, xq, reinterpret_cast<const uint16_t *>(xscale), tiles[wave], lane, gu);
-    }
-    if (lane == 0 && r < a.F) act[r] = silu_ggml(gu[0]) * gu[1];
-    mark(a, 1, 3);
+        __syncthreads();
+        mark(a, 1, 2);
+        const int e = s_expert;
+        if (e < 0 || e >= a.E) return;  // the wait ran out (status is set): leave without touching memory
+        const uint8_t *gate = mat_ptr_expert<0>(a.gate_up, e);
+        const uint8_t *up = mat_ptr_expert<1>(a.gate_up, e);
+        float *act = a.act + static_cast<size_t>(j) * a.F;
+        const int r = rg * 8 + wave;
+        float gu[2];
+        if (kIq) {
+            const int nb = a.H >> 8;
+            const size_t rb = static_cast<size_t>(nb) * (TYPE == 21 ? 110 : 82);
+            const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
+            const uint8_t *const rows[2] = {uniform_ptr(gate + off), uniform_ptr(up + off)};  // one row pair per wave
+            if (COAL && NB == 10)
+                iq_rows10_coal<(kIq ? TYPE : 21), 2>(rows, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
+                                                     lds_ab + ((4 * a.H + 16 + 15) & ~15) + wave * 2 * kIqStage10Bytes);
+            else if (COAL)
+                iq_rows8_coal<(kIq ? TYPE : 21), 2>(rows, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
+                                                    lds_ab + ((4 * a.H + 16 + 15) & ~15) + wave * 2 * kIqStageBytes);
+            else
+                iq_rows_q8k<(kIq ? TYPE : 21), 2, false>(rows, nb, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
+                                                          nullptr, 0);
+        } else {
+            Q8RowTile *tiles = reinterpret_cast<Q8RowTile *>(s_union);
+            const int nb = a.H >> 5;
+            const size_t rb = static_cast<size_t>(nb) * 34;
+            const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
+            const uint8_t *const rows[2] = {gate + off, up + off};
+            q8_row_wave<2>(rows, nb, xq, reinterpret_cast<const uint16_t *>(xscale), tiles[wave], lane, gu);
+        }
+        if (lane == 0 && r < a.F) act[r] = silu_ggml(gu[0]) * gu[1];
+        mark(a, 1, 3);
+        if (LOOP) {
+            item += n_routed_wgs;
+            __syncthreads();  // s_expert is free for the next item
+        }
+    } while (LOOP && item < a.n_routed_items);
 }
 
 // ---- dispatch B -----------------------------------------------------------------------------------------
