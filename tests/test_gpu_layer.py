@@ -104,6 +104,20 @@ def test_model_shape_layers(g, oracle, gate_t, down_t):
     check_layer(g, oracle, L, x)
 
 
+@pytest.mark.parametrize("H,F,gate_t,down_t,shared", [(2048, 512, synth.IQ3_S, synth.Q8_0, True),
+                                                      (2560, 640, synth.IQ2_S, synth.IQ4_NL, True),
+                                                      (1792, 512, synth.IQ3_S, synth.Q8_0, False),
+                                                      (2048, 512, synth.Q8_0, synth.Q8_0, True)])
+def test_more_routed_items_than_the_device_holds(g, oracle, H, F, gate_t, down_t, shared):
+    """Top-16: 16 * ffn / 8 = 1024 or 1280 (rung, row group) items of routed gate/up work, more than the workgroups an
+    MI355X holds at once, so the routed workgroups of the merged dispatch walk them in a loop; 17 matrices in the down
+    dispatch (waves with two matrices each at hidden 2560, one of them without a second)."""
+    E, k = 32, 16
+    L = synth.make_layer(H, F, E, k, gate_t, down_t, shared, seed=SEED, layer=79, router_sigma=1.0 / np.sqrt(H))
+    x = synth.rms_normed(synth.rng_for(SEED, 51, H), H)
+    check_layer(g, oracle, L, x)
+
+
 @pytest.mark.parametrize("shared", [True, False])
 def test_iq4_nl_down_rows_of_16_blocks(g, oracle, shared):
     """IQ4_NL down projection at ffn 512: the aligned fetch of four 16-block rows (with and without the Q8_0 shared

@@ -492,8 +492,9 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
     // One wave per matrix (k routed and the shared one).  A compute unit holds two such workgroups; when the grid has
     // more than the chip holds at once (hidden > 2048), waves take two matrices each instead, so that the smaller
     // workgroups all run together rather than in two rounds.
-    int waves_c = n_act < 16 ? n_act : 16;
-    if (grid_c > 512) waves_c = (n_act + 1) / 2;
+    // (With k = 16 and a shared expert there are 17 matrices, more than the 16 waves of a workgroup: halved as well.)
+    int waves_c = n_act;
+    if (grid_c > 512 || n_act > 16) waves_c = (n_act + 1) / 2;
     const size_t per_wave = (static_cast<size_t>(F) + F / 16 + 15) & ~static_cast<size_t>(15);
     const bool two = waves_c < n_act;  // halved above: n_act <= 2 * waves_c
     // such a wave keeps both quantised activations and the second row group (at most 4 rows of F / 32 34-byte blocks) in LDS
@@ -506,6 +507,7 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
     const dim3 grid(grid_c), block(64 * waves_c);
     const bool q8 = L->down_type == WD_TYPE_Q8_0;
     if (coal && two) {
+        if (waves_c > 9) return fail(WD_ERR_ARG, "fused layer: %d waves in the paired down dispatch (at most 9)", waves_c);
         if (F == 512 && q8) k_layer_c<0, true, 16, true><<<grid, block, lds_c, st>>>(a);
         else if (F == 512) k_layer_c<1, true, 16, true><<<grid, block, lds_c, st>>>(a);
         else if (q8) k_layer_c<0, true, 20, true><<<grid, block, lds_c, st>>>(a);
