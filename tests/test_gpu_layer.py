@@ -118,6 +118,20 @@ def test_more_routed_items_than_the_device_holds(g, oracle, H, F, gate_t, down_t
     check_layer(g, oracle, L, x)
 
 
+@pytest.mark.parametrize("H,F,E,k,gate_t,down_t,shared", [
+    (256, 32, 8, 1, synth.IQ3_S, synth.Q8_0, False),          # the smallest layer the limits allow
+    (256, 32, 1024, 16, synth.IQ2_S, synth.IQ4_NL, True),     # most experts, largest top-k
+    (2560, 640, 8, 1, synth.IQ2_S, synth.IQ4_NL, False),      # one matrix in the down dispatch
+    (2560, 640, 16, 2, synth.IQ3_S, synth.Q8_0, False),       # two: one paired wave
+    (512, 32, 8, 8, synth.Q8_0, synth.Q8_0, True),            # every expert selected
+    (3072, 96, 16, 4, synth.IQ3_S, synth.IQ4_NL, True),       # more than 2560 columns, odd number of down blocks
+    (4096, 1024, 16, 4, synth.Q8_0, synth.Q8_0, True)])       # two full spans, down rows of 32 blocks
+def test_corners_of_the_documented_limits(g, oracle, H, F, E, k, gate_t, down_t, shared):
+    L = synth.make_layer(H, F, E, k, gate_t, down_t, shared, seed=SEED, layer=80 + k, router_sigma=1.0 / np.sqrt(H))
+    x = synth.rms_normed(synth.rng_for(SEED, 52, H + E), H)
+    check_layer(g, oracle, L, x)
+
+
 @pytest.mark.parametrize("shared", [True, False])
 def test_iq4_nl_down_rows_of_16_blocks(g, oracle, shared):
     """IQ4_NL down projection at ffn 512: the aligned fetch of four 16-block rows (with and without the Q8_0 shared
