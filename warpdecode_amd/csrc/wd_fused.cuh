@@ -305,10 +305,15 @@ WD_DEV void topk_wave_m(const float *logits, int n, int k, float w_scale, int32_
 //      If not (ties - which also make the counted ranks collide -, rounding inversions, rows with -inf or NaN,
 //      a dead row) wave 0 runs the reference's rungs over the probabilities themselves.
 // lds: 4 * (512 * M + 600) bytes of scratch.  The results are written by wave 0 (lanes 0..k-1).
+// tagged != null: as soon as the ids are known - before the renormalisation, which only the weights need - id j
+// goes to tagged[c * 16 + j] of the `copies` replicas with device-scope atomic stores (the readers poll them).
+// Ids given by the caller (override_ids) are requested up front, so their round trip is not behind the selection.
 template <int M>
 WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32_t *ids, float *weights,
                          const int32_t *__restrict__ override_ids, uint8_t *lds, int lane, int wave,
-                         unsigned long long *stamps = nullptr) {
+                         unsigned long long *stamps = nullptr, uint32_t *tagged = nullptr, int copies = 0) {
+    int id_given = 0;
+    if (override_ids && wave == 0 && lane < k) id_given = override_ids[lane];
 #define WD_STAMP(i) do { if (stamps && wave == 0 && lane == 0) stamps[i] = wall_clock64(); } while (0)
     float *p = reinterpret_cast<float *>(lds);        // [512 M] probabilities by expert id
     float *wmax = p + 512 * M;                        // [8] largest logit of each wave
@@ -478,8 +483,15 @@ WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32
                 for (int i = 0; i < 8; ++i) v[8 * m + i] = p[(lane + 64 * m) * 8 + i];
             rungs_on_probs<M>(v, k, lane, top_mine, id_mine);
         }
+        if (override_ids) id_mine = id_given;
         WD_STAMP(6);
-        finish_weights(top_mine, id_mine, k, w_scale, ids, weights, override_ids, lane);
+        if (tagged && lane < k) {
+#pragma unroll 4
+            for (int c = 0; c < copies; ++c)
+                __hip_atomic_store(tagged + c * 16 + lane, static_cast<uint32_t>(id_mine), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        }
+        finish_weights(top_mine, id_mine, k, w_scale, ids, weights, nullptr, lane);
         WD_STAMP(7);
     }
 #undef WD_STAMP
@@ -487,11 +499,11 @@ WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32
 
 WD_DEV void topk_block(const float *logits, int n, int k, float w_scale, int32_t *ids, float *weights,
                        const int32_t *__restrict__ override_ids, uint8_t *lds, int lane, int wave,
-                       unsigned long long *stamps = nullptr) {
+                       unsigned long long *stamps = nullptr, uint32_t *tagged = nullptr, int copies = 0) {
     if (n <= 512)
-        topk_block_m<1>(logits, n, k, w_scale, ids, weights, override_ids, lds, lane, wave, stamps);
+        topk_block_m<1>(logits, n, k, w_scale, ids, weights, override_ids, lds, lane, wave, stamps, tagged, copies);
     else
-        topk_block_m<2>(logits, n, k, w_scale, ids, weights, override_ids, lds, lane, wave, stamps);
+        topk_block_m<2>(logits, n, k, w_scale, ids, weights, override_ids, lds, lane, wave, stamps, tagged, copies);
 }
 
 template <bool COHERENT>
@@ -773,19 +785,14 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
             // results land behind the selection's own scratch
             int32_t *lds_ids = reinterpret_cast<int32_t *>(s_union + 4 * (1024 + 600));
             float *lds_w = reinterpret_cast<float *>(s_union + 4 * (1024 + 600) + 64);
+            // the selection itself publishes the replicas that the routed workgroups wait for, ahead of the weights
             topk_block(a.logits, a.E, a.k, a.w_scale, lds_ids, lds_w, a.ids_override, s_union, lane, wave,
-                       a.trace ? a.trace + (0 * 16 + 9) * 8 : nullptr);
+                       a.trace ? a.trace + (0 * 16 + 9) * 8 : nullptr, a.ids_tagged, kTagCopies);
             if (wave == 0) {
                 wave_lds_fence();
-                const int id = lds_ids[lane & 15];
-                // replicas first (the routed workgroups wait for them), then the plain copies for dispatch C
-#pragma unroll 4
-                for (int c = 0; c < kTagCopies; ++c)
-                    if (lane < a.k)
-                        __hip_atomic_store(a.ids_tagged + c * 16 + lane, static_cast<uint32_t>(id), __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
+                // the plain copies for dispatch C
                 if (lane < a.k) {
-                    a.ids[lane] = id;
+                    a.ids[lane] = lds_ids[lane];
                     a.weights[lane] = lds_w[lane];
                 }
                 if (a.trace && lane == 0) a.trace[(0 * 16 + 8) * 8 + 1] = wall_clock64();
