@@ -218,6 +218,21 @@ def test_selection_edge_rows(g, oracle, flags):
         r[E // 2 + 1] = r[E // 2]
         spike["router"] = r
         _fused_vs_oracle(g, oracle, spike, x, flags)
+        # near-ties: pairs of experts whose logits differ in the last places only, so that their exponentials are
+        # equal or adjacent floats and the order of the probabilities is decided by rounding
+        near = dict(L)
+        r = L["router"].copy()
+        r[1::2] = r[0::2]
+        j = int(np.argmax(np.abs(x)))
+        r[1::2, j] = np.nextafter(r[1::2, j], np.float32(np.inf))
+        near["router"] = r
+        _fused_vs_oracle(g, oracle, near, x, flags)
+        # logits of minus infinity: all but two experts, i.e. fewer finite logits than k
+        minf = dict(L)
+        r = L["router"].copy()
+        r[2:] = np.where(x > 0, np.float32(-np.inf), np.float32(np.inf))[None, :]
+        minf["router"] = r
+        _fused_vs_oracle(g, oracle, minf, x, flags)
 
 
 def test_selection_more_than_512_experts(g, oracle):

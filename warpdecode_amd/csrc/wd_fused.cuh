@@ -300,10 +300,12 @@ WD_DEV void topk_wave_m(const float *logits, int n, int k, float w_scale, int32_
 //      candidates and adds the counts in LDS); rank r < k makes it candidate r.  Meanwhile the exponentials and
 //      the per-8 sums (a group is eight consecutive lanes) are computed eight waves wide;
 //   3. exp is monotone only up to rounding and equal probabilities must go to the lower id, so the candidates
-//      are checked against the probabilities: they are the reference's selection exactly when their
-//      probabilities are strictly decreasing and the last one is strictly above every probability left.
-//      If not (ties - which also make the counted ranks collide -, rounding inversions, rows with -inf or NaN,
-//      a dead row) wave 0 runs the reference's rungs over the probabilities themselves.
+//      are checked: they are the reference's selection exactly when their probabilities are strictly decreasing
+//      and the last one is strictly above every probability left.  The test is made on the exponentials, with a
+//      margin that carries it over to the probabilities (see there), so that the ids go out before the
+//      denominator is summed.  If it fails (ties - which also make the counted ranks collide -, near-ties,
+//      rounding inversions, rows with -inf or NaN, a dead row) wave 0 runs the reference's rungs over the
+//      probabilities themselves.
 // lds: 4 * (512 * M + 600) bytes of scratch.  The results are written by wave 0 (lanes 0..k-1).
 // tagged != null: as soon as the ids are known - before the renormalisation, which only the weights need - id j
 // goes to tagged[c * 16 + j] of the `copies` replicas with device-scope atomic stores (the readers poll them).
@@ -324,7 +326,6 @@ WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32
     int *sel = rank + 128;                            // [16] candidate r
     float *selp = reinterpret_cast<float *>(sel + 16);  // [16] its probability
     float *rest = selp + 16;                          // [8] largest unselected probability of each wave
-    float *bc = rest + 8;                             // [2] 1 / sum, dead flag
     const int groups = n >> 3;
     WD_STAMP(0);
 
@@ -407,17 +408,8 @@ WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32
     __syncthreads();
     WD_STAMP(3);
 
-    // wave 0: the denominator.  Waves 1, 2: candidates with rank < k take their place.
-    if (wave == 0) {
-        float gs[M];
-#pragma unroll
-        for (int m = 0; m < M; ++m) gs[m] = (lane + 64 * m < groups) ? gsum[m * 64 + lane] : 0.0f;
-        const double sum = sum_groups<M>(gs, groups, lane);
-        if (lane == 0) {
-            bc[0] = (sum == 0.0) ? 0.0f : static_cast<float>(1.0 / sum);
-            bc[1] = (sum == 0.0) ? 1.0f : 0.0f;
-        }
-    } else if (wave <= 2) {
+    // Waves 1, 2: candidates with rank < k take their place.
+    if (wave >= 1 && wave <= 2) {
         const int c = (wave - 1) * 64 + lane;
         const int r = rank[c];
         if (ci[c] >= 0 && r < k) sel[r] = ci[c];
@@ -425,15 +417,14 @@ WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32
     __syncthreads();
     WD_STAMP(4);
 
-    // 3. probabilities; the candidates' ones and the largest of the rest
-    const float inv = bc[0];
-    const bool dead = bc[1] != 0.0f;
-    float pv[M];
+    // 3. the candidates' exponentials and the largest of the rest.  The ids do not wait for the denominator:
+    //    p = e * inv with one inv in [2^-10, 1] for the whole row is monotone in e, and two exponentials that differ
+    //    by more than a few units in the last place (and are not tiny) cannot round to the same product, so the test
+    //    below on the exponentials implies the one on the probabilities.  A NaN counts as larger than everything.
     bool taken[M];
 #pragma unroll
     for (int m = 0; m < M; ++m) {
-        pv[m] = (id[m] < n && !dead) ? e[m] * inv : -INFINITY;
-        p[id[m]] = pv[m];
+        p[id[m]] = e[m];
         taken[m] = false;
     }
     {
@@ -449,15 +440,15 @@ WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32
                 for (int m = 0; m < M; ++m) {
                     if (4 * t + u < k && id[m] == sj[u]) {
                         taken[m] = true;
-                        selp[4 * t + u] = pv[m];
+                        selp[4 * t + u] = e[m];
                     }
                 }
             }
         }
     }
-    float rm = -INFINITY;
+    float rm = 0.0f;
 #pragma unroll
-    for (int m = 0; m < M; ++m) rm = __builtin_fmaxf(rm, taken[m] ? -INFINITY : pv[m]);
+    for (int m = 0; m < M; ++m) rm = __builtin_fmaxf(rm, taken[m] ? 0.0f : (e[m] != e[m] ? INFINITY : e[m]));
     rm = wave_max(rm);
     if (lane == 0) rest[wave] = rm;
     __syncthreads();
@@ -466,30 +457,49 @@ WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32
     if (wave == 0) {
         const int idc = (lane < k) ? sel[lane] : -1;
         const bool have = idc >= 0 && idc < n;
-        const float top = have ? selp[lane] : 0.0f;
+        const float top_e = have ? selp[lane] : 0.0f;
         float rest_all = rest[0];
 #pragma unroll
         for (int w = 1; w < 8; ++w) rest_all = __builtin_fmaxf(rest_all, rest[w]);
-        const float nxt = dpp_f<kDppShl1>(0.0f, top);  // k <= 16: the candidates sit in one row of lanes
-        const bool good = lane >= k || (have && (lane == k - 1 ? top > rest_all : top > nxt));
-        const bool all_good = !dead && __builtin_amdgcn_ballot_w64(good) == ~0ull;
-        float top_mine = top;
-        int id_mine = idc;
-        if (!all_good) {
-            float v[8 * M];
-#pragma unroll
-            for (int m = 0; m < M; ++m)
-#pragma unroll
-                for (int i = 0; i < 8; ++i) v[8 * m + i] = p[(lane + 64 * m) * 8 + i];
-            rungs_on_probs<M>(v, k, lane, top_mine, id_mine);
-        }
-        if (override_ids) id_mine = id_given;
-        WD_STAMP(6);
-        if (tagged && lane < k) {
+        const float nxt = dpp_f<kDppShl1>(0.0f, top_e);  // k <= 16: the candidates sit in one row of lanes
+        const float below = (lane == k - 1 ? rest_all : nxt) * 1.000001f;
+        const bool good = lane >= k || (have && top_e >= 0x1p-100f && top_e > below);
+        const bool all_good = __builtin_amdgcn_ballot_w64(good) == ~0ull;
+        int id_mine = override_ids ? id_given : idc;
+        if (all_good && tagged && lane < k) {
 #pragma unroll 4
             for (int c = 0; c < copies; ++c)
                 __hip_atomic_store(tagged + c * 16 + lane, static_cast<uint32_t>(id_mine), __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
+        }
+        WD_STAMP(6);
+
+        // the denominator (only the weights and the slow path need it)
+        float gs[M];
+#pragma unroll
+        for (int m = 0; m < M; ++m) gs[m] = (lane + 64 * m < groups) ? gsum[m * 64 + lane] : 0.0f;
+        const double sum = sum_groups<M>(gs, groups, lane);
+        const float inv = (sum == 0.0) ? 0.0f : static_cast<float>(1.0 / sum);
+        const bool dead = sum == 0.0;
+        float top_mine = top_e * inv;
+        if (!all_good) {
+            // ties, rounding inversions, -inf or NaN logits, a dead row: the reference's rungs over the probabilities
+            float v[8 * M];
+#pragma unroll
+            for (int m = 0; m < M; ++m)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int ix = (lane + 64 * m) * 8 + i;
+                    v[8 * m + i] = (ix < n && !dead) ? p[ix] * inv : -INFINITY;
+                }
+            rungs_on_probs<M>(v, k, lane, top_mine, id_mine);
+            if (override_ids) id_mine = id_given;
+            if (tagged && lane < k) {
+#pragma unroll 4
+                for (int c = 0; c < copies; ++c)
+                    __hip_atomic_store(tagged + c * 16 + lane, static_cast<uint32_t>(id_mine), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
         finish_weights(top_mine, id_mine, k, w_scale, ids, weights, nullptr, lane);
         WD_STAMP(7);
