@@ -291,21 +291,22 @@ WD_DEV void topk_wave_m(const float *logits, int n, int k, float w_scale, int32_
 
 // The same selection by a workgroup of eight waves (every thread must call it; it contains barriers).
 // Expert m * 512 + 64 * wave + lane belongs to (wave, lane): one or two logits per lane.  A wave instruction
-// takes four cycles and a chain of k dependent arg-max steps costs about 0.2 us each, so candidates are found by
-// counting instead:
-//   1. every lane counts how many LOGITS of its wave are larger than its own (one uniform read and a compare per
-//      value): its rank in the wave.  Ranks below k form the wave's sorted candidate list;
-//   2. the eight lists are merged the same way: the rank of a candidate is its rank in its own list plus, for
-//      every other list, the number of entries ahead of it (each wave counts its own list against all
-//      candidates and adds the counts in LDS); rank r < k makes it candidate r.  Meanwhile the exponentials and
-//      the per-8 sums (a group is eight consecutive lanes) are computed eight waves wide;
-//   3. exp is monotone only up to rounding and equal probabilities must go to the lower id, so the candidates
-//      are checked: they are the reference's selection exactly when their probabilities are strictly decreasing
-//      and the last one is strictly above every probability left.  The test is made on the exponentials, with a
-//      margin that carries it over to the probabilities (see there), so that the ids go out before the
-//      denominator is summed.  If it fails (ties - which also make the counted ranks collide -, near-ties,
-//      rounding inversions, rows with -inf or NaN, a dead row) wave 0 runs the reference's rungs over the
-//      probabilities themselves.
+// takes four cycles and a chain of k dependent arg-max steps costs about 0.2 us each, so the selection is made by
+// thresholding and counting instead:
+//   1. every row of 16 lanes publishes its largest logit (32 rows in the workgroup);
+//   2. every wave finds T, the smallest of the row maxima that have fewer than k larger ones: at least k logits are
+//      >= T, so the k largest are among the candidates {logit >= T} - a few dozen at most for any row that is not
+//      nearly constant.  The candidates (logit, exponential, id) are compacted into one list in LDS (ballot, one
+//      LDS atomic per wave); meanwhile the exponentials and the per-8 sums (a group is eight consecutive lanes)
+//      are computed eight waves wide, and every wave notes its largest exponential outside the candidates;
+//   3. wave 0 ranks the candidates by counting (one uniform read and a compare per candidate); rank r < k makes
+//      a candidate the r-th selected.  exp is monotone only up to rounding and equal probabilities must go to the
+//      lower id, so the result is checked: it is the reference's selection exactly when the probabilities are
+//      strictly decreasing and the last one is strictly above every probability left.  The test is made on the
+//      exponentials, with a margin that carries it over to the probabilities (see there), so that the ids go out
+//      before the denominator is summed.  If it fails (ties - which also make the counted ranks collide -,
+//      near-ties, rounding inversions, rows with -inf or NaN, a dead row, more than 64 candidates) wave 0 runs the
+//      reference's rungs over the probabilities themselves.
 // lds: 4 * (512 * M + 600) bytes of scratch.  The results are written by wave 0 (lanes 0..k-1).
 // tagged != null: as soon as the ids are known - before the renormalisation, which only the weights need - id j
 // goes to tagged[c * 16 + j] of the `copies` replicas with device-scope atomic stores (the readers poll them).
@@ -314,22 +315,24 @@ template <int M>
 WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32_t *ids, float *weights,
                          const int32_t *__restrict__ override_ids, uint8_t *lds, int lane, int wave,
                          unsigned long long *stamps = nullptr, uint32_t *tagged = nullptr, int copies = 0) {
+#define WD_STAMP(i) do { if (stamps && wave == 0 && lane == 0) stamps[i] = wall_clock64(); } while (0)
+    float *p = reinterpret_cast<float *>(lds);        // [512 M] exponentials by expert id
+    float *gsum = p + 512 * M;                        // [64 M] per-8 sums by group
+    float *rmx = gsum + 64 * M;                       // [32] largest logit of every row of 16 lanes
+    float *cl = rmx + 32;                             // [64] candidates: logit,
+    float *ce = cl + 64;                              // [64] exponential,
+    int *cid = reinterpret_cast<int *>(ce + 64);      // [64] id
+    int *ncand = cid + 64;                            // [4] their number
+    int *sel = ncand + 4;                             // [16] the r-th selected id
+    float *selp = reinterpret_cast<float *>(sel + 16);  // [16] its exponential
+    float *rest = selp + 16;                          // [8] largest exponential outside the candidates, by wave
+    const int groups = n >> 3;
+    auto nan_is_large = [](float v) { return v != v ? INFINITY : v; };
+    WD_STAMP(0);
     int id_given = 0;
     if (override_ids && wave == 0 && lane < k) id_given = override_ids[lane];
-#define WD_STAMP(i) do { if (stamps && wave == 0 && lane == 0) stamps[i] = wall_clock64(); } while (0)
-    float *p = reinterpret_cast<float *>(lds);        // [512 M] probabilities by expert id
-    float *wmax = p + 512 * M;                        // [8] largest logit of each wave
-    float *gsum = wmax + 8;                           // [64 M] per-8 sums by group
-    float *cv = gsum + 64 * M;                        // [8][16] sorted candidate logits of each wave
-    int *ci = reinterpret_cast<int *>(cv + 128);      // [8][16] their ids (-1: none)
-    int *rank = ci + 128;                             // [8][16] global ranks
-    int *sel = rank + 128;                            // [16] candidate r
-    float *selp = reinterpret_cast<float *>(sel + 16);  // [16] its probability
-    float *rest = selp + 16;                          // [8] largest unselected probability of each wave
-    const int groups = n >> 3;
-    WD_STAMP(0);
 
-    // 1. logits, largest of the wave, rank of every value inside the wave
+    // 1. logits, largest of every row
     float l[M];
     int id[M];
 #pragma unroll
@@ -337,131 +340,95 @@ WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32
         id[m] = m * 512 + wave * 64 + lane;
         l[m] = (id[m] < n) ? __hip_atomic_load(logits + id[m], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
     }
-    if (lane < 16) {
-        cv[wave * 16 + lane] = -INFINITY;
-        ci[wave * 16 + lane] = -1;
-        rank[wave * 16 + lane] = lane;
-        if (wave == 0) sel[lane] = -1;
-    }
-    float lm = l[0];
-#pragma unroll
-    for (int m = 1; m < M; ++m) lm = __builtin_fmaxf(lm, l[m]);
-    lm = wave_max(lm);
-    if (lane == 0) wmax[wave] = lm;
-    WD_STAMP(1);
+    if (wave == 0 && lane == 0) ncand[0] = 0;
     {
-        int larger[M];
+        float lm = l[0];
 #pragma unroll
-        for (int m = 0; m < M; ++m) larger[m] = 0;
-#pragma unroll
-        for (int m2 = 0; m2 < M; ++m2) {
-            // (partial unroll: a full one keeps every broadcast value in a scalar register at once)
-#pragma unroll 16
-            for (int src = 0; src < 64; ++src) {
-                const float other = readlane_f(l[m2], src);
-#pragma unroll
-                for (int m = 0; m < M; ++m) larger[m] += (other > l[m]) ? 1 : 0;
-            }
-        }
-        wave_lds_fence();
-#pragma unroll
-        for (int m = 0; m < M; ++m) {
-            if (larger[m] < k && l[m] > -INFINITY) {
-                cv[wave * 16 + larger[m]] = l[m];
-                ci[wave * 16 + larger[m]] = id[m];
-            }
-        }
+        for (int m = 1; m < M; ++m) lm = __builtin_fmaxf(lm, l[m]);
+        lm = __builtin_fmaxf(lm, dpp_f<kDppXor1>(lm, lm));
+        lm = __builtin_fmaxf(lm, dpp_f<kDppXor2>(lm, lm));
+        lm = __builtin_fmaxf(lm, dpp_f<kDppRor4>(lm, lm));
+        lm = __builtin_fmaxf(lm, dpp_f<kDppRor8>(lm, lm));
+        if ((lane & 15) == 0) rmx[wave * 4 + (lane >> 4)] = lm;
     }
     __syncthreads();
-    WD_STAMP(2);
+    WD_STAMP(1);
 
-    // 2. exponentials and per-8 sums; this wave's list counted against every candidate of the other lists
-    float mx = wmax[0];
+    // 2. threshold, exponentials and per-8 sums, candidate list
+    const float r = rmx[lane & 31];
+    const float mx = wave_max(r);
+    float thr;
+    {
+        int larger = 0;
 #pragma unroll
-    for (int w = 1; w < 8; ++w) mx = __builtin_fmaxf(mx, wmax[w]);
+        for (int src = 0; src < 32; ++src) larger += (readlane_f(r, src) > r) ? 1 : 0;
+        thr = -wave_max(larger < k ? -r : -INFINITY);
+    }
     float e[M];
+    float rme = 0.0f;
 #pragma unroll
     for (int m = 0; m < M; ++m) {
         e[m] = (id[m] < n) ? exp_ggml(l[m] - mx) : 0.0f;
         const float gs = close_lanes8(e[m]);
         if ((lane & 7) == 0) gsum[m * 64 + wave * 8 + (lane >> 3)] = gs;
-    }
-    {
-        float4 own_v[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) own_v[t] = *reinterpret_cast<const float4 *>(cv + wave * 16 + 4 * t);
-        const float val0 = cv[lane], val1 = cv[64 + lane];
-        int ahead0 = 0, ahead1 = 0;
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const float vv[4] = {own_v[t].x, own_v[t].y, own_v[t].z, own_v[t].w};
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                // empty entries hold -inf and are ahead of nothing; equal values collide (and fail the check)
-                ahead0 += (vv[u] > val0) ? 1 : 0;
-                ahead1 += (vv[u] > val1) ? 1 : 0;
-            }
-        }
-        if ((lane >> 4) != wave && ahead0) atomicAdd(&rank[lane], ahead0);
-        if ((4 + (lane >> 4)) != wave && ahead1) atomicAdd(&rank[64 + lane], ahead1);
-    }
-    __syncthreads();
-    WD_STAMP(3);
-
-    // Waves 1, 2: candidates with rank < k take their place.
-    if (wave >= 1 && wave <= 2) {
-        const int c = (wave - 1) * 64 + lane;
-        const int r = rank[c];
-        if (ci[c] >= 0 && r < k) sel[r] = ci[c];
-    }
-    __syncthreads();
-    WD_STAMP(4);
-
-    // 3. the candidates' exponentials and the largest of the rest.  The ids do not wait for the denominator:
-    //    p = e * inv with one inv in [2^-10, 1] for the whole row is monotone in e, and two exponentials that differ
-    //    by more than a few units in the last place (and are not tiny) cannot round to the same product, so the test
-    //    below on the exponentials implies the one on the probabilities.  A NaN counts as larger than everything.
-    bool taken[M];
-#pragma unroll
-    for (int m = 0; m < M; ++m) {
         p[id[m]] = e[m];
-        taken[m] = false;
-    }
-    {
-        int4 sq[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) sq[t] = *reinterpret_cast<const int4 *>(sel + 4 * t);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const int sj[4] = {sq[t].x, sq[t].y, sq[t].z, sq[t].w};
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-#pragma unroll
-                for (int m = 0; m < M; ++m) {
-                    if (4 * t + u < k && id[m] == sj[u]) {
-                        taken[m] = true;
-                        selp[4 * t + u] = e[m];
-                    }
-                }
+        const bool c = l[m] >= thr && l[m] > -INFINITY;
+        const unsigned long long cm = __builtin_amdgcn_ballot_w64(c);
+        if (cm != 0ull) {
+            int base = 0;
+            if (lane == 0) base = atomicAdd(ncand, static_cast<int>(__builtin_popcountll(cm)));
+            base = __builtin_amdgcn_readfirstlane(base);
+            const int pos = base + static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<unsigned>(cm >> 32),
+                                                        __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(cm), 0u)));
+            if (c && pos < 64) {
+                cl[pos] = l[m];
+                ce[pos] = e[m];
+                cid[pos] = id[m];
             }
         }
+        rme = __builtin_fmaxf(rme, c ? 0.0f : nan_is_large(e[m]));
     }
-    float rm = 0.0f;
-#pragma unroll
-    for (int m = 0; m < M; ++m) rm = __builtin_fmaxf(rm, taken[m] ? 0.0f : (e[m] != e[m] ? INFINITY : e[m]));
-    rm = wave_max(rm);
-    if (lane == 0) rest[wave] = rm;
+    rme = wave_max(rme);
+    if (lane == 0) rest[wave] = rme;
     __syncthreads();
-    WD_STAMP(5);
+    WD_STAMP(2);
 
     if (wave == 0) {
+        // 3. ranks of the candidates
+        const int nc = ncand[0];
+        const bool fits = nc <= 64;
+        const bool mine = fits && lane < nc;
+        const float my_l = mine ? cl[lane] : -INFINITY;
+        const float my_e = mine ? ce[lane] : 0.0f;
+        const int my_id = mine ? cid[lane] : -1;
+        if (lane < 16) sel[lane] = -1;
+        int rk = 0;
+        const int steps = fits ? (nc + 3) & ~3 : 0;  // lanes past the list hold -inf, which is ahead of nothing
+        for (int src = 0; src < steps; src += 4) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) rk += (readlane_f(my_l, src + u) > my_l) ? 1 : 0;
+        }
+        wave_lds_fence();
+        if (mine && rk < k) {
+            sel[rk] = my_id;  // equal logits collide here; the loser stays among the rest and fails the test below
+            selp[rk] = my_e;
+        }
+        wave_lds_fence();
+        const bool taken = mine && rk < k && sel[rk < k ? rk : 0] == my_id;
+        float rest_all = wave_max((mine && !taken) ? nan_is_large(my_e) : 0.0f);
+#pragma unroll
+        for (int w = 0; w < 8; ++w) rest_all = __builtin_fmaxf(rest_all, rest[w]);
+        if (!fits) rest_all = INFINITY;
+        WD_STAMP(3);
+
+        // The ids do not wait for the denominator: p = e * inv with one inv in [2^-10, 1] for the whole row is
+        // monotone in e, and two exponentials that differ by more than a few units in the last place (and are not
+        // tiny) cannot round to the same product, so this test on the exponentials implies the one on the
+        // probabilities.  A NaN counts as larger than everything.
         const int idc = (lane < k) ? sel[lane] : -1;
         const bool have = idc >= 0 && idc < n;
         const float top_e = have ? selp[lane] : 0.0f;
-        float rest_all = rest[0];
-#pragma unroll
-        for (int w = 1; w < 8; ++w) rest_all = __builtin_fmaxf(rest_all, rest[w]);
-        const float nxt = dpp_f<kDppShl1>(0.0f, top_e);  // k <= 16: the candidates sit in one row of lanes
+        const float nxt = dpp_f<kDppShl1>(0.0f, top_e);  // k <= 16: the selected sit in one row of lanes
         const float below = (lane == k - 1 ? rest_all : nxt) * 1.000001f;
         const bool good = lane >= k || (have && top_e >= 0x1p-100f && top_e > below);
         const bool all_good = __builtin_amdgcn_ballot_w64(good) == ~0ull;
@@ -483,7 +450,6 @@ WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32
         const bool dead = sum == 0.0;
         float top_mine = top_e * inv;
         if (!all_good) {
-            // ties, rounding inversions, -inf or NaN logits, a dead row: the reference's rungs over the probabilities
             float v[8 * M];
 #pragma unroll
             for (int m = 0; m < M; ++m)
