@@ -235,6 +235,37 @@ def test_selection_edge_rows(g, oracle, flags):
         _fused_vs_oracle(g, oracle, minf, x, flags)
 
 
+@pytest.mark.parametrize("E,k", [(8, 1), (64, 8), (128, 8), (512, 10), (512, 16), (520, 10), (1024, 16)])
+def test_selection_many_rows(g, oracle, E, k):
+    """Ids and weights of many random rows at three logit scales (the selection thresholds on row maxima and ranks the
+    candidates above the threshold), and a row whose large logits all sit in a few rows of lanes, so that there are
+    more candidates than the fast path holds."""
+    H, F = 256, 32
+    for si, sigma in enumerate((1e-3, 1.0 / 16, 0.5)):
+        L = synth.make_layer(H, F, E, k, synth.Q8_0, synth.Q8_0, False, seed=SEED, layer=960 + si, router_sigma=sigma)
+        dl = g.DeviceLayer(L)
+        sc = g.Scratch(H, F, E, k)
+        out = g.empty(H, np.float32)
+        for t in range(10):
+            x = synth.rms_normed(synth.rng_for(SEED, 48, 1000 * E + 16 * si + t), H)
+            want, d = oracle.moe_layer(L, x)
+            dx = g.dev(x)
+            capi.call("wd_moe_layer_f32", C.byref(dl.desc), g.ptr(dx), g.ptr(out), sc.h, 0, g.stream())
+            g.sync()
+            assert np.array_equal(sc.get("ids", k, np.int32), d["ids"]), (E, k, sigma, t)
+            assert g.same_bits(sc.get("weights", k, np.float32), d["weights"]), (E, k, sigma, t)
+            assert g.same_bits(g.host(out), want), (E, k, sigma, t)
+        sc.close()
+    if E >= 512:
+        L = synth.make_layer(H, F, E, k, synth.Q8_0, synth.Q8_0, False, seed=SEED, layer=970, router_sigma=1.0 / 16)
+        x = synth.rms_normed(synth.rng_for(SEED, 49, E), H)
+        r = L["router"].copy()
+        for i in range(144):                     # logits 3 + i / 144 in nine rows of 16 lanes
+            r[i] = x * np.float32((3.0 + i / 144.0) / H)
+        L["router"] = r
+        _fused_vs_oracle(g, oracle, L, x)
+
+
 def test_selection_more_than_512_experts(g, oracle):
     H, F, k = 256, 32, 10
     for E in (520, 1024):
