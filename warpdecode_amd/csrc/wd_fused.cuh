@@ -361,7 +361,10 @@ WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32
     {
         int larger = 0;
 #pragma unroll
-        for (int src = 0; src < 32; ++src) larger += (readlane_f(r, src) > r) ? 1 : 0;
+        for (int t = 0; t < 8; ++t) {  // the same 16 bytes for every lane: broadcast reads
+            const float4 q = *reinterpret_cast<const float4 *>(rmx + 4 * t);
+            larger += (q.x > r ? 1 : 0) + (q.y > r ? 1 : 0) + (q.z > r ? 1 : 0) + (q.w > r ? 1 : 0);
+        }
         thr = -wave_max(larger < k ? -r : -INFINITY);
     }
     float e[M];
@@ -396,11 +399,13 @@ WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32
     if (wave == 0) {
         // 3. ranks of the candidates
         const int nc = ncand[0];
+        const float got_l = cl[lane], got_e = ce[lane];  // requested together with the count, not behind it
+        const int got_id = cid[lane];
         const bool fits = nc <= 64;
         const bool mine = fits && lane < nc;
-        const float my_l = mine ? cl[lane] : -INFINITY;
-        const float my_e = mine ? ce[lane] : 0.0f;
-        const int my_id = mine ? cid[lane] : -1;
+        const float my_l = mine ? got_l : -INFINITY;
+        const float my_e = mine ? got_e : 0.0f;
+        const int my_id = mine ? got_id : -1;
         if (lane < 16) sel[lane] = -1;
         int rk = 0;
         const int steps = fits ? (nc + 3) & ~3 : 0;  // lanes past the list hold -inf, which is ahead of nothing
