@@ -192,6 +192,11 @@ int wd_moe_scratch_enable_partials(wd_moe_scratch *s, int gate_type, int down_ty
  * workgroups, 2 = dispatch C.  Only the traced workgroup pays for it.
  * Counterpart of the reference's kernel profiler sites, src/qwen38_moe.cuh:296-535. */
 unsigned long long *wd_moe_scratch_trace(wd_moe_scratch *s, int wg);
+/* The same for the one-launch form of wd_moe_stack_f32: uint64 [12][16] = [wave][point] of workgroup `wg` in layer
+ * `layer` (waves 0..9 routed rungs, 10 shared expert, 11 router row; points: 0 layer begin, 1 input seen, 2 input in
+ * LDS, 3 logits seen / logit stored, 4 id seen, 5 activation stored, 6 activations seen, 7 down rows done, 8/9 begin
+ * and end of the combine).  wg == -1: uint64 [512][4][16], waves 0, 9, 10 and 11 of every workgroup. */
+unsigned long long *wd_moe_scratch_trace_resident(wd_moe_scratch *s, int wg, int layer);
 
 /* flags for wd_moe_layer_f32 */
 #define WD_MOE_PRESELECTED 1u      /* ids/weights already in scratch: skip the router (reference `preselected`) */
@@ -204,6 +209,7 @@ unsigned long long *wd_moe_scratch_trace(wd_moe_scratch *s, int wg);
 #define WD_MOE_ONLY_C 0x40u /* down projections + combine */
 #define WD_MOE_SPLIT_AB 0x100u /* router and routed gate/up as two launches instead of one with an in-dispatch hand-off */
 #define WD_MOE_DRY 0x80u    /* every workgroup of the fused dispatches returns at once: the launch floor */
+#define WD_MOE_PER_LAYER 0x200u /* wd_moe_stack_f32: launch every layer's dispatches instead of one resident launch for the stack */
 
 /* One decode step of one layer: router -> top-k -> grouped gate/up -> SwiGLU -> Q8_0 ->
  * grouped down -> ordered weighted sum -> + shared * sigmoid gate.  d_out is f32 [hidden]
@@ -244,7 +250,14 @@ int wd_shared_expert_f32(const wd_moe_layer *layer, const float *d_x, wd_moe_scr
  * layer's output.  d_ids_trace (device int32 [n_layers][top_k], may be NULL) replays a routing trace:
  * the router still runs and its weights are used, but the expert ids come from the trace.
  * `layers` is a host array.  No counterpart in the reference, whose caller loops over layers
- * (Qwen38Decoder::step, src/qwen38_forward.cuh:2923-3371). */
+ * (Qwen38Decoder::step, src/qwen38_forward.cuh:2923-3371).
+ * Stacks of up to 64 layers of the 512-expert layer shape (hidden 2048, ffn 512, at most 512 experts, top-k <= 10,
+ * IQ3_S or IQ2_S gate/up, Q8_0 down, 16-byte aligned tensors, experts addressed directly) run as ONE launch of 512
+ * workgroups that stay on the device for the whole step and hand values to each other through global memory; this
+ * needs a device that holds the whole grid at once (checked) and flags == 0.  Everything else, and
+ * WD_MOE_PER_LAYER, takes the per-layer dispatches.  The results are the same bits either way.  The first call with
+ * a given set of layers allocates and uploads their descriptors (synchronous; not under stream capture, where an
+ * unseen set takes the per-layer dispatches). */
 int wd_moe_stack_f32(const wd_moe_layer *layers, int n_layers, float *d_x, float *d_layer_out,
                      wd_moe_scratch *scratch, const int32_t *d_ids_trace, float residual_scale, unsigned flags,
                      void *stream);

@@ -15,6 +15,7 @@ HEADER = os.path.join(os.path.dirname(HERE), "include", "warpdecode_amd.h")
 F32, F16, Q4_0, Q8_0, IQ4_NL, IQ3_S, IQ2_S = 0, 1, 2, 8, 20, 21, 22
 Q6_K = 14
 MOE_PRESELECTED, MOE_KEEP_EXPERT_OUT, MOE_STAGED = 1, 2, 4
+MOE_PER_LAYER = 0x200
 
 vp, i32, f32, sz, u32 = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint
 
@@ -89,6 +90,7 @@ _SIGS = {
     "wd_moe_scratch_destroy": (i32, [vp]),
     "wd_moe_scratch_enable_partials": (i32, [vp, i32, i32]),
     "wd_moe_scratch_trace": (vp, [vp, i32]),
+    "wd_moe_scratch_trace_resident": (vp, [vp, i32, i32]),
     "wd_moe_layer_f32": (i32, [C.POINTER(MoeLayer), vp, vp, vp, u32, vp]),
     "wd_moe_stack_cached_f32": (i32, [C.POINTER(MoeLayer), i32, vp, vp, vp, vp, vp, vp, f32, u32, vp]),
     "wd_moe_scratch_status": (i32, [vp]),

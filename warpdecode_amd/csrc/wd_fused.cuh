@@ -311,170 +311,196 @@ WD_DEV void topk_wave_m(const float *logits, int n, int k, float w_scale, int32_
 // tagged != null: as soon as the ids are known - before the renormalisation, which only the weights need - id j
 // goes to tagged[c * 16 + j] of the `copies` replicas with device-scope atomic stores (the readers poll them).
 // Ids given by the caller (override_ids) are requested up front, so their round trip is not behind the selection.
+// The three steps as functions of their own, so that a caller with the logits already in registers (or with waves
+// that only keep the barriers company) can compose them.  LDS layout of the selection's scratch:
 template <int M>
-WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32_t *ids, float *weights,
-                         const int32_t *__restrict__ override_ids, uint8_t *lds, int lane, int wave,
-                         unsigned long long *stamps = nullptr, uint32_t *tagged = nullptr, int copies = 0) {
-#define WD_STAMP(i) do { if (stamps && wave == 0 && lane == 0) stamps[i] = wall_clock64(); } while (0)
-    float *p = reinterpret_cast<float *>(lds);        // [512 M] exponentials by expert id
-    float *gsum = p + 512 * M;                        // [64 M] per-8 sums by group
-    float *rmx = gsum + 64 * M;                       // [32] largest logit of every row of 16 lanes
-    float *cl = rmx + 32;                             // [64] candidates: logit,
-    float *ce = cl + 64;                              // [64] exponential,
-    int *cid = reinterpret_cast<int *>(ce + 64);      // [64] id
-    int *ncand = cid + 64;                            // [4] their number
-    int *sel = ncand + 4;                             // [16] the r-th selected id
-    float *selp = reinterpret_cast<float *>(sel + 16);  // [16] its exponential
-    float *rest = selp + 16;                          // [8] largest exponential outside the candidates, by wave
-    const int groups = n >> 3;
+struct TopkLds {
+    float *p, *gsum, *rmx, *cl, *ce, *rest, *selp;
+    int *cid, *ncand, *sel;
+    WD_DEV explicit TopkLds(uint8_t *lds) {
+        p = reinterpret_cast<float *>(lds);        // [512 M] exponentials by expert id
+        gsum = p + 512 * M;                        // [64 M] per-8 sums by group
+        rmx = gsum + 64 * M;                       // [32] largest logit of every row of 16 lanes
+        cl = rmx + 32;                             // [64] candidates: logit,
+        ce = cl + 64;                              // [64] exponential,
+        cid = reinterpret_cast<int *>(ce + 64);    // [64] id
+        ncand = cid + 64;                          // [4] their number
+        sel = ncand + 4;                           // [16] the r-th selected id
+        selp = reinterpret_cast<float *>(sel + 16);  // [16] its exponential
+        rest = selp + 16;                          // [8] largest exponential outside the candidates, by wave
+    }
+};
+constexpr int kTopkLdsBytes1 = 4 * (512 + 600), kTopkLdsBytes2 = 4 * (1024 + 600);
+
+// Step 1 (waves 0..7, before the first barrier): the row maxima of the logits held in l[] (expert m * 512 + 64 * wave + lane).
+template <int M>
+WD_DEV void topk_block_step1(const float (&l)[M], const TopkLds<M> &s, int lane, int wave) {
+    if (wave == 0 && lane == 0) s.ncand[0] = 0;
+    float lm = l[0];
+#pragma unroll
+    for (int m = 1; m < M; ++m) lm = __builtin_fmaxf(lm, l[m]);
+    lm = __builtin_fmaxf(lm, dpp_f<kDppXor1>(lm, lm));
+    lm = __builtin_fmaxf(lm, dpp_f<kDppXor2>(lm, lm));
+    lm = __builtin_fmaxf(lm, dpp_f<kDppRor4>(lm, lm));
+    lm = __builtin_fmaxf(lm, dpp_f<kDppRor8>(lm, lm));
+    if ((lane & 15) == 0) s.rmx[wave * 4 + (lane >> 4)] = lm;
+}
+
+// Step 2 (waves 0..7, between the barriers): threshold, exponentials and per-8 sums, candidate list.
+template <int M>
+WD_DEV void topk_block_step2(const float (&l)[M], int n, int k, const TopkLds<M> &s, int lane, int wave) {
     auto nan_is_large = [](float v) { return v != v ? INFINITY : v; };
-    WD_STAMP(0);
-    int id_given = 0;
-    if (override_ids && wave == 0 && lane < k) id_given = override_ids[lane];
-
-    // 1. logits, largest of every row
-    float l[M];
-    int id[M];
-#pragma unroll
-    for (int m = 0; m < M; ++m) {
-        id[m] = m * 512 + wave * 64 + lane;
-        l[m] = (id[m] < n) ? __hip_atomic_load(logits + id[m], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
-    }
-    if (wave == 0 && lane == 0) ncand[0] = 0;
-    {
-        float lm = l[0];
-#pragma unroll
-        for (int m = 1; m < M; ++m) lm = __builtin_fmaxf(lm, l[m]);
-        lm = __builtin_fmaxf(lm, dpp_f<kDppXor1>(lm, lm));
-        lm = __builtin_fmaxf(lm, dpp_f<kDppXor2>(lm, lm));
-        lm = __builtin_fmaxf(lm, dpp_f<kDppRor4>(lm, lm));
-        lm = __builtin_fmaxf(lm, dpp_f<kDppRor8>(lm, lm));
-        if ((lane & 15) == 0) rmx[wave * 4 + (lane >> 4)] = lm;
-    }
-    __syncthreads();
-    WD_STAMP(1);
-
-    // 2. threshold, exponentials and per-8 sums, candidate list
-    const float r = rmx[lane & 31];
+    const float r = s.rmx[lane & 31];
     const float mx = wave_max(r);
     float thr;
     {
         int larger = 0;
 #pragma unroll
         for (int t = 0; t < 8; ++t) {  // the same 16 bytes for every lane: broadcast reads
-            const float4 q = *reinterpret_cast<const float4 *>(rmx + 4 * t);
+            const float4 q = *reinterpret_cast<const float4 *>(s.rmx + 4 * t);
             larger += (q.x > r ? 1 : 0) + (q.y > r ? 1 : 0) + (q.z > r ? 1 : 0) + (q.w > r ? 1 : 0);
         }
         thr = -wave_max(larger < k ? -r : -INFINITY);
     }
-    float e[M];
     float rme = 0.0f;
 #pragma unroll
     for (int m = 0; m < M; ++m) {
-        e[m] = (id[m] < n) ? exp_ggml(l[m] - mx) : 0.0f;
-        const float gs = close_lanes8(e[m]);
-        if ((lane & 7) == 0) gsum[m * 64 + wave * 8 + (lane >> 3)] = gs;
-        p[id[m]] = e[m];
+        const int id = m * 512 + wave * 64 + lane;
+        const float e = (id < n) ? exp_ggml(l[m] - mx) : 0.0f;
+        const float gs = close_lanes8(e);
+        if ((lane & 7) == 0) s.gsum[m * 64 + wave * 8 + (lane >> 3)] = gs;
+        s.p[id] = e;
         const bool c = l[m] >= thr && l[m] > -INFINITY;
         const unsigned long long cm = __builtin_amdgcn_ballot_w64(c);
         if (cm != 0ull) {
             int base = 0;
-            if (lane == 0) base = atomicAdd(ncand, static_cast<int>(__builtin_popcountll(cm)));
+            if (lane == 0) base = atomicAdd(s.ncand, static_cast<int>(__builtin_popcountll(cm)));
             base = __builtin_amdgcn_readfirstlane(base);
             const int pos = base + static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<unsigned>(cm >> 32),
                                                         __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(cm), 0u)));
             if (c && pos < 64) {
-                cl[pos] = l[m];
-                ce[pos] = e[m];
-                cid[pos] = id[m];
+                s.cl[pos] = l[m];
+                s.ce[pos] = e;
+                s.cid[pos] = id;
             }
         }
-        rme = __builtin_fmaxf(rme, c ? 0.0f : nan_is_large(e[m]));
+        rme = __builtin_fmaxf(rme, c ? 0.0f : nan_is_large(e));
     }
     rme = wave_max(rme);
-    if (lane == 0) rest[wave] = rme;
-    __syncthreads();
-    WD_STAMP(2);
+    if (lane == 0) s.rest[wave] = rme;
+}
 
-    if (wave == 0) {
-        // 3. ranks of the candidates
-        const int nc = ncand[0];
-        const float got_l = cl[lane], got_e = ce[lane];  // requested together with the count, not behind it
-        const int got_id = cid[lane];
-        const bool fits = nc <= 64;
-        const bool mine = fits && lane < nc;
-        const float my_l = mine ? got_l : -INFINITY;
-        const float my_e = mine ? got_e : 0.0f;
-        const int my_id = mine ? got_id : -1;
-        if (lane < 16) sel[lane] = -1;
-        int rk = 0;
-        const int steps = fits ? (nc + 3) & ~3 : 0;  // lanes past the list hold -inf, which is ahead of nothing
-        for (int src = 0; src < steps; src += 4) {
+// Step 3 (wave 0, after the second barrier): ranks, check, publication of the ids, denominator, weights.
+// id_given: the caller's id for lane j < k when the ids are replaced (override), requested before step 1.
+template <int M>
+WD_DEV void topk_block_step3(int n, int k, float w_scale, int32_t *ids, float *weights, bool override_ids, int id_given,
+                             const TopkLds<M> &s, int lane, unsigned long long *stamps, uint32_t *tagged, int copies) {
+#define WD_STAMP(i) do { if (stamps && lane == 0) stamps[i] = wall_clock64(); } while (0)
+    auto nan_is_large = [](float v) { return v != v ? INFINITY : v; };
+    const int groups = n >> 3;
+    // ranks of the candidates
+    const int nc = s.ncand[0];
+    const float got_l = s.cl[lane], got_e = s.ce[lane];  // requested together with the count, not behind it
+    const int got_id = s.cid[lane];
+    const bool fits = nc <= 64;
+    const bool mine = fits && lane < nc;
+    const float my_l = mine ? got_l : -INFINITY;
+    const float my_e = mine ? got_e : 0.0f;
+    const int my_id = mine ? got_id : -1;
+    if (lane < 16) s.sel[lane] = -1;
+    int rk = 0;
+    const int steps = fits ? (nc + 3) & ~3 : 0;  // lanes past the list hold -inf, which is ahead of nothing
+    for (int src = 0; src < steps; src += 4) {
 #pragma unroll
-            for (int u = 0; u < 4; ++u) rk += (readlane_f(my_l, src + u) > my_l) ? 1 : 0;
-        }
-        wave_lds_fence();
-        if (mine && rk < k) {
-            sel[rk] = my_id;  // equal logits collide here; the loser stays among the rest and fails the test below
-            selp[rk] = my_e;
-        }
-        wave_lds_fence();
-        const bool taken = mine && rk < k && sel[rk < k ? rk : 0] == my_id;
-        float rest_all = wave_max((mine && !taken) ? nan_is_large(my_e) : 0.0f);
+        for (int u = 0; u < 4; ++u) rk += (readlane_f(my_l, src + u) > my_l) ? 1 : 0;
+    }
+    wave_lds_fence();
+    if (mine && rk < k) {
+        s.sel[rk] = my_id;  // equal logits collide here; the loser stays among the rest and fails the test below
+        s.selp[rk] = my_e;
+    }
+    wave_lds_fence();
+    const bool taken = mine && rk < k && s.sel[rk < k ? rk : 0] == my_id;
+    float rest_all = wave_max((mine && !taken) ? nan_is_large(my_e) : 0.0f);
 #pragma unroll
-        for (int w = 0; w < 8; ++w) rest_all = __builtin_fmaxf(rest_all, rest[w]);
-        if (!fits) rest_all = INFINITY;
-        WD_STAMP(3);
+    for (int w = 0; w < 8; ++w) rest_all = __builtin_fmaxf(rest_all, s.rest[w]);
+    if (!fits) rest_all = INFINITY;
+    WD_STAMP(3);
 
-        // The ids do not wait for the denominator: p = e * inv with one inv in [2^-10, 1] for the whole row is
-        // monotone in e, and two exponentials that differ by more than a few units in the last place (and are not
-        // tiny) cannot round to the same product, so this test on the exponentials implies the one on the
-        // probabilities.  A NaN counts as larger than everything.
-        const int idc = (lane < k) ? sel[lane] : -1;
-        const bool have = idc >= 0 && idc < n;
-        const float top_e = have ? selp[lane] : 0.0f;
-        const float nxt = dpp_f<kDppShl1>(0.0f, top_e);  // k <= 16: the selected sit in one row of lanes
-        const float below = (lane == k - 1 ? rest_all : nxt) * 1.000001f;
-        const bool good = lane >= k || (have && top_e >= 0x1p-100f && top_e > below);
-        const bool all_good = __builtin_amdgcn_ballot_w64(good) == ~0ull;
-        int id_mine = override_ids ? id_given : idc;
-        if (all_good && tagged && lane < k) {
+    // The ids do not wait for the denominator: p = e * inv with one inv in [2^-10, 1] for the whole row is
+    // monotone in e, and two exponentials that differ by more than a few units in the last place (and are not
+    // tiny) cannot round to the same product, so this test on the exponentials implies the one on the
+    // probabilities.  A NaN counts as larger than everything.
+    const int idc = (lane < k) ? s.sel[lane] : -1;
+    const bool have = idc >= 0 && idc < n;
+    const float top_e = have ? s.selp[lane] : 0.0f;
+    const float nxt = dpp_f<kDppShl1>(0.0f, top_e);  // k <= 16: the selected sit in one row of lanes
+    const float below = (lane == k - 1 ? rest_all : nxt) * 1.000001f;
+    const bool good = lane >= k || (have && top_e >= 0x1p-100f && top_e > below);
+    const bool all_good = __builtin_amdgcn_ballot_w64(good) == ~0ull;
+    int id_mine = override_ids ? id_given : idc;
+    if (all_good && tagged && lane < k) {
+#pragma unroll 4
+        for (int c = 0; c < copies; ++c)
+            __hip_atomic_store(tagged + c * 16 + lane, static_cast<uint32_t>(id_mine), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+    }
+    WD_STAMP(6);
+
+    // the denominator (only the weights and the slow path need it)
+    float gs[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) gs[m] = (lane + 64 * m < groups) ? s.gsum[m * 64 + lane] : 0.0f;
+    const double sum = sum_groups<M>(gs, groups, lane);
+    const float inv = (sum == 0.0) ? 0.0f : static_cast<float>(1.0 / sum);
+    const bool dead = sum == 0.0;
+    float top_mine = top_e * inv;
+    if (!all_good) {
+        float v[8 * M];
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int ix = (lane + 64 * m) * 8 + i;
+                v[8 * m + i] = (ix < n && !dead) ? s.p[ix] * inv : -INFINITY;
+            }
+        rungs_on_probs<M>(v, k, lane, top_mine, id_mine);
+        if (override_ids) id_mine = id_given;
+        if (tagged && lane < k) {
 #pragma unroll 4
             for (int c = 0; c < copies; ++c)
                 __hip_atomic_store(tagged + c * 16 + lane, static_cast<uint32_t>(id_mine), __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
         }
-        WD_STAMP(6);
-
-        // the denominator (only the weights and the slow path need it)
-        float gs[M];
-#pragma unroll
-        for (int m = 0; m < M; ++m) gs[m] = (lane + 64 * m < groups) ? gsum[m * 64 + lane] : 0.0f;
-        const double sum = sum_groups<M>(gs, groups, lane);
-        const float inv = (sum == 0.0) ? 0.0f : static_cast<float>(1.0 / sum);
-        const bool dead = sum == 0.0;
-        float top_mine = top_e * inv;
-        if (!all_good) {
-            float v[8 * M];
-#pragma unroll
-            for (int m = 0; m < M; ++m)
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const int ix = (lane + 64 * m) * 8 + i;
-                    v[8 * m + i] = (ix < n && !dead) ? p[ix] * inv : -INFINITY;
-                }
-            rungs_on_probs<M>(v, k, lane, top_mine, id_mine);
-            if (override_ids) id_mine = id_given;
-            if (tagged && lane < k) {
-#pragma unroll 4
-                for (int c = 0; c < copies; ++c)
-                    __hip_atomic_store(tagged + c * 16 + lane, static_cast<uint32_t>(id_mine), __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
-        finish_weights(top_mine, id_mine, k, w_scale, ids, weights, nullptr, lane);
-        WD_STAMP(7);
     }
+    finish_weights(top_mine, id_mine, k, w_scale, ids, weights, nullptr, lane);
+    WD_STAMP(7);
+#undef WD_STAMP
+}
+
+template <int M>
+WD_DEV void topk_block_m(const float *logits, int n, int k, float w_scale, int32_t *ids, float *weights,
+                         const int32_t *__restrict__ override_ids, uint8_t *lds, int lane, int wave,
+                         unsigned long long *stamps = nullptr, uint32_t *tagged = nullptr, int copies = 0) {
+#define WD_STAMP(i) do { if (stamps && wave == 0 && lane == 0) stamps[i] = wall_clock64(); } while (0)
+    const TopkLds<M> s(lds);
+    WD_STAMP(0);
+    int id_given = 0;
+    if (override_ids && wave == 0 && lane < k) id_given = override_ids[lane];
+    float l[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+        const int id = m * 512 + wave * 64 + lane;
+        l[m] = (id < n) ? __hip_atomic_load(logits + id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : -INFINITY;
+    }
+    topk_block_step1<M>(l, s, lane, wave);
+    __syncthreads();
+    WD_STAMP(1);
+    topk_block_step2<M>(l, n, k, s, lane, wave);
+    __syncthreads();
+    WD_STAMP(2);
+    if (wave == 0)
+        topk_block_step3<M>(n, k, w_scale, ids, weights, override_ids != nullptr, id_given, s, lane, stamps, tagged, copies);
 #undef WD_STAMP
 }
 
@@ -764,8 +790,9 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
             if (a.trace && threadIdx.x == 0) a.trace[(0 * 16 + 8) * 8 + 0] = wall_clock64();
             // results land behind the selection's own scratch
-            int32_t *lds_ids = reinterpret_cast<int32_t *>(s_union + 4 * (1024 + 600));
-            float *lds_w = reinterpret_cast<float *>(s_union + 4 * (1024 + 600) + 64);
+            static_assert(sizeof(s_union) >= kTopkLdsBytes2 + 128, "selection scratch, ids and weights must fit the shared area");
+            int32_t *lds_ids = reinterpret_cast<int32_t *>(s_union + kTopkLdsBytes2);
+            float *lds_w = reinterpret_cast<float *>(s_union + kTopkLdsBytes2 + 64);
             // the selection itself publishes the replicas that the routed workgroups wait for, ahead of the weights
             topk_block(a.logits, a.E, a.k, a.w_scale, lds_ids, lds_w, a.ids_override, s_union, lane, wave,
                        a.trace ? a.trace + (0 * 16 + 9) * 8 : nullptr, a.ids_tagged, kTagCopies);

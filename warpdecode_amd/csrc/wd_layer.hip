@@ -2,8 +2,12 @@
 // every stage a stand-alone operator of wd_ops.hip resolved against the device-side ids).
 #include "wd_common.h"
 #include "wd_tokens.cuh"
+#include "wd_resident.cuh"
 
+#include <cstdlib>
+#include <cstring>
 #include <new>
+#include <vector>
 
 using namespace wd;
 
@@ -37,6 +41,13 @@ struct wd_moe_scratch {
     unsigned *status = nullptr;           // [0] != 0: a bounded wait inside a dispatch ran out
     unsigned spin_limit = kSpinLimit;
     int compute_units = 256;              // of the device the scratch lives on
+    // the resident stack kernel (wd_resident.cuh): hand-off buffers, device copy of the layer descriptors
+    uint8_t *res_block = nullptr;
+    ResidentLayer *res_layers = nullptr;          // device [kResMaxLayers], then one ResidentViews
+    std::vector<ResidentLayer> res_shadow;        // what res_layers holds
+    int res_fits = -1;                            // -1 not asked yet; 1: the device holds the whole grid at once
+    int trace_layer = 0;
+    bool trace_all = false;                       // the trace buffer has the resident kernel's size
 };
 
 namespace {
@@ -124,6 +135,8 @@ int wd_moe_scratch_destroy(wd_moe_scratch *s) {
     (void)hipFree(s->gup);
     (void)hipFree(s->dp);
     (void)hipFree(s->trace);
+    (void)hipFree(s->res_block);
+    (void)hipFree(s->res_layers);
     (void)hipHostFree(s->h_ids);
     delete s;
     return WD_OK;
@@ -141,6 +154,7 @@ int wd_moe_scratch_set_wait_limit(wd_moe_scratch *s, unsigned polls) {
     // a fresh start: clear the status word and make the published ids invalid again
     WD_HIP(hipMemset(s->status, 0, sizeof(unsigned)));
     WD_HIP(hipMemset(s->tagged, 0xff, sizeof(uint32_t) * kTagRecords * kTagCopies * 16));
+    if (s->res_block) WD_HIP(hipMemset(s->res_block, 0xff, kHandFin));
     return WD_OK;
 }
 float *wd_moe_scratch_logits(wd_moe_scratch *s) { return s->logits; }
@@ -171,6 +185,24 @@ unsigned long long *wd_moe_scratch_trace(wd_moe_scratch *s, int wg) {
         (void)hipMemset(s->trace + (d * 16 + 15) * 8 + 1, 0, sizeof(big));
     }
     s->trace_wg = wg;
+    return s->trace;
+}
+
+// Profiling aid of the resident stack kernel: 12 x 16 time stamps (100 MHz counter; per wave, per marked point) of
+// workgroup `wg` in layer `layer`; returns the device address of the buffer (shared with wd_moe_scratch_trace).
+unsigned long long *wd_moe_scratch_trace_resident(wd_moe_scratch *s, int wg, int layer) {
+    if (!s) return nullptr;
+    const size_t bytes = sizeof(unsigned long long) * kResWgs * 4 * 16;  // also covers the per-layer kernels' 3 x 16 x 8
+    if (s->trace && !s->trace_all) {
+        (void)hipFree(s->trace);
+        s->trace = nullptr;
+    }
+    if (!s->trace) {
+        if (hipMalloc(reinterpret_cast<void **>(&s->trace), bytes) != hipSuccess) return nullptr;
+        s->trace_all = true;
+    }
+    (void)hipMemset(s->trace, 0, bytes);
+    s->trace_wg = wg, s->trace_layer = layer;
     return s->trace;
 }
 
@@ -609,6 +641,100 @@ extern "C" int wd_shared_expert_f32(const wd_moe_layer *L, const float *d_x, wd_
     return grouped_gemv(WD_TYPE_Q8_0, d, 1, H, F, s, aq, ad, 0, s->down_f32, nullptr, st);
 }
 
+namespace {
+
+// The hand-off buffers and the descriptor array of the resident stack kernel, allocated on first use.
+int resident_prepare(wd_moe_scratch *s) {
+    if (s->res_block) return WD_OK;
+    uint8_t *b = nullptr;
+    WD_HIP(hipMalloc(reinterpret_cast<void **>(&b), kHandBytes));
+    const size_t desc_bytes = sizeof(ResidentLayer) * kResMaxLayers + sizeof(ResidentViews);
+    if (hipMalloc(reinterpret_cast<void **>(&s->res_layers), desc_bytes) != hipSuccess) {
+        (void)hipFree(b);
+        return fail(WD_ERR_HIP, "hipMalloc of the resident stack's layer descriptors failed");
+    }
+    (void)hipMemset(b, 0xff, kHandFin);                      // every hand-off word "not yet written"
+    (void)hipMemset(b + kHandFin, 0, kHandBytes - kHandFin);  // launch numbers
+    const ResidentViews v{s->logits, s->weights, s->accum, s->down_f32, s->shared_gate, s->ids};
+    (void)hipMemcpy(s->res_layers + kResMaxLayers, &v, sizeof(v), hipMemcpyHostToDevice);
+    s->res_block = b;
+    return WD_OK;
+}
+
+bool aligned16(const void *p, size_t stride) { return reinterpret_cast<uintptr_t>(p) % 16 == 0 && stride % 16 == 0; }
+
+// Whether the stack can run as one resident launch (see wd_resident.cuh for the geometry it is written for).
+bool resident_shape(const wd_moe_layer *layers, int n_layers, const wd_moe_scratch *s, unsigned flags) {
+    if (flags != 0 || n_layers > kResMaxLayers || s->gup != nullptr) return false;
+    const wd_moe_layer &f = layers[0];
+    if (f.hidden != kResH || f.expert_ffn != kResF || f.n_experts > 512 || f.n_experts % 8 != 0 || f.top_k > kResMaxK) return false;
+    if (!consumes_q8k(f.gate_type)) return false;
+    for (int l = 0; l < n_layers; ++l) {
+        const wd_moe_layer &L = layers[l];
+        if (L.hidden != f.hidden || L.expert_ffn != f.expert_ffn || L.n_experts != f.n_experts || L.top_k != f.top_k) return false;
+        if (L.gate_type != f.gate_type || L.up_type != f.gate_type || L.down_type != WD_TYPE_Q8_0 || L.slot_of_expert) return false;
+        if (L.gate_stride != f.gate_stride || L.up_stride != f.up_stride || L.down_stride != f.down_stride) return false;
+        if ((L.shared_gate_inp != nullptr) != (f.shared_gate_inp != nullptr)) return false;
+        if (!aligned16(L.gate, L.gate_stride) || !aligned16(L.up, L.up_stride) || !aligned16(L.down, L.down_stride)) return false;
+        if (reinterpret_cast<uintptr_t>(L.router) % 16 != 0) return false;
+        if (L.shared_gate_inp && (!aligned16(L.shared_down, 0) || reinterpret_cast<uintptr_t>(L.shared_gate_inp) % 4 != 0)) return false;
+    }
+    return true;
+}
+
+template <int TYPE>
+int resident_launch(const ResidentArgs &a, wd_moe_scratch *s, hipStream_t st) {
+    if (s->res_fits < 0) {
+        int per_cu = 0;
+        const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_stack_resident<TYPE>, kResThreads, kResLdsBytes);
+        s->res_fits = (e == hipSuccess && per_cu * s->compute_units >= kResWgs) ? 1 : 0;
+    }
+    if (!s->res_fits) return -1;  // the workgroups would wait for each other without all being on the device
+    k_stack_resident<TYPE><<<dim3(kResWgs), dim3(kResThreads), kResLdsBytes, st>>>(a);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+// Returns -1 when the stack has to take the per-layer dispatches instead.
+int stack_resident(const wd_moe_layer *layers, int n_layers, float *d_x, float *d_layer_out, wd_moe_scratch *s,
+                   const int32_t *d_ids_trace, float residual_scale, hipStream_t st) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) != hipSuccess) return -1;
+    const bool capturing = cap != hipStreamCaptureStatusNone;
+    if (!s->res_block) {
+        if (capturing) return -1;  // nothing may be allocated while a graph is recorded
+        if (const int rc = resident_prepare(s)) return rc;
+    }
+    std::vector<ResidentLayer> want(n_layers);
+    for (int l = 0; l < n_layers; ++l) {
+        const wd_moe_layer &L = layers[l];
+        ResidentLayer &d = want[l];
+        std::memset(&d, 0, sizeof(d));
+        d.router = L.router, d.sh_inp = L.shared_gate_inp;
+        d.sh_gate = L.shared_gate, d.sh_up = L.shared_up, d.sh_down = L.shared_down;
+        d.gate = L.gate, d.up = L.up, d.down = L.down;
+        d.w_scale = L.expert_scale;
+    }
+    if (s->res_shadow.size() != want.size() || std::memcmp(s->res_shadow.data(), want.data(), sizeof(ResidentLayer) * want.size()) != 0) {
+        if (capturing) return -1;
+        WD_HIP(hipStreamSynchronize(st));  // an earlier launch on this stream may still read the old descriptors
+        WD_HIP(hipMemcpy(s->res_layers, want.data(), sizeof(ResidentLayer) * want.size(), hipMemcpyHostToDevice));
+        s->res_shadow = want;
+    }
+    ResidentArgs a{};
+    a.layers = s->res_layers, a.n_layers = n_layers, a.E = layers[0].n_experts, a.k = layers[0].top_k;
+    a.shared = layers[0].shared_gate_inp != nullptr;
+    a.gate_stride = layers[0].gate_stride, a.up_stride = layers[0].up_stride, a.down_stride = layers[0].down_stride;
+    a.x = d_x, a.out = d_layer_out, a.residual_scale = residual_scale, a.ids_trace = d_ids_trace;
+    a.views = reinterpret_cast<const ResidentViews *>(s->res_layers + kResMaxLayers);
+    a.hand = s->res_block, a.status = s->status, a.spin_limit = s->spin_limit;
+    a.trace = s->trace, a.trace_wg = s->trace_wg, a.trace_layer = s->trace_layer;
+    if (const char *dbg = getenv("WD_RES_DEBUG")) a.debug = atoi(dbg);
+    return layers[0].gate_type == WD_TYPE_IQ3_S ? resident_launch<21>(a, s, st) : resident_launch<22>(a, s, st);
+}
+
+}  // namespace
+
 extern "C" int wd_moe_stack_f32(const wd_moe_layer *layers, int n_layers, float *d_x, float *d_layer_out,
                                 wd_moe_scratch *s, const int32_t *d_ids_trace, float residual_scale, unsigned flags,
                                 void *stream) {
@@ -617,6 +743,11 @@ extern "C" int wd_moe_stack_f32(const wd_moe_layer *layers, int n_layers, float 
     for (int l = 0; l < n_layers; ++l) {
         if (const int rc = check_layer(&layers[l], s)) return rc;
     }
+    if (resident_shape(layers, n_layers, s, flags)) {
+        const int rc = stack_resident(layers, n_layers, d_x, d_layer_out, s, d_ids_trace, residual_scale, as_stream(stream));
+        if (rc >= 0) return rc;
+    }
+    flags &= ~WD_MOE_PER_LAYER;
     const unsigned only = flags & (WD_MOE_ONLY_A | WD_MOE_ONLY_B | WD_MOE_ONLY_C);
     for (int l = 0; l < n_layers; ++l) {
         const int32_t *trace = d_ids_trace ? d_ids_trace + static_cast<size_t>(l) * layers[l].top_k : nullptr;

@@ -306,22 +306,33 @@ WD_DEV IqFields iq_fields_lds(const uint8_t *blk, int ib, int sb) {
 
 // iq_rows_q8k<TYPE, NR, false> for nb == 8 and 16-byte aligned rows.  stage: NR * kIqStageBytes bytes of LDS owned by
 // the wave, 16-byte aligned.
+// The fetch and the rest apart, for callers that put other requests in flight between the two.
 template <int TYPE, int NR>
-WD_DEV void iq_rows8_coal(const uint8_t *const (&rows)[NR], const IqTables &t, const int8_t *act_qs, const float *act_d,
-                          int lane, float (&y)[NR], uint8_t *stage) {
-    constexpr int kBlk = (TYPE == 21) ? 110 : 82;
-    constexpr int kWords = 8 * kBlk / 16;
+struct IqRows8Raw {
+    static constexpr int kBlk = (TYPE == 21) ? 110 : 82, kWords = 8 * kBlk / 16;
+    uint4 u[NR];
+};
+template <int TYPE, int NR>
+WD_DEV IqRows8Raw<TYPE, NR> iq_rows8_coal_request(const uint8_t *const (&rows)[NR], int lane) {
+    IqRows8Raw<TYPE, NR> raw;
+#pragma unroll
+    for (int i = 0; i < NR; ++i) raw.u[i] = gld_u128_aligned(rows[i] + 16 * min(lane, IqRows8Raw<TYPE, NR>::kWords - 1));
+    return raw;
+}
+template <int TYPE, int NR>
+WD_DEV void iq_rows8_coal_park(const IqRows8Raw<TYPE, NR> &raw, int lane, uint8_t *stage) {
+#pragma unroll
+    for (int i = 0; i < NR; ++i)
+        if (lane < IqRows8Raw<TYPE, NR>::kWords) reinterpret_cast<uint4 *>(stage + i * kIqStageBytes)[lane] = raw.u[i];
+    wave_lds_fence();
+}
+// The dot products of the NR rows parked in `stage`.
+template <int TYPE, int NR>
+WD_DEV void iq_rows8_coal_dots(const IqTables &t, const int8_t *act_qs, const float *act_d, int lane, float (&y)[NR],
+                               const uint8_t *stage) {
+    constexpr int kBlk = IqRows8Raw<TYPE, NR>::kBlk;
     const int ib = lane >> 3, sb = lane & 7;
     const bool first = sb == 0;
-    {
-        uint4 raw[NR];
-#pragma unroll
-        for (int i = 0; i < NR; ++i) raw[i] = gld_u128_aligned(rows[i] + 16 * min(lane, kWords - 1));
-#pragma unroll
-        for (int i = 0; i < NR; ++i)
-            if (lane < kWords) reinterpret_cast<uint4 *>(stage + i * kIqStageBytes)[lane] = raw[i];
-    }
-    wave_lds_fence();
     const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32);
     const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32 + 16);
     const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
@@ -343,6 +354,18 @@ WD_DEV void iq_rows8_coal(const uint8_t *const (&rows)[NR], const IqTables &t, c
         const float r = close_lanes8_strided(v);
         y[i] = (TYPE == 22) ? 0.125f * r : r;
     }
+}
+template <int TYPE, int NR>
+WD_DEV void iq_rows8_coal_finish(const IqRows8Raw<TYPE, NR> &raw, const IqTables &t, const int8_t *act_qs, const float *act_d,
+                                 int lane, float (&y)[NR], uint8_t *stage) {
+    iq_rows8_coal_park<TYPE, NR>(raw, lane, stage);
+    iq_rows8_coal_dots<TYPE, NR>(t, act_qs, act_d, lane, y, stage);
+}
+template <int TYPE, int NR>
+WD_DEV void iq_rows8_coal(const uint8_t *const (&rows)[NR], const IqTables &t, const int8_t *act_qs, const float *act_d,
+                          int lane, float (&y)[NR], uint8_t *stage) {
+    const IqRows8Raw<TYPE, NR> raw = iq_rows8_coal_request<TYPE, NR>(rows, lane);
+    iq_rows8_coal_finish<TYPE, NR>(raw, t, act_qs, act_d, lane, y, stage);
 }
 
 constexpr int kIqStage10Bytes = 1120;  // per row of ten super-blocks: the 70 words that cover 12 + 1100 bytes
@@ -894,10 +917,54 @@ struct Q8RowTile {
 };
 
 // rows[i]: the row of matrix i.  y[i] valid in lane 0 (every aligned group of 8 lanes runs the same chain).
+// One pass of the row chains: block `bi` of every matrix (wb[i], loaded by the caller; lanes with on == false
+// contribute nothing) against the activation; acc[i] is chunk lane (lane & 7)'s accumulator.
+template <int NM>
+WD_DEV void q8_row_wave_pass(const Q8Block (&wb)[NM], bool on, int bi, const int8_t *act_qs, const uint16_t *act_d,
+                             Q8RowTile &tile, int lane, float (&acc)[NM]) {
+    const int c = lane & 7;
+    uint32_t a[8];
+    float dx = 0.0f;
+    if (on) {
+        const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + bi * 32);
+        const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + bi * 32 + 16);
+        a[0] = a0.x, a[1] = a0.y, a[2] = a0.z, a[3] = a0.w, a[4] = a1.x, a[5] = a1.y, a[6] = a1.z, a[7] = a1.w;
+        dx = h2f(act_d[bi]);
+    }
+#pragma unroll
+    for (int i = 0; i < NM; ++i) {
+        int p[8];
+        float ds = 0.0f;
+        if (on) {
+            q8_chunks<0>(wb[i], a, p);
+            ds = h2f(wb[i].d) * dx;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) p[j] = 0;
+        }
+        wave_lds_fence();  // earlier reads of the tile are done before it is overwritten
+#pragma unroll
+        for (int j = 0; j < 8; ++j) tile.pf[j][lane] = static_cast<float>(p[j]);
+        tile.ds[lane] = ds;
+        wave_lds_fence();
+        // blocks past the end of the row contribute fma(0, 0, acc) == acc
+        // (partial unroll: a full one makes the compiler hold all 128 tile values in registers at once)
+#pragma unroll 4
+        for (int s4 = 0; s4 < 16; ++s4) {
+            const float4 pv = *reinterpret_cast<const float4 *>(&tile.pf[c][4 * s4]);
+            const float4 dv = *reinterpret_cast<const float4 *>(&tile.ds[4 * s4]);
+            acc[i] = __builtin_fmaf(dv.x, pv.x, acc[i]);
+            acc[i] = __builtin_fmaf(dv.y, pv.y, acc[i]);
+            acc[i] = __builtin_fmaf(dv.z, pv.z, acc[i]);
+            acc[i] = __builtin_fmaf(dv.w, pv.w, acc[i]);
+        }
+    }
+}
+
+// rows[i]: the row of matrix i.  y[i] valid in lane 0 (every aligned group of 8 lanes runs the same chain).
 template <int NM, typename Pre = NoPre>
 WD_DEV void q8_row_wave(const uint8_t *const (&rows)[NM], int nb, const int8_t *act_qs, const uint16_t *act_d,
                         Q8RowTile &tile, int lane, float (&y)[NM], Pre pre = Pre()) {
-    const int c = lane & 7;
     float acc[NM];
 #pragma unroll
     for (int i = 0; i < NM; ++i) acc[i] = 0.0f;
@@ -910,42 +977,7 @@ WD_DEV void q8_row_wave(const uint8_t *const (&rows)[NM], int nb, const int8_t *
             for (int i = 0; i < NM; ++i) wb[i] = q8_load<0>(rows[i] + static_cast<size_t>(bi) * 34);
         }
         if (base == 0) pre();
-        uint32_t a[8];
-        float dx = 0.0f;
-        if (on) {
-            const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + bi * 32);
-            const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + bi * 32 + 16);
-            a[0] = a0.x, a[1] = a0.y, a[2] = a0.z, a[3] = a0.w, a[4] = a1.x, a[5] = a1.y, a[6] = a1.z, a[7] = a1.w;
-            dx = h2f(act_d[bi]);
-        }
-#pragma unroll
-        for (int i = 0; i < NM; ++i) {
-            int p[8];
-            float ds = 0.0f;
-            if (on) {
-                q8_chunks<0>(wb[i], a, p);
-                ds = h2f(wb[i].d) * dx;
-            } else {
-#pragma unroll
-                for (int j = 0; j < 8; ++j) p[j] = 0;
-            }
-            wave_lds_fence();  // earlier reads of the tile are done before it is overwritten
-#pragma unroll
-            for (int j = 0; j < 8; ++j) tile.pf[j][lane] = static_cast<float>(p[j]);
-            tile.ds[lane] = ds;
-            wave_lds_fence();
-            // blocks past the end of the row contribute fma(0, 0, acc) == acc
-            // (partial unroll: a full one makes the compiler hold all 128 tile values in registers at once)
-#pragma unroll 4
-            for (int s4 = 0; s4 < 16; ++s4) {
-                const float4 pv = *reinterpret_cast<const float4 *>(&tile.pf[c][4 * s4]);
-                const float4 dv = *reinterpret_cast<const float4 *>(&tile.ds[4 * s4]);
-                acc[i] = __builtin_fmaf(dv.x, pv.x, acc[i]);
-                acc[i] = __builtin_fmaf(dv.y, pv.y, acc[i]);
-                acc[i] = __builtin_fmaf(dv.z, pv.z, acc[i]);
-                acc[i] = __builtin_fmaf(dv.w, pv.w, acc[i]);
-            }
-        }
+        q8_row_wave_pass<NM>(wb, on, bi, act_qs, act_d, tile, lane, acc);
     }
 #pragma unroll
     for (int i = 0; i < NM; ++i) y[i] = close_lanes8(acc[i]);

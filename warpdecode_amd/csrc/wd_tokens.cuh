@@ -62,8 +62,9 @@ __global__ __launch_bounds__(512, 6) void k_tokens_a(TokenArgs ta) {
         if (!s_last) return;
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         if (!a.preselected) {
-            int32_t *lds_ids = reinterpret_cast<int32_t *>(s_work + 4 * (1024 + 600));  // behind the selection's own scratch
-            float *lds_w = reinterpret_cast<float *>(s_work + 4 * (1024 + 600) + 64);
+            static_assert(sizeof(s_work) >= kTopkLdsBytes2 + 128, "selection scratch, ids and weights must fit the shared area");
+            int32_t *lds_ids = reinterpret_cast<int32_t *>(s_work + kTopkLdsBytes2);  // behind the selection's own scratch
+            float *lds_w = reinterpret_cast<float *>(s_work + kTopkLdsBytes2 + 64);
             topk_block(s.logits, a.E, a.k, a.w_scale, lds_ids, lds_w, nullptr, s_work, lane, wave);
             if (wave == 0) {
                 wave_lds_fence();
