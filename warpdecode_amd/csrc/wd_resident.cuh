@@ -41,6 +41,7 @@ constexpr int kResWgs = 512, kResWaves = 12, kResThreads = kResWaves * 64;
 constexpr int kResH = 2048, kResF = 512, kResMaxK = 10, kResSharedSlot = 10, kResActSlots = 11;
 constexpr uint32_t kResEmpty = 0xffffffffu;
 constexpr int kResIdCopies = 16;   // replicas of the published ids (pollers spread over lines)
+constexpr int kResXtRow = 68;      // floats per row of the transposed input in LDS (64 + bank spread)
 constexpr int kResGateSlot = 15;   // word of the weights record that holds the shared expert's sigmoid gate
 
 struct ResidentLayer {
@@ -64,13 +65,13 @@ constexpr unsigned kHandRec = 0;          // [layers][512] records of 128 bytes,
 constexpr unsigned kRecBytes = 128;       //   word 0 router logit, word 1 the shared expert's gate logit (workgroup 1 only),
 constexpr unsigned kRecAct = 16;          //   words 4..14 SwiGLU activations of slots 0..10 (word 15 zero),
 constexpr unsigned kRecX = 64;            //   words 16..19 the workgroup's four values of the next layer's input
-// Gathered copies: hub workgroup g (g < kResHubs) collects the records of a layer and lays the values out contiguously for
-// the workgroups r with r % kResHubs == g, which then fetch them with a few coalesced requests instead of one per record.
+// Gathered copies of the layer inputs: hub workgroup g (g < kResHubs) collects the four values of every record and lays the
+// vector out contiguously for the workgroups r with r % kResHubs == g, which fetch it with coalesced requests instead of
+// one per record.  (The same for the activations - as floats, or quantised to Q8_0 by the hubs - measured slower than
+// every workgroup reading the 512 records itself: 5 to 7 us against 4 to 5.)
 constexpr int kResHubs = 8;
 constexpr unsigned kHandXc = kHandRec + kRecBytes * kResMaxLayers * kResWgs;          // f32 [layers][hubs][2048] layer inputs
-constexpr unsigned kHandAc = kHandXc + 4u * kResMaxLayers * kResHubs * kResH;         // f32 [layers][hubs][11][512] activations
-constexpr unsigned kAcWords16 = kResActSlots * 512 / 4;                               // 16-byte words of one such copy
-constexpr unsigned kHandIdh = kHandAc + 16u * kAcWords16 * kResMaxLayers * kResHubs;  // u32 [layers][copies][16] selected ids
+constexpr unsigned kHandIdh = kHandXc + 4u * kResMaxLayers * kResHubs * kResH;        // u32 [layers][copies][16] selected ids
 constexpr unsigned kHandWh = kHandIdh + 4u * kResMaxLayers * kResIdCopies * 16;  // u32 [layers][16] router weights, [15] the shared gate
 constexpr unsigned kHandFin = kHandWh + 4u * kResMaxLayers * 16;              // u32 [512] number of the last launch each workgroup finished
 constexpr unsigned kHandEpoch = kHandFin + 4u * kResWgs;                      // u32 launches finished
@@ -78,7 +79,6 @@ constexpr unsigned kHandBytes = kHandEpoch + 256u;
 static_assert(kHandIdh % 128 == 0 && kHandWh % 16 == 0 && kHandFin % 16 == 0, "hand-off block alignment");
 WD_DEV unsigned rec_off(int l, int wg) { return kHandRec + static_cast<unsigned>(l * kResWgs + wg) * kRecBytes; }
 WD_DEV unsigned xc_off(int l, int hub) { return kHandXc + static_cast<unsigned>(l * kResHubs + hub) * (4u * kResH); }
-WD_DEV unsigned ac_off(int l, int hub) { return kHandAc + static_cast<unsigned>(l * kResHubs + hub) * (16u * kAcWords16); }
 
 struct ResidentArgs {
     const ResidentLayer *layers;  // device array [n_layers]
@@ -190,20 +190,22 @@ WD_DEV void res_router_fetch(const float *__restrict__ row, float (&wv)[32], int
 #pragma unroll
     for (int u = 0; u < 32; ++u) wv[u] = p[32 * u];
 }
-// The row's dot product with xs (LDS, f32 [2048]); valid in lane 32.
-WD_DEV float res_router_dot(const float (&wv)[32], const float *xs, int lane) {
+// The row's dot product with the input (LDS, transposed: xt[t][v] = x[32 v + t], rows of kResXtRow floats); valid in lane 32.
+WD_DEV float res_router_dot(const float (&wv)[32], const float *xt, int lane) {
     const int t = lane & 31;
     const bool upper = lane >= 32;
-    const float *xp = xs + (upper ? 1024 : 0) + t;
+    const float4 *xp = reinterpret_cast<const float4 *>(xt + t * kResXtRow + (upper ? 32 : 0));
+    float4 xv[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) xv[q] = xp[q];
     auto run_half = [&](float start) {
         float v = start;
 #pragma unroll
-        for (int ub = 0; ub < 32; ub += 8) {
-            float xv[8];
-#pragma unroll
-            for (int q = 0; q < 8; ++q) xv[q] = xp[32 * (ub + q)];
-#pragma unroll
-            for (int q = 0; q < 8; ++q) v = __builtin_fmaf(wv[ub + q], xv[q], v);
+        for (int q = 0; q < 8; ++q) {
+            v = __builtin_fmaf(wv[4 * q + 0], xv[q].x, v);
+            v = __builtin_fmaf(wv[4 * q + 1], xv[q].y, v);
+            v = __builtin_fmaf(wv[4 * q + 2], xv[q].z, v);
+            v = __builtin_fmaf(wv[4 * q + 3], xv[q].w, v);
         }
         return v;
     };
@@ -225,8 +227,9 @@ WD_DEV float res_router_dot(const float (&wv)[32], const float *xs, int lane) {
 }
 
 // ---- LDS layout -----------------------------------------------------------------------------------------------
-constexpr int kResLdsXs = 0;                                  // f32 [2048] layer input
-constexpr int kResLdsXq = kResLdsXs + 4 * kResH;              // int8 [2048] its Q8_K quants
+constexpr int kResLdsXs = 0;                                  // f32 [32][68] layer input, xt[t][v] = x[32 v + t]: the 64 values that
+                                                              //   accumulator t of a router row meets are contiguous
+constexpr int kResLdsXq = kResLdsXs + 4 * 32 * kResXtRow;     // int8 [2048] its Q8_K quants
 constexpr int kResLdsXd = kResLdsXq + kResH;                  // f32 [8] Q8_K scales
 constexpr int kResLdsX0q = kResLdsXd + 32;                    // int8 [2048] its Q8_0 quants
 constexpr int kResLdsX0d = kResLdsX0q + kResH;                // f16 [64] Q8_0 scales
@@ -240,7 +243,7 @@ constexpr int kResLdsRoles = kResLdsSel + kTopkLdsBytes1 + 128;       // int [12
 constexpr int kResLdsActv = kResLdsRoles + 64;                        // f32 [12] this workgroup's activations (word 11 zero)
 constexpr int kResLdsBytes = kResLdsActv + 64;
 constexpr int kResLdsLand = kResLdsWave;  // f32 [11][512] all activations of the layer, while no slot area is in use
-static_assert(kResLdsTables % 16 == 0 && kResLdsWave % 16 == 0 && kResWaveBytes % 16 == 0 && kResLdsSel % 16 == 0, "LDS alignment");
+static_assert(kResLdsXq % 16 == 0 && kResLdsTables % 16 == 0 && kResLdsWave % 16 == 0 && kResWaveBytes % 16 == 0 && kResLdsSel % 16 == 0, "LDS alignment");
 static_assert(sizeof(Q8RowTile) <= sizeof(Q8TileNB<16>) && 2 * kIqStageBytes <= kResTileBytes, "a slot's area serves every stage");
 static_assert(kResLdsBytes <= 65536, "LDS of the resident stack kernel");
 static_assert(4 * kResActSlots * 512 <= kResActSlots * kResWaveBytes, "the activations land in the slot areas");
@@ -262,7 +265,8 @@ struct ResCtx {
     uint8_t *lds;
     int r, lane, wave, slot;
     __amdgpu_buffer_rsrc_t hb;  // the hand-off block
-    WD_DEV float *xs() const { return reinterpret_cast<float *>(lds + kResLdsXs); }
+    WD_DEV float *xt() const { return reinterpret_cast<float *>(lds + kResLdsXs); }
+    WD_DEV float x_at(int e) const { return xt()[(e & 31) * kResXtRow + (e >> 5)]; }
     WD_DEV int8_t *xq() const { return reinterpret_cast<int8_t *>(lds + kResLdsXq); }
     WD_DEV float *xd() const { return reinterpret_cast<float *>(lds + kResLdsXd); }
     WD_DEV int8_t *x0q() const { return reinterpret_cast<int8_t *>(lds + kResLdsX0q); }
@@ -308,8 +312,7 @@ WD_DEV void res_exchange(const ResidentArgs &a, const ResCtx &c, int l, bool has
         const float4 p = reinterpret_cast<const float4 *>(c.actv())[lane];
         hand_store16(c.hb, rec_off(l, c.r) + kRecAct + 16u * lane, make_uint4(f_bits(p.x), f_bits(p.y), f_bits(p.z), f_bits(p.w)));
     }
-    const int hub = c.r & (kResHubs - 1);
-    if (wave < 8 && c.r < kResHubs) {  // hub: one request per record; the values go to LDS and, laid out by slot, to the copy
+    if (wave < 8) {  // every workgroup reads the records themselves, one per lane
         const int i = wave * 64 + lane;
         const unsigned base = rec_off(l, i) + kRecAct;
         const unsigned off[3] = {base, base + 16u, base + 32u};
@@ -317,23 +320,8 @@ WD_DEV void res_exchange(const ResidentArgs &a, const ResCtx &c, int l, bool has
         hand_wait16<3>(a, c.hb, off, true, v, dead);
         const uint32_t w[11] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w, v[2].x, v[2].y, v[2].z};
         float *land = c.land() + i;
-        const unsigned dst = ac_off(l, hub) + 4u * i;
 #pragma unroll
-        for (int m = 0; m < kResActSlots; ++m) {
-            land[m * 512] = bits_f(w[m]);
-            hand_store4(c.hb, dst + 2048u * m, w[m]);
-        }
-    } else if (wave < 8) {             // the others copy the hub's layout, 16 bytes per lane and turn
-        const int i = wave * 64 + lane;
-        const unsigned base = ac_off(l, hub) + 16u * i;
-        const unsigned off[3] = {base, base + 16u * 512, base + 16u * 1024};
-        const bool third = i + 1024 < static_cast<int>(kAcWords16);  // (the third turn covers only part of the lanes)
-        const bool on[3] = {true, true, third};
-        uint4 v[3];
-        hand_wait16<3>(a, c.hb, off, on, v, dead);
-        uint4 *land = reinterpret_cast<uint4 *>(c.land()) + i;
-        land[0] = v[0], land[512] = v[1];
-        if (third) land[1024] = v[2];
+        for (int m = 0; m < kResActSlots; ++m) land[m * 512] = bits_f(w[m]);
     }
     __syncthreads();  // B3: every activation of the layer is in LDS
     res_mark(a, c, l, 6);
@@ -388,7 +376,10 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                 xv = make_float4(bits_f(v[0].x), bits_f(v[0].y), bits_f(v[0].z), bits_f(v[0].w));
             }
             res_mark(a, c, l, 1);
-            reinterpret_cast<float4 *>(c.xs())[i] = xv;
+            {   // values 4 i .. 4 i + 3 are accumulators 4 (i % 8) .. + 3 at step i / 8
+                float *dst = c.xt() + (4 * (i & 7)) * kResXtRow + (i >> 3);
+                dst[0] = xv.x, dst[kResXtRow] = xv.y, dst[2 * kResXtRow] = xv.z, dst[3 * kResXtRow] = xv.w;
+            }
             wave_quantize_q8_k_regs(xv, c.xq() + 256 * wave, c.xd() + wave, lane);
             if (shared) {  // Q8_0: a block is eight lanes
                 float amax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(xv.x), __builtin_fabsf(xv.y)),
@@ -401,14 +392,14 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         }
         __syncthreads();  // B1: x and its quantised forms are in LDS
         res_mark(a, c, l, 2);
-        const float res_pre = c.xs()[4 * r + (lane & 3)];  // (rung 0 adds the layer's output to these)
+        const float res_pre = c.x_at(4 * r + (lane & 3));  // (rung 0 adds the layer's output to these)
         // this layer's routed tensors (the wave has nothing else to do until the ids appear)
         const uint8_t *const gate_base = res_field(&L->gate), *const up_base = res_field(&L->up), *const down_base = res_field(&L->down);
 
         if (gate_row) {  // (needed by the combine only: its weights are requested now)
             float gw[32];
             res_router_fetch(res_field(&L->sh_inp), gw, lane);
-            const float s = res_router_dot(gw, c.xs(), lane);
+            const float s = res_router_dot(gw, c.xt(), lane);
             if (lane == 32) hand_store4(c.hb, rec_off(l, 1) + 4u, f_bits(s));
         }
 
@@ -572,7 +563,7 @@ WD_DEV void res_router_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         __syncthreads();  // B1
         res_mark(a, c, l, 2);
         if (on) {
-            const float s = res_router_dot(wv, c.xs(), lane);
+            const float s = res_router_dot(wv, c.xt(), lane);
             if (lane == 32) hand_store4(c.hb, rec_off(l, r), f_bits(s));
             res_mark(a, c, l, 3);
             if (!last) res_router_fetch(res_field(&a.layers[l + 1].router) + static_cast<size_t>(r) * kResH, wv, lane);
@@ -667,9 +658,8 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 
     for (int i = threadIdx.x; i < n * 8; i += kResThreads)  // this workgroup's records, 16 bytes per thread
         hand_store16(hb, rec_off(i >> 3, r) + 16u * (i & 7), empty4);
     // the gathered copies of layers 0..n-1, shared out over the grid
-    const unsigned xc16 = static_cast<unsigned>(n) * kResHubs * (kResH / 4), ac16 = static_cast<unsigned>(n) * kResHubs * kAcWords16;
+    const unsigned xc16 = static_cast<unsigned>(n) * kResHubs * (kResH / 4);
     for (unsigned i = static_cast<unsigned>(r) * kResThreads + threadIdx.x; i < xc16; i += kResWgs * kResThreads) hand_store16(hb, kHandXc + 16u * i, empty4);
-    for (unsigned i = static_cast<unsigned>(r) * kResThreads + threadIdx.x; i < ac16; i += kResWgs * kResThreads) hand_store16(hb, kHandAc + 16u * i, empty4);
     if (r == 0) {
         for (int i = threadIdx.x; i < n * kResIdCopies * 4; i += kResThreads) hand_store16(hb, kHandIdh + static_cast<unsigned>(i * 16), empty4);
         for (int i = threadIdx.x; i < n * 4; i += kResThreads) hand_store16(hb, kHandWh + static_cast<unsigned>(i * 16), empty4);
