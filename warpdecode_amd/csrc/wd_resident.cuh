@@ -61,24 +61,26 @@ struct ResidentViews {
 };
 
 // Byte offsets inside the hand-off block.
-constexpr unsigned kHandRec = 0;          // [layers][512] records of 128 bytes, one per (layer, workgroup):
-constexpr unsigned kRecBytes = 128;       //   word 0 router logit, word 1 the shared expert's gate logit (workgroup 1 only),
-constexpr unsigned kRecAct = 16;          //   words 4..14 SwiGLU activations of slots 0..10 (word 15 zero),
-constexpr unsigned kRecX = 64;            //   words 16..19 the workgroup's four values of the next layer's input
-// Gathered copies of the layer inputs: hub workgroup g (g < kResHubs) collects the four values of every record and lays the
-// vector out contiguously for the workgroups r with r % kResHubs == g, which fetch it with coalesced requests instead of
-// one per record.  (The same for the activations - as floats, or quantised to Q8_0 by the hubs - measured slower than
-// every workgroup reading the 512 records itself: 5 to 7 us against 4 to 5.)
-constexpr int kResHubs = 8;
-constexpr unsigned kHandXc = kHandRec + kRecBytes * kResMaxLayers * kResWgs;          // f32 [layers][hubs][2048] layer inputs
-constexpr unsigned kHandIdh = kHandXc + 4u * kResMaxLayers * kResHubs * kResH;        // u32 [layers][copies][16] selected ids
+constexpr unsigned kHandRec = 0;          // [layers][512] records of 128 bytes, one per (layer, workgroup): word 0 the router
+constexpr unsigned kRecBytes = 128;       //   logit of row r, word 1 the shared expert's gate logit (workgroup 1 only)
+// What every workgroup needs from every other - four values of the next input, eleven activations - is written by its
+// producer into kResCopies copies, one per group of workgroups (r % kResCopies; on this device the workgroups of a group
+// share an L2), laid out contiguously: the consumers of a group fetch their copy with coalesced requests, and a line is
+// polled from one L2 only.
+constexpr int kResCopies = 8;
+constexpr unsigned kHandXc = kHandRec + kRecBytes * kResMaxLayers * kResWgs;           // f32 [layers][copies][2048] layer inputs
+constexpr unsigned kAcRec = 48;                                                        // bytes of a workgroup's activations: slots 0..10, a zero
+constexpr unsigned kAcBytes = kAcRec * kResWgs;                                        // 24 KB per copy
+constexpr unsigned kHandAc = kHandXc + 4u * kResMaxLayers * kResCopies * kResH;        // f32 [layers][copies][512][12] activations
+constexpr unsigned kHandIdh = kHandAc + kAcBytes * kResMaxLayers * kResCopies;         // u32 [layers][copies][16] selected ids
 constexpr unsigned kHandWh = kHandIdh + 4u * kResMaxLayers * kResIdCopies * 16;  // u32 [layers][16] router weights, [15] the shared gate
 constexpr unsigned kHandFin = kHandWh + 4u * kResMaxLayers * 16;              // u32 [512] number of the last launch each workgroup finished
 constexpr unsigned kHandEpoch = kHandFin + 4u * kResWgs;                      // u32 launches finished
 constexpr unsigned kHandBytes = kHandEpoch + 256u;
-static_assert(kHandIdh % 128 == 0 && kHandWh % 16 == 0 && kHandFin % 16 == 0, "hand-off block alignment");
+static_assert(kHandXc % 128 == 0 && kHandAc % 128 == 0 && kHandIdh % 128 == 0 && kHandWh % 16 == 0 && kHandFin % 16 == 0, "hand-off block alignment");
 WD_DEV unsigned rec_off(int l, int wg) { return kHandRec + static_cast<unsigned>(l * kResWgs + wg) * kRecBytes; }
-WD_DEV unsigned xc_off(int l, int hub) { return kHandXc + static_cast<unsigned>(l * kResHubs + hub) * (4u * kResH); }
+WD_DEV unsigned xc_off(int l, int copy) { return kHandXc + static_cast<unsigned>(l * kResCopies + copy) * (4u * kResH); }
+WD_DEV unsigned ac_off(int l, int copy) { return kHandAc + static_cast<unsigned>(l * kResCopies + copy) * kAcBytes; }
 
 struct ResidentArgs {
     const ResidentLayer *layers;  // device array [n_layers]
@@ -308,20 +310,24 @@ WD_DEV void res_exchange(const ResidentArgs &a, const ResCtx &c, int l, bool has
     const int lane = c.lane, wave = c.wave;
     if (has && lane == 0) c.actv()[c.slot] = mine;
     __syncthreads();  // B2: the workgroup's activations are in LDS, and no slot area is in use any more
-    if (wave == 0 && lane < 3) {
-        const float4 p = reinterpret_cast<const float4 *>(c.actv())[lane];
-        hand_store16(c.hb, rec_off(l, c.r) + kRecAct + 16u * lane, make_uint4(f_bits(p.x), f_bits(p.y), f_bits(p.z), f_bits(p.w)));
+    if (wave == 0 && lane < 3 * kResCopies) {  // piece lane % 3 of the workgroup's 48 bytes, to copy lane / 3
+        const int piece = lane % 3, copy = lane / 3;
+        const float4 p = reinterpret_cast<const float4 *>(c.actv())[piece];
+        hand_store16(c.hb, ac_off(l, copy) + kAcRec * c.r + 16u * piece, make_uint4(f_bits(p.x), f_bits(p.y), f_bits(p.z), f_bits(p.w)));
     }
-    if (wave < 8) {  // every workgroup reads the records themselves, one per lane
+    if (wave < 8) {  // the group's copy, three 16-byte words per lane: word w is piece w % 3 of workgroup w / 3
         const int i = wave * 64 + lane;
-        const unsigned base = rec_off(l, i) + kRecAct;
-        const unsigned off[3] = {base, base + 16u, base + 32u};
+        const unsigned base = ac_off(l, c.r & (kResCopies - 1)) + 16u * i;
+        const unsigned off[3] = {base, base + 16u * 512, base + 16u * 1024};
         uint4 v[3];
         hand_wait16<3>(a, c.hb, off, true, v, dead);
-        const uint32_t w[11] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w, v[2].x, v[2].y, v[2].z};
-        float *land = c.land() + i;
 #pragma unroll
-        for (int m = 0; m < kResActSlots; ++m) land[m * 512] = bits_f(w[m]);
+        for (int t = 0; t < 3; ++t) {
+            const int w = i + 512 * t, wg = w / 3, piece = w - 3 * wg;
+            float *land = c.land() + (4 * piece) * 512 + wg;
+            land[0] = bits_f(v[t].x), land[512] = bits_f(v[t].y), land[1024] = bits_f(v[t].z);
+            if (piece < 2) land[1536] = bits_f(v[t].w);
+        }
     }
     __syncthreads();  // B3: every activation of the layer is in LDS
     res_mark(a, c, l, 6);
@@ -367,12 +373,10 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             float4 xv;
             if (l == 0) {
                 xv = reinterpret_cast<const float4 *>(a.x)[i];
-            } else {  // hubs collect the four values of every workgroup's record and hand the whole vector on
-                const bool is_hub = r < kResHubs;
-                const unsigned off[1] = {is_hub ? rec_off(l - 1, i) + kRecX : xc_off(l, r & (kResHubs - 1)) + 16u * i};
+            } else {
+                const unsigned off[1] = {xc_off(l, r & (kResCopies - 1)) + 16u * i};
                 uint4 v[1];
                 hand_wait16<1>(a, c.hb, off, true, v, dead);
-                if (is_hub) hand_store16(c.hb, xc_off(l, r) + 16u * i, v[0]);
                 xv = make_float4(bits_f(v[0].x), bits_f(v[0].y), bits_f(v[0].z), bits_f(v[0].w));
             }
             res_mark(a, c, l, 1);
@@ -504,7 +508,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             } else {
                 const uint4 piece = make_uint4(f_bits(readlane_f(xn, 0)), f_bits(readlane_f(xn, 1)), f_bits(readlane_f(xn, 2)),
                                                f_bits(readlane_f(xn, 3)));
-                if (lane == 0) hand_store16(c.hb, rec_off(l, r) + kRecX, piece);
+                if (lane < kResCopies) hand_store16(c.hb, xc_off(l + 1, lane) + 16u * r, piece);
             }
             res_mark(a, c, l, 9);
         }
@@ -655,11 +659,11 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 
     if (__hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return;
     const int n = a.n_layers;
     const uint4 empty4 = make_uint4(kResEmpty, kResEmpty, kResEmpty, kResEmpty);
-    for (int i = threadIdx.x; i < n * 8; i += kResThreads)  // this workgroup's records, 16 bytes per thread
-        hand_store16(hb, rec_off(i >> 3, r) + 16u * (i & 7), empty4);
-    // the gathered copies of layers 0..n-1, shared out over the grid
-    const unsigned xc16 = static_cast<unsigned>(n) * kResHubs * (kResH / 4);
+    for (int l = threadIdx.x; l < n; l += kResThreads) hand_store16(hb, rec_off(l, r), empty4);  // this workgroup's records
+    // the copies of layers 0..n-1, shared out over the grid
+    const unsigned xc16 = static_cast<unsigned>(n) * kResCopies * (kResH / 4), ac16 = static_cast<unsigned>(n) * kResCopies * (kAcBytes / 16);
     for (unsigned i = static_cast<unsigned>(r) * kResThreads + threadIdx.x; i < xc16; i += kResWgs * kResThreads) hand_store16(hb, kHandXc + 16u * i, empty4);
+    for (unsigned i = static_cast<unsigned>(r) * kResThreads + threadIdx.x; i < ac16; i += kResWgs * kResThreads) hand_store16(hb, kHandAc + 16u * i, empty4);
     if (r == 0) {
         for (int i = threadIdx.x; i < n * kResIdCopies * 4; i += kResThreads) hand_store16(hb, kHandIdh + static_cast<unsigned>(i * 16), empty4);
         for (int i = threadIdx.x; i < n * 4; i += kResThreads) hand_store16(hb, kHandWh + static_cast<unsigned>(i * 16), empty4);
