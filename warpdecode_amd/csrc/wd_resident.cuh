@@ -33,8 +33,14 @@
 
 namespace wd {
 
+#ifndef WD_RES_SLEEP4
+#define WD_RES_SLEEP4 2
+#endif
+#ifndef WD_RES_XDELAY
+#define WD_RES_XDELAY 24
+#endif
 #ifndef WD_RES_SLEEP16
-#define WD_RES_SLEEP16 1
+#define WD_RES_SLEEP16 2
 #endif
 constexpr int kResMaxLayers = 64;
 constexpr int kResWgs = 512, kResWaves = 12, kResThreads = kResWaves * 64;
@@ -181,6 +187,7 @@ WD_DEV uint32_t hand_wait4(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, uns
         need = need && v == kResEmpty;
         if (__builtin_amdgcn_ballot_w64(need) == 0ull) return v;
         if (res_give_up(a, spins, dead)) return v;
+        __builtin_amdgcn_s_sleep(WD_RES_SLEEP4);
     }
 }
 
@@ -374,6 +381,9 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             if (l == 0) {
                 xv = reinterpret_cast<const float4 *>(a.x)[i];
             } else {
+                // (the other waves of the workgroup come here while rung 0 still folds the previous layer: nothing
+                // can have arrived yet)
+                if (rung != 0 && WD_RES_XDELAY) __builtin_amdgcn_s_sleep(WD_RES_XDELAY);
                 const unsigned off[1] = {xc_off(l, r & (kResCopies - 1)) + 16u * i};
                 uint4 v[1];
                 hand_wait16<1>(a, c.hb, off, true, v, dead);
@@ -425,12 +435,15 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                 topk_block_step1<1>(lv, s, lane, wave);
             }
             __syncthreads();
+            res_mark(a, c, l, 12);
             if (wave < 8) topk_block_step2<1>(lv, a.E, a.k, s, lane, wave);
             __syncthreads();
+            res_mark(a, c, l, 13);
             if (wave == 0) {
                 const float w_scale = *const_cast<const volatile float *>(&L->w_scale);
                 topk_block_step3<1>(a.E, a.k, w_scale, lds_ids, lds_w, ids_given != nullptr, id_given, s, lane, nullptr,
                                     reinterpret_cast<uint32_t *>(a.hand + kHandIdh) + static_cast<size_t>(l) * kResIdCopies * 16, kResIdCopies);
+                res_mark(a, c, l, 14);
                 wave_lds_fence();
                 if (lane < a.k) {
                     hand_store4(c.hb, kHandWh + static_cast<unsigned>((l * 16 + lane) * 4), f_bits(lds_w[lane]));
