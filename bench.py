@@ -64,6 +64,9 @@ def parse():
     ap.add_argument("--cache-warm-tokens", type=int, default=256,
                     help="lru mode: tokens run before the warm-up steps so that the slot pool is in steady state")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a captured HIP graph")
+    ap.add_argument("--path", choices=["resident", "per-layer"], default="resident",
+                    help="resident mode: the stack as ONE launch of resident workgroups (default), or two dispatches per layer")
+    ap.add_argument("--repeats", type=int, default=5, help="further repeats of the timed region, for the spread in the JSON line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=6.0,
                     help="wall-clock seconds of CPU layer passes to accumulate for cpu_baseline (all host threads busy)")
@@ -805,9 +808,28 @@ def main():
     d_out = torch.zeros(H, dtype=torch.float32, device="cuda")
     trace_ptr = C.c_void_p(d_trace.data_ptr()) if args.routing == "zipf" else None
 
-    def launch_stack():
+    PER_LAYER = 0x200   # WD_MOE_PER_LAYER
+    stack_flags = STACK_FLAGS | (PER_LAYER if args.path == "per-layer" else 0)
+
+    def launch_stack(flags=None):
         capi.call("wd_moe_stack_f32", layers, NL, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()), scratch,
-                  trace_ptr, RESIDUAL_SCALE, STACK_FLAGS, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+                  trace_ptr, RESIDUAL_SCALE, stack_flags if flags is None else flags,
+                  C.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+    def captured(fn):
+        """fn() warmed on a side stream, then captured into a HIP graph (None with --no-graph)."""
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        if args.no_graph:
+            return None
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        return g
 
     if args.check:
         from oracle import pyoracle
@@ -823,21 +845,12 @@ def main():
             sys.exit(1)
 
     note("inputs and routing trace ready")
-    graph = None
-    if not args.no_graph:
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            launch_stack()                       # warm the launch path outside capture
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            launch_stack()
+    graph = captured(launch_stack)
 
     note("launch mode: %s" % ("eager" if graph is None else "hip-graph replay"))
 
     def step(i):
+        i %= total_steps
         d_x.copy_(d_xs[i], non_blocking=True)
         d_trace.copy_(d_trace_all[i], non_blocking=True)
         if graph is not None:
@@ -845,19 +858,22 @@ def main():
         else:
             launch_stack()
 
+    def timed_region(first):
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for i in range(args.steps):
+            step(first + i)
+        ev1.record()
+        torch.cuda.synchronize()
+        return ev0.elapsed_time(ev1) / args.steps
+
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
     note("warm-up done, timing %d steps" % args.steps)
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
-    ev0.record()
-    for i in range(args.steps):
-        step(args.warmup + i)
-    ev1.record()
-    torch.cuda.synchronize()
+    ms_per_step = timed_region(args.warmup)
     wall = time.perf_counter() - t0
-    ms_per_step = ev0.elapsed_time(ev1) / args.steps
     tok_s = 1000.0 / ms_per_step
     finite = bool(torch.isfinite(d_x).all().item())
     waits_ok = capi.load().wd_moe_scratch_status(scratch) == 0   # no bounded wait inside a dispatch ran out
@@ -865,6 +881,10 @@ def main():
     if not (finite and waits_ok):
         print("bench.py: invalid run (finite=%s, in-dispatch waits ok=%s)" % (finite, waits_ok), file=sys.stderr)
         sys.exit(1)
+    repeats = sorted([ms_per_step] + [timed_region(args.warmup + (j + 1) * 7) for j in range(args.repeats)])
+    spread = dict(min=round(repeats[0], 4), median=round(repeats[len(repeats) // 2], 4), max=round(repeats[-1], 4),
+                  regions=len(repeats))
+    note("spread of %d timed regions: %s" % (len(repeats), spread))
 
     # Algorithmic bytes of the two dispatches of one layer (weights only, as the workload prices them):
     #   AB router f32 [E][H] + the shared expert's gate vector + its Q8_0 gate and up matrices
@@ -876,30 +896,7 @@ def main():
     assert E != 512 or bytes_per_layer == 27697152
     bytes_per_step = bytes_per_layer * NL
 
-    # Per-kernel launch time, live: the stack is replayed with one dispatch per layer only (the other two
-    # left out), so the timed region is a chain of NL launches of that one kernel over NL layers' weights
-    # (plus, for k_layer_ab, one small fill launch per chain that resets the in-dispatch hand-off words).
-    # HIP events on the launch stream bracket `reps` replays; the period includes the gap between two
-    # dependent launches on a stream (about 1.5 us in a graph), which a profiler's begin-to-end time omits.
-    only = {"k_layer_ab": 0x30, "k_layer_c": 0x40}
-    per_kernel, reps = {}, 20
-    step(0)
-    for name, flag in only.items():
-        def chain():
-            capi.call("wd_moe_stack_f32", layers, NL, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()), scratch,
-                      trace_ptr, RESIDUAL_SCALE, flag | CHAIN_FLAGS, C.c_void_p(torch.cuda.current_stream().cuda_stream))
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            chain()
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        runner = chain
-        if graph is not None:
-            g1 = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g1):
-                chain()
-            runner = g1.replay
+    def period_ms(runner, reps):
         for _ in range(3):
             runner()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -908,10 +905,58 @@ def main():
             runner()
         e1.record()
         torch.cuda.synchronize()
-        us = e0.elapsed_time(e1) * 1e3 / (reps * NL)
-        per_kernel[name] = dict(us_per_launch=round(us, 3), bytes_per_launch=alg[name],
-                                achieved=round(alg[name] / (us * 1e-6) / 1e9, 1))
-    dominant = max(per_kernel, key=lambda n: per_kernel[n]["us_per_launch"])
+        return e0.elapsed_time(e1) / reps
+
+    per_kernel, reps = {}, 20
+    step(0)
+    if args.path == "resident":
+        # The dominant kernel is the step itself: one launch of k_stack_resident covers the 48 layers.  Timed live with HIP
+        # events on the launch stream over `reps` launches (graph replays) without the input copies of step().
+        # (fresh input and routing trace before every launch, as in the timed region; the events bracket the launch alone)
+        run_it = graph.replay if graph is not None else launch_stack
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        for j, (e0, e1) in enumerate(pairs):
+            d_x.copy_(d_xs[j % total_steps], non_blocking=True)
+            d_trace.copy_(d_trace_all[j % total_steps], non_blocking=True)
+            e0.record()
+            run_it()
+            e1.record()
+        torch.cuda.synchronize()
+        us = sum(e0.elapsed_time(e1) for e0, e1 in pairs) / reps * 1e3
+        per_kernel["k_stack_resident"] = dict(us_per_launch=round(us, 2), bytes_per_launch=bytes_per_step,
+                                              achieved=round(bytes_per_step / (us * 1e-6) / 1e9, 1), layers_per_launch=NL,
+                                              us_per_layer=round(us / NL, 3))
+        # the same step as two dispatches per layer, for comparison
+        g2 = captured(lambda: launch_stack(STACK_FLAGS | PER_LAYER))
+        run_alt = g2.replay if g2 is not None else (lambda: launch_stack(STACK_FLAGS | PER_LAYER))
+
+        def alt_step(j):
+            d_x.copy_(d_xs[j % total_steps], non_blocking=True)
+            d_trace.copy_(d_trace_all[j % total_steps], non_blocking=True)
+            run_alt()
+        for j in range(4):
+            alt_step(j)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for j in range(reps):
+            alt_step(4 + j)
+        e1.record()
+        torch.cuda.synchronize()
+        per_kernel["per_layer_dispatches"] = dict(ms_per_step=round(e0.elapsed_time(e1) / reps, 4))
+        dominant = "k_stack_resident"
+    else:
+        # Per-kernel launch time, live: the stack is replayed with one dispatch per layer only (the other left out), so
+        # the timed region is a chain of NL launches of that one kernel over NL layers' weights.  The period includes
+        # the gap between two dependent launches on a stream, which a profiler's begin-to-end time omits.
+        only = {"k_layer_ab": 0x30, "k_layer_c": 0x40}
+        for name, flag in only.items():
+            def chain():
+                launch_stack(flag | CHAIN_FLAGS | PER_LAYER)
+            g1 = captured(chain)
+            us = period_ms(g1.replay if g1 is not None else chain, reps) * 1e3 / NL
+            per_kernel[name] = dict(us_per_launch=round(us, 3), bytes_per_launch=alg[name],
+                                    achieved=round(alg[name] / (us * 1e-6) / 1e9, 1))
+        dominant = max(per_kernel, key=lambda n: per_kernel[n]["us_per_launch"])
     note("per-kernel launch periods: %s; dominant: %s" % (per_kernel, dominant))
     traffic = recorded_traffic(dominant)
     dom = per_kernel[dominant]
@@ -941,6 +986,8 @@ def main():
                                % NL,
                    "layers": NL, "experts": E, "top_k": k, "routing": args.routing,
                    "launch": "eager" if graph is None else "hip-graph replay",
+                   "path": "one resident launch per step" if args.path == "resident" else "two dispatches per layer",
+                   "spread_ms_per_step": spread,
                    "bytes_per_token": bytes_per_step, "wall_s": round(wall, 3), "finite": finite,
                    "in_dispatch_waits_ok": waits_ok},
         "roofline": roofline,

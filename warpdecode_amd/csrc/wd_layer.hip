@@ -154,7 +154,7 @@ int wd_moe_scratch_set_wait_limit(wd_moe_scratch *s, unsigned polls) {
     // a fresh start: clear the status word and make the published ids invalid again
     WD_HIP(hipMemset(s->status, 0, sizeof(unsigned)));
     WD_HIP(hipMemset(s->tagged, 0xff, sizeof(uint32_t) * kTagRecords * kTagCopies * 16));
-    if (s->res_block) WD_HIP(hipMemset(s->res_block, 0xff, kHandFin));
+    if (s->res_block) WD_HIP(hipMemset(s->res_block, 0xff, kHandEpoch));
     return WD_OK;
 }
 float *wd_moe_scratch_logits(wd_moe_scratch *s) { return s->logits; }
@@ -653,8 +653,8 @@ int resident_prepare(wd_moe_scratch *s) {
         (void)hipFree(b);
         return fail(WD_ERR_HIP, "hipMalloc of the resident stack's layer descriptors failed");
     }
-    (void)hipMemset(b, 0xff, kHandFin);                      // every hand-off word "not yet written"
-    (void)hipMemset(b + kHandFin, 0, kHandBytes - kHandFin);  // launch numbers
+    (void)hipMemset(b, 0xff, kHandEpoch);                        // every hand-off word of both sets "not yet written"
+    (void)hipMemset(b + kHandEpoch, 0, kHandBytes - kHandEpoch);  // launches finished
     const ResidentViews v{s->logits, s->weights, s->accum, s->down_f32, s->shared_gate, s->ids};
     (void)hipMemcpy(s->res_layers + kResMaxLayers, &v, sizeof(v), hipMemcpyHostToDevice);
     s->res_block = b;

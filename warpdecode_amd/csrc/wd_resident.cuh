@@ -24,8 +24,8 @@
 // its own, one 128-byte line per (layer, workgroup): a line that several compute units write piece by piece while
 // the whole grid polls it changes hands once per write, and thirty-two writers per line made a hand-off take 17 us.  (An f32 result with
 // that very bit pattern - a NaN that no arithmetic here produces by itself - would be taken for "not yet" and end in
-// a timeout.)  After the last layer the workgroups meet once more (a barrier on words tagged with the launch number)
-// and every producer resets the words it wrote.  Waits are bounded: a wait that runs out sets status[0], after which
+// a timeout.)  There are two sets of these buffers: a launch works in one and resets the other as it goes (the router
+// waves, which have time to spare), so nothing has to be cleaned up when a launch ends.  Waits are bounded: a wait that runs out sets status[0], after which
 // every wait in the grid ends at once and later launches return immediately until the scratch is reset.
 #pragma once
 
@@ -80,10 +80,12 @@ constexpr unsigned kAcBytes = kAcRec * kResWgs;                                 
 constexpr unsigned kHandAc = kHandXc + 4u * kResMaxLayers * kResCopies * kResH;        // f32 [layers][copies][512][12] activations
 constexpr unsigned kHandIdh = kHandAc + kAcBytes * kResMaxLayers * kResCopies;         // u32 [layers][copies][16] selected ids
 constexpr unsigned kHandWh = kHandIdh + 4u * kResMaxLayers * kResIdCopies * 16;  // u32 [layers][16] router weights, [15] the shared gate
-constexpr unsigned kHandFin = kHandWh + 4u * kResMaxLayers * 16;              // u32 [512] number of the last launch each workgroup finished
-constexpr unsigned kHandEpoch = kHandFin + 4u * kResWgs;                      // u32 launches finished
+constexpr unsigned kHandSet = kHandWh + 4u * kResMaxLayers * 16;             // bytes of one set of hand-off buffers
+// The block holds two such sets and the number of launches finished.  Launch e works in set e % 2 and, layer by layer and
+// off its critical path, puts set (e + 1) % 2 back to "not yet written": no launch has to clean up behind itself.
+constexpr unsigned kHandEpoch = 2u * kHandSet;
 constexpr unsigned kHandBytes = kHandEpoch + 256u;
-static_assert(kHandXc % 128 == 0 && kHandAc % 128 == 0 && kHandIdh % 128 == 0 && kHandWh % 16 == 0 && kHandFin % 16 == 0, "hand-off block alignment");
+static_assert(kHandXc % 128 == 0 && kHandAc % 128 == 0 && kHandIdh % 128 == 0 && kHandWh % 16 == 0 && kHandSet % 128 == 0, "hand-off block alignment");
 WD_DEV unsigned rec_off(int l, int wg) { return kHandRec + static_cast<unsigned>(l * kResWgs + wg) * kRecBytes; }
 WD_DEV unsigned xc_off(int l, int copy) { return kHandXc + static_cast<unsigned>(l * kResCopies + copy) * (4u * kResH); }
 WD_DEV unsigned ac_off(int l, int copy) { return kHandAc + static_cast<unsigned>(l * kResCopies + copy) * kAcBytes; }
@@ -363,7 +365,7 @@ WD_DEV void res_down(const ResidentArgs &a, const ResCtx &c, int l, const Q8Coal
 // Waves 0..7 (always rungs 0..7) also fetch and quantise the layer's input, and in workgroup 0 select the experts.
 template <int TYPE>
 WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, int lane0, int wave0, int slot0,
-                            __amdgpu_buffer_rsrc_t hb, bool &dead) {
+                            __amdgpu_buffer_rsrc_t hb, unsigned set_base, bool &dead) {
     constexpr int kRow = 8 * ((TYPE == 21) ? 110 : 82);
     const bool shared = a.shared != 0;
     for (int l = 0; l < a.n_layers; ++l) {
@@ -442,7 +444,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             if (wave == 0) {
                 const float w_scale = *const_cast<const volatile float *>(&L->w_scale);
                 topk_block_step3<1>(a.E, a.k, w_scale, lds_ids, lds_w, ids_given != nullptr, id_given, s, lane, nullptr,
-                                    reinterpret_cast<uint32_t *>(a.hand + kHandIdh) + static_cast<size_t>(l) * kResIdCopies * 16, kResIdCopies);
+                                    reinterpret_cast<uint32_t *>(a.hand + set_base + kHandIdh) + static_cast<size_t>(l) * kResIdCopies * 16, kResIdCopies);
                 res_mark(a, c, l, 14);
                 wave_lds_fence();
                 if (lane < a.k) {
@@ -568,8 +570,10 @@ WD_DEV void res_shared_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
 }
 
 // ---- the router wave: row r --------------------------------------------------------------------------------------------
+// It also puts the other set of hand-off buffers (`ob`) back to "not yet written": in layer l this workgroup's share of
+// layers l, l + n, l + 2n, ... of that set (all kResMaxLayers layers, whatever the launch that wrote them used).
 WD_DEV void res_router_role(const ResidentArgs &a, uint8_t *lds_base, int r0, int lane0, int wave0,
-                            __amdgpu_buffer_rsrc_t hb, bool &dead) {
+                            __amdgpu_buffer_rsrc_t hb, __amdgpu_buffer_rsrc_t ob, bool &dead) {
     const bool on = r0 < a.E;
     float wv[32];
     if (on) res_router_fetch(res_field(&a.layers->router) + static_cast<size_t>(r0) * kResH, wv, lane0);
@@ -584,6 +588,17 @@ WD_DEV void res_router_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             if (lane == 32) hand_store4(c.hb, rec_off(l, r), f_bits(s));
             res_mark(a, c, l, 3);
             if (!last) res_router_fetch(res_field(&a.layers[l + 1].router) + static_cast<size_t>(r) * kResH, wv, lane);
+        }
+        for (int ll = l; ll < kResMaxLayers; ll += a.n_layers) {
+            const uint4 empty4 = make_uint4(kResEmpty, kResEmpty, kResEmpty, kResEmpty);
+            // 8 lanes the workgroup's record, 8 its 128 bytes of the layer's input copies, 24 its 384 bytes of the activations'
+            const unsigned off = lane < 8 ? rec_off(ll, r) + 16u * lane
+                               : lane < 16 ? xc_off(ll, 0) + 16u * (8 * r + lane - 8) : ac_off(ll, 0) + 16u * (24 * r + lane - 16);
+            if (lane < 40) hand_store16(ob, off, empty4);
+            if (r == 0) {
+                hand_store16(ob, kHandIdh + static_cast<unsigned>(ll * kResIdCopies * 64 + 16 * lane), empty4);
+                if (lane < 4) hand_store16(ob, kHandWh + static_cast<unsigned>(ll * 64 + 16 * lane), empty4);
+            }
         }
         if (r == 0) {
             __syncthreads();
@@ -609,8 +624,9 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = blockIdx.x;
     if (__hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return;  // an earlier launch failed
-    const __amdgpu_buffer_rsrc_t hb = hand_rsrc(a.hand, kHandBytes);
-    const unsigned epoch = hand_load4(hb, kHandEpoch);
+    const unsigned epoch = __hip_atomic_load(reinterpret_cast<const unsigned *>(a.hand + kHandEpoch), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned set_base = (epoch & 1u) ? kHandSet : 0u;
+    const __amdgpu_buffer_rsrc_t hb = hand_rsrc(a.hand + set_base, kHandSet), ob = hand_rsrc(a.hand + (kHandSet - set_base), kHandSet);
     stage_tables<TYPE == 21, TYPE == 22>(*reinterpret_cast<IqTables *>(lds_res + kResLdsTables), threadIdx.x, kResThreads);
 
     // Roles.  The twelve waves of a workgroup sit three to a SIMD (waves w, w + 4, w + 8 share one), and two
@@ -649,39 +665,15 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 
 
     bool dead = false;
     if (slot < 0)
-        res_router_role(a, lds_res, r, lane, wave, hb, dead);
+        res_router_role(a, lds_res, r, lane, wave, hb, ob, dead);
     else if (slot == kResSharedSlot)
         res_shared_role(a, lds_res, r, lane, wave, hb, dead);
     else
-        res_routed_role<TYPE>(a, lds_res, r, lane, wave, slot, hb, dead);
+        res_routed_role<TYPE>(a, lds_res, r, lane, wave, slot, hb, set_base, dead);
 
-    // ---- the end of the launch: every workgroup has finished every layer before any hand-off word is reset
-    __syncthreads();
-    if (threadIdx.x == 0) hand_store4(hb, kHandFin + static_cast<unsigned>(r * 4), epoch + 1u);
-    if (wave < 8 && !dead) {
-        const unsigned off = kHandFin + static_cast<unsigned>((wave * 64 + lane) * 4);
-        unsigned spins = 0;
-        for (;;) {
-            const bool need = hand_load4(hb, off) != epoch + 1u;
-            if (__builtin_amdgcn_ballot_w64(need) == 0ull) break;
-            if (res_give_up(a, spins, dead)) break;
-        }
-    }
-    __syncthreads();
-    // (after a failed wait the words stay as they are: the scratch has to be reset before it is used again)
-    if (__hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return;
-    const int n = a.n_layers;
-    const uint4 empty4 = make_uint4(kResEmpty, kResEmpty, kResEmpty, kResEmpty);
-    for (int l = threadIdx.x; l < n; l += kResThreads) hand_store16(hb, rec_off(l, r), empty4);  // this workgroup's records
-    // the copies of layers 0..n-1, shared out over the grid
-    const unsigned xc16 = static_cast<unsigned>(n) * kResCopies * (kResH / 4), ac16 = static_cast<unsigned>(n) * kResCopies * (kAcBytes / 16);
-    for (unsigned i = static_cast<unsigned>(r) * kResThreads + threadIdx.x; i < xc16; i += kResWgs * kResThreads) hand_store16(hb, kHandXc + 16u * i, empty4);
-    for (unsigned i = static_cast<unsigned>(r) * kResThreads + threadIdx.x; i < ac16; i += kResWgs * kResThreads) hand_store16(hb, kHandAc + 16u * i, empty4);
-    if (r == 0) {
-        for (int i = threadIdx.x; i < n * kResIdCopies * 4; i += kResThreads) hand_store16(hb, kHandIdh + static_cast<unsigned>(i * 16), empty4);
-        for (int i = threadIdx.x; i < n * 4; i += kResThreads) hand_store16(hb, kHandWh + static_cast<unsigned>(i * 16), empty4);
-        if (threadIdx.x == 0) hand_store4(hb, kHandEpoch, epoch + 1u);
-    }
+    // the next launch takes the other set (workgroup 0 can only get here after every workgroup has read the number)
+    if (r == 0 && threadIdx.x == 0 && !dead)
+        __hip_atomic_store(reinterpret_cast<unsigned *>(a.hand + kHandEpoch), epoch + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace wd
