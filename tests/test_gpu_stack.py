@@ -165,3 +165,79 @@ def test_graph_replayed_c2_stack(g, oracle):
         assert g.same_bits(d_x.cpu().numpy(), wx), token
     assert capi.load().wd_moe_scratch_status(sc.h) == 0
     sc.close()
+
+
+# ---- the stack as ONE launch of resident workgroups (layers of the 512-expert shape: hidden 2048, ffn 512) -------------
+PER_LAYER = 0x200
+VIEWS = (("ids", "k", np.int32), ("weights", "k", np.float32), ("logits", "E", np.float32), ("accum", "H", np.float32),
+         ("down_f32", "H", np.float32), ("shared_gate", 1, np.float32))
+
+
+def _run_stack(g, arr, n, x, tr, sc, flags):
+    dx, out = g.dev(x), g.empty(2048, np.float32)
+    dtr = g.dev(tr) if tr is not None else None
+    capi.call("wd_moe_stack_f32", arr, n, g.ptr(dx), g.ptr(out), sc.h, g.ptr(dtr), float(2.0 ** -12), flags, g.stream())
+    g.sync()
+    views = {}
+    for name, n_, dt in VIEWS:
+        cnt = {"k": sc.k, "E": sc.E, "H": sc.H}.get(n_, n_)
+        views[name] = sc.get(name, cnt, dt)
+    return g.host(dx), g.host(out), views
+
+
+@pytest.mark.parametrize("gate_type,experts,k,shared", [(synth.IQ3_S, 64, 10, True), (synth.IQ2_S, 40, 6, True),
+                                                        (synth.IQ3_S, 128, 9, False)],
+                         ids=["iq3s-64x10-shared", "iq2s-40x6-shared", "iq3s-128x9"])
+def test_one_launch_stack_matches_per_layer_and_oracle(g, oracle, gate_type, experts, k, shared):
+    """The resident launch against the per-layer dispatches (every output and every view of the last layer, bit for
+    bit) over launches in a row with stacks of different depth, with and without a routing trace; the first token
+    also against the oracle applied layer by layer."""
+    nl = 5
+    Ls = [synth.make_layer(2048, 512, experts, k, gate_type, synth.Q8_0, shared=shared, layer=300 + l,
+                           router_sigma=1.0 / np.sqrt(2048.0)) for l in range(nl)]
+    dls, arr = _descs(g, Ls)
+    sc_a, sc_b = g.Scratch(2048, 512, experts, k), g.Scratch(2048, 512, experts, k)
+    rng = np.random.default_rng(SEED + 400)
+    for token, depth in enumerate([nl, 2, nl, nl, 3, nl]):
+        x = synth.rms_normed(synth.rng_for(SEED, 84, token), 2048)
+        tr = None
+        if token % 2 == 1:
+            tr = np.stack([rng.choice(experts, size=k, replace=False) for _ in range(depth)]).astype(np.int32)
+        got = _run_stack(g, arr, depth, x, tr, sc_a, 0)
+        want = _run_stack(g, arr, depth, x, tr, sc_b, PER_LAYER)
+        assert g.same_bits(got[0], want[0]) and g.same_bits(got[1], want[1]), (token, depth)
+        for name, _, dt in VIEWS:
+            if name in ("down_f32", "shared_gate") and not shared:
+                continue
+            assert np.array_equal(got[2][name].view(np.uint32), want[2][name].view(np.uint32)), (token, name)
+        if token == 0:
+            wx = x.copy()
+            for L in Ls:
+                wout, _ = oracle.moe_layer(L, wx)
+                wx = (wx + (wout * np.float32(2.0 ** -12)).astype(np.float32)).astype(np.float32)
+            assert g.same_bits(got[0], wx) and g.same_bits(got[1], wout)
+    assert capi.load().wd_moe_scratch_status(sc_a.h) == 0
+    sc_a.close()
+    sc_b.close()
+
+
+def test_one_launch_stack_wait_that_runs_out(g):
+    """A wait limit of one poll: the launch ends normally with the status word set, later launches return at once
+    until the scratch is reset, and after the reset the results are right again."""
+    Ls = [synth.make_c2(layer=320 + l, n_experts=64) for l in range(3)]
+    dls, arr = _descs(g, Ls)
+    sc, ref = g.Scratch(2048, 512, 64, 10), g.Scratch(2048, 512, 64, 10)
+    x = synth.rms_normed(synth.rng_for(SEED, 85), 2048)
+    want = _run_stack(g, arr, 3, x, None, ref, PER_LAYER)
+    capi.call("wd_moe_scratch_set_wait_limit", sc.h, 1)
+    _run_stack(g, arr, 3, x, None, sc, 0)
+    assert capi.load().wd_moe_scratch_status(sc.h) == 1
+    _run_stack(g, arr, 3, x, None, sc, 0)            # refused on the device: nothing waits, nothing is written
+    assert capi.load().wd_moe_scratch_status(sc.h) == 1
+    capi.call("wd_moe_scratch_set_wait_limit", sc.h, 0)
+    assert capi.load().wd_moe_scratch_status(sc.h) == 0
+    for _ in range(3):
+        got = _run_stack(g, arr, 3, x, None, sc, 0)
+        assert g.same_bits(got[0], want[0]) and g.same_bits(got[1], want[1])
+    sc.close()
+    ref.close()
