@@ -300,6 +300,7 @@ def test_bounded_wait_gives_up_and_recovers(g, oracle):
     capi.call("wd_moe_layer_f32", C.byref(dl.desc), g.ptr(dx), g.ptr(out), sc.h, 0, g.stream())
     g.sync()
     assert lib.wd_moe_scratch_status(sc.h) == 1
+    assert np.isnan(g.host(out)).all()       # the failure is in the data too: no caller takes garbage for a result
     capi.call("wd_moe_scratch_set_wait_limit", sc.h, 0)
     assert lib.wd_moe_scratch_status(sc.h) == 0
     capi.call("wd_moe_layer_f32", C.byref(dl.desc), g.ptr(dx), g.ptr(out), sc.h, 0, g.stream())

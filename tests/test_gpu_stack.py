@@ -230,10 +230,12 @@ def test_one_launch_stack_wait_that_runs_out(g):
     x = synth.rms_normed(synth.rng_for(SEED, 85), 2048)
     want = _run_stack(g, arr, 3, x, None, ref, PER_LAYER)
     capi.call("wd_moe_scratch_set_wait_limit", sc.h, 1)
-    _run_stack(g, arr, 3, x, None, sc, 0)
+    bad = _run_stack(g, arr, 3, x, None, sc, 0)
     assert capi.load().wd_moe_scratch_status(sc.h) == 1
-    _run_stack(g, arr, 3, x, None, sc, 0)            # refused on the device: nothing waits, nothing is written
+    assert np.isnan(bad[0]).all() and np.isnan(bad[1]).all()   # the failure is in the data too
+    bad = _run_stack(g, arr, 3, x, None, sc, 0)      # refused on the device: nothing waits
     assert capi.load().wd_moe_scratch_status(sc.h) == 1
+    assert np.isnan(bad[0]).all() and np.isnan(bad[1]).all()
     capi.call("wd_moe_scratch_set_wait_limit", sc.h, 0)
     assert capi.load().wd_moe_scratch_status(sc.h) == 0
     for _ in range(3):

@@ -1023,7 +1023,9 @@ void k_layer_c(LayerArgs a) {
     mark(a, 2, 0);
     // combine operands, requested early: lane m keeps router weight m, lane 16 the shared gate
     float wreg = 0.0f, res_pre = 0.0f, inject = 0.0f;
+    unsigned bad = 0u;  // a bounded wait of this layer pass ran out: the results below are replaced by NaN
     if (wave == 0) {
+        bad = __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (lane < a.k) wreg = a.weights[lane];
         if (lane == 16 && shared) wreg = a.shared_gate[0];
         // the residual values this workgroup updates at its end (nothing else writes them meanwhile): lane 4c + r
@@ -1167,6 +1169,7 @@ void k_layer_c(LayerArgs a) {
             o = acc + prod;
             if (on) a.down_f32[row] = y;
         }
+        if (bad) acc = o = __builtin_nanf("");  // the caller sees the failure in its data, without a synchronisation
         if (on) {
             a.accum[row] = acc;
             a.out[row] = o;

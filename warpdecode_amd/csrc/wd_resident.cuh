@@ -511,8 +511,10 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                 o = acc + prod;
             }
             const float scaled = o * a.residual_scale;
-            const float xn = res_pre + scaled;
+            float xn = res_pre + scaled;
             if (last) {
+                // a wait that ran out anywhere in the grid: the caller sees it in its data, without a synchronisation
+                if (dead || __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) xn = o = acc = __builtin_nanf("");
                 if (lane < 4) {
                     const int row = 4 * r + lane;
                     a.x[row] = xn;
@@ -623,7 +625,10 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 
     extern __shared__ __align__(16) uint8_t lds_res[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = blockIdx.x;
-    if (__hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return;  // an earlier launch failed
+    if (__hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {  // an earlier launch failed
+        if (threadIdx.x < 4) a.x[4 * r + threadIdx.x] = a.out[4 * r + threadIdx.x] = __builtin_nanf("");
+        return;
+    }
     const unsigned epoch = __hip_atomic_load(reinterpret_cast<const unsigned *>(a.hand + kHandEpoch), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const unsigned set_base = (epoch & 1u) ? kHandSet : 0u;
     const __amdgpu_buffer_rsrc_t hb = hand_rsrc(a.hand + set_base, kHandSet), ob = hand_rsrc(a.hand + (kHandSet - set_base), kHandSet);
