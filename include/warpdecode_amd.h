@@ -245,6 +245,15 @@ int wd_moe_layer_hc_f32(const wd_moe_layer *layer, const float *d_x, float *d_ou
  *   q38_moe_run_shared_expert_f32_input (:3915-3948). */
 int wd_shared_expert_f32(const wd_moe_layer *layer, const float *d_x, wd_moe_scratch *scratch, void *stream);
 
+/* wd_moe_layer_f32 for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc): the same fused dispatches, with the intermediate values in a static device array of 128 KiB instead
+ * of a wd_moe_scratch object; the call allocates and frees nothing.  No counterpart in the reference.
+ * Limits: hidden <= 4096, expert_ffn <= 1024, n_experts <= 1024, top_k <= 16 (larger layers are refused with
+ * WD_ERR_ARG); flags 0 or WD_MOE_SPLIT_AB.  Only d_out is handed back (no views of ids, weights or partial sums).
+ * Every call on a GPU uses that GPU's one array: calls that overlap on a GPU race.  If a bounded wait inside the
+ * dispatches runs out, d_out is filled with NaN. */
+int wd_moe_layer_noalloc_f32(const wd_moe_layer *layer, const float *d_x, float *d_out, unsigned flags, void *stream);
+
 /* One decode step through a stack of layers: for each layer, x += residual_scale * layer(x) (the scaled
  * residual add stands in for the caller's own glue between two MoE blocks).  d_layer_out f32 [hidden] receives the last
  * layer's output.  d_ids_trace (device int32 [n_layers][top_k], may be NULL) replays a routing trace:

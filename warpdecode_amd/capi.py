@@ -97,6 +97,7 @@ _SIGS = {
     "wd_moe_scratch_set_wait_limit": (i32, [vp, u32]),
     "wd_shared_expert_f32": (i32, [C.POINTER(MoeLayer), vp, vp, vp]),
     "wd_moe_stack_f32": (i32, [C.POINTER(MoeLayer), i32, vp, vp, vp, vp, f32, u32, vp]),
+    "wd_moe_layer_noalloc_f32": (i32, [C.POINTER(MoeLayer), vp, vp, u32, vp]),
 }
 for _n in ("logits", "ids", "weights", "gate_up", "act", "act_qs", "act_scales", "expert_out", "accum", "down_f32",
            "shared_gate", "gate_up_partials", "down_partials"):

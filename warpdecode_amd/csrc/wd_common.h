@@ -16,6 +16,9 @@ std::string &last_error_slot();
 int fail(int code, const char *fmt, ...);
 
 inline hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
+// wd_noalloc.hip: looks up, once per device, where that device holds the static scratch array of the layer pass that
+// allocates nothing (the current device; wd_init calls it)
+int noalloc_setup_current_device();
 
 #define WD_HIP(call)                                                                         \
     do {                                                                                     \

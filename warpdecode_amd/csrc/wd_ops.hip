@@ -37,7 +37,7 @@ int wd_init(int device) {
     WD_HIP(hipGetDeviceProperties(&prop, device));
     WD_REQUIRE(prop.warpSize == 64, "wd_init: device %s has %d-wide waves; this library is built for gfx950",
                prop.name, prop.warpSize);
-    return WD_OK;
+    return noalloc_setup_current_device();
 }
 
 size_t wd_row_bytes(int type, int cols) { return row_bytes(type, cols); }
