@@ -161,9 +161,13 @@ typedef struct {
 typedef struct wd_moe_scratch wd_moe_scratch;
 int wd_moe_scratch_create(wd_moe_scratch **out, int hidden, int expert_ffn, int n_experts, int max_k);
 int wd_moe_scratch_destroy(wd_moe_scratch *s);
-/* 0 when every bounded wait inside the fused dispatches was satisfied so far, 1 when one ran out (the layer's
- * results are then invalid), -1 on error.  Synchronous read of one device word. */
+/* 0 when every bounded wait inside the fused dispatches was satisfied so far, 1 when one ran out, 2 when a kernel
+ * was asked for an expert whose entry in slot_of_expert is negative (not in the slot pool: the kernel read slot 0
+ * instead); the layer's results are then invalid and the fused combine has written NaN.  -1 on error.
+ * Synchronous read of one device word. */
 int wd_moe_scratch_status(wd_moe_scratch *s);
+/* The device word behind it (u32), for callers that copy it beside other results instead of a read of its own. */
+const unsigned *wd_moe_scratch_status_word(wd_moe_scratch *s);
 /* Sets the number of polls after which such a wait gives up (0 = the default, seconds of waiting) and clears the
  * status word.  For tests of the failure path: with a limit of 1 the waiting workgroups give up at once, set the
  * status and leave without touching memory; every kernel still ends normally.  Synchronous. */

@@ -227,6 +227,44 @@ static void host_only_checks() {
     }
     CHECK(throws([&] { GgufFile missing(path + ".nope"); }), "opening an absent file must throw");
     unlink(path.c_str());
+
+    // The reference's own files (copied as data) with the answers its tests check or print:
+    // tests/gguf_parser_test.cpp:6-8 prints version, tensor count and data offset of tests/min.gguf (3, 1, 160: the
+    // header ends at byte 134 and general.alignment is 32); tests/gguf_array_test.cpp:11-27 asserts the arrays of the
+    // fixture tests/make_qwen38_fixture.py writes; tests/gguf_type_size_test.cpp:17-25 the block sizes.
+    const char *env = std::getenv("WD_GOLDEN_DIR");
+    const std::string golden = env ? env : "tests/golden";
+    {
+        GgufFile g(golden + "/gguf/min.gguf");
+        CHECK(g.version() == 3 && g.tensors().size() == 1 && g.data_offset() == 160, "min.gguf: %u %zu %zu", g.version(), g.tensors().size(), g.data_offset());
+        CHECK(g.string_meta("general.architecture") == "llama" && g.uint_meta("general.alignment") == 32, "min.gguf metadata");
+        const TensorInfo &t = g.tensor("vec");
+        const float want[4] = {1.0f, 2.0f, 3.0f, 4.0f};
+        CHECK(t.type == GgmlType::F32 && t.dims == std::vector<uint64_t>({4}) && t.byte_size() == 16 && g.tensor_file_offset(t) == 160 &&
+                  std::memcmp(t.data, want, 16) == 0, "min.gguf tensor");
+    }
+    {
+        GgufFile g(golden + "/gguf/qwen38-fixture-00001-of-00002.gguf");
+        CHECK(g.version() == 3 && g.tensors().empty() && g.data_offset() == 2400, "fixture header: %u %zu %zu", g.version(), g.tensors().size(), g.data_offset());
+        const std::vector<int64_t> ratios = g.int_array_meta("qwen4exp.attention.compress_ratios");
+        CHECK(ratios.size() == 49 && ratios[3] == 8 && ratios[48] == 0, "compress_ratios");
+        const std::vector<uint64_t> ple = g.uint_array_meta("qwen4exp.ple.layers");
+        CHECK(ple.size() == 1 && ple[0] == 0, "ple.layers (an int32 array read as unsigned)");
+        CHECK(g.uint_array_meta("qwen4exp.ple.layer_multipliers") == std::vector<uint64_t>({3, 5, 7}), "ple.layer_multipliers");
+        const std::vector<uint64_t> offsets = g.uint_array_meta("qwen4exp.ple.head_offsets"), sizes = g.uint_array_meta("qwen4exp.ple.head_vocab_sizes");
+        CHECK(offsets.size() == 16 && sizes.size() == 16 && offsets.back() == 150 && sizes.back() == 10, "ple head arrays");
+        CHECK(g.number_array_meta("qwen4exp.rope.dimension_sections") == std::vector<double>({11, 11, 10, 0}), "rope sections as numbers");
+        CHECK(g.number_meta("qwen4exp.expert_weights_scale", 0.0) == 1.25 && g.uint_meta("qwen4exp.hyper_connection.count") == 4, "fixture scalars");
+        CHECK(g.has_meta("qwen4exp.ple.layers") && !g.has_meta("qwen4exp.absent"), "has_meta");
+        CHECK(throws([&] { g.int_array_meta("qwen4exp.absent"); }) && throws([&] { g.uint_array_meta("qwen4exp.expert_weights_scale"); }), "array accessors refuse absent keys and scalars");
+    }
+    auto size_of = [](GgmlType type, uint64_t n) {
+        TensorInfo ti{"test", {n}, type, 0, nullptr};
+        return ti.byte_size();
+    };
+    CHECK(size_of(GgmlType::F32, 32) == 128 && size_of(GgmlType::F16, 32) == 64 && size_of(GgmlType::BF16, 32) == 64, "float type sizes");
+    CHECK(size_of(GgmlType::Q4_0, 32) == 18 && size_of(GgmlType::Q8_0, 32) == 34 && size_of(GgmlType::Q6_K, 256) == 210, "Q4_0 / Q8_0 / Q6_K sizes");
+    CHECK(size_of(GgmlType::IQ4_NL, 32) == 18 && size_of(GgmlType::IQ3_S, 256) == 110 && size_of(GgmlType::IQ2_S, 256) == 82, "IQ type sizes");
 }
 
 // The reference's three calls, then the read-back a caller does.
@@ -353,6 +391,34 @@ static void gpu_checks() {
                 std::vector<float> acc(H);
                 check(wd_memcpy_d2h(acc.data(), scratch.d_accum(), sizeof(float) * H, nullptr), "accum");
                 CHECK(same_bits(acc.data(), routed.data(), H), "mode %d token %d layer %d: routed sum differs", mode, token, l);
+                if (mode == 1) {
+                    // the one-call wrappers with a cache that cannot hold the layer: the ids go through the host instead of
+                    // the kernels indexing a slot table with holes in it
+                    CHECK(!cache.layer_resident(l), "layer %d cannot be resident in 10 slots", l);
+                    run_qwen38_moe_layer_f32_x(l, dx.data, routers[l], L[l].t_gate, L[l].t_up, L[l].t_down, cache, shared[l], scratch, dout.data, 1.0f, stream);
+                    check(wd_stream_sync(stream), "sync");
+                    std::vector<float> fused(H);
+                    dout.download(fused.data());
+                    CHECK(same_bits(fused.data(), want.data(), H), "token %d layer %d: one-call wrapper over the LRU cache differs from the oracle", token, l);
+                    CHECK(wd_moe_scratch_status(scratch.handle()) == 0, "token %d layer %d: status word set", token, l);
+                    const int hc = 4;
+                    Qwen38HcF32DebugScratch hcs;
+                    hcs.initialize(H, hc);
+                    std::vector<float> res0(static_cast<size_t>(hc) * H), inject(hc);
+                    for (auto &v : res0) v = r.normal();
+                    for (auto &v : inject) v = 2.0f * r.normal();
+                    check(wd_memcpy_h2d(hcs.inject(), inject.data(), sizeof(float) * hc, nullptr), "inject");
+                    std::vector<float> want_res = res0;
+                    wdo_hc_combine_f32(want_res.data(), want.data(), inject.data(), H, hc, 0);
+                    DeviceFloatArray dres;
+                    dres.upload(res0.data(), res0.size());
+                    run_qwen38_moe_layer_hc_f32_x(l, dx.data, routers[l], L[l].t_gate, L[l].t_up, L[l].t_down, cache, shared[l], scratch, dout.data,
+                                                  dres.data, hcs, 1.0f, stream);
+                    check(wd_stream_sync(stream), "sync");
+                    std::vector<float> got_res(res0.size());
+                    dres.download(got_res.data());
+                    CHECK(same_bits(got_res.data(), want_res.data(), got_res.size()), "token %d layer %d: wrapper with combine over the LRU cache differs", token, l);
+                }
                 if (mode == 0) {
                     run_qwen38_moe_layer_f32_x(l, dx.data, routers[l], L[l].t_gate, L[l].t_up, L[l].t_down, cache, shared[l], scratch, dout.data, 1.0f, stream);
                     check(wd_stream_sync(stream), "sync");

@@ -110,6 +110,61 @@ def test_malformed_files_are_refused(tmp_path):
     _open_fails(p, "dimensions")
 
 
+    # dimensions whose product wraps around 64 bits (2^32 x 2^32 x 2 F32 elements would read as 0 bytes)
+    wrap = (struct.pack("<IIQQ", 0x46554747, 3, 1, 0) + struct.pack("<Q", 1) + b"t" + struct.pack("<I", 3) +
+            struct.pack("<QQQ", 1 << 32, 1 << 32, 2) + struct.pack("<IQ", 0, 0))
+    p.write_bytes(wrap + b"\0" * 64)
+    _open_fails(p, "does not fit 64 bits")
+
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gguf")
+
+
+def test_reference_fixtures_read_as_the_reference_tests_expect():
+    """The two GGUF files the reference ships for its parser tests (copied as data), with the answers those tests check:
+    tests/gguf_parser_test.cpp:6-8 prints version, tensor count and data offset of tests/min.gguf - 3, 1 and 160 (the
+    header ends at byte 134, general.alignment is 32; the file's 16 data bytes are the floats 1..4);
+    tests/gguf_array_test.cpp:11-27 asserts the arrays of the first shard of tests/qwen38-fixture (written by
+    tests/make_qwen38_fixture.py: no tensors, 2400 bytes of header)."""
+    with ggufio.GgufFile(os.path.join(GOLDEN, "min.gguf")) as g:
+        assert (g.version, len(g.tensors), g.data_offset) == (3, 1, 160)
+        assert g.string("general.architecture") == "llama" and g.number("general.alignment") == 32
+        t = g.tensors["vec"]
+        assert t["dims"] == [4] and t["type"] == 0 and t["relative_offset"] == 0 and t["bytes"] == 16
+        assert g.bytes_of("vec").view(np.float32).tolist() == [1.0, 2.0, 3.0, 4.0]
+    with ggufio.GgufFile(os.path.join(GOLDEN, "qwen38-fixture-00001-of-00002.gguf")) as g:
+        assert (g.version, len(g.tensors), g.data_offset) == (3, 0, 2400)
+        ratios = g.array("qwen4exp.attention.compress_ratios")
+        assert ratios.dtype == np.int32 and len(ratios) == 49 and ratios[3] == 8 and ratios[48] == 0
+        assert ratios.tolist() == [0, 0, 0, 8] * 12 + [0]
+        assert g.array("qwen4exp.ple.layers").tolist() == [0]
+        mult = g.array("qwen4exp.ple.layer_multipliers")
+        assert mult.dtype == np.uint64 and mult.tolist() == [3, 5, 7]
+        offsets, sizes = g.array("qwen4exp.ple.head_offsets"), g.array("qwen4exp.ple.head_vocab_sizes")
+        assert len(offsets) == 16 and len(sizes) == 16 and offsets[-1] == 150 and sizes[-1] == 10
+        assert g.array("qwen4exp.rope.dimension_sections").tolist() == [11, 11, 10, 0]
+        assert g.number("qwen4exp.expert_weights_scale") == 1.25 and g.number("qwen4exp.hyper_connection.count") == 4
+        assert g.number("qwen4exp.ple.eos_token_id") == 248044 and g.array("qwen4exp.absent") is None
+
+
+def test_block_sizes_as_the_reference_test_lists_them():
+    """tests/gguf_type_size_test.cpp:17-25 (the types this library computes with; F16 and BF16 are 2 bytes a value)."""
+    lib = capi.load()
+    for gtype, n, want in [(capi.Q4_0, 32, 18), (capi.Q8_0, 32, 34), (capi.Q6_K, 256, 210), (capi.IQ4_NL, 32, 18),
+                           (capi.IQ3_S, 256, 110), (capi.IQ2_S, 256, 82)]:
+        assert lib.wd_row_bytes(gtype, n) == want, gtype
+
+
+def test_float_tensor_sizes(tmp_path):
+    """F32 32 values = 128 bytes, F16 and BF16 32 values = 64 bytes (tests/gguf_type_size_test.cpp:17-19), as the
+    reader sizes tensors of those types in a directory."""
+    path = tmp_path / "f.gguf"
+    ggufio.write_gguf(path, [("a", [32], 0, np.zeros(128, np.uint8)), ("b", [32], 1, np.zeros(64, np.uint8)),
+                             ("c", [32], 30, np.zeros(64, np.uint8))])
+    with ggufio.GgufFile(path) as g:
+        assert [g.tensors[n]["bytes"] for n in "abc"] == [128, 64, 64]
+
+
 def test_unknown_tensor_type_is_listed_without_size(tmp_path):
     path = tmp_path / "q6.gguf"
     ggufio.write_gguf(path, [("output.weight", [256, 4], 12, np.zeros(4 * 144, np.uint8)),   # Q4_K: not computed here

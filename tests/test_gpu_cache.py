@@ -125,6 +125,73 @@ def test_cache_errors(g):
     capi.call("wd_expert_cache_destroy", cache)
 
 
+def test_state_after_a_failing_acquire(g, tmp_path):
+    """A call that fails part-way (the file behind the experts has lost its tail, so the read of one expert comes up
+    short) must leave the host's index, the device's slot table and the pool agreeing with each other: the experts
+    acquired before the failure are resident with their bytes in place, the failing one and those after it are not.
+    An id out of range is refused before anything changes.  Every failure here is a host-side error return."""
+    import mmap
+    import os
+    E, gb, ub, db = 8, 4096, 4096, 2048
+    slot = gb + ub + db
+    rng = np.random.default_rng(SEED + 17)
+    data = rng.integers(0, 256, E * slot, dtype=np.uint8)
+    path = tmp_path / "experts.bin"
+    data.tofile(path)
+    fd = os.open(path, os.O_RDWR)
+    mm = mmap.mmap(fd, E * slot)
+    base = np.frombuffer(mm, dtype=np.uint8).ctypes.data
+    lib = capi.load()
+    cache = C.c_void_p()
+    capi.call("wd_expert_cache_create", C.byref(cache), 5 * slot, gb, ub, db, 1, E, 0)
+    capi.call("wd_expert_cache_register_layer", cache, 0, C.c_void_p(base), C.c_void_p(base + E * gb), C.c_void_p(base + E * (gb + ub)))
+    capi.call("wd_expert_cache_attach_file", cache, C.c_void_p(base), E * slot, fd, 2)
+    os.ftruncate(fd, E * slot - db // 2)        # the last expert's down slice is no longer whole
+
+    def acquire(ids):
+        a = np.asarray(ids, np.int32)
+        hit = np.zeros(len(a), np.uint8)
+        rc = lib.wd_expert_cache_acquire(cache, 0, a.ctypes.data_as(C.c_void_p), len(a), hit.ctypes.data_as(C.c_void_p), g.stream())
+        g.sync()
+        return rc, hit
+
+    def expert_bytes(e):
+        return np.concatenate([data[e * gb:(e + 1) * gb], data[E * gb + e * ub:E * gb + (e + 1) * ub],
+                               data[E * (gb + ub) + e * db:E * (gb + ub) + (e + 1) * db]])
+
+    def check_state(resident):
+        table = g.view(lib.wd_expert_cache_slot_table(cache, 0), E, np.int32)
+        pool = g.view(lib.wd_expert_cache_pool(cache), 5 * slot, np.uint8)
+        for e in range(E):
+            s_host = lib.wd_expert_cache_slot_of(cache, 0, e)
+            assert s_host == table[e], (e, s_host, table[e])
+            assert (s_host >= 0) == (e in resident), (e, s_host)
+            if s_host >= 0:
+                assert np.array_equal(pool[s_host * slot:(s_host + 1) * slot], expert_bytes(e)), e
+        st = capi.CacheStats()
+        capi.call("wd_expert_cache_get_stats", cache, C.byref(st))
+        assert st.resident == len(resident)
+
+    rc, _ = acquire([0, 9, 1])                    # an id out of range: nothing changes
+    assert rc == -1
+    check_state(set())
+    rc, hit = acquire([0, 1, 7, 2])               # 0 and 1 are filled, 7 cannot be read, 2 is never reached
+    assert rc < 0 and "pread" in lib.wd_last_error().decode()
+    check_state({0, 1})
+    rc, hit = acquire([1, 0, 2])
+    assert rc == 0 and hit.tolist() == [1, 1, 0]
+    check_state({0, 1, 2})
+    rc, hit = acquire([3, 4, 5])                  # recycles slots: the one given back by the failed fill among them
+    assert rc == 0 and hit.tolist() == [0, 0, 0]
+    st = capi.CacheStats()
+    capi.call("wd_expert_cache_get_stats", cache, C.byref(st))
+    assert st.evictions == 1
+    check_state({0, 2, 3, 4, 5} if lib.wd_expert_cache_slot_of(cache, 0, 1) < 0 else {1, 2, 3, 4, 5})
+    capi.call("wd_expert_cache_destroy", cache)
+    del base
+    os.close(fd)
+
+
 def test_layer_through_slot_table(g, oracle):
     """A C2-shaped layer (fewer experts) whose routed tensors live only in the slot pool."""
     L = synth.make_c2(n_experts=64)
@@ -161,6 +228,22 @@ def test_layer_through_slot_table(g, oracle):
     st = capi.CacheStats()
     capi.call("wd_expert_cache_get_stats", cache, C.byref(st))
     assert st.misses > 24 and st.evictions > 0 and st.hits > 0
+    # The router's own selection over a pool that holds 24 of the 64 experts: the kernels meet negative entries of the
+    # slot table.  They read slot 0 instead (memory that exists), report it through the status word, and the fused
+    # combine hands NaN to the caller.
+    table = g.view(lib.wd_expert_cache_slot_table(cache, 0), E, np.int32)
+    x = synth.rms_normed(synth.rng_for(SEED, 61, 99), H)
+    _, dump = oracle.moe_layer(L, x)
+    assert any(table[e] < 0 for e in dump["ids"]), "the selection should include an expert without a slot"
+    dx, out = g.dev(x), g.empty(H, np.float32)
+    for flags in (0, capi.MOE_SPLIT_AB, capi.MOE_STAGED):
+        capi.call("wd_moe_layer_f32", C.byref(d), g.ptr(dx), g.ptr(out), sc.h, flags, g.stream())
+        g.sync()
+        assert lib.wd_moe_scratch_status(sc.h) == 2, flags
+        if flags != capi.MOE_STAGED:
+            assert np.isnan(g.host(out)).all(), flags
+        capi.call("wd_moe_scratch_set_wait_limit", sc.h, 0)
+        assert lib.wd_moe_scratch_status(sc.h) == 0
     sc.close()
     capi.call("wd_expert_cache_destroy", cache)
 

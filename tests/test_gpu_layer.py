@@ -280,6 +280,24 @@ def test_selection_more_than_512_experts(g, oracle):
         _fused_vs_oracle(g, oracle, dup, x)
 
 
+def test_expert_counts_the_selection_cannot_take_are_refused(g, oracle):
+    """The router's selection sums probabilities in groups of eight experts and holds at most 1024 of them
+    (src/qwen38_moe.cuh:686-688): other counts are an error on every path that selects, not a silently different
+    result; a pass on a given selection takes any count."""
+    L = synth.make_layer(256, 64, 12, 2, synth.IQ3_S, synth.Q8_0, shared=True)
+    dl, sc = g.DeviceLayer(L), g.Scratch(256, 64, 12, 2)
+    x = synth.rms_normed(synth.rng_for(SEED, 45), 256)
+    dx, out = g.dev(x), g.empty(256, np.float32)
+    lib = capi.load()
+    for flags in (0, capi.MOE_SPLIT_AB, capi.MOE_STAGED):
+        assert lib.wd_moe_layer_f32(C.byref(dl.desc), g.ptr(dx), g.ptr(out), sc.h, flags, g.stream()) == -1, flags
+        assert "multiple of 8" in lib.wd_last_error().decode()
+    arr = (capi.MoeLayer * 1)(dl.desc)
+    assert lib.wd_moe_stack_f32(arr, 1, g.ptr(dx), g.ptr(out), sc.h, None, 1.0, 0, g.stream()) == -1
+    sc.close()
+    check_layer(g, oracle, L, x, flags=capi.MOE_PRESELECTED, ids=np.array([11, 3], np.int32), weights=np.array([0.25, 0.5], np.float32))
+
+
 def test_status_word_is_clear(g):
     sc = g.Scratch(512, 64, 8, 2)
     assert capi.load().wd_moe_scratch_status(sc.h) == 0

@@ -10,7 +10,8 @@ EXE = os.path.join(ROOT, "tests", "host", "test_wd_ops")
 
 
 def _run(args):
-    p = subprocess.run([EXE] + args, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    env = dict(os.environ, WD_GOLDEN_DIR=os.path.join(ROOT, "tests", "golden"))
+    p = subprocess.run([EXE] + args, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300, env=env)
     assert p.returncode == 0, p.stdout
     assert " 0 failures" in p.stdout, p.stdout
     return p.stdout

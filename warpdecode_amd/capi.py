@@ -15,6 +15,7 @@ HEADER = os.path.join(os.path.dirname(HERE), "include", "warpdecode_amd.h")
 F32, F16, Q4_0, Q8_0, IQ4_NL, IQ3_S, IQ2_S = 0, 1, 2, 8, 20, 21, 22
 Q6_K = 14
 MOE_PRESELECTED, MOE_KEEP_EXPERT_OUT, MOE_STAGED = 1, 2, 4
+MOE_ONLY_A, MOE_ONLY_B, MOE_ONLY_C, MOE_DRY, MOE_SPLIT_AB = 0x10, 0x20, 0x40, 0x80, 0x100
 MOE_PER_LAYER = 0x200
 
 vp, i32, f32, sz, u32 = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint
@@ -94,6 +95,7 @@ _SIGS = {
     "wd_moe_layer_f32": (i32, [C.POINTER(MoeLayer), vp, vp, vp, u32, vp]),
     "wd_moe_stack_cached_f32": (i32, [C.POINTER(MoeLayer), i32, vp, vp, vp, vp, vp, vp, f32, u32, vp]),
     "wd_moe_scratch_status": (i32, [vp]),
+    "wd_moe_scratch_status_word": (vp, [vp]),
     "wd_moe_scratch_set_wait_limit": (i32, [vp, u32]),
     "wd_shared_expert_f32": (i32, [C.POINTER(MoeLayer), vp, vp, vp]),
     "wd_moe_stack_f32": (i32, [C.POINTER(MoeLayer), i32, vp, vp, vp, vp, f32, u32, vp]),

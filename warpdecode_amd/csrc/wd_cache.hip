@@ -27,11 +27,13 @@
 #include <fcntl.h>
 #include <unistd.h>
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <condition_variable>
 #include <cstdio>
 #include <cstring>
+#include <functional>
 #include <list>
 #include <mutex>
 #include <new>
@@ -588,6 +590,9 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
     Partition &P = c->parts[c->partitioned ? layer : 0];
     WD_REQUIRE(P.end - P.begin >= static_cast<size_t>(k), "expert cache: %zu slots cannot hold %d experts at once",
                P.end - P.begin, k);
+    // every id is checked before anything changes: a bad one must not leave half of the call applied
+    for (int j = 0; j < k; ++j)
+        WD_REQUIRE(h_ids[j] >= 0 && h_ids[j] < c->n_experts, "expert index out of range: %d", h_ids[j]);
     hipStream_t st = as_stream(stream);
     const auto t_begin = std::chrono::steady_clock::now();
     struct Timer {
@@ -630,9 +635,12 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
     int n_fill = 0;
     uint32_t max_words = 0;
 
+    // A failure inside the loop (no slot may be recycled, a short read from the file) ends the loop, not the call: the
+    // fills and slot-table changes of the experts acquired before it are still issued below, so that the host's index
+    // and the device's table describe the same pool when the error is returned.
+    int rc_late = WD_OK;
     for (int j = 0; j < k; ++j) {
         const int e = h_ids[j];
-        WD_REQUIRE(e >= 0 && e < c->n_experts, "expert index out of range: %d", e);
         const uint64_t key = (static_cast<uint64_t>(static_cast<uint32_t>(layer)) << 32) | static_cast<uint32_t>(e);
         ++c->clock;
         ++c->stats.accesses;
@@ -659,8 +667,10 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
         } else {
             slot = P.lru.front();
             Slot &victim = c->slots[slot];
-            if (victim.last_use > victim_floor)
-                return fail(WD_ERR_STATE, "expert cache: all slots are held by the experts being acquired");
+            if (victim.last_use > victim_floor) {
+                rc_late = fail(WD_ERR_STATE, "expert cache: all slots are held by the experts being acquired");
+                break;
+            }
             P.lru.pop_front();
             c->index.erase(victim.key);
             updates[n_updates++] = {static_cast<int32_t>((victim.key >> 32) * c->n_experts + (victim.key & 0xffffffffu)), -1};
@@ -708,8 +718,16 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
                 }
                 at += len3[q];
             }
-            if (!c->pread_pool->run(pieces, n_pieces))
-                return fail(WD_ERR_STATE, "expert cache: pread of layer %d expert %d failed or came up short", layer, e);
+            if (!c->pread_pool->run(pieces, n_pieces)) {
+                // this expert never reached its slot: take it out of the index again (the victim stays evicted)
+                c->index.erase(key);
+                P.lru.pop_back();
+                s.valid = false;
+                P.free.insert(std::upper_bound(P.free.begin(), P.free.end(), slot, std::greater<size_t>()), slot);
+                --n_updates;
+                rc_late = fail(WD_ERR_STATE, "expert cache: pread of layer %d expert %d failed or came up short", layer, e);
+                break;
+            }
             c->pread_ms += std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
             WD_HIP(hipMemcpyAsync(dst, entry, c->slot_bytes, hipMemcpyHostToDevice, c->copy_stream));
             WD_HIP(hipEventRecord(c->stage_done[r], c->copy_stream));
@@ -757,7 +775,7 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
                 WD_HIP(hipStreamWaitEvent(st, c->ev_done, 0));
         }
     }
-    return WD_OK;
+    return rc_late;
 }
 
 // Acquires the experts of every layer of one token before any of the token's layers is launched, so that the host
@@ -772,9 +790,12 @@ int acquire_token_ahead(wd_expert_cache *c, int n_layers, const int32_t *h_ids, 
             if (!ev) WD_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
     }
     AheadState ahead{c->clock, false, {}};
-    for (int l = 0; l < n_layers; ++l)
-        if (const int rc = acquire_impl(c, l, h_ids + static_cast<size_t>(l) * k, k, nullptr, stream, true, &ahead)) return rc;
-    return flush_slot_updates(c, ahead.updates.data(), static_cast<int>(ahead.updates.size()), as_stream(stream));
+    int rc_late = WD_OK;
+    for (int l = 0; l < n_layers && rc_late == WD_OK; ++l)
+        rc_late = acquire_impl(c, l, h_ids + static_cast<size_t>(l) * k, k, nullptr, stream, true, &ahead);
+    // also after a failure: the table must describe what the layers before it did to the pool
+    const int rc = flush_slot_updates(c, ahead.updates.data(), static_cast<int>(ahead.updates.size()), as_stream(stream));
+    return rc_late != WD_OK ? rc_late : rc;
 }
 
 int wait_layer_fills(wd_expert_cache *c, int layer, hipStream_t st) {

@@ -1169,6 +1169,8 @@ void k_layer_c(LayerArgs a) {
             o = acc + prod;
             if (on) a.down_f32[row] = y;
         }
+        // an expert without a slot was reported by the waves above (or by the dispatch before)
+        if (a.down.slot_of_expert) bad |= __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (bad) acc = o = __builtin_nanf("");  // the caller sees the failure in its data, without a synchronisation
         if (on) {
             a.accum[row] = acc;

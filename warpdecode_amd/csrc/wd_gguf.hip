@@ -100,18 +100,22 @@ bool read_scalar(Reader &r, uint32_t t, GgufValue &v) {
     return r.ok;
 }
 
-uint64_t tensor_bytes(const GgufTensor &t) {
+// Bytes of a tensor's data; false when the element count or the byte count does not fit 64 bits (a crafted header
+// whose product wraps would otherwise pass the bounds test with a small size).
+bool tensor_bytes(const GgufTensor &t, uint64_t *bytes) {
     uint64_t n = 1;
-    for (uint32_t d = 0; d < t.n_dims; ++d) n *= t.dims[d];
+    for (uint32_t d = 0; d < t.n_dims; ++d)
+        if (__builtin_mul_overflow(n, t.dims[d], &n)) return false;
     switch (t.type) {
-        case 0: return n * 4;            // F32
-        case 1: case 30: return n * 2;   // F16, BF16
+        case 0: return !__builtin_mul_overflow(n, uint64_t{4}, bytes);            // F32
+        case 1: case 30: return !__builtin_mul_overflow(n, uint64_t{2}, bytes);   // F16, BF16
         default: break;
     }
-    const uint64_t cols = t.dims[0];
-    if (cols == 0 || cols > 0x7fffffffu) return 0;
-    const size_t row = row_bytes(static_cast<int>(t.type), static_cast<int>(cols));
-    return row ? (n / cols) * row : 0;
+    const uint64_t cols = t.n_dims ? t.dims[0] : 0;
+    *bytes = 0;
+    if (cols == 0 || cols > 0x7fffffffu) return true;
+    const uint64_t row = row_bytes(static_cast<int>(t.type), static_cast<int>(cols));
+    return !__builtin_mul_overflow(n / cols, row, bytes);
 }
 
 }  // namespace
@@ -208,7 +212,11 @@ int wd_gguf_open(wd_gguf **out, const char *path) {
     g->data_offset = (r.at + alignment - 1) & ~(alignment - 1);
     if (g->data_offset > g->size) return bail("tensor data would start past the end of the file");
     for (GgufTensor &t : g->tensors) {
-        t.bytes = tensor_bytes(t);
+        if (!tensor_bytes(t, &t.bytes)) {
+            const int rc = fail(WD_ERR_ARG, "GGUF %s: the size of tensor %s does not fit 64 bits", path, t.name.c_str());
+            wd_gguf_close(g);
+            return rc;
+        }
         if (t.relative_offset > g->size - g->data_offset || t.bytes > g->size - g->data_offset - t.relative_offset) {
             const int rc = fail(WD_ERR_ARG, "GGUF %s: tensor %s lies outside the file", path, t.name.c_str());
             wd_gguf_close(g);

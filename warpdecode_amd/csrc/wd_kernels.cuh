@@ -22,14 +22,25 @@ struct MatSrc {
     const uint8_t *pool;
     size_t slot_bytes;
     size_t slot_off[2];
+    unsigned *slot_status;  // set to 2 when an expert without a slot is asked for (may be null)
 };
+
+// The slot of an expert that is not in the pool is -1: such a request is reported through the status word and reads
+// slot 0 (memory that exists, values that mean nothing) instead of an address before the pool.
+WD_DEV size_t checked_slot(const MatSrc &s, int slot) {
+    if (slot < 0) {
+        if (s.slot_status) __hip_atomic_store(s.slot_status, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        slot = 0;
+    }
+    return static_cast<size_t>(slot);
+}
 
 WD_DEV const uint8_t *mat_ptr(const MatSrc &s, int m) {
     if (s.table) return s.table[m];
     if (s.ids) {
         const int j = m / s.per_expert, t = m - j * s.per_expert;
         const int e = s.ids[j];
-        if (s.slot_of_expert) return s.pool + static_cast<size_t>(s.slot_of_expert[e]) * s.slot_bytes + s.slot_off[t];
+        if (s.slot_of_expert) return s.pool + checked_slot(s, s.slot_of_expert[e]) * s.slot_bytes + s.slot_off[t];
         return s.base[t] + static_cast<size_t>(e) * s.stride[t];
     }
     return s.single;
@@ -40,7 +51,7 @@ WD_DEV const uint8_t *mat_ptr(const MatSrc &s, int m) {
 // without waiting for e) instead of a lookup by a computed index.
 template <int T>
 WD_DEV const uint8_t *mat_ptr_expert(const MatSrc &s, int e) {
-    if (s.slot_of_expert) return s.pool + static_cast<size_t>(s.slot_of_expert[e]) * s.slot_bytes + s.slot_off[T];
+    if (s.slot_of_expert) return s.pool + checked_slot(s, s.slot_of_expert[e]) * s.slot_bytes + s.slot_off[T];
     return s.base[T] + static_cast<size_t>(e) * s.stride[T];
 }
 
@@ -48,7 +59,7 @@ WD_DEV const uint8_t *mat_ptr_expert(const MatSrc &s, int e) {
 // waits for nor is counted among the wave's vector loads.
 template <int T>
 WD_DEV const uint8_t *mat_ptr_expert_uniform(const MatSrc &s, int e) {
-    if (s.slot_of_expert) return s.pool + static_cast<size_t>(sld_i32(s.slot_of_expert + e)) * s.slot_bytes + s.slot_off[T];
+    if (s.slot_of_expert) return s.pool + checked_slot(s, sld_i32(s.slot_of_expert + e)) * s.slot_bytes + s.slot_off[T];
     return s.base[T] + static_cast<size_t>(e) * s.stride[T];
 }
 

@@ -148,6 +148,7 @@ int wd_moe_scratch_status(wd_moe_scratch *s) {
     if (hipMemcpy(&v, s->status, sizeof(v), hipMemcpyDeviceToHost) != hipSuccess) return -1;
     return static_cast<int>(v);
 }
+const unsigned *wd_moe_scratch_status_word(wd_moe_scratch *s) { return s ? s->status : nullptr; }
 int wd_moe_scratch_set_wait_limit(wd_moe_scratch *s, unsigned polls) {
     WD_REQUIRE(s != nullptr, "wd_moe_scratch_set_wait_limit: null scratch");
     s->spin_limit = polls ? polls : kSpinLimit;
@@ -223,7 +224,7 @@ int wd_moe_scratch_enable_partials(wd_moe_scratch *s, int gate_type, int down_ty
 
 namespace {
 
-int check_layer(const wd_moe_layer *L, const wd_moe_scratch *s) {
+int check_layer(const wd_moe_layer *L, const wd_moe_scratch *s, unsigned flags) {
     WD_REQUIRE(L && s, "MoE layer: null layer or scratch");
     WD_REQUIRE(L->hidden == s->hidden && L->expert_ffn == s->ffn, "MoE layer geometry mismatch: layer %d/%d, scratch %d/%d",
                L->hidden, L->expert_ffn, s->hidden, s->ffn);
@@ -238,6 +239,10 @@ int check_layer(const wd_moe_layer *L, const wd_moe_scratch *s) {
     WD_REQUIRE(L->down_type == WD_TYPE_Q8_0 || L->down_type == WD_TYPE_IQ4_NL, "MoE layer: unsupported down type %d",
                L->down_type);
     WD_REQUIRE(L->router != nullptr, "MoE layer: null router");
+    // the selection sums the probabilities in groups of eight experts and holds at most 1024 of them (src/qwen38_moe.cuh:686-688)
+    if (!(flags & WD_MOE_PRESELECTED))
+        WD_REQUIRE(L->n_experts % 8 == 0 && L->n_experts <= 1024,
+                   "MoE layer: the router's selection needs n_experts (%d) to be a multiple of 8, at most 1024", L->n_experts);
     if (L->slot_of_expert) {
         WD_REQUIRE(L->slot_pool != nullptr && L->slot_bytes > 0, "MoE layer: slot table without a slot pool");
     } else {
@@ -247,9 +252,10 @@ int check_layer(const wd_moe_layer *L, const wd_moe_scratch *s) {
     return WD_OK;
 }
 
-MatSrc routed_src(const wd_moe_layer *L, const int32_t *ids, bool down) {
+MatSrc routed_src(const wd_moe_layer *L, const wd_moe_scratch *s, const int32_t *ids, bool down) {
     MatSrc m{};
     m.ids = ids;
+    m.slot_status = s->status;
     m.per_expert = down ? 1 : 2;
     if (L->slot_of_expert) {
         m.slot_of_expert = L->slot_of_expert;
@@ -332,7 +338,6 @@ int layer_staged(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_s
         k_router_gemv<<<dim3((E + (shared ? 1 : 0) + 7) / 8), dim3(256), 0, st>>>(
             L->router, d_x, s->logits, E, H, shared ? L->shared_gate_inp : nullptr, s->shared_gate);
         WD_LAUNCH_CHECK();
-        if (E % 8 != 0 || E > 1024) return fail(WD_ERR_UNSUPPORTED, "router: n_experts %d must be a multiple of 8 <= 1024", E);
         k_topk_softmax<<<dim3(1), dim3(64), 0, st>>>(s->logits, E, k, L->expert_scale, s->ids, s->weights,
                                                      shared ? s->shared_gate : nullptr, ids_override);
         WD_LAUNCH_CHECK();
@@ -355,7 +360,7 @@ int layer_staged(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_s
 
     // 3. gate/up of the k selected experts in one dispatch (2k matrices), then the shared expert's
     const bool part = s->gup != nullptr && s->gup_type == L->gate_type && s->dp_type == L->down_type;
-    if (const int rc = grouped_gemv(L->gate_type, routed_src(L, s->ids, false), 2 * k, F, H, s, s->x0_qs, s->x0_d, 0,
+    if (const int rc = grouped_gemv(L->gate_type, routed_src(L, s, s->ids, false), 2 * k, F, H, s, s->x0_qs, s->x0_d, 0,
                                     s->gate_up, part ? s->gup : nullptr, st))
         return rc;
     if (shared) {
@@ -374,7 +379,7 @@ int layer_staged(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_s
     WD_LAUNCH_CHECK();
 
     // 6. down projections: k routed matrices with their own activations, then the shared expert
-    if (const int rc = grouped_gemv(L->down_type, routed_src(L, s->ids, true), k, H, F, s, s->act_qs, s->act_d, F,
+    if (const int rc = grouped_gemv(L->down_type, routed_src(L, s, s->ids, true), k, H, F, s, s->act_qs, s->act_d, F,
                                     s->expert_out, part ? s->dp : nullptr, st))
         return rc;
     if (shared) {
@@ -407,8 +412,8 @@ LayerArgs fused_args(const wd_moe_layer *L, const float *d_x, float *d_out, wd_m
     a.w_scale = L->expert_scale;
     a.x = d_x;
     a.router = L->router;
-    a.gate_up = routed_src(L, s->ids, false);
-    a.down = routed_src(L, s->ids, true);
+    a.gate_up = routed_src(L, s, s->ids, false);
+    a.down = routed_src(L, s, s->ids, true);
     a.sh_inp = L->shared_gate_inp;
     a.sh_gate = L->shared_gate, a.sh_up = L->shared_up, a.sh_down = L->shared_down;
     a.logits = s->logits, a.ids = s->ids, a.weights = s->weights;
@@ -573,7 +578,7 @@ int layer_dispatch(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe
 
 extern "C" int wd_moe_layer_f32(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s,
                                 unsigned flags, void *stream) {
-    if (const int rc = check_layer(L, s)) return rc;
+    if (const int rc = check_layer(L, s, flags)) return rc;
     WD_REQUIRE(d_x && d_out, "MoE layer: null activation or output pointer");
     return layer_dispatch(L, d_x, d_out, s, flags, nullptr, nullptr, 0.0f, as_stream(stream));
 }
@@ -581,7 +586,7 @@ extern "C" int wd_moe_layer_f32(const wd_moe_layer *L, const float *d_x, float *
 extern "C" int wd_moe_layer_hc_f32(const wd_moe_layer *L, const float *d_x, float *d_out, float *d_residual,
                                    const float *d_inject, int hc, int round_half, wd_moe_scratch *s, unsigned flags,
                                    void *stream) {
-    if (const int rc = check_layer(L, s)) return rc;
+    if (const int rc = check_layer(L, s, flags)) return rc;
     WD_REQUIRE(d_x && d_out && d_residual && d_inject, "MoE layer with combine: null activation, output, residual or inject pointer");
     WD_REQUIRE(hc >= 1 && hc <= 16, "MoE layer with combine: 1..16 residual streams (got %d)", hc);
     WD_REQUIRE(!(flags & (WD_MOE_ONLY_A | WD_MOE_ONLY_B | WD_MOE_ONLY_C | WD_MOE_DRY)), "MoE layer with combine: measurement flags are not supported");
@@ -741,7 +746,7 @@ extern "C" int wd_moe_stack_f32(const wd_moe_layer *layers, int n_layers, float 
     WD_REQUIRE(layers && n_layers > 0, "MoE stack: no layers");
     WD_REQUIRE(d_x && d_layer_out, "MoE stack: null activation or output pointer");
     for (int l = 0; l < n_layers; ++l) {
-        if (const int rc = check_layer(&layers[l], s)) return rc;
+        if (const int rc = check_layer(&layers[l], s, flags)) return rc;
     }
     if (resident_shape(layers, n_layers, s, flags)) {
         const int rc = stack_resident(layers, n_layers, d_x, d_layer_out, s, d_ids_trace, residual_scale, as_stream(stream));
@@ -771,7 +776,7 @@ extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, 
         WD_REQUIRE(scratch_per_token[t] != nullptr, "multi-token pass: null scratch for token %d", t);
         for (int q = 0; q < t; ++q)
             WD_REQUIRE(scratch_per_token[q] != scratch_per_token[t], "multi-token pass: tokens %d and %d share a scratch", q, t);
-        if (const int rc = check_layer(L, scratch_per_token[t])) return rc;
+        if (const int rc = check_layer(L, scratch_per_token[t], flags)) return rc;
     }
     hipStream_t st = as_stream(stream);
     const int H = L->hidden, F = L->expert_ffn, k = L->top_k;
@@ -792,8 +797,8 @@ extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, 
     TokenArgs ta{};
     ta.T = tokens;
     ta.common = fused_args(L, d_x, d_out, scratch_per_token[0], flags, nullptr, nullptr, 0.0f);
-    ta.common.gate_up = routed_src(L, nullptr, false);  // the kernels pass the expert id themselves
-    ta.common.down = routed_src(L, nullptr, true);
+    ta.common.gate_up = routed_src(L, scratch_per_token[0], nullptr, false);  // the kernels pass the expert id themselves
+    ta.common.down = routed_src(L, scratch_per_token[0], nullptr, true);
     for (int t = 0; t < tokens; ++t) {
         wd_moe_scratch *s = scratch_per_token[t];
         TokenSlots &k_ = ta.tok[t];

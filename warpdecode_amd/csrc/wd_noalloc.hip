@@ -89,7 +89,7 @@ extern "C" int wd_moe_layer_noalloc_f32(const wd_moe_layer *L, const float *d_x,
     view.down_f32 = reinterpret_cast<float *>(ptr + off_down);
     view.act = reinterpret_cast<float *>(ptr + off_act);
     view.compute_units = g_compute_units[dev];
-    if (const int rc = check_layer(L, &view)) return rc;
+    if (const int rc = check_layer(L, &view, flags)) return rc;
     const hipStream_t st = as_stream(stream);
     k_noalloc_clean<<<dim3(1), dim3(512), 0, st>>>(reinterpret_cast<uint32_t *>(ptr));
     WD_LAUNCH_CHECK();

@@ -28,7 +28,7 @@ extern "C" int wd_moe_stack_cached_f32(const wd_moe_layer *layers, int n_layers,
     };
     for (int l = 0; l < n_layers; ++l) {
         const wd_moe_layer L = bind(l);
-        if (const int rc = check_layer(&L, s)) return rc;
+        if (const int rc = check_layer(&L, s, flags)) return rc;
         WD_REQUIRE(L.n_experts == cache->n_experts, "cached MoE stack: layer %d has %d experts, the cache %d", l, L.n_experts, cache->n_experts);
     }
     const int k = layers[0].top_k;
@@ -71,7 +71,9 @@ extern "C" int wd_moe_stack_cached_f32(const wd_moe_layer *layers, int n_layers,
 
     for (int l = 0; l < n_layers; ++l) {
         const wd_moe_layer L = bind(l);
-        if (!(flags & WD_MOE_PRESELECTED)) {
+        // dispatch A also carries the shared expert's gate/up rows and its gate: it runs whenever there is something in it
+        // (with ids given by the caller it leaves the router rows out)
+        if (!(flags & WD_MOE_PRESELECTED) || L.shared_gate_inp) {
             if (const int rc = layer_fused(&L, d_x, d_layer_out, s, flags | WD_MOE_ONLY_A, nullptr, d_x, residual_scale, st)) return rc;
         }
         WD_HIP(hipMemcpyAsync(s->h_ids, s->ids, sizeof(int32_t) * L.top_k, hipMemcpyDeviceToHost, st));

@@ -7,6 +7,8 @@
 #pragma once
 #include "wd_ops.hpp"
 
+#include <cstdint>
+#include <cstring>
 #include <unordered_map>
 
 namespace wd {
@@ -58,6 +60,45 @@ public:
         double v = 0.0;
         return wd_gguf_meta_number(g_, key.c_str(), &v) == WD_OK ? v : fallback;
     }
+    // src/gguf.hpp:334-339: an unsigned scalar (a signed one when it is not negative), an exception otherwise
+    uint64_t uint_meta(const std::string &key) const {
+        double v = 0.0;
+        if (wd_gguf_meta_number(g_, key.c_str(), &v) != WD_OK || v < 0.0 || v != static_cast<double>(static_cast<uint64_t>(v)))
+            throw std::runtime_error("GGUF metadata is not an unsigned integer: " + key);
+        return static_cast<uint64_t>(v);
+    }
+    // src/gguf.hpp:358-402: integer arrays convert between signed and unsigned when every value fits, float arrays are
+    // numbers only; a missing key or an array of another kind throws.
+    std::vector<uint64_t> uint_array_meta(const std::string &key) const {
+        std::vector<uint64_t> out;
+        read_array(key, false, [&](int kind, uint64_t u, int64_t i, double) {
+            if (kind == 1 && i < 0) throw std::runtime_error("GGUF metadata array holds a negative value: " + key);
+            out.push_back(kind == 0 ? u : static_cast<uint64_t>(i));
+        });
+        return out;
+    }
+    std::vector<int64_t> int_array_meta(const std::string &key) const {
+        std::vector<int64_t> out;
+        read_array(key, false, [&](int kind, uint64_t u, int64_t i, double) {
+            if (kind == 0 && u > static_cast<uint64_t>(INT64_MAX)) throw std::runtime_error("GGUF metadata array value does not fit int64: " + key);
+            out.push_back(kind == 0 ? static_cast<int64_t>(u) : i);
+        });
+        return out;
+    }
+    std::vector<double> number_array_meta(const std::string &key) const {
+        std::vector<double> out;
+        read_array(key, true, [&](int kind, uint64_t u, int64_t i, double f) {
+            out.push_back(kind == 0 ? static_cast<double>(u) : (kind == 1 ? static_cast<double>(i) : f));
+        });
+        return out;
+    }
+    bool has_meta(const std::string &key) const {
+        double v;
+        uint32_t et;
+        const void *p;
+        return wd_gguf_meta_number(g_, key.c_str(), &v) == WD_OK || wd_gguf_meta_string(g_, key.c_str()) != nullptr ||
+               wd_gguf_meta_array(g_, key.c_str(), &et, &p) >= 0;
+    }
     // The read-only mapping of the whole file and its descriptor, for readers that bypass the mapping.
     const uint8_t *map_base() const { return wd_gguf_map_base(g_); }
     size_t map_bytes() const { return wd_gguf_map_bytes(g_); }
@@ -68,6 +109,38 @@ public:
     }
 
 private:
+    // Walks an array of fixed-size elements: f(kind, u, i, d) with kind 0 unsigned (and bool), 1 signed, 2 float.
+    template <typename F>
+    void read_array(const std::string &key, bool floats_allowed, F &&f) const {
+        uint32_t et = 0;
+        const void *p = nullptr;
+        const long long n = wd_gguf_meta_array(g_, key.c_str(), &et, &p);
+        if (n < 0) throw std::runtime_error("GGUF metadata array not found: " + key);
+        const uint8_t *b = static_cast<const uint8_t *>(p);
+        auto get = [&](auto tag, long long at) {
+            decltype(tag) v;
+            std::memcpy(&v, b + static_cast<size_t>(at) * sizeof(v), sizeof(v));
+            return v;
+        };
+        for (long long at = 0; at < n; ++at) {
+            switch (et) {
+                case 0: case 7: f(0, get(uint8_t{}, at), 0, 0.0); break;
+                case 1: f(1, 0, get(int8_t{}, at), 0.0); break;
+                case 2: f(0, get(uint16_t{}, at), 0, 0.0); break;
+                case 3: f(1, 0, get(int16_t{}, at), 0.0); break;
+                case 4: f(0, get(uint32_t{}, at), 0, 0.0); break;
+                case 5: f(1, 0, get(int32_t{}, at), 0.0); break;
+                case 10: f(0, get(uint64_t{}, at), 0, 0.0); break;
+                case 11: f(1, 0, get(int64_t{}, at), 0.0); break;
+                case 6: case 12:
+                    if (!floats_allowed) throw std::runtime_error("GGUF metadata array is not an integer array: " + key);
+                    f(2, 0, 0, et == 6 ? static_cast<double>(get(float{}, at)) : get(double{}, at));
+                    break;
+                default: throw std::runtime_error("GGUF metadata array of an unsupported element type: " + key);
+            }
+        }
+    }
+
     wd_gguf *g_ = nullptr;
     std::vector<TensorInfo> tensors_;
     std::unordered_map<std::string, size_t> index_;

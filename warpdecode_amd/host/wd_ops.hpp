@@ -34,6 +34,7 @@ enum class GgmlType : uint32_t {
     IQ4_NL = 20,
     IQ3_S = 21,
     IQ2_S = 22,
+    BF16 = 30,
 };
 
 inline void check(int rc, const char *what) {
@@ -56,7 +57,7 @@ struct TensorInfo {
     size_t byte_size() const {
         const uint64_t n = elements();
         if (type == GgmlType::F32) return static_cast<size_t>(n * 4);
-        if (type == GgmlType::F16) return static_cast<size_t>(n * 2);
+        if (type == GgmlType::F16 || type == GgmlType::BF16) return static_cast<size_t>(n * 2);
         const uint64_t cols = dims.empty() ? 0 : dims[0];
         const size_t row = wd_row_bytes(static_cast<int>(type), static_cast<int>(cols));
         if (row == 0 || cols == 0) throw std::runtime_error("tensor size is not a whole number of blocks, or unsupported type: " + name);
@@ -242,8 +243,9 @@ public:
         check(wd_moe_scratch_create(&s_, hidden, expert_ffn, n_experts, k), "MoE scratch allocation failed");
         n_experts_ = n_experts, k_ = k, hidden_ = hidden, expert_ffn_ = expert_ffn;
         void *p = nullptr;
-        check(wd_malloc_host(&p, sizeof(int) * k), "pinned allocation failed");
+        check(wd_malloc_host(&p, sizeof(int) * (k + 1)), "pinned allocation failed");  // [k] receives the status word
         h_ids_ = static_cast<int *>(p);
+        h_ids_[k] = 0;
         check(wd_malloc_host(&p, sizeof(float) * k), "pinned allocation failed");
         h_weights_ = static_cast<float *>(p);
     }
@@ -274,6 +276,17 @@ public:
     half_bits *rx_batch_q8_0_scales() const { return wd_moe_scratch_act_scales(s_); }
     float *rx_batch_down() const { return wd_moe_scratch_expert_out(s_); }
     int *h_ids() const { return h_ids_; }
+    // The scratch's status word travels to the host with the next synchronisation of `stream`; afterwards
+    // throw_if_failed() reports a layer pass on this scratch whose results are invalid (a bounded wait that ran out,
+    // an expert that had no slot).
+    void queue_status_copy(Stream stream) {
+        check(wd_memcpy_d2h(h_ids_ + k_, wd_moe_scratch_status_word(s_), sizeof(int), stream), "status copy failed");
+    }
+    void throw_if_failed() const {
+        if (h_ids_[k_] == 1) throw std::runtime_error("MoE layer pass failed: a wait between its workgroups ran out");
+        if (h_ids_[k_] == 2) throw std::runtime_error("MoE layer pass failed: an expert without a cache slot was selected");
+        if (h_ids_[k_] != 0) throw std::runtime_error("MoE layer pass failed");
+    }
     float *h_weights() const { return h_weights_; }
     wd_moe_scratch *handle() const { return s_; }
 
@@ -581,6 +594,21 @@ inline void fill_routed(wd_moe_layer &L, int layer, const GpuMatrix &router, con
     L.slot_bytes = cache.slot_bytes(), L.slot_gate_bytes = cache.gate_bytes(), L.slot_up_bytes = cache.up_bytes();
     if (!L.slot_of_expert) throw std::runtime_error("MoE layer is outside the expert cache's layer range");
 }
+// The layer pass for a layer whose experts are not all in the slot pool: dispatch A (router, selection, the shared
+// expert's first half), the ids to the host, the cache acquires them, then the routed dispatches on that selection.
+// The wait for the ids is also where a failure recorded by an earlier pass on this scratch surfaces.
+inline void routed_through_host(const wd_moe_layer &L, int layer, const float *x, const TensorInfo &gate, const TensorInfo &up,
+                                const TensorInfo &down, GpuExpertCache &cache, Qwen38MoeScratch &scratch, float *dst, bool run_a,
+                                Stream stream) {
+    if (run_a) check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), WD_MOE_ONLY_A, stream), "MoE router failed");
+    check(wd_memcpy_d2h(scratch.h_ids(), scratch.d_ids(), sizeof(int) * L.top_k, stream), "routed ids copy failed");
+    scratch.queue_status_copy(stream);
+    check(wd_stream_sync(stream), "stream synchronisation failed");
+    scratch.throw_if_failed();
+    cache.register_layer_experts(layer, gate, up, down);
+    cache.acquire_ids(layer, scratch.h_ids(), L.top_k, stream);
+    check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), WD_MOE_PRESELECTED | WD_MOE_ONLY_B | WD_MOE_ONLY_C, stream), "MoE experts failed");
+}
 }  // namespace detail
 
 // Routed experts of one layer: router -> top-k -> (host ids, cache acquire) -> grouped gate/up -> SwiGLU ->
@@ -598,12 +626,7 @@ inline void run_qwen38_routed_moe_separate_f32_x(int layer, const float *x, cons
         check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), preselected ? WD_MOE_PRESELECTED : 0u, stream), "MoE layer failed");
         return;
     }
-    if (!preselected) check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), WD_MOE_ONLY_A, stream), "MoE router failed");
-    check(wd_memcpy_d2h(scratch.h_ids(), scratch.d_ids(), sizeof(int) * L.top_k, stream), "routed ids copy failed");
-    check(wd_stream_sync(stream), "stream synchronisation failed");
-    cache.register_layer_experts(layer, gate_exps, up_exps, down_exps);
-    cache.acquire_ids(layer, scratch.h_ids(), L.top_k, stream);
-    check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), WD_MOE_PRESELECTED | WD_MOE_ONLY_B | WD_MOE_ONLY_C, stream), "MoE experts failed");
+    detail::routed_through_host(L, layer, x, gate_exps, up_exps, down_exps, cache, scratch, dst, !preselected, stream);
 }
 
 // The same with the gate and up projections stored as one tensor of 2 * ffn rows per expert
@@ -657,6 +680,10 @@ inline void run_qwen38_moe_layer_f32_x(int layer, const float *x, const GpuMatri
     detail::fill_routed(L, layer, router, gate_exps, up_exps, down_exps, cache, scratch, expert_scale);
     L.shared_gate_inp = shared.gate_input_f32.data;
     L.shared_gate = shared.gate.data, L.shared_up = shared.up.data, L.shared_down = shared.down.data;
+    if (!cache.layer_resident(layer)) {  // the device cannot resolve every selection by itself: the ids go through the host
+        detail::routed_through_host(L, layer, x, gate_exps, up_exps, down_exps, cache, scratch, out, true, stream);
+        return;
+    }
     check(wd_moe_layer_f32(&L, x, out, scratch.handle(), 0u, stream), "MoE layer failed");
 }
 
@@ -687,8 +714,10 @@ inline void run_qwen38_moe_tokens_f32_x(int layer, const float *x, int tokens, c
         check(wd_moe_layer_f32(&L, x + static_cast<size_t>(t) * H, out + static_cast<size_t>(t) * H, handles[t], WD_MOE_ONLY_A, stream),
               "MoE router failed");
         check(wd_memcpy_d2h(scratch[t]->h_ids(), scratch[t]->d_ids(), sizeof(int) * k, stream), "routed ids copy failed");
+        scratch[t]->queue_status_copy(stream);
     }
     check(wd_stream_sync(stream), "stream synchronisation failed");
+    for (const Qwen38MoeScratch *s : scratch) s->throw_if_failed();
     std::vector<int> unique;
     for (int t = 0; t < tokens; ++t)
         for (int j = 0; j < k; ++j) {
@@ -754,6 +783,11 @@ inline void run_qwen38_moe_layer_hc_f32_x(int layer, const float *x, const GpuMa
     detail::fill_routed(L, layer, router, gate_exps, up_exps, down_exps, cache, scratch, expert_scale);
     L.shared_gate_inp = shared.gate_input_f32.data;
     L.shared_gate = shared.gate.data, L.shared_up = shared.up.data, L.shared_down = shared.down.data;
+    if (!cache.layer_resident(layer)) {  // the ids go through the host, the combine runs as a call of its own
+        detail::routed_through_host(L, layer, x, gate_exps, up_exps, down_exps, cache, scratch, out, true, stream);
+        run_qwen38_hc_combine_f32_block_f32_inject(residual, out, hc, stream, round_half);
+        return;
+    }
     check(wd_moe_layer_hc_f32(&L, x, out, residual, hc.inject(), hc.hc(), round_half ? 1 : 0, scratch.handle(), 0u, stream),
           "MoE layer with combine failed");
 }
