@@ -68,7 +68,7 @@ def parse():
                     help="resident mode: the stack as ONE launch of resident workgroups (default), or two dispatches per layer")
     ap.add_argument("--repeats", type=int, default=5, help="further repeats of the timed region, for the spread in the JSON line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-seconds", type=float, default=6.0,
+    ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="wall-clock seconds of CPU layer passes to accumulate for cpu_baseline (all host threads busy)")
     ap.add_argument("--check", action="store_true", help="verify one layer pass against the CPU oracle first")
     return ap.parse_args()
@@ -133,21 +133,58 @@ def layer_dict(torch, synth, t, n_experts):
     return L
 
 
-def cpu_child(seconds, threads, kind):
-    """Child process of the cpu_baseline leg: no GPU.  Times C2 layer passes of the reference CPU MoE
-    path (its run_layer + thread pool for the routed experts, its Q8_0 row kernels for the shared
-    expert; router through the C port) or of the C port alone, and prints one progress line per pass."""
+CPU_LAYERS, CPU_EXPERTS = 4, 512      # 4 x 1.03 GB of weights: far beyond any last-level cache
+
+
+def cpu_weights(folder):
+    """Writes the cpu_baseline leg's weights as .npy files that its children map: 128 experts generated like the GPU
+    workload's, every layer made of those blocks four times over in an order of its own (1.03 GB of distinct memory
+    per layer), with small tensors of its own."""
+    from warpdecode_amd import synth
+    made = 128
+    base = synth.make_c2(layer=0, n_experts=made)
+    rng = synth.rng_for(synth.BASE_SEED, 9003)
+    for l in range(CPU_LAYERS):
+        order = rng.permutation(np.tile(np.arange(made), CPU_EXPERTS // made))
+        small = base if l == 0 else synth.make_c2(layer=l, n_experts=8)
+        for name, a in base.items():
+            if not isinstance(a, np.ndarray):
+                continue
+            if name in ("gate", "up", "down", "router"):
+                a = a.reshape(made, -1)[order].reshape((CPU_EXPERTS,) + a.shape[1:])
+            elif l > 0:
+                a = small[name]
+            np.save(os.path.join(folder, "%d.%s.npy" % (l, name)), a)
+
+
+def cpu_child(seconds, threads, kind, folder):
+    """Child process of the cpu_baseline leg: no GPU.  Times layer passes of the headline workload's shape (512
+    experts per layer, ids Zipf(1.1) over a permutation of its own per layer, 4 layers' weights taken in turn) in the
+    C port of the layer, or in the reference CPU MoE path (its run_layer + thread pool for the routed experts, its
+    Q8_0 row kernels for the shared expert; router through the C port), and prints one progress line per pass."""
     from oracle import pyoracle
     from warpdecode_amd import synth
-    n_exp = 64
-    layers = [synth.make_c2(layer=l, n_experts=n_exp) for l in range(2)]       # 2 x 129 MB of expert bytes
+    proto = synth.make_c2(layer=0, n_experts=8)
+    layers = []
+    for l in range(CPU_LAYERS):
+        L = {k: v for k, v in proto.items() if not isinstance(v, np.ndarray)}
+        L["n_experts"] = CPU_EXPERTS
+        for name, a in proto.items():
+            if isinstance(a, np.ndarray):
+                L[name] = np.load(os.path.join(folder, "%d.%s.npy" % (l, name)), mmap_mode="r")
+        layers.append(L)
     rng = synth.rng_for(synth.BASE_SEED, 9002)
+    perms = [rng.permutation(CPU_EXPERTS) for _ in range(CPU_LAYERS)]
     x = synth.rms_normed(rng, 2048)
+    for L in layers:                      # fault the mappings in before the clock starts
+        for name in ("gate", "up", "down", "router"):
+            np.add.reduce(L[name].reshape(-1)[::4096], dtype=np.uint64 if L[name].dtype == np.uint8 else None)
     print("READY", flush=True)
     passes, t0 = 0, time.perf_counter()
     while True:
-        L = layers[passes % 2]
-        ids = synth.zipf_ids(rng, n_exp, 10, 1.1)
+        l = passes % CPU_LAYERS
+        L = layers[l]
+        ids = synth.zipf_ids(rng, CPU_EXPERTS, 10, 1.1, perms[l])
         logits = pyoracle.router_logits(L["router"], x)
         _, wts = pyoracle.route(logits, 10)
         if kind == "reference":
@@ -164,56 +201,80 @@ def cpu_child(seconds, threads, kind):
             break
 
 
-def cpu_baseline(seconds):
-    """Runs cpu_child in a subprocess under a watchdog (the reference's fork-join pool can dead-lock
-    when a late worker picks up a task of the next parallel_for; a stalled child is killed and the
-    passes it completed are used) and converts ms/layer to tokens/s of a 48-layer stack."""
+def cpu_leg(kind, seconds, threads, folder, max_children):
+    """Runs cpu_child as fresh child processes until `seconds` of timed passes have accumulated (or the children run
+    out).  A child that prints nothing for 2.5 s after its first pass has stalled (the reference's fork-join pool can
+    dead-lock when a late worker picks up a task of the next parallel_for): it is killed, the passes it completed
+    count, and a fresh child continues.  Returns (passes, seconds, stalled children)."""
     import subprocess
     import threading
+    tot_passes, tot_time, stalls = 0, 0.0, 0
+    for _ in range(max_children):
+        remaining = seconds - tot_time
+        if remaining <= 0.5:
+            break
+        proc = subprocess.Popen([sys.executable, os.path.abspath(__file__), "--cpu-child", str(remaining), str(threads), kind, folder],
+                                stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True)
+        last = [0, 0.0, time.perf_counter()]
+
+        def reader():
+            for line in proc.stdout:
+                f = line.split()
+                if f and f[0] == "P":
+                    last[0], last[1] = int(f[1]), float(f[2])
+                last[2] = time.perf_counter()
+
+        th = threading.Thread(target=reader, daemon=True)
+        th.start()
+        while proc.poll() is None:
+            time.sleep(0.25)
+            # a pass takes milliseconds; only the start-up (mapping 4 GB of weights) is slow
+            if time.perf_counter() - last[2] > (90.0 if last[0] == 0 else 2.5):
+                stalls += 1
+                proc.kill()
+                break
+        proc.wait()
+        th.join(timeout=5)
+        tot_passes += last[0]
+        tot_time += last[1]
+    return tot_passes, tot_time, stalls
+
+
+def cpu_baseline(seconds):
+    """The layer pass on the host cores, on the headline workload's shape: the C port (one child, no restarts) is the
+    figure reported; the reference's own CPU path is reported beside it with the number of children that stalled.
+    ms/layer is converted to tokens/s of a 48-layer stack."""
+    import shutil
+    import tempfile
     from oracle import pyoracle
     cpus = len(os.sched_getaffinity(0))
     threads = max(1, min(cpus, 16))
-    kinds = (["reference"] if pyoracle.ref() is not None else []) + ["port"]
-    for kind in kinds:
-        tot_passes, tot_time, stalls = 0, 0.0, 0
-        for attempt in range(40):
-            remaining = seconds - tot_time
-            if remaining <= 0.5:
-                break
-            proc = subprocess.Popen([sys.executable, os.path.abspath(__file__), "--cpu-child", str(remaining), str(threads), kind],
-                                    stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True)
-            last = [0, 0.0, time.perf_counter()]
-
-            def reader():
-                for line in proc.stdout:
-                    f = line.split()
-                    if f and f[0] == "P":
-                        last[0], last[1] = int(f[1]), float(f[2])
-                    last[2] = time.perf_counter()
-
-            th = threading.Thread(target=reader, daemon=True)
-            th.start()
-            while proc.poll() is None:
-                time.sleep(0.25)
-                # a pass takes milliseconds; only the start-up (weight generation) is slow
-                if time.perf_counter() - last[2] > (60.0 if last[0] == 0 else 2.5):
-                    stalls += 1
-                    proc.kill()
-                    break
-            th.join(timeout=5)
-            tot_passes += last[0]
-            tot_time += last[1]
-        note("cpu baseline (%s): %d passes in %.1f s, %d stalled children" % (kind, tot_passes, tot_time, stalls))
-        if tot_passes >= 8:
-            per_layer = tot_time / tot_passes
-            return dict(value=round(1.0 / (per_layer * 48), 3), unit="tok/s", cores=threads, kind=kind,
-                        sample="%d C2 layer passes (512-expert layer shape, ids Zipf(1.1) over 64 resident experts, "
-                               "2 layers' weights alternating) in %.1f s = %.2f ms/layer, x48 layers per token; "
-                               "%d threads on %d host cores%s"
-                               % (tot_passes, tot_time, per_layer * 1e3, threads, cpus,
-                                  ("; the reference thread pool dead-locked %d times, each time the child was "
-                                   "restarted and only completed passes are counted" % stalls) if stalls else ""))
-    return dict(value=None, unit="tok/s", cores=threads, kind="port", sample="no CPU pass completed")
+    folder = tempfile.mkdtemp(prefix="wd_cpu_", dir="/dev/shm" if os.path.isdir("/dev/shm") else None)
+    workload = ("layer passes of the headline shape (hidden 2048, ffn 512, top-10 of %d experts + shared expert, ids "
+                "Zipf(1.1) over a per-layer permutation, %d layers = %.1f GB of weights taken in turn)"
+                % (CPU_EXPERTS, CPU_LAYERS, CPU_LAYERS * 1.039))
+    try:
+        note("cpu baseline: writing %d layers of weights to %s" % (CPU_LAYERS, folder))
+        cpu_weights(folder)
+        passes, secs, stalls = cpu_leg("port", seconds, threads, folder, 1)
+        note("cpu baseline (port): %d passes in %.1f s, %d stalled children" % (passes, secs, stalls))
+        if passes < 8:
+            return dict(value=None, unit="tok/s", cores=threads, kind="port", sample="no CPU pass completed")
+        per_layer = secs / passes
+        out = dict(value=round(1.0 / (per_layer * 48), 3), unit="tok/s", cores=threads, kind="port",
+                   sample="%d %s in %.1f s = %.2f ms/layer, x48 layers per token; %d threads on %d host cores, one "
+                          "child process, no restarts" % (passes, workload, secs, per_layer * 1e3, threads, cpus))
+        if pyoracle.ref() is not None:
+            passes, secs, stalls = cpu_leg("reference", seconds, threads, folder, 12)
+            note("cpu baseline (reference): %d passes in %.1f s, %d stalled children" % (passes, secs, stalls))
+            ref = dict(value=round(passes / (secs * 48), 3) if passes >= 8 else None, unit="tok/s", cores=threads,
+                       passes=passes, seconds=round(secs, 2), stalled_children=stalls,
+                       sample="the reference's own CPU MoE path on the same workload; a child whose thread pool "
+                              "dead-locked was killed and replaced by a fresh one, only completed passes count")
+            out["reference"] = ref
+        return out
+    finally:
+        shutil.rmtree(folder, ignore_errors=True)
 
 
 def recorded_traffic(kernel):
@@ -759,8 +820,8 @@ def bench_tokens(args, torch, capi, synth):
 
 
 def main():
-    if len(sys.argv) >= 5 and sys.argv[1] == "--cpu-child":
-        cpu_child(float(sys.argv[2]), int(sys.argv[3]), sys.argv[4])
+    if len(sys.argv) >= 6 and sys.argv[1] == "--cpu-child":
+        cpu_child(float(sys.argv[2]), int(sys.argv[3]), sys.argv[4], sys.argv[5])
         return
     args = parse()
     if args.gpus != 1:
