@@ -74,10 +74,15 @@ constexpr unsigned kRecBytes = 128;       //   logit of row r, word 1 the shared
 // share an L2), laid out contiguously: the consumers of a group fetch their copy with coalesced requests, and a line is
 // polled from one L2 only.
 constexpr int kResCopies = 8;
-constexpr unsigned kHandXc = kHandRec + kRecBytes * kResMaxLayers * kResWgs;           // f32 [layers][copies][2048] layer inputs
+#ifndef WD_RES_XSTRIDE
+#define WD_RES_XSTRIDE 16
+#endif
+constexpr unsigned kXcStride = WD_RES_XSTRIDE;  // bytes from one workgroup's four values of a layer input to the next one's
+constexpr unsigned kXcBytes = kXcStride * kResWgs;                                     // one copy
+constexpr unsigned kHandXc = kHandRec + kRecBytes * kResMaxLayers * kResWgs;           // [layers][copies][512] pieces of four f32: layer inputs
 constexpr unsigned kAcRec = 48;                                                        // bytes of a workgroup's activations: slots 0..10, a zero
 constexpr unsigned kAcBytes = kAcRec * kResWgs;                                        // 24 KB per copy
-constexpr unsigned kHandAc = kHandXc + 4u * kResMaxLayers * kResCopies * kResH;        // f32 [layers][copies][512][12] activations
+constexpr unsigned kHandAc = kHandXc + kXcBytes * kResMaxLayers * kResCopies;        // f32 [layers][copies][512][12] activations
 constexpr unsigned kHandIdh = kHandAc + kAcBytes * kResMaxLayers * kResCopies;         // u32 [layers][copies][16] selected ids
 constexpr unsigned kHandWh = kHandIdh + 4u * kResMaxLayers * kResIdCopies * 16;  // u32 [layers][16] router weights, [15] the shared gate
 constexpr unsigned kHandSet = kHandWh + 4u * kResMaxLayers * 16;             // bytes of one set of hand-off buffers
@@ -87,7 +92,7 @@ constexpr unsigned kHandEpoch = 2u * kHandSet;
 constexpr unsigned kHandBytes = kHandEpoch + 256u;
 static_assert(kHandXc % 128 == 0 && kHandAc % 128 == 0 && kHandIdh % 128 == 0 && kHandWh % 16 == 0 && kHandSet % 128 == 0, "hand-off block alignment");
 WD_DEV unsigned rec_off(int l, int wg) { return kHandRec + static_cast<unsigned>(l * kResWgs + wg) * kRecBytes; }
-WD_DEV unsigned xc_off(int l, int copy) { return kHandXc + static_cast<unsigned>(l * kResCopies + copy) * (4u * kResH); }
+WD_DEV unsigned xc_off(int l, int copy) { return kHandXc + static_cast<unsigned>(l * kResCopies + copy) * kXcBytes; }
 WD_DEV unsigned ac_off(int l, int copy) { return kHandAc + static_cast<unsigned>(l * kResCopies + copy) * kAcBytes; }
 
 struct ResidentArgs {
@@ -111,15 +116,16 @@ struct ResidentArgs {
 // ---- device-scope access to the hand-off buffers ------------------------------------------------------------
 typedef unsigned wd_u4v __attribute__((ext_vector_type(4)));
 constexpr int kAuxDevice = 16;  // sc1: the access is coherent across the device's L2 caches
+constexpr int kAuxPoll = static_cast<int>(0x80000010u);  // the same, volatile: two polls of one address are two requests
 WD_DEV __amdgpu_buffer_rsrc_t hand_rsrc(const void *p, unsigned bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, static_cast<int>(bytes), 0x00020000);
 }
 WD_DEV uint4 hand_load16(__amdgpu_buffer_rsrc_t rs, unsigned off) {
-    const wd_u4v v = __builtin_amdgcn_raw_buffer_load_b128(rs, static_cast<int>(off), 0, kAuxDevice);
+    const wd_u4v v = __builtin_amdgcn_raw_buffer_load_b128(rs, static_cast<int>(off), 0, kAuxPoll);
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 WD_DEV uint32_t hand_load4(__amdgpu_buffer_rsrc_t rs, unsigned off) {
-    return __builtin_amdgcn_raw_buffer_load_b32(rs, static_cast<int>(off), 0, kAuxDevice);
+    return __builtin_amdgcn_raw_buffer_load_b32(rs, static_cast<int>(off), 0, kAuxPoll);
 }
 WD_DEV void hand_store16(__amdgpu_buffer_rsrc_t rs, unsigned off, uint4 v) {
     const wd_u4v w = {v.x, v.y, v.z, v.w};
@@ -146,8 +152,97 @@ WD_DEV bool res_full(const uint4 &v) { return v.x != kResEmpty && v.y != kResEmp
 
 // N 16-byte pieces per lane (lanes with on == false take no part): returns when every word of every piece has been
 // written.  Only pieces that are still incomplete are requested again.
+// WD_RES_PIPE16 / WD_RES_PIPE4 > 1: that many polls are kept in flight.  A poll that has to travel to memory and back
+// before the next one is issued notices a value up to one round trip late; several polls under way notice it within the
+// interval at which they were issued.
+#ifndef WD_RES_PIPE16
+#define WD_RES_PIPE16 1
+#endif
+#ifndef WD_RES_PIPE4
+#define WD_RES_PIPE4 1
+#endif
+#ifndef WD_RES_PIPE16_MAXN
+#define WD_RES_PIPE16_MAXN 1
+#endif
+template <int N, int D>
+WD_DEV void hand_wait16_piped(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, const unsigned (&off)[N], const bool (&on)[N], uint4 (&v)[N], bool &dead) {
+    static_assert(D == 2, "two polls in flight");
+    bool need[N];
+    uint4 p0[N], p1[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        need[i] = on[i];
+        v[i] = p0[i] = p1[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
+    if (dead) return;
+    auto issue = [&](uint4 (&p)[N]) {
+#pragma unroll
+        for (int i = 0; i < N; ++i)
+            if (need[i]) p[i] = hand_load16(rs, off[i]);
+    };
+    auto arrived = [&](const uint4 (&p)[N]) {  // true when nothing is missing any more (or the wait is given up)
+        bool any = false;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            if (need[i]) {
+                v[i] = p[i];
+                need[i] = !res_full(v[i]);
+            }
+            any = any || need[i];
+        }
+        return __builtin_amdgcn_ballot_w64(any) == 0ull;
+    };
+    issue(p0);
+    __builtin_amdgcn_s_sleep(WD_RES_SLEEP16);
+    issue(p1);
+    unsigned spins = 0;
+    for (;;) {
+        if (arrived(p0) || res_give_up(a, spins, dead)) return;
+        issue(p0);
+        __builtin_amdgcn_s_sleep(WD_RES_SLEEP16);
+        if (arrived(p1) || res_give_up(a, spins, dead)) return;
+        issue(p1);
+        __builtin_amdgcn_s_sleep(WD_RES_SLEEP16);
+    }
+}
+template <int D>
+WD_DEV uint32_t hand_wait4_piped(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, unsigned off, bool on, bool &dead) {
+    uint32_t v = 0u;
+    if (dead) return v;
+    bool need = on;
+    uint32_t s[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        s[d] = 0u;
+        if (need) s[d] = hand_load4(rs, off);
+        if (d + 1 < D) __builtin_amdgcn_s_sleep(WD_RES_SLEEP4);
+    }
+    unsigned spins = 0;
+    bool done = false;
+    while (!done) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            if (!done) {
+                if (need) {
+                    v = s[d];
+                    need = v == kResEmpty;
+                }
+                done = __builtin_amdgcn_ballot_w64(need) == 0ull || res_give_up(a, spins, dead);
+                if (!done) {
+                    if (need) s[d] = hand_load4(rs, off);
+                    __builtin_amdgcn_s_sleep(WD_RES_SLEEP4);
+                }
+            }
+        }
+    }
+    return v;
+}
 template <int N>
 WD_DEV void hand_wait16(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, const unsigned (&off)[N], const bool (&on)[N], uint4 (&v)[N], bool &dead) {
+    if constexpr (WD_RES_PIPE16 > 1 && N <= WD_RES_PIPE16_MAXN) {
+        hand_wait16_piped<N, WD_RES_PIPE16>(a, rs, off, on, v, dead);
+        return;
+    }
     bool need[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) {
@@ -180,6 +275,7 @@ WD_DEV void hand_wait16(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, const 
 }
 // One word per lane.
 WD_DEV uint32_t hand_wait4(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, unsigned off, bool on, bool &dead) {
+    if constexpr (WD_RES_PIPE4 > 1) return hand_wait4_piped<WD_RES_PIPE4>(a, rs, off, on, dead);
     uint32_t v = 0u;
     if (dead) return v;
     bool need = on;
@@ -386,7 +482,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                 // (the other waves of the workgroup come here while rung 0 still folds the previous layer: nothing
                 // can have arrived yet)
                 if (rung != 0 && WD_RES_XDELAY) __builtin_amdgcn_s_sleep(WD_RES_XDELAY);
-                const unsigned off[1] = {xc_off(l, r & (kResCopies - 1)) + 16u * i};
+                const unsigned off[1] = {xc_off(l, r & (kResCopies - 1)) + kXcStride * i};
                 uint4 v[1];
                 hand_wait16<1>(a, c.hb, off, true, v, dead);
                 xv = make_float4(bits_f(v[0].x), bits_f(v[0].y), bits_f(v[0].z), bits_f(v[0].w));
@@ -428,6 +524,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             const int32_t *ids_given = a.ids_trace ? a.ids_trace + l * a.k : nullptr;
             int id_given = 0;
             if (ids_given && wave == 0 && lane < a.k) id_given = ids_given[lane];
+            const float w_scale = *const_cast<const volatile float *>(&L->w_scale);  // (asked for ahead of the logits)
             float lv[1] = {-INFINITY};
             const int id = wave * 64 + lane;
             if (wave < 8) {
@@ -442,7 +539,6 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             __syncthreads();
             res_mark(a, c, l, 13);
             if (wave == 0) {
-                const float w_scale = *const_cast<const volatile float *>(&L->w_scale);
                 topk_block_step3<1>(a.E, a.k, w_scale, lds_ids, lds_w, ids_given != nullptr, id_given, s, lane, nullptr,
                                     reinterpret_cast<uint32_t *>(a.hand + set_base + kHandIdh) + static_cast<size_t>(l) * kResIdCopies * 16, kResIdCopies);
                 res_mark(a, c, l, 14);
@@ -483,14 +579,20 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             act = silu_ggml(gu[0]) * gu[1];
             res_mark(a, c, l, 5);
         }
+        // rung 0 folds the results with the router's weights and the shared expert's gate: published long before this
+        // point as a rule, so one request now, answered while the activations are exchanged, replaces a round trip
+        // between the down rows and the fold
+        const bool wlane = rung == 0 && (lane < a.k || (shared && lane == 16));
+        const unsigned woff = kHandWh + static_cast<unsigned>((l * 16 + (lane == 16 ? kResGateSlot : lane)) * 4);
+        uint32_t wbits = kResEmpty;
+        if (wlane && !dead) wbits = hand_load4(c.hb, woff);
         float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
         res_exchange(a, c, l, on, act, v0, v1, dead);
         if (on) res_down(a, c, l, draw, v0, v1);
-        // rung 0 folds the results; the router's weights and the gate it needs are fetched on this side of the barrier
         float wreg = 0.0f;
         if (rung == 0) {
-            const bool wlane = lane < a.k || (shared && lane == 16);
-            wreg = bits_f(hand_wait4(a, c.hb, kHandWh + static_cast<unsigned>((l * 16 + (lane == 16 ? kResGateSlot : lane)) * 4), wlane, dead));
+            if (__builtin_amdgcn_ballot_w64(wlane && wbits == kResEmpty) != 0ull) wbits = hand_wait4(a, c.hb, woff, wlane, dead);
+            wreg = wlane ? bits_f(wbits) : 0.0f;
         }
         __syncthreads();  // B5: the eleven results of rows 4r..4r+3 are in LDS
 
@@ -525,7 +627,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             } else {
                 const uint4 piece = make_uint4(f_bits(readlane_f(xn, 0)), f_bits(readlane_f(xn, 1)), f_bits(readlane_f(xn, 2)),
                                                f_bits(readlane_f(xn, 3)));
-                if (lane < kResCopies) hand_store16(c.hb, xc_off(l + 1, lane) + 16u * r, piece);
+                if (lane < kResCopies) hand_store16(c.hb, xc_off(l + 1, lane) + kXcStride * r, piece);
             }
             res_mark(a, c, l, 9);
         }
@@ -563,11 +665,11 @@ WD_DEV void res_shared_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         }
         float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
         res_exchange(a, c, l, a.shared != 0, act, v0, v1, dead);
-        if (a.shared) {
-            res_down(a, c, l, draw, v0, v1);
-            if (l + 1 < a.n_layers) fetch(a.layers + l + 1, r, lane);
-        }
+        if (a.shared) res_down(a, c, l, draw, v0, v1);
         __syncthreads();  // B5
+        // the next layer's rows, asked for on this side of the barrier: the fold of this layer must not wait for a
+        // wave that is busy issuing requests
+        if (a.shared && l + 1 < a.n_layers) fetch(a.layers + l + 1, r, lane);
     }
 }
 
@@ -595,7 +697,7 @@ WD_DEV void res_router_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             const uint4 empty4 = make_uint4(kResEmpty, kResEmpty, kResEmpty, kResEmpty);
             // 8 lanes the workgroup's record, 8 its 128 bytes of the layer's input copies, 24 its 384 bytes of the activations'
             const unsigned off = lane < 8 ? rec_off(ll, r) + 16u * lane
-                               : lane < 16 ? xc_off(ll, 0) + 16u * (8 * r + lane - 8) : ac_off(ll, 0) + 16u * (24 * r + lane - 16);
+                               : lane < 16 ? xc_off(ll, 0) + kXcStride * (8 * r + lane - 8) : ac_off(ll, 0) + 16u * (24 * r + lane - 16);
             if (lane < 40) hand_store16(ob, off, empty4);
             if (r == 0) {
                 hand_store16(ob, kHandIdh + static_cast<unsigned>(ll * kResIdCopies * 64 + 16 * lane), empty4);
