@@ -155,6 +155,9 @@ WD_DEV bool res_full(const uint4 &v) { return v.x != kResEmpty && v.y != kResEmp
 // WD_RES_PIPE16 / WD_RES_PIPE4 > 1: that many polls are kept in flight.  A poll that has to travel to memory and back
 // before the next one is issued notices a value up to one round trip late; several polls under way notice it within the
 // interval at which they were issued.
+#ifndef WD_RES_DOWN_AT
+#define WD_RES_DOWN_AT 0  // the down rows are requested 0: when the gate/up rows have arrived, 1: after the decode, 2: after the exchange
+#endif
 #ifndef WD_RES_PIPE16
 #define WD_RES_PIPE16 1
 #endif
@@ -539,7 +542,12 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             __syncthreads();
             res_mark(a, c, l, 13);
             if (wave == 0) {
-                topk_block_step3<1>(a.E, a.k, w_scale, lds_ids, lds_w, ids_given != nullptr, id_given, s, lane, nullptr,
+#ifdef WD_RES_SEL_STAMPS
+                unsigned long long *st3 = (a.trace && l == a.trace_layer && a.trace_wg == 0) ? a.trace + 11 * 16 + 5 : nullptr;
+#else
+                unsigned long long *st3 = nullptr;
+#endif
+                topk_block_step3<1>(a.E, a.k, w_scale, lds_ids, lds_w, ids_given != nullptr, id_given, s, lane, st3,
                                     reinterpret_cast<uint32_t *>(a.hand + set_base + kHandIdh) + static_cast<size_t>(l) * kResIdCopies * 16, kResIdCopies);
                 res_mark(a, c, l, 14);
                 wave_lds_fence();
@@ -559,6 +567,9 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         Q8CoalRaw<0, 16> draw;
         draw.u[0] = draw.u[1] = draw.u[2] = make_uint4(0u, 0u, 0u, 0u);
         float act = 0.0f;
+#if WD_RES_DOWN_AT != 0
+        uint32_t e_keep = 0;
+#endif
         if (on) {
             uint32_t e = hand_wait4(a, c.hb, kHandIdh + static_cast<unsigned>(((l * kResIdCopies + (r & (kResIdCopies - 1))) * 16 + rung) * 4), true, dead);
             e = __builtin_amdgcn_readfirstlane(e);
@@ -573,11 +584,18 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             iq_rows8_coal_park<TYPE, 2>(raw, lane, c.area());
             // the down rows are asked for once the gate/up rows are here: requested together, the down rows of the
             // waves served first would delay the gate/up rows of the others, which the whole grid waits for
+#if WD_RES_DOWN_AT == 0
             if (!(a.debug & 2)) draw = q8_rows4_coal_request<0, 16>(down_base + e * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
+#else
+            e_keep = e;
+#endif
             res_mark(a, c, l, 11);
             if (!(a.debug & 1)) iq_rows8_coal_dots<TYPE, 2>(tables, c.xq(), c.xd(), lane, gu, c.area());
             act = silu_ggml(gu[0]) * gu[1];
             res_mark(a, c, l, 5);
+#if WD_RES_DOWN_AT == 1
+            draw = q8_rows4_coal_request<0, 16>(down_base + e_keep * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
+#endif
         }
         // rung 0 folds the results with the router's weights and the shared expert's gate: published long before this
         // point as a rule, so one request now, answered while the activations are exchanged, replaces a round trip
@@ -588,6 +606,9 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         if (wlane && !dead) wbits = hand_load4(c.hb, woff);
         float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
         res_exchange(a, c, l, on, act, v0, v1, dead);
+#if WD_RES_DOWN_AT == 2
+        if (on) draw = q8_rows4_coal_request<0, 16>(down_base + e_keep * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
+#endif
         if (on) res_down(a, c, l, draw, v0, v1);
         float wreg = 0.0f;
         if (rung == 0) {
