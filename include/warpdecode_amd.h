@@ -78,6 +78,23 @@ int wd_device_sync(void);
 int wd_q8_k_quantize_f32(const float *d_x, int elements, int8_t *d_qs, float *d_scales, int16_t *d_bsums,
                          void *stream);
 int wd_q8_0_quantize_f32(const float *d_x, int elements, int8_t *d_qs, uint16_t *d_scales, void *stream);
+/* The same from half input, as the dense Q4_0 path quantises its activations (values widened to float, inv = 127 / amax,
+ * q = lrintf(v * inv) clamped to +-127, scale = half(amax / 127) by IEEE rounding).
+ *   reference: q8_0_quantize_half_kernel, src/warodecode.cu:1504-1520.  d_x: half bits, 8-byte aligned. */
+int wd_q8_0_quantize_f16(const uint16_t *d_x, int elements, int8_t *d_qs, uint16_t *d_scales, void *stream);
+/* Q8_1 activation of the reference's plain Q8_0 GEMV: d = amax / 127, q = roundf(x / d), scale = half(d).
+ *   reference: q8_1_quantize_f32_kernel, src/lowbit.cuh:287-308 (buffer: Q8_1Buffer, :251-285). */
+int wd_q8_1_quantize_f32(const float *d_x, int elements, int8_t *d_qs, uint16_t *d_scales, void *stream);
+/* y[r] = sum over the row's Q8_0 blocks in ascending order of (d_w * d_x) * (float)dot32 (three roundings per block).
+ *   reference: q8_0_q8_1_gemv_f32_kernel / launch_q8_0_gemv_q8_1_f32, src/lowbit.cuh:310-362.
+ * d_block_sums: NULL or int32 [rows][cols / 32], the exact integer sums. */
+int wd_gemv_q8_0_q8_1_f32(const uint8_t *d_w, int rows, int cols, const int8_t *d_qs, const uint16_t *d_scales, float *d_y,
+                          int32_t *d_block_sums, void *stream);
+/* Element-wise half <-> float (IEEE round-to-nearest-even on the way down, the reference's __float2half / __half2float):
+ * what a caller with half activations or half outputs puts around the F32 layer calls
+ * (reference: q38_moe_select_experts_input<__half>, q38_finish_moe, src/qwen38_moe.cuh:2384-2453). */
+int wd_convert_f16_to_f32(const uint16_t *d_src, float *d_dst, size_t n, void *stream);
+int wd_convert_f32_to_f16(const float *d_src, uint16_t *d_dst, size_t n, void *stream);
 
 /* ---- router ----------------------------------------------------------------
  * logits[r] = dot(w[r,:], x) in the 4x8-accumulator order of ggml_vec_dot_f32.

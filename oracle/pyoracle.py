@@ -71,6 +71,14 @@ def _load():
     lib.wdo_f32_to_f16.argtypes = [C.c_float]
     lib.wdo_quantize_q8_0.argtypes = [_f32p, C.c_int, _i8p, _u16p]
     lib.wdo_quantize_q8_K.argtypes = [_f32p, C.c_int, _i8p, _f32p, _i16p]
+    lib.wdo_f32_to_f16_rn.restype = C.c_uint16
+    lib.wdo_f32_to_f16_rn.argtypes = [C.c_float]
+    lib.wdo_quantize_q8_1.restype = None
+    lib.wdo_quantize_q8_1.argtypes = [_f32p, C.c_int, _i8p, _u16p]
+    lib.wdo_gemv_q8_0_q8_1.restype = None
+    lib.wdo_gemv_q8_0_q8_1.argtypes = [_u8p, C.c_int, C.c_int, _i8p, _u16p, _f32p, _i32p]
+    lib.wdo_quantize_q8_0_f16.restype = None
+    lib.wdo_quantize_q8_0_f16.argtypes = [_u16p, C.c_int, _i8p, _u16p]
     lib.wdo_gemv.argtypes = [C.c_int, _u8p, C.c_int, C.c_int, _i8p, C.c_void_p, _f32p, _i32p]
     lib.wdo_dequant_row.argtypes = [C.c_int, _u8p, C.c_int, _f32p]
     lib.wdo_gemv_q6_K.argtypes = [_u8p, C.c_int, C.c_int, _i8p, _f32p, _i16p, _f32p, _i32p]
@@ -152,6 +160,37 @@ def quantize_q8_0(x):
     qs = np.empty(n, np.int8)
     d = np.empty(n // 32, np.uint16)
     lib().wdo_quantize_q8_0(_ptr(x, _f32p), n, _ptr(qs, _i8p), _ptr(d, _u16p))
+    return qs, d
+
+
+def f32_to_f16_rn(vals):
+    """IEEE round-to-nearest-even float -> half bits."""
+    vals = np.asarray(vals, dtype=np.float32)
+    return np.array([lib().wdo_f32_to_f16_rn(float(v)) for v in vals.ravel()], dtype=np.uint16).reshape(vals.shape)
+
+
+def quantize_q8_1(x):
+    """src/lowbit.cuh:287-308: q = roundf(x / d), d = amax / 127, scale as half(d)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    qs, d = np.empty(x.size, np.int8), np.empty(x.size // 32, np.uint16)
+    lib().wdo_quantize_q8_1(_ptr(x, _f32p), x.size, _ptr(qs, _i8p), _ptr(d, _u16p))
+    return qs, d
+
+
+def gemv_q8_0_q8_1(w, rows, cols, qs, d):
+    """src/lowbit.cuh:310-341.  Returns (y f32[rows], block sums int32[rows][cols/32])."""
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    y, sums = np.empty(rows, np.float32), np.empty((rows, cols // 32), np.int32)
+    lib().wdo_gemv_q8_0_q8_1(_ptr(w, _u8p), rows, cols, _ptr(np.ascontiguousarray(qs, np.int8), _i8p),
+                             _ptr(np.ascontiguousarray(d, np.uint16), _u16p), _ptr(y, _f32p), _ptr(sums, _i32p))
+    return y, sums
+
+
+def quantize_q8_0_f16(x_bits):
+    """src/warodecode.cu:1504-1520: Q8_0 activation from half input (bits)."""
+    x_bits = np.ascontiguousarray(x_bits, dtype=np.uint16)
+    qs, d = np.empty(x_bits.size, np.int8), np.empty(x_bits.size // 32, np.uint16)
+    lib().wdo_quantize_q8_0_f16(_ptr(x_bits, _u16p), x_bits.size, _ptr(qs, _i8p), _ptr(d, _u16p))
     return qs, d
 
 

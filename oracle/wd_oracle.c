@@ -628,6 +628,69 @@ void wdo_round_half_n(const float *x, int n, float *out) {
     for (int i = 0; i < n; ++i) out[i] = wdo_round_half(x[i]);
 }
 
+/* IEEE round-to-nearest-even float -> half bits (the device's __float2half): the rounded value is representable, so
+ * the block-scale conversion above is exact on it (its flush of magnitudes below 2^-24 cannot apply). */
+uint16_t wdo_f32_to_f16_rn(float value) {
+    if (value != value) return 0x7e00u;
+    return wdo_f32_to_f16(wdo_round_half(value));
+}
+
+/* Q8_1 activation of the reference's plain Q8_0 GEMV (q8_1_quantize_f32_kernel, src/lowbit.cuh:287-308): per block of
+ * 32, d = amax / 127, q = roundf(x / d) (halves away from zero, a division - not a multiplication by the inverse),
+ * scale stored as half(d). */
+void wdo_quantize_q8_1(const float *x, int n, int8_t *qs, uint16_t *d) {
+    for (int b = 0; b < n / 32; ++b) {
+        const float *src = x + (size_t)b * 32;
+        float amax = 0.0f;
+        for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(src[i]));
+        const float scale = amax / 127.0f;
+        for (int i = 0; i < 32; ++i) qs[(size_t)b * 32 + i] = amax == 0.0f ? 0 : (int8_t)roundf(src[i] / scale);
+        d[b] = wdo_f32_to_f16_rn(scale);
+    }
+}
+
+/* y[row] = sum over the row's blocks, in ascending order, of (d_w * d_x) * (float)dot32 - one rounded multiply of the
+ * two scales, one of the product with the integer sum, one rounded add (q8_0_q8_1_gemv_f32_kernel,
+ * src/lowbit.cuh:310-341; the reference builds with --use_fast_math, which may fuse the last two: results there are
+ * defined up to that).  block_sums (optional): int32 [rows][cols / 32]. */
+void wdo_gemv_q8_0_q8_1(const uint8_t *w, int rows, int cols, const int8_t *qs, const uint16_t *d, float *y, int32_t *block_sums) {
+    const int nb = cols / 32;
+    for (int r = 0; r < rows; ++r) {
+        const uint8_t *row = w + (size_t)r * nb * 34;
+        float sum = 0.0f;
+        for (int b = 0; b < nb; ++b) {
+            const uint8_t *blk = row + (size_t)b * 34;
+            int dot = 0;
+            for (int i = 0; i < 32; ++i) dot += (int)(int8_t)blk[2 + i] * (int)qs[b * 32 + i];
+            if (block_sums) block_sums[(size_t)r * nb + b] = dot;
+            const float scale = half_at(blk) * wdo_f16_to_f32(d[b]);
+            const float prod = scale * (float)dot;
+            sum = sum + prod;
+        }
+        y[r] = sum;
+    }
+}
+
+/* Q8_0 activation from half input (q8_0_quantize_half_kernel, src/warodecode.cu:1504-1520): the values widened to
+ * float, inv = 127 / amax, q = lrintf(v * inv) clamped to +-127, scale = half(amax / 127) by IEEE rounding. */
+void wdo_quantize_q8_0_f16(const uint16_t *x, int n, int8_t *qs, uint16_t *d) {
+    for (int b = 0; b < n / 32; ++b) {
+        float v[32], amax = 0.0f;
+        for (int i = 0; i < 32; ++i) {
+            v[i] = wdo_f16_to_f32(x[(size_t)b * 32 + i]);
+            amax = fmaxf(amax, fabsf(v[i]));
+        }
+        const float inv = amax == 0.0f ? 0.0f : 127.0f / amax;
+        for (int i = 0; i < 32; ++i) {
+            long q = lrintf(v[i] * inv);
+            if (q > 127) q = 127;
+            if (q < -127) q = -127;
+            qs[(size_t)b * 32 + i] = (int8_t)q;
+        }
+        d[b] = wdo_f32_to_f16_rn(amax / 127.0f);
+    }
+}
+
 float wdo_moe_branch_f32(float routed, float shared, float gate) {
     const float weighted = shared * gate;
     return routed + weighted;

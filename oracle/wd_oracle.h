@@ -50,6 +50,12 @@ uint16_t wdo_f32_to_f16(float value);
 /* src/qwen38_cpu_moe.cuh:220-263.  n is a multiple of 32 / 256. */
 void wdo_quantize_q8_0(const float *x, int n, int8_t *qs, uint16_t *d);
 void wdo_quantize_q8_K(const float *x, int n, int8_t *qs, float *d, int16_t *bsums);
+/* The reference's plain Q8_0 x Q8_1 path (src/lowbit.cuh:287-362) and its half-input Q8_0 quantiser
+ * (src/warodecode.cu:1504-1520); wdo_f32_to_f16_rn is IEEE round-to-nearest-even (the device's __float2half). */
+uint16_t wdo_f32_to_f16_rn(float value);
+void wdo_quantize_q8_1(const float *x, int n, int8_t *qs, uint16_t *d);
+void wdo_gemv_q8_0_q8_1(const uint8_t *w, int rows, int cols, const int8_t *qs, const uint16_t *d, float *y, int32_t *block_sums);
+void wdo_quantize_q8_0_f16(const uint16_t *x, int n, int8_t *qs, uint16_t *d);
 
 /*
  * Row dots.  `partials` (may be NULL) receives the exact int32 chunk sums:

@@ -228,6 +228,18 @@ static void host_only_checks() {
     CHECK(throws([&] { GgufFile missing(path + ".nope"); }), "opening an absent file must throw");
     unlink(path.c_str());
 
+    // the slot pool's default size (src/qwen38_tuning.hpp:88-116 names 40 GB -> 22 GiB and 80 GB -> 52 GiB)
+    unsetenv("WARODECODE_EXPERT_CACHE_MIB");
+    CHECK(default_expert_cache_mib(size_t{40} << 30) == 22 * 1024 && default_expert_cache_mib(size_t{80} << 30) == 52 * 1024, "cache size rule");
+    CHECK(default_expert_cache_mib(size_t{8} << 30) == 512 && default_expert_cache_mib(size_t{288} << 30) == 64 * 1024, "cache size clamps");
+    setenv("WARODECODE_EXPERT_CACHE_MIB", "20000", 1);
+    CHECK(default_expert_cache_mib(size_t{80} << 30) == 20000, "cache size override");
+    unsetenv("WARODECODE_EXPERT_CACHE_MIB");
+    CHECK(default_expert_prefetch_depth(size_t{130} << 30) == 3 && default_expert_prefetch_depth(size_t{80} << 30) == 2 &&
+              default_expert_prefetch_depth(size_t{24} << 30) == 1, "read-ahead depth rule");
+    Q8_1Buffer q81;
+    CHECK(throws([&] { q81.initialize(33); }) && throws([&] { q81.initialize(0); }), "Q8_1 buffer needs a positive multiple of 32");
+
     // The reference's own files (copied as data) with the answers its tests check or print:
     // tests/gguf_parser_test.cpp:6-8 prints version, tensor count and data offset of tests/min.gguf (3, 1, 160: the
     // header ends at byte 134 and general.alignment is 32); tests/gguf_array_test.cpp:11-27 asserts the arrays of the
@@ -342,6 +354,32 @@ static void gpu_checks() {
         CHECK(throws([&] { launch_q6_k_gemv_q8_k_f32(w, nullptr, nullptr, nullptr, y.data, stream, 48); }), "threads must be a multiple of 32");
     }
 
+    {   // launch_q8_0_gemv_q8_1_f32 through Q8_1Buffer (src/lowbit.cuh:251-362)
+        const int R = 96;
+        Rng r(4242);
+        const std::vector<uint8_t> wq = random_blocks(r, WDO_Q8_0, R, H, 0.02f / 127.0f);
+        TensorInfo tw{"w", {static_cast<uint64_t>(H), static_cast<uint64_t>(R)}, GgmlType::Q8_0, 0, wq.data()};
+        LowBitMatrix w = upload_lowbit_matrix(tw);
+        const std::vector<float> x = rms_normed(r, H);
+        DeviceFloatArray dx(H), dy(R);
+        dx.upload(x.data(), H);
+        Q8_1Buffer buf;
+        buf.initialize(H);
+        CHECK(throws([&] { buf.initialize(H); }), "double initialisation of the Q8_1 buffer must throw");
+        launch_q8_0_gemv_q8_1_f32(w, dx.data, dy.data, buf, stream);
+        check(wd_stream_sync(stream), "sync");
+        std::vector<float> got(R), want(R);
+        dy.download(got.data());
+        std::vector<int8_t> q(H);
+        std::vector<uint16_t> d(H / 32);
+        wdo_quantize_q8_1(x.data(), H, q.data(), d.data());
+        wdo_gemv_q8_0_q8_1(wq.data(), R, H, q.data(), d.data(), want.data(), nullptr);
+        CHECK(same_bits(got.data(), want.data(), R), "launch_q8_0_gemv_q8_1_f32 differs from the oracle");
+        Q8_1Buffer small;
+        small.initialize(H / 2);
+        CHECK(throws([&] { launch_q8_0_gemv_q8_1_f32(w, dx.data, dy.data, small, stream); }), "a buffer smaller than the row must be refused");
+    }
+
     std::vector<GpuMatrix> routers;
     std::vector<Qwen38SharedExpertWeights> shared(layers);
     for (int l = 0; l < layers; ++l) {
@@ -391,6 +429,44 @@ static void gpu_checks() {
                 std::vector<float> acc(H);
                 check(wd_memcpy_d2h(acc.data(), scratch.d_accum(), sizeof(float) * H, nullptr), "accum");
                 CHECK(same_bits(acc.data(), routed.data(), H), "mode %d token %d layer %d: routed sum differs", mode, token, l);
+                if (token == 0) {
+                    // the runners by element type (src/qwen38_moe.cuh:3521-3534): half input, half output, the selected
+                    // experts' down outputs captured as half - against the oracle on the widened input
+                    std::vector<uint16_t> xh(H);
+                    std::vector<float> xw(H);
+                    for (int i = 0; i < H; ++i) xh[i] = wdo_f32_to_f16_rn(x[i]), xw[i] = wdo_f16_to_f32(xh[i]);
+                    DeviceArray<half_bits> dxh(H), dout_h(H);
+                    check(wd_memcpy_h2d(dxh.data, xh.data(), sizeof(uint16_t) * H, nullptr), "half input");
+                    std::vector<float> want_h(H), routed_h(H), eo(static_cast<size_t>(k) * H);
+                    wdo_dump dh{};
+                    dh.routed = routed_h.data(), dh.expert_out = eo.data();
+                    wdo_moe_layer(&L[l].o, xw.data(), want_h.data(), &dh, 0);
+                    run_qwen38_routed_moe_separate<true, half_bits, half_bits>(l, dxh.data, routers[l], L[l].t_gate, L[l].t_up, L[l].t_down, cache,
+                                                                              scratch, dout_h.data, 1.0f, stream, false, scratch.selected_output_trace());
+                    check(wd_stream_sync(stream), "sync");
+                    std::vector<uint16_t> got_h(H), got_tr(static_cast<size_t>(k) * H);
+                    check(wd_memcpy_d2h(got_h.data(), dout_h.data, sizeof(uint16_t) * H, nullptr), "half output");
+                    check(wd_memcpy_d2h(got_tr.data(), scratch.selected_output_trace(), sizeof(uint16_t) * got_tr.size(), nullptr), "trace");
+                    bool ok_h = true, ok_tr = true;
+                    for (int i = 0; i < H; ++i) ok_h = ok_h && got_h[i] == wdo_f32_to_f16_rn(routed_h[i]);
+                    for (size_t i = 0; i < got_tr.size(); ++i) ok_tr = ok_tr && got_tr[i] == wdo_f32_to_f16_rn(eo[i]);
+                    CHECK(ok_h, "mode %d layer %d: half-in half-out routed sum differs from the rounded oracle", mode, l);
+                    CHECK(ok_tr, "mode %d layer %d: selected expert trace differs from the rounded oracle", mode, l);
+                    // float output from half input equals the float runner on the widened input
+                    DeviceFloatArray dxw(H), o1(H), o2(H);
+                    dxw.upload(xw.data(), H);
+                    run_qwen38_routed_moe_separate<false, float, half_bits>(l, dxh.data, routers[l], L[l].t_gate, L[l].t_up, L[l].t_down, cache,
+                                                                           scratch, o1.data, 1.0f, stream);
+                    run_qwen38_routed_moe_separate<false, float, float>(l, dxw.data, routers[l], L[l].t_gate, L[l].t_up, L[l].t_down, cache, scratch,
+                                                                       o2.data, 1.0f, stream);
+                    check(wd_stream_sync(stream), "sync");
+                    std::vector<float> a1(H), a2(H);
+                    o1.download(a1.data()), o2.download(a2.data());
+                    CHECK(same_bits(a1.data(), a2.data(), H) && same_bits(a1.data(), routed_h.data(), H), "mode %d layer %d: half-input runner differs", mode, l);
+                    CHECK(throws([&] { run_qwen38_routed_moe_separate<true, float, float>(l, dxw.data, routers[l], L[l].t_gate, L[l].t_up, L[l].t_down,
+                                                                                         cache, scratch, o2.data, 1.0f, stream); }),
+                          "a capturing run without a trace buffer must throw");
+                }
                 if (mode == 1) {
                     // the one-call wrappers with a cache that cannot hold the layer: the ids go through the host instead of
                     // the kernels indexing a slot table with holes in it

@@ -323,3 +323,77 @@ def test_error_paths(g):
     assert lib.wd_gemv_q8_k_f32(synth.IQ3_S, g.ptr(x), 4, 100, g.ptr(x), g.ptr(x), g.ptr(x), None, None) == -1
     assert lib.wd_gemv_q6_k_q8_k_f32(g.ptr(x), 4, 300, g.ptr(x), g.ptr(x), g.ptr(x), g.ptr(x), None, None) == -1
     assert lib.wd_gemv_q6_k_q8_k_f32(g.ptr(x), 4, 65536, g.ptr(x), g.ptr(x), g.ptr(x), g.ptr(x), None, None) == -1
+
+
+# ---- the plain Q8_0 x Q8_1 path, the half-input quantiser, the element-wise conversions ------------------------------
+@pytest.mark.parametrize("n", [32, 2048, 6144, 32 * 37])
+def test_quantize_q8_1(g, oracle, n):
+    for x in _act_cases(max(n, 256), SEED + 13 * n):
+        x = x[:n].copy()
+        dx = g.dev(x)
+        qs, d = g.empty(n, np.int8), g.empty(n // 32, np.uint16)
+        capi.call("wd_q8_1_quantize_f32", g.ptr(dx), n, g.ptr(qs), g.ptr(d), g.stream())
+        g.sync()
+        oq, od = oracle.quantize_q8_1(x)
+        assert np.array_equal(g.host(qs), oq)
+        assert np.array_equal(g.host(d, np.uint16), od)
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 2048), (5, 96), (9, 2048 + 64), (320, 2048), (2048, 320), (3, 4096 + 32)])
+def test_gemv_q8_0_q8_1(g, oracle, rows, cols):
+    """launch_q8_0_gemv_q8_1_f32 (src/lowbit.cuh:343-362): quantise, then the row sums in block order - quants, scales,
+    int32 block sums and f32 results all bit-identical to the oracle."""
+    rng = synth.rng_for(SEED, 77, rows, cols)
+    w = np.ascontiguousarray(synth.q8_0_matrix(rng, rows, cols)).reshape(-1)
+    for x in _act_cases(max(cols, 256), SEED + rows + cols)[:4]:
+        x = x[:cols].copy()
+        dw, dx = g.dev(w), g.dev(x)
+        qs, d = g.empty(cols, np.int8), g.empty(cols // 32, np.uint16)
+        y, sums = g.empty(rows, np.float32), g.empty(rows * (cols // 32), np.int32)
+        capi.call("wd_q8_1_quantize_f32", g.ptr(dx), cols, g.ptr(qs), g.ptr(d), g.stream())
+        capi.call("wd_gemv_q8_0_q8_1_f32", g.ptr(dw), rows, cols, g.ptr(qs), g.ptr(d), g.ptr(y), g.ptr(sums), g.stream())
+        g.sync()
+        oq, od = oracle.quantize_q8_1(x)
+        oy, osums = oracle.gemv_q8_0_q8_1(w, rows, cols, oq, od)
+        assert np.array_equal(g.host(qs), oq) and np.array_equal(g.host(d, np.uint16), od)
+        assert np.array_equal(g.host(sums).reshape(rows, -1), osums)
+        assert g.same_bits(g.host(y), oy)
+    lib = capi.load()
+    assert lib.wd_gemv_q8_0_q8_1_f32(g.ptr(dw), rows, 33, g.ptr(qs), g.ptr(d), g.ptr(y), None, g.stream()) == -1
+
+
+@pytest.mark.parametrize("n", [32, 2048, 32 * 37])
+def test_quantize_q8_0_from_half(g, oracle, n):
+    rng = np.random.default_rng(SEED + 17 * n)
+    for scale in (1.0, 1e-3, 3e-6, 300.0):
+        xh = (rng.normal(0, 1, n) * scale).astype(np.float16)
+        xh[:8] = 0
+        dx = g.dev(xh.view(np.uint16))
+        qs, d = g.empty(n, np.int8), g.empty(n // 32, np.uint16)
+        capi.call("wd_q8_0_quantize_f16", g.ptr(dx), n, g.ptr(qs), g.ptr(d), g.stream())
+        g.sync()
+        oq, od = oracle.quantize_q8_0_f16(xh.view(np.uint16))
+        assert np.array_equal(g.host(qs), oq), scale
+        assert np.array_equal(g.host(d, np.uint16), od), scale
+
+
+def test_half_float_conversions(g, oracle):
+    """Every half widens exactly; floats narrow by IEEE round-to-nearest-even (numpy's float16 conversion and the oracle's
+    agree, tests/test_oracle_pins.py)."""
+    halves = np.arange(65536, dtype=np.uint16)
+    dh, df = g.dev(halves), g.empty(65536, np.float32)
+    capi.call("wd_convert_f16_to_f32", g.ptr(dh), g.ptr(df), 65536, g.stream())
+    g.sync()
+    want = halves.view(np.float16).astype(np.float32)
+    got = g.host(df)
+    finite = ~np.isnan(want)
+    assert g.same_bits(got[finite], want[finite]) and np.isnan(got[~finite]).all()
+    rng = np.random.default_rng(SEED + 31)
+    v = (rng.normal(size=100001) * 10.0 ** rng.integers(-9, 5, 100001)).astype(np.float32)
+    v[:6] = [65504, 65520, 2.0 ** -25, 1 + 2.0 ** -11, 1 + 3 * 2.0 ** -11, -0.0]
+    dv, dout = g.dev(v), g.empty(v.size, np.uint16)
+    capi.call("wd_convert_f32_to_f16", g.ptr(dv), g.ptr(dout), v.size, g.stream())
+    g.sync()
+    with np.errstate(over="ignore"):
+        assert np.array_equal(g.host(dout, np.uint16), v.astype(np.float16).view(np.uint16))
+    assert np.array_equal(g.host(dout, np.uint16)[:2000], oracle.f32_to_f16_rn(v[:2000]))

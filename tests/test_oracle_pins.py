@@ -657,3 +657,102 @@ def test_hc_combine_against_numpy(oracle, hc, hidden, round_half):
     assert np.array_equal(got.view(np.uint32), want16.view(np.uint32))
     for c in range(hc):                 # the weight itself: 2 / (1 + exp(-inject / hc)) to float accuracy
         assert abs(float(w[c]) - 2.0 / (1.0 + np.exp(-float(inject[c]) / hc))) < 1e-6
+
+
+# ---- the plain Q8_0 x Q8_1 path and the half-input quantiser (src/lowbit.cuh:287-362, src/warodecode.cu:1504-1520) ----
+def test_f32_to_f16_rn_equals_numpy(oracle):
+    """IEEE round-to-nearest-even against numpy's float16 conversion (an implementation of its own): ties, the subnormal
+    range, overflow to infinity, and 200,000 values over thirteen decades."""
+    edge = np.array([1.0, 65504, 65519.996, 65520, 2.0 ** -24, 2.0 ** -25, np.nextafter(np.float32(2.0 ** -25), np.float32(1)),
+                     1 + 2.0 ** -11, 1 + 3 * 2.0 ** -11, -(1 + 2.0 ** -11), 0.0, -0.0, 6.0e-8, 3.0e-8], np.float32)
+    rng = np.random.default_rng(SEED + 901)
+    many = (rng.normal(size=200000) * 10.0 ** rng.integers(-9, 5, 200000)).astype(np.float32)
+    for v in (edge, many):
+        with np.errstate(over="ignore"):
+            assert np.array_equal(oracle.f32_to_f16_rn(v), v.astype(np.float16).view(np.uint16))
+
+
+def test_q8_1_quantiser_closed_forms(oracle):
+    """d = amax / 127 and q = roundf(x / d): with amax = 63.5 the scale is exactly 0.5, so x = j / 2 must give q = j; halves
+    go away from zero (2.5 -> 3, -2.5 -> -3, where the Q8_0 quantiser's round-to-even gives 2 and -2); a zero block stays
+    zero with a zero scale; the scale is half(d)."""
+    x = np.zeros(96, np.float32)
+    x[:32] = np.arange(-16, 16) * 0.5
+    x[31] = 63.5
+    x[64:96] = [127, 2.5, -2.5, 3.5, -3.5, 0.49999997, 126.5, -126.5] + [0] * 24
+    q, d = oracle.quantize_q8_1(x)
+    assert q[:31].tolist() == list(range(-16, 15)) and q[31] == 127
+    assert not q[32:64].any() and d[1] == 0
+    assert q[64:72].tolist() == [127, 3, -3, 4, -4, 0, 127, -127]
+    assert oracle.quantize_q8_0(x[64:96])[0][:5].tolist() == [127, 2, -2, 4, -4]      # the other rounding, for contrast
+    assert oracle.f16_to_f32(d).tolist() == [0.5, 0.0, 1.0]
+    rng = np.random.default_rng(SEED + 902)
+    x = rng.normal(0, 3, 4096).astype(np.float32)
+    q, d = oracle.quantize_q8_1(x)
+    amax = np.abs(x.reshape(-1, 32)).max(axis=1)
+    scale = (amax / np.float32(127)).astype(np.float32)
+    want = np.where(x.reshape(-1, 32) / scale[:, None] >= 0, np.floor(x.reshape(-1, 32) / scale[:, None] + np.float32(0.5)),
+                    np.ceil(x.reshape(-1, 32) / scale[:, None] - np.float32(0.5)))
+    # (floor(t + 0.5) in float32 can differ from roundf(t) only when t + 0.5 rounds up across an integer: none here)
+    assert np.array_equal(q.reshape(-1, 32), want.astype(np.int8))
+    assert np.array_equal(d, scale.astype(np.float16).view(np.uint16))
+
+
+def test_q8_0_q8_1_gemv_against_exact_integers_and_a_sequential_sum(oracle):
+    """With unit scales and small quants every product and partial sum is an integer below 2^24: the row sum must equal the
+    integer dot product whatever the order.  With real scales the sum is order-dependent: it must equal the plain
+    sequential float32 loop over the blocks (multiply the scales, multiply by the integer sum, add) and differ from a
+    pairwise sum on this sample; the exported block sums are the exact int32 dot products."""
+    rng = np.random.default_rng(SEED + 903)
+    rows, cols = 7, 2048
+    nb = cols // 32
+    one = np.float16(1.0).view(np.uint16)
+
+    def pack(dw, qw):
+        w = np.empty((rows, nb, 34), np.uint8)
+        w[:, :, :2] = dw.astype(np.uint16).reshape(rows, nb, 1).view(np.uint8).reshape(rows, nb, 2)
+        w[:, :, 2:] = qw.view(np.uint8).reshape(rows, nb, 32)
+        return w.reshape(-1)
+
+    qw = rng.integers(-8, 9, (rows, nb, 32)).astype(np.int8)
+    qx = rng.integers(-8, 9, cols).astype(np.int8)
+    y, sums = oracle.gemv_q8_0_q8_1(pack(np.full((rows, nb), one), qw), rows, cols, qx, np.full(nb, one, np.uint16))
+    exact = (qw.reshape(rows, cols).astype(np.int64) * qx.astype(np.int64)).sum(axis=1)
+    assert np.array_equal(y, exact.astype(np.float32))
+    assert np.array_equal(sums, (qw.astype(np.int64) * qx.reshape(nb, 32)).sum(axis=2))
+
+    qw = rng.integers(-127, 128, (rows, nb, 32)).astype(np.int8)
+    qx = rng.integers(-127, 128, cols).astype(np.int8)
+    dw = rng.uniform(0.001, 0.02, (rows, nb)).astype(np.float16)
+    dx = rng.uniform(0.001, 0.02, nb).astype(np.float16)
+    y, sums = oracle.gemv_q8_0_q8_1(pack(dw.view(np.uint16), qw), rows, cols, qx, dx.view(np.uint16))
+    dots = (qw.astype(np.int64) * qx.reshape(nb, 32)).sum(axis=2)
+    assert np.array_equal(sums, dots)
+    seq = np.zeros(rows, np.float32)
+    for b in range(nb):
+        scale = dw[:, b].astype(np.float32) * dx[b].astype(np.float32)
+        seq = (seq + scale * dots[:, b].astype(np.float32)).astype(np.float32)
+    assert np.array_equal(y.view(np.uint32), seq.view(np.uint32))
+    prods = (dw.astype(np.float32) * dx.astype(np.float32)[None, :] * dots.astype(np.float32)).astype(np.float32)
+    pairwise = prods.copy()
+    while pairwise.shape[1] > 1:
+        pairwise = (pairwise[:, 0::2] + pairwise[:, 1::2]).astype(np.float32)
+    assert not np.array_equal(pairwise[:, 0].view(np.uint32), y.view(np.uint32))
+
+
+def test_q8_0_quantiser_from_half_input(oracle):
+    """The values widened to float go through inv = 127 / amax and lrintf (half to even), clamped to +-127; on input that
+    is representable in half the quants equal the float quantiser's; the scale is the IEEE half of amax / 127, which for
+    a block of tiny values is a subnormal half where the float quantiser's block-scale conversion stores zero."""
+    rng = np.random.default_rng(SEED + 904)
+    xh = rng.normal(0, 2, 2048).astype(np.float16)
+    xh[32:64] = 0
+    xh[64:96] = (2.0 ** -24 * rng.integers(-80, 81, 32)).astype(np.float16)   # amax / 127 between 2^-25 and 2^-24
+    xh[64] = np.float16(84 * 2.0 ** -24)
+    q, d = oracle.quantize_q8_0_f16(xh.view(np.uint16))
+    qf, df = oracle.quantize_q8_0(xh.astype(np.float32))
+    assert np.array_equal(q, qf)
+    amax = np.abs(xh.astype(np.float32).reshape(-1, 32)).max(axis=1)
+    assert np.array_equal(d, (amax / np.float32(127)).astype(np.float32).astype(np.float16).view(np.uint16))
+    assert d[1] == 0 and d[2] == 1 and df[2] == 0
+    assert np.array_equal(d[3:], df[3:])

@@ -57,6 +57,11 @@ class CacheStats(C.Structure):
 _SIGS = {
     "wd_init": (i32, [i32]),
     "wd_row_bytes": (sz, [i32, i32]),
+    "wd_q8_0_quantize_f16": (i32, [vp, i32, vp, vp, vp]),
+    "wd_q8_1_quantize_f32": (i32, [vp, i32, vp, vp, vp]),
+    "wd_gemv_q8_0_q8_1_f32": (i32, [vp, i32, i32, vp, vp, vp, vp, vp]),
+    "wd_convert_f16_to_f32": (i32, [vp, vp, sz, vp]),
+    "wd_convert_f32_to_f16": (i32, [vp, vp, sz, vp]),
     "wd_gemv_q6_k_q8_k_f32": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp]),
     "wd_file_mapping_of": (i32, [vp, C.POINTER(FileMapping)]),
     "wd_expert_cache_attach_mappings": (i32, [vp, i32, C.POINTER(i32)]),

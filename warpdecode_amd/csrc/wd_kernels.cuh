@@ -126,6 +126,103 @@ __global__ __launch_bounds__(256) void k_q8_0_quantize(const float *__restrict__
     if (sub == 0) scales[blk] = f2h_ref(amax / 127.0f);
 }
 
+// ---- the reference's plain Q8_0 x Q8_1 path and its half-input quantiser ----------------------------------------
+// IEEE float -> half bits (the reference's __float2half), unlike f2h_ref.
+WD_DEV uint16_t f2h_rn(float v) {
+    const _Float16 f = static_cast<_Float16>(v);
+    uint16_t h;
+    __builtin_memcpy(&h, &f, 2);
+    return h;
+}
+// The largest |v| of the block of 32 values held four per lane by eight consecutive lanes.
+WD_DEV float block32_amax(const float4 &v) {
+    float amax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)),
+                                 __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
+    amax = quad_max(amax);
+    return __builtin_fmaxf(amax, dpp_f<0x141>(amax, amax));  // row_half_mirror pairs the two quads of a block
+}
+// q8_1_quantize_f32_kernel, src/lowbit.cuh:287-308: d = amax / 127, q = roundf(x / d) (a division; halves away from
+// zero), scale = half(d).  Eight lanes per block, four values per lane.
+__global__ __launch_bounds__(256) void k_q8_1_quantize(const float *__restrict__ x, int blocks, int8_t *__restrict__ qs,
+                                                        uint16_t *__restrict__ scales) {
+    const int sub = threadIdx.x & 7;
+    const int blk = blockIdx.x * 32 + (threadIdx.x >> 3);
+    const bool on = blk < blocks;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (on) v = reinterpret_cast<const float4 *>(x + static_cast<size_t>(blk) * 32)[sub];
+    const float amax = block32_amax(v);
+    if (!on) return;
+    const float d = amax / 127.0f;
+    auto q = [&](float t) { return amax == 0.0f ? 0 : static_cast<int>(__builtin_roundf(t / d)); };
+    const int q0 = q(v.x), q1 = q(v.y), q2 = q(v.z), q3 = q(v.w);
+    reinterpret_cast<uint32_t *>(qs + static_cast<size_t>(blk) * 32)[sub] =
+        (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | (static_cast<uint32_t>(q3 & 0xff) << 24);
+    if (sub == 0) scales[blk] = f2h_rn(d);
+}
+// q8_0_quantize_half_kernel, src/warodecode.cu:1504-1520: half input, inv = 127 / amax, q = lrintf(v * inv) clamped to
+// +-127, scale = half(amax / 127).
+__global__ __launch_bounds__(256) void k_q8_0_quantize_f16(const uint16_t *__restrict__ x, int blocks, int8_t *__restrict__ qs,
+                                                            uint16_t *__restrict__ scales) {
+    const int sub = threadIdx.x & 7;
+    const int blk = blockIdx.x * 32 + (threadIdx.x >> 3);
+    const bool on = blk < blocks;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (on) {
+        const uint2 h = reinterpret_cast<const uint2 *>(x + static_cast<size_t>(blk) * 32)[sub];
+        v = make_float4(h2f(static_cast<uint16_t>(h.x)), h2f(static_cast<uint16_t>(h.x >> 16)), h2f(static_cast<uint16_t>(h.y)),
+                        h2f(static_cast<uint16_t>(h.y >> 16)));
+    }
+    const float amax = block32_amax(v);
+    if (!on) return;
+    const float inv = amax == 0.0f ? 0.0f : 127.0f / amax;
+    auto q = [&](float t) { return max(-127, min(127, static_cast<int>(__builtin_rintf(t * inv)))); };
+    const int q0 = q(v.x), q1 = q(v.y), q2 = q(v.z), q3 = q(v.w);
+    reinterpret_cast<uint32_t *>(qs + static_cast<size_t>(blk) * 32)[sub] =
+        (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | (static_cast<uint32_t>(q3 & 0xff) << 24);
+    if (sub == 0) scales[blk] = f2h_rn(amax / 127.0f);
+}
+// q8_0_q8_1_gemv_f32_kernel, src/lowbit.cuh:310-341: one wave per row, lane = block (64 blocks a pass); the row's sum
+// runs over the blocks in ascending order, one rounded multiply of the two scales, one with the integer sum, one add.
+// block_sums (optional): int32 [rows][cols / 32].
+__global__ __launch_bounds__(256) void k_gemv_q8_0_q8_1(const uint8_t *__restrict__ w, int rows, int cols,
+                                                         const int8_t *__restrict__ qs, const uint16_t *__restrict__ scales,
+                                                         float *__restrict__ y, int32_t *__restrict__ block_sums) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int nb = cols >> 5;
+    const uint8_t *wr = w + static_cast<size_t>(row) * nb * 34;
+    float sum = 0.0f;
+    for (int base = 0; base < nb; base += 64) {
+        const int b = base + lane;
+        float prod = 0.0f;
+        if (b < nb) {
+            const uint8_t *blk = wr + static_cast<size_t>(b) * 34;
+            int dot = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t wq = static_cast<uint32_t>(ldu<uint16_t>(blk + 2 + 4 * i)) | (static_cast<uint32_t>(ldu<uint16_t>(blk + 4 + 4 * i)) << 16);
+                dot = sdot4(wq, *reinterpret_cast<const uint32_t *>(qs + b * 32 + 4 * i), dot);
+            }
+            if (block_sums) block_sums[static_cast<size_t>(row) * nb + b] = dot;
+            const float scale = h2f(ldu<uint16_t>(blk)) * h2f(scales[b]);
+            prod = scale * static_cast<float>(dot);
+        }
+        const int n = min(64, nb - base);
+        for (int i = 0; i < n; ++i) sum = sum + readlane_f(prod, i);
+    }
+    if (lane == 0) y[row] = sum;
+}
+// Element-wise half <-> float (IEEE rounding on the way down).
+__global__ void k_f16_to_f32(const uint16_t *__restrict__ src, float *__restrict__ dst, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = h2f(src[i]);
+}
+__global__ void k_f32_to_f16(const float *__restrict__ src, uint16_t *__restrict__ dst, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = f2h_rn(src[i]);
+}
+
 // ---- router GEMV: 32 lanes per row, lane t owns accumulator t of the 4x8 scheme --------------
 // (src/qwen38_moe.cuh:198-245).  Optional extra row (the shared expert's gate vector).
 __global__ __launch_bounds__(256) void k_router_gemv(const float *__restrict__ w, const float *__restrict__ x,

@@ -135,6 +135,45 @@ int wd_q8_0_quantize_f32(const float *d_x, int elements, int8_t *d_qs, uint16_t 
     return WD_OK;
 }
 
+int wd_q8_1_quantize_f32(const float *d_x, int elements, int8_t *d_qs, uint16_t *d_scales, void *stream) {
+    WD_REQUIRE(elements > 0 && elements % 32 == 0, "Q8_1 input must be a positive multiple of 32 (got %d)", elements);
+    WD_REQUIRE(d_x && d_qs && d_scales, "wd_q8_1_quantize_f32: null pointer");
+    const int blocks = elements / 32;
+    k_q8_1_quantize<<<dim3((blocks + 31) / 32), dim3(256), 0, as_stream(stream)>>>(d_x, blocks, d_qs, d_scales);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+int wd_q8_0_quantize_f16(const uint16_t *d_x, int elements, int8_t *d_qs, uint16_t *d_scales, void *stream) {
+    WD_REQUIRE(elements > 0 && elements % 32 == 0, "Q8_0 quantisation requires a positive multiple of 32 elements (got %d)", elements);
+    WD_REQUIRE(d_x && d_qs && d_scales, "wd_q8_0_quantize_f16: null pointer");
+    WD_REQUIRE(reinterpret_cast<uintptr_t>(d_x) % 8 == 0, "wd_q8_0_quantize_f16: the input must be 8-byte aligned");
+    const int blocks = elements / 32;
+    k_q8_0_quantize_f16<<<dim3((blocks + 31) / 32), dim3(256), 0, as_stream(stream)>>>(d_x, blocks, d_qs, d_scales);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+int wd_gemv_q8_0_q8_1_f32(const uint8_t *d_w, int rows, int cols, const int8_t *d_qs, const uint16_t *d_scales, float *d_y,
+                          int32_t *d_block_sums, void *stream) {
+    WD_REQUIRE(rows > 0 && cols > 0 && cols % 32 == 0, "Q8_0 x Q8_1 GEMV geometry mismatch (%d x %d)", rows, cols);
+    WD_REQUIRE(d_w && d_qs && d_scales && d_y, "wd_gemv_q8_0_q8_1_f32: null pointer");
+    WD_REQUIRE(reinterpret_cast<uintptr_t>(d_qs) % 4 == 0, "wd_gemv_q8_0_q8_1_f32: the quantised input must be 4-byte aligned");
+    k_gemv_q8_0_q8_1<<<dim3((rows + 3) / 4), dim3(256), 0, as_stream(stream)>>>(d_w, rows, cols, d_qs, d_scales, d_y, d_block_sums);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+int wd_convert_f16_to_f32(const uint16_t *d_src, float *d_dst, size_t n, void *stream) {
+    WD_REQUIRE(d_src && d_dst && n > 0, "wd_convert_f16_to_f32: invalid arguments");
+    k_f16_to_f32<<<dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, as_stream(stream)>>>(d_src, d_dst, n);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+int wd_convert_f32_to_f16(const float *d_src, uint16_t *d_dst, size_t n, void *stream) {
+    WD_REQUIRE(d_src && d_dst && n > 0, "wd_convert_f32_to_f16: invalid arguments");
+    k_f32_to_f16<<<dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, as_stream(stream)>>>(d_src, d_dst, n);
+    WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
 // ---- router -------------------------------------------------------------------------------
 int wd_router_gemv_f32(const float *d_w, const float *d_x, float *d_logits, int rows, int cols, void *stream) {
     WD_REQUIRE(rows > 0 && cols > 0, "router GEMV: invalid shape %d x %d", rows, cols);

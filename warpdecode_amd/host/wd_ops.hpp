@@ -11,7 +11,9 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <cstdlib>
 #include <cstring>
+#include <type_traits>
 #include <stdexcept>
 #include <string>
 #include <utility>
@@ -254,11 +256,21 @@ public:
         if (h_ids_) wd_free_host(h_ids_);
         if (h_weights_) wd_free_host(h_weights_);
         s_ = nullptr, h_ids_ = nullptr, h_weights_ = nullptr;
-        moe_out_.reset();
+        moe_out_.reset(), x_f32_.reset(), trace_.reset();
     }
     float *moe_out_f32() {
         if (moe_out_.empty()) moe_out_.allocate(static_cast<size_t>(hidden_));
         return moe_out_.data;
+    }
+    // the layer's input widened to float, for callers that hold it as half
+    float *x_f32() {
+        if (x_f32_.empty()) x_f32_.allocate(static_cast<size_t>(hidden_));
+        return x_f32_.data;
+    }
+    // src/qwen38_moe.cuh:1769-1775: half [k][hidden], the selected experts' down outputs of a capturing run
+    half_bits *selected_output_trace() {
+        if (trace_.empty()) trace_.allocate(static_cast<size_t>(k_) * hidden_);
+        return trace_.data;
     }
     int n_experts() const { return n_experts_; }
     int k() const { return k_; }
@@ -295,7 +307,8 @@ private:
     int n_experts_ = 0, k_ = 0, hidden_ = 0, expert_ffn_ = 0;
     int *h_ids_ = nullptr;
     float *h_weights_ = nullptr;
-    DeviceFloatArray moe_out_;
+    DeviceFloatArray moe_out_, x_f32_;
+    DeviceArray<half_bits> trace_;
 };
 
 // src/expert_cache.cuh:76-115 (the file-backed staging knobs have no meaning here: sources are host memory)
@@ -471,6 +484,75 @@ inline void q38_moe_quantize_activation_q8_0(const float *input, int elements, i
     check(wd_q8_0_quantize_f32(input, elements, quantized, scales, stream), "Q8_0 quantisation failed");
 }
 
+// src/warodecode.cu:1504-1520 (the dense Q4_0 path's activation quantiser: half input)
+inline void launch_q8_0_quantize_half(const half_bits *x, int elements, int8_t *quantized, half_bits *scales, Stream stream) {
+    check(wd_q8_0_quantize_f16(x, elements, quantized, scales, stream), "Q8_0 quantisation of half input failed");
+}
+
+// src/lowbit.cuh:251-285: the activation buffer of the plain Q8_0 x Q8_1 GEMV
+class Q8_1Buffer {
+public:
+    Q8_1Buffer() = default;
+    Q8_1Buffer(const Q8_1Buffer &) = delete;
+    Q8_1Buffer &operator=(const Q8_1Buffer &) = delete;
+    ~Q8_1Buffer() { reset(); }
+
+    void initialize(int elements) {
+        if (values_) throw std::runtime_error("Q8_1 buffer already initialized");
+        if (elements <= 0 || elements % 32 != 0) throw std::runtime_error("Q8_1 input must be a positive multiple of 32");
+        void *p = nullptr;
+        check(wd_malloc(&p, static_cast<size_t>(elements)), "Q8_1 values allocation failed");
+        values_ = static_cast<int8_t *>(p);
+        if (wd_malloc(&p, static_cast<size_t>(elements / 32) * sizeof(half_bits)) != WD_OK) {
+            reset();
+            throw std::runtime_error(std::string("Q8_1 scales allocation failed: ") + wd_last_error());
+        }
+        scales_ = static_cast<half_bits *>(p);
+        elements_ = elements;
+    }
+    int elements() const { return elements_; }
+    int8_t *values() const { return values_; }
+    half_bits *scales() const { return scales_; }
+
+private:
+    void reset() {
+        if (values_) wd_free(values_);
+        if (scales_) wd_free(scales_);
+        values_ = nullptr, scales_ = nullptr, elements_ = 0;
+    }
+    int elements_ = 0;
+    int8_t *values_ = nullptr;
+    half_bits *scales_ = nullptr;
+};
+
+// src/lowbit.cuh:343-362: quantise the input to Q8_1, then one row sum per output (blocks in ascending order)
+inline void launch_q8_0_gemv_q8_1_f32(const LowBitMatrix &weights, const float *input, float *output, Q8_1Buffer &scratch, Stream stream) {
+    if (weights.type != GgmlType::Q8_0 || weights.rows <= 0 || weights.cols > scratch.elements() || weights.cols % 32 != 0)
+        throw std::runtime_error("Q8_0 x Q8_1 GEMV geometry mismatch");
+    check(wd_q8_1_quantize_f32(input, weights.cols, scratch.values(), scratch.scales(), stream), "Q8_1 quantisation failed");
+    check(wd_gemv_q8_0_q8_1_f32(weights.data, weights.rows, weights.cols, scratch.values(), scratch.scales(), output, nullptr, stream),
+          "Q8_0 x Q8_1 GEMV failed");
+}
+
+// The slot pool's default size for a device with `vram_bytes` of memory: three quarters of the card minus 8 GiB, at least
+// 512 MiB, at most 64 GiB; WARODECODE_EXPERT_CACHE_MIB overrides it (src/qwen38_tuning.hpp:88-116: 40 GB -> 22 GiB,
+// 80 GB -> 52 GiB).  A device that holds the whole model needs no pool at all: the layer calls take resident tensors.
+inline int default_expert_cache_mib(size_t vram_bytes) {
+    long long cache = static_cast<long long>(vram_bytes >> 20) * 3 / 4 - 8 * 1024;
+    if (cache < 512) cache = 512;
+    if (cache > 64 * 1024) cache = 64 * 1024;
+    if (const char *v = std::getenv("WARODECODE_EXPERT_CACHE_MIB")) {
+        const int mib = std::atoi(v);
+        if (mib > 0) cache = mib;
+    }
+    return static_cast<int>(cache);
+}
+// How many layers ahead the expert read-ahead works, by device memory (src/qwen38_tuning.hpp:97-112).
+inline int default_expert_prefetch_depth(size_t vram_bytes) {
+    const long long mib = static_cast<long long>(vram_bytes >> 20);
+    return mib >= 120 * 1024 ? 3 : (mib >= 40 * 1024 ? 2 : 1);
+}
+
 // src/qwen38_moe.cuh:247-263
 inline void launch_q38_router_gemv_f32(const GpuMatrix &w, const float *x, float *y, Stream stream, int threads = 256) {
     if (!matrix_has_f32_weights(w)) throw std::runtime_error("router F32 warp GEMV requires an F32 dense matrix");
@@ -599,7 +681,7 @@ inline void fill_routed(wd_moe_layer &L, int layer, const GpuMatrix &router, con
 // The wait for the ids is also where a failure recorded by an earlier pass on this scratch surfaces.
 inline void routed_through_host(const wd_moe_layer &L, int layer, const float *x, const TensorInfo &gate, const TensorInfo &up,
                                 const TensorInfo &down, GpuExpertCache &cache, Qwen38MoeScratch &scratch, float *dst, bool run_a,
-                                Stream stream) {
+                                Stream stream, unsigned extra_flags = 0u) {
     if (run_a) check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), WD_MOE_ONLY_A, stream), "MoE router failed");
     check(wd_memcpy_d2h(scratch.h_ids(), scratch.d_ids(), sizeof(int) * L.top_k, stream), "routed ids copy failed");
     scratch.queue_status_copy(stream);
@@ -607,7 +689,7 @@ inline void routed_through_host(const wd_moe_layer &L, int layer, const float *x
     scratch.throw_if_failed();
     cache.register_layer_experts(layer, gate, up, down);
     cache.acquire_ids(layer, scratch.h_ids(), L.top_k, stream);
-    check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), WD_MOE_PRESELECTED | WD_MOE_ONLY_B | WD_MOE_ONLY_C, stream), "MoE experts failed");
+    check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), WD_MOE_PRESELECTED | WD_MOE_ONLY_B | WD_MOE_ONLY_C | extra_flags, stream), "MoE experts failed");
 }
 }  // namespace detail
 
@@ -618,22 +700,23 @@ inline void routed_through_host(const wd_moe_layer &L, int layer, const float *x
 inline void run_qwen38_routed_moe_separate_f32_x(int layer, const float *x, const GpuMatrix &router, const TensorInfo &gate_exps,
                                                  const TensorInfo &up_exps, const TensorInfo &down_exps, GpuExpertCache &cache,
                                                  Qwen38MoeScratch &scratch, float *out, float expert_scale, Stream stream,
-                                                 bool preselected = false) {
+                                                 bool preselected = false, bool keep_expert_outputs = false) {
     wd_moe_layer L;
     detail::fill_routed(L, layer, router, gate_exps, up_exps, down_exps, cache, scratch, expert_scale);
     float *dst = out ? out : scratch.moe_out_f32();
+    const unsigned keep = keep_expert_outputs ? WD_MOE_KEEP_EXPERT_OUT : 0u;  // scratch.rx_batch_down(): [k][hidden]
     if (cache.layer_resident(layer)) {
-        check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), preselected ? WD_MOE_PRESELECTED : 0u, stream), "MoE layer failed");
+        check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), (preselected ? WD_MOE_PRESELECTED : 0u) | keep, stream), "MoE layer failed");
         return;
     }
-    detail::routed_through_host(L, layer, x, gate_exps, up_exps, down_exps, cache, scratch, dst, !preselected, stream);
+    detail::routed_through_host(L, layer, x, gate_exps, up_exps, down_exps, cache, scratch, dst, !preselected, stream, keep);
 }
 
 // The same with the gate and up projections stored as one tensor of 2 * ffn rows per expert
 // (run_qwen38_routed_moe_fused, src/qwen38_moe.cuh:3522-3647).
 inline void run_qwen38_routed_moe_fused_f32_x(int layer, const float *x, const GpuMatrix &router, const TensorInfo &gate_up_exps,
                                               const TensorInfo &down_exps, GpuExpertCache &cache, Qwen38MoeScratch &scratch, float *out,
-                                              float expert_scale, Stream stream, bool preselected = false) {
+                                              float expert_scale, Stream stream, bool preselected = false, bool keep_expert_outputs = false) {
     if (gate_up_exps.dims.size() != 3 || gate_up_exps.dims[1] % 2 != 0) throw std::runtime_error("fused gate_up tensor must be 3D with an even row count: " + gate_up_exps.name);
     TensorInfo half = gate_up_exps;   // geometry of one projection; the data pointer is only used for registration
     half.dims[1] = gate_up_exps.dims[1] / 2;
@@ -644,7 +727,72 @@ inline void run_qwen38_routed_moe_fused_f32_x(int layer, const float *x, const G
     TensorInfo g = half, u = half;
     g.data = gate_up_exps.data, u.data = gate_up_exps.data;
     // expert_slice() checks contiguity against byte_size(): give it tensors of the half geometry
-    run_qwen38_routed_moe_separate_f32_x(layer, x, router, g, u, down_exps, cache, scratch, out, expert_scale, stream, preselected);
+    run_qwen38_routed_moe_separate_f32_x(layer, x, router, g, u, down_exps, cache, scratch, out, expert_scale, stream, preselected,
+                                         keep_expert_outputs);
+}
+
+// The reference's runners by element type (src/qwen38_moe.cuh:3521-3534, :3650-3668): XT the type of the layer's input
+// (half bits or float), OutT that of the routed output, CaptureSelectedOutput the k selected experts' down outputs as half
+// into selected_output_trace [k][hidden].  Half input is widened once (every half is a float, so the result is that of the
+// float runner on the widened input - the reference's own statement, :3607-3610); half output is the F32 routed sum
+// rounded once, as the reference's F32-mid lifetime rounds it (q38_finish_moe, :2401-2453).
+namespace detail {
+template <typename XT>
+inline const float *widened_input(const XT *x, Qwen38MoeScratch &scratch, Stream stream) {
+    if constexpr (std::is_same<XT, float>::value) {
+        return x;
+    } else {
+        static_assert(std::is_same<XT, half_bits>::value, "MoE input is float or half bits");
+        check(wd_convert_f16_to_f32(x, scratch.x_f32(), static_cast<size_t>(scratch.hidden()), stream), "widening the MoE input failed");
+        return scratch.x_f32();
+    }
+}
+template <bool Capture, typename OutT>
+inline void narrowed_output(Qwen38MoeScratch &scratch, const float *routed, OutT *out, half_bits *trace, Stream stream) {
+    if constexpr (!std::is_same<OutT, float>::value) {
+        static_assert(std::is_same<OutT, half_bits>::value, "MoE output is float or half bits");
+        check(wd_convert_f32_to_f16(routed, out, static_cast<size_t>(scratch.hidden()), stream), "rounding the MoE output failed");
+    }
+    if constexpr (Capture)
+        check(wd_convert_f32_to_f16(scratch.rx_batch_down(), trace, static_cast<size_t>(scratch.k()) * scratch.hidden(), stream),
+              "selected expert trace failed");
+}
+}  // namespace detail
+
+template <bool CaptureSelectedOutput = false, typename OutT = half_bits, typename XT = half_bits>
+inline void run_qwen38_routed_moe_separate(int layer, const XT *x, const GpuMatrix &router, const TensorInfo &gate_exps,
+                                           const TensorInfo &up_exps, const TensorInfo &down_exps, GpuExpertCache &cache,
+                                           Qwen38MoeScratch &scratch, OutT *out, float expert_scale, Stream stream,
+                                           bool preselected = false, half_bits *selected_output_trace = nullptr) {
+    if (CaptureSelectedOutput && !selected_output_trace) throw std::runtime_error("selected expert trace buffer is null");
+    if (!out) throw std::runtime_error("MoE output buffer is null");
+    const float *xf = detail::widened_input<XT>(x, scratch, stream);
+    float *routed = std::is_same<OutT, float>::value ? reinterpret_cast<float *>(out) : scratch.moe_out_f32();
+    run_qwen38_routed_moe_separate_f32_x(layer, xf, router, gate_exps, up_exps, down_exps, cache, scratch, routed, expert_scale, stream,
+                                         preselected, CaptureSelectedOutput);
+    detail::narrowed_output<CaptureSelectedOutput, OutT>(scratch, routed, out, selected_output_trace, stream);
+}
+template <bool CaptureSelectedOutput = false, typename OutT = half_bits, typename XT = half_bits>
+inline void run_qwen38_routed_moe_fused(int layer, const XT *x, const GpuMatrix &router, const TensorInfo &gate_up_exps,
+                                        const TensorInfo &down_exps, GpuExpertCache &cache, Qwen38MoeScratch &scratch, OutT *out,
+                                        float expert_scale, Stream stream, bool preselected = false,
+                                        half_bits *selected_output_trace = nullptr) {
+    if (CaptureSelectedOutput && !selected_output_trace) throw std::runtime_error("selected expert trace buffer is null");
+    if (!out) throw std::runtime_error("MoE output buffer is null");
+    const float *xf = detail::widened_input<XT>(x, scratch, stream);
+    float *routed = std::is_same<OutT, float>::value ? reinterpret_cast<float *>(out) : scratch.moe_out_f32();
+    run_qwen38_routed_moe_fused_f32_x(layer, xf, router, gate_up_exps, down_exps, cache, scratch, routed, expert_scale, stream, preselected,
+                                      CaptureSelectedOutput);
+    detail::narrowed_output<CaptureSelectedOutput, OutT>(scratch, routed, out, selected_output_trace, stream);
+}
+// src/qwen38_moe.cuh:3588-3604: float output from half input
+template <bool CaptureSelectedOutput = false>
+inline void run_qwen38_routed_moe_fused_f32(int layer, const half_bits *x, const GpuMatrix &router, const TensorInfo &gate_up_exps,
+                                            const TensorInfo &down_exps, GpuExpertCache &cache, Qwen38MoeScratch &scratch, float *out,
+                                            float expert_scale, Stream stream, bool preselected = false,
+                                            half_bits *selected_output_trace = nullptr) {
+    run_qwen38_routed_moe_fused<CaptureSelectedOutput, float, half_bits>(layer, x, router, gate_up_exps, down_exps, cache, scratch, out,
+                                                                         expert_scale, stream, preselected, selected_output_trace);
 }
 
 // src/qwen38_moe.cuh:3963-3969
