@@ -298,6 +298,18 @@ int wd_moe_stack_f32(const wd_moe_layer *layers, int n_layers, float *d_x, float
  * (which re-reads the weights per (token, expert) pair). */
 int wd_moe_layer_tokens_f32(const wd_moe_layer *layer, const float *d_x, float *d_out, int tokens,
                             wd_moe_scratch *const *scratch_per_token, unsigned flags, void *stream);
+/* The same pass over the experts a caller holds as separate views instead of tensors that contain every expert (the
+ * form in which the reference's token batch receives them, one (gate, up, down) triple per acquired expert:
+ * Qwen38MoeTokenBatch::set_pair_weights / run, src/qwen38_moe.cuh:2907-3109).  h_gate / h_up / h_down: host arrays of
+ * n_entries (<= 128) device pointers; the ids in the scratches are entry numbers, the weights the router weights, and
+ * flags must contain WD_MOE_PRESELECTED.  `layer` supplies geometry, tensor types and (optionally) the shared expert;
+ * its routed tensor pointers are ignored.  IQ3_S / IQ2_S gate and up; Q8_0 down with ffn <= 512, or 16-byte aligned
+ * down views with ffn 512 / 640.  The table travels through a small pinned ring owned by the first scratch (allocated
+ * at first use); every expert's bytes are read once for all tokens that selected it, results are those of one pass
+ * per token. */
+int wd_moe_layer_tokens_pairs_f32(const wd_moe_layer *layer, const uint8_t *const *h_gate, const uint8_t *const *h_up,
+                                  const uint8_t *const *h_down, int n_entries, const float *d_x, float *d_out, int tokens,
+                                  wd_moe_scratch *const *scratch_per_token, unsigned flags, void *stream);
 
 /* ---- expert-slot cache -----------------------------------------------------------
  * LRU pool of fixed-size slots in HBM, key (layer << 32 | expert); a miss copies the expert's

@@ -566,6 +566,70 @@ static void gpu_checks() {
                     wdo_moe_layer(&L[l].o, xs.data() + static_cast<size_t>(t) * H, want.data(), nullptr, 0);
                     CHECK(same_bits(got.data() + static_cast<size_t>(t) * H, want.data(), H), "mode %d layer %d token %d of the batch differs from the oracle", mode, l, t);
                 }
+                // the same tokens through the reference's batch object, driven as its caller drives it
+                // (src/qwen38_mtp.cuh:702-747): selection of all tokens, the union acquired expert by expert, every pair
+                // told its views, one pass, the routed sums out as float and as half
+                {
+                    Qwen38MoeTokenBatch batch;
+                    CHECK(batch.compatible(cache, scratch, L[l].t_gate, L[l].t_up, L[l].t_down, T) == (mode == 0), "mode %d: batch compatibility (8 slots per selection)", mode);
+                    CHECK(!batch.compatible(cache, scratch, L[l].t_gate, L[l].t_up, L[l].t_down, kMoeBatchTokenMax + 1) &&
+                              !batch.compatible(cache, scratch, L[l].t_down, L[l].t_up, L[l].t_down, T), "batch bound and tensor types");
+                    std::vector<const float *> acts;
+                    for (int t = 0; t < T; ++t) acts.push_back(dxs.data + static_cast<size_t>(t) * H);
+                    batch.open_all(scratch, routers[l], acts, 1.0f, stream, false);
+                    std::vector<int> union_expert, union_slot(static_cast<size_t>(T) * k);
+                    std::vector<ExpertDeviceWeights> union_weights;
+                    for (int p = 0; p < T * k; ++p) {
+                        const int expert = scratch.h_ids()[p];
+                        int at = -1;
+                        for (size_t q = 0; q < union_expert.size(); ++q)
+                            if (union_expert[q] == expert) at = static_cast<int>(q);
+                        if (at < 0) {
+                            at = static_cast<int>(union_expert.size());
+                            union_expert.push_back(expert);
+                            union_weights.push_back(cache.acquire(l, expert, L[l].t_gate, L[l].t_up, L[l].t_down, stream));
+                        }
+                        union_slot[static_cast<size_t>(p)] = at;
+                    }
+                    CHECK(!batch.resolved(), "pairs without views are not resolved");
+                    for (int p = 0; p < T * k; ++p) {
+                        const ExpertDeviceWeights &w = union_weights[static_cast<size_t>(union_slot[static_cast<size_t>(p)])];
+                        batch.set_pair_weights(p, w.gate, w.up, w.down);
+                    }
+                    CHECK(batch.resolved(true), "mode %d layer %d: the batch should be runnable", mode, l);
+                    batch.run(scratch, L[l].t_gate, L[l].t_up, L[l].t_down, stream);
+                    DeviceFloatArray bo(static_cast<size_t>(T) * H);
+                    DeviceArray<half_bits> bh(static_cast<size_t>(T) * H);
+                    batch.write_output(scratch, bo.data, nullptr, stream);
+                    batch.write_output(scratch, nullptr, bh.data, stream);
+                    check(wd_stream_sync(stream), "sync");
+                    std::vector<float> sums(static_cast<size_t>(T) * H), routed(H);
+                    std::vector<uint16_t> halves(sums.size());
+                    bo.download(sums.data());
+                    check(wd_memcpy_d2h(halves.data(), bh.data, sizeof(uint16_t) * halves.size(), nullptr), "half sums");
+                    CHECK(batch.tokens() == T && batch.accumulated(scratch) != nullptr, "batch accessors");
+                    for (int t = 0; t < T; ++t) {
+                        wdo_dump dd{};
+                        std::vector<int> oids(k);
+                        dd.routed = routed.data(), dd.ids = oids.data();
+                        wdo_moe_layer(&L[l].o, xs.data() + static_cast<size_t>(t) * H, want.data(), &dd, 0);
+                        CHECK(std::equal(oids.begin(), oids.end(), scratch.h_ids() + t * k), "mode %d layer %d token %d: batch selection differs", mode, l, t);
+                        CHECK(same_bits(sums.data() + static_cast<size_t>(t) * H, routed.data(), H), "mode %d layer %d token %d: batch routed sum differs from the oracle", mode, l, t);
+                        bool okh = true;
+                        for (int i = 0; i < H; ++i) okh = okh && halves[static_cast<size_t>(t) * H + i] == wdo_f32_to_f16_rn(routed[i]);
+                        CHECK(okh, "mode %d layer %d token %d: batch half output differs", mode, l, t);
+                    }
+                    // a slot recycled under an earlier pair shows as two pairs with one view and two experts
+                    if (union_expert.size() >= 2) {
+                        const ExpertDeviceWeights &w0 = union_weights[0];
+                        int other = -1;
+                        for (int p = 0; p < T * k; ++p)
+                            if (union_slot[static_cast<size_t>(p)] == 1) other = p;
+                        batch.set_pair_weights(other, w0.gate, w0.up, w0.down);
+                        CHECK(batch.resolved(false) && !batch.resolved(true), "a recycled slot must fail the slot check");
+                    }
+                    CHECK(throws([&] { batch.set_pair_weights(kMoeBatchTokenMax * 16, union_weights[0].gate, union_weights[0].up, union_weights[0].down); }), "pair index bound");
+                }
             }
         }
     }

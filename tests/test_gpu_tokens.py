@@ -125,3 +125,59 @@ def test_tokens_errors(g):
     assert lib.wd_moe_layer_tokens_f32(C.byref(dl.desc), g.ptr(x), g.ptr(x), 2, arr, 0, None) == -1   # shared scratch
     assert lib.wd_moe_layer_tokens_f32(C.byref(dl.desc), g.ptr(x), g.ptr(x), 9, arr, 0, None) == -1
     sc.close()
+
+
+@pytest.mark.parametrize("shape", ["c2", "model", "small-unaligned"])
+def test_tokens_on_a_table_of_expert_views(g, oracle, shape):
+    """wd_moe_layer_tokens_pairs_f32: the pass over (gate, up, down) views given expert by expert - the form in which the
+    reference's token batch receives acquired experts (src/qwen38_moe.cuh:2907-3109) - with entry numbers as ids.  The
+    views here point into resident tensors, in a shuffled order with a few entries nobody selects; every token must
+    come out as from the pass over the tensors themselves, i.e. as from the oracle."""
+    if shape == "c2":
+        L, T = synth.make_c2(n_experts=64), 4
+    elif shape == "model":
+        L, T = synth.make_layer(2560, 640, 32, 8, synth.IQ2_S, synth.IQ4_NL, shared=True, seed=SEED + 3), 3
+    else:
+        L, T = synth.make_layer(512, 64, 16, 4, synth.IQ3_S, synth.Q8_0, shared=False, seed=SEED + 4), 5
+    H, F, E, k = L["hidden"], L["expert_ffn"], L["n_experts"], L["top_k"]
+    dl = g.DeviceLayer(L)
+    if shape == "small-unaligned":     # views that are only 2-byte aligned: the tensors copied to an odd-word offset
+        for name in ("gate", "up", "down"):
+            raw = np.concatenate([np.zeros(2, np.uint8), np.ascontiguousarray(L[name]).reshape(-1)])
+            dl.keep[name + "_shifted"] = g.dev(raw)
+            setattr(dl.desc, name, dl.keep[name + "_shifted"].data_ptr() + 2)
+    xs = correlated_tokens(H, T, 31 + T)
+    ref = run_tokens(g, dl, L, xs)
+    rng = np.random.default_rng(SEED + 55)
+    union = sorted(set(ref["ids"].ravel().tolist()))
+    entries = union + [e for e in range(E) if e not in union][:3]
+    order = rng.permutation(len(entries))
+    entries = [entries[i] for i in order]
+    entry_of = {e: i for i, e in enumerate(entries)}
+    d = dl.desc
+    P = C.c_void_p * len(entries)
+    hg = P(*[d.gate + e * d.gate_stride for e in entries])
+    hu = P(*[d.up + e * d.up_stride for e in entries])
+    hd = P(*[d.down + e * d.down_stride for e in entries])
+    scs = [g.Scratch(H, F, E, k) for _ in range(T)]
+    for t in range(T):
+        vids = np.array([entry_of[e] for e in ref["ids"][t]], np.int32)
+        capi.call("wd_memcpy_h2d", C.c_void_p(scs[t].raw("ids")), vids.ctypes.data_as(C.c_void_p), 4 * k, None)
+        capi.call("wd_memcpy_h2d", C.c_void_p(scs[t].raw("weights")), np.ascontiguousarray(ref["weights"][t]).ctypes.data_as(C.c_void_p), 4 * k, None)
+    arr = (C.c_void_p * T)(*[s.h for s in scs])
+    dx, out = g.dev(xs), g.empty((T, H), np.float32)
+    lib = capi.load()
+    for rep in range(6):       # more calls than the ring of pointer tables has entries
+        capi.call("wd_moe_layer_tokens_pairs_f32", C.byref(d), hg, hu, hd, len(entries), g.ptr(dx), g.ptr(out), T, arr,
+                  capi.MOE_PRESELECTED, g.stream())
+    g.sync()
+    got = g.host(out)
+    for t in range(T):
+        want, dump = oracle.moe_layer(L, xs[t])
+        assert g.same_bits(got[t], want), (shape, t)
+        assert g.same_bits(scs[t].get("accum", H, np.float32), dump["routed"]), (shape, t)
+        assert g.same_bits(got[t], ref["out"][t])
+    assert lib.wd_moe_layer_tokens_pairs_f32(C.byref(d), hg, hu, hd, len(entries), g.ptr(dx), g.ptr(out), T, arr, 0, g.stream()) == -1
+    assert lib.wd_moe_layer_tokens_pairs_f32(C.byref(d), hg, hu, hd, 129, g.ptr(dx), g.ptr(out), T, arr, capi.MOE_PRESELECTED, g.stream()) == -1
+    for s in scs:
+        s.close()

@@ -48,7 +48,13 @@ struct wd_moe_scratch {
     int res_fits = -1;                            // -1 not asked yet; 1: the device holds the whole grid at once
     int trace_layer = 0;
     bool trace_all = false;                       // the trace buffer has the resident kernel's size
+    // wd_moe_layer_tokens_pairs_f32: a ring of pointer tables (pinned staging + device copy), kPairRing x [kPairEntries][3]
+    const uint8_t **pair_host = nullptr, **pair_dev = nullptr;
+    hipEvent_t pair_done[4] = {nullptr, nullptr, nullptr, nullptr};
+    bool pair_used[4] = {false, false, false, false};
+    int pair_next = 0;
 };
+constexpr int kPairRing = 4, kPairEntries = 128;
 
 namespace {
 constexpr int kTagRecords = 64;  // one record per layer of a stack (modulo), so that a chain of layers needs no reset in between
@@ -138,6 +144,10 @@ int wd_moe_scratch_destroy(wd_moe_scratch *s) {
     (void)hipFree(s->res_block);
     (void)hipFree(s->res_layers);
     (void)hipHostFree(s->h_ids);
+    (void)hipFree(s->pair_dev);
+    (void)hipHostFree(s->pair_host);
+    for (hipEvent_t ev : s->pair_done)
+        if (ev) (void)hipEventDestroy(ev);
     delete s;
     return WD_OK;
 }
@@ -768,8 +778,11 @@ extern "C" int wd_moe_stack_f32(const wd_moe_layer *layers, int n_layers, float 
     return WD_OK;
 }
 
-extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, float *d_out, int tokens,
-                                       wd_moe_scratch *const *scratch_per_token, unsigned flags, void *stream) {
+namespace {
+// gu_table / down_table: null, or device tables of pointers ([entry][2] gate and up, [entry] down) that take the place of
+// the layer's routed tensors, the ids of the pass being entry numbers; tables_aligned: every pointer in them is 16-byte aligned.
+int tokens_pass(const wd_moe_layer *L, const float *d_x, float *d_out, int tokens, wd_moe_scratch *const *scratch_per_token,
+                unsigned flags, void *stream, const uint8_t *const *gu_table, const uint8_t *const *down_table, bool tables_aligned) {
     WD_REQUIRE(tokens > 0 && tokens <= kMaxTokens, "multi-token pass: 1..%d tokens (got %d)", kMaxTokens, tokens);
     WD_REQUIRE(scratch_per_token != nullptr && d_x && d_out, "multi-token pass: null pointer");
     for (int t = 0; t < tokens; ++t) {
@@ -786,6 +799,7 @@ extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, 
                             scratch_per_token[0]->gup == nullptr &&
                             !(flags & (WD_MOE_ONLY_A | WD_MOE_ONLY_B | WD_MOE_ONLY_C | WD_MOE_DRY));
     const bool down_tokens = L->down_type == WD_TYPE_Q8_0 && F <= 512;
+    if (gu_table) WD_REQUIRE(union_path, "multi-token pass on a pointer table: IQ3_S / IQ2_S gate and up tensors, at most 128 (token, expert) pairs, no staging flags");
     if (!union_path) {
         // same results, one pass per token (every pass reads its own experts)
         for (int t = 0; t < tokens; ++t)
@@ -799,6 +813,10 @@ extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, 
     ta.common = fused_args(L, d_x, d_out, scratch_per_token[0], flags, nullptr, nullptr, 0.0f);
     ta.common.gate_up = routed_src(L, scratch_per_token[0], nullptr, false);  // the kernels pass the expert id themselves
     ta.common.down = routed_src(L, scratch_per_token[0], nullptr, true);
+    if (gu_table) {
+        ta.common.gate_up.table = gu_table, ta.common.gate_up.per_expert = 2;
+        ta.common.down.table = down_table, ta.common.down.per_expert = 1;
+    }
     for (int t = 0; t < tokens; ++t) {
         wd_moe_scratch *s = scratch_per_token[t];
         TokenSlots &k_ = ta.tok[t];
@@ -821,8 +839,9 @@ extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, 
     // rows of eight or ten super-blocks of aligned tensors: the aligned fetch, one item ahead
     auto al16b = [](const void *p_, size_t v) { return reinterpret_cast<uintptr_t>(p_) % 16 == 0 && v % 16 == 0; };
     const bool coal_b = (H == 2048 || H == 2560) &&
-                        (L->slot_of_expert ? al16b(L->slot_pool, L->slot_bytes) && L->slot_gate_bytes % 16 == 0
-                                           : al16b(L->gate, L->gate_stride) && al16b(L->up, L->up_stride));
+                        (gu_table ? tables_aligned
+                                  : (L->slot_of_expert ? al16b(L->slot_pool, L->slot_bytes) && L->slot_gate_bytes % 16 == 0
+                                                       : al16b(L->gate, L->gate_stride) && al16b(L->up, L->up_stride)));
     const size_t lds_b_coal = ((lds_b + 15) & ~static_cast<size_t>(15)) + 8 * 2 * static_cast<size_t>(H == 2048 ? kIqStageBytes : kIqStage10Bytes);
     const dim3 gb(grid_b), bb(512);
 #define WD_TOKENS_B(TYPE_)                                                                              \
@@ -848,8 +867,9 @@ extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, 
     auto al16t = [](const void *p_, size_t v) { return reinterpret_cast<uintptr_t>(p_) % 16 == 0 && v % 16 == 0; };
     const bool down_tokens_nb = !down_tokens && (F == 512 || F == 640) && H % 8 == 0 && tokens <= 16 &&
                                 (!L->shared_down || al16t(L->shared_down, 0)) &&
-                                (L->slot_of_expert ? al16t(L->slot_pool, L->slot_bytes) && (L->slot_gate_bytes + L->slot_up_bytes) % 16 == 0
-                                                   : al16t(L->down, L->down_stride));
+                                (down_table ? tables_aligned
+                                            : (L->slot_of_expert ? al16t(L->slot_pool, L->slot_bytes) && (L->slot_gate_bytes + L->slot_up_bytes) % 16 == 0
+                                                                 : al16t(L->down, L->down_stride)));
     if (down_tokens_nb) {
         const size_t per_wave_n = (static_cast<size_t>(F) + F / 16 + 15) & ~static_cast<size_t>(15);
         const size_t lds_n = 16 * per_wave_n + sizeof(float) * 8 * tokens * (k + 1);
@@ -862,6 +882,7 @@ extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, 
         return WD_OK;
     }
     if (!down_tokens) {
+        WD_REQUIRE(!down_table, "multi-token pass on a pointer table: this down tensor (type %d, %d columns) has no multi-token dispatch", L->down_type, F);
         for (int t = 0; t < tokens; ++t)
             if (const int rc = layer_fused(L, d_x + static_cast<size_t>(t) * H, d_out + static_cast<size_t>(t) * H, scratch_per_token[t],
                                            flags | WD_MOE_ONLY_C, nullptr, nullptr, 0.0f, st))
@@ -874,4 +895,46 @@ extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, 
     k_tokens_c<<<dim3((H + 7) / 8), dim3(64 * waves_c), lds_c, st>>>(ta);
     WD_LAUNCH_CHECK();
     return WD_OK;
+}
+}  // namespace
+
+extern "C" int wd_moe_layer_tokens_f32(const wd_moe_layer *L, const float *d_x, float *d_out, int tokens,
+                                       wd_moe_scratch *const *scratch_per_token, unsigned flags, void *stream) {
+    return tokens_pass(L, d_x, d_out, tokens, scratch_per_token, flags, stream, nullptr, nullptr, false);
+}
+
+extern "C" int wd_moe_layer_tokens_pairs_f32(const wd_moe_layer *L, const uint8_t *const *h_gate, const uint8_t *const *h_up,
+                                             const uint8_t *const *h_down, int n_entries, const float *d_x, float *d_out, int tokens,
+                                             wd_moe_scratch *const *scratch_per_token, unsigned flags, void *stream) {
+    WD_REQUIRE(L && h_gate && h_up && h_down && scratch_per_token && scratch_per_token[0], "multi-token pass on a pointer table: null argument");
+    WD_REQUIRE(n_entries > 0 && n_entries <= kPairEntries, "multi-token pass on a pointer table: 1..%d entries (got %d)", kPairEntries, n_entries);
+    WD_REQUIRE(flags & WD_MOE_PRESELECTED, "multi-token pass on a pointer table: the selection (entry numbers) must be in the scratches");
+    bool aligned = true;
+    for (int i = 0; i < n_entries; ++i) {
+        WD_REQUIRE(h_gate[i] && h_up[i] && h_down[i], "multi-token pass on a pointer table: entry %d has a null pointer", i);
+        WD_REQUIRE((reinterpret_cast<uintptr_t>(h_gate[i]) | reinterpret_cast<uintptr_t>(h_up[i]) | reinterpret_cast<uintptr_t>(h_down[i])) % 2 == 0,
+                   "multi-token pass on a pointer table: entry %d is not 2-byte aligned", i);
+        aligned = aligned && (reinterpret_cast<uintptr_t>(h_gate[i]) | reinterpret_cast<uintptr_t>(h_up[i]) | reinterpret_cast<uintptr_t>(h_down[i])) % 16 == 0;
+    }
+    wd_moe_layer Lt = *L;  // the routed tensors come from the table: the descriptor's own are placeholders for the checks
+    Lt.slot_of_expert = nullptr;
+    Lt.gate = h_gate[0], Lt.up = h_up[0], Lt.down = h_down[0];
+    Lt.n_experts = n_entries < Lt.top_k ? Lt.top_k : n_entries;
+    wd_moe_scratch *s = scratch_per_token[0];
+    hipStream_t st = as_stream(stream);
+    if (!s->pair_dev) {  // once per scratch
+        WD_HIP(hipHostMalloc(reinterpret_cast<void **>(&s->pair_host), sizeof(void *) * 3 * kPairEntries * kPairRing, hipHostMallocDefault));
+        WD_HIP(hipMalloc(reinterpret_cast<void **>(&s->pair_dev), sizeof(void *) * 3 * kPairEntries * kPairRing));
+        for (hipEvent_t &ev : s->pair_done) WD_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+    }
+    const int slot = s->pair_next;
+    s->pair_next = (slot + 1) % kPairRing;
+    if (s->pair_used[slot]) WD_HIP(hipEventSynchronize(s->pair_done[slot]));  // the pass that read this entry of the ring has run
+    const uint8_t **h = s->pair_host + static_cast<size_t>(slot) * 3 * kPairEntries, **d = s->pair_dev + static_cast<size_t>(slot) * 3 * kPairEntries;
+    for (int i = 0; i < n_entries; ++i) h[2 * i] = h_gate[i], h[2 * i + 1] = h_up[i], h[2 * kPairEntries + i] = h_down[i];
+    WD_HIP(hipMemcpyAsync(d, h, sizeof(void *) * 3 * kPairEntries, hipMemcpyHostToDevice, st));
+    const int rc = tokens_pass(&Lt, d_x, d_out, tokens, scratch_per_token, flags, stream, d, d + 2 * kPairEntries, aligned);
+    WD_HIP(hipEventRecord(s->pair_done[slot], st));
+    s->pair_used[slot] = true;
+    return rc;
 }

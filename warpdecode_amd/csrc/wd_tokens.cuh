@@ -18,6 +18,14 @@ namespace wd {
 
 constexpr int kMaxTokens = 8;
 
+// Tensor T of "expert" e when the pass was given a table of pointers instead of tensors that hold every expert: e is
+// then an index into the table ([entry][tensors per entry]).
+template <int T>
+WD_DEV const uint8_t *mat_ptr_entry(const MatSrc &s, int e) {
+    if (s.table) return s.table[e * s.per_expert + T];
+    return mat_ptr_expert<T>(s, e);
+}
+
 struct TokenSlots {
     const float *x;
     float *logits;
@@ -234,7 +242,7 @@ __global__ __launch_bounds__(512, 4) void k_tokens_b(TokenArgs ta) {
         const int u = item / groups, rg = item - u * groups;
         const int e = un.expert[u];
         const size_t off = static_cast<size_t>(min(rg * 8 + wave, a.F - 1)) * rb;
-        rows[0] = uniform_ptr(mat_ptr_expert<0>(a.gate_up, e) + off), rows[1] = uniform_ptr(mat_ptr_expert<1>(a.gate_up, e) + off);
+        rows[0] = uniform_ptr(mat_ptr_entry<0>(a.gate_up, e) + off), rows[1] = uniform_ptr(mat_ptr_entry<1>(a.gate_up, e) + off);
     };
     if (NB != 0 && static_cast<int>(blockIdx.x) < n_items) {
         const uint8_t *rows[2];
@@ -393,7 +401,7 @@ __global__ __launch_bounds__(1024) void k_tokens_c(TokenArgs ta) {
             const bool is_shared = it_j[i] == a.k;
             const int pair = it_t[i] * a.k + (is_shared ? 0 : it_j[i]);
             const int e = pair < 64 ? __builtin_amdgcn_readlane(id_lo, pair) : __builtin_amdgcn_readlane(id_hi, pair - 64);
-            const uint8_t *w = is_shared ? a.sh_down : mat_ptr_expert<0>(a.down, e);
+            const uint8_t *w = is_shared ? a.sh_down : mat_ptr_entry<0>(a.down, e);
 #pragma unroll
             for (int g = 0; g < 2; ++g) {
                 const int row = min(r0 + 4 * g + r4, a.H - 1);
@@ -531,7 +539,7 @@ __global__ __launch_bounds__(1024) void k_tokens_c_nb(TokenArgs ta) {
             const bool is_shared = it_j[i] == a.k;
             const int pair = it_t[i] * a.k + (is_shared ? 0 : it_j[i]);
             const int e = pair < 64 ? __builtin_amdgcn_readlane(id_lo, pair) : __builtin_amdgcn_readlane(id_hi, pair - 64);
-            const uint8_t *w = is_shared ? a.sh_down : mat_ptr_expert<0>(a.down, e);
+            const uint8_t *w = is_shared ? a.sh_down : mat_ptr_entry<0>(a.down, e);
 #pragma unroll
             for (int g = 0; g < 2; ++g) {
                 if (KIND == 0 || is_shared) {  // wave-uniform

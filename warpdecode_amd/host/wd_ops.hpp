@@ -13,6 +13,7 @@
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 #include <type_traits>
 #include <stdexcept>
 #include <string>
@@ -229,6 +230,8 @@ struct Qwen38SharedExpertWeights {
     LowBitMatrix gate, up, down;      // Q8_0
 };
 
+constexpr int kMoeBatchTokenMax = 8;  // tokens of one batch pass (src/qwen38_moe.cuh:2711 allows 32; larger batches take the serial loop)
+
 // src/qwen38_moe.cuh:1701-2150.  The device buffers belong to the library's scratch object; the accessors
 // keep the reference's names for the views a caller reads after a layer pass.
 class Qwen38MoeScratch {
@@ -245,10 +248,12 @@ public:
         check(wd_moe_scratch_create(&s_, hidden, expert_ffn, n_experts, k), "MoE scratch allocation failed");
         n_experts_ = n_experts, k_ = k, hidden_ = hidden, expert_ffn_ = expert_ffn;
         void *p = nullptr;
-        check(wd_malloc_host(&p, sizeof(int) * (k + 1)), "pinned allocation failed");  // [k] receives the status word
+        // room for a token batch's ids and weights ([kMoeBatchTokenMax][k], as the reference's batch buffers); the word
+        // behind the ids receives the status word
+        check(wd_malloc_host(&p, sizeof(int) * (kMoeBatchTokenMax * k + 1)), "pinned allocation failed");
         h_ids_ = static_cast<int *>(p);
-        h_ids_[k] = 0;
-        check(wd_malloc_host(&p, sizeof(float) * k), "pinned allocation failed");
+        h_ids_[kMoeBatchTokenMax * k] = 0;
+        check(wd_malloc_host(&p, sizeof(float) * kMoeBatchTokenMax * k), "pinned allocation failed");
         h_weights_ = static_cast<float *>(p);
     }
     void reset() {
@@ -292,12 +297,13 @@ public:
     // throw_if_failed() reports a layer pass on this scratch whose results are invalid (a bounded wait that ran out,
     // an expert that had no slot).
     void queue_status_copy(Stream stream) {
-        check(wd_memcpy_d2h(h_ids_ + k_, wd_moe_scratch_status_word(s_), sizeof(int), stream), "status copy failed");
+        check(wd_memcpy_d2h(h_ids_ + kMoeBatchTokenMax * k_, wd_moe_scratch_status_word(s_), sizeof(int), stream), "status copy failed");
     }
     void throw_if_failed() const {
-        if (h_ids_[k_] == 1) throw std::runtime_error("MoE layer pass failed: a wait between its workgroups ran out");
-        if (h_ids_[k_] == 2) throw std::runtime_error("MoE layer pass failed: an expert without a cache slot was selected");
-        if (h_ids_[k_] != 0) throw std::runtime_error("MoE layer pass failed");
+        const int st = h_ids_[kMoeBatchTokenMax * k_];
+        if (st == 1) throw std::runtime_error("MoE layer pass failed: a wait between its workgroups ran out");
+        if (st == 2) throw std::runtime_error("MoE layer pass failed: an expert without a cache slot was selected");
+        if (st != 0) throw std::runtime_error("MoE layer pass failed");
     }
     float *h_weights() const { return h_weights_; }
     wd_moe_scratch *handle() const { return s_; }
@@ -879,6 +885,185 @@ inline void run_qwen38_moe_tokens_f32_x(int layer, const float *x, int tokens, c
         if (wd_expert_cache_slot_of(cache.handle(), layer, e) < 0) throw std::runtime_error("token batch: the expert cache is too small for the union of the tokens' experts");
     check(wd_moe_layer_tokens_f32(&L, x, out, tokens, handles.data(), WD_MOE_PRESELECTED, stream), "MoE token batch failed");
 }
+
+// The MTP block's token batch with the reference's interface (Qwen38MoeTokenBatch, src/qwen38_moe.cuh:2743-3237; its
+// caller: src/qwen38_mtp.cuh:674-795): open_all selects the experts of every token with one synchronisation, the caller
+// acquires the union of the experts and names each pair's (token * k + rank) views with set_pair_weights, resolved()
+// decides whether the pass may run, run() computes every token's routed sum with each distinct expert read once, and
+// write_output() hands the sums on as float or half.  After open_all, scratch.h_ids() / h_weights() hold [tokens][k].
+class Qwen38MoeTokenBatch {
+public:
+    Qwen38MoeTokenBatch() = default;
+    Qwen38MoeTokenBatch(const Qwen38MoeTokenBatch &) = delete;
+    Qwen38MoeTokenBatch &operator=(const Qwen38MoeTokenBatch &) = delete;
+
+    int batch_k() const { return 16; }
+    int tokens() const { return tokens_; }
+
+    // src/qwen38_moe.cuh:2767-2791: the pass exists for IQ2_S / IQ3_S gate and up tensors; the down tensors this library
+    // batches are Q8_0 rows of at most 16 blocks and aligned IQ4_NL / Q8_0 rows of 16 or 20 blocks.  The slot bound is the
+    // reference's (8 slots per selection).
+    bool compatible(const GpuExpertCache &cache, const Qwen38MoeScratch &scratch, const TensorInfo &gate_exps, const TensorInfo &up_exps,
+                    const TensorInfo &down_exps, int tokens) const {
+        if (tokens < 1 || tokens > kMoeBatchTokenMax) return false;
+        if (scratch.k() < 1 || scratch.k() > batch_k() || tokens * scratch.k() > 128) return false;
+        auto iq = [](GgmlType t) { return t == GgmlType::IQ2_S || t == GgmlType::IQ3_S; };
+        if (!iq(gate_exps.type) || gate_exps.type != up_exps.type) return false;
+        const int F = scratch.expert_ffn();
+        if (!(down_exps.type == GgmlType::Q8_0 && F <= 512) && !((down_exps.type == GgmlType::IQ4_NL || down_exps.type == GgmlType::Q8_0) && (F == 512 || F == 640)))
+            return false;
+        if (gate_exps.dims.size() != 3 || up_exps.dims.size() != 3 || down_exps.dims.size() != 3) return false;
+        if (static_cast<int>(gate_exps.dims[0]) != scratch.hidden() || static_cast<int>(gate_exps.dims[1]) != F ||
+            static_cast<int>(up_exps.dims[0]) != scratch.hidden() || static_cast<int>(up_exps.dims[1]) != F ||
+            static_cast<int>(down_exps.dims[0]) != F || static_cast<int>(down_exps.dims[1]) != scratch.hidden())
+            return false;
+        return cache.slot_count() >= 8u * static_cast<size_t>(scratch.k());
+    }
+
+    // src/qwen38_moe.cuh:2798-2888.  activations: one device pointer per token (float [hidden]).  preselected: the caller
+    // has put ids and weights into scratch.h_ids() / h_weights() ([tokens][k]) itself (or will, with set_pair_experts).
+    void open_all(Qwen38MoeScratch &scratch, const GpuMatrix &router, const std::vector<const float *> &activations, float expert_scale,
+                  Stream stream, bool preselected) {
+        tokens_ = static_cast<int>(activations.size());
+        if (tokens_ < 1 || tokens_ > kMoeBatchTokenMax) throw std::runtime_error("MoE token batch holds one to the batch bound of tokens");
+        if (!(expert_scale > 0.0f)) throw std::runtime_error("MoE token batch needs a positive expert scale");
+        for (const float *x : activations)
+            if (!x) throw std::runtime_error("MoE token batch got a null activation");
+        k_ = scratch.k(), hidden_ = scratch.hidden();
+        activations_ = activations;
+        ids_ = scratch.h_ids(), weights_ = scratch.h_weights();
+        while (tok_.size() < static_cast<size_t>(tokens_)) {
+            tok_.emplace_back(new Qwen38MoeScratch);
+            tok_.back()->initialize(scratch.n_experts(), scratch.k(), scratch.hidden(), scratch.expert_ffn());
+        }
+        for (int p = 0; p < kMoeBatchTokenMax * 16; ++p) pair_[p] = Pair();
+        router_ = router.dense_f32.data;
+        if (preselected) return;
+        if (!matrix_has_f32_weights(router)) throw std::runtime_error("MoE router must be an F32 matrix");
+        if (router.rows != scratch.n_experts() || router.cols != hidden_) throw std::runtime_error("Qwen3.8 router matrix geometry mismatch");
+        for (int t = 0; t < tokens_; ++t) {
+            Qwen38MoeScratch &q = *tok_[static_cast<size_t>(t)];
+            check(wd_router_gemv_f32(router.dense_f32.data, activations[static_cast<size_t>(t)], q.d_logits(), router.rows, router.cols, stream),
+                  "MoE token batch router failed");
+            check(wd_topk_softmax(q.d_logits(), router.rows, k_, expert_scale, q.d_ids(), q.d_weights(), stream), "MoE token batch selection failed");
+            check(wd_memcpy_d2h(ids_ + t * k_, q.d_ids(), sizeof(int) * k_, stream), "MoE token batch ids copy failed");
+            check(wd_memcpy_d2h(weights_ + t * k_, q.d_weights(), sizeof(float) * k_, stream), "MoE token batch weights copy failed");
+        }
+        check(wd_stream_sync(stream), "MoE token batch selection failed");
+        queued_ = false;
+    }
+
+    // src/qwen38_moe.cuh:2897-2904
+    void set_pair_experts(int pair, int expert, const std::vector<float> &weights_by_pair) {
+        if (pair < 0 || pair >= kMoeBatchTokenMax * 16) throw std::runtime_error("MoE token batch pair index out of range");
+        if (ids_) ids_[pair] = expert;
+        if (weights_) weights_[pair] = weights_by_pair[static_cast<size_t>(pair)];
+    }
+    // src/qwen38_moe.cuh:2907-2922
+    void set_pair_weights(int pair, const LowBitMatrix &gate, const LowBitMatrix &up, const LowBitMatrix &down) {
+        if (pair < 0 || pair >= kMoeBatchTokenMax * 16) throw std::runtime_error("MoE token batch pair index out of range");
+        pair_[pair].gate = gate.data, pair_[pair].up = up.data, pair_[pair].down = down.data;
+        if (pair == 0) gate_type_ = gate.type, down_type_ = down.type, ffn_ = gate.rows;
+    }
+    // src/qwen38_moe.cuh:2933-2951: every pair has its three views, 2-byte aligned, of the types the pass takes; with
+    // check_slots, two pairs that share a slot must name the same expert (otherwise a later acquire recycled the slot
+    // under an earlier pair and the batch must give way to the serial loop).
+    bool resolved(bool check_slots = false) {
+        if (gate_type_ != GgmlType::IQ2_S && gate_type_ != GgmlType::IQ3_S) return false;
+        const int pairs = tokens_ * k_;
+        for (int p = 0; p < pairs; ++p) {
+            const Pair &e = pair_[p];
+            if (!e.gate || !e.up || !e.down) return false;
+            if ((reinterpret_cast<uintptr_t>(e.gate) | reinterpret_cast<uintptr_t>(e.up) | reinterpret_cast<uintptr_t>(e.down)) & 1u) return false;
+        }
+        if (!check_slots || !ids_) return true;
+        for (int a = 0; a < pairs; ++a)
+            for (int b = a + 1; b < pairs; ++b)
+                if (pair_[b].gate == pair_[a].gate && pair_[b].down == pair_[a].down && ids_[a] != ids_[b]) return false;
+        return true;
+    }
+
+    // src/qwen38_moe.cuh:2955-3109: the routed experts of every token in one pass.  The tensors are named for the
+    // interface's sake; the pass works on the views given pair by pair.
+    void run(Qwen38MoeScratch &scratch, const TensorInfo &, const TensorInfo &, const TensorInfo &, Stream stream) {
+        const int pairs = tokens_ * k_;
+        if (tokens_ < 1 || k_ < 1 || pairs <= 0 || pairs > 128) throw std::runtime_error("MoE token batch pass is not staged");
+        if (!resolved(false)) throw std::runtime_error("MoE token batch pass has unresolved pairs");
+        if (queued_) check(wd_stream_sync(stream), "MoE token batch: waiting for the previous pass failed");  // its copies read the staging below
+        // distinct experts in order of first appearance; a pair's id is the number of its expert's entry
+        std::vector<const uint8_t *> g, u, d;
+        if (!stage_) {
+            void *p = nullptr;
+            check(wd_malloc_host(&p, sizeof(int) * kMoeBatchTokenMax * 16), "pinned allocation failed");
+            stage_ = static_cast<int *>(p);
+        }
+        for (int p = 0; p < pairs; ++p) {
+            int entry = -1;
+            for (size_t q = 0; q < g.size(); ++q)
+                if (g[q] == pair_[p].gate && d[q] == pair_[p].down) entry = static_cast<int>(q);
+            if (entry < 0) {
+                entry = static_cast<int>(g.size());
+                g.push_back(pair_[p].gate), u.push_back(pair_[p].up), d.push_back(pair_[p].down);
+            }
+            stage_[p] = entry;
+        }
+        if (static_cast<int>(g.size()) > scratch.n_experts()) throw std::runtime_error("MoE token batch: more distinct experts than the scratch was made for");
+        std::vector<wd_moe_scratch *> handles;
+        for (int t = 0; t < tokens_; ++t) {
+            Qwen38MoeScratch &q = *tok_[static_cast<size_t>(t)];
+            check(wd_memcpy_h2d(q.d_ids(), stage_ + t * k_, sizeof(int) * k_, stream), "MoE token batch ids upload failed");
+            check(wd_memcpy_h2d(q.d_weights(), weights_ + t * k_, sizeof(float) * k_, stream), "MoE token batch weights upload failed");
+            handles.push_back(q.handle());
+        }
+        if (x_.count < static_cast<size_t>(tokens_) * hidden_) x_.reset(), x_.allocate(static_cast<size_t>(kMoeBatchTokenMax) * hidden_);
+        if (out_.count < static_cast<size_t>(tokens_) * hidden_) out_.reset(), out_.allocate(static_cast<size_t>(kMoeBatchTokenMax) * hidden_);
+        for (int t = 0; t < tokens_; ++t)
+            check(wd_memcpy_d2d(x_.data + static_cast<size_t>(t) * hidden_, activations_[static_cast<size_t>(t)], sizeof(float) * hidden_, stream),
+                  "MoE token batch activation copy failed");
+        wd_moe_layer L;
+        std::memset(&L, 0, sizeof(L));
+        L.hidden = hidden_, L.expert_ffn = ffn_, L.n_experts = scratch.n_experts(), L.top_k = k_, L.expert_scale = 1.0f;
+        L.gate_type = L.up_type = static_cast<int>(gate_type_), L.down_type = static_cast<int>(down_type_);
+        L.router = router_ ? router_ : reinterpret_cast<const float *>(g[0]);  // (not read: the selection is given)
+        check(wd_moe_layer_tokens_pairs_f32(&L, g.data(), u.data(), d.data(), static_cast<int>(g.size()), x_.data, out_.data, tokens_, handles.data(),
+                                            WD_MOE_PRESELECTED, stream),
+              "MoE token batch pass failed");
+        queued_ = true;
+    }
+
+    // src/qwen38_moe.cuh:3111-3113: float [tokens][hidden], every token's routed weighted sum
+    float *accumulated(Qwen38MoeScratch &) { return out_.data; }
+
+    // src/qwen38_moe.cuh:3119-3147: the sums as they are, or rounded to half once
+    void write_output(Qwen38MoeScratch &scratch, float *out_f32_or_null, half_bits *out_half_or_null, Stream stream) {
+        const size_t n = static_cast<size_t>(tokens_) * scratch.hidden();
+        if (out_half_or_null)
+            check(wd_convert_f32_to_f16(out_.data, out_half_or_null, n, stream), "MoE token batch output failed");
+        else if (out_f32_or_null)
+            check(wd_memcpy_d2d(out_f32_or_null, out_.data, sizeof(float) * n, stream), "MoE token batch output failed");
+        else
+            throw std::runtime_error("MoE token batch output failed: no output buffer");
+    }
+
+    ~Qwen38MoeTokenBatch() {
+        if (stage_) wd_free_host(stage_);
+    }
+
+private:
+    struct Pair {
+        const uint8_t *gate = nullptr, *up = nullptr, *down = nullptr;
+    };
+    int tokens_ = 0, k_ = 0, hidden_ = 0, ffn_ = 0;
+    int *ids_ = nullptr, *stage_ = nullptr;
+    float *weights_ = nullptr;
+    const float *router_ = nullptr;
+    bool queued_ = false;
+    GgmlType gate_type_ = GgmlType::F32, down_type_ = GgmlType::F32;
+    std::vector<const float *> activations_;
+    std::vector<std::unique_ptr<Qwen38MoeScratch>> tok_;
+    Pair pair_[kMoeBatchTokenMax * 16];
+    DeviceFloatArray x_, out_;
+};
 
 // The F32 inject projections of the hyper-connection combine (the part of the reference's Qwen38HcF32DebugScratch that
 // the combine reads: hidden(), hc(), inject(); src/qwen38_hc.cuh:2263-2330).
