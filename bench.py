@@ -382,6 +382,7 @@ def bench_lru(args, torch, capi, synth):
     for i in range(args.steps):
         step(base + args.warmup + i)
     ev1.record()
+    host_ms = (time.perf_counter() - t0) * 1e3 / args.steps      # the host's share: queueing a token, nothing awaited
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     s1 = stats()
@@ -410,6 +411,7 @@ def bench_lru(args, torch, capi, synth):
                    "hit_rate": round(hits / max(1, acc), 4), "misses_per_token": round(miss / args.steps, 2),
                    "host_link_bytes_per_token": int(moved / args.steps),
                    "host_link_GBps": round(moved / (ms_per_step * 1e-3 * args.steps) / 1e9, 2),
+                   "host_ms_per_step": round(host_ms, 4),
                    "wall_s": round(wall, 3), "finite": bool(torch.isfinite(d_x).all().item()),
                    "monitor_whole_run": monitor},
         "roofline": {"bound": "hbm", "achieved": round(whole, 1) if whole else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",

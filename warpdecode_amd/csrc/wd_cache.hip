@@ -59,18 +59,37 @@ struct FillSegments {
     uint8_t *dst[kMaxFillSegments];
     uint32_t words[kMaxFillSegments];      // 16-byte words
 };
-__global__ __launch_bounds__(256) void k_fill_slots(FillSegments f) {
-    const int seg = blockIdx.y;
-    const uint4 *src = reinterpret_cast<const uint4 *>(f.src[seg]);
-    uint4 *dst = reinterpret_cast<uint4 *>(f.dst[seg]);
-    const uint32_t n = f.words[seg];
+#ifndef WD_FILL_WGS
+#define WD_FILL_WGS 8      // workgroups of a fill launch, whatever the number of segments (4: the link is no longer kept busy)
+#endif
+#ifndef WD_FILL_UNROLL
+#define WD_FILL_UNROLL 8   // 16-byte words a thread moves per round, all requested before the first is stored
+#endif
+// A few workgroups walk all the segments together.  The link, not the number of workgroups, bounds the rate (256 threads x
+// WD_FILL_UNROLL requests x 16 bytes per workgroup in flight), and every workgroup lives as long as the launch: a launch with
+// one workgroup per piece of every segment filled the compute units with hundreds of workgroups that each waited on the
+// link for most of a millisecond, and the layer kernels of the same period could not place theirs.
+__global__ __launch_bounds__(256) void k_fill_slots(FillSegments f, int n_seg) {
     const uint32_t stride = gridDim.x * 256;
-    uint32_t i = blockIdx.x * 256 + threadIdx.x;
-    for (; i + 3 * stride < n; i += 4 * stride) {  // four requests in flight per thread
-        const uint4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
-        dst[i] = a, dst[i + stride] = b, dst[i + 2 * stride] = c, dst[i + 3 * stride] = d;
+    for (int seg = 0; seg < n_seg; ++seg) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(f.src[seg]);
+        uint4 *dst = reinterpret_cast<uint4 *>(f.dst[seg]);
+        const uint32_t n = f.words[seg];
+        // every round: WD_FILL_UNROLL requests per thread in flight (lanes past the end repeat the last word and store nothing)
+        for (uint32_t base = blockIdx.x * 256 + threadIdx.x; base < n; base += WD_FILL_UNROLL * stride) {
+            uint4 v[WD_FILL_UNROLL];
+#pragma unroll
+            for (int u = 0; u < WD_FILL_UNROLL; ++u) {
+                const uint32_t i = base + u * stride;
+                v[u] = src[i < n ? i : n - 1];
+            }
+#pragma unroll
+            for (int u = 0; u < WD_FILL_UNROLL; ++u) {
+                const uint32_t i = base + u * stride;
+                if (i < n) dst[i] = v[u];
+            }
+        }
     }
-    for (; i < n; i += stride) dst[i] = src[i];
 }
 
 // One thread, in order: a batch may name the same table entry twice (evicted, then filled again).
@@ -302,6 +321,12 @@ struct wd_expert_cache {
     uint64_t prev_floor = 0;     // clock value before the previous acquire call
     bool fills_pending = false;  // a deferred acquire's fills have not been waited for yet
     std::vector<hipEvent_t> ev_layer;      // token-ahead acquires: the fills of layer l are complete
+    std::vector<int> layer_event;          //   ... when ev_layer[layer_event[l]] has passed (fills are launched by groups of layers)
+    int last_waited = -1;                  // the event the caller's stream was last made to wait for in this token
+    hipEvent_t ev_token[2] = {nullptr, nullptr};  // recorded on the caller's stream when a token-ahead acquire begins, alternately
+    int token_parity = 0;
+    bool have_prev_token = false;
+    uint64_t prev_token_floor = 0;         // the clock when the previous token-ahead acquire began
     std::vector<uint8_t> layer_pending;    // ev_layer[l] has been recorded and not yet waited for
     std::vector<const uint8_t *> h_gate, h_up, h_down;
     std::vector<size_t> s_gate, s_up, s_down;  // bytes from one expert to the next in the host tensors
@@ -441,6 +466,8 @@ int wd_expert_cache_destroy(wd_expert_cache *c) {
     (void)hipFree(c->d_updates);
     if (c->h_updates) (void)hipHostFree(c->h_updates);
     if (c->ev_retire) (void)hipEventDestroy(c->ev_retire);
+    for (hipEvent_t ev : c->ev_token)
+        if (ev) (void)hipEventDestroy(ev);
     if (c->ev_done) (void)hipEventDestroy(c->ev_done);
     for (hipEvent_t ev : c->ev_layer)
         if (ev) (void)hipEventDestroy(ev);
@@ -560,8 +587,18 @@ namespace {
 struct AheadState {
     uint64_t floor;
     bool retired;
+    hipEvent_t before = nullptr;  // not null: the fills may start once this event of the caller's stream has passed
     std::vector<SlotUpdate> updates;
+    // Copy-kernel fills are collected over a group of layers and launched together: a launch that moves one expert
+    // reaches 31 GB/s over the host link, one that moves eight 46 GB/s (the fixed cost of a launch is about 20 us).
+    FillSegments fills;
+    int n_fill = 0;
+    uint32_t max_words = 0;
+    std::vector<int> group;  // layers whose fills are queued but not yet covered by an event
 };
+
+int launch_fill_segments(wd_expert_cache *c, FillSegments &fills, int &n_fill, uint32_t &max_words);
+
 
 // Uploads a batch of slot-table changes and applies them in order on the caller's stream.
 int flush_slot_updates(wd_expert_cache *c, const SlotUpdate *updates, int n_updates, hipStream_t st) {
@@ -631,9 +668,12 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
     const bool by_kernel = c->use_copy_kernel && static_cast<size_t>(layer) < c->gpu_readable.size() && c->gpu_readable[layer];
     const bool by_file = !by_kernel && static_cast<size_t>(layer) < c->layer_file.size() && c->layer_file[layer] >= 0 &&
                          !(static_cast<size_t>(layer) < c->gpu_readable.size() && c->gpu_readable[layer]);
-    FillSegments fills;
-    int n_fill = 0;
-    uint32_t max_words = 0;
+    FillSegments own_fills;
+    int own_n_fill = 0;
+    uint32_t own_max_words = 0;
+    FillSegments &fills = ahead ? ahead->fills : own_fills;
+    int &n_fill = ahead ? ahead->n_fill : own_n_fill;
+    uint32_t &max_words = ahead ? ahead->max_words : own_max_words;
 
     // A failure inside the loop (no slot may be recycled, a short read from the file) ends the loop, not the call: the
     // fills and slot-table changes of the experts acquired before it are still issued below, so that the host's index
@@ -686,8 +726,12 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
         if (!waited) {
             // kernels already queued on the caller's stream may still read the victim slot
             if (!ahead || !ahead->retired) {
-                WD_HIP(hipEventRecord(c->ev_retire, st));
-                WD_HIP(hipStreamWaitEvent(c->copy_stream, c->ev_retire, 0));
+                if (ahead && ahead->before) {
+                    WD_HIP(hipStreamWaitEvent(c->copy_stream, ahead->before, 0));
+                } else {
+                    WD_HIP(hipEventRecord(c->ev_retire, st));
+                    WD_HIP(hipStreamWaitEvent(c->copy_stream, c->ev_retire, 0));
+                }
                 if (ahead) ahead->retired = true;
             }
             waited = true;
@@ -734,6 +778,8 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
             c->stage_used[r] = true;
             ++c->pread_fills;
         } else if (by_kernel) {
+            if (n_fill + 3 > kMaxFillSegments)  // (token-ahead groups only: one call alone never has that many)
+                if (const int rc = launch_fill_segments(c, fills, n_fill, max_words)) return rc;
             for (int q = 0; q < 3; ++q) {
                 fills.src[n_fill] = src3[q], fills.dst[n_fill] = dst3[q];
                 fills.words[n_fill] = static_cast<uint32_t>(len3[q] / 16);
@@ -749,12 +795,8 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
         c->stats.bytes_copied += c->slot_bytes;
     }
     c->stats.resident = c->index.size();
-    if (n_fill > 0) {
-        // enough workgroups per segment to keep the host link busy, few enough to leave the decode its compute units
-        const uint32_t per_seg = (max_words + 256 * 16 - 1) / (256 * 16);
-        k_fill_slots<<<dim3(per_seg < 32 ? (per_seg ? per_seg : 1) : 32, n_fill), dim3(256), 0, c->copy_stream>>>(fills);
-        WD_LAUNCH_CHECK();
-    }
+    if (!ahead)
+        if (const int rc = launch_fill_segments(c, fills, n_fill, max_words)) return rc;
 
     if (n_updates > 0) {
         if (ahead) {  // applied once for the whole token, before its first layer
@@ -765,8 +807,7 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
     }
     if (waited) {
         if (ahead) {
-            WD_HIP(hipEventRecord(c->ev_layer[layer], c->copy_stream));
-            c->layer_pending[layer] = 1;
+            ahead->group.push_back(layer);  // the event that covers the layer is recorded when its group is closed
         } else {
             WD_HIP(hipEventRecord(c->ev_done, c->copy_stream));
             if (defer_wait)
@@ -778,6 +819,31 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
     return rc_late;
 }
 
+int launch_fill_segments(wd_expert_cache *c, FillSegments &fills, int &n_fill, uint32_t &max_words) {
+    if (n_fill > 0) {
+        // enough workgroups per segment to keep the host link busy, few enough to leave the decode its compute units
+        const uint32_t per_seg = (max_words + 256 * WD_FILL_UNROLL - 1) / (256 * WD_FILL_UNROLL);
+        k_fill_slots<<<dim3(per_seg < WD_FILL_WGS ? (per_seg ? per_seg : 1) : WD_FILL_WGS), dim3(256), 0, c->copy_stream>>>(fills, n_fill);
+        WD_LAUNCH_CHECK();
+    }
+    n_fill = 0, max_words = 0;
+    return WD_OK;
+}
+// Launches what the group has collected and records the event its layers wait for.
+int close_ahead_group(wd_expert_cache *c, AheadState &ahead) {
+    if (const int rc = launch_fill_segments(c, ahead.fills, ahead.n_fill, ahead.max_words)) return rc;
+    if (!ahead.group.empty()) {
+        const int last = ahead.group.back();
+        WD_HIP(hipEventRecord(c->ev_layer[last], c->copy_stream));
+        for (int l : ahead.group) c->layer_pending[l] = 1, c->layer_event[l] = last;
+        ahead.group.clear();
+    }
+    return WD_OK;
+}
+
+#ifndef WD_AHEAD_GROUP
+#define WD_AHEAD_GROUP 8  // layers per group of fills at most (the first groups are 1, 1, 2, 4 layers: the first layers wait least)
+#endif
 // Acquires the experts of every layer of one token before any of the token's layers is launched, so that the host
 // link streams the token's misses back to back while the layers compute; wait_layer_fills(l) then makes the stream
 // wait for layer l's fills only.  Needs a pool that holds a whole token: the slots a token touches are not evicted
@@ -786,13 +852,36 @@ int acquire_token_ahead(wd_expert_cache *c, int n_layers, const int32_t *h_ids, 
     if (c->ev_layer.size() < static_cast<size_t>(c->n_layers)) {
         c->ev_layer.resize(c->n_layers, nullptr);
         c->layer_pending.assign(c->n_layers, 0);
+        c->layer_event.assign(c->n_layers, 0);
         for (hipEvent_t &ev : c->ev_layer)
             if (!ev) WD_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
     }
-    AheadState ahead{c->clock, false, {}};
-    int rc_late = WD_OK;
-    for (int l = 0; l < n_layers && rc_late == WD_OK; ++l)
+    AheadState ahead;
+    ahead.floor = c->clock, ahead.retired = false;
+    c->last_waited = -1;
+    // A pool that holds three tokens' experts always has a victim that the previous token did not touch either: such a
+    // slot was last read by work queued before the previous token, so this token's fills need not wait for the previous
+    // token's layers - they wait for the event recorded when the previous token was queued, and cross the host link
+    // while its layers compute.
+    if (!c->ev_token[0])
+        for (hipEvent_t &ev : c->ev_token) WD_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+    const Partition &P0 = c->parts[0];
+    const bool relaxed = !c->partitioned && c->have_prev_token && P0.end - P0.begin >= 3 * static_cast<size_t>(n_layers) * k;
+    WD_HIP(hipEventRecord(c->ev_token[c->token_parity], as_stream(stream)));  // everything queued before this token
+    if (relaxed) {
+        ahead.floor = c->prev_token_floor;
+        ahead.before = c->ev_token[c->token_parity ^ 1];
+    }
+    c->prev_token_floor = c->clock, c->have_prev_token = true, c->token_parity ^= 1;
+    int rc_late = WD_OK, group_end = 1, group_len = 1;
+    for (int l = 0; l < n_layers && rc_late == WD_OK; ++l) {
         rc_late = acquire_impl(c, l, h_ids + static_cast<size_t>(l) * k, k, nullptr, stream, true, &ahead);
+        if (l + 1 == group_end || l + 1 == n_layers || rc_late != WD_OK) {
+            if (const int rc = close_ahead_group(c, ahead)) return rc;
+            group_len = l + 1 < 2 ? 1 : (2 * group_len < WD_AHEAD_GROUP ? 2 * group_len : WD_AHEAD_GROUP);
+            group_end = l + 1 + group_len;
+        }
+    }
     // also after a failure: the table must describe what the layers before it did to the pool
     const int rc = flush_slot_updates(c, ahead.updates.data(), static_cast<int>(ahead.updates.size()), as_stream(stream));
     return rc_late != WD_OK ? rc_late : rc;
@@ -800,7 +889,9 @@ int acquire_token_ahead(wd_expert_cache *c, int n_layers, const int32_t *h_ids, 
 
 int wait_layer_fills(wd_expert_cache *c, int layer, hipStream_t st) {
     if (static_cast<size_t>(layer) < c->layer_pending.size() && c->layer_pending[layer]) {
-        WD_HIP(hipStreamWaitEvent(st, c->ev_layer[layer], 0));
+        // the layers of a group wait for one event: the stream is told once (the call costs the host about 20 us)
+        if (c->layer_event[layer] != c->last_waited) WD_HIP(hipStreamWaitEvent(st, c->ev_layer[c->layer_event[layer]], 0));
+        c->last_waited = c->layer_event[layer];
         c->layer_pending[layer] = 0;
     }
     return WD_OK;
