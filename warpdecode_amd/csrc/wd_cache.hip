@@ -60,23 +60,30 @@ struct FillSegments {
     uint32_t words[kMaxFillSegments];      // 16-byte words
 };
 #ifndef WD_FILL_WGS
-#define WD_FILL_WGS 8      // workgroups of a fill launch, whatever the number of segments (4: the link is no longer kept busy)
+#define WD_FILL_WGS 20     // workgroups of a fill launch, whatever the number of segments
 #endif
 #ifndef WD_FILL_UNROLL
 #define WD_FILL_UNROLL 8   // 16-byte words a thread moves per round, all requested before the first is stored
 #endif
-// A few workgroups walk all the segments together.  The link, not the number of workgroups, bounds the rate (256 threads x
-// WD_FILL_UNROLL requests x 16 bytes per workgroup in flight), and every workgroup lives as long as the launch: a launch with
-// one workgroup per piece of every segment filled the compute units with hundreds of workgroups that each waited on the
-// link for most of a millisecond, and the layer kernels of the same period could not place theirs.
-__global__ __launch_bounds__(256) void k_fill_slots(FillSegments f, int n_seg) {
-    const uint32_t stride = gridDim.x * 256;
+// A few one-wave workgroups walk all the segments together.  The link, not the number of workgroups, bounds the rate
+// (160 KB in flight keep it at 50 GB/s and more), and every workgroup lives as long as the launch, so what matters is
+// how little the launch disturbs the layer kernels that run beside it.  Measured on the mode B workload (tokens per
+// second at a hit rate of 0.93): one workgroup of 256 threads per piece of every segment 400 (hundreds of workgroups
+// that each wait on the link for most of a millisecond: the layer kernels could not place theirs); 8 x 256 threads for
+// the whole launch 570 (k_layer_ab 22.6 instead of 16 us: the compute units that host a fill workgroup serve their
+// layer workgroups late, and the grid waits for those); 32 x 64 threads 589, 24 x 64 642, 20 x 64 670, 16 x 64 582
+// (the link is no longer kept busy).
+#ifndef WD_FILL_THREADS
+#define WD_FILL_THREADS 64
+#endif
+__global__ __launch_bounds__(WD_FILL_THREADS) void k_fill_slots(FillSegments f, int n_seg) {
+    const uint32_t stride = gridDim.x * WD_FILL_THREADS;
     for (int seg = 0; seg < n_seg; ++seg) {
         const uint4 *src = reinterpret_cast<const uint4 *>(f.src[seg]);
         uint4 *dst = reinterpret_cast<uint4 *>(f.dst[seg]);
         const uint32_t n = f.words[seg];
         // every round: WD_FILL_UNROLL requests per thread in flight (lanes past the end repeat the last word and store nothing)
-        for (uint32_t base = blockIdx.x * 256 + threadIdx.x; base < n; base += WD_FILL_UNROLL * stride) {
+        for (uint32_t base = blockIdx.x * WD_FILL_THREADS + threadIdx.x; base < n; base += WD_FILL_UNROLL * stride) {
             uint4 v[WD_FILL_UNROLL];
 #pragma unroll
             for (int u = 0; u < WD_FILL_UNROLL; ++u) {
@@ -822,8 +829,8 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
 int launch_fill_segments(wd_expert_cache *c, FillSegments &fills, int &n_fill, uint32_t &max_words) {
     if (n_fill > 0) {
         // enough workgroups per segment to keep the host link busy, few enough to leave the decode its compute units
-        const uint32_t per_seg = (max_words + 256 * WD_FILL_UNROLL - 1) / (256 * WD_FILL_UNROLL);
-        k_fill_slots<<<dim3(per_seg < WD_FILL_WGS ? (per_seg ? per_seg : 1) : WD_FILL_WGS), dim3(256), 0, c->copy_stream>>>(fills, n_fill);
+        const uint32_t per_seg = (max_words + WD_FILL_THREADS * WD_FILL_UNROLL - 1) / (WD_FILL_THREADS * WD_FILL_UNROLL);
+        k_fill_slots<<<dim3(per_seg < WD_FILL_WGS ? (per_seg ? per_seg : 1) : WD_FILL_WGS), dim3(WD_FILL_THREADS), 0, c->copy_stream>>>(fills, n_fill);
         WD_LAUNCH_CHECK();
     }
     n_fill = 0, max_words = 0;
