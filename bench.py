@@ -61,6 +61,13 @@ def parse():
                          "misses read with pread into the cache's pinned ring; the same file as a plain (pageable) mapping")
     ap.add_argument("--file-dir", default="/tmp", help="lru mode with --source file/mapping: directory of the model file")
     ap.add_argument("--pread-threads", type=int, default=4)
+    ap.add_argument("--lru-driver", choices=["trace", "router"], default="trace",
+                    help="lru mode: the host knows the routing trace and acquires a token's experts ahead (default), or every layer's "
+                         "selection comes back from the device before its experts are acquired (what a decode loop without a "
+                         "predictor does)")
+    ap.add_argument("--read-ahead", type=int, default=0,
+                    help="lru mode with --lru-driver router and --source file: layers of read-ahead (the previous token's experts are "
+                         "read from the file into a pinned ring while the layers compute)")
     ap.add_argument("--cache-warm-tokens", type=int, default=256,
                     help="lru mode: tokens run before the warm-up steps so that the slot pool is in steady state")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a captured HIP graph")
@@ -354,8 +361,15 @@ def bench_lru(args, torch, capi, synth):
     d_out = torch.zeros(H, dtype=torch.float32, device="cuda")
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
+    if args.read_ahead:
+        capi.call("wd_expert_cache_set_read_ahead", cache, args.read_ahead, 0)
+
     def step(i):
         d_x.copy_(d_xs[i % 64], non_blocking=True)
+        if args.lru_driver == "router":   # the router's own selection, layer by layer through the host
+            capi.call("wd_moe_stack_cached_f32", layers, NL, cache, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()),
+                      scratch, None, None, RESIDUAL_SCALE, 0, stream)
+            return
         capi.call("wd_moe_stack_cached_f32", layers, NL, cache, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()),
                   scratch, trace[i].ctypes.data_as(C.c_void_p), C.c_void_p(d_trace_all[i].data_ptr()), RESIDUAL_SCALE, 0, stream)
 
@@ -406,7 +420,8 @@ def bench_lru(args, torch, capi, synth):
         "data": "synthetic",
         "config": {"workload": "C3 mode B: %d-layer stack of the 512-expert top-10 IQ3_S/Q8_0 MoE layer, batch=1, routed "
                                "experts in pinned host memory behind a %.0f GiB LRU slot pool in HBM, Zipf(1.1) trace" % (NL, args.cache_gib),
-                   "layers": NL, "experts": E, "top_k": k, "routing": "zipf", "launch": "eager", "source": args.source,
+                   "layers": NL, "experts": E, "top_k": k, "routing": "zipf" if args.lru_driver == "trace" else "router", "launch": "eager",
+                   "source": args.source, "driver": args.lru_driver, "read_ahead": args.read_ahead,
                    "slots": int(s1.slots), "slot_bytes": int(slot_bytes), "cache_warm_tokens": args.cache_warm_tokens,
                    "hit_rate": round(hits / max(1, acc), 4), "misses_per_token": round(miss / args.steps, 2),
                    "host_link_bytes_per_token": int(moved / args.steps),

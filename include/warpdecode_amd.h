@@ -353,6 +353,15 @@ int wd_expert_cache_get_stats(wd_expert_cache *c, wd_expert_cache_stats *out);
  * and 16-byte aligned (default), else - or with enabled = 0 - by hipMemcpyAsync per piece.  No counterpart in the
  * reference (its fills are cudaMemcpyAsync per contiguous run, src/expert_cache.cuh:1166-1254). */
 int wd_expert_cache_set_copy_kernel(wd_expert_cache *c, int enabled);
+/* Read-ahead for file-backed layers when the router decides layer by layer what is needed (no trace known to the host):
+ * at a layer's first acquire of a token, the experts the previous token took in this layer and the next depth - 1 ones,
+ * as far as they are not resident, are read from the file by a reader thread into a ring of `slots` pinned buffers laid
+ * out like a slot (0: depth * 16); an acquire that then wants one of them queues its DMA from that buffer instead of
+ * reading the file itself.  A prediction that comes true puts the same bytes into the slot as the on-demand read; one
+ * that does not only wastes a read.  depth 0 switches it off.  Counters: "read_ahead" in wd_expert_cache_dump_json.
+ * reference: ExpertReadAhead, ExpertStagePath::note_access / post_prefetch, ExpertCacheOptions::prefetch_depth
+ * (src/expert_cache.cuh:105-114, :547-824, :1094-1153). */
+int wd_expert_cache_set_read_ahead(wd_expert_cache *c, int depth, int slots);
 /* File-backed fills: a read-only mapping [map_base, map_base + map_bytes) of the file behind `fd` (the cache keeps its
  * own duplicate of the descriptor).  Layers whose registered host tensors lie inside the mapping and are not pinned are
  * then filled by pread() of the expert's slices into a pinned ring (`threads` readers share every expert) and one DMA per

@@ -159,3 +159,55 @@ def test_cached_stack_streams_experts_from_the_mapping(g, oracle, layers, tmp_pa
             assert mon["fills_by_pread"] == st.misses and mon["fills_by_memcpy"] == 0 and mon["fills_by_copy_kernel"] == 0
         sc.close()
         capi.call("wd_expert_cache_destroy", cache)
+
+
+@pytest.mark.parametrize("depth", [1, 2])
+def test_read_ahead_serves_router_driven_misses(g, oracle, layers, tmp_path, depth):
+    """No trace known to the host: every layer's selection comes back from the device before its experts are acquired.
+    With read-ahead on, the experts the previous token took are read from the file while the layers compute, and a miss
+    that was predicted is filled from the ring.  The pool (8 slots for 3 layers x 4 experts per token) cannot keep a
+    token's experts until the next token, so a token that repeats the previous input misses everywhere and every
+    prediction comes true.  Whatever the source of a fill, the results are the oracle's."""
+    import json
+    gb = F * synth.row_bytes(synth.IQ3_S, H)
+    db = H * synth.row_bytes(synth.Q8_0, F)
+    with ggufio.GgufFile(_write(tmp_path, layers, False)) as gf:
+        Ls = [_layer_from_file(gf, l) for l in range(NL)]
+        cache = C.c_void_p()
+        capi.call("wd_expert_cache_create", C.byref(cache), 8 * (2 * gb + db), gb, gb, db, NL, E, 0)
+        capi.call("wd_expert_cache_attach_file", cache, C.c_void_p(gf.map_base), gf.map_bytes, gf.fd, 2)
+        for l, L in enumerate(Ls):
+            ptr = lambda a: C.c_void_p(a.ctypes.data)
+            capi.call("wd_expert_cache_register_layer", cache, l, ptr(L["gate"]), ptr(L["up"]), ptr(L["down"]))
+        capi.call("wd_expert_cache_set_read_ahead", cache, depth, 0)
+        dls, arr = _descs(g, [dict(L, gate=L["gate"][:1], up=L["up"][:1], down=L["down"][:1]) for L in Ls])
+        for i in range(NL):
+            arr[i].gate = arr[i].up = arr[i].down = None
+        sc = g.Scratch(H, F, E, K)
+        lib = capi.load()
+        xs = [synth.rms_normed(synth.rng_for(SEED, 143, i // 2), H) for i in range(8)]     # every input twice in a row
+        for step, x in enumerate(xs):
+            dx, out = g.dev(x), g.empty(H, np.float32)
+            capi.call("wd_moe_stack_cached_f32", arr, NL, cache, g.ptr(dx), g.ptr(out), sc.h, None, None, float(SCALE), 0, g.stream())
+            g.sync()
+            wx, wout = _oracle_stack(oracle, layers, x)
+            assert g.same_bits(g.host(dx), wx), step
+            assert g.same_bits(g.host(out), wout), step
+            import time
+            time.sleep(0.05)         # the reader works in the background: give it the time a real layer stack would
+        buf = C.create_string_buffer(1 << 16)
+        lib.wd_expert_cache_dump_json(cache, buf, len(buf))
+        mon = json.loads(buf.value.decode())
+        ra = mon["read_ahead"]
+        assert ra["depth"] == depth and ra["slots"] == 16 * depth
+        assert ra["posted"] > 0 and ra["delivered"] > 0 and ra["failed"] == 0
+        assert ra["fills"] > 0, ra                                           # predictions that came true were served from the ring
+        assert ra["fills"] + mon["fills_by_pread"] == mon["misses"]          # every other miss took the on-demand path
+        capi.call("wd_expert_cache_set_read_ahead", cache, 0, 0)             # off again: the ring is released
+        dx, out = g.dev(xs[0]), g.empty(H, np.float32)
+        capi.call("wd_moe_stack_cached_f32", arr, NL, cache, g.ptr(dx), g.ptr(out), sc.h, None, None, float(SCALE), 0, g.stream())
+        g.sync()
+        assert g.same_bits(g.host(out), _oracle_stack(oracle, layers, xs[0])[1])
+        assert lib.wd_expert_cache_set_read_ahead(cache, 9, 0) == -1
+        sc.close()
+        capi.call("wd_expert_cache_destroy", cache)

@@ -123,6 +123,7 @@ _OPTIONAL = {
     "wd_expert_cache_slot_of": (C.c_longlong, [vp, i32, i32]),
     "wd_expert_cache_add_shadow": (i32, [vp, i32, sz]),
     "wd_expert_cache_set_copy_kernel": (i32, [vp, i32]),
+    "wd_expert_cache_set_read_ahead": (i32, [vp, i32, i32]),
     "wd_expert_cache_attach_file": (i32, [vp, vp, sz, i32, i32]),
     "wd_expert_cache_dump_json": (sz, [vp, C.c_char_p, sz]),
     "wd_gguf_open": (i32, [C.POINTER(vp), C.c_char_p]),

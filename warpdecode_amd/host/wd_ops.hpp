@@ -322,6 +322,8 @@ struct ExpertCacheOptions {
     bool stats = false;
     bool layer_evict = false;
     int layer_count = 0;
+    int prefetch_depth = 0;  // layers of read-ahead for file-backed experts (src/expert_cache.cuh:105-112); 0 = off
+    int prefetch_slots = 0;  // 0 = prefetch_depth * 16
 };
 
 // src/expert_cache.cuh:2148-2154
@@ -374,7 +376,11 @@ public:
         wd_expert_cache_stats st{};
         wd_expert_cache_get_stats(c_, &st);
         n_slots_ = static_cast<size_t>(st.slots);
+        if (options.prefetch_depth > 0)
+            check(wd_expert_cache_set_read_ahead(c_, options.prefetch_depth, options.prefetch_slots), "expert read-ahead setup failed");
     }
+    // layers of read-ahead in force (src/expert_cache.cuh:2229)
+    void set_prefetch_depth(int depth, int slots = 0) { check(wd_expert_cache_set_read_ahead(c_, depth, slots), "expert read-ahead setup failed"); }
 
     size_t slot_count() const { return n_slots_; }
     size_t slot_bytes() const { return slot_bytes_; }
