@@ -204,7 +204,9 @@ float *wd_moe_scratch_shared_gate(wd_moe_scratch *s); /* f32 [1] sigmoid gate (d
 int32_t *wd_moe_scratch_gate_up_partials(wd_moe_scratch *s); /* NULL until enabled */
 int32_t *wd_moe_scratch_down_partials(wd_moe_scratch *s);
 /* Allocates the int32 chunk-sum dumps ([k][2][ffn][P_gate] and [k][hidden][P_down]) and makes the
- * layer pass fill them.  Parity harness only. */
+ * layer pass fill them: variants of the fused dispatches store them beside their results when the
+ * gate/up rows are IQ3_S or IQ2_S; other layers, and WD_MOE_STAGED, take one dispatch per operator.
+ * The shared expert's sums are not part of the dump.  Parity harness only. */
 int wd_moe_scratch_enable_partials(wd_moe_scratch *s, int gate_type, int down_type);
 
 /* Profiling aid: makes the fused layer dispatches record 100 MHz time stamps of workgroup `wg` and returns the

@@ -51,34 +51,29 @@ def run_layer(g, L, x, partials=True, flags=0, ids=None, weights=None):
 
 
 def check_layer(g, oracle, L, x, **kw):
-    """Staged pass (one dispatch per operator, int32 chunk sums exported) and fused pass (three
-    dispatches) against the oracle."""
+    """Three passes against the oracle: the fused dispatches, the fused dispatches with the int32 chunk sums
+    exported (layers whose gate rows are not of a kind the fused kernels export take the staged dispatches for
+    this by themselves), and the staged dispatches (one per operator, which also leave the quantised activation
+    in the scratch)."""
     want, d = oracle.moe_layer(L, x, ids=kw.get("ids"), weights=kw.get("weights"), want_partials=True)
-    fused = run_layer(g, L, x, partials=False, **kw)
-    assert np.array_equal(fused["ids"], d["ids"])
-    assert g.same_bits(fused["weights"], d["weights"])
-    if kw.get("ids") is None:
-        assert g.same_bits(fused["logits"], d["logits"])
-    assert g.same_bits(fused["act"], d["act"])
-    assert g.same_bits(fused["accum"], d["routed"])
-    if L.get("shared_gate_inp") is not None:
-        assert g.same_bits(fused["shared_gate"], d["shared_gate"])
-        assert g.same_bits(fused["down_f32"], d["shared_out"])
-    assert g.same_bits(fused["out"], want)
-    got = run_layer(g, L, x, **kw)
-    assert np.array_equal(got["ids"], d["ids"])
-    assert g.same_bits(got["weights"], d["weights"])
-    if kw.get("ids") is None:
-        assert g.same_bits(got["logits"], d["logits"])
-    assert np.array_equal(got["gate_up_partials"], d["gate_up_partials"])
-    assert g.same_bits(got["act"], d["act"])
-    assert np.array_equal(got["act_qs"], d["act_qs"]) and np.array_equal(got["act_d"], d["act_d"])
-    assert np.array_equal(got["down_partials"], d["down_partials"])
-    assert g.same_bits(got["accum"], d["routed"])
-    if L.get("shared_gate_inp") is not None:
-        assert g.same_bits(got["shared_gate"], d["shared_gate"])
-        assert g.same_bits(got["down_f32"], d["shared_out"])
-    assert g.same_bits(got["out"], want)
+    base = kw.pop("flags", 0)
+    for partials, flags in ((False, base), (True, base), (True, base | capi.MOE_STAGED)):
+        got = run_layer(g, L, x, partials=partials, flags=flags, **kw)
+        assert np.array_equal(got["ids"], d["ids"])
+        assert g.same_bits(got["weights"], d["weights"])
+        if kw.get("ids") is None:
+            assert g.same_bits(got["logits"], d["logits"])
+        assert g.same_bits(got["act"], d["act"])
+        assert g.same_bits(got["accum"], d["routed"])
+        if partials:
+            assert np.array_equal(got["gate_up_partials"], d["gate_up_partials"])
+            assert np.array_equal(got["down_partials"], d["down_partials"])
+        if flags & capi.MOE_STAGED:
+            assert np.array_equal(got["act_qs"], d["act_qs"]) and np.array_equal(got["act_d"], d["act_d"])
+        if L.get("shared_gate_inp") is not None:
+            assert g.same_bits(got["shared_gate"], d["shared_gate"])
+            assert g.same_bits(got["down_f32"], d["shared_out"])
+        assert g.same_bits(got["out"], want)
     rel = np.linalg.norm(got["out"] - want) / max(np.linalg.norm(want), 1e-30)
     assert rel <= 1e-5
     return got

@@ -47,6 +47,9 @@ struct LayerArgs {
     unsigned spin_limit;         // polls (about a microsecond each) before such a wait gives up
     unsigned long long *trace;   // profiling aid: null, or [3][16][8] time stamps (100 MHz) of workgroup trace_wg
     int trace_wg;
+    // the PART variants of the dispatches also store the exact int32 chunk sums of the routed rows:
+    int32_t *gup_part;           // [k][2][F][8 * H / 256]
+    int32_t *down_part;          // [k][H][8 * F / 32]
 };
 
 constexpr int kTagCopies = 16;           // replicas of the published ids, 64 bytes apart, so that pollers spread over lines
@@ -762,7 +765,7 @@ __global__ __launch_bounds__(512) void k_layer_a(LayerArgs a) {
 // NB (COAL only): super-blocks per row, 8 (hidden 2048) or 10 (hidden 2560).
 // LOOP: the grid has fewer routed workgroups than there are (expert rung, group of eight rows) items; they walk them
 // with the stride of their number.
-template <int TYPE, bool COAL, int NB = 8, bool LOOP = false>
+template <int TYPE, bool COAL, int NB = 8, bool LOOP = false, bool PART = false>
 __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
     constexpr bool kIq = (TYPE == 21 || TYPE == 22);
     extern __shared__ __align__(16) uint8_t lds_ab[];
@@ -877,15 +880,18 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
             const size_t rb = static_cast<size_t>(nb) * (TYPE == 21 ? 110 : 82);
             const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
             const uint8_t *const rows[2] = {uniform_ptr(gate + off), uniform_ptr(up + off)};  // one row pair per wave
+            // (PART) the chunk sums of the pair: gate row r of rung j, the up row F rows further on
+            const size_t pg = static_cast<size_t>(nb) * 8;
+            int32_t *pp = PART ? a.gup_part + (static_cast<size_t>(j) * 2 * a.F + min(r, a.F - 1)) * pg : nullptr;
             if (COAL && NB == 10)
-                iq_rows10_coal<(kIq ? TYPE : 21), 2>(rows, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
-                                                     lds_ab + ((4 * a.H + 16 + 15) & ~15) + wave * 2 * kIqStage10Bytes);
+                iq_rows10_coal<(kIq ? TYPE : 21), 2, PART>(rows, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
+                                                           lds_ab + ((4 * a.H + 16 + 15) & ~15) + wave * 2 * kIqStage10Bytes, pp, a.F * pg);
             else if (COAL)
-                iq_rows8_coal<(kIq ? TYPE : 21), 2>(rows, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
-                                                    lds_ab + ((4 * a.H + 16 + 15) & ~15) + wave * 2 * kIqStageBytes);
+                iq_rows8_coal<(kIq ? TYPE : 21), 2, PART>(rows, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
+                                                          lds_ab + ((4 * a.H + 16 + 15) & ~15) + wave * 2 * kIqStageBytes, pp, a.F * pg);
             else
-                iq_rows_q8k<(kIq ? TYPE : 21), 2, false>(rows, nb, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
-                                                          nullptr, 0);
+                iq_rows_q8k<(kIq ? TYPE : 21), 2, PART>(rows, nb, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu, pp,
+                                                         a.F * pg);
         } else {
             Q8RowTile *tiles = reinterpret_cast<Q8RowTile *>(s_union);
             const int nb = a.H >> 5;
@@ -909,7 +915,7 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
 // IQ4_NL: 256-thread workgroups, four row pairs per wave, grid = k * ceil(F / 16).
 // Every wave first requests its weight bytes; the workgroup then stages the codebooks and quantises x
 // while they are in flight.  dynamic LDS: quantised x (H bytes + scales).
-template <int TYPE>
+template <int TYPE, bool PART = false>
 __global__ __launch_bounds__(TYPE == 20 ? 256 : 512) void k_layer_b(LayerArgs a) {
     constexpr bool kIq = (TYPE == 21 || TYPE == 22);
     constexpr int kThreads = (TYPE == 20) ? 256 : 512;
@@ -938,8 +944,10 @@ __global__ __launch_bounds__(TYPE == 20 ? 256 : 512) void k_layer_b(LayerArgs a)
         const size_t off = static_cast<size_t>(min(r, a.F - 1)) * rb;
         const uint8_t *const rows[2] = {gate + off, up + off};
         float gu[2];
-        iq_rows_q8k<(kIq ? TYPE : 21), 2, false>(rows, nb, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
-                                                  nullptr, 0, [&]() {
+        const size_t pg = static_cast<size_t>(nb) * 8;
+        int32_t *pp = PART ? a.gup_part + (static_cast<size_t>(j) * 2 * a.F + min(r, a.F - 1)) * pg : nullptr;
+        iq_rows_q8k<(kIq ? TYPE : 21), 2, PART>(rows, nb, tables, xq, reinterpret_cast<const float *>(xscale), lane, gu,
+                                                 pp, a.F * pg, [&]() {
             stage_tables<TYPE == 21, TYPE == 22>(tables, threadIdx.x, kThreads);
             for (int b = wave; b < (a.H >> 8); b += kThreads / 64)
                 wave_quantize_q8_k_block(a.x + b * 256, xq + b * 256, reinterpret_cast<float *>(xscale) + b, lane);
@@ -996,7 +1004,7 @@ __global__ __launch_bounds__(TYPE == 20 ? 256 : 512) void k_layer_b(LayerArgs a)
 // products, which keeps it within 80 registers: the waves of a workgroup go to the four SIMDs in turn, so three
 // workgroups of six waves need six wave slots on two of them.  dynamic LDS per wave: two quantised activations and a
 // staging area of 4 * NB * 34 bytes.
-template <int KIND, bool COAL, int NB = 16, bool TWO = false>
+template <int KIND, bool COAL, int NB = 16, bool TWO = false, bool PART = false>
 __global__ __launch_bounds__(TWO ? 576 : 1024) __attribute__((amdgpu_waves_per_eu(TWO ? 6 : 4)))
 void k_layer_c(LayerArgs a) {
     extern __shared__ __align__(16) uint8_t lds_c[];
@@ -1098,8 +1106,14 @@ void k_layer_c(LayerArgs a) {
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
             if (q == 1 && !second) break;
-            const float y = (KIND == 0 || sh[q]) ? q8_rows4_coal_dots<0, NB>(stage2[q], aq2[q], ad2[q], tiles[wave], lane)
-                                                 : q8_rows4_coal_dots<KIND, NB>(stage2[q], aq2[q], ad2[q], tiles[wave], lane);
+            float y;
+            if (PART && !sh[q]) {  // (the shared expert's sums are not part of the dump)
+                int32_t *pp = a.down_part + (static_cast<size_t>(mm[q]) * a.H + r0) * (NB * 8);
+                y = q8_rows4_coal_dots<KIND, NB, PART>(stage2[q], aq2[q], ad2[q], tiles[wave], lane, pp);
+            } else {
+                y = (KIND == 0 || sh[q]) ? q8_rows4_coal_dots<0, NB>(stage2[q], aq2[q], ad2[q], tiles[wave], lane)
+                                         : q8_rows4_coal_dots<KIND, NB>(stage2[q], aq2[q], ad2[q], tiles[wave], lane);
+            }
             if ((lane & 15) == 0) ybuf[mm[q] * 4 + r4] = y;
             mark(a, 2, q == 0 ? 2 : 5);
         }
@@ -1118,13 +1132,17 @@ void k_layer_c(LayerArgs a) {
                 wave_lds_fence();
                 quantise_act(v, aq, ad);
                 mark(a, 2, 1);
-                y = q8_rows4_coal_finish<0, NB>(raw, aq, ad, tiles[wave], lane);
+                if (PART && !is_shared)
+                    y = q8_rows4_coal_finish<0, NB, PART>(raw, aq, ad, tiles[wave], lane, a.down_part + (static_cast<size_t>(m) * a.H + r0) * (NB * 8));
+                else
+                    y = q8_rows4_coal_finish<0, NB>(raw, aq, ad, tiles[wave], lane);
             } else {
                 const auto raw = q8_rows4_coal_request<1, NB>(w + static_cast<size_t>(r0) * NB * 18, lane);
                 wave_lds_fence();
                 quantise_act(v, aq, ad);
                 mark(a, 2, 1);
-                y = q8_rows4_coal_finish<1, NB>(raw, aq, ad, tiles[wave], lane);
+                y = q8_rows4_coal_finish<1, NB, PART>(raw, aq, ad, tiles[wave], lane,
+                                                      PART ? a.down_part + (static_cast<size_t>(m) * a.H + r0) * (NB * 8) : nullptr);
             }
             if ((lane & 15) == 0) ybuf[m * 4 + r4] = y;
         } else {
@@ -1139,10 +1157,13 @@ void k_layer_c(LayerArgs a) {
                 wave_lds_fence();
                 mark(a, 2, 1);
             };
-            if (KIND == 0 || is_shared)
+            int32_t *pp = (PART && !is_shared) ? a.down_part + (static_cast<size_t>(m) * a.H + r0) * (static_cast<size_t>(nb) * 8) : nullptr;
+            if (PART && !is_shared && KIND == 0)
+                q8_rows4_multi<0, 1, 1, PART>(rows, nrows, nb, aq, ad, tiles[wave], lane, y, pp, 0, quantise);
+            else if (KIND == 0 || is_shared)
                 q8_rows4_multi<0, 1, 1, false>(rows, nrows, nb, aq, ad, tiles[wave], lane, y, nullptr, 0, quantise);
             else
-                q8_rows4_multi<1, 1, 1, false>(rows, nrows, nb, aq, ad, tiles[wave], lane, y, nullptr, 0, quantise);
+                q8_rows4_multi<1, 1, 1, PART>(rows, nrows, nb, aq, ad, tiles[wave], lane, y, pp, 0, quantise);
             if ((lane & 15) == 0) ybuf[m * 4 + r4] = y[0];
         }
         mark(a, 2, 2);

@@ -444,6 +444,10 @@ LayerArgs fused_args(const wd_moe_layer *L, const float *d_x, float *d_out, wd_m
     a.clear_tagged = 1;
     a.status = s->status;
     a.spin_limit = s->spin_limit;
+    // the chunk sums go out of the fused dispatches when the scratch was asked to keep them and the gate/up rows are of
+    // the kinds whose fused kernels export them (other layers take the staged dispatches for that)
+    if (s->gup && !(flags & WD_MOE_STAGED) && consumes_q8k(L->gate_type) && s->gup_type == L->gate_type && s->dp_type == L->down_type)
+        a.gup_part = s->gup, a.down_part = s->dp;
     return a;
 }
 
@@ -460,10 +464,22 @@ int launch_a(const LayerArgs &a, hipStream_t st) {
 // One layer in three dispatches (router + shared gate/up, routed gate/up, down + combine).
 template <int TYPE, bool COAL, int NB>
 void launch_layer_ab(bool loop, dim3 grid, dim3 block, size_t lds, hipStream_t st, const LayerArgs &m) {
-    if (loop)
+    const bool part = m.gup_part != nullptr;  // the variants that also store the int32 chunk sums
+    if (loop && part)
+        k_layer_ab<TYPE, COAL, NB, true, true><<<grid, block, lds, st>>>(m);
+    else if (loop)
         k_layer_ab<TYPE, COAL, NB, true><<<grid, block, lds, st>>>(m);
+    else if (part)
+        k_layer_ab<TYPE, COAL, NB, false, true><<<grid, block, lds, st>>>(m);
     else
         k_layer_ab<TYPE, COAL, NB, false><<<grid, block, lds, st>>>(m);
+}
+template <int KIND, bool COAL, int NB, bool TWO>
+void launch_layer_c(dim3 grid, dim3 block, size_t lds, hipStream_t st, const LayerArgs &a) {
+    if (a.down_part)
+        k_layer_c<KIND, COAL, NB, TWO, true><<<grid, block, lds, st>>>(a);
+    else
+        k_layer_c<KIND, COAL, NB, TWO><<<grid, block, lds, st>>>(a);
 }
 
 int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_scratch *s, unsigned flags,
@@ -525,8 +541,14 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
     const int grid_b = k * (L->gate_type == WD_TYPE_IQ4_NL ? (F + 15) / 16 : (F + 7) / 8);
     if (run_b && !merged) {
         switch (L->gate_type) {
-            case WD_TYPE_IQ3_S: k_layer_b<21><<<dim3(grid_b), dim3(512), lds_b, st>>>(a); break;
-            case WD_TYPE_IQ2_S: k_layer_b<22><<<dim3(grid_b), dim3(512), lds_b, st>>>(a); break;
+            case WD_TYPE_IQ3_S:
+                if (a.gup_part) k_layer_b<21, true><<<dim3(grid_b), dim3(512), lds_b, st>>>(a);
+                else k_layer_b<21><<<dim3(grid_b), dim3(512), lds_b, st>>>(a);
+                break;
+            case WD_TYPE_IQ2_S:
+                if (a.gup_part) k_layer_b<22, true><<<dim3(grid_b), dim3(512), lds_b, st>>>(a);
+                else k_layer_b<22><<<dim3(grid_b), dim3(512), lds_b, st>>>(a);
+                break;
             case WD_TYPE_Q8_0: k_layer_b<8><<<dim3(grid_b), dim3(512), lds_b, st>>>(a); break;
             case WD_TYPE_IQ4_NL: k_layer_b<20><<<dim3(grid_b), dim3(256), lds_b, st>>>(a); break;
             default: return fail(WD_ERR_UNSUPPORTED, "fused layer: unsupported gate/up type %d", L->gate_type);
@@ -555,22 +577,22 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
     const bool q8 = L->down_type == WD_TYPE_Q8_0;
     if (coal && two) {
         if (waves_c > 9) return fail(WD_ERR_ARG, "fused layer: %d waves in the paired down dispatch (at most 9)", waves_c);
-        if (F == 512 && q8) k_layer_c<0, true, 16, true><<<grid, block, lds_c, st>>>(a);
-        else if (F == 512) k_layer_c<1, true, 16, true><<<grid, block, lds_c, st>>>(a);
-        else if (q8) k_layer_c<0, true, 20, true><<<grid, block, lds_c, st>>>(a);
-        else k_layer_c<1, true, 20, true><<<grid, block, lds_c, st>>>(a);
+        if (F == 512 && q8) launch_layer_c<0, true, 16, true>(grid, block, lds_c, st, a);
+        else if (F == 512) launch_layer_c<1, true, 16, true>(grid, block, lds_c, st, a);
+        else if (q8) launch_layer_c<0, true, 20, true>(grid, block, lds_c, st, a);
+        else launch_layer_c<1, true, 20, true>(grid, block, lds_c, st, a);
     } else if (coal && F == 512 && q8)
-        k_layer_c<0, true><<<grid, block, lds_c, st>>>(a);
+        launch_layer_c<0, true, 16, false>(grid, block, lds_c, st, a);
     else if (coal && F == 512)
-        k_layer_c<1, true, 16><<<grid, block, lds_c, st>>>(a);
+        launch_layer_c<1, true, 16, false>(grid, block, lds_c, st, a);
     else if (coal && q8)
-        k_layer_c<0, true, 20><<<grid, block, lds_c, st>>>(a);
+        launch_layer_c<0, true, 20, false>(grid, block, lds_c, st, a);
     else if (coal)
-        k_layer_c<1, true, 20><<<grid, block, lds_c, st>>>(a);
+        launch_layer_c<1, true, 20, false>(grid, block, lds_c, st, a);
     else if (q8)
-        k_layer_c<0, false><<<grid, block, lds_c, st>>>(a);
+        launch_layer_c<0, false, 16, false>(grid, block, lds_c, st, a);
     else
-        k_layer_c<1, false><<<grid, block, lds_c, st>>>(a);
+        launch_layer_c<1, false, 16, false>(grid, block, lds_c, st, a);
     WD_LAUNCH_CHECK();
     return WD_OK;
 }
@@ -579,7 +601,8 @@ int layer_dispatch(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe
                    const int32_t *ids_override, float *residual, float residual_scale, hipStream_t st, int rec = 0,
                    const HcSpec *hc = nullptr) {
     const bool want_partials = s->gup != nullptr;
-    if ((flags & WD_MOE_STAGED) || want_partials)
+    const bool fused_exports = consumes_q8k(L->gate_type) && s->gup_type == L->gate_type && s->dp_type == L->down_type;
+    if ((flags & WD_MOE_STAGED) || (want_partials && !fused_exports))
         return layer_staged(L, d_x, d_out, s, flags, ids_override, residual, residual_scale, st, hc);
     return layer_fused(L, d_x, d_out, s, flags, ids_override, residual, residual_scale, st, rec, hc);
 }

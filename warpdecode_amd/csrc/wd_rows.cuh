@@ -327,9 +327,10 @@ WD_DEV void iq_rows8_coal_park(const IqRows8Raw<TYPE, NR> &raw, int lane, uint8_
     wave_lds_fence();
 }
 // The dot products of the NR rows parked in `stage`.
-template <int TYPE, int NR>
+// PART: the int32 chunk sums go out as well ([8 super-blocks][8 chunk lanes] per row, rows `pstride` ints apart).
+template <int TYPE, int NR, bool PART = false>
 WD_DEV void iq_rows8_coal_dots(const IqTables &t, const int8_t *act_qs, const float *act_d, int lane, float (&y)[NR],
-                               const uint8_t *stage) {
+                               const uint8_t *stage, int32_t *partials = nullptr, size_t pstride = 0) {
     constexpr int kBlk = IqRows8Raw<TYPE, NR>::kBlk;
     const int ib = lane >> 3, sb = lane & 7;
     const bool first = sb == 0;
@@ -343,7 +344,9 @@ WD_DEV void iq_rows8_coal_dots(const IqTables &t, const int8_t *act_qs, const fl
         int p[8];
         iq_chunks<TYPE>(f, ib, t, a, p);
         const float ds = h2f(f.d) * dx;
-        const float pf = static_cast<float>(reduce_scatter_ib(p, lane));  // lane (c = ib, sb): chunk c of super-block sb
+        const int P = reduce_scatter_ib(p, lane);  // lane (c = ib, sb): chunk c of super-block sb
+        if (PART) partials[i * pstride + sb * 8 + ib] = P;
+        const float pf = static_cast<float>(P);
         float v = __builtin_fmaf(ds, pf, 0.0f);
 #pragma unroll
         for (int s = 1; s < 8; ++s) {
@@ -355,17 +358,17 @@ WD_DEV void iq_rows8_coal_dots(const IqTables &t, const int8_t *act_qs, const fl
         y[i] = (TYPE == 22) ? 0.125f * r : r;
     }
 }
-template <int TYPE, int NR>
+template <int TYPE, int NR, bool PART = false>
 WD_DEV void iq_rows8_coal_finish(const IqRows8Raw<TYPE, NR> &raw, const IqTables &t, const int8_t *act_qs, const float *act_d,
-                                 int lane, float (&y)[NR], uint8_t *stage) {
+                                 int lane, float (&y)[NR], uint8_t *stage, int32_t *partials = nullptr, size_t pstride = 0) {
     iq_rows8_coal_park<TYPE, NR>(raw, lane, stage);
-    iq_rows8_coal_dots<TYPE, NR>(t, act_qs, act_d, lane, y, stage);
+    iq_rows8_coal_dots<TYPE, NR, PART>(t, act_qs, act_d, lane, y, stage, partials, pstride);
 }
-template <int TYPE, int NR>
+template <int TYPE, int NR, bool PART = false>
 WD_DEV void iq_rows8_coal(const uint8_t *const (&rows)[NR], const IqTables &t, const int8_t *act_qs, const float *act_d,
-                          int lane, float (&y)[NR], uint8_t *stage) {
+                          int lane, float (&y)[NR], uint8_t *stage, int32_t *partials = nullptr, size_t pstride = 0) {
     const IqRows8Raw<TYPE, NR> raw = iq_rows8_coal_request<TYPE, NR>(rows, lane);
-    iq_rows8_coal_finish<TYPE, NR>(raw, t, act_qs, act_d, lane, y, stage);
+    iq_rows8_coal_finish<TYPE, NR, PART>(raw, t, act_qs, act_d, lane, y, stage, partials, pstride);
 }
 
 constexpr int kIqStage10Bytes = 1120;  // per row of ten super-blocks: the 70 words that cover 12 + 1100 bytes
@@ -400,9 +403,9 @@ struct IqRowFetch {
 // first two lanes of every group of eight, the chain carried over as in iq_rows_q8k.
 // rows[i]: 4-byte aligned, inside a tensor whose end is 16-byte aligned.  stage: NR * kIqStage10Bytes bytes of LDS
 // owned by the wave, 16-byte aligned.
-template <int TYPE, int NR>
+template <int TYPE, int NR, bool PART = false>
 WD_DEV void iq_rows10_coal(const uint8_t *const (&rows)[NR], const IqTables &t, const int8_t *act_qs, const float *act_d,
-                           int lane, float (&y)[NR], uint8_t *stage) {
+                           int lane, float (&y)[NR], uint8_t *stage, int32_t *partials = nullptr, size_t pstride = 0) {
     constexpr int kBlk = (TYPE == 21) ? 110 : 82, kRow = 10 * kBlk;
     constexpr bool kTwoLoads = 12 + kRow > 1024;
     const int ib = lane >> 3, sbl = lane & 7;
@@ -443,6 +446,7 @@ WD_DEV void iq_rows10_coal(const uint8_t *const (&rows)[NR], const IqTables &t, 
             iq_chunks<TYPE>(f, ib, t, a, p);
             const float ds = on ? h2f(f.d) * dx : 0.0f;
             const int P = reduce_scatter_ib(p, lane);  // lane (c = ib, sb): chunk c of super-block sb
+            if (PART && on) partials[i * pstride + sb * 8 + ib] = P;
             const float pf = on ? static_cast<float>(P) : 0.0f;
             // carry of the first pass: last lane of the group -> first lane (lanes past the row's end pass the
             // accumulator through unchanged, fma(0, 0, acc) == acc)
@@ -846,8 +850,10 @@ WD_DEV void q8_rows4_coal_stage_any(const Q8CoalRaw<0, NB> &raw, uint8_t *stage,
 }
 // The dot products of the four staged rows; `stage` may be the tile itself (its chunk-sum area is overwritten only
 // after the staged bytes have been read).  y of row r4 valid in lane 16 r4.  The float order is that of q8_rows4_multi.
-template <int KIND, int NB>
-WD_DEV float q8_rows4_coal_dots(const uint8_t *stage, const int8_t *act_qs, const uint16_t *act_d, Q8TileNB<NB> &tile, int lane) {
+// partials (PART): int32 [4 rows][NB blocks][8 chunk lanes].
+template <int KIND, int NB, bool PART = false>
+WD_DEV float q8_rows4_coal_dots(const uint8_t *stage, const int8_t *act_qs, const uint16_t *act_d, Q8TileNB<NB> &tile, int lane,
+                                int32_t *partials = nullptr) {
     constexpr int kSecond = 4 * NB - 64, kRow = Q8TileNB<NB>::kRow;
     const int t1 = 64 + min(lane, max(kSecond, 1) - 1);
     const Q8Block w0 = q8_block_from_lds<KIND>(stage, lane);
@@ -861,6 +867,10 @@ WD_DEV float q8_rows4_coal_dots(const uint8_t *stage, const int8_t *act_qs, cons
         const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
         int p[8];
         q8_chunks<KIND>(w, a, p);
+        if (PART) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) partials[(row * NB + bi) * 8 + j] = p[j];
+        }
         float4 *dst = reinterpret_cast<float4 *>(&tile.pf[row * kRow + bi * 8]);
         dst[0] = make_float4(static_cast<float>(p[0]), static_cast<float>(p[1]), static_cast<float>(p[2]), static_cast<float>(p[3]));
         dst[1] = make_float4(static_cast<float>(p[4]), static_cast<float>(p[5]), static_cast<float>(p[6]), static_cast<float>(p[7]));
@@ -881,14 +891,14 @@ WD_DEV float q8_rows4_coal_dots(const uint8_t *stage, const int8_t *act_qs, cons
     }
     return close_lanes8(KIND == 1 ? acc + acc_odd : acc);
 }
-template <int KIND, int NB>
+template <int KIND, int NB, bool PART = false>
 WD_DEV float q8_rows4_coal_finish(const Q8CoalRaw<KIND, NB> &raw, const int8_t *act_qs, const uint16_t *act_d, Q8TileNB<NB> &tile,
-                                  int lane) {
+                                  int lane, int32_t *partials = nullptr) {
     uint8_t *stage = reinterpret_cast<uint8_t *>(&tile);  // chunk sums and scales together are large enough
     wave_lds_fence();  // earlier reads of the tile are done before it is overwritten
     q8_rows4_coal_stage<KIND, NB>(raw, stage, lane);
     wave_lds_fence();
-    return q8_rows4_coal_dots<KIND, NB>(stage, act_qs, act_d, tile, lane);
+    return q8_rows4_coal_dots<KIND, NB, PART>(stage, act_qs, act_d, tile, lane, partials);
 }
 // rows: first of the four rows.  `pre` runs between the request and the first read of the activation.
 template <int KIND, int NB, typename Pre = NoPre>
