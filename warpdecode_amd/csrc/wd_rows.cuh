@@ -328,12 +328,48 @@ WD_DEV void iq_rows8_coal_park(const IqRows8Raw<TYPE, NR> &raw, int lane, uint8_
 }
 // The dot products of the NR rows parked in `stage`.
 // PART: the int32 chunk sums go out as well ([8 super-blocks][8 chunk lanes] per row, rows `pstride` ints apart).
+//
+// Lane layout (differs from iq_rows_q8k): super-block sb = (lane >> 1) & 7, 32-value block ib = 2 (lane >> 4) + (lane & 1).
+// The integer fold over the eight ib-lanes is a half swap (ib bit 2), a row-pair swap (ib bit 1) and a swap of
+// neighbours (ib bit 0); it leaves chunk c of super-block sb in the lane that decoded (ib = c, sb).  The eight lanes of
+// one chain then sit two apart inside one row of 16 lanes, in super-block order, so a chain step is row_shr:2 in place:
+// the first lane of a chain has no source there and reads zero, which makes its fma the chain's first term again -
+// no lane has to be excluded from a step - and the finished chains sit in lanes 14, 15 of every row, where two swaps
+// and one shifted add form ggml's closing tree.
+WD_DEV int reduce_scatter_ib_pairs(const int (&p)[8], int lane) {
+    int q[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const wd_uint2v r = __builtin_amdgcn_permlane32_swap(static_cast<unsigned>(p[j]), static_cast<unsigned>(p[j + 4]),
+                                                            false, false);
+        q[j] = static_cast<int>(r.x + r.y);  // lanes < 32: chunk j, lanes >= 32: chunk j + 4
+    }
+    int s2[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const wd_uint2v r = __builtin_amdgcn_permlane16_swap(static_cast<unsigned>(q[j]), static_cast<unsigned>(q[j + 2]),
+                                                            false, false);
+        s2[j] = static_cast<int>(r.x + r.y);  // even rows: q[j] family, odd rows: q[j + 2] family
+    }
+    const bool odd = (lane & 1) != 0;
+    const int keep = odd ? s2[1] : s2[0];
+    const int send = odd ? s2[0] : s2[1];
+    return keep + dpp_i<kDppXor1>(0, send);
+}
+// ((l0 + l4) + (l2 + l6)) + ((l1 + l5) + (l3 + l7)) with chain c in lane 16 (c >> 1) + 14 + (c & 1); uniform result.
+WD_DEV float close_chains_pairs(float v) {
+    const wd_uint2v h = __builtin_amdgcn_permlane32_swap(f_bits(v), f_bits(v), false, false);
+    const float a = bits_f(h.x) + bits_f(h.y);  // lanes 14, 15, 30, 31: l0 + l4, l1 + l5, l2 + l6, l3 + l7
+    const wd_uint2v w = __builtin_amdgcn_permlane16_swap(f_bits(a), f_bits(a), false, false);
+    const float b = bits_f(w.x) + bits_f(w.y);  // lane 14: (l0 + l4) + (l2 + l6), lane 15: (l1 + l5) + (l3 + l7)
+    const float c = b + dpp_f<kDppShr1>(0.0f, b);
+    return readlane_f(c, 15);
+}
 template <int TYPE, int NR, bool PART = false>
 WD_DEV void iq_rows8_coal_dots(const IqTables &t, const int8_t *act_qs, const float *act_d, int lane, float (&y)[NR],
                                const uint8_t *stage, int32_t *partials = nullptr, size_t pstride = 0) {
     constexpr int kBlk = IqRows8Raw<TYPE, NR>::kBlk;
-    const int ib = lane >> 3, sb = lane & 7;
-    const bool first = sb == 0;
+    const int ib = ((lane >> 4) << 1) | (lane & 1), sb = (lane >> 1) & 7;
     const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32);
     const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32 + 16);
     const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
@@ -344,17 +380,13 @@ WD_DEV void iq_rows8_coal_dots(const IqTables &t, const int8_t *act_qs, const fl
         int p[8];
         iq_chunks<TYPE>(f, ib, t, a, p);
         const float ds = h2f(f.d) * dx;
-        const int P = reduce_scatter_ib(p, lane);  // lane (c = ib, sb): chunk c of super-block sb
+        const int P = reduce_scatter_ib_pairs(p, lane);  // lane (c = ib, sb): chunk c of super-block sb
         if (PART) partials[i * pstride + sb * 8 + ib] = P;
         const float pf = static_cast<float>(P);
         float v = __builtin_fmaf(ds, pf, 0.0f);
 #pragma unroll
-        for (int s = 1; s < 8; ++s) {
-            const float up = dpp_f<kDppShr1>(0.0f, v);
-            const float nxt = __builtin_fmaf(ds, pf, up);
-            v = first ? v : nxt;
-        }
-        const float r = close_lanes8_strided(v);
+        for (int s = 1; s < 8; ++s) v = __builtin_fmaf(ds, pf, dpp_f<kDppShr2, 0xf, 0xf, true>(0.0f, v));
+        const float r = close_chains_pairs(v);
         y[i] = (TYPE == 22) ? 0.125f * r : r;
     }
 }
