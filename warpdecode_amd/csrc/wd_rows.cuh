@@ -142,13 +142,19 @@ template <int TYPE>
 WD_DEV void iq_chunks(const IqFields &f, int ib, const IqTables &t, const uint32_t (&a)[8], int (&p)[8]) {
     if (TYPE == 21) {
         const int ls = 1 + 2 * static_cast<int>((f.sc >> (4 * (ib & 1))) & 15u);
+        // all sixteen lookups first, the arithmetic after: a lane's block then waits for the LDS once, not eight times
+        uint32_t g[8];
+        uint2 sm[8];
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
             const uint32_t q = ((c < 4 ? f.qs.x : f.qs.y) >> (8 * (c & 3))) & 0xffu;
             const uint32_t idx = q | ((f.qh << (8 - c)) & 0x100u);
             const uint32_t sbits = (f.sg >> (4 * c)) & 15u;  // sign byte c>>1, nibble c&1
-            p[c] = __mul24(ls, sdot4(apply_signs(t.grid3[idx], t.sign[sbits]), a[c], 0));
+            g[c] = t.grid3[idx];
+            sm[c] = t.sign[sbits];
         }
+#pragma unroll
+        for (int c = 0; c < 8; ++c) p[c] = __mul24(ls, sdot4(apply_signs(g[c], sm[c]), a[c], 0));
     } else {
         const int ls_lo = 1 + 2 * static_cast<int>(f.sc & 15u);
         const int ls_hi = 1 + 2 * static_cast<int>(f.sc >> 4);
