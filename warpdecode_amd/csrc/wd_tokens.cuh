@@ -232,7 +232,10 @@ __global__ __launch_bounds__(512, 4) void k_tokens_b(TokenArgs ta) {
     __syncthreads();
     mark(a, 1, 2);
     const int n_items = un.count * groups;
-    const int ib = lane >> 3, sbl = lane & 7;
+    // rows of eight super-blocks are one pass: the lane layout of iq_rows8_coal_dots then (a chain's lanes two apart inside
+    // a row, no carry between passes, no lane excluded from a chain step)
+    constexpr bool kPairs = NB == 8;
+    const int ib = kPairs ? ((lane >> 4) << 1) | (lane & 1) : lane >> 3, sbl = kPairs ? (lane >> 1) & 7 : lane & 7;
     const bool first = sbl == 0;
     constexpr int kStage = (NB == 10) ? kIqStage10Bytes : kIqStageBytes;
     uint8_t *stage = lds_tb + ((static_cast<size_t>(ta.T) * (a.H + sizeof(float) * nb) + 15) & ~static_cast<size_t>(15)) +
@@ -316,6 +319,14 @@ __global__ __launch_bounds__(512, 4) void k_tokens_b(TokenArgs ta) {
 #pragma unroll
                         for (int c = 0; c < 8; ++c) p[c] = 0;
                     }
+                    if (kPairs) {
+                        const float pf = static_cast<float>(reduce_scatter_ib_pairs(p, lane));
+                        float v = __builtin_fmaf(ds, pf, 0.0f);
+#pragma unroll
+                        for (int s = 1; s < 8; ++s) v = __builtin_fmaf(ds, pf, dpp_f<kDppShr2, 0xf, 0xf, true>(0.0f, v));
+                        acc[t][i] = v;
+                        continue;
+                    }
                     const float pf = static_cast<float>(reduce_scatter_ib(p, lane));
                     const float carry = dpp_f<kDppShl7>(0.0f, acc[t][i]);
                     float v = __builtin_fmaf(ds, pf, base == 0 ? 0.0f : carry);
@@ -332,7 +343,8 @@ __global__ __launch_bounds__(512, 4) void k_tokens_b(TokenArgs ta) {
 #pragma unroll
         for (int t = 0; t < MAXT; ++t) {
             if (rank[t] < 0) continue;
-            float g = close_lanes8_strided(acc[t][0]), up = close_lanes8_strided(acc[t][1]);
+            float g = kPairs ? close_chains_pairs(acc[t][0]) : close_lanes8_strided(acc[t][0]);
+            float up = kPairs ? close_chains_pairs(acc[t][1]) : close_lanes8_strided(acc[t][1]);
             if (TYPE == 22) {
                 g = 0.125f * g;
                 up = 0.125f * up;
