@@ -945,11 +945,16 @@ extern "C" int wd_moe_layer_tokens_pairs_f32(const wd_moe_layer *L, const uint8_
     Lt.n_experts = n_entries < Lt.top_k ? Lt.top_k : n_entries;
     wd_moe_scratch *s = scratch_per_token[0];
     hipStream_t st = as_stream(stream);
-    if (!s->pair_dev) {  // once per scratch
+    // the table goes up through a ring of pinned entries that this call may have to wait for: not something a graph
+    // can record
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    WD_HIP(hipStreamIsCapturing(st, &cap));
+    WD_REQUIRE(cap == hipStreamCaptureStatusNone, "multi-token pass on a pointer table: the stream is being captured (the table upload cannot be recorded)");
+    if (!s->pair_host)  // once per scratch
         WD_HIP(hipHostMalloc(reinterpret_cast<void **>(&s->pair_host), sizeof(void *) * 3 * kPairEntries * kPairRing, hipHostMallocDefault));
-        WD_HIP(hipMalloc(reinterpret_cast<void **>(&s->pair_dev), sizeof(void *) * 3 * kPairEntries * kPairRing));
-        for (hipEvent_t &ev : s->pair_done) WD_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
-    }
+    if (!s->pair_dev) WD_HIP(hipMalloc(reinterpret_cast<void **>(&s->pair_dev), sizeof(void *) * 3 * kPairEntries * kPairRing));
+    for (hipEvent_t &ev : s->pair_done)
+        if (!ev) WD_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
     const int slot = s->pair_next;
     s->pair_next = (slot + 1) % kPairRing;
     if (s->pair_used[slot]) WD_HIP(hipEventSynchronize(s->pair_done[slot]));  // the pass that read this entry of the ring has run
