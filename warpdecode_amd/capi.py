@@ -97,6 +97,7 @@ _SIGS = {
     "wd_moe_scratch_enable_partials": (i32, [vp, i32, i32]),
     "wd_moe_scratch_trace": (vp, [vp, i32]),
     "wd_moe_scratch_trace_resident": (vp, [vp, i32, i32]),
+    "wd_moe_scratch_omit_resident": (i32, [vp, i32]),
     "wd_moe_layer_f32": (i32, [C.POINTER(MoeLayer), vp, vp, vp, u32, vp]),
     "wd_moe_stack_cached_f32": (i32, [C.POINTER(MoeLayer), i32, vp, vp, vp, vp, vp, vp, f32, u32, vp]),
     "wd_moe_scratch_status": (i32, [vp]),

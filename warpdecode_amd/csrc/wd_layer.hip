@@ -47,6 +47,7 @@ struct wd_moe_scratch {
     std::vector<ResidentLayer> res_shadow;        // what res_layers holds
     int res_fits = -1;                            // -1 not asked yet; 1: the device holds the whole grid at once
     int trace_layer = 0;
+    int res_omit = 0;                             // measurement aid: parts of the resident launch left out (wd_moe_scratch_omit_resident)
     bool trace_all = false;                       // the trace buffer has the resident kernel's size
     // wd_moe_layer_tokens_pairs_f32: a ring of pointer tables (pinned staging + device copy), kPairRing x [kPairEntries][3]
     const uint8_t **pair_host = nullptr, **pair_dev = nullptr;
@@ -215,6 +216,14 @@ unsigned long long *wd_moe_scratch_trace_resident(wd_moe_scratch *s, int wg, int
     (void)hipMemset(s->trace, 0, bytes);
     s->trace_wg = wg, s->trace_layer = layer;
     return s->trace;
+}
+
+// Measurement aid: leaves parts of the resident launch out (results are then invalid), to time what remains.
+int wd_moe_scratch_omit_resident(wd_moe_scratch *s, int mask) {
+    WD_REQUIRE(s != nullptr, "omit parts of the resident launch: null scratch");
+    WD_REQUIRE(mask >= 0 && mask < 16, "omit parts of the resident launch: mask 0..15 (got %d)", mask);
+    s->res_omit = mask;
+    return WD_OK;
 }
 
 int wd_moe_scratch_enable_partials(wd_moe_scratch *s, int gate_type, int down_type) {
@@ -767,7 +776,7 @@ int stack_resident(const wd_moe_layer *layers, int n_layers, float *d_x, float *
     a.views = reinterpret_cast<const ResidentViews *>(s->res_layers + kResMaxLayers);
     a.hand = s->res_block, a.status = s->status, a.spin_limit = s->spin_limit;
     a.trace = s->trace, a.trace_wg = s->trace_wg, a.trace_layer = s->trace_layer;
-    if (const char *dbg = getenv("WD_RES_DEBUG")) a.debug = atoi(dbg);
+    a.debug = s->res_omit;
     return layers[0].gate_type == WD_TYPE_IQ3_S ? resident_launch<21>(a, s, st) : resident_launch<22>(a, s, st);
 }
 
