@@ -437,16 +437,21 @@ struct IqRowFetch {
 
 // iq_rows_q8k<TYPE, NR, false> for nb == 10 (hidden 2560) with the aligned fetch.  A row of ten super-blocks is 1100
 // or 820 bytes: 4-byte but not 16-byte aligned, so the wave fetches the 16-byte words that cover it (at most 70) and
-// the fields are picked behind the row's offset in its first word.  Two passes: super-blocks 0..7, then 8 and 9 in the
-// first two lanes of every group of eight, the chain carried over as in iq_rows_q8k.
+// the fields are picked behind the row's offset in its first word.
+// Lane layout as in iq_rows8_coal_dots (ib = 2 (lane >> 4) + (lane & 1), the other three lane bits a position 0..7
+// inside the chain): one pass per row over super-blocks 0..7, then ONE pass for super-blocks 8 and 9 of all NR rows
+// together - position 2 i takes super-block 8 of row i, position 2 i + 1 super-block 9 - instead of a mostly idle
+// second pass per row.  The chain of row i continues there: its value moves from the main pass's last position to
+// position 2 i (a row shift), two more steps follow, and the result moves back to the last position for the closing tree.
 // rows[i]: 4-byte aligned, inside a tensor whose end is 16-byte aligned.  stage: NR * kIqStage10Bytes bytes of LDS
-// owned by the wave, 16-byte aligned.
+// owned by the wave, 16-byte aligned.  NR <= 4.
 template <int TYPE, int NR, bool PART = false>
 WD_DEV void iq_rows10_coal(const uint8_t *const (&rows)[NR], const IqTables &t, const int8_t *act_qs, const float *act_d,
                            int lane, float (&y)[NR], uint8_t *stage, int32_t *partials = nullptr, size_t pstride = 0) {
+    static_assert(NR >= 1 && NR <= 4, "the tails of the rows share one pass of eight positions");
     constexpr int kBlk = (TYPE == 21) ? 110 : 82, kRow = 10 * kBlk;
     constexpr bool kTwoLoads = 12 + kRow > 1024;
-    const int ib = lane >> 3, sbl = lane & 7;
+    const int ib = ((lane >> 4) << 1) | (lane & 1), pos = (lane >> 1) & 7;
     uint32_t lead[NR];
     {
         uint4 raw0[NR], raw1[NR];
@@ -468,39 +473,63 @@ WD_DEV void iq_rows10_coal(const uint8_t *const (&rows)[NR], const IqTables &t, 
     }
     wave_lds_fence();
     float acc[NR];
-#pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
-        const int sb = 8 * pass + sbl;
-        const bool on = sb < 10;
-        const int sbc = min(sb, 9);  // lanes without a super-block read the last one and contribute zero
-        const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + sbc * 256 + ib * 32);
-        const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + sbc * 256 + ib * 32 + 16);
+    {   // super-blocks 0..7 of every row
+        const int sb = pos;
+        const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32);
+        const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32 + 16);
         const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
-        const float dx = act_d[sbc];
+        const float dx = act_d[sb];
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
-            const IqFields f = iq_fields_lds<TYPE>(stage + i * kIqStage10Bytes + lead[i] + sbc * kBlk, ib, sbc);
+            const IqFields f = iq_fields_lds<TYPE>(stage + i * kIqStage10Bytes + lead[i] + sb * kBlk, ib, sb);
             int p[8];
             iq_chunks<TYPE>(f, ib, t, a, p);
-            const float ds = on ? h2f(f.d) * dx : 0.0f;
-            const int P = reduce_scatter_ib(p, lane);  // lane (c = ib, sb): chunk c of super-block sb
-            if (PART && on) partials[i * pstride + sb * 8 + ib] = P;
-            const float pf = on ? static_cast<float>(P) : 0.0f;
-            // carry of the first pass: last lane of the group -> first lane (lanes past the row's end pass the
-            // accumulator through unchanged, fma(0, 0, acc) == acc)
-            float v = __builtin_fmaf(ds, pf, pass == 0 ? 0.0f : dpp_f<kDppShl7>(0.0f, acc[i]));
+            const float ds = h2f(f.d) * dx;
+            const int P = reduce_scatter_ib_pairs(p, lane);  // lane (c = ib, sb): chunk c of super-block sb
+            if (PART) partials[i * pstride + sb * 8 + ib] = P;
+            const float pf = static_cast<float>(P);
+            float v = __builtin_fmaf(ds, pf, 0.0f);
 #pragma unroll
-            for (int s = 1; s < 8; ++s) {
-                const float up = dpp_f<kDppShr1>(0.0f, v);
-                const float nxt = __builtin_fmaf(ds, pf, up);
-                v = (sbl == 0) ? v : nxt;
-            }
-            acc[i] = v;
+            for (int s = 1; s < 8; ++s) v = __builtin_fmaf(ds, pf, dpp_f<kDppShr2, 0xf, 0xf, true>(0.0f, v));
+            acc[i] = v;  // the chain over super-blocks 0..7: valid at position 7
         }
+    }
+    {   // super-blocks 8 and 9 of all rows in one pass
+        const int ri = min(pos >> 1, NR - 1), sb = 8 + (pos & 1);
+        const bool on = pos < 2 * NR;
+        const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32);
+        const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32 + 16);
+        const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        const float dx = act_d[sb];
+        uint32_t my_lead = lead[0];
+#pragma unroll
+        for (int i = 1; i < NR; ++i) my_lead = (ri == i) ? lead[i] : my_lead;
+        const IqFields f = iq_fields_lds<TYPE>(stage + ri * kIqStage10Bytes + my_lead + sb * kBlk, ib, sb);
+        int p[8];
+        iq_chunks<TYPE>(f, ib, t, a, p);
+        const float ds = on ? h2f(f.d) * dx : 0.0f;
+        const int P = reduce_scatter_ib_pairs(p, lane);
+        if (PART && on) partials[ri * pstride + sb * 8 + ib] = P;
+        const float pf = on ? static_cast<float>(P) : 0.0f;
+        // the chain value of row i, from position 7 of its own pass to position 2 i of this one (row_shl by 14 - 4 i lanes;
+        // only the four lanes of positions 2 i and 2 i + 1 are written, and of these only position 2 i has a source)
+        float carry = 0.0f;
+        if (NR > 0) carry = dpp_f<0x10E, 0xf, 0x1>(carry, acc[0]);
+        if (NR > 1) carry = dpp_f<0x10A, 0xf, 0x2>(carry, acc[NR > 1 ? 1 : 0]);
+        if (NR > 2) carry = dpp_f<0x106, 0xf, 0x4>(carry, acc[NR > 2 ? 2 : 0]);
+        if (NR > 3) carry = dpp_f<0x102, 0xf, 0x8>(carry, acc[NR > 3 ? 3 : 0]);
+        const float v8 = __builtin_fmaf(ds, pf, carry);                       // valid at the even positions
+        const float v9 = __builtin_fmaf(ds, pf, dpp_f<kDppShr2, 0xf, 0xf, true>(0.0f, v8));  // valid at the odd ones
+        // back to position 7 for the closing tree: row_shr by 12 - 4 i lanes
+        if (NR > 0) acc[0] = dpp_f<0x11C>(0.0f, v9);
+        if (NR > 1) acc[NR > 1 ? 1 : 0] = dpp_f<0x118>(0.0f, v9);
+        if (NR > 2) acc[NR > 2 ? 2 : 0] = dpp_f<0x114>(0.0f, v9);
+        // (NR == 4: row 3's result is already at position 7)
+        if (NR > 3) acc[NR > 3 ? 3 : 0] = v9;
     }
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
-        const float r = close_lanes8_strided(acc[i]);
+        const float r = close_chains_pairs(acc[i]);
         y[i] = (TYPE == 22) ? 0.125f * r : r;
     }
 }
