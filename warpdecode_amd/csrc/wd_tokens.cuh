@@ -234,7 +234,9 @@ __global__ __launch_bounds__(512, 4) void k_tokens_b(TokenArgs ta) {
     const int n_items = un.count * groups;
     // rows of eight super-blocks are one pass: the lane layout of iq_rows8_coal_dots then (a chain's lanes two apart inside
     // a row, no carry between passes, no lane excluded from a chain step)
-    constexpr bool kPairs = NB == 8;
+    // (NB == 10: the same layout for super-blocks 0..7, and super-blocks 8 and 9 of both rows in one shared pass, as in
+    // iq_rows10_coal)
+    constexpr bool kPairs = NB == 8 || NB == 10;
     const int ib = kPairs ? ((lane >> 4) << 1) | (lane & 1) : lane >> 3, sbl = kPairs ? (lane >> 1) & 7 : lane & 7;
     const bool first = sbl == 0;
     constexpr int kStage = (NB == 10) ? kIqStage10Bytes : kIqStageBytes;
@@ -275,7 +277,7 @@ __global__ __launch_bounds__(512, 4) void k_tokens_b(TokenArgs ta) {
         float acc[MAXT][2];
 #pragma unroll
         for (int t = 0; t < MAXT; ++t) acc[t][0] = acc[t][1] = 0.0f;
-        for (int base = 0; base < nb; base += 8) {
+        for (int base = 0; base < (NB == 10 ? 8 : nb); base += 8) {
             const int sb = base + sbl;
             const bool on = sb < nb;
             uint32_t w[2][8];
@@ -338,6 +340,35 @@ __global__ __launch_bounds__(512, 4) void k_tokens_b(TokenArgs ta) {
                     }
                     acc[t][i] = v;
                 }
+            }
+        }
+        if (NB == 10) {
+            // super-blocks 8 and 9: position 0/1 of the pass = row 0, position 2/3 = row 1 (positions 4..7 idle)
+            const int ri = min(sbl >> 1, 1), sb = 8 + (sbl & 1);
+            const bool on = sbl < 4;
+            const IqFields f = iq_fields_lds<TYPE>(stage + ri * kStage + (ri ? lead[1] : lead[0]) + sb * kBlk, ib, sb);
+            uint32_t w[8];
+            int ls[2];
+            iq_decode<TYPE>(f, ib, tables, w, ls);
+            const float dw = h2f(f.d);
+#pragma unroll
+            for (int t = 0; t < MAXT; ++t) {
+                if (rank[t] < 0) continue;  // uniform
+                const int8_t *aq = xq + static_cast<size_t>(t) * a.H + sb * 256 + ib * 32;
+                const uint4 a0 = *reinterpret_cast<const uint4 *>(aq);
+                const uint4 a1 = *reinterpret_cast<const uint4 *>(aq + 16);
+                const uint32_t av[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+                int p[8];
+                iq_dot_decoded(w, ls, av, p);
+                const float ds = on ? dw * xd[t * nb + sb] : 0.0f;
+                const int P = reduce_scatter_ib_pairs(p, lane);
+                const float pf = on ? static_cast<float>(P) : 0.0f;
+                float carry = dpp_f<0x10E, 0xf, 0x1>(0.0f, acc[t][0]);  // row 0's chain: position 7 -> position 0
+                carry = dpp_f<0x10A, 0xf, 0x2>(carry, acc[t][1]);       // row 1's chain: position 7 -> position 2
+                const float v8 = __builtin_fmaf(ds, pf, carry);
+                const float v9 = __builtin_fmaf(ds, pf, dpp_f<kDppShr2, 0xf, 0xf, true>(0.0f, v8));
+                acc[t][0] = dpp_f<0x11C>(0.0f, v9);  // back to position 7 for the closing tree
+                acc[t][1] = dpp_f<0x118>(0.0f, v9);
             }
         }
 #pragma unroll
