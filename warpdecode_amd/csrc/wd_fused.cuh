@@ -688,6 +688,90 @@ WD_DEV void router_rows_wave(const float *__restrict__ w, const float *__restric
     }
 }
 
+// The same for rows of 2049..4096 columns, two waves per row: wave 2 w takes the first 2048 columns of row (4 wg + w),
+// wave 2 w + 1 the rest, both with every load of theirs in flight from the start - one trip to memory instead of one per
+// span.  The chains still see their columns in ascending order: the second wave starts from the 32 accumulators the
+// first one leaves in LDS (`hand`: 4 x 32 floats).  Every thread of the (512-thread) workgroup must call it.
+WD_DEV void router_rows_wave_pair(const float *__restrict__ w, const float *__restrict__ x, float *xs, float *hand, float *logits,
+                                  int rows, int cols, const float *__restrict__ extra_w, float *extra_out, int wg) {
+    const int lane = threadIdx.x & 63, t = lane & 31, wave = static_cast<int>(threadIdx.x >> 6);
+    const bool upper = lane >= 32, second = (wave & 1) != 0;
+    const int row = wg * 4 + (wave >> 1);
+    const int total = rows + (extra_w ? 1 : 0);
+    const bool on = row < total;
+    const float *wr = on ? (row < rows ? w + static_cast<size_t>(row) * cols : extra_w) : x;
+    const int np = cols & ~31;
+    const int c0 = (second ? 2048 : 0) + (upper ? 1024 : 0) + t;  // this lane's first column
+    float wv[32];
+    if (on) {
+#pragma unroll
+        for (int u = 0; u < 32; ++u) {
+            const int c = c0 + 32 * u;
+            wv[u] = (c < np) ? wr[c] : 0.0f;
+        }
+    }
+    for (int i = static_cast<int>(threadIdx.x) * 4; i < cols; i += static_cast<int>(blockDim.x) * 4) {
+        if (i + 4 <= cols) {
+            *reinterpret_cast<float4 *>(xs + i) = *reinterpret_cast<const float4 *>(x + i);
+        } else {
+            for (int c = i; c < cols; ++c) xs[c] = x[c];
+        }
+    }
+    __syncthreads();
+    auto run_half = [&](float start) {
+        float v = start;
+#pragma unroll
+        for (int ub = 0; ub < 32; ub += 8) {
+            float xv[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int c = c0 + 32 * (ub + q);
+                xv[q] = xs[c < np ? c : 0];
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int c = c0 + 32 * (ub + q);
+                const float nv = __builtin_fmaf(wv[ub + q], xv[q], v);
+                v = (c < np) ? nv : v;
+            }
+        }
+        return v;
+    };
+    // one copy of the chain code for both waves of a pair: round 0 is run by the first wave, round 1 by the second
+    float s = 0.0f;
+#pragma unroll 1
+    for (int round = 0; round < 2; ++round) {
+        if (second == (round == 1)) {
+            const float start = s;
+            if (on && !upper) s = run_half(start);
+            const wd_uint2v fwd = __builtin_amdgcn_permlane32_swap(f_bits(s), f_bits(s), false, false);
+            if (upper) s = on ? run_half(bits_f(fwd.x)) : bits_f(fwd.x);
+        }
+        if (round == 0) {
+            if (!second && upper) hand[(wave >> 1) * 32 + t] = s;
+            __syncthreads();
+            if (second) s = hand[(wave >> 1) * 32 + t];
+        }
+    }
+    if (!second) return;
+    // the 32 accumulators are final in the upper half (lanes 32..63): ggml's closing tree
+    float o = __shfl_down(s, 16, 32);
+    if (t < 16) s = s + o;
+    o = __shfl_down(s, 8, 32);
+    if (t < 8) s = s + o;
+    o = __shfl_down(s, 4, 32);
+    if (t < 4) s = s + o;
+    o = __shfl_down(s, 1, 32);
+    if (t == 0 || t == 2) s = s + o;
+    o = __shfl_down(s, 2, 32);
+    float acc = s + o;
+    if (on && lane == 32) {
+        for (int c = np; c < cols; ++c) acc = acc + wr[c] * xs[c];
+        float *dst = (row < rows) ? logits + row : extra_out;
+        __hip_atomic_store(dst, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 // ---- dispatch A -----------------------------------------------------------------------------------------
 // grid = n_router_wgs + ceil(F / 8) (the second part only with a shared expert); 512 threads.
 // Router workgroups: 16 rows each.  Shared-expert workgroups: 8 (gate, up) row pairs, one per wave.
@@ -779,8 +863,12 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
 
     mark(a, wg < a.n_router_wgs + n_shared_wgs ? 0 : 1, 0);
     if (wg < a.n_router_wgs) {
-        router_rows_wave<true>(a.router, a.x, reinterpret_cast<float *>(lds_ab), a.logits, a.E, a.H, a.sh_inp,
-                               a.shared_gate, wg);
+        if (COAL && NB == 10)  // rows of 2560 columns: two waves per row, four rows per workgroup (the host sizes the grid for it)
+            router_rows_wave_pair(a.router, a.x, reinterpret_cast<float *>(lds_ab), reinterpret_cast<float *>(s_union), a.logits, a.E,
+                                  a.H, a.sh_inp, a.shared_gate, wg);
+        else
+            router_rows_wave<true>(a.router, a.x, reinterpret_cast<float *>(lds_ab), a.logits, a.E, a.H, a.sh_inp,
+                                   a.shared_gate, wg);
         mark(a, 0, 1);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_waitcnt(0);  // this wave's stores have been acknowledged

@@ -518,14 +518,19 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
         const int capacity = 3 * s->compute_units;
         const int routed_wgs = m.n_routed_items <= capacity - 8 ? m.n_routed_items
                                                                 : std::min(m.n_routed_items, std::max(capacity - fixed_wgs, (F + 7) / 8));
-        const int grid_ab = fixed_wgs + routed_wgs;
-        const size_t lds_ab = sizeof(float) * static_cast<size_t>(H) + 16;  // f32 x of the router rows; the quantised x of the others fits inside
         // rows of eight super-blocks on 16-byte boundaries: coalesced fetch with a per-wave staging area behind lds_ab
         auto al16_ = [](const void *p_, size_t v) { return reinterpret_cast<uintptr_t>(p_) % 16 == 0 && v % 16 == 0; };
         // (rows of ten super-blocks are 4-byte aligned then, and F rows end on a 16-byte boundary)
         const bool coal_ab = iq && (H == 2048 || H == 2560) &&
                              (L->slot_of_expert ? al16_(L->slot_pool, L->slot_bytes) && L->slot_gate_bytes % 16 == 0
                                                 : al16_(L->gate, L->gate_stride) && al16_(L->up, L->up_stride));
+        if (coal_ab && H == 2560) {
+            // these variants give a router row two waves, every weight of the row requested at once: twice the router
+            // workgroups (they leave long before the routed ones stop waiting, so the routed workgroups keep their number)
+            m.n_router_wgs = (a.E + (shared ? 1 : 0) + 3) / 4;
+        }
+        const int grid_ab = m.n_router_wgs + (shared ? (F + 7) / 8 : 0) + routed_wgs;
+        const size_t lds_ab = sizeof(float) * static_cast<size_t>(H) + 16;  // f32 x of the router rows; the quantised x of the others fits inside
         const size_t lds_stage = 16 + 8 * 2 * static_cast<size_t>(H == 2048 ? kIqStageBytes : kIqStage10Bytes);
         const dim3 grid(grid_ab), block(512);
         const bool loop = routed_wgs < m.n_routed_items;
