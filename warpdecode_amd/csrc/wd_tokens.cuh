@@ -49,7 +49,7 @@ struct TokenArgs {
 // one-token merged dispatch: router rows one per wave, the last router workgroup of the token selects its experts
 // with the whole workgroup, the other workgroups run the shared expert's gate/up.
 // dynamic LDS: 4 * H bytes (x as f32 for the router rows; the shared workgroups use H + H/16 of it).
-__global__ __launch_bounds__(512, 6) void k_tokens_a(TokenArgs ta) {
+__global__ __launch_bounds__(512, 4) void k_tokens_a(TokenArgs ta) {
     extern __shared__ __align__(16) uint8_t lds_ta[];
     __shared__ __align__(16) uint8_t s_work[sizeof(Q8RowTile) * 8];
     __shared__ int s_last;
