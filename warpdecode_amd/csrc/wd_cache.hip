@@ -73,7 +73,11 @@ struct FillSegments {
 // that each wait on the link for most of a millisecond: the layer kernels could not place theirs); 8 x 256 threads for
 // the whole launch 570 (k_layer_ab 22.6 instead of 16 us: the compute units that host a fill workgroup serve their
 // layer workgroups late, and the grid waits for those); 32 x 64 threads 589, 24 x 64 642, 20 x 64 670, 16 x 64 582
-// (the link is no longer kept busy).
+// (the link is no longer kept busy).  The loop below keeps a round's words in a private array that the compiler
+// places in scratch memory (the stores are conditional): the words go link -> registers -> scratch -> registers ->
+// slot, one store at a time.  Forms that keep them in registers (unconditional stores of a plain vector type; 20 x 64
+// x 8, 20 x 64 x 4, 40 x 64 x 4, 40 x 64 x 2, 64 x 64 x 2) all measured 530..590 against 669 on the same box: a copy
+// that runs through its stores faster takes more from the layer kernels than it gains on the link.
 #ifndef WD_FILL_THREADS
 #define WD_FILL_THREADS 64
 #endif
