@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the batch=1 MoE decode hot path on one MI355X.
 
-Workload (BASELINE.json configs[3], mode A): a stack of 48 MoE layers (hidden 2048, 512 experts,
+Workload (the 48-layer stack of the full-scale layer, mode A): a stack of 48 MoE layers (hidden 2048, 512 experts,
 top-10, ffn 512, IQ3_S gate/up, Q8_0 down, Q8_0 shared expert gated by sigmoid(w.x), f32 router),
 all 24,576 experts resident in HBM, one token per step.  Per layer the router runs and its weights
 are used; the expert ids are replayed from a seeded Zipf(1.1) trace, as the workload prescribes.
@@ -460,7 +460,7 @@ def graph_period_us(torch, launch, launches, reps):
 
 
 def bench_q4_sweep(args, torch, capi, synth):
-    """Dense Q4_0 x Q8_0 GEMV at batch=1 over the Llama-3.2-1B shapes (BASELINE.json configs[1]).  Every launch
+    """Dense Q4_0 x Q8_0 GEMV at batch=1 over the Llama-3.2-1B shapes (the dense sweep workload).  Every launch
     of a chain reads another copy of the matrix, with enough copies (>= 1.5 GB) that nothing is served from the
     256 MB last-level cache; the period is taken over a captured chain, so it includes the launch gap."""
     shapes = [(2048, 2048), (8192, 2048), (2048, 8192), (128256, 2048)]     # rows x cols of the weight
@@ -711,7 +711,7 @@ def bench_hc(args, torch, capi, synth):
 
 
 def bench_c0(args, torch, capi, synth):
-    """BASELINE.json configs[0] at stack depth: the 64-expert top-8 layer with Q8_0 gate/up/down and no shared expert
+    """The single-layer parity workload at stack depth: the 64-expert top-8 layer with Q8_0 gate/up/down and no shared expert
     (hidden 2048, ffn 512), `--layers` independent layers chained as in the headline workload, router-selected."""
     H, F, k, E, NL = 2048, 512, 8, 64, args.layers
     g = torch.Generator(device="cuda")
@@ -766,7 +766,7 @@ def bench_c0(args, torch, capi, synth):
 
 
 def bench_tokens(args, torch, capi, synth):
-    """Speculative-verify batch (BASELINE.json configs[4]): T correlated tokens through each of the C2 layers in one
+    """Speculative-verify batch: T correlated tokens through each of the C2 layers in one
     pass that reads every selected expert once, against T one-token passes over the same layers.  The router picks
     the experts; the tokens are mixed from a common direction so that their top-10 sets overlap by about half."""
     H, F, k, E, NL, T = 2048, 512, 10, args.experts, args.layers, args.tokens

@@ -737,17 +737,17 @@ WD_DEV void router_rows_wave_pair(const float *__restrict__ w, const float *__re
         }
         return v;
     };
-    // one copy of the chain code for both waves of a pair: round 0 is run by the first wave, round 1 by the second
+    // one copy of the chain code for both waves of a pair: turn 0 is the first wave's, turn 1 the second's
     float s = 0.0f;
 #pragma unroll 1
-    for (int round = 0; round < 2; ++round) {
-        if (second == (round == 1)) {
+    for (int turn = 0; turn < 2; ++turn) {
+        if (second == (turn == 1)) {
             const float start = s;
             if (on && !upper) s = run_half(start);
             const wd_uint2v fwd = __builtin_amdgcn_permlane32_swap(f_bits(s), f_bits(s), false, false);
             if (upper) s = on ? run_half(bits_f(fwd.x)) : bits_f(fwd.x);
         }
-        if (round == 0) {
+        if (turn == 0) {
             if (!second && upper) hand[(wave >> 1) * 32 + t] = s;
             __syncthreads();
             if (second) s = hand[(wave >> 1) * 32 + t];
