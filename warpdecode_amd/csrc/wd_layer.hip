@@ -738,11 +738,14 @@ template <int TYPE>
 int resident_launch(const ResidentArgs &a, wd_moe_scratch *s, hipStream_t st) {
     if (s->res_fits < 0) {
         int per_cu = 0;
-        const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_stack_resident<TYPE>, kResThreads, kResLdsBytes);
+        const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_stack_resident<TYPE, true>, kResThreads, kResLdsBytes);
         s->res_fits = (e == hipSuccess && per_cu * s->compute_units >= kResWgs) ? 1 : 0;
     }
     if (!s->res_fits) return -1;  // the workgroups would wait for each other without all being on the device
-    k_stack_resident<TYPE><<<dim3(kResWgs), dim3(kResThreads), kResLdsBytes, st>>>(a);
+    if (a.trace)  // (the variant with the time stamps only when they are asked for)
+        k_stack_resident<TYPE, true><<<dim3(kResWgs), dim3(kResThreads), kResLdsBytes, st>>>(a);
+    else
+        k_stack_resident<TYPE, false><<<dim3(kResWgs), dim3(kResThreads), kResLdsBytes, st>>>(a);
     WD_LAUNCH_CHECK();
     return WD_OK;
 }

@@ -110,7 +110,10 @@ struct ResidentArgs {
     unsigned spin_limit;
     unsigned long long *trace;  // null, or [12][16] time stamps (100 MHz) of workgroup trace_wg in layer trace_layer
     int trace_wg, trace_layer;
-    int debug;  // experiments: 1 no gate/up decode, 2 no weight loads, 4 no wait for the activations, 8 no down dots
+    int debug;  // experiments: 1 no gate/up decode, 2 no weight loads, 4 no wait for the activations, 8 no down dots.
+                // (The tests of these bits stay in the kernel on purpose: as branches around the weight requests and the
+                // dot products they keep the compiler from moving these against each other - the down rows' request in
+                // particular must follow the gate/up rows' arrival -, and the kernel measured 5 % slower without them.)
 };
 
 // ---- device-scope access to the hand-off buffers ------------------------------------------------------------
@@ -396,7 +399,10 @@ WD_DEV ResCtx res_ctx(uint8_t *base, int r, int lane, int wave, int slot, __amdg
 }
 // Time stamp i of this wave in layer l.  trace_wg >= 0: every wave of that workgroup ([12][16] stamps);
 // trace_wg == -1: waves 0, 9, 10 and 11 of every workgroup ([wg][4][16] stamps).
+// (STAMPS: the time stamps are compiled in; the variant without them keeps their pointers and tests out of the layer loop)
+template <bool STAMPS>
 WD_DEV void res_mark(const ResidentArgs &a, const ResCtx &c, int l, int i) {
+    if (!STAMPS) return;
     if (!a.trace || l != a.trace_layer || c.lane != 0) return;
     if (a.trace_wg >= 0) {
         if (c.r == a.trace_wg) a.trace[c.wave * 16 + i] = wall_clock64();
@@ -414,6 +420,7 @@ WD_DEV T *res_field(T *const *field) {
 // activation, for routed rungs in use and the shared expert).  The workgroup's eleven activations go out as one store
 // of its record; waves 0..7 then wait for the records of all 512 workgroups and lay the values out in LDS by slot;
 // v0, v1 receive values 8 lane .. 8 lane + 7 of this wave's slot.
+template <bool STAMPS>
 WD_DEV void res_exchange(const ResidentArgs &a, const ResCtx &c, int l, bool has, float mine, float4 &v0, float4 &v1, bool &dead) {
     const int lane = c.lane, wave = c.wave;
     if (has && lane == 0) c.actv()[c.slot] = mine;
@@ -438,7 +445,7 @@ WD_DEV void res_exchange(const ResidentArgs &a, const ResCtx &c, int l, bool has
         }
     }
     __syncthreads();  // B3: every activation of the layer is in LDS
-    res_mark(a, c, l, 6);
+    res_mark<STAMPS>(a, c, l, 6);
     if (has) {
         const float4 *row = reinterpret_cast<const float4 *>(c.land() + c.slot * 512 + 8 * lane);
         v0 = row[0], v1 = row[1];
@@ -448,6 +455,7 @@ WD_DEV void res_exchange(const ResidentArgs &a, const ResCtx &c, int l, bool has
 
 // The down rows 4r..4r+3 of one matrix against the activation values v0, v1 (8 lane .. 8 lane + 7) of slot `c.slot`:
 // quantises them to Q8_0 and runs the four row chains; the result of row 4r + i lands in ybuf[slot * 4 + i].
+template <bool STAMPS>
 WD_DEV void res_down(const ResidentArgs &a, const ResCtx &c, int l, const Q8CoalRaw<0, 16> &draw, const float4 &v0, const float4 &v1) {
     const int lane = c.lane;
     uint8_t *area = c.area();
@@ -457,12 +465,12 @@ WD_DEV void res_down(const ResidentArgs &a, const ResCtx &c, int l, const Q8Coal
     float y = 1.0f;
     if (!(a.debug & 8)) y = q8_rows4_coal_finish<0, 16>(draw, aq, ad, *reinterpret_cast<Q8TileNB<16> *>(area), lane);
     if ((lane & 15) == 0) c.ybuf()[c.slot * 4 + (lane >> 4)] = y;
-    res_mark(a, c, l, 7);
+    res_mark<STAMPS>(a, c, l, 7);
 }
 
 // ---- the ten routed waves -------------------------------------------------------------------------------------
 // Waves 0..7 (always rungs 0..7) also fetch and quantise the layer's input, and in workgroup 0 select the experts.
-template <int TYPE>
+template <int TYPE, bool STAMPS>
 WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, int lane0, int wave0, int slot0,
                             __amdgpu_buffer_rsrc_t hb, unsigned set_base, bool &dead) {
     constexpr int kRow = 8 * ((TYPE == 21) ? 110 : 82);
@@ -475,7 +483,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         const bool last = l == a.n_layers - 1;
         const bool gate_row = shared && r == 1 && rung == 9;  // the shared expert's gate logit: one more row of the router's kind
         // ---- the layer's input: 16 bytes per lane of waves 0..7, quantised from the registers they arrive in
-        res_mark(a, c, l, 0);
+        res_mark<STAMPS>(a, c, l, 0);
         if (wave < 8) {
             const int i = wave * 64 + lane;
             float4 xv;
@@ -490,7 +498,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                 hand_wait16<1>(a, c.hb, off, true, v, dead);
                 xv = make_float4(bits_f(v[0].x), bits_f(v[0].y), bits_f(v[0].z), bits_f(v[0].w));
             }
-            res_mark(a, c, l, 1);
+            res_mark<STAMPS>(a, c, l, 1);
             {   // values 4 i .. 4 i + 3 are accumulators 4 (i % 8) .. + 3 at step i / 8
                 float *dst = c.xt() + (4 * (i & 7)) * kResXtRow + (i >> 3);
                 dst[0] = xv.x, dst[kResXtRow] = xv.y, dst[2 * kResXtRow] = xv.z, dst[3 * kResXtRow] = xv.w;
@@ -506,7 +514,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             }
         }
         __syncthreads();  // B1: x and its quantised forms are in LDS
-        res_mark(a, c, l, 2);
+        res_mark<STAMPS>(a, c, l, 2);
         const float res_pre = c.x_at(4 * r + (lane & 3));  // (rung 0 adds the layer's output to these)
         // this layer's routed tensors (the wave has nothing else to do until the ids appear)
         const uint8_t *const gate_base = res_field(&L->gate), *const up_base = res_field(&L->up), *const down_base = res_field(&L->down);
@@ -533,23 +541,23 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             if (wave < 8) {
                 const uint32_t b = hand_wait4(a, c.hb, rec_off(l, id), id < a.E, dead);
                 if (id < a.E) lv[0] = bits_f(b);
-                res_mark(a, c, l, 3);
+                res_mark<STAMPS>(a, c, l, 3);
                 topk_block_step1<1>(lv, s, lane, wave);
             }
             __syncthreads();
-            res_mark(a, c, l, 12);
+            res_mark<STAMPS>(a, c, l, 12);
             if (wave < 8) topk_block_step2<1>(lv, a.E, a.k, s, lane, wave);
             __syncthreads();
-            res_mark(a, c, l, 13);
+            res_mark<STAMPS>(a, c, l, 13);
             if (wave == 0) {
 #ifdef WD_RES_SEL_STAMPS
-                unsigned long long *st3 = (a.trace && l == a.trace_layer && a.trace_wg == 0) ? a.trace + 11 * 16 + 5 : nullptr;
+                unsigned long long *st3 = (STAMPS && a.trace && l == a.trace_layer && a.trace_wg == 0) ? a.trace + 11 * 16 + 5 : nullptr;
 #else
                 unsigned long long *st3 = nullptr;
 #endif
                 topk_block_step3<1>(a.E, a.k, w_scale, lds_ids, lds_w, ids_given != nullptr, id_given, s, lane, st3,
                                     reinterpret_cast<uint32_t *>(a.hand + set_base + kHandIdh) + static_cast<size_t>(l) * kResIdCopies * 16, kResIdCopies);
-                res_mark(a, c, l, 14);
+                res_mark<STAMPS>(a, c, l, 14);
                 wave_lds_fence();
                 if (lane < a.k) {
                     hand_store4(c.hb, kHandWh + static_cast<unsigned>((l * 16 + lane) * 4), f_bits(lds_w[lane]));
@@ -574,7 +582,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             uint32_t e = hand_wait4(a, c.hb, kHandIdh + static_cast<unsigned>(((l * kResIdCopies + (r & (kResIdCopies - 1))) * 16 + rung) * 4), true, dead);
             e = __builtin_amdgcn_readfirstlane(e);
             if (e >= static_cast<uint32_t>(a.E)) e = 0;  // only after a wait that ran out (status is set)
-            res_mark(a, c, l, 4);
+            res_mark<STAMPS>(a, c, l, 4);
             const uint8_t *const rows[2] = {gate_base + e * a.gate_stride + static_cast<size_t>(r) * kRow,
                                             up_base + e * a.up_stride + static_cast<size_t>(r) * kRow};
             IqRows8Raw<TYPE, 2> raw;
@@ -589,10 +597,10 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
 #else
             e_keep = e;
 #endif
-            res_mark(a, c, l, 11);
+            res_mark<STAMPS>(a, c, l, 11);
             if (!(a.debug & 1)) iq_rows8_coal_dots<TYPE, 2>(tables, c.xq(), c.xd(), lane, gu, c.area());
             act = silu_ggml(gu[0]) * gu[1];
-            res_mark(a, c, l, 5);
+            res_mark<STAMPS>(a, c, l, 5);
 #if WD_RES_DOWN_AT == 1
             draw = q8_rows4_coal_request<0, 16>(down_base + e_keep * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
 #endif
@@ -605,11 +613,11 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         uint32_t wbits = kResEmpty;
         if (wlane && !dead) wbits = hand_load4(c.hb, woff);
         float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
-        res_exchange(a, c, l, on, act, v0, v1, dead);
+        res_exchange<STAMPS>(a, c, l, on, act, v0, v1, dead);
 #if WD_RES_DOWN_AT == 2
         if (on) draw = q8_rows4_coal_request<0, 16>(down_base + e_keep * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
 #endif
-        if (on) res_down(a, c, l, draw, v0, v1);
+        if (on) res_down<STAMPS>(a, c, l, draw, v0, v1);
         float wreg = 0.0f;
         if (rung == 0) {
             if (__builtin_amdgcn_ballot_w64(wlane && wbits == kResEmpty) != 0ull) wbits = hand_wait4(a, c.hb, woff, wlane, dead);
@@ -619,7 +627,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
 
         // ---- ordered weighted sum, shared branch, next input
         if (rung == 0) {
-            res_mark(a, c, l, 8);
+            res_mark<STAMPS>(a, c, l, 8);
             const float *ybuf = c.ybuf();
             float acc = 0.0f;
             for (int m = 0; m < a.k; ++m) {
@@ -650,12 +658,13 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                                                f_bits(readlane_f(xn, 3)));
                 if (lane < kResCopies) hand_store16(c.hb, xc_off(l + 1, lane) + kXcStride * r, piece);
             }
-            res_mark(a, c, l, 9);
+            res_mark<STAMPS>(a, c, l, 9);
         }
     }
 }
 
 // ---- the shared expert's wave ------------------------------------------------------------------------------------
+template <bool STAMPS>
 WD_DEV void res_shared_role(const ResidentArgs &a, uint8_t *lds_base, int r0, int lane0, int wave0,
                             __amdgpu_buffer_rsrc_t hb, bool &dead) {
     Q8Block gb[2];
@@ -676,17 +685,17 @@ WD_DEV void res_shared_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         }
         float act = 0.0f;
         if (a.shared) {
-            res_mark(a, c, l, 2);
+            res_mark<STAMPS>(a, c, l, 2);
             Q8RowTile &tile = *reinterpret_cast<Q8RowTile *>(c.area());
             float acc[2] = {0.0f, 0.0f};
             q8_row_wave_pass<2>(gb, true, lane, c.x0q(), c.x0d(), tile, lane, acc);
             const float g = close_lanes8(acc[0]), u = close_lanes8(acc[1]);
             act = silu_ggml(g) * u;
-            res_mark(a, c, l, 5);
+            res_mark<STAMPS>(a, c, l, 5);
         }
         float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
-        res_exchange(a, c, l, a.shared != 0, act, v0, v1, dead);
-        if (a.shared) res_down(a, c, l, draw, v0, v1);
+        res_exchange<STAMPS>(a, c, l, a.shared != 0, act, v0, v1, dead);
+        if (a.shared) res_down<STAMPS>(a, c, l, draw, v0, v1);
         __syncthreads();  // B5
         // the next layer's rows, asked for on this side of the barrier: the fold of this layer must not wait for a
         // wave that is busy issuing requests
@@ -697,6 +706,7 @@ WD_DEV void res_shared_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
 // ---- the router wave: row r --------------------------------------------------------------------------------------------
 // It also puts the other set of hand-off buffers (`ob`) back to "not yet written": in layer l this workgroup's share of
 // layers l, l + n, l + 2n, ... of that set (all kResMaxLayers layers, whatever the launch that wrote them used).
+template <bool STAMPS>
 WD_DEV void res_router_role(const ResidentArgs &a, uint8_t *lds_base, int r0, int lane0, int wave0,
                             __amdgpu_buffer_rsrc_t hb, __amdgpu_buffer_rsrc_t ob, bool &dead) {
     const bool on = r0 < a.E;
@@ -707,11 +717,11 @@ WD_DEV void res_router_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         const int r = c.r, lane = c.lane;
         const bool last = l == a.n_layers - 1;
         __syncthreads();  // B1
-        res_mark(a, c, l, 2);
+        res_mark<STAMPS>(a, c, l, 2);
         if (on) {
             const float s = res_router_dot(wv, c.xt(), lane);
             if (lane == 32) hand_store4(c.hb, rec_off(l, r), f_bits(s));
-            res_mark(a, c, l, 3);
+            res_mark<STAMPS>(a, c, l, 3);
             if (!last) res_router_fetch(res_field(&a.layers[l + 1].router) + static_cast<size_t>(r) * kResH, wv, lane);
         }
         for (int ll = l; ll < kResMaxLayers; ll += a.n_layers) {
@@ -738,12 +748,12 @@ WD_DEV void res_router_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             }
         }
         float4 v0, v1;
-        res_exchange(a, c, l, false, 0.0f, v0, v1, dead);
+        res_exchange<STAMPS>(a, c, l, false, 0.0f, v0, v1, dead);
         __syncthreads();  // B5
     }
 }
 
-template <int TYPE>
+template <int TYPE, bool STAMPS>
 __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 6))) void k_stack_resident(ResidentArgs a) {
     extern __shared__ __align__(16) uint8_t lds_res[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -793,11 +803,11 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 
 
     bool dead = false;
     if (slot < 0)
-        res_router_role(a, lds_res, r, lane, wave, hb, ob, dead);
+        res_router_role<STAMPS>(a, lds_res, r, lane, wave, hb, ob, dead);
     else if (slot == kResSharedSlot)
-        res_shared_role(a, lds_res, r, lane, wave, hb, dead);
+        res_shared_role<STAMPS>(a, lds_res, r, lane, wave, hb, dead);
     else
-        res_routed_role<TYPE>(a, lds_res, r, lane, wave, slot, hb, set_base, dead);
+        res_routed_role<TYPE, STAMPS>(a, lds_res, r, lane, wave, slot, hb, set_base, dead);
 
     // the next launch takes the other set (workgroup 0 can only get here after every workgroup has read the number)
     if (r == 0 && threadIdx.x == 0 && !dead)
