@@ -57,7 +57,10 @@ constexpr uint32_t kTagInvalid = 0xffffffffu;
 constexpr unsigned kSpinLimit = 1u << 21;  // default number of polls before a wait gives up (seconds)
 
 // Time stamp `i` of dispatch `d` (0 = A, 1 = B, 2 = C) for the traced workgroup; lane 0 of every wave.
+// TRACE false: compiled out (the kernels that take the stamps as a template parameter run without their tests then).
+template <bool TRACE = true>
 WD_DEV void mark(const LayerArgs &a, int d, int i) {
+    if (!TRACE) return;
     if (a.trace && static_cast<int>(blockIdx.x) == a.trace_wg && (threadIdx.x & 63) == 0 && (threadIdx.x >> 6) < 15)
         a.trace[(d * 16 + (threadIdx.x >> 6)) * 8 + i] = wall_clock64();
 }
@@ -849,7 +852,7 @@ __global__ __launch_bounds__(512) void k_layer_a(LayerArgs a) {
 // NB (COAL only): super-blocks per row, 8 (hidden 2048) or 10 (hidden 2560).
 // LOOP: the grid has fewer routed workgroups than there are (expert rung, group of eight rows) items; they walk them
 // with the stride of their number.
-template <int TYPE, bool COAL, int NB = 8, bool LOOP = false, bool PART = false>
+template <int TYPE, bool COAL, int NB = 8, bool LOOP = false, bool PART = false, bool TRACE = false>
 __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
     constexpr bool kIq = (TYPE == 21 || TYPE == 22);
     extern __shared__ __align__(16) uint8_t lds_ab[];
@@ -861,7 +864,7 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
     const int groups = (a.F + 7) / 8;
     const int n_shared_wgs = a.sh_inp ? groups : 0;
 
-    mark(a, wg < a.n_router_wgs + n_shared_wgs ? 0 : 1, 0);
+    mark<TRACE>(a, wg < a.n_router_wgs + n_shared_wgs ? 0 : 1, 0);
     if (wg < a.n_router_wgs) {
         if (COAL && NB == 10)  // rows of 2560 columns: two waves per row, four rows per workgroup (the host sizes the grid for it)
             router_rows_wave_pair(a.router, a.x, reinterpret_cast<float *>(lds_ab), reinterpret_cast<float *>(s_union), a.logits, a.E,
@@ -869,7 +872,7 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
         else
             router_rows_wave<true>(a.router, a.x, reinterpret_cast<float *>(lds_ab), a.logits, a.E, a.H, a.sh_inp,
                                    a.shared_gate, wg);
-        mark(a, 0, 1);
+        mark<TRACE>(a, 0, 1);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_waitcnt(0);  // this wave's stores have been acknowledged
         __syncthreads();
@@ -879,14 +882,14 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
         __syncthreads();
         if (s_last) {
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-            if (a.trace && threadIdx.x == 0) a.trace[(0 * 16 + 8) * 8 + 0] = wall_clock64();
+            if (TRACE && a.trace && threadIdx.x == 0) a.trace[(0 * 16 + 8) * 8 + 0] = wall_clock64();
             // results land behind the selection's own scratch
             static_assert(sizeof(s_union) >= kTopkLdsBytes2 + 128, "selection scratch, ids and weights must fit the shared area");
             int32_t *lds_ids = reinterpret_cast<int32_t *>(s_union + kTopkLdsBytes2);
             float *lds_w = reinterpret_cast<float *>(s_union + kTopkLdsBytes2 + 64);
             // the selection itself publishes the replicas that the routed workgroups wait for, ahead of the weights
             topk_block(a.logits, a.E, a.k, a.w_scale, lds_ids, lds_w, a.ids_override, s_union, lane, wave,
-                       a.trace ? a.trace + (0 * 16 + 9) * 8 : nullptr, a.ids_tagged, kTagCopies);
+                       (TRACE && a.trace) ? a.trace + (0 * 16 + 9) * 8 : nullptr, a.ids_tagged, kTagCopies);
             if (wave == 0) {
                 wave_lds_fence();
                 // the plain copies for dispatch C
@@ -894,7 +897,7 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
                     a.ids[lane] = lds_ids[lane];
                     a.weights[lane] = lds_w[lane];
                 }
-                if (a.trace && lane == 0) a.trace[(0 * 16 + 8) * 8 + 1] = wall_clock64();
+                if (TRACE && a.trace && lane == 0) a.trace[(0 * 16 + 8) * 8 + 1] = wall_clock64();
             } else if (wave == 5 && lane == 0) {
                 // off the selection's path: the shared expert's gate, and the counter for the next layer pass
                 if (a.sh_inp) {
@@ -904,7 +907,7 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
                 a.arrive[0] = 0u;
             }
         }
-        mark(a, 0, 2);
+        mark<TRACE>(a, 0, 2);
         return;
     }
 
@@ -936,7 +939,7 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
     } else {
         lds_quantize_q8_0(a.x, a.H, xq, reinterpret_cast<uint16_t *>(xscale), threadIdx.x, 512);
     }
-    mark(a, 1, 1);
+    mark<TRACE>(a, 1, 1);
     __shared__ int s_expert;
     const int n_routed_wgs = LOOP ? static_cast<int>(gridDim.x) - a.n_router_wgs - n_shared_wgs : 0;
     int item = bw;
@@ -955,7 +958,7 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
             s_expert = static_cast<int>(e);
         }
         __syncthreads();
-        mark(a, 1, 2);
+        mark<TRACE>(a, 1, 2);
         const int e = s_expert;
         if (e < 0 || e >= a.E) return;  // the wait ran out (status is set): leave without touching memory
         const uint8_t *gate = mat_ptr_expert<0>(a.gate_up, e);
@@ -989,7 +992,7 @@ __global__ __launch_bounds__(512, 6) void k_layer_ab(LayerArgs a) {
             q8_row_wave<2>(rows, nb, xq, reinterpret_cast<const uint16_t *>(xscale), tiles[wave], lane, gu);
         }
         if (lane == 0 && r < a.F) act[r] = silu_ggml(gu[0]) * gu[1];
-        mark(a, 1, 3);
+        mark<TRACE>(a, 1, 3);
         if (LOOP) {
             item += n_routed_wgs;
             __syncthreads();  // s_expert is free for the next item
@@ -1092,7 +1095,7 @@ __global__ __launch_bounds__(TYPE == 20 ? 256 : 512) void k_layer_b(LayerArgs a)
 // products, which keeps it within 80 registers: the waves of a workgroup go to the four SIMDs in turn, so three
 // workgroups of six waves need six wave slots on two of them.  dynamic LDS per wave: two quantised activations and a
 // staging area of 4 * NB * 34 bytes.
-template <int KIND, bool COAL, int NB = 16, bool TWO = false, bool PART = false>
+template <int KIND, bool COAL, int NB = 16, bool TWO = false, bool PART = false, bool TRACE = false>
 __global__ __launch_bounds__(TWO ? 576 : 1024) __attribute__((amdgpu_waves_per_eu(TWO ? 6 : 4)))
 void k_layer_c(LayerArgs a) {
     extern __shared__ __align__(16) uint8_t lds_c[];
@@ -1116,7 +1119,7 @@ void k_layer_c(LayerArgs a) {
     if (a.clear_tagged && blockIdx.x == 0)
         for (int i = threadIdx.x; i < kTagCopies * 16; i += blockDim.x)
             __hip_atomic_store(a.ids_tagged + i, kTagInvalid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    mark(a, 2, 0);
+    mark<TRACE>(a, 2, 0);
     // combine operands, requested early: lane m keeps router weight m, lane 16 the shared gate
     float wreg = 0.0f, res_pre = 0.0f, inject = 0.0f;
     unsigned bad = 0u;  // a bounded wait of this layer pass ran out: the results below are replaced by NaN
@@ -1183,11 +1186,11 @@ void k_layer_c(LayerArgs a) {
             words[q] = q8 ? RawQ8::kWords : RawW::kWords;
             raw[q] = q8_rows4_coal_request_any<NB>(w + static_cast<size_t>(r0) * NB * (q8 ? 34 : RawW::kBlk), words[q], lane);
         }
-        mark(a, 2, 1);
+        mark<TRACE>(a, 2, 1);
         wave_lds_fence();
 #pragma unroll
         for (int q = 0; q < 2; ++q) quantise_act(v[q], aq2[q], ad2[q]);
-        mark(a, 2, 6);
+        mark<TRACE>(a, 2, 6);
 #pragma unroll
         for (int q = 0; q < 2; ++q) q8_rows4_coal_stage_any<NB>(raw[q], stage2[q], words[q], lane);
         wave_lds_fence();
@@ -1203,7 +1206,7 @@ void k_layer_c(LayerArgs a) {
                                          : q8_rows4_coal_dots<KIND, NB>(stage2[q], aq2[q], ad2[q], tiles[wave], lane);
             }
             if ((lane & 15) == 0) ybuf[mm[q] * 4 + r4] = y;
-            mark(a, 2, q == 0 ? 2 : 5);
+            mark<TRACE>(a, 2, q == 0 ? 2 : 5);
         }
     } else
     for (int m = wave; m < n_act; m += nwaves) {
@@ -1219,7 +1222,7 @@ void k_layer_c(LayerArgs a) {
                 const auto raw = q8_rows4_coal_request<0, NB>(w + static_cast<size_t>(r0) * NB * 34, lane);
                 wave_lds_fence();
                 quantise_act(v, aq, ad);
-                mark(a, 2, 1);
+                mark<TRACE>(a, 2, 1);
                 if (PART && !is_shared)
                     y = q8_rows4_coal_finish<0, NB, PART>(raw, aq, ad, tiles[wave], lane, a.down_part + (static_cast<size_t>(m) * a.H + r0) * (NB * 8));
                 else
@@ -1228,7 +1231,7 @@ void k_layer_c(LayerArgs a) {
                 const auto raw = q8_rows4_coal_request<1, NB>(w + static_cast<size_t>(r0) * NB * 18, lane);
                 wave_lds_fence();
                 quantise_act(v, aq, ad);
-                mark(a, 2, 1);
+                mark<TRACE>(a, 2, 1);
                 y = q8_rows4_coal_finish<1, NB, PART>(raw, aq, ad, tiles[wave], lane,
                                                       PART ? a.down_part + (static_cast<size_t>(m) * a.H + r0) * (NB * 8) : nullptr);
             }
@@ -1243,7 +1246,7 @@ void k_layer_c(LayerArgs a) {
                 wave_lds_fence();
                 lds_quantize_q8_0(a.act + static_cast<size_t>(m) * a.F, a.F, aq, ad, lane, 64);
                 wave_lds_fence();
-                mark(a, 2, 1);
+                mark<TRACE>(a, 2, 1);
             };
             int32_t *pp = (PART && !is_shared) ? a.down_part + (static_cast<size_t>(m) * a.H + r0) * (static_cast<size_t>(nb) * 8) : nullptr;
             if (PART && !is_shared && KIND == 0)
@@ -1254,10 +1257,10 @@ void k_layer_c(LayerArgs a) {
                 q8_rows4_multi<1, 1, 1, PART>(rows, nrows, nb, aq, ad, tiles[wave], lane, y, pp, 0, quantise);
             if ((lane & 15) == 0) ybuf[m * 4 + r4] = y[0];
         }
-        mark(a, 2, 2);
+        mark<TRACE>(a, 2, 2);
     }
     __syncthreads();
-    mark(a, 2, 3);
+    mark<TRACE>(a, 2, 3);
     if (wave == 0) {
         // every lane folds row r0 + (lane & 3); lanes 0..3 store it
         const int row = r0 + lane;
@@ -1299,7 +1302,7 @@ void k_layer_c(LayerArgs a) {
             }
         }
     }
-    mark(a, 2, 4);
+    mark<TRACE>(a, 2, 4);
 }
 
 }  // namespace wd

@@ -474,12 +474,19 @@ int launch_a(const LayerArgs &a, hipStream_t st) {
 template <int TYPE, bool COAL, int NB>
 void launch_layer_ab(bool loop, dim3 grid, dim3 block, size_t lds, hipStream_t st, const LayerArgs &m) {
     const bool part = m.gup_part != nullptr;  // the variants that also store the int32 chunk sums
+    // (the time stamps are a variant of their own, so that the others run without their tests; no stamps are taken
+    // while the chunk sums are exported)
+    const bool trace = m.trace != nullptr && !part;
     if (loop && part)
         k_layer_ab<TYPE, COAL, NB, true, true><<<grid, block, lds, st>>>(m);
+    else if (loop && trace)
+        k_layer_ab<TYPE, COAL, NB, true, false, true><<<grid, block, lds, st>>>(m);
     else if (loop)
         k_layer_ab<TYPE, COAL, NB, true><<<grid, block, lds, st>>>(m);
     else if (part)
         k_layer_ab<TYPE, COAL, NB, false, true><<<grid, block, lds, st>>>(m);
+    else if (trace)
+        k_layer_ab<TYPE, COAL, NB, false, false, true><<<grid, block, lds, st>>>(m);
     else
         k_layer_ab<TYPE, COAL, NB, false><<<grid, block, lds, st>>>(m);
 }
@@ -487,6 +494,8 @@ template <int KIND, bool COAL, int NB, bool TWO>
 void launch_layer_c(dim3 grid, dim3 block, size_t lds, hipStream_t st, const LayerArgs &a) {
     if (a.down_part)
         k_layer_c<KIND, COAL, NB, TWO, true><<<grid, block, lds, st>>>(a);
+    else if (a.trace)
+        k_layer_c<KIND, COAL, NB, TWO, false, true><<<grid, block, lds, st>>>(a);
     else
         k_layer_c<KIND, COAL, NB, TWO><<<grid, block, lds, st>>>(a);
 }
