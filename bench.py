@@ -59,6 +59,10 @@ def parse():
     ap.add_argument("--source", choices=["pinned", "file", "mapping"], default="pinned",
                     help="lru mode: where the routed experts live - pinned host memory; a GGUF file written to --file-dir, "
                          "misses read with pread into the cache's pinned ring; the same file as a plain (pageable) mapping")
+    ap.add_argument("--host-layout", choices=["tensors", "packed"], default="tensors",
+                    help="lru mode with --source pinned: the host copy as three tensors per layer (as in a model file), or packed "
+                         "per expert - gate, up and down of an expert back to back, one slot apart - so that a miss is one "
+                         "contiguous piece")
     ap.add_argument("--file-dir", default="/tmp", help="lru mode with --source file/mapping: directory of the model file")
     ap.add_argument("--pread-threads", type=int, default=4)
     ap.add_argument("--lru-driver", choices=["trace", "router"], default="trace",
@@ -81,9 +85,11 @@ def parse():
     return ap.parse_args()
 
 
-def build_stack(torch, synth, capi, n_layers, n_experts, seed, offload=False):
+def build_stack(torch, synth, capi, n_layers, n_experts, seed, offload=False, packed=False):
     """Random GGUF-layout weights for n_layers C2 layers, generated on the device.  With `offload` the routed
-    tensors are moved to pinned host memory (returned per layer) and their device copies dropped."""
+    tensors are moved to pinned host memory (returned per layer) and their device copies dropped; `packed` lays
+    them out per expert (gate, up, down of expert e back to back, experts one slot apart) in ONE buffer per layer and
+    returns that buffer's three starting points."""
     H, F, k = 2048, 512, 10
     g = torch.Generator(device="cuda")
     g.manual_seed(seed)
@@ -117,7 +123,19 @@ def build_stack(torch, synth, capi, n_layers, n_experts, seed, offload=False):
             setattr(d, name, tensor.data_ptr())
         d.gate_stride = d.up_stride = F * rb_iq3
         d.down_stride = H * rb_q8f
-        if offload:
+        if offload and packed:
+            gbytes, dbytes = F * rb_iq3, H * rb_q8f
+            slot = torch.cat([t["gate"].view(n_experts, gbytes), t["up"].view(n_experts, gbytes),
+                              t["down"].view(n_experts, dbytes)], dim=1).contiguous()
+            h = C.c_void_p()
+            capi.call("wd_malloc_host", C.byref(h), slot.numel())
+            capi.call("wd_memcpy_d2h", h, C.c_void_p(slot.data_ptr()), slot.numel(), None)
+            del slot
+            for name in ("gate", "up", "down"):
+                t[name] = None
+                setattr(d, name, None)
+            pinned.append([h, C.c_void_p(h.value + gbytes), C.c_void_p(h.value + 2 * gbytes)])
+        elif offload:
             host = []
             for name in ("gate", "up", "down"):
                 h = C.c_void_p()      # exact-size pinned buffer (torch's pinned allocator rounds sizes up to 2^n)
@@ -309,12 +327,16 @@ def bench_lru(args, torch, capi, synth):
     model_file = None
     if args.source == "pinned":
         note("generating %d layers x %d experts, routed tensors to pinned host memory" % (NL, E))
-        layers, keep, pinned = build_stack(torch, synth, capi, NL, E, synth.BASE_SEED, offload=True)
+        packed = args.host_layout == "packed"
+        layers, keep, pinned = build_stack(torch, synth, capi, NL, E, synth.BASE_SEED, offload=True, packed=packed)
         torch.cuda.synchronize()
         capi.call("wd_expert_cache_create", C.byref(cache), int(args.cache_gib * (1 << 30)), gb, gb, db, NL, E, 0)
         capi.call("wd_expert_cache_set_copy_kernel", cache, 1 if args.fill == "kernel" else 0)
         for l in range(NL):
-            capi.call("wd_expert_cache_register_layer", cache, l, *pinned[l])
+            if packed:
+                capi.call("wd_expert_cache_register_layer_strided", cache, l, *pinned[l], slot_bytes, slot_bytes, slot_bytes)
+            else:
+                capi.call("wd_expert_cache_register_layer", cache, l, *pinned[l])
     else:
         # the routed tensors go into a GGUF file (names of the model files), are dropped from the device, and come back
         # through the library's reader: the cache's host sources are pointers into its mapping

@@ -2,6 +2,7 @@
 (src/expert_cache.cuh:2252-2326, :2467-2493), device slot table contents, bytes in the slots, and a
 layer pass through the slot table that is bit-identical to the all-resident pass."""
 import ctypes as C
+import json
 
 import numpy as np
 import pytest
@@ -106,6 +107,56 @@ def test_lru_semantics_and_contents(g, partition):
     assert (st.hits, st.misses, st.evictions) == (model.hits, model.misses, model.evictions)
     assert st.accesses == 60 * k and st.bytes_copied == model.misses * (gb + ub + db)
     assert st.slots == n_slots and st.resident == sum(s is not None for s in model.slots)
+    capi.call("wd_expert_cache_destroy", cache)
+
+
+@pytest.mark.parametrize("copy_kernel", [1, 0])
+def test_host_copy_packed_per_expert(g, copy_kernel):
+    """A host copy that holds each expert's gate, up and down bytes back to back (one record per expert, the three
+    strides all one record) is filled as one piece; the slots must read as they do from three separate tensors."""
+    import torch
+    n_layers, E, k = 2, 12, 3
+    gb, ub, db = 512, 256, 1024
+    rec = gb + ub + db
+    n_slots = 7
+    host = _host_layers(n_layers, E, gb, ub, db, SEED + 21)
+    packed = []
+    for l in range(n_layers):
+        p = np.concatenate([host[l][0].reshape(E, gb), host[l][1].reshape(E, ub), host[l][2].reshape(E, db)], axis=1)
+        packed.append(torch.from_numpy(np.ascontiguousarray(p).reshape(-1)).pin_memory())
+    cache = C.c_void_p()
+    capi.call("wd_expert_cache_create", C.byref(cache), n_slots * rec, gb, ub, db, n_layers, E, 0)
+    capi.call("wd_expert_cache_set_copy_kernel", cache, copy_kernel)
+    for l in range(n_layers):
+        base = packed[l].data_ptr()
+        capi.call("wd_expert_cache_register_layer_strided", cache, l, C.c_void_p(base), C.c_void_p(base + gb),
+                  C.c_void_p(base + gb + ub), rec, rec, rec)
+    model = ModelCache(n_slots, n_layers, False)
+    rng = np.random.default_rng(SEED + 22)
+    lib = capi.load()
+    pool = lib.wd_expert_cache_pool(cache)
+    for step in range(30):
+        layer = int(rng.integers(0, n_layers))
+        ids = rng.choice(E, size=k, replace=False).astype(np.int32)
+        capi.call("wd_expert_cache_acquire", cache, layer, ids.ctypes.data_as(C.c_void_p), k, None, g.stream())
+        want = [model.acquire(layer, int(e)) for e in ids]
+        g.sync()
+        table = g.view(lib.wd_expert_cache_slot_table(cache, layer), E, np.int32)
+        for e, (slot, _) in zip(ids, want):
+            assert table[e] == slot
+            got = g.view(pool + slot * rec, rec, np.uint8)
+            assert np.array_equal(got[:gb], host[layer][0][e * gb:(e + 1) * gb])
+            assert np.array_equal(got[gb:gb + ub], host[layer][1][e * ub:(e + 1) * ub])
+            assert np.array_equal(got[gb + ub:], host[layer][2][e * db:(e + 1) * db])
+    st = capi.CacheStats()
+    capi.call("wd_expert_cache_get_stats", cache, C.byref(st))
+    assert (st.hits, st.misses) == (model.hits, model.misses) and st.bytes_copied == model.misses * rec
+    need = lib.wd_expert_cache_dump_json(cache, None, 0)
+    buf = C.create_string_buffer(need + 1)
+    lib.wd_expert_cache_dump_json(cache, buf, need + 1)
+    d = json.loads(buf.value.decode())
+    by = ("fills_by_copy_kernel", "fills_by_memcpy")
+    assert d[by[1 - copy_kernel]] == model.misses and d[by[copy_kernel]] == 0
     capi.call("wd_expert_cache_destroy", cache)
 
 
@@ -251,7 +302,6 @@ def test_layer_through_slot_table(g, oracle):
 def test_monitor_and_shadow_caches(g):
     """Counters and counterfactual caches against a direct model: an LRU shadow with the pool's own capacity must
     hit exactly as often as the pool, a larger one at least as often, and the JSON dump must carry the counters."""
-    import json
     E, NL, k = 16, 2, 4
     gb, ub, db = 256, 256, 512
     slots = 6

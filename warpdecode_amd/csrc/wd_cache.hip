@@ -809,6 +809,7 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
                                   c->h_down[layer] + static_cast<size_t>(e) * c->s_down[layer]};
         uint8_t *dst3[3] = {dst, dst + c->gate_bytes, dst + c->gate_bytes + c->up_bytes};
         const size_t len3[3] = {c->gate_bytes, c->up_bytes, c->down_bytes};
+        const bool one_piece = src3[0] + len3[0] == src3[1] && src3[1] + len3[1] == src3[2];
         int ra_entry = -1;
         uint8_t *ra_buf = by_file && c->ra.enabled() ? c->ra.borrow(key, &ra_entry) : nullptr;
         if (ra_buf) {
@@ -855,16 +856,22 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
         } else if (by_kernel) {
             if (n_fill + 3 > kMaxFillSegments)  // (token-ahead groups only: one call alone never has that many)
                 if (const int rc = launch_fill_segments(c, fills, n_fill, max_words)) return rc;
-            for (int q = 0; q < 3; ++q) {
+            // an expert whose three pieces lie back to back on the host (a copy packed per expert) is one segment
+            const int n_seg = one_piece ? 1 : 3;
+            for (int q = 0; q < n_seg; ++q) {
                 fills.src[n_fill] = src3[q], fills.dst[n_fill] = dst3[q];
-                fills.words[n_fill] = static_cast<uint32_t>(len3[q] / 16);
+                fills.words[n_fill] = static_cast<uint32_t>((one_piece ? c->slot_bytes : len3[q]) / 16);
                 max_words = fills.words[n_fill] > max_words ? fills.words[n_fill] : max_words;
                 ++n_fill;
             }
             ++c->kernel_fills;
         } else {
-            for (int q = 0; q < 3; ++q)
-                WD_HIP(hipMemcpyAsync(dst3[q], src3[q], len3[q], hipMemcpyHostToDevice, c->copy_stream));
+            if (one_piece) {
+                WD_HIP(hipMemcpyAsync(dst, src3[0], c->slot_bytes, hipMemcpyHostToDevice, c->copy_stream));
+            } else {
+                for (int q = 0; q < 3; ++q)
+                    WD_HIP(hipMemcpyAsync(dst3[q], src3[q], len3[q], hipMemcpyHostToDevice, c->copy_stream));
+            }
             ++c->dma_fills;
         }
         c->stats.bytes_copied += c->slot_bytes;
