@@ -79,6 +79,9 @@ def parse():
                     help="resident mode: the stack as ONE launch of resident workgroups (default), or two dispatches per layer")
     ap.add_argument("--repeats", type=int, default=5, help="further repeats of the timed region, for the spread in the JSON line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--site-profile", type=int, default=0, metavar="TOKENS",
+                    help="resident mode: afterwards run TOKENS eager steps with the library's site profiler on (device, host and "
+                         "gap time per bracketed site and token), print its report and add it to the JSON line")
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="wall-clock seconds of CPU layer passes to accumulate for cpu_baseline (all host threads busy)")
     ap.add_argument("--check", action="store_true", help="verify one layer pass against the CPU oracle first")
@@ -1075,6 +1078,29 @@ def main():
     torch.cuda.synchronize()
     del cal_src, cal_dst
 
+    site_profile = None
+    if args.site_profile > 0:
+        # eager launches: a bracket on a capturing stream is not recorded.  One pass per form of the stack.
+        import re
+        site_profile = {}
+        lib = capi.load()
+        for form, flags in (("resident_launch", STACK_FLAGS), ("per_layer_dispatches", STACK_FLAGS | PER_LAYER)):
+            capi.call("wd_profile_enable", 1)
+            capi.call("wd_profile_reset")
+            for j in range(args.site_profile):
+                d_x.copy_(d_xs[j % total_steps], non_blocking=True)
+                d_trace.copy_(d_trace_all[j % total_steps], non_blocking=True)
+                launch_stack(flags)
+                torch.cuda.synchronize()
+                capi.call("wd_profile_flush_token")
+            need = lib.wd_profile_report(None, 0)
+            buf = C.create_string_buffer(need + 1)
+            lib.wd_profile_report(buf, need + 1)
+            capi.call("wd_profile_enable", 0)
+            print("site profile, %s:\n%s" % (form, buf.value.decode()), file=sys.stderr, flush=True)
+            site_profile[form] = {line.split()[1]: {key: float(v) for key, v in re.findall(r"([a-z/]+)=\s*([-0-9.]+)", line)}
+                                  for line in buf.value.decode().splitlines()[1:]}
+
     out = {
         "metric": "MoE layer batch=1 decode: synthetic 48-layer tok/s (achieved HBM GB/s in roofline)",
         "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -1092,6 +1118,8 @@ def main():
                    "in_dispatch_waits_ok": waits_ok},
         "roofline": roofline,
     }
+    if site_profile is not None:
+        out["config"]["site_profile_ms_per_token"] = site_profile
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
     print(json.dumps(out))

@@ -405,6 +405,56 @@ int wd_moe_stack_cached_f32(const wd_moe_layer *layers, int n_layers, wd_expert_
                             const int32_t *d_ids_trace, float residual_scale, unsigned flags, void *stream);
 
 
+/* ---- site profiler ---------------------------------------------------------------------------
+ * Event brackets around regions of the MoE path, accumulated per decode token into device time (HIP events on the
+ * bracket's stream), host time (steady clock) and their gap; one report line per site.  reference:
+ * Q38MoeKernelProfiler / Q38MoeKernelScope and its sites, src/qwen38_moe.cuh:296-535.  Sites 0..23 carry the
+ * reference's numbers and names; a caller brackets them exactly where the reference does, and the library brackets
+ * the ones its own code covers: moe.routed_total (a layer call), moe.acquire, moe.shared, moe.finish, and - on the
+ * WD_MOE_STAGED path, whose dispatches are the reference's stages - moe.router.gemv, moe.router.topk, moe.rx_quant,
+ * moe.batch.gate_up, moe.batch.silu, moe.batch.q8_quant, moe.batch.down, moe.batch.accum.  Sites from
+ * WD_PROFILE_FIRST_OWN_SITE on are dispatches that only exist here.  Off by default: every hook is then one load
+ * and a branch.  A bracket on a stream that is being captured is not recorded and counts as dropped.  Process-wide;
+ * brackets of one site must not overlap across threads. */
+enum {
+    WD_SITE_STAGE_TOTAL = 0, WD_SITE_ROUTED_TOTAL, WD_SITE_ROUTER, WD_SITE_ROUTER_QUANT, WD_SITE_ROUTER_GEMV,
+    WD_SITE_ROUTER_TOPK, WD_SITE_ROUTER_D2H, WD_SITE_ROUTER_SYNC, WD_SITE_ACCUM_ZERO, WD_SITE_RX_QUANT,
+    WD_SITE_ACQUIRE, WD_SITE_PTR_H2D, WD_SITE_BATCH_TOTAL, WD_SITE_GATE_UP_GEMV, WD_SITE_SILU,
+    WD_SITE_Q8_QUANT, WD_SITE_DOWN_GEMV, WD_SITE_ACCUM, WD_SITE_CAPTURE, WD_SITE_LOOP_TOTAL,
+    WD_SITE_FINISH, WD_SITE_SHARED, WD_SITE_SHARED_GATE, WD_SITE_MIRROR,
+    WD_PROFILE_FIRST_OWN_SITE,
+    WD_SITE_FUSED_AB = WD_PROFILE_FIRST_OWN_SITE, /* router + selection + shared and routed gate/up in one launch */
+    WD_SITE_FUSED_A,        /* router + selection + shared gate/up as a launch of its own */
+    WD_SITE_FUSED_B,        /* routed gate/up + SwiGLU as a launch of its own */
+    WD_SITE_FUSED_C,        /* down projections + ordered combine */
+    WD_SITE_STACK_TOTAL,    /* one wd_moe_stack_f32 / wd_moe_stack_cached_f32 call */
+    WD_SITE_STACK_RESIDENT, /* the one-launch form of the stack */
+    WD_SITE_CACHE_FILL,     /* the fills of one acquire, on the cache's copy stream */
+    WD_SITE_TOKENS_TOTAL,   /* one multi-token pass */
+    WD_SITE_TOKENS_A, WD_SITE_TOKENS_B, WD_SITE_TOKENS_C,
+    WD_SITE_HC_COMBINE,     /* the hyper-connection combine as a launch of its own */
+    WD_PROFILE_SITE_COUNT
+};
+typedef struct {
+    unsigned long long calls;      /* brackets whose two events were read */
+    unsigned long long recorded;   /* brackets that recorded both events */
+    unsigned long long dropped;    /* brackets without room, on a capturing stream, or whose event record failed */
+    unsigned long long unreadable; /* brackets whose elapsed time could not be read at the flush */
+    double device_ms, host_ms;     /* totals over all flushed tokens */
+} wd_profile_site_stat;
+int wd_profile_enable(int on);                       /* the first enable creates the events */
+int wd_profile_enabled(void);
+int wd_profile_begin(int site, void *stream);        /* reference mark_begin; nested brackets of a site count once */
+int wd_profile_end(int site, void *stream);          /* reference mark_end */
+int wd_profile_flush_token(void);                    /* once per token, after the bracketed streams were synchronised */
+int wd_profile_site(int site, wd_profile_site_stat *out, unsigned long long *tokens);
+const char *wd_profile_site_name(int site);          /* "unknown" outside 0..WD_PROFILE_SITE_COUNT-1 */
+/* The reference's summary (print_summary): "[moe-profile] <site> dev= host= gap= calls/token= recorded= dropped=
+ * evfail=", per token, one line per site that saw anything.  Returns the bytes needed without the terminator. */
+size_t wd_profile_report(char *buf, size_t cap);
+int wd_profile_reset(void);                          /* forgets every total; keeps the events and the switch */
+
+
 /* ---- GGUF container ---------------------------------------------------------------------------
  * Read-only memory map of a GGUF file (versions 2 and 3) with its metadata and tensor directory parsed; tensor
  * views point into the mapping (raw block bytes, as the expert cache, wd_memcpy_h2d and the layer descriptors

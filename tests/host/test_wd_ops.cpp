@@ -700,6 +700,53 @@ static void gpu_checks() {
         }
         CHECK(wd_moe_scratch_status(scratch.handle()) == 0, "an in-dispatch wait ran out");
     }
+    // the site profiler, bracketed the way the reference's stage code brackets a token (src/qwen38_moe.cuh:296-535):
+    // a ten-slot pool, so every layer goes selection -> ids to the host -> acquire -> expert dispatches
+    {
+        Q38MoeKernelProfiler &prof = Q38MoeKernelProfiler::instance();
+        CHECK(!prof.enabled(), "the profiler is off unless WARODECODE_MOE_PROFILE is set");
+        check(wd_profile_enable(1), "profiler on");
+        check(wd_profile_reset(), "profiler reset");
+        GpuExpertCache cache;
+        cache.initialize((10 * slot + (1u << 20) - 1) >> 20, L[0].t_gate, L[0].t_up, L[0].t_down, 0, 0, 0, opt);
+        for (int l = 0; l < layers; ++l) cache.register_layer_experts(l, L[l].t_gate, L[l].t_up, L[l].t_down);
+        Rng r(321);
+        DeviceFloatArray dx(H), dout(H);
+        const int tokens = 2;
+        for (int token = 0; token < tokens; ++token) {
+            {
+                Q38MoeKernelScope stage(kQ38MoeSiteStageTotal, stream);
+                for (int l = 0; l < layers; ++l) {
+                    const std::vector<float> x = rms_normed(r, H);
+                    dx.upload(x.data(), H);
+                    const std::vector<float> got = run_three_calls(l, L[l], routers[l], cache, shared[l], scratch, dx, dout, stream);
+                    std::vector<float> want(H);
+                    wdo_moe_layer(&L[l].o, x.data(), want.data(), nullptr, 0);
+                    CHECK(same_bits(got.data(), want.data(), H), "profiled token %d layer %d: output differs from the oracle", token, l);
+                }
+            }
+            check(wd_device_sync(), "sync");
+            prof.flush_token();
+        }
+        const unsigned long long n = static_cast<unsigned long long>(tokens) * layers;
+        const Q38MoeSiteStat stage = prof.site(kQ38MoeSiteStageTotal), routed = prof.site(kQ38MoeSiteRoutedTotal),
+                             select = prof.site(kQ38MoeSiteRouter), sync = prof.site(kQ38MoeSiteRouterSync),
+                             acquire = prof.site(kQ38MoeSiteAcquire), sh = prof.site(kQ38MoeSiteShared), fin = prof.site(kQ38MoeSiteFinish);
+        CHECK(stage.calls == tokens && stage.overflow == 0 && stage.elapsed_fail == 0, "stage brackets: %llu", stage.calls);
+        CHECK(routed.calls == n && select.calls == n && sync.calls == n && acquire.calls == n, "per-layer brackets: %llu %llu %llu %llu of %llu",
+              routed.calls, select.calls, sync.calls, acquire.calls, n);
+        CHECK(sh.calls == n && fin.calls == n, "shared expert and finish brackets: %llu %llu", sh.calls, fin.calls);
+        CHECK(stage.total_ms >= 0.98 * routed.total_ms && routed.total_ms >= 0.98 * select.total_ms && select.total_ms > 0.0, "device times nest");
+        CHECK(stage.total_host_ms >= routed.total_host_ms && routed.total_host_ms >= select.total_host_ms && select.total_host_ms >= sync.total_host_ms &&
+                  sync.total_host_ms > 0.0, "host times nest");
+        const std::string text = prof.summary();
+        CHECK(text.find("[moe-profile] tokens=2 unit=ms_per_token") == 0 && text.find("moe.router_select") != std::string::npos &&
+                  text.find("moe.fused.c") != std::string::npos && text.find("moe.batch.gate_up") == std::string::npos,
+              "summary:\n%s", text.c_str());
+        CHECK(std::string(q38_moe_site_name(kQ38MoeSiteRouterTopk)) == "moe.router.topk" && kQ38MoeSiteCount == 24, "site names");
+        check(wd_profile_enable(0), "profiler off");
+        check(wd_profile_reset(), "profiler reset");
+    }
     wd_stream_destroy(stream);
 }
 

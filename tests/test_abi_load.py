@@ -34,3 +34,28 @@ def test_argument_errors_are_reported():
     assert lib.wd_gemv_q8_k_f32(synth.Q8_0, C.c_void_p(8), 4, 256, None, None, None, None, None) == -1
     with pytest.raises(capi.WdError):
         capi.call("wd_q8_0_quantize_f32", None, 33, None, None, None)
+
+
+def test_profiler_switched_off_touches_nothing():
+    """The site profiler's names follow the reference's numbering (src/qwen38_moe.cuh:296-352), and with the switch off
+    its hooks are no-ops that need no device."""
+    from warpdecode_amd import capi
+    lib = capi.load()
+    names = [lib.wd_profile_site_name(i).decode() for i in range(24)]
+    assert names[0] == "moe.stage_total" and names[1] == "moe.routed_total" and names[2] == "moe.router_select"
+    assert names[10] == "moe.acquire" and names[13] == "moe.batch.gate_up" and names[17] == "moe.batch.accum"
+    assert names[20] == "moe.finish" and names[23] == "moe.mirror" and len(set(names)) == 24
+    assert lib.wd_profile_site_name(24) == b"moe.fused.ab"
+    assert lib.wd_profile_site_name(-1) == b"unknown" and lib.wd_profile_site_name(1000) == b"unknown"
+    assert lib.wd_profile_enabled() == 0
+    capi.call("wd_profile_begin", 0, None)
+    capi.call("wd_profile_end", 0, None)
+    capi.call("wd_profile_flush_token")
+    st, tokens = capi.ProfileSiteStat(), C.c_ulonglong(7)
+    capi.call("wd_profile_site", 0, C.byref(st), C.byref(tokens))
+    assert (st.calls, st.recorded, st.dropped, st.host_ms, tokens.value) == (0, 0, 0, 0.0, 0)
+    assert lib.wd_profile_begin(1000, None) != 0 and b"out of range" in lib.wd_last_error()
+    need = lib.wd_profile_report(None, 0)
+    buf = C.create_string_buffer(need + 1)
+    assert lib.wd_profile_report(buf, need + 1) == need
+    assert buf.value == b"[moe-profile] tokens=0 unit=ms_per_token\n"

@@ -49,6 +49,11 @@ class GgufTensorInfo(C.Structure):
                 ("relative_offset", C.c_uint64), ("bytes", C.c_uint64), ("data", vp)]
 
 
+class ProfileSiteStat(C.Structure):
+    _fields_ = [("calls", C.c_ulonglong), ("recorded", C.c_ulonglong), ("dropped", C.c_ulonglong),
+                ("unreadable", C.c_ulonglong), ("device_ms", C.c_double), ("host_ms", C.c_double)]
+
+
 class CacheStats(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in ("accesses", "hits", "misses", "evictions", "bytes_copied", "slots",
                                           "slot_bytes", "resident")]
@@ -98,6 +103,15 @@ _SIGS = {
     "wd_moe_scratch_trace": (vp, [vp, i32]),
     "wd_moe_scratch_trace_resident": (vp, [vp, i32, i32]),
     "wd_moe_scratch_omit_resident": (i32, [vp, i32]),
+    "wd_profile_enable": (i32, [i32]),
+    "wd_profile_enabled": (i32, []),
+    "wd_profile_begin": (i32, [i32, vp]),
+    "wd_profile_end": (i32, [i32, vp]),
+    "wd_profile_flush_token": (i32, []),
+    "wd_profile_site": (i32, [i32, C.POINTER(ProfileSiteStat), C.POINTER(C.c_ulonglong)]),
+    "wd_profile_site_name": (C.c_char_p, [i32]),
+    "wd_profile_report": (sz, [C.c_char_p, sz]),
+    "wd_profile_reset": (i32, []),
     "wd_moe_layer_f32": (i32, [C.POINTER(MoeLayer), vp, vp, vp, u32, vp]),
     "wd_moe_stack_cached_f32": (i32, [C.POINTER(MoeLayer), i32, vp, vp, vp, vp, vp, vp, f32, u32, vp]),
     "wd_moe_scratch_status": (i32, [vp]),

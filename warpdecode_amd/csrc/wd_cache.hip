@@ -23,6 +23,7 @@
 //     reference's ExpertFileMap / ExpertPreadPool / pinned ring (src/expert_cache.cuh:204-508, :858-1583); the file
 //     is named by the caller or found through /proc/self/maps (wd_expert_cache_attach_mappings).
 #include "wd_common.h"
+#include "wd_profile.hpp"
 #include "wd_readahead.hpp"
 
 #include <fcntl.h>
@@ -678,6 +679,7 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
     for (int j = 0; j < k; ++j)
         WD_REQUIRE(h_ids[j] >= 0 && h_ids[j] < c->n_experts, "expert index out of range: %d", h_ids[j]);
     hipStream_t st = as_stream(stream);
+    SiteScope site(WD_SITE_ACQUIRE, st);
     const auto t_begin = std::chrono::steady_clock::now();
     struct Timer {
         wd_expert_cache *c;
@@ -903,6 +905,7 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
 
 int launch_fill_segments(wd_expert_cache *c, FillSegments &fills, int &n_fill, uint32_t &max_words) {
     if (n_fill > 0) {
+        SiteScope site(WD_SITE_CACHE_FILL, c->copy_stream);
         // enough workgroups per segment to keep the host link busy, few enough to leave the decode its compute units
         const uint32_t per_seg = (max_words + WD_FILL_THREADS * WD_FILL_UNROLL - 1) / (WD_FILL_THREADS * WD_FILL_UNROLL);
         k_fill_slots<<<dim3(per_seg < WD_FILL_WGS ? (per_seg ? per_seg : 1) : WD_FILL_WGS), dim3(WD_FILL_THREADS), 0, c->copy_stream>>>(fills, n_fill);

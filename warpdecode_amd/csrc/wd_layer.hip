@@ -1,5 +1,6 @@
 // Whole-layer entry points: scratch object and the staged layer pass (one launch per stage,
 // every stage a stand-alone operator of wd_ops.hip resolved against the device-side ids).
+#include "wd_profile.hpp"
 #include "wd_common.h"
 #include "wd_tokens.cuh"
 #include "wd_resident.cuh"
@@ -354,13 +355,18 @@ int layer_staged(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_s
 
     // 1. router logits (+ the shared expert's gate logit as one more row), softmax/top-k, sigmoid
     if (!pre) {
-        k_router_gemv<<<dim3((E + (shared ? 1 : 0) + 7) / 8), dim3(256), 0, st>>>(
-            L->router, d_x, s->logits, E, H, shared ? L->shared_gate_inp : nullptr, s->shared_gate);
-        WD_LAUNCH_CHECK();
+        {
+            SiteScope site(WD_SITE_ROUTER_GEMV, st);
+            k_router_gemv<<<dim3((E + (shared ? 1 : 0) + 7) / 8), dim3(256), 0, st>>>(
+                L->router, d_x, s->logits, E, H, shared ? L->shared_gate_inp : nullptr, s->shared_gate);
+            WD_LAUNCH_CHECK();
+        }
+        SiteScope site(WD_SITE_ROUTER_TOPK, st);
         k_topk_softmax<<<dim3(1), dim3(64), 0, st>>>(s->logits, E, k, L->expert_scale, s->ids, s->weights,
                                                      shared ? s->shared_gate : nullptr, ids_override);
         WD_LAUNCH_CHECK();
     } else if (shared) {
+        SiteScope site(WD_SITE_SHARED_GATE, st);
         k_router_gemv<<<dim3(1), dim3(256), 0, st>>>(L->router, d_x, s->logits, 0, H, L->shared_gate_inp, s->shared_gate);
         WD_LAUNCH_CHECK();
         k_sigmoid1<<<dim3(1), dim3(64), 0, st>>>(s->shared_gate);
@@ -368,21 +374,28 @@ int layer_staged(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_s
     }
 
     // 2. quantise the layer input for the consumers that need it
-    if (consumes_q8k(L->gate_type)) {
-        k_q8_k_quantize<<<dim3((H / 256 + 3) / 4), dim3(256), 0, st>>>(d_x, H / 256, s->xk_qs, s->xk_d, s->xk_bs);
-        WD_LAUNCH_CHECK();
-    }
-    if (!consumes_q8k(L->gate_type) || shared) {
-        k_q8_0_quantize<<<dim3((H / 32 + 31) / 32), dim3(256), 0, st>>>(d_x, H / 32, s->x0_qs, s->x0_d);
-        WD_LAUNCH_CHECK();
+    {
+        SiteScope site(WD_SITE_RX_QUANT, st);
+        if (consumes_q8k(L->gate_type)) {
+            k_q8_k_quantize<<<dim3((H / 256 + 3) / 4), dim3(256), 0, st>>>(d_x, H / 256, s->xk_qs, s->xk_d, s->xk_bs);
+            WD_LAUNCH_CHECK();
+        }
+        if (!consumes_q8k(L->gate_type) || shared) {
+            k_q8_0_quantize<<<dim3((H / 32 + 31) / 32), dim3(256), 0, st>>>(d_x, H / 32, s->x0_qs, s->x0_d);
+            WD_LAUNCH_CHECK();
+        }
     }
 
     // 3. gate/up of the k selected experts in one dispatch (2k matrices), then the shared expert's
     const bool part = s->gup != nullptr && s->gup_type == L->gate_type && s->dp_type == L->down_type;
-    if (const int rc = grouped_gemv(L->gate_type, routed_src(L, s, s->ids, false), 2 * k, F, H, s, s->x0_qs, s->x0_d, 0,
-                                    s->gate_up, part ? s->gup : nullptr, st))
-        return rc;
+    {
+        SiteScope site(WD_SITE_GATE_UP_GEMV, st);
+        if (const int rc = grouped_gemv(L->gate_type, routed_src(L, s, s->ids, false), 2 * k, F, H, s, s->x0_qs, s->x0_d, 0,
+                                        s->gate_up, part ? s->gup : nullptr, st))
+            return rc;
+    }
     if (shared) {
+        SiteScope site(WD_SITE_SHARED, st);
         MatSrc g{}, u{};
         g.single = L->shared_gate, u.single = L->shared_up;
         float *gu = s->gate_up + static_cast<size_t>(2) * k * F;
@@ -392,16 +405,26 @@ int layer_staged(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_s
 
     // 4. SwiGLU in f32, 5. Q8_0 re-quantisation, for k (+1) experts at once
     const int n_act = k + (shared ? 1 : 0);
-    k_silu_mul_experts<<<dim3((F + 255) / 256, n_act), dim3(256), 0, st>>>(s->gate_up, s->act, F);
-    WD_LAUNCH_CHECK();
-    k_q8_0_quantize<<<dim3((n_act * F / 32 + 31) / 32), dim3(256), 0, st>>>(s->act, n_act * F / 32, s->act_qs, s->act_d);
-    WD_LAUNCH_CHECK();
+    {
+        SiteScope site(WD_SITE_SILU, st);
+        k_silu_mul_experts<<<dim3((F + 255) / 256, n_act), dim3(256), 0, st>>>(s->gate_up, s->act, F);
+        WD_LAUNCH_CHECK();
+    }
+    {
+        SiteScope site(WD_SITE_Q8_QUANT, st);
+        k_q8_0_quantize<<<dim3((n_act * F / 32 + 31) / 32), dim3(256), 0, st>>>(s->act, n_act * F / 32, s->act_qs, s->act_d);
+        WD_LAUNCH_CHECK();
+    }
 
     // 6. down projections: k routed matrices with their own activations, then the shared expert
-    if (const int rc = grouped_gemv(L->down_type, routed_src(L, s, s->ids, true), k, H, F, s, s->act_qs, s->act_d, F,
-                                    s->expert_out, part ? s->dp : nullptr, st))
-        return rc;
+    {
+        SiteScope site(WD_SITE_DOWN_GEMV, st);
+        if (const int rc = grouped_gemv(L->down_type, routed_src(L, s, s->ids, true), k, H, F, s, s->act_qs, s->act_d, F,
+                                        s->expert_out, part ? s->dp : nullptr, st))
+            return rc;
+    }
     if (shared) {
+        SiteScope site(WD_SITE_SHARED, st);
         MatSrc d{};
         d.single = L->shared_down;
         if (const int rc = grouped_gemv(WD_TYPE_Q8_0, d, 1, H, F, s, s->act_qs + static_cast<size_t>(k) * F,
@@ -410,11 +433,15 @@ int layer_staged(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_s
     }
 
     // 7. ordered weighted sum and the shared branch
-    k_combine<<<dim3((H + 255) / 256), dim3(256), 0, st>>>(s->expert_out, s->weights, k, shared ? s->down_f32 : nullptr,
-                                                            s->shared_gate, s->accum, d_out, hc ? nullptr : residual,
-                                                            residual_scale, H);
-    WD_LAUNCH_CHECK();
+    {
+        SiteScope site(WD_SITE_ACCUM, st);
+        k_combine<<<dim3((H + 255) / 256), dim3(256), 0, st>>>(s->expert_out, s->weights, k, shared ? s->down_f32 : nullptr,
+                                                                s->shared_gate, s->accum, d_out, hc ? nullptr : residual,
+                                                                residual_scale, H);
+        WD_LAUNCH_CHECK();
+    }
     if (hc && residual) {
+        SiteScope site(WD_SITE_HC_COMBINE, st);
         k_hc_combine<0><<<dim3((H * hc->hc + 255) / 256), dim3(256), 0, st>>>(residual, d_out, nullptr, nullptr, hc->inject, H,
                                                                              hc->hc, hc->round_half);
         WD_LAUNCH_CHECK();
@@ -515,6 +542,7 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
     const bool merged = run_a && run_b && !a.preselected && !(flags & WD_MOE_SPLIT_AB) &&
                         (iq || L->gate_type == WD_TYPE_Q8_0);
     if (merged) {
+        SiteScope site(WD_SITE_FUSED_AB, st);
         LayerArgs m = a;
         m.n_router_wgs = (a.E + (shared ? 1 : 0) + 7) / 8;  // one router row per wave in the merged dispatch
         // A compute unit holds three of these workgroups.  The router and shared ones leave well before the ids are
@@ -558,11 +586,13 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
         }
         WD_LAUNCH_CHECK();
     } else if (run_a) {
+        SiteScope site(WD_SITE_FUSED_A, st);
         if (const int rc = launch_a(a, st)) return rc;
     }
     const size_t lds_b = H + (iq ? sizeof(float) * (H / 256) : sizeof(uint16_t) * (H / 32));
     const int grid_b = k * (L->gate_type == WD_TYPE_IQ4_NL ? (F + 15) / 16 : (F + 7) / 8);
     if (run_b && !merged) {
+        SiteScope site(WD_SITE_FUSED_B, st);
         switch (L->gate_type) {
             case WD_TYPE_IQ3_S:
                 if (a.gup_part) k_layer_b<21, true><<<dim3(grid_b), dim3(512), lds_b, st>>>(a);
@@ -598,6 +628,7 @@ int layer_fused(const wd_moe_layer *L, const float *d_x, float *d_out, wd_moe_sc
                                          : al16(L->down, L->down_stride));
     const dim3 grid(grid_c), block(64 * waves_c);
     const bool q8 = L->down_type == WD_TYPE_Q8_0;
+    SiteScope site(WD_SITE_FUSED_C, st);
     if (coal && two) {
         if (waves_c > 9) return fail(WD_ERR_ARG, "fused layer: %d waves in the paired down dispatch (at most 9)", waves_c);
         if (F == 512 && q8) launch_layer_c<0, true, 16, true>(grid, block, lds_c, st, a);
@@ -636,6 +667,7 @@ extern "C" int wd_moe_layer_f32(const wd_moe_layer *L, const float *d_x, float *
                                 unsigned flags, void *stream) {
     if (const int rc = check_layer(L, s, flags)) return rc;
     WD_REQUIRE(d_x && d_out, "MoE layer: null activation or output pointer");
+    SiteScope site(WD_SITE_ROUTED_TOTAL, as_stream(stream));
     return layer_dispatch(L, d_x, d_out, s, flags, nullptr, nullptr, 0.0f, as_stream(stream));
 }
 
@@ -647,6 +679,7 @@ extern "C" int wd_moe_layer_hc_f32(const wd_moe_layer *L, const float *d_x, floa
     WD_REQUIRE(hc >= 1 && hc <= 16, "MoE layer with combine: 1..16 residual streams (got %d)", hc);
     WD_REQUIRE(!(flags & (WD_MOE_ONLY_A | WD_MOE_ONLY_B | WD_MOE_ONLY_C | WD_MOE_DRY)), "MoE layer with combine: measurement flags are not supported");
     const HcSpec spec{d_inject, hc, round_half ? 1 : 0};
+    SiteScope site(WD_SITE_ROUTED_TOTAL, as_stream(stream));
     return layer_dispatch(L, d_x, d_out, s, flags, nullptr, d_residual, 0.0f, as_stream(stream), 0, &spec);
 }
 
@@ -654,6 +687,7 @@ extern "C" int wd_hc_combine_f32(float *d_residual, const float *d_block_out, co
                                  int round_half, void *stream) {
     WD_REQUIRE(d_residual && d_block_out && d_inject, "combine: null pointer");
     WD_REQUIRE(hidden > 0 && hc > 0 && static_cast<long long>(hidden) * hc < (1LL << 31), "combine: bad geometry %d x %d", hc, hidden);
+    SiteScope site(WD_SITE_HC_COMBINE, as_stream(stream));
     k_hc_combine<0><<<dim3((hidden * hc + 255) / 256), dim3(256), 0, as_stream(stream)>>>(d_residual, d_block_out, nullptr, nullptr,
                                                                                           d_inject, hidden, hc, round_half ? 1 : 0);
     WD_LAUNCH_CHECK();
@@ -665,6 +699,7 @@ extern "C" int wd_hc_combine_moe_f32(float *d_residual, const float *d_routed, c
                                      void *stream) {
     WD_REQUIRE(d_residual && d_routed && d_shared && d_shared_gate && d_inject, "combine: null pointer");
     WD_REQUIRE(hidden > 0 && hc > 0 && static_cast<long long>(hidden) * hc < (1LL << 31), "combine: bad geometry %d x %d", hc, hidden);
+    SiteScope site(WD_SITE_HC_COMBINE, as_stream(stream));
     const dim3 grid((hidden * hc + 255) / 256), block(256);
     if (shared_is_half)
         k_hc_combine<2><<<grid, block, 0, as_stream(stream)>>>(d_residual, d_routed, d_shared, d_shared_gate, d_inject, hidden, hc, round_half ? 1 : 0);
@@ -681,6 +716,7 @@ extern "C" int wd_shared_expert_f32(const wd_moe_layer *L, const float *d_x, wd_
     WD_REQUIRE(L->shared_gate_inp && L->shared_gate && L->shared_up && L->shared_down, "shared expert: incomplete weights");
     const int H = L->hidden, F = L->expert_ffn, slot = s->max_k;
     const hipStream_t st = as_stream(stream);
+    SiteScope site(WD_SITE_SHARED, st);
     k_router_gemv<<<dim3(1), dim3(256), 0, st>>>(L->router, d_x, s->logits, 0, H, L->shared_gate_inp, s->shared_gate);
     WD_LAUNCH_CHECK();
     k_sigmoid1<<<dim3(1), dim3(64), 0, st>>>(s->shared_gate);
@@ -751,6 +787,7 @@ int resident_launch(const ResidentArgs &a, wd_moe_scratch *s, hipStream_t st) {
         s->res_fits = (e == hipSuccess && per_cu * s->compute_units >= kResWgs) ? 1 : 0;
     }
     if (!s->res_fits) return -1;  // the workgroups would wait for each other without all being on the device
+    SiteScope site(WD_SITE_STACK_RESIDENT, st);
     if (a.trace)  // (the variant with the time stamps only when they are asked for)
         k_stack_resident<TYPE, true><<<dim3(kResWgs), dim3(kResThreads), kResLdsBytes, st>>>(a);
     else
@@ -807,6 +844,7 @@ extern "C" int wd_moe_stack_f32(const wd_moe_layer *layers, int n_layers, float 
     for (int l = 0; l < n_layers; ++l) {
         if (const int rc = check_layer(&layers[l], s, flags)) return rc;
     }
+    SiteScope site(WD_SITE_STACK_TOTAL, as_stream(stream));
     if (resident_shape(layers, n_layers, s, flags)) {
         const int rc = stack_resident(layers, n_layers, d_x, d_layer_out, s, d_ids_trace, residual_scale, as_stream(stream));
         if (rc >= 0) return rc;
@@ -821,6 +859,7 @@ extern "C" int wd_moe_stack_f32(const wd_moe_layer *layers, int n_layers, float 
             k_fill_u32<<<dim3((n + 255) / 256), dim3(256), 0, as_stream(stream)>>>(s->tagged, kTagInvalid, n);
             WD_LAUNCH_CHECK();
         }
+        SiteScope layer_site(WD_SITE_ROUTED_TOTAL, as_stream(stream));
         if (const int rc = layer_dispatch(&layers[l], d_x, d_layer_out, s, flags, trace, d_x, residual_scale, as_stream(stream), l))
             return rc;
     }
@@ -842,6 +881,7 @@ int tokens_pass(const wd_moe_layer *L, const float *d_x, float *d_out, int token
     }
     hipStream_t st = as_stream(stream);
     const int H = L->hidden, F = L->expert_ffn, k = L->top_k;
+    SiteScope total_site(WD_SITE_TOKENS_TOTAL, st);
     // the union pass over the gate/up tensors needs the IQ types; the multi-token down dispatch needs Q8_0 rows of at
     // most 16 blocks (other down tensors take the one-token dispatch per token, on the activations the union pass left)
     const bool union_path = !(flags & WD_MOE_STAGED) && consumes_q8k(L->gate_type) && tokens * k <= 128 &&
@@ -879,6 +919,7 @@ int tokens_pass(const wd_moe_layer *L, const float *d_x, float *d_out, int token
     a.n_router_wgs = ((a.preselected ? 0 : a.E) + (a.sh_inp ? 1 : 0) + 7) / 8;  // one router row per wave
     const int grid_a = a.n_router_wgs + (a.sh_inp ? (F + 7) / 8 : 0);
     if (grid_a > 0) {  // router, selection and shared gate/up of every token
+        SiteScope site(WD_SITE_TOKENS_A, st);
         k_tokens_a<<<dim3(grid_a, tokens), dim3(512), static_cast<size_t>(H) * 4 + 16, st>>>(ta);
         WD_LAUNCH_CHECK();
     }
@@ -906,12 +947,15 @@ int tokens_pass(const wd_moe_layer *L, const float *d_x, float *d_out, int token
             else k_tokens_b<TYPE_, kMaxTokens><<<gb, bb, lds_b, st>>>(ta);                              \
         }                                                                                               \
     } while (0)
-    if (L->gate_type == WD_TYPE_IQ3_S)
-        WD_TOKENS_B(21);
-    else
-        WD_TOKENS_B(22);
+    {
+        SiteScope site(WD_SITE_TOKENS_B, st);
+        if (L->gate_type == WD_TYPE_IQ3_S)
+            WD_TOKENS_B(21);
+        else
+            WD_TOKENS_B(22);
+        WD_LAUNCH_CHECK();
+    }
 #undef WD_TOKENS_B
-    WD_LAUNCH_CHECK();
     // other down tensors in aligned groups of four 16- or 20-block rows: the same dispatch with the aligned fetch
     auto al16t = [](const void *p_, size_t v) { return reinterpret_cast<uintptr_t>(p_) % 16 == 0 && v % 16 == 0; };
     const bool down_tokens_nb = !down_tokens && (F == 512 || F == 640) && H % 8 == 0 && tokens <= 16 &&
@@ -919,6 +963,7 @@ int tokens_pass(const wd_moe_layer *L, const float *d_x, float *d_out, int token
                                 (down_table ? tables_aligned
                                             : (L->slot_of_expert ? al16t(L->slot_pool, L->slot_bytes) && (L->slot_gate_bytes + L->slot_up_bytes) % 16 == 0
                                                                  : al16t(L->down, L->down_stride)));
+    SiteScope c_site(WD_SITE_TOKENS_C, st);
     if (down_tokens_nb) {
         const size_t per_wave_n = (static_cast<size_t>(F) + F / 16 + 15) & ~static_cast<size_t>(15);
         const size_t lds_n = 16 * per_wave_n + sizeof(float) * 8 * tokens * (k + 1);

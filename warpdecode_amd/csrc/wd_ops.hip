@@ -2,8 +2,11 @@
 // softmax/top-k, low-bit GEMVs (one matrix or one dispatch over several expert matrices)
 // and the elementwise stages.  Each extern "C" entry point mirrors one launcher of the
 // reference operator surface (see include/warpdecode_amd.h for the citations).
+#include <cstring>
+
 #include "wd_common.h"
 #include "wd_fused.cuh"
+#include "wd_profile.hpp"
 
 namespace wd {
 
@@ -407,8 +410,44 @@ int wd_weighted_accum_experts_f32(const float *d_experts, const float *d_weights
 
 int wd_add_shared_f32(float *d_routed, const float *d_shared, const float *d_gate, int n, void *stream) {
     WD_REQUIRE(n > 0 && d_routed && d_shared && d_gate, "add shared: invalid arguments");
+    SiteScope site(WD_SITE_FINISH, as_stream(stream));
     k_add_shared<<<dim3((n + 255) / 256), dim3(256), 0, as_stream(stream)>>>(d_routed, d_shared, d_gate, d_routed, n);
     WD_LAUNCH_CHECK();
+    return WD_OK;
+}
+
+// ---- site profiler -----------------------------------------------------------------------
+int wd_profile_enable(int on) { return SiteProfiler::instance().enable(on != 0); }
+int wd_profile_enabled(void) { return SiteProfiler::instance().enabled() ? 1 : 0; }
+int wd_profile_begin(int site, void *stream) {
+    WD_REQUIRE(site >= 0 && site < WD_PROFILE_SITE_COUNT, "profiler: site %d out of range", site);
+    SiteProfiler::instance().begin(site, as_stream(stream));
+    return WD_OK;
+}
+int wd_profile_end(int site, void *stream) {
+    WD_REQUIRE(site >= 0 && site < WD_PROFILE_SITE_COUNT, "profiler: site %d out of range", site);
+    SiteProfiler::instance().end(site, as_stream(stream));
+    return WD_OK;
+}
+int wd_profile_flush_token(void) { return SiteProfiler::instance().flush_token(); }
+int wd_profile_site(int site, wd_profile_site_stat *out, unsigned long long *tokens) {
+    WD_REQUIRE(site >= 0 && site < WD_PROFILE_SITE_COUNT && out, "profiler: site %d out of range, or a null output", site);
+    *out = SiteProfiler::instance().stat(site);
+    if (tokens) *tokens = SiteProfiler::instance().tokens();
+    return WD_OK;
+}
+const char *wd_profile_site_name(int site) { return profile_site_name(site); }
+size_t wd_profile_report(char *buf, size_t cap) {
+    const std::string r = SiteProfiler::instance().report();
+    if (buf && cap) {
+        const size_t n = r.size() < cap - 1 ? r.size() : cap - 1;
+        std::memcpy(buf, r.data(), n);
+        buf[n] = 0;
+    }
+    return r.size();
+}
+int wd_profile_reset(void) {
+    SiteProfiler::instance().reset();
     return WD_OK;
 }
 

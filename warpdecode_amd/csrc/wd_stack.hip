@@ -19,6 +19,7 @@ extern "C" int wd_moe_stack_cached_f32(const wd_moe_layer *layers, int n_layers,
     WD_REQUIRE((h_ids_trace == nullptr) == (d_ids_trace == nullptr), "cached MoE stack: the routing trace needs its host and device copy");
     WD_REQUIRE(!(flags & (WD_MOE_ONLY_A | WD_MOE_ONLY_B | WD_MOE_ONLY_C | WD_MOE_STAGED)), "cached MoE stack: unsupported flags");
     const hipStream_t st = as_stream(stream);
+    SiteScope total_site(WD_SITE_STACK_TOTAL, st);
     auto bind = [&](int l) {
         wd_moe_layer L = layers[l];
         L.slot_of_expert = cache->d_table + static_cast<size_t>(l) * cache->n_experts;
@@ -73,11 +74,19 @@ extern "C" int wd_moe_stack_cached_f32(const wd_moe_layer *layers, int n_layers,
         const wd_moe_layer L = bind(l);
         // dispatch A also carries the shared expert's gate/up rows and its gate: it runs whenever there is something in it
         // (with ids given by the caller it leaves the router rows out)
-        if (!(flags & WD_MOE_PRESELECTED) || L.shared_gate_inp) {
-            if (const int rc = layer_fused(&L, d_x, d_layer_out, s, flags | WD_MOE_ONLY_A, nullptr, d_x, residual_scale, st)) return rc;
+        SiteScope layer_site(WD_SITE_ROUTED_TOTAL, st);
+        {   // the reference's router_select bracket: router and selection, ids to the host, the synchronisation that closes it
+            SiteScope select_site(WD_SITE_ROUTER, st);
+            if (!(flags & WD_MOE_PRESELECTED) || L.shared_gate_inp) {
+                if (const int rc = layer_fused(&L, d_x, d_layer_out, s, flags | WD_MOE_ONLY_A, nullptr, d_x, residual_scale, st)) return rc;
+            }
+            {
+                SiteScope d2h_site(WD_SITE_ROUTER_D2H, st);
+                WD_HIP(hipMemcpyAsync(s->h_ids, s->ids, sizeof(int32_t) * L.top_k, hipMemcpyDeviceToHost, st));
+            }
+            SiteScope sync_site(WD_SITE_ROUTER_SYNC, st);
+            WD_HIP(hipStreamSynchronize(st));
         }
-        WD_HIP(hipMemcpyAsync(s->h_ids, s->ids, sizeof(int32_t) * L.top_k, hipMemcpyDeviceToHost, st));
-        WD_HIP(hipStreamSynchronize(st));
         if (const int rc = wd_expert_cache_acquire(cache, l, s->h_ids, L.top_k, nullptr, stream)) return rc;
         if (const int rc = layer_fused(&L, d_x, d_layer_out, s, flags | WD_MOE_ONLY_B | WD_MOE_ONLY_C, nullptr, d_x, residual_scale, st))
             return rc;

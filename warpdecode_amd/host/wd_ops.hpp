@@ -11,6 +11,7 @@
 
 #include <algorithm>
 #include <cstdint>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <memory>
@@ -565,6 +566,109 @@ inline int default_expert_prefetch_depth(size_t vram_bytes) {
     return mib >= 120 * 1024 ? 3 : (mib >= 40 * 1024 ? 2 : 1);
 }
 
+// Site profiler (src/qwen38_moe.cuh:296-535): the reference's site numbers, its process-wide profiler object and its
+// scope bracket, over the library's profiler.  As there, WARODECODE_MOE_PROFILE=1 switches it on when the object is
+// first used and the summary goes to stderr when the process ends; the library brackets its own dispatches while it
+// is on (the sites beyond kQ38MoeSiteCount), a caller brackets the regions of its own code with Q38MoeKernelScope and
+// calls flush_token() once per token after its stream synchronisation.
+enum Q38MoeSite : int {
+    kQ38MoeSiteStageTotal = WD_SITE_STAGE_TOTAL,
+    kQ38MoeSiteRoutedTotal = WD_SITE_ROUTED_TOTAL,
+    kQ38MoeSiteRouter = WD_SITE_ROUTER,
+    kQ38MoeSiteRouterQuant = WD_SITE_ROUTER_QUANT,
+    kQ38MoeSiteRouterGemv = WD_SITE_ROUTER_GEMV,
+    kQ38MoeSiteRouterTopk = WD_SITE_ROUTER_TOPK,
+    kQ38MoeSiteRouterD2h = WD_SITE_ROUTER_D2H,
+    kQ38MoeSiteRouterSync = WD_SITE_ROUTER_SYNC,
+    kQ38MoeSiteAccumZero = WD_SITE_ACCUM_ZERO,
+    kQ38MoeSiteRxQuant = WD_SITE_RX_QUANT,
+    kQ38MoeSiteAcquire = WD_SITE_ACQUIRE,
+    kQ38MoeSitePtrH2d = WD_SITE_PTR_H2D,
+    kQ38MoeSiteBatchTotal = WD_SITE_BATCH_TOTAL,
+    kQ38MoeSiteGateUpGemv = WD_SITE_GATE_UP_GEMV,
+    kQ38MoeSiteSilu = WD_SITE_SILU,
+    kQ38MoeSiteQ8Quant = WD_SITE_Q8_QUANT,
+    kQ38MoeSiteDownGemv = WD_SITE_DOWN_GEMV,
+    kQ38MoeSiteAccum = WD_SITE_ACCUM,
+    kQ38MoeSiteCapture = WD_SITE_CAPTURE,
+    kQ38MoeSiteLoopTotal = WD_SITE_LOOP_TOTAL,
+    kQ38MoeSiteFinish = WD_SITE_FINISH,
+    kQ38MoeSiteShared = WD_SITE_SHARED,
+    kQ38MoeSiteSharedGate = WD_SITE_SHARED_GATE,
+    kQ38MoeSiteMirror = WD_SITE_MIRROR,
+    kQ38MoeSiteCount = WD_PROFILE_FIRST_OWN_SITE
+};
+inline const char *q38_moe_site_name(int site) { return wd_profile_site_name(site); }
+
+struct Q38MoeSiteStat {
+    unsigned long long calls = 0;
+    double total_ms = 0.0;
+    double total_host_ms = 0.0;
+    unsigned long long overflow = 0;
+    unsigned long long elapsed_fail = 0;
+    unsigned long long recorded = 0;
+};
+
+class Q38MoeKernelProfiler {
+public:
+    static Q38MoeKernelProfiler &instance() {
+        static Q38MoeKernelProfiler profiler;
+        return profiler;
+    }
+    bool enabled() const { return wd_profile_enabled() != 0; }
+    void mark_begin(int site, Stream stream) {
+        if (site >= 0 && site < WD_PROFILE_SITE_COUNT) (void)wd_profile_begin(site, stream);
+    }
+    void mark_end(int site, Stream stream) {
+        if (site >= 0 && site < WD_PROFILE_SITE_COUNT) (void)wd_profile_end(site, stream);
+    }
+    void flush_token() { check(wd_profile_flush_token(), "profiler flush"); }
+    Q38MoeSiteStat site(int site_index) const {
+        wd_profile_site_stat raw{};
+        check(wd_profile_site(site_index, &raw, nullptr), "profiler site");
+        Q38MoeSiteStat out;
+        out.calls = raw.calls, out.total_ms = raw.device_ms, out.total_host_ms = raw.host_ms;
+        out.overflow = raw.dropped, out.elapsed_fail = raw.unreadable, out.recorded = raw.recorded;
+        return out;
+    }
+    std::string summary() const {
+        std::string text(wd_profile_report(nullptr, 0), '\0');
+        if (!text.empty()) wd_profile_report(&text[0], text.size() + 1);
+        return text;
+    }
+    void print_summary() const {
+        if (!enabled()) return;
+        wd_profile_site_stat raw{};
+        unsigned long long tokens = 0;
+        if (wd_profile_site(0, &raw, &tokens) != WD_OK || tokens == 0) return;
+        std::fputs(summary().c_str(), stderr);
+    }
+
+private:
+    Q38MoeKernelProfiler() {
+        const char *v = std::getenv("WARODECODE_MOE_PROFILE");
+        if (v != nullptr && v[0] != '\0' && v[0] != '0') (void)wd_profile_enable(1);
+    }
+    ~Q38MoeKernelProfiler() { print_summary(); }
+    Q38MoeKernelProfiler(const Q38MoeKernelProfiler &) = delete;
+    Q38MoeKernelProfiler &operator=(const Q38MoeKernelProfiler &) = delete;
+};
+
+// RAII bracket for one region of a MoE layer.
+class Q38MoeKernelScope {
+public:
+    Q38MoeKernelScope(int site, Stream stream) : site_(site), stream_(stream) {
+        Q38MoeKernelProfiler::instance().mark_begin(site_, stream_);
+    }
+    ~Q38MoeKernelScope() { Q38MoeKernelProfiler::instance().mark_end(site_, stream_); }
+    Q38MoeKernelScope(const Q38MoeKernelScope &) = delete;
+    Q38MoeKernelScope &operator=(const Q38MoeKernelScope &) = delete;
+
+private:
+    int site_;
+    Stream stream_;
+};
+
 // src/qwen38_moe.cuh:247-263
 inline void launch_q38_router_gemv_f32(const GpuMatrix &w, const float *x, float *y, Stream stream, int threads = 256) {
     if (!matrix_has_f32_weights(w)) throw std::runtime_error("router F32 warp GEMV requires an F32 dense matrix");
@@ -694,10 +798,17 @@ inline void fill_routed(wd_moe_layer &L, int layer, const GpuMatrix &router, con
 inline void routed_through_host(const wd_moe_layer &L, int layer, const float *x, const TensorInfo &gate, const TensorInfo &up,
                                 const TensorInfo &down, GpuExpertCache &cache, Qwen38MoeScratch &scratch, float *dst, bool run_a,
                                 Stream stream, unsigned extra_flags = 0u) {
-    if (run_a) check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), WD_MOE_ONLY_A, stream), "MoE router failed");
-    check(wd_memcpy_d2h(scratch.h_ids(), scratch.d_ids(), sizeof(int) * L.top_k, stream), "routed ids copy failed");
-    scratch.queue_status_copy(stream);
-    check(wd_stream_sync(stream), "stream synchronisation failed");
+    {   // the reference's brackets of this stretch (src/qwen38_moe.cuh:2323-2380): selection, ids to the host, the wait
+        Q38MoeKernelScope select_scope(kQ38MoeSiteRouter, stream);
+        if (run_a) check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), WD_MOE_ONLY_A, stream), "MoE router failed");
+        {
+            Q38MoeKernelScope d2h_scope(kQ38MoeSiteRouterD2h, stream);
+            check(wd_memcpy_d2h(scratch.h_ids(), scratch.d_ids(), sizeof(int) * L.top_k, stream), "routed ids copy failed");
+            scratch.queue_status_copy(stream);
+        }
+        Q38MoeKernelScope sync_scope(kQ38MoeSiteRouterSync, stream);
+        check(wd_stream_sync(stream), "stream synchronisation failed");
+    }
     scratch.throw_if_failed();
     cache.register_layer_experts(layer, gate, up, down);
     cache.acquire_ids(layer, scratch.h_ids(), L.top_k, stream);
@@ -717,6 +828,7 @@ inline void run_qwen38_routed_moe_separate_f32_x(int layer, const float *x, cons
     detail::fill_routed(L, layer, router, gate_exps, up_exps, down_exps, cache, scratch, expert_scale);
     float *dst = out ? out : scratch.moe_out_f32();
     const unsigned keep = keep_expert_outputs ? WD_MOE_KEEP_EXPERT_OUT : 0u;  // scratch.rx_batch_down(): [k][hidden]
+    Q38MoeKernelScope routed_scope(kQ38MoeSiteRoutedTotal, stream);  // (the library's own brackets of this site nest inside)
     if (cache.layer_resident(layer)) {
         check(wd_moe_layer_f32(&L, x, dst, scratch.handle(), (preselected ? WD_MOE_PRESELECTED : 0u) | keep, stream), "MoE layer failed");
         return;
@@ -825,6 +937,7 @@ inline void run_qwen38_shared_expert_f32_x(const float *x, const Qwen38SharedExp
 // out = routed weighted sum + shared expert * gate (src/qwen38_moe.cuh:2442-2453)
 inline void q38_finish_moe_f32(Qwen38MoeScratch &scratch, float *out, Stream stream) {
     if (out == scratch.d_accum()) throw std::runtime_error("F32 MoE output must not alias the routed accumulation buffer");
+    Q38MoeKernelScope finish_scope(kQ38MoeSiteFinish, stream);
     check(wd_memcpy_d2d(out, scratch.d_accum(), sizeof(float) * scratch.hidden(), stream), "routed sum copy failed");
     q38_moe_add_shared_f32(out, scratch.down_f32(), scratch.d_shared_gate(), scratch.hidden(), stream);
 }
