@@ -71,7 +71,7 @@ public:
         if (l.depth++ != 0) return;  // a nested bracket of the same site stays one interval
         l.host_begin = std::chrono::steady_clock::now();
         l.armed = false;
-        if (l.written >= kCap || capturing(st) || hipEventRecord(start_[index(site, l.written)], st) != hipSuccess) {
+        if (l.written >= kCap || capturing(st) || !record(start_[index(site, l.written)], st)) {
             ++l.dropped;
             return;
         }
@@ -86,7 +86,7 @@ public:
         l.host_ms += std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - l.host_begin).count();
         if (!l.armed) return;  // counted as dropped when it began
         l.armed = false;
-        if (capturing(st) || hipEventRecord(stop_[index(site, l.written)], st) != hipSuccess) {
+        if (capturing(st) || !record(stop_[index(site, l.written)], st)) {
             ++l.dropped;
             return;
         }
@@ -166,7 +166,16 @@ private:
     static size_t index(int site, int slot) { return static_cast<size_t>(site) * kCap + static_cast<size_t>(slot); }
     static bool capturing(hipStream_t st) {
         hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-        return hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &cs) != hipSuccess) {
+            (void)hipGetLastError();  // (the legacy stream while another stream captures): not the caller's next launch's error
+            return true;
+        }
+        return cs != hipStreamCaptureStatusNone;
+    }
+    static bool record(hipEvent_t ev, hipStream_t st) {
+        if (hipEventRecord(ev, st) == hipSuccess) return true;
+        (void)hipGetLastError();
+        return false;
     }
     void release_events() {
         for (hipEvent_t e : start_)
