@@ -956,9 +956,9 @@ int tokens_pass(const wd_moe_layer *L, const float *d_x, float *d_out, int token
         WD_LAUNCH_CHECK();
     }
 #undef WD_TOKENS_B
-    // other down tensors in aligned groups of four 16- or 20-block rows: the same dispatch with the aligned fetch
+    // down tensors in aligned groups of four 16- or 20-block rows (either type): the dispatch with the aligned fetch
     auto al16t = [](const void *p_, size_t v) { return reinterpret_cast<uintptr_t>(p_) % 16 == 0 && v % 16 == 0; };
-    const bool down_tokens_nb = !down_tokens && (F == 512 || F == 640) && H % 8 == 0 && tokens <= 16 &&
+    const bool down_tokens_nb = (F == 512 || F == 640) && H % 8 == 0 && tokens <= 16 &&
                                 (!L->shared_down || al16t(L->shared_down, 0)) &&
                                 (down_table ? tables_aligned
                                             : (L->slot_of_expert ? al16t(L->slot_pool, L->slot_bytes) && (L->slot_gate_bytes + L->slot_up_bytes) % 16 == 0
@@ -970,6 +970,7 @@ int tokens_pass(const wd_moe_layer *L, const float *d_x, float *d_out, int token
         const dim3 grid(H / 8), block(1024);
         const bool q8 = L->down_type == WD_TYPE_Q8_0;
         if (F == 512 && !q8) k_tokens_c_nb<1, 16><<<grid, block, lds_n, st>>>(ta);
+        else if (F == 512) k_tokens_c_nb<0, 16><<<grid, block, lds_n, st>>>(ta);
         else if (q8) k_tokens_c_nb<0, 20><<<grid, block, lds_n, st>>>(ta);
         else k_tokens_c_nb<1, 20><<<grid, block, lds_n, st>>>(ta);
         WD_LAUNCH_CHECK();

@@ -527,8 +527,8 @@ __global__ __launch_bounds__(1024) void k_tokens_c(TokenArgs ta) {
     mark(a, 2, 6);
 }
 
-// The same for down tensors that k_tokens_c does not take: IQ4_NL (KIND 1) or Q8_0 (KIND 0) rows of NB = 16 or 20 blocks
-// in 16-byte aligned groups of four, fetched as aligned words (q8_rows4_coal).  Eight rows per workgroup, 16 waves, an
+// The same for IQ4_NL (KIND 1) or Q8_0 (KIND 0) rows of NB = 16 or 20 blocks in 16-byte aligned groups of four, fetched as
+// aligned words (q8_rows4_coal): preferred over k_tokens_c where both apply (aligned Q8_0 rows of 16 blocks).  Eight rows per workgroup, 16 waves, an
 // item is (token, matrix) with the shared expert (always Q8_0) as matrix k; a wave has the two row groups of two items
 // in flight.  dynamic LDS per wave: F bytes + F/32 halves (+ pad), then [T][k+1][8] floats.
 template <int KIND, int NB>
