@@ -917,10 +917,10 @@ int tokens_pass(const wd_moe_layer *L, const float *d_x, float *d_out, int token
     }
     LayerArgs &a = ta.common;
     a.n_router_wgs = ((a.preselected ? 0 : a.E) + (a.sh_inp ? 1 : 0) + 7) / 8;  // one router row per wave
-    const int grid_a = a.n_router_wgs + (a.sh_inp ? (F + 7) / 8 : 0);
+    const int grid_a = tokens_a_grid(a.n_router_wgs, a.sh_inp ? (F + 7) / 8 : 0).total(tokens);
     if (grid_a > 0) {  // router, selection and shared gate/up of every token
         SiteScope site(WD_SITE_TOKENS_A, st);
-        k_tokens_a<<<dim3(grid_a, tokens), dim3(512), static_cast<size_t>(H) * 4 + 16, st>>>(ta);
+        k_tokens_a<<<dim3(grid_a), dim3(512), static_cast<size_t>(H) * 4 + 16, st>>>(ta);
         WD_LAUNCH_CHECK();
     }
     const size_t lds_b = static_cast<size_t>(tokens) * (H + sizeof(float) * (H / 256));

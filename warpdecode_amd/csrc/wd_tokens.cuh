@@ -45,17 +45,42 @@ struct TokenArgs {
 };
 
 // ---- dispatch A for T tokens ----------------------------------------------------------------------------
-// grid = (n_router_wgs + ceil(F / 8), T), 512 threads; blockIdx.y is the token.  Per token this is the front of the
+// grid = T * (router_stride + shared_stride), 512 threads, the strides being the router and the shared workgroups of a
+// token rounded up to a multiple of 8 (tokens_a_grid): first the router workgroups of every token, token by token, then
+// the shared ones.  The router workgroups are on the pass's critical path and start first; and workgroup w of every
+// token - the same weight rows - lands on the same XCD (workgroups go to the eight XCDs in turn), so its L2 serves the
+// rows to the tokens after the first.  The padding workgroups return at once.  Per token this is the front of the
 // one-token merged dispatch: router rows one per wave, the last router workgroup of the token selects its experts
 // with the whole workgroup, the other workgroups run the shared expert's gate/up.
 // dynamic LDS: 4 * H bytes (x as f32 for the router rows; the shared workgroups use H + H/16 of it).
+struct TokensAGrid {
+    int router_stride, shared_stride;
+    __host__ __device__ int total(int tokens) const { return tokens * (router_stride + shared_stride); }
+};
+__host__ __device__ inline TokensAGrid tokens_a_grid(int n_router_wgs, int n_shared_wgs) {
+    return TokensAGrid{(n_router_wgs + 7) & ~7, (n_shared_wgs + 7) & ~7};
+}
 __global__ __launch_bounds__(512, 4) void k_tokens_a(TokenArgs ta) {
     extern __shared__ __align__(16) uint8_t lds_ta[];
     __shared__ __align__(16) uint8_t s_work[sizeof(Q8RowTile) * 8];
     __shared__ int s_last;
     const LayerArgs &a = ta.common;
-    const TokenSlots &s = ta.tok[blockIdx.y];
-    const int wg = blockIdx.x;
+    const int n_shared_wgs = a.sh_inp ? (a.F + 7) / 8 : 0;
+    const TokensAGrid gr = tokens_a_grid(a.n_router_wgs, n_shared_wgs);
+    int token, wg;
+    {
+        const int b = blockIdx.x, router_part = ta.T * gr.router_stride;
+        if (b < router_part) {
+            token = b / gr.router_stride, wg = b - token * gr.router_stride;
+            if (wg >= a.n_router_wgs) return;
+        } else {
+            token = (b - router_part) / gr.shared_stride;
+            const int w = b - router_part - token * gr.shared_stride;
+            if (w >= n_shared_wgs) return;
+            wg = a.n_router_wgs + w;
+        }
+    }
+    const TokenSlots &s = ta.tok[token];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     if (wg < a.n_router_wgs) {
         router_rows_wave<true, true>(a.router, s.x, reinterpret_cast<float *>(lds_ta), s.logits, a.preselected ? 0 : a.E, a.H,
