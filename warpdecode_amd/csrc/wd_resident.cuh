@@ -67,8 +67,12 @@ struct ResidentViews {
 };
 
 // Byte offsets inside the hand-off block.
-constexpr unsigned kHandRec = 0;          // [layers][512] records of 128 bytes, one per (layer, workgroup): word 0 the router
-constexpr unsigned kRecBytes = 128;       //   logit of row r, word 1 the shared expert's gate logit (workgroup 1 only)
+constexpr unsigned kHandRec = 0;          // [layers][512] records of kRecBytes, one per (layer, workgroup): word 0 the router
+// (Measured on one box: records of 128 / 64 / 32 / 16 bytes 0.869 / 0.861 / 0.856 / 0.851 ms per token - workgroup 0 polls
+// 64 lines instead of 512; the gate logit moved into the line of the router weights, which every workgroup polls, costs
+// 1.2 % again, and records of 8 bytes are no better than 16.)
+constexpr unsigned kRecBytes = 16;        //   logit of row r, word 1 the shared expert's gate logit (workgroup 1 only)
+static_assert(kRecBytes % 16 == 0 && kRecBytes <= 128, "records are reset in 16-byte pieces by eight lanes");
 // What every workgroup needs from every other - four values of the next input, eleven activations - is written by its
 // producer into kResCopies copies, one per group of workgroups (r % kResCopies; on this device the workgroups of a group
 // share an L2), laid out contiguously: the consumers of a group fetch their copy with coalesced requests, and a line is
@@ -726,10 +730,10 @@ WD_DEV void res_router_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         }
         for (int ll = l; ll < kResMaxLayers; ll += a.n_layers) {
             const uint4 empty4 = make_uint4(kResEmpty, kResEmpty, kResEmpty, kResEmpty);
-            // 8 lanes the workgroup's record, 8 its 128 bytes of the layer's input copies, 24 its 384 bytes of the activations'
+            // lane 0 the workgroup's record (of the first 8 lanes), 8 lanes its 128 bytes of the layer's input copies, 24 its 384 bytes of the activations'
             const unsigned off = lane < 8 ? rec_off(ll, r) + 16u * lane
                                : lane < 16 ? xc_off(ll, 0) + kXcStride * (8 * r + lane - 8) : ac_off(ll, 0) + 16u * (24 * r + lane - 16);
-            if (lane < 40) hand_store16(ob, off, empty4);
+            if (lane < 8 ? lane < static_cast<int>(kRecBytes / 16) : lane < 40) hand_store16(ob, off, empty4);
             if (r == 0) {
                 hand_store16(ob, kHandIdh + static_cast<unsigned>(ll * kResIdCopies * 64 + 16 * lane), empty4);
                 if (lane < 4) hand_store16(ob, kHandWh + static_cast<unsigned>(ll * 64 + 16 * lane), empty4);
