@@ -445,11 +445,16 @@ WD_DEV void topk_block_step3(int n, int k, float w_scale, int32_t *ids, float *w
     const bool good = lane >= k || (have && top_e >= 0x1p-100f && top_e > below);
     const bool all_good = __builtin_amdgcn_ballot_w64(good) == ~0ull;
     int id_mine = override_ids ? id_given : idc;
-    if (all_good && tagged && lane < k) {
+    if (all_good && tagged) {
+        // the ids (lanes 0..k-1, k <= 16) into every row of 16 lanes, then four replicas per store instruction: the last
+        // replica goes out a quarter of the stores after the first
+        const wd_uint2v t16 = __builtin_amdgcn_permlane16_swap(static_cast<uint32_t>(id_mine), static_cast<uint32_t>(id_mine), false, false);
+        const wd_uint2v t32 = __builtin_amdgcn_permlane32_swap(t16.x, t16.x, false, false);
+        const int j = lane & 15, c4 = lane >> 4;
 #pragma unroll 4
-        for (int c = 0; c < copies; ++c)
-            __hip_atomic_store(tagged + c * 16 + lane, static_cast<uint32_t>(id_mine), __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
+        for (int c0 = 0; c0 < copies; c0 += 4)
+            if (j < k && c0 + c4 < copies)
+                __hip_atomic_store(tagged + (c0 + c4) * 16 + j, t32.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     WD_STAMP(6);
 
