@@ -20,9 +20,11 @@
 // Hand-off buffers.  Every layer of a launch has its own copy of each buffer, so no word is written twice during a
 // launch.  A word holds kResEmpty (0xffffffff) until its producer stores the value; consumers poll the data words
 // themselves with device-scope loads, so no flag, counter or ordering between stores is needed.  What a workgroup
-// hands on in a layer - its logit, its eleven activations, its four values of the next input - lies in a record of
-// its own, one 128-byte line per (layer, workgroup): a line that several compute units write piece by piece while
-// the whole grid polls it changes hands once per write, and thirty-two writers per line made a hand-off take 17 us.  (An f32 result with
+// hands on in a layer: its logit, in a 16-byte record that only workgroup 0 polls (64 lines for the 512 logits); its
+// eleven activations (48 bytes) and its four values of the next input (16 bytes), pushed into eight contiguous
+// copies, one per group of workgroups, each of which polls its own.  A line that many compute units write piece
+// by piece while the whole grid polls it changes hands once per write: thirty-two writers per line made a hand-off
+// take 17 us, hence pieces of 16 bytes or more.  (An f32 result with
 // that very bit pattern - a NaN that no arithmetic here produces by itself - would be taken for "not yet" and end in
 // a timeout.)  There are two sets of these buffers: a launch works in one and resets the other as it goes (the router
 // waves, which have time to spare), so nothing has to be cleaned up when a launch ends.  Waits are bounded: a wait that runs out sets status[0], after which
