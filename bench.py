@@ -934,17 +934,39 @@ def main():
             fn()
         return g
 
+    def first_token(flags, n_layers=NL):
+        """x and out (host copies) of token 0 through the first n_layers layers by the given form of the stack."""
+        d_x.copy_(d_xs[0])
+        d_trace.copy_(d_trace_all[0])
+        capi.call("wd_moe_stack_f32", layers, n_layers, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()), scratch,
+                  trace_ptr, RESIDUAL_SCALE, flags, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        return d_x.cpu().numpy().copy(), d_out.cpu().numpy().copy()
+
+    # The launch that is timed, against the other form of the stack on the same token: all layers at full width, bit for bit.
+    got, alt = first_token(stack_flags), first_token(stack_flags ^ PER_LAYER)
+    forms_agree = all(np.array_equal(a.view(np.uint32), b.view(np.uint32)) for a, b in zip(got, alt))
+    note("token 0 through %d layers: resident launch and per-layer dispatches bit-identical: %s" % (NL, forms_agree))
+    if not forms_agree:
+        print("bench.py: the two forms of the stack disagree on token 0", file=sys.stderr)
+        sys.exit(1)
+    oracle_checked = None
     if args.check:
+        # the measured form of the stack on layer 0 alone against the CPU oracle (ids from the trace, the router's weights)
         from oracle import pyoracle
         L0 = layer_dict(torch, synth, keep[0], E)
-        want, _ = pyoracle.moe_layer(L0, xs[0])
-        o = torch.zeros(H, dtype=torch.float32, device="cuda")
-        capi.call("wd_moe_layer_f32", C.byref(layers[0]), C.c_void_p(d_xs[0].data_ptr()), C.c_void_p(o.data_ptr()),
-                  scratch, 0, C.c_void_p(torch.cuda.current_stream().cuda_stream))
-        torch.cuda.synchronize()
-        same = np.array_equal(o.cpu().numpy().view(np.uint32), want.view(np.uint32))
-        print("check: layer 0 output bit-identical to the CPU oracle: %s" % same, file=sys.stderr)
-        if not same:
+        if trace_ptr is None:
+            want, _ = pyoracle.moe_layer(L0, xs[0])
+        else:
+            _, wts = pyoracle.route(pyoracle.router_logits(L0["router"], xs[0]), k)
+            want, _ = pyoracle.moe_layer(L0, xs[0], ids=trace[0][0], weights=wts)
+        want_x = (xs[0] + (want * np.float32(RESIDUAL_SCALE)).astype(np.float32)).astype(np.float32)
+        got_x, got_out = first_token(stack_flags, 1)
+        oracle_checked = bool(np.array_equal(got_out.view(np.uint32), want.view(np.uint32)) and
+                              np.array_equal(got_x.view(np.uint32), want_x.view(np.uint32)))
+        print("check: layer 0 through the measured form of the stack bit-identical to the CPU oracle: %s" % oracle_checked,
+              file=sys.stderr)
+        if not oracle_checked:
             sys.exit(1)
 
     note("inputs and routing trace ready")
@@ -1115,7 +1137,8 @@ def main():
                    "path": "one resident launch per step" if args.path == "resident" else "two dispatches per layer",
                    "spread_ms_per_step": spread,
                    "bytes_per_token": bytes_per_step, "wall_s": round(wall, 3), "finite": finite,
-                   "in_dispatch_waits_ok": waits_ok},
+                   "in_dispatch_waits_ok": waits_ok, "forms_bit_identical_on_token_0": forms_agree,
+                   "layer_0_equals_cpu_oracle": oracle_checked},
         "roofline": roofline,
     }
     if site_profile is not None:

@@ -185,20 +185,21 @@ def _run_stack(g, arr, n, x, tr, sc, flags):
     return g.host(dx), g.host(out), views
 
 
-@pytest.mark.parametrize("gate_type,experts,k,shared", [(synth.IQ3_S, 64, 10, True), (synth.IQ2_S, 40, 6, True),
-                                                        (synth.IQ3_S, 128, 9, False)],
-                         ids=["iq3s-64x10-shared", "iq2s-40x6-shared", "iq3s-128x9"])
-def test_one_launch_stack_matches_per_layer_and_oracle(g, oracle, gate_type, experts, k, shared):
+# The last case is the shape the benchmark measures: 512 experts (every workgroup owns a router row, all eight selecting
+# waves of workgroup 0 hold live logits, the poll of the logit records is full), top-10, a shared expert.
+@pytest.mark.parametrize("gate_type,experts,k,shared,nl", [(synth.IQ3_S, 64, 10, True, 5), (synth.IQ2_S, 40, 6, True, 5),
+                                                           (synth.IQ3_S, 128, 9, False, 5), (synth.IQ3_S, 512, 10, True, 3)],
+                         ids=["iq3s-64x10-shared", "iq2s-40x6-shared", "iq3s-128x9", "iq3s-512x10-shared"])
+def test_one_launch_stack_matches_per_layer_and_oracle(g, oracle, gate_type, experts, k, shared, nl):
     """The resident launch against the per-layer dispatches (every output and every view of the last layer, bit for
     bit) over launches in a row with stacks of different depth, with and without a routing trace; the first token
-    also against the oracle applied layer by layer."""
-    nl = 5
+    (router-selected ids) and the second (ids from a trace) also against the oracle applied layer by layer."""
     Ls = [synth.make_layer(2048, 512, experts, k, gate_type, synth.Q8_0, shared=shared, layer=300 + l,
                            router_sigma=1.0 / np.sqrt(2048.0)) for l in range(nl)]
     dls, arr = _descs(g, Ls)
     sc_a, sc_b = g.Scratch(2048, 512, experts, k), g.Scratch(2048, 512, experts, k)
     rng = np.random.default_rng(SEED + 400)
-    for token, depth in enumerate([nl, 2, nl, nl, 3, nl]):
+    for token, depth in enumerate([nl, 2, nl, nl, min(3, nl), nl]):
         x = synth.rms_normed(synth.rng_for(SEED, 84, token), 2048)
         tr = None
         if token % 2 == 1:
@@ -210,12 +211,16 @@ def test_one_launch_stack_matches_per_layer_and_oracle(g, oracle, gate_type, exp
             if name in ("down_f32", "shared_gate") and not shared:
                 continue
             assert np.array_equal(got[2][name].view(np.uint32), want[2][name].view(np.uint32)), (token, name)
-        if token == 0:
+        if token < 2:
             wx = x.copy()
-            for L in Ls:
-                wout, _ = oracle.moe_layer(L, wx)
+            for l, L in enumerate(Ls[:depth]):
+                if tr is None:
+                    wout, _ = oracle.moe_layer(L, wx)
+                else:
+                    _, wts = oracle.route(oracle.router_logits(L["router"], wx), k)
+                    wout, _ = oracle.moe_layer(L, wx, ids=tr[l], weights=wts)
                 wx = (wx + (wout * np.float32(2.0 ** -12)).astype(np.float32)).astype(np.float32)
-            assert g.same_bits(got[0], wx) and g.same_bits(got[1], wout)
+            assert g.same_bits(got[0], wx) and g.same_bits(got[1], wout), token
     assert capi.load().wd_moe_scratch_status(sc_a.h) == 0
     sc_a.close()
     sc_b.close()
