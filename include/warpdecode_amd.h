@@ -220,10 +220,6 @@ unsigned long long *wd_moe_scratch_trace(wd_moe_scratch *s, int wg);
  * LDS, 3 logits seen / logit stored, 4 id seen, 5 activation stored, 6 activations seen, 7 down rows done, 8/9 begin
  * and end of the combine).  wg == -1: uint64 [512][4][16], waves 0, 9, 10 and 11 of every workgroup. */
 unsigned long long *wd_moe_scratch_trace_resident(wd_moe_scratch *s, int wg, int layer);
-/* Measurement aid for the same launch, in the spirit of WD_MOE_DRY: leaves parts of it out so that what remains can be
- * timed - 1 the gate/up decode and dots, 2 the routed weight loads, 4 the wait for the activations, 8 the down dots
- * (a bit mask; 0 restores the whole launch).  The results of a launch with a non-zero mask are not valid. */
-int wd_moe_scratch_omit_resident(wd_moe_scratch *s, int mask);
 
 /* flags for wd_moe_layer_f32 */
 #define WD_MOE_PRESELECTED 1u      /* ids/weights already in scratch: skip the router (reference `preselected`) */

@@ -227,24 +227,87 @@ def test_one_launch_stack_matches_per_layer_and_oracle(g, oracle, gate_type, exp
 
 
 def test_one_launch_stack_wait_that_runs_out(g):
-    """A wait limit of one poll: the launch ends normally with the status word set, later launches return at once
-    until the scratch is reset, and after the reset the results are right again."""
+    """A wait limit of one poll: the launch ends normally with the status word set and NaN in its outputs; the next call
+    on that scratch is refused by the host (the status word has a mirror in host memory), a replay of a graph recorded
+    earlier returns NaN at once; after the reset the results are right again."""
+    import torch
     Ls = [synth.make_c2(layer=320 + l, n_experts=64) for l in range(3)]
     dls, arr = _descs(g, Ls)
     sc, ref = g.Scratch(2048, 512, 64, 10), g.Scratch(2048, 512, 64, 10)
     x = synth.rms_normed(synth.rng_for(SEED, 85), 2048)
     want = _run_stack(g, arr, 3, x, None, ref, PER_LAYER)
+    # a graph of the launch, recorded while all is well
+    d_x, d_out = g.dev(x), g.empty(2048, np.float32)
+
+    def launch():
+        capi.call("wd_moe_stack_f32", arr, 3, g.ptr(d_x), g.ptr(d_out), sc.h, None, float(2.0 ** -12), 0,
+                  C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    assert g.same_bits(g.host(d_x), want[0])
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        launch()
     capi.call("wd_moe_scratch_set_wait_limit", sc.h, 1)
     bad = _run_stack(g, arr, 3, x, None, sc, 0)
     assert capi.load().wd_moe_scratch_status(sc.h) == 1
     assert np.isnan(bad[0]).all() and np.isnan(bad[1]).all()   # the failure is in the data too
-    bad = _run_stack(g, arr, 3, x, None, sc, 0)      # refused on the device: nothing waits
+    dx, out = g.dev(x), g.empty(2048, np.float32)
+    rc = capi.load().wd_moe_stack_f32(arr, 3, g.ptr(dx), g.ptr(out), sc.h, None, float(2.0 ** -12), 0, g.stream())
+    assert rc == -3 and "ran out" in capi.load().wd_last_error().decode()   # WD_ERR_STATE: refused by the host
+    d_x.copy_(torch.from_numpy(x).cuda())
+    graph.replay()                                   # refused on the device: nothing waits
+    g.sync()
+    assert np.isnan(g.host(d_x)).all() and np.isnan(g.host(d_out)).all()
     assert capi.load().wd_moe_scratch_status(sc.h) == 1
-    assert np.isnan(bad[0]).all() and np.isnan(bad[1]).all()
     capi.call("wd_moe_scratch_set_wait_limit", sc.h, 0)
     assert capi.load().wd_moe_scratch_status(sc.h) == 0
     for _ in range(3):
         got = _run_stack(g, arr, 3, x, None, sc, 0)
         assert g.same_bits(got[0], want[0]) and g.same_bits(got[1], want[1])
+    d_x.copy_(torch.from_numpy(x).cuda())
+    graph.replay()
+    g.sync()
+    assert g.same_bits(g.host(d_x), want[0]) and g.same_bits(g.host(d_out), want[1])
+    sc.close()
+    ref.close()
+
+
+def test_one_launch_stack_keeps_the_descriptors_of_a_recorded_graph(g):
+    """A graph recorded for one stack still computes that stack after the same scratch has run another one: every stack a
+    scratch has seen keeps a device copy of its layer descriptors of its own."""
+    import torch
+    Ls = [synth.make_c2(layer=330 + l, n_experts=64) for l in range(4)]
+    dls, arr = _descs(g, Ls)
+    other = (capi.MoeLayer * 2)(arr[3], arr[2])
+    sc, ref = g.Scratch(2048, 512, 64, 10), g.Scratch(2048, 512, 64, 10)
+    x = synth.rms_normed(synth.rng_for(SEED, 86), 2048)
+    want = _run_stack(g, arr, 2, x, None, ref, PER_LAYER)
+    want_other = _run_stack(g, other, 2, x, None, ref, PER_LAYER)
+    d_x, d_out = g.dev(x), g.empty(2048, np.float32)
+
+    def launch():
+        capi.call("wd_moe_stack_f32", arr, 2, g.ptr(d_x), g.ptr(d_out), sc.h, None, float(2.0 ** -12), 0,
+                  C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        launch()
+    got_other = _run_stack(g, other, 2, x, None, sc, 0)     # another stack on the same scratch, eagerly
+    assert g.same_bits(got_other[0], want_other[0]) and g.same_bits(got_other[1], want_other[1])
+    d_x.copy_(torch.from_numpy(x).cuda())
+    graph.replay()
+    g.sync()
+    assert g.same_bits(g.host(d_x), want[0]) and g.same_bits(g.host(d_out), want[1])
+    assert capi.load().wd_moe_scratch_status(sc.h) == 0
     sc.close()
     ref.close()

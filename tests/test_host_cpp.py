@@ -32,13 +32,13 @@ def test_reference_style_caller_matches_oracle():
     assert int(out.split(" checks")[0].split()[-1]) > 60, out
 
 
-def test_read_ahead_ring_host_checks():
-    """tests/host/test_readahead.cpp: the expert read-ahead ring and its history, no GPU
+def test_expert_prefetcher_host_checks():
+    """tests/host/test_prefetch.cpp: the expert prefetcher and its planner, no GPU
     (the contract of the reference's tests/expert_prefetch_host_test.cpp)."""
     from warpdecode_amd import build
     if not os.path.exists(build.LIB):
         pytest.skip("HIP library not built")
     build.build_host_test()
-    exe = os.path.join(ROOT, "tests", "host", "test_readahead")
+    exe = os.path.join(ROOT, "tests", "host", "test_prefetch")
     p = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     assert p.returncode == 0 and " 0 failures" in p.stdout, p.stdout

@@ -35,9 +35,9 @@ def build_host_test(verbose=False):
     if verbose:
         print(" ".join(cmd))
     subprocess.check_call(cmd)
-    # the read-ahead ring's host test: no GPU library at all
-    cmd = ["g++", "-std=c++17", "-O2", "-Wall", "-Wextra", "-pthread", "-I" + CSRC, os.path.join(root, "tests", "host", "test_readahead.cpp"),
-           "-o", os.path.join(root, "tests", "host", "test_readahead")]
+    # the expert prefetcher's host test: no GPU library at all
+    cmd = ["g++", "-std=c++17", "-O2", "-Wall", "-Wextra", "-pthread", "-I" + CSRC, os.path.join(root, "tests", "host", "test_prefetch.cpp"),
+           "-o", os.path.join(root, "tests", "host", "test_prefetch")]
     if verbose:
         print(" ".join(cmd))
     subprocess.check_call(cmd)

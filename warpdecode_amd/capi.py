@@ -102,7 +102,6 @@ _SIGS = {
     "wd_moe_scratch_enable_partials": (i32, [vp, i32, i32]),
     "wd_moe_scratch_trace": (vp, [vp, i32]),
     "wd_moe_scratch_trace_resident": (vp, [vp, i32, i32]),
-    "wd_moe_scratch_omit_resident": (i32, [vp, i32]),
     "wd_profile_enable": (i32, [i32]),
     "wd_profile_enabled": (i32, []),
     "wd_profile_begin": (i32, [i32, vp]),

@@ -24,7 +24,7 @@
 //     is named by the caller or found through /proc/self/maps (wd_expert_cache_attach_mappings).
 #include "wd_common.h"
 #include "wd_profile.hpp"
-#include "wd_readahead.hpp"
+#include "wd_prefetch.hpp"
 
 #include <fcntl.h>
 #include <unistd.h>
@@ -336,11 +336,11 @@ struct wd_expert_cache {
     std::vector<hipEvent_t> ev_layer;      // token-ahead acquires: the fills of layer l are complete
     std::vector<int> layer_event;          //   ... when ev_layer[layer_event[l]] has passed (fills are launched by groups of layers)
     int last_waited = -1;                  // the event the caller's stream was last made to wait for in this token
-    // read-ahead of predicted experts from the model file (wd_readahead.hpp); the reader thread touches ra_mem only
-    wd::ReadAheadRing ra;
-    wd::ReadAheadHistory ra_hist;
-    uint8_t *ra_mem = nullptr;             // pinned, one slot per ring entry
-    std::vector<hipEvent_t> ra_done;       // per entry: the DMA that last read its buffer
+    // read-ahead of predicted experts from the model file (wd_prefetch.hpp); the reader thread touches ra_mem only
+    wd::ExpertPrefetcher ra;
+    wd::PrefetchPlanner ra_plan;
+    uint8_t *ra_mem = nullptr;             // pinned, one slot per shelf
+    std::vector<hipEvent_t> ra_done;       // per shelf: the DMA that last read it
     uint64_t ra_fills = 0, ra_candidates = 0, ra_resident_skips = 0;
     hipEvent_t ev_token[2] = {nullptr, nullptr};  // recorded on the caller's stream when a token-ahead acquire begins, alternately
     int token_parity = 0;
@@ -480,7 +480,7 @@ int wd_expert_cache_create(wd_expert_cache **out, size_t capacity_bytes, size_t 
 int wd_expert_cache_destroy(wd_expert_cache *c) {
     if (!c) return WD_OK;
     if (c->copy_stream) (void)hipStreamSynchronize(c->copy_stream);
-    c->ra.release();  // (joins the reader before its buffers go)
+    c->ra.stop();  // (joins the reader before its buffers go)
     if (c->ra_mem) (void)hipHostFree(c->ra_mem);
     for (hipEvent_t ev : c->ra_done)
         if (ev) (void)hipEventDestroy(ev);
@@ -596,14 +596,14 @@ int wd_expert_cache_set_read_ahead(wd_expert_cache *c, int depth, int slots) {
     WD_REQUIRE(c != nullptr, "expert cache is not initialized");
     WD_REQUIRE(depth >= 0 && depth <= 8 && slots >= 0 && slots <= 1024, "expert cache read-ahead: depth 0..8, slots 0..1024 (got %d, %d)", depth, slots);
     if (c->copy_stream) WD_HIP(hipStreamSynchronize(c->copy_stream));  // no DMA reads the old ring any more
-    c->ra.release();
+    c->ra.stop();
     if (c->ra_mem) (void)hipHostFree(c->ra_mem);
     c->ra_mem = nullptr;
     for (hipEvent_t ev : c->ra_done)
         if (ev) (void)hipEventDestroy(ev);
     c->ra_done.clear();
-    c->ra_hist = wd::ReadAheadHistory();
-    c->ra_hist.set_depth(depth);
+    c->ra_plan = wd::PrefetchPlanner();
+    c->ra_plan.set_depth(depth);
     if (depth == 0) return WD_OK;
     const int n = slots > 0 ? slots : depth * 16;  // (the reference's default, src/expert_cache.cuh:995)
     WD_HIP(hipHostMalloc(reinterpret_cast<void **>(&c->ra_mem), static_cast<size_t>(n) * c->slot_bytes, hipHostMallocDefault));
@@ -613,7 +613,7 @@ int wd_expert_cache_set_read_ahead(wd_expert_cache *c, int depth, int slots) {
         bufs.push_back(c->ra_mem + static_cast<size_t>(i) * c->slot_bytes);
         WD_HIP(hipEventCreateWithFlags(&c->ra_done[i], hipEventDisableTiming));
     }
-    c->ra.configure(bufs, [c](int entry) { return hipEventQuery(c->ra_done[static_cast<size_t>(entry)]) == hipSuccess; });
+    c->ra.start(bufs, [c](int shelf) { return hipEventQuery(c->ra_done[static_cast<size_t>(shelf)]) == hipSuccess; });
     return WD_OK;
 }
 
@@ -736,9 +736,9 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
         ++c->layer_access[layer];
         c->distinct.insert(key);
         for (Shadow &sh : c->shadows) sh.access(key);
-        if (c->ra.enabled() && !ahead) {
+        if (c->ra.running() && !ahead) {
             // what the previous token took in this layer (and the next ones): read it from the file while the layers compute
-            for (uint64_t cand : c->ra_hist.note_access(layer, key)) {
+            for (uint64_t cand : c->ra_plan.on_acquire(layer, key)) {
                 ++c->ra_candidates;
                 if (c->index.find(cand) != c->index.end()) {
                     ++c->ra_resident_skips;
@@ -750,10 +750,10 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
                     continue;
                 const FileSource &fs = c->files[c->layer_file[cl]];
                 const uint8_t *src[3] = {c->h_gate[cl] + ce * c->s_gate[cl], c->h_up[cl] + ce * c->s_up[cl], c->h_down[cl] + ce * c->s_down[cl]};
-                const uint64_t file_off[3] = {fs.file_off + static_cast<uint64_t>(src[0] - fs.base), fs.file_off + static_cast<uint64_t>(src[1] - fs.base),
-                                              fs.file_off + static_cast<uint64_t>(src[2] - fs.base)};
-                const size_t at[3] = {0, c->gate_bytes, c->gate_bytes + c->up_bytes}, len[3] = {c->gate_bytes, c->up_bytes, c->down_bytes};
-                c->ra.post(cand, fs.fd, file_off, at, len, 3);
+                const wd::PrefetchRun runs[3] = {{fs.file_off + static_cast<uint64_t>(src[0] - fs.base), 0, c->gate_bytes},
+                                                 {fs.file_off + static_cast<uint64_t>(src[1] - fs.base), c->gate_bytes, c->up_bytes},
+                                                 {fs.file_off + static_cast<uint64_t>(src[2] - fs.base), c->gate_bytes + c->up_bytes, c->down_bytes}};
+                c->ra.request(cand, fs.fd, runs, 3);
             }
         }
         auto it = c->index.find(key);
@@ -812,13 +812,14 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
         uint8_t *dst3[3] = {dst, dst + c->gate_bytes, dst + c->gate_bytes + c->up_bytes};
         const size_t len3[3] = {c->gate_bytes, c->up_bytes, c->down_bytes};
         const bool one_piece = src3[0] + len3[0] == src3[1] && src3[1] + len3[1] == src3[2];
-        int ra_entry = -1;
-        uint8_t *ra_buf = by_file && c->ra.enabled() ? c->ra.borrow(key, &ra_entry) : nullptr;
-        if (ra_buf) {
+        const int shelf = by_file ? c->ra.claim(key) : -1;
+        if (shelf >= 0) {
             // a prediction that came true: the slot's bytes are in pinned memory already, laid out like the slot
-            WD_HIP(hipMemcpyAsync(dst, ra_buf, c->slot_bytes, hipMemcpyHostToDevice, c->copy_stream));
-            WD_HIP(hipEventRecord(c->ra_done[static_cast<size_t>(ra_entry)], c->copy_stream));
-            c->ra.finish_borrow(key);
+            const hipError_t e1 = hipMemcpyAsync(dst, c->ra.data(shelf), c->slot_bytes, hipMemcpyHostToDevice, c->copy_stream);
+            const hipError_t e2 = hipEventRecord(c->ra_done[static_cast<size_t>(shelf)], c->copy_stream);
+            c->ra.copy_queued(shelf);  // (also after an error: the event then speaks of whatever was queued before)
+            WD_HIP(e1);
+            WD_HIP(e2);
             ++c->ra_fills;
         } else if (by_file) {
             // the three slices land in one ring entry in slot order, then the slot is filled with one DMA
@@ -1052,9 +1053,9 @@ size_t wd_expert_cache_dump_json(wd_expert_cache *c, char *buf, size_t cap) {
     s += ",\"acquire_calls\":" + std::to_string(c->acquire_calls) + ",\"acquire_ms\":" + fixed(c->acquire_ms, 1);
     s += ",\"fills_by_copy_kernel\":" + std::to_string(c->kernel_fills) + ",\"fills_by_memcpy\":" + std::to_string(c->dma_fills);
     s += ",\"fills_by_pread\":" + std::to_string(c->pread_fills) + ",\"pread_ms\":" + fixed(c->pread_ms, 1);
-    s += ",\"read_ahead\":{\"depth\":" + std::to_string(c->ra_hist.depth()) + ",\"slots\":" + std::to_string(c->ra.slots()) +
+    s += ",\"read_ahead\":{\"depth\":" + std::to_string(c->ra_plan.depth()) + ",\"slots\":" + std::to_string(c->ra.shelves()) +
          ",\"candidates\":" + std::to_string(c->ra_candidates) + ",\"already_resident\":" + std::to_string(c->ra_resident_skips) +
-         ",\"posted\":" + std::to_string(c->ra.posted()) + ",\"dropped\":" + std::to_string(c->ra.dropped()) +
+         ",\"posted\":" + std::to_string(c->ra.requested()) + ",\"dropped\":" + std::to_string(c->ra.dropped()) +
          ",\"delivered\":" + std::to_string(c->ra.delivered()) + ",\"failed\":" + std::to_string(c->ra.failed()) +
          ",\"fills\":" + std::to_string(c->ra_fills) + "}";
     s += ",\"prev_token_ready\":" + std::to_string(c->prev_ready);

@@ -54,7 +54,7 @@ struct LayerArgs {
 
 constexpr int kTagCopies = 16;           // replicas of the published ids, 64 bytes apart, so that pollers spread over lines
 constexpr uint32_t kTagInvalid = 0xffffffffu;
-constexpr unsigned kSpinLimit = 1u << 21;  // default number of polls before a wait gives up (seconds)
+constexpr unsigned kSpinLimit = 1u << 16;  // default number of polls before a wait gives up (tens of milliseconds; a wait lasts microseconds)
 
 // Time stamp `i` of dispatch `d` (0 = A, 1 = B, 2 = C) for the traced workgroup; lane 0 of every wave.
 // TRACE false: compiled out (the kernels that take the stamps as a template parameter run without their tests then).
@@ -533,6 +533,136 @@ WD_DEV void topk_wave(const float *logits, int n, int k, float w_scale, int32_t 
         topk_wave_m<2, COHERENT>(logits, n, k, w_scale, ids, weights, override_ids, lane);
 }
 
+// ---- the same selection by ONE wave that holds eight logits per lane ------------------------------------------------
+// lv[j] is the logit of expert 64 j + lane (-inf at and beyond n; n <= 512, k <= 15).  A single wave pays for every trip
+// through LDS or the scalar unit with hundreds of idle cycles, so step A stays in the vector registers: every logit
+// becomes a 32-bit key - its bits mapped so that unsigned order is float order, the low nine bits replaced by
+// 511 - expert - , every lane sorts its eight keys (a network of 19 exchanges), and k + 1 rounds of "largest head of any
+// lane" (a DPP reduction; the lane that held it moves its keys up) give the k + 1 largest keys in order, key j in
+// lane j.  The keys order the logits up to their low nine bits, so the result is accepted as the selection only when
+//   * the keys' upper 23 bits are strictly decreasing over the k + 1 - any logit that was not taken then lies below
+//     the grid point at or below the k-th taken logit -, and
+//   * the exponentials e_0 > e_1 > ... > e_k of the k + 1 exact logits are strictly decreasing by a relative margin:
+//     exp_ggml is within two units in the last place of the true exponential (relative error below 2^-22) on normal
+//     results, so every logit not above the (k+1)-th has an exponential below e_k (1 + 2^-21), and
+//     e_(k-1) > e_k (1 + 2^-18) puts the k-th selected strictly above everything left, also after the product with the
+//     row's 1/sum has been rounded.
+// Rows the test does not accept (ties, near-ties, NaN, +inf, fewer than k + 1 finite logits, selected exponentials below
+// 2^-100) take the reference's rungs over all probabilities in step B.
+struct SelWaveState {
+    float mx;      // the row's largest logit
+    float e;       // lane j <= k: exponential of the j-th largest logit (accepted rows)
+    int id;        // lane j <= k: its expert
+    bool fast;     // step A accepted the row (the same in every lane)
+};
+
+WD_DEV uint32_t wave_max_u32(uint32_t v) {  // the result is uniform
+    v = max(v, static_cast<uint32_t>(dpp_i<kDppXor1>(static_cast<int>(v), static_cast<int>(v))));
+    v = max(v, static_cast<uint32_t>(dpp_i<kDppXor2>(static_cast<int>(v), static_cast<int>(v))));
+    v = max(v, static_cast<uint32_t>(dpp_i<kDppRor4>(static_cast<int>(v), static_cast<int>(v))));
+    v = max(v, static_cast<uint32_t>(dpp_i<kDppRor8>(static_cast<int>(v), static_cast<int>(v))));  // every lane: its row's largest
+    const wd_uint2v t = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    v = max(t.x, t.y);                                                                            // rows 0|2 and 1|3
+    return max(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), 0)),
+               static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), 16)));
+}
+
+// Step A.  Returns with st.fast, and for accepted rows the ids of the selection in lanes 0..k-1 of st.id.
+// Registers and cross-lane moves only: no LDS is written or read.
+WD_DEV void sel_wave_ids(const float (&lv)[8], int n, int k, int lane, SelWaveState &st) {
+    uint32_t h[8];
+    bool odd = false;
+    float lm = lv[0];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int id = 64 * j + lane;
+        odd = odd || lv[j] != lv[j];
+        lm = __builtin_fmaxf(lm, lv[j]);
+        const uint32_t b = f_bits(lv[j]);
+        const uint32_t ord = b ^ ((b & 0x80000000u) ? 0xffffffffu : 0x80000000u);  // unsigned order = float order
+        h[j] = id < n ? ((ord & ~0x1ffu) | static_cast<uint32_t>(511 - id)) : 0u;
+    }
+    const float mx = wave_max(lm);
+    auto exchange = [&](int i, int j) {  // the larger key to the lower register
+        const uint32_t hi = max(h[i], h[j]), lo = min(h[i], h[j]);
+        h[i] = hi, h[j] = lo;
+    };
+    exchange(0, 1), exchange(2, 3), exchange(4, 5), exchange(6, 7);
+    exchange(0, 2), exchange(1, 3), exchange(4, 6), exchange(5, 7);
+    exchange(1, 2), exchange(5, 6);
+    exchange(0, 4), exchange(1, 5), exchange(2, 6), exchange(3, 7);
+    exchange(2, 4), exchange(3, 5);
+    exchange(1, 2), exchange(3, 4), exchange(5, 6);
+    uint32_t mine = 0u;  // lane j: the j-th largest key of the row
+    for (int j = 0; j <= k; ++j) {
+        const uint32_t m = wave_max_u32(h[0]);
+        const bool won = h[0] == m;  // (keys are distinct: they end in the expert's number)
+#pragma unroll
+        for (int i = 0; i < 7; ++i) h[i] = won ? h[i + 1] : h[i];
+        h[7] = won ? 0u : h[7];
+        mine = lane == j ? m : mine;
+    }
+    // the exact logit behind key j: register idc / 64 of lane idc % 64
+    const int idc = 511 - static_cast<int>(mine & 0x1ffu);
+    const bool have = lane <= k && mine != 0u && idc < n;
+    float l = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float from = __shfl(lv[j], idc & 63, kWave);
+        l = (have && (idc >> 6) == j) ? from : l;
+    }
+    const float e = (have && l > -INFINITY) ? exp_ggml(l - mx) : 0.0f;
+    const float nxt = dpp_f<kDppShl1>(0.0f, e);  // k + 1 <= 16: these lanes are one row
+    const uint32_t grid = mine >> 9, grid_nxt = static_cast<uint32_t>(dpp_i<kDppShl1>(0, static_cast<int>(grid)));
+    const bool good = lane > k || (have && l > -INFINITY &&
+                                   (lane == k || (grid > grid_nxt && e >= 0x1p-100f && e > nxt * (lane == k - 1 ? 1.000004f : 1.000001f))));
+    st.mx = mx, st.e = e, st.id = idc;
+    st.fast = __builtin_amdgcn_ballot_w64(odd) == 0ull && mx < INFINITY && __builtin_amdgcn_ballot_w64(good) == ~0ull;
+}
+
+// Step B, first half (any wave that holds the logits; it need not be the wave of step A): every exponential into s.p,
+// the per-8 sums, and the row's 1/sum as the reference takes it (0 for a row whose exponentials all vanished: `dead`).
+WD_DEV float sel_wave_denominator(const float (&lv)[8], int n, const TopkLds<1> &s, int lane, bool &dead) {
+    const int groups = n >> 3;
+    float lm = lv[0];
+#pragma unroll
+    for (int j = 1; j < 8; ++j) lm = __builtin_fmaxf(lm, lv[j]);
+    const float mx = wave_max(lm);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int id = 64 * j + lane;
+        const float e = (id < n) ? exp_ggml(lv[j] - mx) : 0.0f;
+        const float gs = close_lanes8(e);
+        if ((lane & 7) == 0) s.gsum[8 * j + (lane >> 3)] = gs;
+        s.p[id] = e;
+    }
+    wave_lds_fence();
+    const float g1[1] = {lane < groups ? s.gsum[lane] : 0.0f};
+    const double sum = sum_groups<1>(g1, groups, lane);
+    dead = sum == 0.0;
+    return dead ? 0.0f : static_cast<float>(1.0 / sum);
+}
+
+// Step B, second half (the wave of step A; s.p and inv as the first half left them, which may have been another wave
+// on the far side of a barrier): for rows step A did not accept the reference's rungs over the probabilities; then lanes
+// 0..k-1 write the weights and the ids (ids_given: id_given instead).
+WD_DEV void sel_wave_weights(int n, int k, float w_scale, const TopkLds<1> &s, int lane, SelWaveState &st, float inv, bool dead,
+                             int32_t *ids, float *weights, bool ids_given, int id_given) {
+    float top_mine = st.e * inv;
+    int id_mine = st.id;
+    if (!st.fast) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int ix = lane * 8 + i;
+            v[i] = (ix < n && !dead) ? s.p[ix] * inv : -INFINITY;
+        }
+        rungs_on_probs<1>(v, k, lane, top_mine, id_mine);
+        st.id = id_mine;
+    }
+    finish_weights(top_mine, ids_given ? id_given : id_mine, k, w_scale, ids, weights, nullptr, lane);
+}
+
 // Stand-alone softmax/top-k dispatch: one wave (src/qwen38_moe.cuh:711-818).
 // If gate_logit != null, gate_logit[0] is replaced by sigmoid_ggml(gate_logit[0]) (shared expert gate).
 // If override_ids != null the selected ids are replaced by override_ids[0..k) after the weights are formed.
@@ -542,6 +672,21 @@ __global__ __launch_bounds__(64) void k_topk_softmax(const float *__restrict__ l
                                                       const int32_t *__restrict__ override_ids) {
     const int lane = threadIdx.x;
     if (gate_logit && lane == 0) gate_logit[0] = sigmoid_ggml(gate_logit[0]);
+    if (n <= 512 && k <= 15) {  // threshold and ranks first, the reference's rungs for the rows that need them
+        __shared__ __align__(16) uint8_t s_sel[kTopkLdsBytes1];
+        const TopkLds<1> s(s_sel);
+        float lv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) lv[j] = (64 * j + lane < n) ? logits[64 * j + lane] : -INFINITY;
+        SelWaveState st;
+        sel_wave_ids(lv, n, k, lane, st);
+        int id_given = 0;
+        if (override_ids && lane < k) id_given = override_ids[lane];
+        bool dead;
+        const float inv = sel_wave_denominator(lv, n, s, lane, dead);
+        sel_wave_weights(n, k, w_scale, s, lane, st, inv, dead, ids, weights, override_ids != nullptr, id_given);
+        return;
+    }
     topk_wave<false>(logits, n, k, w_scale, ids, weights, override_ids, lane);
 }
 

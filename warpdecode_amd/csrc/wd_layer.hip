@@ -5,6 +5,7 @@
 #include "wd_tokens.cuh"
 #include "wd_resident.cuh"
 
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 #include <new>
@@ -37,18 +38,23 @@ struct wd_moe_scratch {
     unsigned *arrive = nullptr;           // device counter used inside the fused dispatch A
     unsigned long long *trace = nullptr;  // device [3][16][8] time stamps, see wd_moe_scratch_trace
     int trace_wg = 0;
-    int32_t *h_ids = nullptr;             // pinned [16]: routed ids for callers that must see them on the host
+    int32_t *h_ids = nullptr;             // pinned [32]: [0..15] routed ids for callers that must see them on the host,
+                                          // [16] mirror of the status word, written by the resident launch when a wait runs out
     uint32_t *tagged = nullptr;           // [kTagRecords][kTagCopies][16] ids published inside the merged dispatch
     unsigned *status = nullptr;           // [0] != 0: a bounded wait inside a dispatch ran out
     unsigned spin_limit = kSpinLimit;
     int compute_units = 256;              // of the device the scratch lives on
     // the resident stack kernel (wd_resident.cuh): hand-off buffers, device copy of the layer descriptors
     uint8_t *res_block = nullptr;
-    ResidentLayer *res_layers = nullptr;          // device [kResMaxLayers], then one ResidentViews
-    std::vector<ResidentLayer> res_shadow;        // what res_layers holds
+    // Device copies of the layer descriptors of the stacks this scratch has run ([kResMaxLayers], then one ResidentViews
+    // each).  A copy is never overwritten: a captured graph keeps the address of the copy it was recorded with.
+    struct ResDescSet {
+        std::vector<ResidentLayer> shadow;
+        ResidentLayer *dev = nullptr;
+    };
+    std::vector<ResDescSet> res_sets;
     int res_fits = -1;                            // -1 not asked yet; 1: the device holds the whole grid at once
     int trace_layer = 0;
-    int res_omit = 0;                             // measurement aid: parts of the resident launch left out (wd_moe_scratch_omit_resident)
     bool trace_all = false;                       // the trace buffer has the resident kernel's size
     // wd_moe_layer_tokens_pairs_f32: a ring of pointer tables (pinned staging + device copy), kPairRing x [kPairEntries][3]
     const uint8_t **pair_host = nullptr, **pair_dev = nullptr;
@@ -56,7 +62,7 @@ struct wd_moe_scratch {
     bool pair_used[4] = {false, false, false, false};
     int pair_next = 0;
 };
-constexpr int kPairRing = 4, kPairEntries = 128;
+constexpr int kPairRing = 4;
 
 namespace {
 constexpr int kTagRecords = 64;  // one record per layer of a stack (modulo), so that a chain of layers needs no reset in between
@@ -128,11 +134,12 @@ int wd_moe_scratch_create(wd_moe_scratch **out, int hidden, int expert_ffn, int 
     s->status = reinterpret_cast<unsigned *>(b + o_status);
     (void)hipMemset(s->block, 0, c.off);
     (void)hipMemset(s->tagged, 0xff, sizeof(uint32_t) * kTagRecords * kTagCopies * 16);
-    if (hipHostMalloc(reinterpret_cast<void **>(&s->h_ids), sizeof(int32_t) * 16, hipHostMallocDefault) != hipSuccess) {
+    if (hipHostMalloc(reinterpret_cast<void **>(&s->h_ids), sizeof(int32_t) * 32, hipHostMallocDefault) != hipSuccess) {
         (void)hipFree(s->block);
         delete s;
         return fail(WD_ERR_HIP, "hipHostMalloc MoE scratch ids failed");
     }
+    std::memset(s->h_ids, 0, sizeof(int32_t) * 32);
     *out = s;
     return WD_OK;
 }
@@ -144,7 +151,7 @@ int wd_moe_scratch_destroy(wd_moe_scratch *s) {
     (void)hipFree(s->dp);
     (void)hipFree(s->trace);
     (void)hipFree(s->res_block);
-    (void)hipFree(s->res_layers);
+    for (wd_moe_scratch::ResDescSet &d : s->res_sets) (void)hipFree(d.dev);
     (void)hipHostFree(s->h_ids);
     (void)hipFree(s->pair_dev);
     (void)hipHostFree(s->pair_host);
@@ -165,7 +172,9 @@ int wd_moe_scratch_set_wait_limit(wd_moe_scratch *s, unsigned polls) {
     WD_REQUIRE(s != nullptr, "wd_moe_scratch_set_wait_limit: null scratch");
     s->spin_limit = polls ? polls : kSpinLimit;
     // a fresh start: clear the status word and make the published ids invalid again
+    WD_HIP(hipDeviceSynchronize());  // (a launch that gave up may still be running and would set the words again)
     WD_HIP(hipMemset(s->status, 0, sizeof(unsigned)));
+    reinterpret_cast<volatile int32_t *>(s->h_ids)[16] = 0;
     WD_HIP(hipMemset(s->tagged, 0xff, sizeof(uint32_t) * kTagRecords * kTagCopies * 16));
     if (s->res_block) WD_HIP(hipMemset(s->res_block, 0xff, kHandEpoch));
     return WD_OK;
@@ -217,14 +226,6 @@ unsigned long long *wd_moe_scratch_trace_resident(wd_moe_scratch *s, int wg, int
     (void)hipMemset(s->trace, 0, bytes);
     s->trace_wg = wg, s->trace_layer = layer;
     return s->trace;
-}
-
-// Measurement aid: leaves parts of the resident launch out (results are then invalid), to time what remains.
-int wd_moe_scratch_omit_resident(wd_moe_scratch *s, int mask) {
-    WD_REQUIRE(s != nullptr, "omit parts of the resident launch: null scratch");
-    WD_REQUIRE(mask >= 0 && mask < 16, "omit parts of the resident launch: mask 0..15 (got %d)", mask);
-    s->res_omit = mask;
-    return WD_OK;
 }
 
 int wd_moe_scratch_enable_partials(wd_moe_scratch *s, int gate_type, int down_type) {
@@ -740,22 +741,36 @@ extern "C" int wd_shared_expert_f32(const wd_moe_layer *L, const float *d_x, wd_
 
 namespace {
 
-// The hand-off buffers and the descriptor array of the resident stack kernel, allocated on first use.
+// The hand-off buffers of the resident stack kernel, allocated on first use.
 int resident_prepare(wd_moe_scratch *s) {
     if (s->res_block) return WD_OK;
     uint8_t *b = nullptr;
     WD_HIP(hipMalloc(reinterpret_cast<void **>(&b), kHandBytes));
-    const size_t desc_bytes = sizeof(ResidentLayer) * kResMaxLayers + sizeof(ResidentViews);
-    if (hipMalloc(reinterpret_cast<void **>(&s->res_layers), desc_bytes) != hipSuccess) {
-        (void)hipFree(b);
-        return fail(WD_ERR_HIP, "hipMalloc of the resident stack's layer descriptors failed");
-    }
     (void)hipMemset(b, 0xff, kHandEpoch);                        // every hand-off word of both sets "not yet written"
     (void)hipMemset(b + kHandEpoch, 0, kHandBytes - kHandEpoch);  // launches finished
-    const ResidentViews v{s->logits, s->weights, s->accum, s->down_f32, s->shared_gate, s->ids};
-    (void)hipMemcpy(s->res_layers + kResMaxLayers, &v, sizeof(v), hipMemcpyHostToDevice);
     s->res_block = b;
     return WD_OK;
+}
+
+// The device copy of these layer descriptors: the one made for an equal stack before, or a new one (null: none may be
+// made now - a graph is being recorded, or the scratch already holds kResMaxDescSets different stacks).
+constexpr size_t kResMaxDescSets = 32;
+ResidentLayer *resident_descriptors(wd_moe_scratch *s, const std::vector<ResidentLayer> &want, bool capturing) {
+    for (const wd_moe_scratch::ResDescSet &d : s->res_sets)
+        if (d.shadow.size() == want.size() && std::memcmp(d.shadow.data(), want.data(), sizeof(ResidentLayer) * want.size()) == 0) return d.dev;
+    if (capturing || s->res_sets.size() >= kResMaxDescSets) return nullptr;
+    wd_moe_scratch::ResDescSet d;
+    const size_t desc_bytes = sizeof(ResidentLayer) * kResMaxLayers + sizeof(ResidentViews);
+    if (hipMalloc(reinterpret_cast<void **>(&d.dev), desc_bytes) != hipSuccess) return nullptr;
+    const ResidentViews v{s->logits, s->weights, s->accum, s->down_f32, s->shared_gate, s->ids};
+    if (hipMemcpy(d.dev, want.data(), sizeof(ResidentLayer) * want.size(), hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemcpy(d.dev + kResMaxLayers, &v, sizeof(v), hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipFree(d.dev);
+        return nullptr;
+    }
+    d.shadow = want;
+    s->res_sets.push_back(d);
+    return d.dev;
 }
 
 bool aligned16(const void *p, size_t stride) { return reinterpret_cast<uintptr_t>(p) % 16 == 0 && stride % 16 == 0; }
@@ -779,14 +794,17 @@ bool resident_shape(const wd_moe_layer *layers, int n_layers, const wd_moe_scrat
     return true;
 }
 
+constexpr int kTakePerLayer = 1;  // (not an error code) the stack cannot run as one resident launch
+
 template <int TYPE>
 int resident_launch(const ResidentArgs &a, wd_moe_scratch *s, hipStream_t st) {
-    if (s->res_fits < 0) {
-        int per_cu = 0;
-        const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_stack_resident<TYPE, true>, kResThreads, kResLdsBytes);
-        s->res_fits = (e == hipSuccess && per_cu * s->compute_units >= kResWgs) ? 1 : 0;
+    if (s->res_fits < 0) {  // both variants of the kernel (with and without the time stamps) must fit
+        int plain = 0, stamped = 0;
+        const hipError_t e0 = hipOccupancyMaxActiveBlocksPerMultiprocessor(&plain, k_stack_resident<TYPE, false>, kResThreads, kResLdsBytes);
+        const hipError_t e1 = hipOccupancyMaxActiveBlocksPerMultiprocessor(&stamped, k_stack_resident<TYPE, true>, kResThreads, kResLdsBytes);
+        s->res_fits = (e0 == hipSuccess && e1 == hipSuccess && std::min(plain, stamped) * s->compute_units >= kResWgs) ? 1 : 0;
     }
-    if (!s->res_fits) return -1;  // the workgroups would wait for each other without all being on the device
+    if (!s->res_fits) return kTakePerLayer;  // the workgroups would wait for each other without all being on the device
     SiteScope site(WD_SITE_STACK_RESIDENT, st);
     if (a.trace)  // (the variant with the time stamps only when they are asked for)
         k_stack_resident<TYPE, true><<<dim3(kResWgs), dim3(kResThreads), kResLdsBytes, st>>>(a);
@@ -796,14 +814,14 @@ int resident_launch(const ResidentArgs &a, wd_moe_scratch *s, hipStream_t st) {
     return WD_OK;
 }
 
-// Returns -1 when the stack has to take the per-layer dispatches instead.
+// Returns kTakePerLayer when the stack has to take the per-layer dispatches instead.
 int stack_resident(const wd_moe_layer *layers, int n_layers, float *d_x, float *d_layer_out, wd_moe_scratch *s,
                    const int32_t *d_ids_trace, float residual_scale, hipStream_t st) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(st, &cap) != hipSuccess) return -1;
+    if (hipStreamIsCapturing(st, &cap) != hipSuccess) return kTakePerLayer;
     const bool capturing = cap != hipStreamCaptureStatusNone;
     if (!s->res_block) {
-        if (capturing) return -1;  // nothing may be allocated while a graph is recorded
+        if (capturing) return kTakePerLayer;  // nothing may be allocated while a graph is recorded
         if (const int rc = resident_prepare(s)) return rc;
     }
     std::vector<ResidentLayer> want(n_layers);
@@ -816,21 +834,21 @@ int stack_resident(const wd_moe_layer *layers, int n_layers, float *d_x, float *
         d.gate = L.gate, d.up = L.up, d.down = L.down;
         d.w_scale = L.expert_scale;
     }
-    if (s->res_shadow.size() != want.size() || std::memcmp(s->res_shadow.data(), want.data(), sizeof(ResidentLayer) * want.size()) != 0) {
-        if (capturing) return -1;
-        WD_HIP(hipStreamSynchronize(st));  // an earlier launch on this stream may still read the old descriptors
-        WD_HIP(hipMemcpy(s->res_layers, want.data(), sizeof(ResidentLayer) * want.size(), hipMemcpyHostToDevice));
-        s->res_shadow = want;
-    }
+    ResidentLayer *const descriptors = resident_descriptors(s, want, capturing);
+    if (!descriptors) return kTakePerLayer;
+    // a wait of an earlier launch on this scratch ran out: its results were NaN, and so would this launch's be
+    if (reinterpret_cast<const volatile int32_t *>(s->h_ids)[16] != 0)
+        return fail(WD_ERR_STATE, "MoE stack: a wait inside an earlier resident launch on this scratch ran out (is other work resident on the device?); "
+                                  "wd_moe_scratch_set_wait_limit resets the scratch");
     ResidentArgs a{};
-    a.layers = s->res_layers, a.n_layers = n_layers, a.E = layers[0].n_experts, a.k = layers[0].top_k;
+    a.layers = descriptors, a.n_layers = n_layers, a.E = layers[0].n_experts, a.k = layers[0].top_k;
     a.shared = layers[0].shared_gate_inp != nullptr;
     a.gate_stride = layers[0].gate_stride, a.up_stride = layers[0].up_stride, a.down_stride = layers[0].down_stride;
     a.x = d_x, a.out = d_layer_out, a.residual_scale = residual_scale, a.ids_trace = d_ids_trace;
-    a.views = reinterpret_cast<const ResidentViews *>(s->res_layers + kResMaxLayers);
+    a.views = reinterpret_cast<const ResidentViews *>(descriptors + kResMaxLayers);
     a.hand = s->res_block, a.status = s->status, a.spin_limit = s->spin_limit;
+    a.status_host = reinterpret_cast<unsigned *>(s->h_ids + 16);
     a.trace = s->trace, a.trace_wg = s->trace_wg, a.trace_layer = s->trace_layer;
-    a.debug = s->res_omit;
     return layers[0].gate_type == WD_TYPE_IQ3_S ? resident_launch<21>(a, s, st) : resident_launch<22>(a, s, st);
 }
 
@@ -847,7 +865,7 @@ extern "C" int wd_moe_stack_f32(const wd_moe_layer *layers, int n_layers, float 
     SiteScope site(WD_SITE_STACK_TOTAL, as_stream(stream));
     if (resident_shape(layers, n_layers, s, flags)) {
         const int rc = stack_resident(layers, n_layers, d_x, d_layer_out, s, d_ids_trace, residual_scale, as_stream(stream));
-        if (rc >= 0) return rc;
+        if (rc != kTakePerLayer) return rc;
     }
     flags &= ~WD_MOE_PER_LAYER;
     const unsigned only = flags & (WD_MOE_ONLY_A | WD_MOE_ONLY_B | WD_MOE_ONLY_C);
@@ -1031,7 +1049,10 @@ extern "C" int wd_moe_layer_tokens_pairs_f32(const wd_moe_layer *L, const uint8_
     s->pair_next = (slot + 1) % kPairRing;
     if (s->pair_used[slot]) WD_HIP(hipEventSynchronize(s->pair_done[slot]));  // the pass that read this entry of the ring has run
     const uint8_t **h = s->pair_host + static_cast<size_t>(slot) * 3 * kPairEntries, **d = s->pair_dev + static_cast<size_t>(slot) * 3 * kPairEntries;
-    for (int i = 0; i < n_entries; ++i) h[2 * i] = h_gate[i], h[2 * i + 1] = h_up[i], h[2 * kPairEntries + i] = h_down[i];
+    for (int i = 0; i < kPairEntries; ++i) {  // entries the caller did not give point at entry 0
+        const int from = i < n_entries ? i : 0;
+        h[2 * i] = h_gate[from], h[2 * i + 1] = h_up[from], h[2 * kPairEntries + i] = h_down[from];
+    }
     WD_HIP(hipMemcpyAsync(d, h, sizeof(void *) * 3 * kPairEntries, hipMemcpyHostToDevice, st));
     const int rc = tokens_pass(&Lt, d_x, d_out, tokens, scratch_per_token, flags, stream, d, d + 2 * kPairEntries, aligned);
     WD_HIP(hipEventRecord(s->pair_done[slot], st));

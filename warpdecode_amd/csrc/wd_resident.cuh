@@ -5,52 +5,57 @@
 //   * no launch lies between two dependent stages - values are handed from workgroup to workgroup through small
 //     buffers in global memory whose words say themselves whether they have been written (see below);
 //   * weights that do not depend on a value still being computed are already on the compute unit when that value
-//     arrives: the router row and the shared expert's rows of layer l + 1 are fetched during layer l, and the routed
-//     down rows are requested together with the routed gate/up rows, as soon as the expert ids are known.
+//     arrives: the router row and the shared expert's rows of layer l + 1 are fetched during layer l; the routed rows
+//     are requested the moment the expert ids are known - with a routing trace (the caller names the experts of every
+//     layer) that is when the layer begins, before its input exists.
 //
 // Geometry (the C2 layer shape): hidden 2048, expert ffn 512, at most 512 experts, top-k <= 10, IQ3_S or IQ2_S gate/up,
 // Q8_0 down, Q8_0 shared expert.  Workgroup r (0..511) has 12 waves:
-//   waves 0..9   routed rung j = wave: row r of gate and up of expert ids[j], then rows 4r..4r+3 of its down tensor
-//   wave 10      the shared expert: row r of its gate/up, rows 4r..4r+3 of its down tensor
-//   wave 11      router row r
-// and wave 0 folds the eleven results of rows 4r..4r+3 in the reference order and publishes these four values of the
-// next layer's input.  Workgroup 0 also selects the experts (its waves are idle until the ids exist anyway).
+//   ten routed rungs  rung j: row r of gate and up of the j-th selected expert, then rows 4r..4r+3 of its down tensor
+//   one wave          the shared expert: row r of its gate/up, rows 4r..4r+3 of its down tensor
+//   one wave          router row r, and the selection
+// and rung 0 folds the eleven results of rows 4r..4r+3 in the reference order and publishes these four values of the
+// next layer's input.
+// The selection.  Every workgroup selects for itself: its router wave pushes its logit into eight copies (one per group of
+// workgroups), gathers the 512 logits of its copy and finds the ids with sel_wave_ids (wd_fused.cuh) - the same logits
+// and the same code in every workgroup, hence the same ids - and hands them to the rungs through LDS.  No workgroup
+// waits for another one's selection, and the ids never cross the device.  Workgroup 0 goes on to the denominator and
+// the weights (sel_wave_finish), which only the fold at the end of the layer needs, and publishes them.  With a routing
+// trace only workgroup 0 gathers the logits (for the weights): the ids are inputs of the launch.
 // The float operations and their order are those of the per-layer kernels: results are bit-identical.
 //
 // Hand-off buffers.  Every layer of a launch has its own copy of each buffer, so no word is written twice during a
 // launch.  A word holds kResEmpty (0xffffffff) until its producer stores the value; consumers poll the data words
 // themselves with device-scope loads, so no flag, counter or ordering between stores is needed.  What a workgroup
-// hands on in a layer: its logit, in a 16-byte record that only workgroup 0 polls (64 lines for the 512 logits); its
-// eleven activations (48 bytes) and its four values of the next input (16 bytes), pushed into eight contiguous
-// copies, one per group of workgroups, each of which polls its own.  A line that many compute units write piece
-// by piece while the whole grid polls it changes hands once per write: thirty-two writers per line made a hand-off
-// take 17 us, hence pieces of 16 bytes or more.  (An f32 result with
-// that very bit pattern - a NaN that no arithmetic here produces by itself - would be taken for "not yet" and end in
-// a timeout.)  There are two sets of these buffers: a launch works in one and resets the other as it goes (the router
-// waves, which have time to spare), so nothing has to be cleaned up when a launch ends.  Waits are bounded: a wait that runs out sets status[0], after which
-// every wait in the grid ends at once and later launches return immediately until the scratch is reset.
+// hands on in a layer: its logit (a 16-byte record), its eleven activations (48 bytes) and its four values of the next
+// input (16 bytes), each pushed into eight contiguous copies, one per group of workgroups, each of which polls its own.
+// A line that many compute units write piece by piece while the whole grid polls it changes hands once per write:
+// thirty-two writers per line made a hand-off take 17 us, hence pieces of 16 bytes or more.  A value whose bits are
+// kResEmpty (one particular NaN) is stored as the default quiet NaN instead (hand_word): it would be taken for "not yet".
+// There are two sets of these buffers: a launch works in one and resets the other as it goes (the router waves, which
+// have time to spare), so nothing has to be cleaned up when a launch ends.  Waits are bounded: a wait that runs out sets
+// status[0] (and its mirror in host memory), after which every wait in the grid ends at once and later launches return
+// immediately until the scratch is reset.
 #pragma once
 
 #include "wd_fused.cuh"
 
 namespace wd {
 
-#ifndef WD_RES_SLEEP4
-#define WD_RES_SLEEP4 2
-#endif
-#ifndef WD_RES_XDELAY
-#define WD_RES_XDELAY 24
-#endif
-#ifndef WD_RES_SLEEP16
-#define WD_RES_SLEEP16 2
-#endif
 constexpr int kResMaxLayers = 64;
 constexpr int kResWgs = 512, kResWaves = 12, kResThreads = kResWaves * 64;
 constexpr int kResH = 2048, kResF = 512, kResMaxK = 10, kResSharedSlot = 10, kResActSlots = 11;
 constexpr uint32_t kResEmpty = 0xffffffffu;
-constexpr int kResIdCopies = 16;   // replicas of the published ids (pollers spread over lines)
 constexpr int kResXtRow = 68;      // floats per row of the transposed input in LDS (64 + bank spread)
 constexpr int kResGateSlot = 15;   // word of the weights record that holds the shared expert's sigmoid gate
+constexpr int kResSleepPoll = 2;   // s_sleep between two polls of a wait (flat from 1 to 8 in measurements)
+constexpr int kResSleepFold = 24;  // waves that reach a layer while rung 0 still folds the one before wait this long first
+
+// The bits a value is handed on with: kResEmpty means "not yet written", so that one NaN travels as the default quiet NaN.
+WD_DEV uint32_t hand_word(float v) {
+    const uint32_t b = f_bits(v);
+    return b == kResEmpty ? 0x7fc00000u : b;
+}
 
 struct ResidentLayer {
     const float *router;      // f32 [E][2048]
@@ -69,28 +74,22 @@ struct ResidentViews {
 };
 
 // Byte offsets inside the hand-off block.
-constexpr unsigned kHandRec = 0;          // [layers][512] records of kRecBytes, one per (layer, workgroup): word 0 the router
-// (Measured on one box: records of 128 / 64 / 32 / 16 bytes 0.869 / 0.861 / 0.856 / 0.851 ms per token - workgroup 0 polls
-// 64 lines instead of 512; the gate logit moved into the line of the router weights, which every workgroup polls, costs
-// 1.2 % again, and records of 8 bytes are no better than 16.)
-constexpr unsigned kRecBytes = 16;        //   logit of row r, word 1 the shared expert's gate logit (workgroup 1 only)
-static_assert(kRecBytes % 16 == 0 && kRecBytes <= 128, "records are reset in 16-byte pieces by eight lanes");
-// What every workgroup needs from every other - four values of the next input, eleven activations - is written by its
-// producer into kResCopies copies, one per group of workgroups (r % kResCopies; on this device the workgroups of a group
-// share an L2), laid out contiguously: the consumers of a group fetch their copy with coalesced requests, and a line is
-// polled from one L2 only.
+// What every workgroup needs from every other - four values of the next input, eleven activations - is
+// written by its producer into kResCopies copies, one per group of workgroups (r % kResCopies; on this device the
+// workgroups of a group share an L2), laid out contiguously: the consumers of a group fetch their copy with coalesced
+// requests, and a line is polled from one L2 only.
 constexpr int kResCopies = 8;
-#ifndef WD_RES_XSTRIDE
-#define WD_RES_XSTRIDE 16
-#endif
-constexpr unsigned kXcStride = WD_RES_XSTRIDE;  // bytes from one workgroup's four values of a layer input to the next one's
+constexpr unsigned kRecBytes = 16;        // a logit record: word 0 the router logit of row r, word 1 (workgroup 1) the shared expert's gate logit
+constexpr unsigned kHandRec = 0;                                                        // [layers][512] records, gathered by workgroup 0 only
+constexpr unsigned kXcStride = 16;        // bytes from one workgroup's four values of a layer input to the next one's
 constexpr unsigned kXcBytes = kXcStride * kResWgs;                                     // one copy
-constexpr unsigned kHandXc = kHandRec + kRecBytes * kResMaxLayers * kResWgs;           // [layers][copies][512] pieces of four f32: layer inputs
+constexpr unsigned kHandXc = kHandRec + kRecBytes * kResWgs * kResMaxLayers;            // [layers][copies][512] pieces of four f32: layer inputs
 constexpr unsigned kAcRec = 48;                                                        // bytes of a workgroup's activations: slots 0..10, a zero
 constexpr unsigned kAcBytes = kAcRec * kResWgs;                                        // 24 KB per copy
-constexpr unsigned kHandAc = kHandXc + kXcBytes * kResMaxLayers * kResCopies;        // f32 [layers][copies][512][12] activations
-constexpr unsigned kHandIdh = kHandAc + kAcBytes * kResMaxLayers * kResCopies;         // u32 [layers][copies][16] selected ids
-constexpr unsigned kHandWh = kHandIdh + 4u * kResMaxLayers * kResIdCopies * 16;  // u32 [layers][16] router weights, [15] the shared gate
+constexpr unsigned kHandAc = kHandXc + kXcBytes * kResMaxLayers * kResCopies;          // f32 [layers][copies][512][12] activations
+constexpr int kResIdCopies = 16;          // replicas of the published ids (pollers spread over lines)
+constexpr unsigned kHandIdh = kHandAc + kAcBytes * kResMaxLayers * kResCopies;         // u32 [layers][replicas][16] selected ids
+constexpr unsigned kHandWh = kHandIdh + 4u * kResMaxLayers * kResIdCopies * 16;        // u32 [layers][16] router weights, [15] the shared gate
 constexpr unsigned kHandSet = kHandWh + 4u * kResMaxLayers * 16;             // bytes of one set of hand-off buffers
 // The block holds two such sets and the number of launches finished.  Launch e works in set e % 2 and, layer by layer and
 // off its critical path, puts set (e + 1) % 2 back to "not yet written": no launch has to clean up behind itself.
@@ -109,17 +108,14 @@ struct ResidentArgs {
     float *x;                     // [2048] in: input of the first layer; out: input of the layer after the last
     float *out;                   // [2048] output of the last layer
     float residual_scale;
-    const int32_t *ids_trace;     // null, or [n_layers][k]: ids that replace the selected ones (the weights stay the router's)
+    const int32_t *ids_trace;     // null, or [n_layers][k]: the experts of every layer (the weights stay the router's)
     const struct ResidentViews *views;  // device: where the last layer's values go
     uint8_t *hand;   // the hand-off block (kHand* offsets below)
     unsigned *status;
+    unsigned *status_host;        // null, or the status word's mirror in pinned host memory (the host reads it without a synchronisation)
     unsigned spin_limit;
     unsigned long long *trace;  // null, or [12][16] time stamps (100 MHz) of workgroup trace_wg in layer trace_layer
     int trace_wg, trace_layer;
-    int debug;  // experiments: 1 no gate/up decode, 2 no weight loads, 4 no wait for the activations, 8 no down dots.
-                // (The tests of these bits stay in the kernel on purpose: as branches around the weight requests and the
-                // dot products they keep the compiler from moving these against each other - the down rows' request in
-                // particular must follow the gate/up rows' arrival -, and the kernel measured 5 % slower without them.)
 };
 
 // ---- device-scope access to the hand-off buffers ------------------------------------------------------------
@@ -151,6 +147,7 @@ WD_DEV bool res_give_up(const ResidentArgs &a, unsigned &spins, bool &dead) {
     ++spins;
     if (spins >= a.spin_limit) {
         __hip_atomic_store(a.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (a.status_host) __hip_atomic_store(a.status_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
         dead = true;
     } else if ((spins & 63u) == 0u && __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
         dead = true;
@@ -160,105 +157,14 @@ WD_DEV bool res_give_up(const ResidentArgs &a, unsigned &spins, bool &dead) {
 WD_DEV bool res_full(const uint4 &v) { return v.x != kResEmpty && v.y != kResEmpty && v.z != kResEmpty && v.w != kResEmpty; }
 
 // N 16-byte pieces per lane (lanes with on == false take no part): returns when every word of every piece has been
-// written.  Only pieces that are still incomplete are requested again.
-// WD_RES_PIPE16 / WD_RES_PIPE4 > 1: that many polls are kept in flight.  A poll that has to travel to memory and back
-// before the next one is issued notices a value up to one round trip late; several polls under way notice it within the
-// interval at which they were issued.
-#ifndef WD_RES_DOWN_AT
-#define WD_RES_DOWN_AT 0  // the down rows are requested 0: when the gate/up rows have arrived, 1: after the decode, 2: after the exchange
-#endif
-#ifndef WD_RES_PIPE16
-#define WD_RES_PIPE16 1
-#endif
-#ifndef WD_RES_PIPE4
-#define WD_RES_PIPE4 1
-#endif
-#ifndef WD_RES_PIPE16_MAXN
-#define WD_RES_PIPE16_MAXN 1
-#endif
-template <int N, int D>
-WD_DEV void hand_wait16_piped(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, const unsigned (&off)[N], const bool (&on)[N], uint4 (&v)[N], bool &dead) {
-    static_assert(D == 2, "two polls in flight");
-    bool need[N];
-    uint4 p0[N], p1[N];
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-        need[i] = on[i];
-        v[i] = p0[i] = p1[i] = make_uint4(0u, 0u, 0u, 0u);
-    }
-    if (dead) return;
-    auto issue = [&](uint4 (&p)[N]) {
-#pragma unroll
-        for (int i = 0; i < N; ++i)
-            if (need[i]) p[i] = hand_load16(rs, off[i]);
-    };
-    auto arrived = [&](const uint4 (&p)[N]) {  // true when nothing is missing any more (or the wait is given up)
-        bool any = false;
-#pragma unroll
-        for (int i = 0; i < N; ++i) {
-            if (need[i]) {
-                v[i] = p[i];
-                need[i] = !res_full(v[i]);
-            }
-            any = any || need[i];
-        }
-        return __builtin_amdgcn_ballot_w64(any) == 0ull;
-    };
-    issue(p0);
-    __builtin_amdgcn_s_sleep(WD_RES_SLEEP16);
-    issue(p1);
-    unsigned spins = 0;
-    for (;;) {
-        if (arrived(p0) || res_give_up(a, spins, dead)) return;
-        issue(p0);
-        __builtin_amdgcn_s_sleep(WD_RES_SLEEP16);
-        if (arrived(p1) || res_give_up(a, spins, dead)) return;
-        issue(p1);
-        __builtin_amdgcn_s_sleep(WD_RES_SLEEP16);
-    }
-}
-template <int D>
-WD_DEV uint32_t hand_wait4_piped(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, unsigned off, bool on, bool &dead) {
-    uint32_t v = 0u;
-    if (dead) return v;
-    bool need = on;
-    uint32_t s[D];
-#pragma unroll
-    for (int d = 0; d < D; ++d) {
-        s[d] = 0u;
-        if (need) s[d] = hand_load4(rs, off);
-        if (d + 1 < D) __builtin_amdgcn_s_sleep(WD_RES_SLEEP4);
-    }
-    unsigned spins = 0;
-    bool done = false;
-    while (!done) {
-#pragma unroll
-        for (int d = 0; d < D; ++d) {
-            if (!done) {
-                if (need) {
-                    v = s[d];
-                    need = v == kResEmpty;
-                }
-                done = __builtin_amdgcn_ballot_w64(need) == 0ull || res_give_up(a, spins, dead);
-                if (!done) {
-                    if (need) s[d] = hand_load4(rs, off);
-                    __builtin_amdgcn_s_sleep(WD_RES_SLEEP4);
-                }
-            }
-        }
-    }
-    return v;
-}
+// written.  Only pieces that are still incomplete are requested again, one poll at a time: two or three polls in flight
+// measured slower (more device-scope loads compete with the stores they wait for).
 template <int N>
-WD_DEV void hand_wait16(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, const unsigned (&off)[N], const bool (&on)[N], uint4 (&v)[N], bool &dead) {
-    if constexpr (WD_RES_PIPE16 > 1 && N <= WD_RES_PIPE16_MAXN) {
-        hand_wait16_piped<N, WD_RES_PIPE16>(a, rs, off, on, v, dead);
-        return;
-    }
+WD_DEV void hand_wait16(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, const unsigned (&off)[N], bool on, uint4 (&v)[N], bool &dead) {
     bool need[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-        need[i] = on[i];
+        need[i] = on;
         v[i] = make_uint4(0u, 0u, 0u, 0u);
     }
     if (dead) return;
@@ -275,30 +181,46 @@ WD_DEV void hand_wait16(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, const 
         }
         if (__builtin_amdgcn_ballot_w64(any) == 0ull) return;
         if (res_give_up(a, spins, dead)) return;
-        __builtin_amdgcn_s_sleep(WD_RES_SLEEP16);
+        __builtin_amdgcn_s_sleep(kResSleepPoll);
+    }
+}
+// N words per lane, word i at off + i * stride (words with on[i] == false take no part; they read as zero).
+// stop(): looked at after every unsuccessful round; true ends the wait early.  Returns whether every word has arrived.
+template <int N, typename Stop>
+WD_DEV bool hand_wait4(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, unsigned off, unsigned stride, const bool (&on)[N], uint32_t (&v)[N], bool &dead, Stop &&stop) {
+    bool need[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        need[i] = on[i];
+        v[i] = 0u;
+    }
+    if (dead) return false;
+    unsigned spins = 0;
+    for (;;) {
+        bool any = false;
+#pragma unroll
+        for (int i = 0; i < N; ++i)
+            if (need[i]) v[i] = hand_load4(rs, off + static_cast<unsigned>(i) * stride);
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            need[i] = need[i] && v[i] == kResEmpty;
+            any = any || need[i];
+        }
+        if (__builtin_amdgcn_ballot_w64(any) == 0ull) return true;
+        if (stop() || res_give_up(a, spins, dead)) return false;
+        __builtin_amdgcn_s_sleep(kResSleepPoll);
     }
 }
 template <int N>
-WD_DEV void hand_wait16(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, const unsigned (&off)[N], bool on, uint4 (&v)[N], bool &dead) {
-    bool each[N];
-#pragma unroll
-    for (int i = 0; i < N; ++i) each[i] = on;
-    hand_wait16<N>(a, rs, off, each, v, dead);
+WD_DEV void hand_wait4(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, unsigned off, unsigned stride, const bool (&on)[N], uint32_t (&v)[N], bool &dead) {
+    (void)hand_wait4<N>(a, rs, off, stride, on, v, dead, [] { return false; });
 }
 // One word per lane.
 WD_DEV uint32_t hand_wait4(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, unsigned off, bool on, bool &dead) {
-    if constexpr (WD_RES_PIPE4 > 1) return hand_wait4_piped<WD_RES_PIPE4>(a, rs, off, on, dead);
-    uint32_t v = 0u;
-    if (dead) return v;
-    bool need = on;
-    unsigned spins = 0;
-    for (;;) {
-        if (need) v = hand_load4(rs, off);
-        need = need && v == kResEmpty;
-        if (__builtin_amdgcn_ballot_w64(need) == 0ull) return v;
-        if (res_give_up(a, spins, dead)) return v;
-        __builtin_amdgcn_s_sleep(WD_RES_SLEEP4);
-    }
+    const bool each[1] = {on};
+    uint32_t v[1];
+    hand_wait4<1>(a, rs, off, 0u, each, v, dead);
+    return v[0];
 }
 
 // ---- router row of 2048 columns, weights fetched ahead --------------------------------------------------------
@@ -359,7 +281,7 @@ constexpr int kResWaveBytes = kResTileBytes + kResF + 64;
 constexpr int kResLdsY = kResLdsWave + kResActSlots * kResWaveBytes;  // f32 [11][4] down results
 constexpr int kResLdsSel = kResLdsY + 4 * 4 * kResActSlots;           // selection scratch, then ids [16], weights [16]
 constexpr int kResLdsRoles = kResLdsSel + kTopkLdsBytes1 + 128;       // int [12] SIMD of every wave
-constexpr int kResLdsActv = kResLdsRoles + 64;                        // f32 [12] this workgroup's activations (word 11 zero)
+constexpr int kResLdsActv = kResLdsRoles + 64;                        // f32 [12] this workgroup's activations (word 11 zero), u32 [1] arrivals
 constexpr int kResLdsBytes = kResLdsActv + 64;
 constexpr int kResLdsLand = kResLdsWave;  // f32 [11][512] all activations of the layer, while no slot area is in use
 static_assert(kResLdsXq % 16 == 0 && kResLdsTables % 16 == 0 && kResLdsWave % 16 == 0 && kResWaveBytes % 16 == 0 && kResLdsSel % 16 == 0, "LDS alignment");
@@ -393,6 +315,8 @@ struct ResCtx {
     WD_DEV uint8_t *area() const { return lds + kResLdsWave + slot * kResWaveBytes; }
     WD_DEV float *ybuf() const { return reinterpret_cast<float *>(lds + kResLdsY); }
     WD_DEV float *actv() const { return reinterpret_cast<float *>(lds + kResLdsActv); }
+    // how many waves have handed in their activation of a layer, summed over the layers so far (every wave but the router's: 11 per layer)
+    WD_DEV unsigned *arrived() const { return reinterpret_cast<unsigned *>(lds + kResLdsActv + 48); }
     WD_DEV float *land() const { return reinterpret_cast<float *>(lds + kResLdsLand); }
 };
 // The context of one layer: the indices made opaque (see fresh_v); `base` is the workgroup's dynamic LDS.
@@ -422,19 +346,36 @@ WD_DEV T *res_field(T *const *field) {
     return uniform_ptr(*const_cast<T *const volatile *>(field));
 }
 
-// Between the gate/up rows and the down rows of a layer (every wave of the workgroup calls it; `mine`: this wave's
-// activation, for routed rungs in use and the shared expert).  The workgroup's eleven activations go out as one store
-// of its record; waves 0..7 then wait for the records of all 512 workgroups and lay the values out in LDS by slot;
-// v0, v1 receive values 8 lane .. 8 lane + 7 of this wave's slot.
-template <bool STAMPS>
-WD_DEV void res_exchange(const ResidentArgs &a, const ResCtx &c, int l, bool has, float mine, float4 &v0, float4 &v1, bool &dead) {
+// The same through the scalar path (the descriptors are written before the launch): the value is wave-uniform, costs no
+// vector register and no vector-memory wait, and is there long before the request that needs it.
+template <typename T>
+WD_DEV T *res_field_s(T *const *field) {
+    const uintptr_t at = reinterpret_cast<uintptr_t>(field);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(at));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(at >> 32));
+    const uint64_t v = *((const __attribute__((address_space(4))) uint64_t *)((static_cast<uintptr_t>(hi) << 32) | lo));
+    return reinterpret_cast<T *>(static_cast<uintptr_t>(v));
+}
+
+// Between the gate/up rows and the down rows of a layer (every wave of the workgroup calls it, the router wave through its
+// own three barriers; `mine`: this wave's activation, for routed rungs in use and the shared expert).  The workgroup's
+// eleven activations go out as one store of its record; waves 0..7 then wait for the records of all 512 workgroups and
+// lay the values out in LDS by slot; v0, v1 receive values 8 lane .. 8 lane + 7 of this wave's slot.
+// before(): work between handing in the activation and the barrier; meanwhile(): work for a wave that does not gather
+// (waves 8..11) while the others wait for the records.
+template <bool STAMPS, typename Before, typename Meanwhile>
+WD_DEV void res_exchange(const ResidentArgs &a, const ResCtx &c, int l, bool has, float mine, float4 &v0, float4 &v1, bool &dead, Before &&before, Meanwhile &&meanwhile) {
     const int lane = c.lane, wave = c.wave;
-    if (has && lane == 0) c.actv()[c.slot] = mine;
+    if (lane == 0) {
+        if (has) c.actv()[c.slot] = mine;
+        __hip_atomic_fetch_add(c.arrived(), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    before();
     __syncthreads();  // B2: the workgroup's activations are in LDS, and no slot area is in use any more
     if (wave == 0 && lane < 3 * kResCopies) {  // piece lane % 3 of the workgroup's 48 bytes, to copy lane / 3
         const int piece = lane % 3, copy = lane / 3;
         const float4 p = reinterpret_cast<const float4 *>(c.actv())[piece];
-        hand_store16(c.hb, ac_off(l, copy) + kAcRec * c.r + 16u * piece, make_uint4(f_bits(p.x), f_bits(p.y), f_bits(p.z), f_bits(p.w)));
+        hand_store16(c.hb, ac_off(l, copy) + kAcRec * c.r + 16u * piece, make_uint4(hand_word(p.x), hand_word(p.y), hand_word(p.z), hand_word(p.w)));
     }
     if (wave < 8) {  // the group's copy, three 16-byte words per lane: word w is piece w % 3 of workgroup w / 3
         const int i = wave * 64 + lane;
@@ -449,6 +390,8 @@ WD_DEV void res_exchange(const ResidentArgs &a, const ResCtx &c, int l, bool has
             land[0] = bits_f(v[t].x), land[512] = bits_f(v[t].y), land[1024] = bits_f(v[t].z);
             if (piece < 2) land[1536] = bits_f(v[t].w);
         }
+    } else {
+        meanwhile();
     }
     __syncthreads();  // B3: every activation of the layer is in LDS
     res_mark<STAMPS>(a, c, l, 6);
@@ -468,28 +411,54 @@ WD_DEV void res_down(const ResidentArgs &a, const ResCtx &c, int l, const Q8Coal
     int8_t *aq = reinterpret_cast<int8_t *>(area + kResTileBytes);
     uint16_t *ad = reinterpret_cast<uint16_t *>(area + kResTileBytes + kResF);
     lds_quantize_q8_0_step(v0, v1, true, lane * 8, aq, ad, lane);
-    float y = 1.0f;
-    if (!(a.debug & 8)) y = q8_rows4_coal_finish<0, 16>(draw, aq, ad, *reinterpret_cast<Q8TileNB<16> *>(area), lane);
+    const float y = q8_rows4_coal_finish<0, 16>(draw, aq, ad, *reinterpret_cast<Q8TileNB<16> *>(area), lane);
     if ((lane & 15) == 0) c.ybuf()[c.slot * 4 + (lane >> 4)] = y;
     res_mark<STAMPS>(a, c, l, 7);
 }
 
 // ---- the ten routed waves -------------------------------------------------------------------------------------
-// Waves 0..7 (always rungs 0..7) also fetch and quantise the layer's input, and in workgroup 0 select the experts.
+// Rungs 0..7 (always waves 0..7) also fetch and quantise the layer's input.
+// Barriers of a layer, the same for every wave of the workgroup: B1 (input in LDS), B2..B4 (exchange of the
+// activations), B5 (down results in LDS).
 template <int TYPE, bool STAMPS>
 WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, int lane0, int wave0, int slot0,
-                            __amdgpu_buffer_rsrc_t hb, unsigned set_base, bool &dead) {
+                            __amdgpu_buffer_rsrc_t hb, bool &dead) {
     constexpr int kRow = 8 * ((TYPE == 21) ? 110 : 82);
     const bool shared = a.shared != 0;
+    const bool traced = a.ids_trace != nullptr;
+    auto expert_in_range = [&](uint32_t e) { return e < static_cast<uint32_t>(a.E) ? e : 0u; };  // (out of range: a wrong trace, or a wait that ran out)
+    // the expert of this rung in layer l according to the routing trace (any layer number: past the end it is the last layer's)
+    auto traced_expert = [&](int l, int rung) {
+        return expert_in_range(static_cast<uint32_t>(sld_i32(a.ids_trace + (l < a.n_layers ? l : a.n_layers - 1) * a.k + rung)));
+    };
+    auto gate_up_rows = [&](const uint8_t *gate_base, const uint8_t *up_base, uint32_t e, int r, int lane) {
+        const uint8_t *const rows[2] = {gate_base + e * a.gate_stride + static_cast<size_t>(r) * kRow,
+                                        up_base + e * a.up_stride + static_cast<size_t>(r) * kRow};
+        return iq_rows8_coal_request<TYPE, 2>(rows, lane);
+    };
+    // With a routing trace the gate/up rows of a layer are requested while the layer before decodes its own (the
+    // registers they arrive in are free from the moment the rows before them lie in LDS), those of the first layer here.
+    IqRows8Raw<TYPE, 2> raw;
+    raw.u[0] = raw.u[1] = make_uint4(0u, 0u, 0u, 0u);
+    if (traced && slot0 < a.k) raw = gate_up_rows(res_field_s(&a.layers->gate), res_field_s(&a.layers->up), traced_expert(0, slot0), r0, lane0);
     for (int l = 0; l < a.n_layers; ++l) {
         const ResCtx c = res_ctx(lds_base, r0, lane0, wave0, slot0, hb);
         const int r = c.r, lane = c.lane, wave = c.wave, rung = c.slot;
         const IqTables &tables = *reinterpret_cast<const IqTables *>(c.lds + kResLdsTables);
         const ResidentLayer *L = a.layers + l;
         const bool last = l == a.n_layers - 1;
-        const bool gate_row = shared && r == 1 && rung == 9;  // the shared expert's gate logit: one more row of the router's kind
-        // ---- the layer's input: 16 bytes per lane of waves 0..7, quantised from the registers they arrive in
+        const bool on = rung < a.k;
         res_mark<STAMPS>(a, c, l, 0);
+        Q8CoalRaw<0, 16> draw;
+        draw.u[0] = draw.u[1] = draw.u[2] = make_uint4(0u, 0u, 0u, 0u);
+        // what the requests below are made of, asked for now (scalar loads): the tensors of this layer and, with a routing
+        // trace, the gate/up tensors and the expert of the next one
+        const ResidentLayer *const Ln = a.layers + (last ? l : l + 1);
+        const uint8_t *const down_base = res_field_s(&L->down);
+        const uint8_t *const gate_base = res_field_s(traced ? &Ln->gate : &L->gate), *const up_base = res_field_s(traced ? &Ln->up : &L->up);
+        uint32_t e = 0, e_next = 0;
+        if (traced && on) e = traced_expert(l, rung), e_next = traced_expert(l + 1, rung);
+        // ---- the layer's input: 16 bytes per lane of waves 0..7, quantised from the registers they arrive in
         if (wave < 8) {
             const int i = wave * 64 + lane;
             float4 xv;
@@ -498,7 +467,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             } else {
                 // (the other waves of the workgroup come here while rung 0 still folds the previous layer: nothing
                 // can have arrived yet)
-                if (rung != 0 && WD_RES_XDELAY) __builtin_amdgcn_s_sleep(WD_RES_XDELAY);
+                if (rung != 0) __builtin_amdgcn_s_sleep(kResSleepFold);
                 const unsigned off[1] = {xc_off(l, r & (kResCopies - 1)) + kXcStride * i};
                 uint4 v[1];
                 hand_wait16<1>(a, c.hb, off, true, v, dead);
@@ -522,94 +491,29 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         __syncthreads();  // B1: x and its quantised forms are in LDS
         res_mark<STAMPS>(a, c, l, 2);
         const float res_pre = c.x_at(4 * r + (lane & 3));  // (rung 0 adds the layer's output to these)
-        // this layer's routed tensors (the wave has nothing else to do until the ids appear)
-        const uint8_t *const gate_base = res_field(&L->gate), *const up_base = res_field(&L->up), *const down_base = res_field(&L->down);
-
-        if (gate_row) {  // (needed by the combine only: its weights are requested now)
-            float gw[32];
-            res_router_fetch(res_field(&L->sh_inp), gw, lane);
-            const float s = res_router_dot(gw, c.xt(), lane);
-            if (lane == 32) hand_store4(c.hb, rec_off(l, 1) + 4u, f_bits(s));
+        if (!traced && on) {  // the id this rung works on, from one of the replicas workgroup 0 publishes
+            e = hand_wait4(a, c.hb, kHandIdh + static_cast<unsigned>(((l * kResIdCopies + (r & (kResIdCopies - 1))) * 16 + rung) * 4), true, dead);
+            e = expert_in_range(static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(e)));
+            raw = gate_up_rows(gate_base, up_base, e, r, lane);
         }
-
-        // ---- selection (workgroup 0): waves 0..7 hold one logit per lane
-        if (r == 0) {
-            uint8_t *sel = c.lds + kResLdsSel;
-            int32_t *lds_ids = reinterpret_cast<int32_t *>(sel + kTopkLdsBytes1);
-            float *lds_w = reinterpret_cast<float *>(sel + kTopkLdsBytes1 + 64);
-            const TopkLds<1> s(sel);
-            const int32_t *ids_given = a.ids_trace ? a.ids_trace + l * a.k : nullptr;
-            int id_given = 0;
-            if (ids_given && wave == 0 && lane < a.k) id_given = ids_given[lane];
-            const float w_scale = *const_cast<const volatile float *>(&L->w_scale);  // (asked for ahead of the logits)
-            float lv[1] = {-INFINITY};
-            const int id = wave * 64 + lane;
-            if (wave < 8) {
-                const uint32_t b = hand_wait4(a, c.hb, rec_off(l, id), id < a.E, dead);
-                if (id < a.E) lv[0] = bits_f(b);
-                res_mark<STAMPS>(a, c, l, 3);
-                topk_block_step1<1>(lv, s, lane, wave);
-            }
-            __syncthreads();
-            res_mark<STAMPS>(a, c, l, 12);
-            if (wave < 8) topk_block_step2<1>(lv, a.E, a.k, s, lane, wave);
-            __syncthreads();
-            res_mark<STAMPS>(a, c, l, 13);
-            if (wave == 0) {
-#ifdef WD_RES_SEL_STAMPS
-                unsigned long long *st3 = (STAMPS && a.trace && l == a.trace_layer && a.trace_wg == 0) ? a.trace + 11 * 16 + 5 : nullptr;
-#else
-                unsigned long long *st3 = nullptr;
-#endif
-                topk_block_step3<1>(a.E, a.k, w_scale, lds_ids, lds_w, ids_given != nullptr, id_given, s, lane, st3,
-                                    reinterpret_cast<uint32_t *>(a.hand + set_base + kHandIdh) + static_cast<size_t>(l) * kResIdCopies * 16, kResIdCopies);
-                res_mark<STAMPS>(a, c, l, 14);
-                wave_lds_fence();
-                if (lane < a.k) {
-                    hand_store4(c.hb, kHandWh + static_cast<unsigned>((l * 16 + lane) * 4), f_bits(lds_w[lane]));
-                    if (last) {
-                        a.views->ids[lane] = lds_ids[lane];
-                        a.views->weights[lane] = lds_w[lane];
-                    }
-                }
-            }
-            if (last && wave < 8 && id < a.E) a.views->logits[id] = lv[0];
-        }
+        res_mark<STAMPS>(a, c, l, 4);
 
         // ---- routed rung: gate/up row r, then down rows 4r..4r+3
-        const bool on = rung < a.k;
-        Q8CoalRaw<0, 16> draw;
-        draw.u[0] = draw.u[1] = draw.u[2] = make_uint4(0u, 0u, 0u, 0u);
         float act = 0.0f;
-#if WD_RES_DOWN_AT != 0
-        uint32_t e_keep = 0;
-#endif
         if (on) {
-            uint32_t e = hand_wait4(a, c.hb, kHandIdh + static_cast<unsigned>(((l * kResIdCopies + (r & (kResIdCopies - 1))) * 16 + rung) * 4), true, dead);
-            e = __builtin_amdgcn_readfirstlane(e);
-            if (e >= static_cast<uint32_t>(a.E)) e = 0;  // only after a wait that ran out (status is set)
-            res_mark<STAMPS>(a, c, l, 4);
-            const uint8_t *const rows[2] = {gate_base + e * a.gate_stride + static_cast<size_t>(r) * kRow,
-                                            up_base + e * a.up_stride + static_cast<size_t>(r) * kRow};
-            IqRows8Raw<TYPE, 2> raw;
-            raw.u[0] = raw.u[1] = make_uint4(0u, 0u, 0u, 0u);
-            if (!(a.debug & 2)) raw = iq_rows8_coal_request<TYPE, 2>(rows, lane);
             float gu[2] = {1.0f, 1.0f};
             iq_rows8_coal_park<TYPE, 2>(raw, lane, c.area());
-            // the down rows are asked for once the gate/up rows are here: requested together, the down rows of the
-            // waves served first would delay the gate/up rows of the others, which the whole grid waits for
-#if WD_RES_DOWN_AT == 0
-            if (!(a.debug & 2)) draw = q8_rows4_coal_request<0, 16>(down_base + e * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
-#else
-            e_keep = e;
-#endif
+            // Nothing below may be requested before the gate/up rows are here (the wave's loads return in order, and
+            // requested together, the down rows of the waves served first would delay the gate/up rows of the others,
+            // which the whole grid waits for): the expert's number passes through a statement the compiler cannot
+            // look into, so that the addresses below do not exist before this point.
+            asm volatile("" : "+s"(e) : : "memory");
+            draw = q8_rows4_coal_request<0, 16>(down_base + e * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
+            if (traced) raw = gate_up_rows(gate_base, up_base, e_next, r, lane);
             res_mark<STAMPS>(a, c, l, 11);
-            if (!(a.debug & 1)) iq_rows8_coal_dots<TYPE, 2>(tables, c.xq(), c.xd(), lane, gu, c.area());
+            iq_rows8_coal_dots<TYPE, 2>(tables, c.xq(), c.xd(), lane, gu, c.area());
             act = silu_ggml(gu[0]) * gu[1];
             res_mark<STAMPS>(a, c, l, 5);
-#if WD_RES_DOWN_AT == 1
-            draw = q8_rows4_coal_request<0, 16>(down_base + e_keep * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
-#endif
         }
         // rung 0 folds the results with the router's weights and the shared expert's gate: published long before this
         // point as a rule, so one request now, answered while the activations are exchanged, replaces a round trip
@@ -619,10 +523,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         uint32_t wbits = kResEmpty;
         if (wlane && !dead) wbits = hand_load4(c.hb, woff);
         float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
-        res_exchange<STAMPS>(a, c, l, on, act, v0, v1, dead);
-#if WD_RES_DOWN_AT == 2
-        if (on) draw = q8_rows4_coal_request<0, 16>(down_base + e_keep * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
-#endif
+        res_exchange<STAMPS>(a, c, l, on, act, v0, v1, dead, [] {}, [] {});
         if (on) res_down<STAMPS>(a, c, l, draw, v0, v1);
         float wreg = 0.0f;
         if (rung == 0) {
@@ -660,8 +561,8 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                     if (shared) a.views->down_f32[row] = ysh;
                 }
             } else {
-                const uint4 piece = make_uint4(f_bits(readlane_f(xn, 0)), f_bits(readlane_f(xn, 1)), f_bits(readlane_f(xn, 2)),
-                                               f_bits(readlane_f(xn, 3)));
+                const uint4 piece = make_uint4(hand_word(readlane_f(xn, 0)), hand_word(readlane_f(xn, 1)), hand_word(readlane_f(xn, 2)),
+                                               hand_word(readlane_f(xn, 3)));
                 if (lane < kResCopies) hand_store16(c.hb, xc_off(l + 1, lane) + kXcStride * r, piece);
             }
             res_mark<STAMPS>(a, c, l, 9);
@@ -680,15 +581,12 @@ WD_DEV void res_shared_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         gb[1] = q8_load<0>(res_field(&L->sh_up) + static_cast<size_t>(r) * (64 * 34) + lane * 34);
         draw = q8_rows4_coal_request<0, 16>(res_field(&L->sh_down) + static_cast<size_t>(r) * (4 * 16 * 34), lane);
     };
+    const bool traced = a.ids_trace != nullptr;
     if (a.shared) fetch(a.layers, r0, lane0);
     for (int l = 0; l < a.n_layers; ++l) {
         const ResCtx c = res_ctx(lds_base, r0, lane0, wave0, kResSharedSlot, hb);
         const int r = c.r, lane = c.lane;
         __syncthreads();  // B1
-        if (r == 0) {     // the selection's two barriers
-            __syncthreads();
-            __syncthreads();
-        }
         float act = 0.0f;
         if (a.shared) {
             res_mark<STAMPS>(a, c, l, 2);
@@ -699,8 +597,47 @@ WD_DEV void res_shared_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             act = silu_ggml(g) * u;
             res_mark<STAMPS>(a, c, l, 5);
         }
+        // Workgroup 0: this wave has time to spare where the router wave has none, so it takes the half of the selection
+        // that nobody waits for until the fold - every exponential of the row and the reference's 1/sum - and leaves it in
+        // LDS for the router wave.  Without a routing trace at once (the rungs are waiting for the ids anyway); with one,
+        // while the other waves wait for the activations: this workgroup's activations must not be late, so ahead of
+        // the barrier the wave only looks for the logits for as long as some other wave is still at work.
+        bool want[8];
+        float lv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) want[j] = 64 * j + lane < a.E, lv[j] = -INFINITY;
+        // all logits of the layer, eight per lane (expert 64 j + lane); patient == false: only until every other wave of the
+        // workgroup has handed in its activation.  True when they are all there.
+        auto gather_logits = [&](bool patient) {
+            uint32_t lb[8];
+            const unsigned all_in = 11u * static_cast<unsigned>(l + 1);
+            const bool got = hand_wait4<8>(a, c.hb, rec_off(l, lane), 64u * kRecBytes, want, lb, dead, [&] {
+                return !patient && __hip_atomic_load(c.arrived(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= all_in;
+            });
+#pragma unroll
+            for (int j = 0; j < 8; ++j) lv[j] = want[j] ? bits_f(lb[j]) : -INFINITY;
+            return got;
+        };
+        auto denominator = [&]() {
+            const TopkLds<1> scratch(c.lds + kResLdsSel);
+            bool dead_row;
+            const float inv = sel_wave_denominator(lv, a.E, scratch, lane, dead_row);
+            if (lane == 0) scratch.rest[0] = inv, scratch.rest[1] = dead_row ? 1.0f : 0.0f;
+        };
+        if (r == 0 && !traced) {
+            (void)gather_logits(true);
+            denominator();
+        }
+        bool got = false;
         float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
-        res_exchange<STAMPS>(a, c, l, a.shared != 0, act, v0, v1, dead);
+        res_exchange<STAMPS>(a, c, l, a.shared != 0, act, v0, v1, dead,
+            [&] { if (r == 0 && traced) got = gather_logits(false); },  // the logits ahead of the barrier, if that holds nobody up
+            [&] {
+                if (r == 0 && traced) {
+                    if (!got) (void)gather_logits(true);
+                    denominator();
+                }
+            });
         if (a.shared) res_down<STAMPS>(a, c, l, draw, v0, v1);
         __syncthreads();  // B5
         // the next layer's rows, asked for on this side of the barrier: the fold of this layer must not wait for a
@@ -709,52 +646,161 @@ WD_DEV void res_shared_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
     }
 }
 
-// ---- the router wave: row r --------------------------------------------------------------------------------------------
-// It also puts the other set of hand-off buffers (`ob`) back to "not yet written": in layer l this workgroup's share of
-// layers l, l + n, l + 2n, ... of that set (all kResMaxLayers layers, whatever the launch that wrote them used).
+// ---- the router wave: row r; in workgroup 0 the selection ----------------------------------------------------------------
+// Workgroup 0's router wave gathers the 512 logits and ranks them (sel_wave_ids, wd_fused.cuh); the workgroup's shared
+// expert's wave takes the denominator (sel_wave_denominator) and leaves it in LDS.  Without a routing trace the ids go
+// out to the rungs of every workgroup (kResIdCopies replicas) as soon as they are known, and the weights - which only
+// the fold at the end of the layer needs - follow behind the next barrier.  With a routing trace nobody waits for the
+// ids, and workgroup 0 must not hold up its own rungs: ranks and weights are then taken between the barriers of the
+// activation exchange, while the rungs wait for the activations.
+// The wave also puts the other set of hand-off buffers (`ob`) back to "not yet written": in layer l this workgroup's
+// share of layers l, l + n, l + 2n, ... of that set (all kResMaxLayers layers, whatever the launch that wrote them used).
 template <bool STAMPS>
 WD_DEV void res_router_role(const ResidentArgs &a, uint8_t *lds_base, int r0, int lane0, int wave0,
                             __amdgpu_buffer_rsrc_t hb, __amdgpu_buffer_rsrc_t ob, bool &dead) {
-    const bool on = r0 < a.E;
+    const bool has_row = r0 < a.E;
+    const bool traced = a.ids_trace != nullptr;
+#ifdef WD_RES_PRIO
+    __builtin_amdgcn_s_setprio(WD_RES_PRIO);
+#endif
+    // (a workgroup without a row keeps row 0 company: one definition of the row's registers per layer, no merge of an
+    // old and a new value - the compiler then holds them as 32 registers, not as one value of 32 that it copies whole)
     float wv[32];
-    if (on) res_router_fetch(res_field(&a.layers->router) + static_cast<size_t>(r0) * kResH, wv, lane0);
+    res_router_fetch(res_field(&a.layers->router) + static_cast<size_t>(has_row ? r0 : 0) * kResH, wv, lane0);
     for (int l = 0; l < a.n_layers; ++l) {
         const ResCtx c = res_ctx(lds_base, r0, lane0, wave0, -1, hb);
         const int r = c.r, lane = c.lane;
         const bool last = l == a.n_layers - 1;
+        const ResidentLayer *L = a.layers + l;
+        uint8_t *sel = c.lds + kResLdsSel;
+        int32_t *lds_ids = reinterpret_cast<int32_t *>(sel + kTopkLdsBytes1);
+        float *lds_w = reinterpret_cast<float *>(sel + kTopkLdsBytes1 + 64);
+        const TopkLds<1> scratch(sel);
+        // (both asked for ahead of the logits)
+        int id_given = 0;
+        if (traced && r == 0 && lane < a.k) id_given = a.ids_trace[l * a.k + lane];
+        const float w_scale = *const_cast<const volatile float *>(&L->w_scale);
         __syncthreads();  // B1
         res_mark<STAMPS>(a, c, l, 2);
-        if (on) {
+        {
             const float s = res_router_dot(wv, c.xt(), lane);
-            if (lane == 32) hand_store4(c.hb, rec_off(l, r), f_bits(s));
+            if (has_row && lane == 32) hand_store4(c.hb, rec_off(l, r), hand_word(s));
             res_mark<STAMPS>(a, c, l, 3);
-            if (!last) res_router_fetch(res_field(&a.layers[l + 1].router) + static_cast<size_t>(r) * kResH, wv, lane);
+        }
+        // (before the selection's values exist: this dot and they together would not fit the registers)
+        if (a.shared && r == 1) {  // the shared expert's gate logit: one more row of the router's kind (the fold needs it)
+            float gw[32];  // (an array of its own: the router row's registers keep one definition per layer)
+            res_router_fetch(res_field(&L->sh_inp), gw, lane);
+            const float s = res_router_dot(gw, c.xt(), lane);
+            if (lane == 32) hand_store4(c.hb, rec_off(l, 1) + 4u, hand_word(s));
+        }
+        bool want[8];
+        float lv[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) want[j] = 64 * j + lane < a.E, lv[j] = -INFINITY;
+        SelWaveState st;
+        st.mx = 0.0f, st.e = 0.0f, st.id = 0, st.fast = false;
+        // all logits of the layer, eight per lane (expert 64 j + lane); patient == false: only until every other wave of the
+        // workgroup has handed in its activation.  True when they are all there.
+        auto gather_logits = [&](bool patient) {
+            uint32_t lb[8];
+            const unsigned all_in = 11u * static_cast<unsigned>(l + 1);
+            const bool got = hand_wait4<8>(a, c.hb, rec_off(l, lane), 64u * kRecBytes, want, lb, dead, [&] {
+                return !patient && __hip_atomic_load(c.arrived(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= all_in;
+            });
+#pragma unroll
+            for (int j = 0; j < 8; ++j) lv[j] = want[j] ? bits_f(lb[j]) : -INFINITY;
+            if (got) res_mark<STAMPS>(a, c, l, 12);
+            return got;
+        };
+        // the ids to every rung of the grid: replica c, rung j at word c * 16 + j
+        auto publish_ids = [&]() {
+            wave_lds_fence();
+            const int j = lane & 15;
+#pragma unroll
+            for (int c0 = 0; c0 < kResIdCopies; c0 += 4)
+                if (j < a.k) hand_store4(c.hb, kHandIdh + static_cast<unsigned>(((l * kResIdCopies + c0 + (lane >> 4)) * 16 + j) * 4), static_cast<uint32_t>(lds_ids[j]));
+            res_mark<STAMPS>(a, c, l, 13);
+        };
+        // what every fold needs: the weights and the shared expert's gate; the last layer's values for the caller
+        auto publish_weights = [&]() {
+            wave_lds_fence();
+            if (lane < a.k) {
+                hand_store4(c.hb, kHandWh + static_cast<unsigned>((l * 16 + lane) * 4), hand_word(lds_w[lane]));
+                if (last) {
+                    a.views->ids[lane] = lds_ids[lane];
+                    a.views->weights[lane] = lds_w[lane];
+                }
+            }
+            if (last) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (want[j]) a.views->logits[64 * j + lane] = lv[j];
+            }
+            if (a.shared) {
+                const float g = bits_f(hand_wait4(a, c.hb, rec_off(l, 1) + 4u, true, dead));
+                const float sg = sigmoid_ggml(g);
+                if (lane == 0) {
+                    hand_store4(c.hb, kHandWh + static_cast<unsigned>((l * 16 + kResGateSlot) * 4), hand_word(sg));
+                    if (last) a.views->shared_gate[0] = sg;
+                }
+            }
+            res_mark<STAMPS>(a, c, l, 14);
+        };
+        // the weights from this wave's ranks and the 1/sum the shared expert's wave left in LDS (on the far side of a barrier)
+        auto weights_from_lds = [&]() {
+            const float inv = scratch.rest[0];
+            const bool dead_row = scratch.rest[1] != 0.0f;
+            sel_wave_weights(a.E, a.k, w_scale, scratch, lane, st, inv, dead_row, lds_ids, lds_w, traced, id_given);
+            publish_weights();
+        };
+        bool weights_out = false;
+        if (r == 0 && !traced) {
+            (void)gather_logits(true);
+            sel_wave_ids(lv, a.E, a.k, lane, st);
+            if (st.fast) {
+                if (lane < a.k) lds_ids[lane] = st.id;
+                publish_ids();
+            } else {
+                // the reference's rungs need every probability, and the rungs of the grid are waiting: no time for the
+                // other wave (which computes the very same values into the same places)
+                bool dead_row;
+                const float inv = sel_wave_denominator(lv, a.E, scratch, lane, dead_row);
+                sel_wave_weights(a.E, a.k, w_scale, scratch, lane, st, inv, dead_row, lds_ids, lds_w, false, 0);
+                publish_ids();
+                publish_weights();
+                weights_out = true;
+            }
         }
         for (int ll = l; ll < kResMaxLayers; ll += a.n_layers) {
             const uint4 empty4 = make_uint4(kResEmpty, kResEmpty, kResEmpty, kResEmpty);
-            // lane 0 the workgroup's record (of the first 8 lanes), 8 lanes its 128 bytes of the layer's input copies, 24 its 384 bytes of the activations'
-            const unsigned off = lane < 8 ? rec_off(ll, r) + 16u * lane
+            // lane 0 the workgroup's logit record, 8 lanes its 128 bytes of the layer's input copies, 24 its 384 bytes of the activations'
+            const unsigned off = lane < 8 ? rec_off(ll, r)
                                : lane < 16 ? xc_off(ll, 0) + kXcStride * (8 * r + lane - 8) : ac_off(ll, 0) + 16u * (24 * r + lane - 16);
-            if (lane < 8 ? lane < static_cast<int>(kRecBytes / 16) : lane < 40) hand_store16(ob, off, empty4);
+            if (lane == 0 || (lane >= 8 && lane < 40)) hand_store16(ob, off, empty4);
             if (r == 0) {
                 hand_store16(ob, kHandIdh + static_cast<unsigned>(ll * kResIdCopies * 64 + 16 * lane), empty4);
                 if (lane < 4) hand_store16(ob, kHandWh + static_cast<unsigned>(ll * 64 + 16 * lane), empty4);
             }
         }
-        if (r == 0) {
-            __syncthreads();
-            __syncthreads();
-            if (a.shared) {  // the shared expert's gate
-                const float g = bits_f(hand_wait4(a, c.hb, rec_off(l, 1) + 4u, true, dead));
-                const float sg = sigmoid_ggml(g);
-                if (lane == 0) {
-                    hand_store4(c.hb, kHandWh + static_cast<unsigned>((l * 16 + kResGateSlot) * 4), f_bits(sg));
-                    if (last) a.views->shared_gate[0] = sg;
-                }
-            }
+        // The exchange of the activations: this wave (never one of waves 0..7) only keeps its three barriers company.
+        // With a routing trace nobody waits for the ranks before the fold: they are taken while the activations travel;
+        // the logits are gathered ahead of the barrier if that holds nobody up.
+        bool got = false;
+        if (r == 0 && traced) got = gather_logits(false);
+        __syncthreads();  // B2
+        if (r == 0 && !traced && !weights_out) weights_from_lds();
+        if (r == 0 && traced) {
+            if (!got) (void)gather_logits(true);
+            sel_wave_ids(lv, a.E, a.k, lane, st);
+            res_mark<STAMPS>(a, c, l, 13);
         }
-        float4 v0, v1;
-        res_exchange<STAMPS>(a, c, l, false, 0.0f, v0, v1, dead);
+        __syncthreads();  // B3
+        __syncthreads();  // B4
+        if (r == 0 && traced) weights_from_lds();
+        // the next layer's row: requested behind the selection, so that its registers are not held while the selection runs,
+        // and behind the exchange, whose polls it would delay
+        res_router_fetch(res_field(&a.layers[last ? l : l + 1].router) + static_cast<size_t>(has_row ? r : 0) * kResH, wv, lane);
         __syncthreads();  // B5
     }
 }
@@ -807,13 +853,16 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 
         slot = __builtin_amdgcn_readfirstlane(slot);
     }
 
+#ifdef WD_RES_PRIO_WG0
+    if (r == 0) __builtin_amdgcn_s_setprio(WD_RES_PRIO_WG0);
+#endif
     bool dead = false;
     if (slot < 0)
         res_router_role<STAMPS>(a, lds_res, r, lane, wave, hb, ob, dead);
     else if (slot == kResSharedSlot)
         res_shared_role<STAMPS>(a, lds_res, r, lane, wave, hb, dead);
     else
-        res_routed_role<TYPE, STAMPS>(a, lds_res, r, lane, wave, slot, hb, set_base, dead);
+        res_routed_role<TYPE, STAMPS>(a, lds_res, r, lane, wave, slot, hb, dead);
 
     // the next launch takes the other set (workgroup 0 can only get here after every workgroup has read the number)
     if (r == 0 && threadIdx.x == 0 && !dead)

@@ -18,11 +18,15 @@ namespace wd {
 
 constexpr int kMaxTokens = 8;
 
+constexpr int kPairEntries = 128;  // entries of a pointer table (wd_moe_layer_tokens_pairs_f32)
+
 // Tensor T of "expert" e when the pass was given a table of pointers instead of tensors that hold every expert: e is
-// then an index into the table ([entry][tensors per entry]).
+// then an index into the table ([entry][tensors per entry]).  The host fills every one of the kPairEntries entries
+// (those past the caller's with entry 0), and a number outside the table reads entry 0: a wrong id in the scratch gives
+// a wrong result, never a load through a pointer nobody set.
 template <int T>
 WD_DEV const uint8_t *mat_ptr_entry(const MatSrc &s, int e) {
-    if (s.table) return s.table[e * s.per_expert + T];
+    if (s.table) return s.table[(static_cast<unsigned>(e) < static_cast<unsigned>(kPairEntries) ? e : 0) * s.per_expert + T];
     return mat_ptr_expert<T>(s, e);
 }
 
