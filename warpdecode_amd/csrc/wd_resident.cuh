@@ -50,6 +50,7 @@ constexpr int kResXtRow = 68;      // floats per row of the transposed input in 
 constexpr int kResGateSlot = 15;   // word of the weights record that holds the shared expert's sigmoid gate
 constexpr int kResSleepPoll = 2;   // s_sleep between two polls of a wait (flat from 1 to 8 in measurements)
 constexpr int kResSleepFold = 24;  // waves that reach a layer while rung 0 still folds the one before wait this long first
+constexpr int kResPrioRouter = 3, kResPrioWg0 = 2;  // s_setprio of the router waves / of workgroup 0's other waves (measured: 2-4 % each)
 
 // The bits a value is handed on with: kResEmpty means "not yet written", so that one NaN travels as the default quiet NaN.
 WD_DEV uint32_t hand_word(float v) {
@@ -236,17 +237,22 @@ WD_DEV float res_router_dot(const float (&wv)[32], const float *xt, int lane) {
     const int t = lane & 31;
     const bool upper = lane >= 32;
     const float4 *xp = reinterpret_cast<const float4 *>(xt + t * kResXtRow + (upper ? 32 : 0));
-    float4 xv[8];
-#pragma unroll
-    for (int q = 0; q < 8; ++q) xv[q] = xp[q];
+    // (the input in two batches of 16 values: with all 32 next to the 32 weights the wave runs out of registers)
     auto run_half = [&](float start) {
         float v = start;
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            v = __builtin_fmaf(wv[4 * q + 0], xv[q].x, v);
-            v = __builtin_fmaf(wv[4 * q + 1], xv[q].y, v);
-            v = __builtin_fmaf(wv[4 * q + 2], xv[q].z, v);
-            v = __builtin_fmaf(wv[4 * q + 3], xv[q].w, v);
+        for (int h = 0; h < 2; ++h) {
+            float4 xv[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) xv[q] = xp[4 * h + q];
+            asm volatile("" ::: "memory");  // (keeps the second batch's reads behind the first batch's arithmetic)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                v = __builtin_fmaf(wv[16 * h + 4 * q + 0], xv[q].x, v);
+                v = __builtin_fmaf(wv[16 * h + 4 * q + 1], xv[q].y, v);
+                v = __builtin_fmaf(wv[16 * h + 4 * q + 2], xv[q].z, v);
+                v = __builtin_fmaf(wv[16 * h + 4 * q + 3], xv[q].w, v);
+            }
         }
         return v;
     };
@@ -320,10 +326,19 @@ struct ResCtx {
     WD_DEV float *land() const { return reinterpret_cast<float *>(lds + kResLdsLand); }
 };
 // The context of one layer: the indices made opaque (see fresh_v); `base` is the workgroup's dynamic LDS.
+// The lane number, counted anew from a mask the compiler cannot see through: one number kept from the start of the kernel
+// would hold a vector register for the whole launch - one that is spilled to scratch memory when registers are short,
+// and a kernel with scratch memory costs tens of microseconds more per launch.
+WD_DEV int fresh_lane() {
+    const unsigned all = static_cast<unsigned>(fresh_s(-1));
+    return static_cast<int>(__builtin_amdgcn_mbcnt_hi(all, __builtin_amdgcn_mbcnt_lo(all, 0u)));
+}
 WD_DEV ResCtx res_ctx(uint8_t *base, int r, int lane, int wave, int slot, __amdgpu_buffer_rsrc_t hb) {
     ResCtx c;
     c.lds = base + fresh_s(0);
-    c.r = fresh_s(r), c.lane = fresh_v(lane), c.wave = fresh_s(wave), c.slot = fresh_s(slot);
+    (void)lane;
+    c.lane = fresh_lane();
+    c.r = fresh_s(r), c.wave = fresh_s(wave), c.slot = fresh_s(slot);
     c.hb = hb;
     return c;
 }
@@ -509,10 +524,12 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             // look into, so that the addresses below do not exist before this point.
             asm volatile("" : "+s"(e) : : "memory");
             draw = q8_rows4_coal_request<0, 16>(down_base + e * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
-            if (traced) raw = gate_up_rows(gate_base, up_base, e_next, r, lane);
             res_mark<STAMPS>(a, c, l, 11);
             iq_rows8_coal_dots<TYPE, 2>(tables, c.xq(), c.xd(), lane, gu, c.area());
             act = silu_ggml(gu[0]) * gu[1];
+            // the next layer's gate/up rows (their registers are free since the rows of this layer lie in LDS; requested
+            // behind the dot products, which need every register there is)
+            if (traced) raw = gate_up_rows(gate_base, up_base, e_next, r, lane);
             res_mark<STAMPS>(a, c, l, 5);
         }
         // rung 0 folds the results with the router's weights and the shared expert's gate: published long before this
@@ -538,14 +555,14 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             const float *ybuf = c.ybuf();
             float acc = 0.0f;
             for (int m = 0; m < a.k; ++m) {
-                const float wm = lane_get(wreg, m);
+                const float wm = readlane_f(wreg, m);
                 const float prod = ybuf[m * 4 + (lane & 3)] * wm;
                 acc = acc + prod;
             }
             float o = acc, ysh = 0.0f;
             if (shared) {
                 ysh = ybuf[kResSharedSlot * 4 + (lane & 3)];
-                const float prod = ysh * lane_get(wreg, 16);
+                const float prod = ysh * readlane_f(wreg, 16);
                 o = acc + prod;
             }
             const float scaled = o * a.residual_scale;
@@ -586,9 +603,10 @@ WD_DEV void res_shared_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
     for (int l = 0; l < a.n_layers; ++l) {
         const ResCtx c = res_ctx(lds_base, r0, lane0, wave0, kResSharedSlot, hb);
         const int r = c.r, lane = c.lane;
+        const bool with_shared = fresh_s(a.shared) != 0;  // (a scalar of this layer, not a vector register kept for the launch)
         __syncthreads();  // B1
         float act = 0.0f;
-        if (a.shared) {
+        if (with_shared) {
             res_mark<STAMPS>(a, c, l, 2);
             Q8RowTile &tile = *reinterpret_cast<Q8RowTile *>(c.area());
             float acc[2] = {0.0f, 0.0f};
@@ -630,7 +648,7 @@ WD_DEV void res_shared_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         }
         bool got = false;
         float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
-        res_exchange<STAMPS>(a, c, l, a.shared != 0, act, v0, v1, dead,
+        res_exchange<STAMPS>(a, c, l, with_shared, act, v0, v1, dead,
             [&] { if (r == 0 && traced) got = gather_logits(false); },  // the logits ahead of the barrier, if that holds nobody up
             [&] {
                 if (r == 0 && traced) {
@@ -638,11 +656,11 @@ WD_DEV void res_shared_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                     denominator();
                 }
             });
-        if (a.shared) res_down<STAMPS>(a, c, l, draw, v0, v1);
+        if (with_shared) res_down<STAMPS>(a, c, l, draw, v0, v1);
         __syncthreads();  // B5
         // the next layer's rows, asked for on this side of the barrier: the fold of this layer must not wait for a
         // wave that is busy issuing requests
-        if (a.shared && l + 1 < a.n_layers) fetch(a.layers + l + 1, r, lane);
+        if (with_shared && l + 1 < a.n_layers) fetch(a.layers + l + 1, r, lane);
     }
 }
 
@@ -660,9 +678,9 @@ WD_DEV void res_router_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                             __amdgpu_buffer_rsrc_t hb, __amdgpu_buffer_rsrc_t ob, bool &dead) {
     const bool has_row = r0 < a.E;
     const bool traced = a.ids_trace != nullptr;
-#ifdef WD_RES_PRIO
-    __builtin_amdgcn_s_setprio(WD_RES_PRIO);
-#endif
+    // The wave's few instructions are on the critical path of the whole grid (the logit; in workgroup 0 the ranks), while
+    // the rungs next to it work through thousands: it goes first whenever it has something to issue.
+    __builtin_amdgcn_s_setprio(kResPrioRouter);
     // (a workgroup without a row keeps row 0 company: one definition of the row's registers per layer, no merge of an
     // old and a new value - the compiler then holds them as 32 registers, not as one value of 32 that it copies whole)
     float wv[32];
@@ -808,7 +826,8 @@ WD_DEV void res_router_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
 template <int TYPE, bool STAMPS>
 __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 6))) void k_stack_resident(ResidentArgs a) {
     extern __shared__ __align__(16) uint8_t lds_res[];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // (the wave's number as a scalar, the lane's counted where it is needed: no vector register is held for the whole launch)
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
     const int r = blockIdx.x;
     if (__hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {  // an earlier launch failed
         if (threadIdx.x < 4) a.x[4 * r + threadIdx.x] = a.out[4 * r + threadIdx.x] = __builtin_nanf("");
@@ -825,7 +844,7 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 
     // of the compute unit carries five of the twenty routed waves.
     if (threadIdx.x < 16) reinterpret_cast<float *>(lds_res + kResLdsActv)[threadIdx.x] = 0.0f;  // slots not in use hand on zeros
     int *simd_of = reinterpret_cast<int *>(lds_res + kResLdsRoles);
-    if (lane == 0) simd_of[wave] = static_cast<int>((__builtin_amdgcn_s_getreg(4 | (31 << 11)) >> 4) & 3u);  // HW_ID.SIMD_ID
+    if (fresh_lane() == 0) simd_of[wave] = static_cast<int>((__builtin_amdgcn_s_getreg(4 | (31 << 11)) >> 4) & 3u);  // HW_ID.SIMD_ID
     __syncthreads();
     int slot;
     {
@@ -853,19 +872,19 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 
         slot = __builtin_amdgcn_readfirstlane(slot);
     }
 
-#ifdef WD_RES_PRIO_WG0
-    if (r == 0) __builtin_amdgcn_s_setprio(WD_RES_PRIO_WG0);
-#endif
+    // Workgroup 0 carries the selection on top of its share of the rows: its waves go ahead of those of the workgroup it
+    // shares a compute unit with, so that it is not the one the grid waits for.
+    if (r == 0) __builtin_amdgcn_s_setprio(kResPrioWg0);
     bool dead = false;
     if (slot < 0)
-        res_router_role<STAMPS>(a, lds_res, r, lane, wave, hb, ob, dead);
+        res_router_role<STAMPS>(a, lds_res, r, fresh_lane(), wave, hb, ob, dead);
     else if (slot == kResSharedSlot)
-        res_shared_role<STAMPS>(a, lds_res, r, lane, wave, hb, dead);
+        res_shared_role<STAMPS>(a, lds_res, r, fresh_lane(), wave, hb, dead);
     else
-        res_routed_role<TYPE, STAMPS>(a, lds_res, r, lane, wave, slot, hb, dead);
+        res_routed_role<TYPE, STAMPS>(a, lds_res, r, fresh_lane(), wave, slot, hb, dead);
 
     // the next launch takes the other set (workgroup 0 can only get here after every workgroup has read the number)
-    if (r == 0 && threadIdx.x == 0 && !dead)
+    if (r == 0 && wave == 0 && fresh_lane() == 0 && !dead)
         __hip_atomic_store(reinterpret_cast<unsigned *>(a.hand + kHandEpoch), epoch + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
