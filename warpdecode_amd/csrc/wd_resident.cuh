@@ -161,12 +161,12 @@ WD_DEV bool res_full(const uint4 &v) { return v.x != kResEmpty && v.y != kResEmp
 // written.  Only pieces that are still incomplete are requested again, one poll at a time: two or three polls in flight
 // measured slower (more device-scope loads compete with the stores they wait for).
 template <int N>
-WD_DEV void hand_wait16(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, const unsigned (&off)[N], bool on, uint4 (&v)[N], bool &dead) {
+WD_DEV void hand_wait16(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, const unsigned (&off)[N], const bool (&on)[N], uint4 (&v)[N], bool &dead) {
     bool need[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-        need[i] = on;
-        v[i] = make_uint4(0u, 0u, 0u, 0u);
+        need[i] = on[i];
+        if (on[i]) v[i] = make_uint4(0u, 0u, 0u, 0u);
     }
     if (dead) return;
     unsigned spins = 0;
@@ -184,6 +184,13 @@ WD_DEV void hand_wait16(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, const 
         if (res_give_up(a, spins, dead)) return;
         __builtin_amdgcn_s_sleep(kResSleepPoll);
     }
+}
+template <int N>
+WD_DEV void hand_wait16(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, const unsigned (&off)[N], bool on, uint4 (&v)[N], bool &dead) {
+    bool each[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) each[i] = on;
+    hand_wait16<N>(a, rs, off, each, v, dead);
 }
 // N words per lane, word i at off + i * stride (words with on[i] == false take no part; they read as zero).
 // stop(): looked at after every unsuccessful round; true ends the wait early.  Returns whether every word has arrived.
@@ -392,12 +399,23 @@ WD_DEV void res_exchange(const ResidentArgs &a, const ResCtx &c, int l, bool has
         const float4 p = reinterpret_cast<const float4 *>(c.actv())[piece];
         hand_store16(c.hb, ac_off(l, copy) + kAcRec * c.r + 16u * piece, make_uint4(hand_word(p.x), hand_word(p.y), hand_word(p.z), hand_word(p.w)));
     }
+    res_mark<STAMPS>(a, c, l, 10);
     if (wave < 8) {  // the group's copy, three 16-byte words per lane: word w is piece w % 3 of workgroup w / 3
         const int i = wave * 64 + lane;
         const unsigned base = ac_off(l, c.r & (kResCopies - 1)) + 16u * i;
         const unsigned off[3] = {base, base + 16u * 512, base + 16u * 1024};
         uint4 v[3];
-        hand_wait16<3>(a, c.hb, off, true, v, dead);
+        {
+            // the first third alone until it is complete, then the rest: by then most of it is there, and a third of the
+            // volume per poll goes through the fabric while the grid waits for its slowest workgroup (1.5 % of the step).
+            // (The rest read through the L2 once the first third is complete, with the pieces that are behind there polled
+            // past it, measured the same: the volume of the polls is not what this hand-off waits for.)
+            const unsigned o1[1] = {off[0]}, o2[2] = {off[1], off[2]};
+            uint4 v1[1], v2[2];
+            hand_wait16<1>(a, c.hb, o1, true, v1, dead);
+            hand_wait16<2>(a, c.hb, o2, true, v2, dead);
+            v[0] = v1[0], v[1] = v2[0], v[2] = v2[1];
+        }
 #pragma unroll
         for (int t = 0; t < 3; ++t) {
             const int w = i + 512 * t, wg = w / 3, piece = w - 3 * wg;
