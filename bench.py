@@ -79,6 +79,8 @@ def parse():
                     help="resident mode: the stack as ONE launch of resident workgroups (default), or two dispatches per layer")
     ap.add_argument("--repeats", type=int, default=5, help="further repeats of the timed region, for the spread in the JSON line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-mode-b", action="store_true",
+                    help="resident mode: leave out the bounded run of the same stack with its experts behind the slot pool")
     ap.add_argument("--site-profile", type=int, default=0, metavar="TOKENS",
                     help="resident mode: afterwards run TOKENS eager steps with the library's site profiler on (device, host and "
                          "gap time per bracketed site and token), print its report and add it to the JSON line")
@@ -86,6 +88,33 @@ def parse():
                     help="wall-clock seconds of CPU layer passes to accumulate for cpu_baseline (all host threads busy)")
     ap.add_argument("--check", action="store_true", help="verify one layer pass against the CPU oracle first")
     return ap.parse_args()
+
+
+def offload_layer(capi, torch, synth, t, d, packed):
+    """Moves one layer's routed tensors (device tensors in `t`, pointers in descriptor `d`) to pinned host memory and
+    drops their device copies; returns the three host pointers.  `packed`: one buffer, gate, up and down of an expert
+    back to back, experts one slot apart."""
+    H, F, n_experts = 2048, 512, d.n_experts
+    gbytes, dbytes = F * synth.row_bytes(synth.IQ3_S, H), H * synth.row_bytes(synth.Q8_0, F)
+    if packed:
+        slot = torch.cat([t["gate"].view(n_experts, gbytes), t["up"].view(n_experts, gbytes),
+                          t["down"].view(n_experts, dbytes)], dim=1).contiguous()
+        h = C.c_void_p()
+        capi.call("wd_malloc_host", C.byref(h), slot.numel())
+        capi.call("wd_memcpy_d2h", h, C.c_void_p(slot.data_ptr()), slot.numel(), None)
+        del slot
+        host = [h, C.c_void_p(h.value + gbytes), C.c_void_p(h.value + 2 * gbytes)]
+    else:
+        host = []
+        for name in ("gate", "up", "down"):
+            h = C.c_void_p()      # exact-size pinned buffer (torch's pinned allocator rounds sizes up to 2^n)
+            capi.call("wd_malloc_host", C.byref(h), t[name].numel())
+            capi.call("wd_memcpy_d2h", h, C.c_void_p(t[name].data_ptr()), t[name].numel(), None)
+            host.append(h)
+    for name in ("gate", "up", "down"):
+        t[name] = None
+        setattr(d, name, None)
+    return host
 
 
 def build_stack(torch, synth, capi, n_layers, n_experts, seed, offload=False, packed=False):
@@ -126,28 +155,8 @@ def build_stack(torch, synth, capi, n_layers, n_experts, seed, offload=False, pa
             setattr(d, name, tensor.data_ptr())
         d.gate_stride = d.up_stride = F * rb_iq3
         d.down_stride = H * rb_q8f
-        if offload and packed:
-            gbytes, dbytes = F * rb_iq3, H * rb_q8f
-            slot = torch.cat([t["gate"].view(n_experts, gbytes), t["up"].view(n_experts, gbytes),
-                              t["down"].view(n_experts, dbytes)], dim=1).contiguous()
-            h = C.c_void_p()
-            capi.call("wd_malloc_host", C.byref(h), slot.numel())
-            capi.call("wd_memcpy_d2h", h, C.c_void_p(slot.data_ptr()), slot.numel(), None)
-            del slot
-            for name in ("gate", "up", "down"):
-                t[name] = None
-                setattr(d, name, None)
-            pinned.append([h, C.c_void_p(h.value + gbytes), C.c_void_p(h.value + 2 * gbytes)])
-        elif offload:
-            host = []
-            for name in ("gate", "up", "down"):
-                h = C.c_void_p()      # exact-size pinned buffer (torch's pinned allocator rounds sizes up to 2^n)
-                capi.call("wd_malloc_host", C.byref(h), t[name].numel())
-                capi.call("wd_memcpy_d2h", h, C.c_void_p(t[name].data_ptr()), t[name].numel(), None)
-                host.append(h)
-                t[name] = None
-                setattr(d, name, None)
-            pinned.append(host)
+        if offload:
+            pinned.append(offload_layer(capi, torch, synth, t, d, packed))
     return (layers, keep, pinned) if offload else (layers, keep)
 
 
@@ -269,9 +278,10 @@ def cpu_leg(kind, seconds, threads, folder, max_children):
 
 
 def cpu_baseline(seconds):
-    """The layer pass on the host cores, on the headline workload's shape: the C port (one child, no restarts) is the
-    figure reported; the reference's own CPU path is reported beside it with the number of children that stalled.
-    ms/layer is converted to tokens/s of a 48-layer stack."""
+    """The layer pass on the host cores, on the headline workload's shape.  `value` is the reference's own CPU MoE path
+    (kind "reference") when its build is present, with the number of its children that stalled beside it; the C port of
+    the layer (one child, no restarts) is reported under "port", and is `value` (kind "port") where the reference
+    build is absent.  ms/layer is converted to tokens/s of a 48-layer stack."""
     import shutil
     import tempfile
     from oracle import pyoracle
@@ -281,25 +291,29 @@ def cpu_baseline(seconds):
     workload = ("layer passes of the headline shape (hidden 2048, ffn 512, top-10 of %d experts + shared expert, ids "
                 "Zipf(1.1) over a per-layer permutation, %d layers = %.1f GB of weights taken in turn)"
                 % (CPU_EXPERTS, CPU_LAYERS, CPU_LAYERS * 1.039))
+
+    def leg(kind, children):
+        passes, secs, stalls = cpu_leg(kind, seconds, threads, folder, children)
+        note("cpu baseline (%s): %d passes in %.1f s, %d stalled children" % (kind, passes, secs, stalls))
+        if passes < 8:
+            return dict(value=None, unit="tok/s", cores=threads, kind=kind, stalled_children=stalls,
+                        sample="fewer than 8 CPU passes completed")
+        per_layer = secs / passes
+        return dict(value=round(1.0 / (per_layer * 48), 3), unit="tok/s", cores=threads, kind=kind, stalled_children=stalls,
+                    passes=passes, seconds=round(secs, 2), ms_per_layer=round(per_layer * 1e3, 3),
+                    sample="%d %s in %.1f s = %.2f ms/layer, x48 layers per token; %d threads on %d host cores"
+                           % (passes, workload, secs, per_layer * 1e3, threads, cpus))
     try:
         note("cpu baseline: writing %d layers of weights to %s" % (CPU_LAYERS, folder))
         cpu_weights(folder)
-        passes, secs, stalls = cpu_leg("port", seconds, threads, folder, 1)
-        note("cpu baseline (port): %d passes in %.1f s, %d stalled children" % (passes, secs, stalls))
-        if passes < 8:
-            return dict(value=None, unit="tok/s", cores=threads, kind="port", sample="no CPU pass completed")
-        per_layer = secs / passes
-        out = dict(value=round(1.0 / (per_layer * 48), 3), unit="tok/s", cores=threads, kind="port",
-                   sample="%d %s in %.1f s = %.2f ms/layer, x48 layers per token; %d threads on %d host cores, one "
-                          "child process, no restarts" % (passes, workload, secs, per_layer * 1e3, threads, cpus))
-        if pyoracle.ref() is not None:
-            passes, secs, stalls = cpu_leg("reference", seconds, threads, folder, 12)
-            note("cpu baseline (reference): %d passes in %.1f s, %d stalled children" % (passes, secs, stalls))
-            ref = dict(value=round(passes / (secs * 48), 3) if passes >= 8 else None, unit="tok/s", cores=threads,
-                       passes=passes, seconds=round(secs, 2), stalled_children=stalls,
-                       sample="the reference's own CPU MoE path on the same workload; a child whose thread pool "
-                              "dead-locked was killed and replaced by a fresh one, only completed passes count")
-            out["reference"] = ref
+        port = leg("port", 1)
+        port["sample"] += "; C restatement of the layer, one child process, no restarts"
+        if pyoracle.ref() is None:
+            return port
+        out = leg("reference", 12)
+        out["sample"] += ("; the reference's own CPU MoE path built from its sources; a child whose thread pool dead-locked "
+                          "was killed and replaced by a fresh one (stalled_children), only completed passes count")
+        out["port"] = port
         return out
     finally:
         shutil.rmtree(folder, ignore_errors=True)
@@ -319,10 +333,12 @@ def recorded_traffic(kernel):
     return None
 
 
-def bench_lru(args, torch, capi, synth):
+def bench_lru(args, torch, capi, synth, stack=None):
     """C3 mode B: the routed experts live in pinned host memory; an LRU pool of --cache-gib in HBM holds the
     recently used ones.  The routing trace is known to the host, so the fills of layer l+1 are queued while
-    layer l computes.  Eager launches (the cache decides per token what to copy)."""
+    layer l computes.  Eager launches (the cache decides per token what to copy).  Returns the JSON object.
+    `stack`: (layers, keep) of a stack already on the device, whose routed tensors are then moved to pinned host
+    memory in place (--source pinned only)."""
     H, F, k, E, NL = 2048, 512, 10, args.experts, args.layers
     gb, db = F * synth.row_bytes(synth.IQ3_S, H), H * synth.row_bytes(synth.Q8_0, F)
     slot_bytes = 2 * gb + db
@@ -331,7 +347,12 @@ def bench_lru(args, torch, capi, synth):
     if args.source == "pinned":
         note("generating %d layers x %d experts, routed tensors to pinned host memory" % (NL, E))
         packed = args.host_layout == "packed"
-        layers, keep, pinned = build_stack(torch, synth, capi, NL, E, synth.BASE_SEED, offload=True, packed=packed)
+        if stack is None:
+            layers, keep, pinned = build_stack(torch, synth, capi, NL, E, synth.BASE_SEED, offload=True, packed=packed)
+        else:
+            layers, keep = stack
+            pinned = [offload_layer(capi, torch, synth, keep[l], layers[l], packed) for l in range(NL)]
+            torch.cuda.empty_cache()
         torch.cuda.synchronize()
         capi.call("wd_expert_cache_create", C.byref(cache), int(args.cache_gib * (1 << 30)), gb, gb, db, NL, E, 0)
         capi.call("wd_expert_cache_set_copy_kernel", cache, 1 if args.fill == "kernel" else 0)
@@ -458,7 +479,14 @@ def bench_lru(args, torch, capi, synth):
                      "frac": round(whole / HBM_PEAK_GBS, 4) if whole else None, "traffic": None,
                      "kernel": "whole step (kernel bytes only; the host-link bytes are in config)"},
     }
-    print(json.dumps(out))
+    torch.cuda.synchronize()
+    capi.call("wd_moe_scratch_destroy", scratch)
+    capi.call("wd_expert_cache_destroy", cache)
+    if args.source == "pinned":
+        for host in pinned:
+            for h in (host[:1] if packed else host):
+                capi.call("wd_free_host", h)
+    return out
 
 
 def graph_period_us(torch, launch, launches, reps):
@@ -890,7 +918,8 @@ def main():
     if args.mode == "tokens":
         return bench_tokens(args, torch, capi, synth)
     if args.mode == "lru":
-        return bench_lru(args, torch, capi, synth)
+        print(json.dumps(bench_lru(args, torch, capi, synth)))
+        return
     if args.mode == "hc":
         return bench_hc(args, torch, capi, synth)
     layers, keep = build_stack(torch, synth, capi, NL, E, synth.BASE_SEED)
@@ -905,11 +934,17 @@ def main():
     trace = np.stack([np.stack([synth.zipf_ids(rng, E, k, 1.1, perms[l]) for l in range(NL)])
                       for _ in range(total_steps)]).astype(np.int32)           # [steps][layers][k]
     xs = np.stack([synth.rms_normed(rng, H) for _ in range(total_steps)])
-    d_trace_all, d_xs = torch.from_numpy(trace).cuda(), torch.from_numpy(xs).cuda()
-    d_trace = torch.zeros((NL, k), dtype=torch.int32, device="cuda")
-    d_x = torch.zeros(H, dtype=torch.float32, device="cuda")
+    # A token's input is one piece of device memory, the activation followed by its routing trace, so that a step brings
+    # its input in with one copy.
+    inputs = np.concatenate([xs.view(np.int32), trace.reshape(total_steps, NL * k)], axis=1)
+    d_inputs = torch.from_numpy(inputs).cuda()
+    d_input = torch.zeros(H + NL * k, dtype=torch.int32, device="cuda")
+    d_x, d_trace = d_input[:H].view(torch.float32), d_input[H:].view(NL, k)
     d_out = torch.zeros(H, dtype=torch.float32, device="cuda")
     trace_ptr = C.c_void_p(d_trace.data_ptr()) if args.routing == "zipf" else None
+
+    def bring_in(i):
+        d_input.copy_(d_inputs[i % total_steps], non_blocking=True)
 
     PER_LAYER = 0x200   # WD_MOE_PER_LAYER
     stack_flags = STACK_FLAGS | (PER_LAYER if args.path == "per-layer" else 0)
@@ -936,8 +971,7 @@ def main():
 
     def first_token(flags, n_layers=NL):
         """x and out (host copies) of token 0 through the first n_layers layers by the given form of the stack."""
-        d_x.copy_(d_xs[0])
-        d_trace.copy_(d_trace_all[0])
+        bring_in(0)
         capi.call("wd_moe_stack_f32", layers, n_layers, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()), scratch,
                   trace_ptr, RESIDUAL_SCALE, flags, C.c_void_p(torch.cuda.current_stream().cuda_stream))
         torch.cuda.synchronize()
@@ -975,9 +1009,7 @@ def main():
     note("launch mode: %s" % ("eager" if graph is None else "hip-graph replay"))
 
     def step(i):
-        i %= total_steps
-        d_x.copy_(d_xs[i], non_blocking=True)
-        d_trace.copy_(d_trace_all[i], non_blocking=True)
+        bring_in(i)
         if graph is not None:
             graph.replay()
         else:
@@ -1032,7 +1064,7 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / reps
 
-    per_kernel, reps = {}, 20
+    per_kernel, reps, router_driven = {}, 20, None
     step(0)
     if args.path == "resident":
         # The dominant kernel is the step itself: one launch of k_stack_resident covers the 48 layers.  Timed live with HIP
@@ -1041,8 +1073,7 @@ def main():
         run_it = graph.replay if graph is not None else launch_stack
         pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
         for j, (e0, e1) in enumerate(pairs):
-            d_x.copy_(d_xs[j % total_steps], non_blocking=True)
-            d_trace.copy_(d_trace_all[j % total_steps], non_blocking=True)
+            bring_in(j)
             e0.record()
             run_it()
             e1.record()
@@ -1056,8 +1087,7 @@ def main():
         run_alt = g2.replay if g2 is not None else (lambda: launch_stack(STACK_FLAGS | PER_LAYER))
 
         def alt_step(j):
-            d_x.copy_(d_xs[j % total_steps], non_blocking=True)
-            d_trace.copy_(d_trace_all[j % total_steps], non_blocking=True)
+            bring_in(j)
             run_alt()
         for j in range(4):
             alt_step(j)
@@ -1069,6 +1099,28 @@ def main():
         torch.cuda.synchronize()
         per_kernel["per_layer_dispatches"] = dict(ms_per_step=round(e0.elapsed_time(e1) / reps, 4))
         dominant = "k_stack_resident"
+        if trace_ptr is not None:
+            # the same launch with nothing known ahead: every layer's ids come from its own router, inside the launch
+            def router_stack():
+                capi.call("wd_moe_stack_f32", layers, NL, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()), scratch,
+                          None, RESIDUAL_SCALE, STACK_FLAGS, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+            g3 = captured(router_stack)
+            run_router = g3.replay if g3 is not None else router_stack
+            for j in range(4):
+                bring_in(j)
+                run_router()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for j in range(args.steps):
+                bring_in(4 + j)
+                run_router()
+            e1.record()
+            torch.cuda.synchronize()
+            ms_router = e0.elapsed_time(e1) / args.steps
+            router_driven = dict(ms_per_step=round(ms_router, 4), tok_s=round(1000.0 / ms_router, 2), steps=args.steps,
+                                 finite=bool(torch.isfinite(d_x).all().item()),
+                                 in_dispatch_waits_ok=capi.load().wd_moe_scratch_status(scratch) == 0)
+            note("router-selected experts, same launch: %s" % router_driven)
     else:
         # Per-kernel launch time, live: the stack is replayed with one dispatch per layer only (the other left out), so
         # the timed region is a chain of NL launches of that one kernel over NL layers' weights.  The period includes
@@ -1110,8 +1162,7 @@ def main():
             capi.call("wd_profile_enable", 1)
             capi.call("wd_profile_reset")
             for j in range(args.site_profile):
-                d_x.copy_(d_xs[j % total_steps], non_blocking=True)
-                d_trace.copy_(d_trace_all[j % total_steps], non_blocking=True)
+                bring_in(j)
                 launch_stack(flags)
                 torch.cuda.synchronize()
                 capi.call("wd_profile_flush_token")
@@ -1138,13 +1189,29 @@ def main():
                    "spread_ms_per_step": spread,
                    "bytes_per_token": bytes_per_step, "wall_s": round(wall, 3), "finite": finite,
                    "in_dispatch_waits_ok": waits_ok, "forms_bit_identical_on_token_0": forms_agree,
-                   "layer_0_equals_cpu_oracle": oracle_checked},
+                   "layer_0_equals_cpu_oracle": oracle_checked, "router_selected_ids_same_launch": router_driven},
         "roofline": roofline,
     }
     if site_profile is not None:
         out["config"]["site_profile_ms_per_token"] = site_profile
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
+    if not args.no_mode_b and args.path == "resident" and E == 512 and NL == 48:
+        # The same stack with its routed experts in pinned host memory behind the slot pool (a bounded run: the tokens
+        # that warm the pool, then --steps tokens).  The resident stack's device copies are given up for it, so it runs last.
+        del graph, g2
+        try:
+            b = bench_lru(args, torch, capi, synth, stack=(layers, keep))
+            c = b["config"]
+            out["mode_b"] = dict(tok_s=b["value"], ms_per_step=b["ms_per_step"], steps=b["steps"], hit_rate=c["hit_rate"],
+                                 misses_per_token=c["misses_per_token"], host_link_bytes_per_token=c["host_link_bytes_per_token"],
+                                 host_link_GBps=c["host_link_GBps"], host_ms_per_step=c["host_ms_per_step"], slots=c["slots"],
+                                 slot_bytes=c["slot_bytes"], cache_gib=args.cache_gib, cache_warm_tokens=c["cache_warm_tokens"],
+                                 source=c["source"], driver=c["driver"], launch=c["launch"], finite=c["finite"],
+                                 workload=c["workload"])
+        except Exception as exc:      # e.g. the box refuses 49.5 GB of pinned host memory
+            out["mode_b"] = dict(skipped="%s: %s" % (type(exc).__name__, exc))
+        note("mode B: %s" % out["mode_b"])
     print(json.dumps(out))
 
 
