@@ -410,6 +410,8 @@ def bench_lru(args, torch, capi, synth, stack=None):
     if args.read_ahead:
         capi.call("wd_expert_cache_set_read_ahead", cache, args.read_ahead, 0)
 
+    lru_flags = 0x200 if args.path == "per-layer" else 0     # WD_MOE_PER_LAYER
+
     def step(i):
         d_x.copy_(d_xs[i % 64], non_blocking=True)
         if args.lru_driver == "router":   # the router's own selection, layer by layer through the host
@@ -417,7 +419,7 @@ def bench_lru(args, torch, capi, synth, stack=None):
                       scratch, None, None, RESIDUAL_SCALE, 0, stream)
             return
         capi.call("wd_moe_stack_cached_f32", layers, NL, cache, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()),
-                  scratch, trace[i].ctypes.data_as(C.c_void_p), C.c_void_p(d_trace_all[i].data_ptr()), RESIDUAL_SCALE, 0, stream)
+                  scratch, trace[i].ctypes.data_as(C.c_void_p), C.c_void_p(d_trace_all[i].data_ptr()), RESIDUAL_SCALE, lru_flags, stream)
 
     def stats():
         st = capi.CacheStats()
@@ -467,6 +469,8 @@ def bench_lru(args, torch, capi, synth, stack=None):
         "config": {"workload": "C3 mode B: %d-layer stack of the 512-expert top-10 IQ3_S/Q8_0 MoE layer, batch=1, routed "
                                "experts in pinned host memory behind a %.0f GiB LRU slot pool in HBM, Zipf(1.1) trace" % (NL, args.cache_gib),
                    "layers": NL, "experts": E, "top_k": k, "routing": "zipf" if args.lru_driver == "trace" else "router", "launch": "eager",
+                   "path": ("one resident launch per token, fills land while it runs" if monitor.get("tokens_in_one_launch", 0) >= total
+                            else "dispatches per layer"),
                    "source": args.source, "driver": args.lru_driver, "read_ahead": args.read_ahead,
                    "slots": int(s1.slots), "slot_bytes": int(slot_bytes), "cache_warm_tokens": args.cache_warm_tokens,
                    "hit_rate": round(hits / max(1, acc), 4), "misses_per_token": round(miss / args.steps, 2),
@@ -1207,7 +1211,7 @@ def main():
                                  misses_per_token=c["misses_per_token"], host_link_bytes_per_token=c["host_link_bytes_per_token"],
                                  host_link_GBps=c["host_link_GBps"], host_ms_per_step=c["host_ms_per_step"], slots=c["slots"],
                                  slot_bytes=c["slot_bytes"], cache_gib=args.cache_gib, cache_warm_tokens=c["cache_warm_tokens"],
-                                 source=c["source"], driver=c["driver"], launch=c["launch"], finite=c["finite"],
+                                 source=c["source"], driver=c["driver"], launch=c["launch"], path=c["path"], finite=c["finite"],
                                  workload=c["workload"])
         except Exception as exc:      # e.g. the box refuses 49.5 GB of pinned host memory
             out["mode_b"] = dict(skipped="%s: %s" % (type(exc).__name__, exc))

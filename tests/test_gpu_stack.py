@@ -226,6 +226,64 @@ def test_one_launch_stack_matches_per_layer_and_oracle(g, oracle, gate_type, exp
     sc_b.close()
 
 
+# 150 slots hold three tokens' experts (a token's fills run beside the launch of the token before), 100 two tokens'
+# (they wait for it); 320 (layer, expert) pairs compete for them
+@pytest.mark.parametrize("slots", [150, 100], ids=["three-tokens-of-slots", "two-tokens-of-slots"])
+def test_one_launch_stack_fed_from_the_slot_cache(g, oracle, slots):
+    """The stack whose routed experts live in pinned host memory behind the slot pool, routing trace known to the host:
+    one resident launch per token (the cache's counter says so), fills landing while it runs, against the all-resident
+    stack on the same trace - outputs and the last layer's views bit for bit - and, with WD_MOE_PER_LAYER, the same
+    through the per-layer dispatches."""
+    import json
+    import torch
+    experts, k, nl, tokens = 64, 10, 5, 8
+    Ls = [synth.make_layer(2048, 512, experts, k, synth.IQ3_S, synth.Q8_0, shared=True, layer=500 + l,
+                           router_sigma=1.0 / np.sqrt(2048.0)) for l in range(nl)]
+    gb, db = 512 * synth.row_bytes(synth.IQ3_S, 2048), 2048 * synth.row_bytes(synth.Q8_0, 512)
+    cache = C.c_void_p()
+    capi.call("wd_expert_cache_create", C.byref(cache), slots * (2 * gb + db), gb, gb, db, nl, experts, 0)
+    pinned = []
+    for l, L in enumerate(Ls):
+        p = [torch.from_numpy(np.ascontiguousarray(L[n]).reshape(-1)).pin_memory() for n in ("gate", "up", "down")]
+        pinned.append(p)
+        capi.call("wd_expert_cache_register_layer", cache, l, *[C.c_void_p(t.data_ptr()) for t in p])
+    dls, arr = _descs(g, Ls)
+    dls_bare, bare = _descs(g, Ls)   # (kept: the descriptors point into these tensors)
+    for i in range(nl):                      # the routed tensors live only in the cache
+        bare[i].gate = bare[i].up = bare[i].down = None
+    sc_a, sc_b = g.Scratch(2048, 512, experts, k), g.Scratch(2048, 512, experts, k)
+    rng = np.random.default_rng(SEED + 500)
+
+    def counter():
+        lib = capi.load()
+        need = lib.wd_expert_cache_dump_json(cache, None, 0)
+        buf = C.create_string_buffer(need + 1)
+        lib.wd_expert_cache_dump_json(cache, buf, need + 1)
+        return json.loads(buf.value.decode())["tokens_in_one_launch"]
+
+    for token in range(tokens):
+        x = synth.rms_normed(synth.rng_for(SEED, 86, token), 2048)
+        tr = np.stack([rng.choice(experts, size=k, replace=False) for _ in range(nl)]).astype(np.int32)
+        flags = PER_LAYER if token == tokens - 1 else 0
+        dx, out, dtr = g.dev(x), g.empty(2048, np.float32), g.dev(tr)
+        capi.call("wd_moe_stack_cached_f32", bare, nl, cache, g.ptr(dx), g.ptr(out), sc_a.h, tr.ctypes.data_as(C.c_void_p),
+                  g.ptr(dtr), float(2.0 ** -12), flags, g.stream())
+        g.sync()
+        views = {name: sc_a.get(name, {"k": k, "E": experts, "H": 2048}.get(n_, n_), dt) for name, n_, dt in VIEWS}
+        want = _run_stack(g, arr, nl, x, tr, sc_b, PER_LAYER)
+        assert g.same_bits(g.host(dx), want[0]) and g.same_bits(g.host(out), want[1]), token
+        for name, _, dt in VIEWS:
+            assert np.array_equal(views[name].view(np.uint32), want[2][name].view(np.uint32)), (token, name)
+        assert counter() == min(token + 1, tokens - 1), token
+    st = capi.CacheStats()
+    capi.call("wd_expert_cache_get_stats", cache, C.byref(st))
+    assert st.accesses == tokens * nl * k and st.evictions > 0 and st.resident <= slots
+    assert capi.load().wd_moe_scratch_status(sc_a.h) == 0
+    sc_a.close()
+    sc_b.close()
+    capi.call("wd_expert_cache_destroy", cache)
+
+
 def test_one_launch_stack_wait_that_runs_out(g):
     """A wait limit of one poll: the launch ends normally with the status word set and NaN in its outputs; the next call
     on that scratch is refused by the host (the status word has a mirror in host memory), a replay of a graph recorded

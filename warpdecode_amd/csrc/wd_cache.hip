@@ -82,6 +82,28 @@ struct FillSegments {
 #ifndef WD_FILL_THREADS
 #define WD_FILL_THREADS 64
 #endif
+// What a fill launch tells a one-launch stack that runs beside it (wd_resident.cuh, fill_need / fill_done): when the
+// launch's last workgroup is through, done[l] = seq for every layer l in `layers` (bit l).
+struct FillMarks {
+    uint32_t *done;               // null: nothing to tell
+    unsigned *arrivals;           // workgroups of this launch that are through (back to 0 when the last one is)
+    unsigned long long layers;
+    uint32_t seq;
+};
+// When the launch's last workgroup is through: the layers are counted off.
+WD_DEV void fill_marks(const FillMarks &m) {
+    if (!m.done) return;
+    __threadfence();  // the stores of the copy are where every compute unit of the device reads them
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned last = gridDim.x - 1;
+        if (atomicInc(m.arrivals, last) == last) {  // (wraps to 0 for the next launch)
+            __threadfence();
+            for (unsigned long long rest = m.layers; rest; rest &= rest - 1)
+                __hip_atomic_store(m.done + (__ffsll(rest) - 1), m.seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
 __global__ __launch_bounds__(WD_FILL_THREADS) void k_fill_slots(FillSegments f, int n_seg) {
     const uint32_t stride = gridDim.x * WD_FILL_THREADS;
     for (int seg = 0; seg < n_seg; ++seg) {
@@ -103,6 +125,30 @@ __global__ __launch_bounds__(WD_FILL_THREADS) void k_fill_slots(FillSegments f, 
             }
         }
     }
+}
+// The same copy for a launch that has to find room beside a one-launch stack, whose workgroups stay on every compute unit
+// until the stack is through: a workgroup of this kernel takes no LDS, no scratch memory and few registers (a round's
+// three words in named registers, every store unconditional: no private array).  Beside the stack's six waves a SIMD has
+// 32 vector registers left, and of the scalar registers what the stack kernel's own cap leaves (see k_stack_resident):
+// a kernel that needs more of either is not started before the stack has ended, which the stack, waiting for it, never does.
+#ifndef WD_FILL_BESIDE_WGS
+#define WD_FILL_BESIDE_WGS 54   // as many bytes in flight as WD_FILL_WGS workgroups of the other form have
+#endif
+constexpr int kFillBesideUnroll = 3;
+__global__ __launch_bounds__(WD_FILL_THREADS) void k_fill_slots_beside(FillSegments f, int n_seg, FillMarks m) {
+    const uint32_t stride = gridDim.x * WD_FILL_THREADS;
+    for (int seg = 0; seg < n_seg; ++seg) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(f.src[seg]);
+        uint4 *dst = reinterpret_cast<uint4 *>(f.dst[seg]);
+        const uint32_t n = f.words[seg];
+        uint32_t base = blockIdx.x * WD_FILL_THREADS + threadIdx.x;
+        for (; base + 2 * stride < n; base += 3 * stride) {
+            const uint4 a = src[base], b = src[base + stride], c = src[base + 2 * stride];
+            dst[base] = a, dst[base + stride] = b, dst[base + 2 * stride] = c;
+        }
+        for (; base < n; base += stride) dst[base] = src[base];
+    }
+    fill_marks(m);
 }
 
 // One thread, in order: a batch may name the same table entry twice (evicted, then filled again).
@@ -319,6 +365,7 @@ bool find_file_mapping(const void *ptr, wd_file_mapping *out) {
 }
 
 constexpr int kStageRing = 16;  // pinned ring entries of one slot each
+constexpr int kRowsRing = 4, kRowsLayers = 64, kRowsK = 16, kRowsEntry = kRowsLayers * (kRowsK + 1);
 
 }  // namespace
 
@@ -369,6 +416,17 @@ struct wd_expert_cache {
     hipEvent_t ring_free[kUpdateRing] = {};
     bool ring_used[kUpdateRing] = {};
     int ring_next = 0;
+    // One-launch stacks (wd_moe_stack_cached_f32): per token, the slot of every expert of the routing trace and per layer
+    // the number its fills carry, uploaded ahead of the launch; the fills count layers off in d_fill_done.
+    int32_t *h_rows = nullptr, *d_rows = nullptr;   // pinned / device ring [kRowsRing][kRowsLayers * (kRowsK + 1)]
+    hipEvent_t rows_free[kRowsRing] = {};
+    bool rows_used[kRowsRing] = {};
+    int rows_next = 0;
+    uint32_t *d_fill_done = nullptr;                // device [kRowsLayers] numbers, then the fill launches' arrival counter
+    uint32_t fill_seq = 0;                          // the number of the last token whose fills count layers off
+    uint32_t mark_seq = 0;                          // not 0: the token-ahead acquire in progress counts layers off with it
+    std::vector<uint32_t> layer_need;               // per layer: the number to wait for in this token, 0 = nothing on its way
+    uint64_t resident_tokens = 0;                   // tokens that went through the one-launch stack
     wd_expert_cache_stats stats{};
     // monitor (reference: ExpertCacheMonitor, src/expert_cache.cuh:1670-2105)
     std::vector<Shadow> shadows;
@@ -488,6 +546,11 @@ int wd_expert_cache_destroy(wd_expert_cache *c) {
     (void)hipFree(c->d_table);
     (void)hipFree(c->d_updates);
     if (c->h_updates) (void)hipHostFree(c->h_updates);
+    (void)hipFree(c->d_rows);
+    (void)hipFree(c->d_fill_done);
+    if (c->h_rows) (void)hipHostFree(c->h_rows);
+    for (hipEvent_t ev : c->rows_free)
+        if (ev) (void)hipEventDestroy(ev);
     if (c->ev_retire) (void)hipEventDestroy(c->ev_retire);
     for (hipEvent_t ev : c->ev_token)
         if (ev) (void)hipEventDestroy(ev);
@@ -645,7 +708,7 @@ struct AheadState {
     std::vector<int> group;  // layers whose fills are queued but not yet covered by an event
 };
 
-int launch_fill_segments(wd_expert_cache *c, FillSegments &fills, int &n_fill, uint32_t &max_words);
+int launch_fill_segments(wd_expert_cache *c, FillSegments &fills, int &n_fill, uint32_t &max_words, unsigned long long mark_layers = 0ull);
 
 
 // Uploads a batch of slot-table changes and applies them in order on the caller's stream.
@@ -904,12 +967,20 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
     return rc_late;
 }
 
-int launch_fill_segments(wd_expert_cache *c, FillSegments &fills, int &n_fill, uint32_t &max_words) {
-    if (n_fill > 0) {
+int launch_fill_segments(wd_expert_cache *c, FillSegments &fills, int &n_fill, uint32_t &max_words, unsigned long long mark_layers) {
+    if (n_fill > 0 || mark_layers != 0ull) {
         SiteScope site(WD_SITE_CACHE_FILL, c->copy_stream);
         // enough workgroups per segment to keep the host link busy, few enough to leave the decode its compute units
-        const uint32_t per_seg = (max_words + WD_FILL_THREADS * WD_FILL_UNROLL - 1) / (WD_FILL_THREADS * WD_FILL_UNROLL);
-        k_fill_slots<<<dim3(per_seg < WD_FILL_WGS ? (per_seg ? per_seg : 1) : WD_FILL_WGS), dim3(WD_FILL_THREADS), 0, c->copy_stream>>>(fills, n_fill);
+        const bool beside = c->mark_seq != 0u;  // the token goes through a one-launch stack: every fill has to find room beside it
+        const uint32_t round_words = WD_FILL_THREADS * (beside ? kFillBesideUnroll : WD_FILL_UNROLL), most = beside ? WD_FILL_BESIDE_WGS : WD_FILL_WGS;
+        const uint32_t per_seg = (max_words + round_words - 1) / round_words;
+        const dim3 grid(per_seg < most ? (per_seg ? per_seg : 1) : most);
+        if (beside) {
+            const FillMarks marks{mark_layers ? c->d_fill_done : nullptr, reinterpret_cast<unsigned *>(c->d_fill_done + kRowsLayers), mark_layers, c->mark_seq};
+            k_fill_slots_beside<<<grid, dim3(WD_FILL_THREADS), 0, c->copy_stream>>>(fills, n_fill, marks);
+        } else {
+            k_fill_slots<<<grid, dim3(WD_FILL_THREADS), 0, c->copy_stream>>>(fills, n_fill);
+        }
         WD_LAUNCH_CHECK();
     }
     n_fill = 0, max_words = 0;
@@ -917,7 +988,11 @@ int launch_fill_segments(wd_expert_cache *c, FillSegments &fills, int &n_fill, u
 }
 // Launches what the group has collected and records the event its layers wait for.
 int close_ahead_group(wd_expert_cache *c, AheadState &ahead) {
-    if (const int rc = launch_fill_segments(c, ahead.fills, ahead.n_fill, ahead.max_words)) return rc;
+    unsigned long long mark_layers = 0ull;
+    if (c->mark_seq != 0u)
+        for (int l : ahead.group)
+            if (l < kRowsLayers) mark_layers |= 1ull << l, c->layer_need[static_cast<size_t>(l)] = c->mark_seq;
+    if (const int rc = launch_fill_segments(c, ahead.fills, ahead.n_fill, ahead.max_words, mark_layers)) return rc;
     if (!ahead.group.empty()) {
         const int last = ahead.group.back();
         WD_HIP(hipEventRecord(c->ev_layer[last], c->copy_stream));
@@ -980,6 +1055,49 @@ int wait_layer_fills(wd_expert_cache *c, int layer, hipStream_t st) {
         c->last_waited = c->layer_event[layer];
         c->layer_pending[layer] = 0;
     }
+    return WD_OK;
+}
+
+// What a one-launch stack needs beside the pool (allocated at the first such token).
+int rows_prepare(wd_expert_cache *c) {
+    if (c->d_fill_done) return WD_OK;
+    WD_HIP(hipHostMalloc(reinterpret_cast<void **>(&c->h_rows), sizeof(int32_t) * kRowsRing * kRowsEntry, hipHostMallocDefault));
+    WD_HIP(hipMalloc(reinterpret_cast<void **>(&c->d_rows), sizeof(int32_t) * kRowsRing * kRowsEntry));
+    for (hipEvent_t &ev : c->rows_free) WD_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+    uint32_t *done = nullptr;
+    WD_HIP(hipMalloc(reinterpret_cast<void **>(&done), sizeof(uint32_t) * (kRowsLayers + 64)));
+    WD_HIP(hipMemset(done, 0, sizeof(uint32_t) * (kRowsLayers + 64)));
+    c->d_fill_done = done;
+    c->layer_need.assign(kRowsLayers, 0u);
+    return WD_OK;
+}
+
+// Begins a token whose fills count layers off: the number they carry (never 0).
+uint32_t rows_begin_token(wd_expert_cache *c) {
+    if (++c->fill_seq == 0u) ++c->fill_seq;
+    std::fill(c->layer_need.begin(), c->layer_need.end(), 0u);
+    return c->fill_seq;
+}
+
+// After the token's acquire: the slot of every (layer, expert) of h_ids [n_layers][k] and every layer's number, on their
+// way to the device behind the work already on `st`.  rows: [n_layers][k] slot numbers; need: [n_layers].
+int rows_upload(wd_expert_cache *c, int n_layers, const int32_t *h_ids, int k, hipStream_t st, const int32_t **rows, const uint32_t **need) {
+    const int r = c->rows_next;
+    c->rows_next = (r + 1) % kRowsRing;
+    if (c->rows_used[r]) WD_HIP(hipEventSynchronize(c->rows_free[r]));  // the copy that last read this entry is through
+    int32_t *h = c->h_rows + static_cast<size_t>(r) * kRowsEntry, *d = c->d_rows + static_cast<size_t>(r) * kRowsEntry;
+    for (int l = 0; l < n_layers; ++l) {
+        for (int j = 0; j < k; ++j) {
+            const auto it = c->index.find((static_cast<uint64_t>(static_cast<uint32_t>(l)) << 32) | static_cast<uint32_t>(h_ids[l * k + j]));
+            WD_REQUIRE(it != c->index.end(), "expert cache: layer %d expert %d has no slot after its acquire", l, h_ids[l * k + j]);
+            h[l * k + j] = static_cast<int32_t>(it->second);
+        }
+        h[n_layers * k + l] = static_cast<int32_t>(c->layer_need[static_cast<size_t>(l)]);
+    }
+    WD_HIP(hipMemcpyAsync(d, h, sizeof(int32_t) * static_cast<size_t>(n_layers) * (k + 1), hipMemcpyHostToDevice, st));
+    WD_HIP(hipEventRecord(c->rows_free[r], st));
+    c->rows_used[r] = true;
+    *rows = d, *need = reinterpret_cast<const uint32_t *>(d + n_layers * k);
     return WD_OK;
 }
 
@@ -1058,6 +1176,7 @@ size_t wd_expert_cache_dump_json(wd_expert_cache *c, char *buf, size_t cap) {
          ",\"posted\":" + std::to_string(c->ra.requested()) + ",\"dropped\":" + std::to_string(c->ra.dropped()) +
          ",\"delivered\":" + std::to_string(c->ra.delivered()) + ",\"failed\":" + std::to_string(c->ra.failed()) +
          ",\"fills\":" + std::to_string(c->ra_fills) + "}";
+    s += ",\"tokens_in_one_launch\":" + std::to_string(c->resident_tokens);
     s += ",\"prev_token_ready\":" + std::to_string(c->prev_ready);
     s += ",\"prev_token_reuse\":" + fixed(c->prev_ready ? static_cast<double>(c->prev_hit) / c->prev_ready : 0.0, 4);
     s += ",\"layer_access\":" + arr(c->layer_access) + ",\"layer_misses\":" + arr(c->layer_misses);

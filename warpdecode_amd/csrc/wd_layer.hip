@@ -814,9 +814,17 @@ int resident_launch(const ResidentArgs &a, wd_moe_scratch *s, hipStream_t st) {
     return WD_OK;
 }
 
+// Routed experts in a slot pool (see ResidentArgs): the layers' gate/up/down point into the pool, their strides are a slot.
+struct ResidentSlots {
+    const int32_t *rows_trace;   // device [n_layers][k] slot numbers
+    const uint32_t *fill_need;   // device [n_layers]
+    const uint32_t *fill_done;   // device [n_layers]
+    unsigned n_slots;
+};
+
 // Returns kTakePerLayer when the stack has to take the per-layer dispatches instead.
 int stack_resident(const wd_moe_layer *layers, int n_layers, float *d_x, float *d_layer_out, wd_moe_scratch *s,
-                   const int32_t *d_ids_trace, float residual_scale, hipStream_t st) {
+                   const int32_t *d_ids_trace, float residual_scale, hipStream_t st, const ResidentSlots *slots = nullptr) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &cap) != hipSuccess) return kTakePerLayer;
     const bool capturing = cap != hipStreamCaptureStatusNone;
@@ -845,6 +853,11 @@ int stack_resident(const wd_moe_layer *layers, int n_layers, float *d_x, float *
     a.shared = layers[0].shared_gate_inp != nullptr;
     a.gate_stride = layers[0].gate_stride, a.up_stride = layers[0].up_stride, a.down_stride = layers[0].down_stride;
     a.x = d_x, a.out = d_layer_out, a.residual_scale = residual_scale, a.ids_trace = d_ids_trace;
+    a.row_limit = static_cast<unsigned>(a.E);
+    if (slots) {
+        if (!d_ids_trace) return kTakePerLayer;  // (the slots of a layer are known before the launch only with a routing trace)
+        a.rows_trace = slots->rows_trace, a.fill_need = slots->fill_need, a.fill_done = slots->fill_done, a.row_limit = slots->n_slots;
+    }
     a.views = reinterpret_cast<const ResidentViews *>(descriptors + kResMaxLayers);
     a.hand = s->res_block, a.status = s->status, a.spin_limit = s->spin_limit;
     a.status_host = reinterpret_cast<unsigned *>(s->h_ids + 16);

@@ -50,7 +50,18 @@ constexpr int kResXtRow = 68;      // floats per row of the transposed input in 
 constexpr int kResGateSlot = 15;   // word of the weights record that holds the shared expert's sigmoid gate
 constexpr int kResSleepPoll = 2;   // s_sleep between two polls of a wait (flat from 1 to 8 in measurements)
 constexpr int kResSleepFold = 24;  // waves that reach a layer while rung 0 still folds the one before wait this long first
-constexpr int kResPrioRouter = 3, kResPrioWg0 = 2;  // s_setprio of the router waves / of workgroup 0's other waves (measured: 2-4 % each)
+#ifndef WD_RES_SGPRS
+#define WD_RES_SGPRS 96
+#endif
+#ifndef WD_RES_FILL_SLEEPS
+#define WD_RES_FILL_SLEEPS 2
+#endif
+constexpr int kResFillSleeps = WD_RES_FILL_SLEEPS;  // s_sleep 127 (about 4 us each) between two polls of a layer's fills
+#ifndef WD_RES_PRIO_ROUTER
+#define WD_RES_PRIO_ROUTER 3
+#define WD_RES_PRIO_WG0 2
+#endif
+constexpr int kResPrioRouter = WD_RES_PRIO_ROUTER, kResPrioWg0 = WD_RES_PRIO_WG0;  // s_setprio of the router waves / of workgroup 0's other waves (measured: 2-4 % each)
 
 // The bits a value is handed on with: kResEmpty means "not yet written", so that one NaN travels as the default quiet NaN.
 WD_DEV uint32_t hand_word(float v) {
@@ -110,6 +121,14 @@ struct ResidentArgs {
     float *out;                   // [2048] output of the last layer
     float residual_scale;
     const int32_t *ids_trace;     // null, or [n_layers][k]: the experts of every layer (the weights stay the router's)
+    // Routed experts that live in a slot pool (with a routing trace only): the tensors of every layer then start at the
+    // pool, one slot apart, and rows_trace names the slot of every traced expert.  A slot may still be on its way from the
+    // host when the launch begins: fill_need[l] != 0 says that layer l's rows may be read once fill_done[l] has reached
+    // that number (fill_done counts up, one number per token; see k_fill_slots).
+    const int32_t *rows_trace;    // null (the trace's ids address the tensors), or [n_layers][k] slot numbers
+    const uint32_t *fill_need;    // null, or [n_layers]
+    const uint32_t *fill_done;    // [n_layers], written by the fills while the launch runs
+    unsigned row_limit;           // ids (or slot numbers) that address the tensors are below this
     const struct ResidentViews *views;  // device: where the last layer's values go
     uint8_t *hand;   // the hand-off block (kHand* offsets below)
     unsigned *status;
@@ -229,6 +248,24 @@ WD_DEV uint32_t hand_wait4(const ResidentArgs &a, __amdgpu_buffer_rsrc_t rs, uns
     uint32_t v[1];
     hand_wait4<1>(a, rs, off, 0u, each, v, dead);
     return v[0];
+}
+
+// Whether the fills of a layer have reached `need` (numbers wrap: compared as a signed difference).
+WD_DEV bool fill_reached(const ResidentArgs &a, int l, uint32_t need) {
+    const uint32_t got = __hip_atomic_load(a.fill_done + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return static_cast<int32_t>(got - need) >= 0;
+}
+// Returns when they have (all lanes ask for the same word).  A fill takes hundreds of microseconds and crosses the host
+// link: the grid asks seldom (about every 8 us per wave), each unsuccessful poll counting as 32 of the waits' polls.
+WD_DEV void fill_wait(const ResidentArgs &a, int l, uint32_t need, bool &dead) {
+    if (dead) return;
+    unsigned spins = 0;
+    while (!fill_reached(a, l, need)) {
+        spins += 31u;
+        if (res_give_up(a, spins, dead)) return;
+#pragma unroll
+        for (int i = 0; i < kResFillSleeps; ++i) __builtin_amdgcn_s_sleep(127);
+    }
 }
 
 // ---- router row of 2048 columns, weights fetched ahead --------------------------------------------------------
@@ -459,11 +496,15 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
     constexpr int kRow = 8 * ((TYPE == 21) ? 110 : 82);
     const bool shared = a.shared != 0;
     const bool traced = a.ids_trace != nullptr;
-    auto expert_in_range = [&](uint32_t e) { return e < static_cast<uint32_t>(a.E) ? e : 0u; };  // (out of range: a wrong trace, or a wait that ran out)
-    // the expert of this rung in layer l according to the routing trace (any layer number: past the end it is the last layer's)
+    auto expert_in_range = [&](uint32_t e) { return e < a.row_limit ? e : 0u; };  // (out of range: a wrong trace, or a wait that ran out)
+    // the expert of this rung in layer l according to the routing trace, by the number that addresses the tensors
+    // (any layer number: past the end it is the last layer's)
+    const int32_t *const addressed = a.rows_trace ? a.rows_trace : a.ids_trace;
     auto traced_expert = [&](int l, int rung) {
-        return expert_in_range(static_cast<uint32_t>(sld_i32(a.ids_trace + (l < a.n_layers ? l : a.n_layers - 1) * a.k + rung)));
+        return expert_in_range(static_cast<uint32_t>(sld_i32(addressed + (l < a.n_layers ? l : a.n_layers - 1) * a.k + rung)));
     };
+    // fill_need of layer l, 0 when nothing has to be waited for
+    auto fill_needed = [&](int l) { return a.fill_need && l < a.n_layers ? static_cast<uint32_t>(sld_i32(reinterpret_cast<const int32_t *>(a.fill_need) + l)) : 0u; };
     auto gate_up_rows = [&](const uint8_t *gate_base, const uint8_t *up_base, uint32_t e, int r, int lane) {
         const uint8_t *const rows[2] = {gate_base + e * a.gate_stride + static_cast<size_t>(r) * kRow,
                                         up_base + e * a.up_stride + static_cast<size_t>(r) * kRow};
@@ -473,7 +514,11 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
     // registers they arrive in are free from the moment the rows before them lie in LDS), those of the first layer here.
     IqRows8Raw<TYPE, 2> raw;
     raw.u[0] = raw.u[1] = make_uint4(0u, 0u, 0u, 0u);
-    if (traced && slot0 < a.k) raw = gate_up_rows(res_field_s(&a.layers->gate), res_field_s(&a.layers->up), traced_expert(0, slot0), r0, lane0);
+    if (traced && slot0 < a.k) {
+        if (const uint32_t need = fill_needed(0)) fill_wait(a, 0, need, dead);
+        raw = gate_up_rows(res_field_s(&a.layers->gate), res_field_s(&a.layers->up), traced_expert(0, slot0), r0, lane0);
+    }
+    bool rows_asked = true;  // with a routing trace: this layer's gate/up rows were requested during the layer before
     for (int l = 0; l < a.n_layers; ++l) {
         const ResCtx c = res_ctx(lds_base, r0, lane0, wave0, slot0, hb);
         const int r = c.r, lane = c.lane, wave = c.wave, rung = c.slot;
@@ -491,6 +536,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         const uint8_t *const gate_base = res_field_s(traced ? &Ln->gate : &L->gate), *const up_base = res_field_s(traced ? &Ln->up : &L->up);
         uint32_t e = 0, e_next = 0;
         if (traced && on) e = traced_expert(l, rung), e_next = traced_expert(l + 1, rung);
+        const uint32_t need_next = traced && on ? fill_needed(l + 1) : 0u;
         // ---- the layer's input: 16 bytes per lane of waves 0..7, quantised from the registers they arrive in
         if (wave < 8) {
             const int i = wave * 64 + lane;
@@ -529,6 +575,10 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             e = expert_in_range(static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(e)));
             raw = gate_up_rows(gate_base, up_base, e, r, lane);
         }
+        if (traced && on && !rows_asked) {  // the layer's slots were still being filled when the layer before asked
+            fill_wait(a, l, fill_needed(l), dead);
+            raw = gate_up_rows(res_field_s(&L->gate), res_field_s(&L->up), e, r, lane);
+        }
         res_mark<STAMPS>(a, c, l, 4);
 
         // ---- routed rung: gate/up row r, then down rows 4r..4r+3
@@ -547,7 +597,10 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             act = silu_ggml(gu[0]) * gu[1];
             // the next layer's gate/up rows (their registers are free since the rows of this layer lie in LDS; requested
             // behind the dot products, which need every register there is)
-            if (traced) raw = gate_up_rows(gate_base, up_base, e_next, r, lane);
+            if (traced) {
+                rows_asked = need_next == 0u || dead || fill_reached(a, l + 1, need_next);
+                if (rows_asked) raw = gate_up_rows(gate_base, up_base, e_next, r, lane);
+            }
             res_mark<STAMPS>(a, c, l, 5);
         }
         // rung 0 folds the results with the router's weights and the shared expert's gate: published long before this
@@ -714,7 +767,7 @@ WD_DEV void res_router_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         const TopkLds<1> scratch(sel);
         // (both asked for ahead of the logits)
         int id_given = 0;
-        if (traced && r == 0 && lane < a.k) id_given = a.ids_trace[l * a.k + lane];
+        if (traced && r == 0 && lane < a.k) id_given = a.ids_trace[l * a.k + lane];  // (the expert's name, whatever addresses its rows)
         const float w_scale = *const_cast<const volatile float *>(&L->w_scale);
         __syncthreads();  // B1
         res_mark<STAMPS>(a, c, l, 2);
@@ -842,7 +895,11 @@ WD_DEV void res_router_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
 }
 
 template <int TYPE, bool STAMPS>
-__global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 6))) void k_stack_resident(ResidentArgs a) {
+// Registers: six waves per SIMD are resident (two workgroups per compute unit), which leaves a wave 80 vector registers.
+// The scalar registers are capped below what six waves could share out (102 each): at 96 a SIMD keeps scalar registers
+// free for the waves of another stream's small kernel - the copy kernel that fills expert slots while the stack runs
+// found no room beside waves of 106.  (The cap is only honoured when the upper bound of waves_per_eu is above six.)
+__global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 7), amdgpu_num_sgpr(WD_RES_SGPRS))) void k_stack_resident(ResidentArgs a) {
     extern __shared__ __align__(16) uint8_t lds_res[];
     // (the wave's number as a scalar, the lane's counted where it is needed: no vector register is held for the whole launch)
     const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));

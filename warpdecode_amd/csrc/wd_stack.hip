@@ -18,6 +18,8 @@ extern "C" int wd_moe_stack_cached_f32(const wd_moe_layer *layers, int n_layers,
     WD_REQUIRE(n_layers <= cache->n_layers, "cached MoE stack: %d layers exceed the cache's %d", n_layers, cache->n_layers);
     WD_REQUIRE((h_ids_trace == nullptr) == (d_ids_trace == nullptr), "cached MoE stack: the routing trace needs its host and device copy");
     WD_REQUIRE(!(flags & (WD_MOE_ONLY_A | WD_MOE_ONLY_B | WD_MOE_ONLY_C | WD_MOE_STAGED)), "cached MoE stack: unsupported flags");
+    const bool per_layer = (flags & WD_MOE_PER_LAYER) != 0;
+    flags &= ~WD_MOE_PER_LAYER;
     const hipStream_t st = as_stream(stream);
     SiteScope total_site(WD_SITE_STACK_TOTAL, st);
     auto bind = [&](int l) {
@@ -41,7 +43,34 @@ extern "C" int wd_moe_stack_cached_f32(const wd_moe_layer *layers, int n_layers,
     if (token_ahead) {
         if (cache->fills_pending)
             if (const int rc = wait_fills(cache, st)) return rc;
-        if (const int rc = acquire_token_ahead(cache, n_layers, h_ids_trace, k, stream)) return rc;
+        // One launch for the whole stack where its shape allows (wd_resident.cuh): to that launch the pool is one tensor of
+        // slots, the routing trace names slots, and the fills of a layer that are still on their way when the launch begins
+        // count the layer off when they are there (they run beside the launch, on the cache's stream).
+        std::vector<wd_moe_layer> pooled;
+        bool one_launch = !per_layer && flags == 0 && n_layers <= kRowsLayers && k <= kRowsK && cache->n_slots < (1u << 31);
+        if (one_launch) {
+            pooled.assign(layers, layers + n_layers);
+            for (wd_moe_layer &L : pooled) {
+                L.gate = cache->pool, L.up = cache->pool + cache->gate_bytes, L.down = cache->pool + cache->gate_bytes + cache->up_bytes;
+                L.gate_stride = L.up_stride = L.down_stride = cache->slot_bytes;
+                L.slot_of_expert = nullptr, L.slot_pool = nullptr;
+            }
+            one_launch = resident_shape(pooled.data(), n_layers, s, 0) && s->res_fits != 0 && rows_prepare(cache) == WD_OK;
+        }
+        cache->mark_seq = one_launch ? rows_begin_token(cache) : 0u;
+        const int rc_acquire = acquire_token_ahead(cache, n_layers, h_ids_trace, k, stream);
+        cache->mark_seq = 0u;
+        if (rc_acquire) return rc_acquire;
+        if (one_launch) {
+            ResidentSlots slots{};
+            if (const int rc = rows_upload(cache, n_layers, h_ids_trace, k, st, &slots.rows_trace, &slots.fill_need)) return rc;
+            slots.fill_done = cache->d_fill_done, slots.n_slots = static_cast<unsigned>(cache->n_slots);
+            const int rc = stack_resident(pooled.data(), n_layers, d_x, d_layer_out, s, d_ids_trace, residual_scale, st, &slots);
+            if (rc != kTakePerLayer) {
+                if (rc == WD_OK) ++cache->resident_tokens;
+                return rc;
+            }
+        }
         for (int l = 0; l < n_layers; ++l) {
             const wd_moe_layer L = bind(l);
             if (const int rc = wait_layer_fills(cache, l, st)) return rc;
