@@ -74,6 +74,9 @@ def parse():
                          "read from the file into a pinned ring while the layers compute)")
     ap.add_argument("--cache-warm-tokens", type=int, default=256,
                     help="lru mode: tokens run before the warm-up steps so that the slot pool is in steady state")
+    ap.add_argument("--cache-timing", action="store_true",
+                    help="lru mode: switch on the cache's device-side timings (the copy stream's waits and fills, in the monitor "
+                         "object); the events they need cost about 4 % of the rate")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a captured HIP graph")
     ap.add_argument("--path", choices=["resident", "per-layer"], default="resident",
                     help="resident mode: the stack as ONE launch of resident workgroups (default), or two dispatches per layer")
@@ -389,6 +392,8 @@ def bench_lru(args, torch, capi, synth, stack=None):
     st_slots = int(args.cache_gib * (1 << 30)) // slot_bytes
     for policy, slots in ((0, st_slots // 2), (0, 2 * st_slots), (1, st_slots)):   # counterfactual pools, same accesses
         capi.call("wd_expert_cache_add_shadow", cache, policy, slots)
+    if args.cache_timing:
+        capi.call("wd_expert_cache_set_timing", cache, 1)
     scratch = C.c_void_p()
     capi.call("wd_moe_scratch_create", C.byref(scratch), H, F, E, k)
     st0 = capi.CacheStats()

@@ -388,6 +388,15 @@ int wd_expert_cache_add_shadow(wd_expert_cache *c, int policy, size_t slots);
  * needed; writes at most `cap` bytes including the terminator.  reference: ExpertCacheMonitor::dump,
  * src/expert_cache.cuh:1879-1960. */
 size_t wd_expert_cache_dump_json(wd_expert_cache *c, char *buf, size_t cap);
+/* Device-side timings for the dump (off by default; on, every acquire with misses records up to four events on the cache's
+ * copy stream): "io_dma_stall_ms/_max_ms/_calls" - how long the copy stream waited for the last readers of the slots it
+ * was about to overwrite - and "io_dma_ms/_max_ms/_calls" - how long the fills of that acquire (of that group of layers,
+ * when a token is acquired ahead) then took.  Always in the dump, from host clocks: "intra_gap_ms" / "layer_gap_ms", the
+ * time between an acquire's return and the next acquire of the same / of another layer, their per-token means,
+ * "acquire_per_token" and "tokens" (an acquire of a lower layer than the one before begins a token).
+ * reference: StagePool::harvest_timing, src/expert_cache.cuh:1395-1416; ExpertCacheMonitor::note_gap_ms, :1833-1847;
+ * the dump's keys, :1908-1930. */
+int wd_expert_cache_set_timing(wd_expert_cache *c, int enabled);
 
 
 /* One decode step through a stack of layers whose routed experts come from `cache` (layer l of the stack is

@@ -311,6 +311,7 @@ def test_monitor_and_shadow_caches(g):
     capi.call("wd_expert_cache_add_shadow", cache, 0, slots)
     capi.call("wd_expert_cache_add_shadow", cache, 0, 3 * slots)
     capi.call("wd_expert_cache_add_shadow", cache, 1, slots)
+    capi.call("wd_expert_cache_set_timing", cache, 1)
     import torch
     pinned = [[torch.from_numpy(a).pin_memory() for a in layer] for layer in host]
     for l in range(NL):
@@ -339,4 +340,14 @@ def test_monitor_and_shadow_caches(g):
     assert d["shadows"][1]["hits"] == big.hits >= model.hits
     assert d["shadows"][2]["policy"] == "lfu" and 0 < d["shadows"][2]["hits"] <= accesses
     assert d["distinct_pairs"] <= NL * E and 0.0 < d["prev_token_reuse"] < 1.0
+    # the timings: one timed interval per acquire call that missed (every slot's events had passed before the dump), the
+    # copy stream's waits and fills of a few 1 KB experts take microseconds each; 40 passes over 2 layers, all gaps between
+    # two calls are between different layers here
+    missed_calls = d["io_dma_calls"]
+    assert d["io_timing"] is True and 0 < missed_calls <= 40 * NL and d["io_dma_stall_calls"] == missed_calls
+    assert d["io_timing_skipped"] + missed_calls >= 1
+    assert 0.0 < d["io_dma_max_ms"] < 50.0 and d["io_dma_ms"] <= missed_calls * d["io_dma_max_ms"] + 0.1
+    assert 0.0 <= d["io_dma_stall_max_ms"] < 50.0
+    assert d["tokens"] == 40 and d["intra_gap_ms"] == 0.0 and d["layer_gap_ms"] > 0.0
+    assert abs(d["layer_gap_per_token"] - d["layer_gap_ms"] / 40) < 0.011 and d["acquire_per_token"] > 0.0
     capi.call("wd_expert_cache_destroy", cache)

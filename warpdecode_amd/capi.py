@@ -129,6 +129,7 @@ _OPTIONAL = {
     "wd_moe_layer_tokens_pairs_f32": (i32, [C.POINTER(MoeLayer), vp, vp, vp, i32, vp, vp, i32, C.POINTER(vp), u32, vp]),
     "wd_expert_cache_create": (i32, [C.POINTER(vp), sz, sz, sz, sz, i32, i32, i32]),
     "wd_expert_cache_destroy": (i32, [vp]),
+    "wd_expert_cache_set_timing": (i32, [vp, i32]),
     "wd_expert_cache_register_layer": (i32, [vp, i32, vp, vp, vp]),
     "wd_expert_cache_acquire": (i32, [vp, i32, vp, i32, vp, vp]),
     "wd_expert_cache_slot_table": (vp, [vp, i32]),

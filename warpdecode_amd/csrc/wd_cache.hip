@@ -365,6 +365,11 @@ bool find_file_mapping(const void *ptr, wd_file_mapping *out) {
 }
 
 constexpr int kStageRing = 16;  // pinned ring entries of one slot each
+constexpr int kTimingSlots = 32;
+struct TimingSlot {
+    hipEvent_t wait_a = nullptr, wait_b = nullptr, begin = nullptr, end = nullptr;  // all recorded on the copy stream
+    bool used = false, has_wait = false, has_dma = false;
+};
 constexpr int kRowsRing = 4, kRowsLayers = 64, kRowsK = 16, kRowsEntry = kRowsLayers * (kRowsK + 1);
 
 }  // namespace
@@ -427,6 +432,19 @@ struct wd_expert_cache {
     uint32_t mark_seq = 0;                          // not 0: the token-ahead acquire in progress counts layers off with it
     std::vector<uint32_t> layer_need;               // per layer: the number to wait for in this token, 0 = nothing on its way
     uint64_t resident_tokens = 0;                   // tokens that went through the one-launch stack
+    // Timings of the monitor (reference: src/expert_cache.cuh:1395-1416, 1833-1847).  Device side, only when switched on
+    // (wd_expert_cache_set_timing): per acquire with misses (per group of layers in a token-ahead acquire), how long the
+    // copy stream waited for the slots' last readers and how long the fills then took.  Host side, always: the time between
+    // two acquire calls, by whether the layer changed.
+    TimingSlot timing[kTimingSlots];
+    bool timing_on = false;
+    int timing_next = 0, timing_cur = -1;           // timing_cur: the slot of the fills being queued, -1 none
+    double dma_ms = 0.0, dma_max_ms = 0.0, stall_ms = 0.0, stall_max_ms = 0.0;
+    uint64_t dma_calls = 0, stall_calls = 0, timing_skipped = 0;
+    std::chrono::steady_clock::time_point last_acquire_exit{};
+    int last_gap_layer = -1;
+    double intra_gap_ms = 0.0, layer_gap_ms = 0.0;
+    uint64_t tokens_seen = 0;
     wd_expert_cache_stats stats{};
     // monitor (reference: ExpertCacheMonitor, src/expert_cache.cuh:1670-2105)
     std::vector<Shadow> shadows;
@@ -546,6 +564,9 @@ int wd_expert_cache_destroy(wd_expert_cache *c) {
     (void)hipFree(c->d_table);
     (void)hipFree(c->d_updates);
     if (c->h_updates) (void)hipHostFree(c->h_updates);
+    for (TimingSlot &t : c->timing)
+        for (hipEvent_t ev : {t.wait_a, t.wait_b, t.begin, t.end})
+            if (ev) (void)hipEventDestroy(ev);
     (void)hipFree(c->d_rows);
     (void)hipFree(c->d_fill_done);
     if (c->h_rows) (void)hipHostFree(c->h_rows);
@@ -711,6 +732,75 @@ struct AheadState {
 int launch_fill_segments(wd_expert_cache *c, FillSegments &fills, int &n_fill, uint32_t &max_words, unsigned long long mark_layers = 0ull);
 
 
+// ---- device-side timings of the fills (only with c->timing_on) ----------------------------------------------------
+// Intervals whose events have passed are added up and their slots given back.
+void timing_harvest(wd_expert_cache *c) {
+    for (TimingSlot &t : c->timing) {
+        if (!t.used) continue;
+        if (hipEventQuery(t.end) != hipSuccess) {
+            (void)hipGetLastError();
+            continue;
+        }
+        float ms = 0.0f;
+        if (t.has_dma && hipEventElapsedTime(&ms, t.begin, t.end) == hipSuccess) {
+            c->dma_ms += ms, ++c->dma_calls;
+            if (ms > c->dma_max_ms) c->dma_max_ms = ms;
+        }
+        if (t.has_wait && hipEventElapsedTime(&ms, t.wait_a, t.wait_b) == hipSuccess) {
+            c->stall_ms += ms, ++c->stall_calls;
+            if (ms > c->stall_max_ms) c->stall_max_ms = ms;
+        }
+        (void)hipGetLastError();
+        t.used = t.has_wait = t.has_dma = false;
+    }
+}
+// The slot the fills being queued are timed in (opened on demand); null when timing is off or every slot is in flight.
+TimingSlot *timing_slot(wd_expert_cache *c) {
+    if (!c->timing_on) return nullptr;
+    if (c->timing_cur >= 0) return &c->timing[c->timing_cur];
+    for (int pass = 0; pass < 2; ++pass) {
+        for (int i = 0; i < kTimingSlots; ++i) {
+            const int idx = (c->timing_next + i) % kTimingSlots;
+            if (!c->timing[idx].used) {
+                c->timing_cur = idx, c->timing_next = (idx + 1) % kTimingSlots;
+                c->timing[idx].has_wait = c->timing[idx].has_dma = false;
+                return &c->timing[idx];
+            }
+        }
+        timing_harvest(c);
+    }
+    ++c->timing_skipped;
+    return nullptr;
+}
+// Around the copy stream's wait for the slots' last readers.
+void timing_wait_begin(wd_expert_cache *c) {
+    if (TimingSlot *t = timing_slot(c)) (void)hipEventRecord(t->wait_a, c->copy_stream);
+}
+void timing_wait_end(wd_expert_cache *c) {
+    if (c->timing_cur >= 0) {
+        TimingSlot &t = c->timing[c->timing_cur];
+        (void)hipEventRecord(t.wait_b, c->copy_stream);
+        t.has_wait = true;
+    }
+}
+// Before the first copy or copy kernel of the fills being queued.
+void timing_dma_begin(wd_expert_cache *c) {
+    TimingSlot *t = timing_slot(c);
+    if (t && !t->has_dma) {
+        (void)hipEventRecord(t->begin, c->copy_stream);
+        t->has_dma = true;
+    }
+}
+// After their last one.
+void timing_close(wd_expert_cache *c) {
+    if (c->timing_cur < 0) return;
+    TimingSlot &t = c->timing[c->timing_cur];
+    if (!t.has_dma) (void)hipEventRecord(t.begin, c->copy_stream);  // (a wait without fills of its own: an empty interval closes the slot)
+    (void)hipEventRecord(t.end, c->copy_stream);
+    t.used = true;
+    c->timing_cur = -1;
+}
+
 // Uploads a batch of slot-table changes and applies them in order on the caller's stream.
 int flush_slot_updates(wd_expert_cache *c, const SlotUpdate *updates, int n_updates, hipStream_t st) {
     for (int done = 0; done < n_updates; done += kMaxUpdates) {
@@ -744,12 +834,20 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
     hipStream_t st = as_stream(stream);
     SiteScope site(WD_SITE_ACQUIRE, st);
     const auto t_begin = std::chrono::steady_clock::now();
+    if (c->last_gap_layer >= 0) {  // the host's time since the previous acquire returned, by whether the layer changed
+        const double gap = std::chrono::duration<double, std::milli>(t_begin - c->last_acquire_exit).count();
+        (layer == c->last_gap_layer ? c->intra_gap_ms : c->layer_gap_ms) += gap;
+    }
+    if (c->last_gap_layer < 0 || layer < c->last_gap_layer) ++c->tokens_seen;  // (a lower layer than the one before begins a token)
+    c->last_gap_layer = layer;
     struct Timer {
         wd_expert_cache *c;
         std::chrono::steady_clock::time_point t0;
         ~Timer() {
-            c->acquire_ms += std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+            const auto now = std::chrono::steady_clock::now();
+            c->acquire_ms += std::chrono::duration<double, std::milli>(now - t0).count();
             ++c->acquire_calls;
+            c->last_acquire_exit = now;
         }
     } timer{c, t_begin};
     if (c->layer_access.size() < static_cast<size_t>(c->n_layers)) {
@@ -858,12 +956,14 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
         if (!waited) {
             // kernels already queued on the caller's stream may still read the victim slot
             if (!ahead || !ahead->retired) {
+                timing_wait_begin(c);
                 if (ahead && ahead->before) {
                     WD_HIP(hipStreamWaitEvent(c->copy_stream, ahead->before, 0));
                 } else {
                     WD_HIP(hipEventRecord(c->ev_retire, st));
                     WD_HIP(hipStreamWaitEvent(c->copy_stream, c->ev_retire, 0));
                 }
+                timing_wait_end(c);
                 if (ahead) ahead->retired = true;
             }
             waited = true;
@@ -878,6 +978,7 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
         const int shelf = by_file ? c->ra.claim(key) : -1;
         if (shelf >= 0) {
             // a prediction that came true: the slot's bytes are in pinned memory already, laid out like the slot
+            timing_dma_begin(c);
             const hipError_t e1 = hipMemcpyAsync(dst, c->ra.data(shelf), c->slot_bytes, hipMemcpyHostToDevice, c->copy_stream);
             const hipError_t e2 = hipEventRecord(c->ra_done[static_cast<size_t>(shelf)], c->copy_stream);
             c->ra.copy_queued(shelf);  // (also after an error: the event then speaks of whatever was queued before)
@@ -915,6 +1016,7 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
                 break;
             }
             c->pread_ms += std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+            timing_dma_begin(c);
             WD_HIP(hipMemcpyAsync(dst, entry, c->slot_bytes, hipMemcpyHostToDevice, c->copy_stream));
             WD_HIP(hipEventRecord(c->stage_done[r], c->copy_stream));
             c->stage_used[r] = true;
@@ -932,6 +1034,7 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
             }
             ++c->kernel_fills;
         } else {
+            timing_dma_begin(c);
             if (one_piece) {
                 WD_HIP(hipMemcpyAsync(dst, src3[0], c->slot_bytes, hipMemcpyHostToDevice, c->copy_stream));
             } else {
@@ -957,6 +1060,7 @@ int acquire_impl(wd_expert_cache *c, int layer, const int32_t *h_ids, int k, uin
         if (ahead) {
             ahead->group.push_back(layer);  // the event that covers the layer is recorded when its group is closed
         } else {
+            timing_close(c);
             WD_HIP(hipEventRecord(c->ev_done, c->copy_stream));
             if (defer_wait)
                 c->fills_pending = true;
@@ -971,6 +1075,7 @@ int launch_fill_segments(wd_expert_cache *c, FillSegments &fills, int &n_fill, u
     if (n_fill > 0 || mark_layers != 0ull) {
         SiteScope site(WD_SITE_CACHE_FILL, c->copy_stream);
         // enough workgroups per segment to keep the host link busy, few enough to leave the decode its compute units
+        timing_dma_begin(c);
         const bool beside = c->mark_seq != 0u;  // the token goes through a one-launch stack: every fill has to find room beside it
         const uint32_t round_words = WD_FILL_THREADS * (beside ? kFillBesideUnroll : WD_FILL_UNROLL), most = beside ? WD_FILL_BESIDE_WGS : WD_FILL_WGS;
         const uint32_t per_seg = (max_words + round_words - 1) / round_words;
@@ -995,6 +1100,7 @@ int close_ahead_group(wd_expert_cache *c, AheadState &ahead) {
     if (const int rc = launch_fill_segments(c, ahead.fills, ahead.n_fill, ahead.max_words, mark_layers)) return rc;
     if (!ahead.group.empty()) {
         const int last = ahead.group.back();
+        timing_close(c);
         WD_HIP(hipEventRecord(c->ev_layer[last], c->copy_stream));
         for (int l : ahead.group) c->layer_pending[l] = 1, c->layer_event[l] = last;
         ahead.group.clear();
@@ -1145,6 +1251,17 @@ int wd_expert_cache_add_shadow(wd_expert_cache *c, int policy, size_t slots) {
     return WD_OK;
 }
 
+int wd_expert_cache_set_timing(wd_expert_cache *c, int enabled) {
+    WD_REQUIRE(c != nullptr, "expert cache is not initialized");
+    if (enabled && !c->timing[0].end) {
+        for (TimingSlot &t : c->timing)
+            for (hipEvent_t *ev : {&t.wait_a, &t.wait_b, &t.begin, &t.end}) WD_HIP(hipEventCreate(ev));
+    }
+    if (!enabled && c->timing_cur >= 0) timing_close(c);
+    c->timing_on = enabled != 0;
+    return WD_OK;
+}
+
 // JSON object with the counters; returns the length needed (without the terminator), writes at most cap bytes.
 size_t wd_expert_cache_dump_json(wd_expert_cache *c, char *buf, size_t cap) {
     if (!c) return 0;
@@ -1159,6 +1276,8 @@ size_t wd_expert_cache_dump_json(wd_expert_cache *c, char *buf, size_t cap) {
         return std::string(num);
     };
     const wd_expert_cache_stats &st = c->stats;
+    timing_harvest(c);
+    const double tokens = c->tokens_seen ? static_cast<double>(c->tokens_seen) : 1.0;
     std::string s = "{";
     s += "\"mode\":\"" + std::string(c->partitioned ? "layer-partitioned" : "shared") + "\"";
     s += ",\"slots\":" + std::to_string(c->n_slots) + ",\"slot_bytes\":" + std::to_string(c->slot_bytes);
@@ -1176,6 +1295,13 @@ size_t wd_expert_cache_dump_json(wd_expert_cache *c, char *buf, size_t cap) {
          ",\"posted\":" + std::to_string(c->ra.requested()) + ",\"dropped\":" + std::to_string(c->ra.dropped()) +
          ",\"delivered\":" + std::to_string(c->ra.delivered()) + ",\"failed\":" + std::to_string(c->ra.failed()) +
          ",\"fills\":" + std::to_string(c->ra_fills) + "}";
+    s += ",\"io_timing\":" + std::string(c->timing_on ? "true" : "false");
+    s += ",\"io_dma_ms\":" + fixed(c->dma_ms, 1) + ",\"io_dma_max_ms\":" + fixed(c->dma_max_ms, 3) + ",\"io_dma_calls\":" + std::to_string(c->dma_calls);
+    s += ",\"io_dma_stall_ms\":" + fixed(c->stall_ms, 1) + ",\"io_dma_stall_max_ms\":" + fixed(c->stall_max_ms, 3) +
+         ",\"io_dma_stall_calls\":" + std::to_string(c->stall_calls) + ",\"io_timing_skipped\":" + std::to_string(c->timing_skipped);
+    s += ",\"intra_gap_ms\":" + fixed(c->intra_gap_ms, 1) + ",\"layer_gap_ms\":" + fixed(c->layer_gap_ms, 1);
+    s += ",\"intra_gap_per_token\":" + fixed(c->intra_gap_ms / tokens, 2) + ",\"layer_gap_per_token\":" + fixed(c->layer_gap_ms / tokens, 2);
+    s += ",\"acquire_per_token\":" + fixed(c->acquire_ms / tokens, 2) + ",\"tokens\":" + std::to_string(c->tokens_seen);
     s += ",\"tokens_in_one_launch\":" + std::to_string(c->resident_tokens);
     s += ",\"prev_token_ready\":" + std::to_string(c->prev_ready);
     s += ",\"prev_token_reuse\":" + fixed(c->prev_ready ? static_cast<double>(c->prev_hit) / c->prev_ready : 0.0, 4);
