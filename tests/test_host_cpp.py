@@ -42,3 +42,16 @@ def test_expert_prefetcher_host_checks():
     exe = os.path.join(ROOT, "tests", "host", "test_prefetch")
     p = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     assert p.returncode == 0 and " 0 failures" in p.stdout, p.stdout
+
+
+def test_hand_off_word_never_reads_as_not_yet_written():
+    """tests/host/test_handword.cpp: the helper every producer of the resident launch passes its values through - the
+    bit pattern that means "not yet written" (one NaN) leaves as the default quiet NaN, every other NaN and a sweep of
+    all other patterns unchanged."""
+    from warpdecode_amd import build
+    if not os.path.exists(build.LIB):
+        pytest.skip("HIP library not built")
+    build.build_host_test()
+    exe = os.path.join(ROOT, "tests", "host", "test_handword")
+    p = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert p.returncode == 0 and "16777214 NaN patterns" in p.stdout and " 0 failures" in p.stdout, p.stdout

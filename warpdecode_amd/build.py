@@ -41,6 +41,12 @@ def build_host_test(verbose=False):
     if verbose:
         print(" ".join(cmd))
     subprocess.check_call(cmd)
+    # the hand-off word helper of the resident launch: a header of plain C++
+    cmd = ["g++", "-std=c++17", "-O2", "-Wall", "-Wextra", "-I" + CSRC, os.path.join(root, "tests", "host", "test_handword.cpp"),
+           "-o", os.path.join(root, "tests", "host", "test_handword")]
+    if verbose:
+        print(" ".join(cmd))
+    subprocess.check_call(cmd)
     return exe
 
 

@@ -7,7 +7,7 @@
 //   * weights that do not depend on a value still being computed are already on the compute unit when that value
 //     arrives: the router row and the shared expert's rows of layer l + 1 are fetched during layer l; the routed rows
 //     are requested the moment the expert ids are known - with a routing trace (the caller names the experts of every
-//     layer) that is when the layer begins, before its input exists.
+//     layer) a layer ahead, while the rungs still work on the layer before.
 //
 // Geometry (the C2 layer shape): hidden 2048, expert ffn 512, at most 512 experts, top-k <= 10, IQ3_S or IQ2_S gate/up,
 // Q8_0 down, Q8_0 shared expert.  Workgroup r (0..511) has 12 waves:
@@ -16,19 +16,27 @@
 //   one wave          router row r, and the selection
 // and rung 0 folds the eleven results of rows 4r..4r+3 in the reference order and publishes these four values of the
 // next layer's input.
-// The selection.  Every workgroup selects for itself: its router wave pushes its logit into eight copies (one per group of
-// workgroups), gathers the 512 logits of its copy and finds the ids with sel_wave_ids (wd_fused.cuh) - the same logits
-// and the same code in every workgroup, hence the same ids - and hands them to the rungs through LDS.  No workgroup
-// waits for another one's selection, and the ids never cross the device.  Workgroup 0 goes on to the denominator and
-// the weights (sel_wave_finish), which only the fold at the end of the layer needs, and publishes them.  With a routing
-// trace only workgroup 0 gathers the logits (for the weights): the ids are inputs of the launch.
+// The selection is central.  Every router wave hands its logit to workgroup 0 (a 16-byte record per workgroup and
+// layer); workgroup 0's router wave gathers the 512 logits, eight per lane, and ranks them in registers (sel_wave_ids,
+// wd_fused.cuh).  Without a routing trace it publishes the ids at once, in sixteen replicas that the rungs of the grid
+// poll, and only then works out the denominator and the weights, which nothing needs before the fold at the end of the
+// layer.  With a routing trace the ids are inputs of the launch: the rungs request the next layer's gate/up rows while
+// they still work on this one, and workgroup 0 ranks between the barriers of its own activation exchange, so that it never
+// holds up its own rungs (the whole grid waits for the slowest workgroup of a layer).  The shared expert's wave of
+// workgroup 0 computes the softmax denominator meanwhile.  The router waves run at a raised wave priority, as do all
+// waves of workgroup 0: their few instructions are on everybody's critical path.
+// Routed experts in a slot pool (the expert cache's stack, with a routing trace): the pool is addressed as one tensor of
+// slots, a second trace names the slot of every expert, and a layer whose slots are still being filled when the launch
+// begins is waited for inside the launch (fill_need / fill_done in ResidentArgs): the fills run beside the launch on
+// another stream and count the layers off.
 // The float operations and their order are those of the per-layer kernels: results are bit-identical.
 //
 // Hand-off buffers.  Every layer of a launch has its own copy of each buffer, so no word is written twice during a
 // launch.  A word holds kResEmpty (0xffffffff) until its producer stores the value; consumers poll the data words
 // themselves with device-scope loads, so no flag, counter or ordering between stores is needed.  What a workgroup
-// hands on in a layer: its logit (a 16-byte record), its eleven activations (48 bytes) and its four values of the next
-// input (16 bytes), each pushed into eight contiguous copies, one per group of workgroups, each of which polls its own.
+// hands on in a layer: its logit (a 16-byte record that only workgroup 0 reads), its eleven activations (48 bytes) and
+// its four values of the next input (16 bytes), the latter two pushed into eight contiguous copies, one per group of
+// workgroups, each of which polls its own.
 // A line that many compute units write piece by piece while the whole grid polls it changes hands once per write:
 // thirty-two writers per line made a hand-off take 17 us, hence pieces of 16 bytes or more.  A value whose bits are
 // kResEmpty (one particular NaN) is stored as the default quiet NaN instead (hand_word): it would be taken for "not yet".
@@ -39,13 +47,14 @@
 #pragma once
 
 #include "wd_fused.cuh"
+#include "wd_handword.hpp"
 
 namespace wd {
 
 constexpr int kResMaxLayers = 64;
 constexpr int kResWgs = 512, kResWaves = 12, kResThreads = kResWaves * 64;
 constexpr int kResH = 2048, kResF = 512, kResMaxK = 10, kResSharedSlot = 10, kResActSlots = 11;
-constexpr uint32_t kResEmpty = 0xffffffffu;
+constexpr uint32_t kResEmpty = kHandEmpty;
 constexpr int kResXtRow = 68;      // floats per row of the transposed input in LDS (64 + bank spread)
 constexpr int kResGateSlot = 15;   // word of the weights record that holds the shared expert's sigmoid gate
 constexpr int kResSleepPoll = 2;   // s_sleep between two polls of a wait (flat from 1 to 8 in measurements)
@@ -63,11 +72,9 @@ constexpr int kResFillSleeps = WD_RES_FILL_SLEEPS;  // s_sleep 127 (about 4 us e
 #endif
 constexpr int kResPrioRouter = WD_RES_PRIO_ROUTER, kResPrioWg0 = WD_RES_PRIO_WG0;  // s_setprio of the router waves / of workgroup 0's other waves (measured: 2-4 % each)
 
-// The bits a value is handed on with: kResEmpty means "not yet written", so that one NaN travels as the default quiet NaN.
-WD_DEV uint32_t hand_word(float v) {
-    const uint32_t b = f_bits(v);
-    return b == kResEmpty ? 0x7fc00000u : b;
-}
+// The bits a value is handed on with: kResEmpty means "not yet written", so that one NaN travels as the default quiet NaN
+// (wd_handword.hpp, checked on the host).
+WD_DEV uint32_t hand_word(float v) { return hand_word_bits(f_bits(v)); }
 
 struct ResidentLayer {
     const float *router;      // f32 [E][2048]
