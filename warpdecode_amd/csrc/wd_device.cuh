@@ -111,6 +111,9 @@ WD_DEV float silu_ggml(float v) { return v / (1.0f + exp_ggml(-v)); }
 WD_DEV float sigmoid_ggml(float v) { return 1.0f / (1.0f + exp_ggml(-v)); }
 
 WD_DEV int sdot4(uint32_t a, uint32_t b, int acc) {
+    // (Not the three-operand form with a constant 0 through inline assembly, although it saves the move that zeroes the
+    // two-operand form's accumulator: the result of a dot instruction needs wait states before another vector instruction
+    // reads it, which the compiler inserts for instructions it knows and not behind assembly text - results were wrong.)
     return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), acc, false);
 }
 

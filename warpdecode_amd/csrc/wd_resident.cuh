@@ -529,7 +529,9 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
     for (int l = 0; l < a.n_layers; ++l) {
         const ResCtx c = res_ctx(lds_base, r0, lane0, wave0, slot0, hb);
         const int r = c.r, lane = c.lane, wave = c.wave, rung = c.slot;
-        const IqTables &tables = *reinterpret_cast<const IqTables *>(c.lds + kResLdsTables);
+        // (the tables at an LDS address written out as a number - the kernel has no LDS but its dynamic block, which
+        // therefore starts at 0, as the kernel checks when it begins)
+        const IqTablesAt<kResLdsTables> tables;
         const ResidentLayer *L = a.layers + l;
         const bool last = l == a.n_layers - 1;
         const bool on = rung < a.k;
@@ -600,7 +602,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             asm volatile("" : "+s"(e) : : "memory");
             draw = q8_rows4_coal_request<0, 16>(down_base + e * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
             res_mark<STAMPS>(a, c, l, 11);
-            iq_rows8_coal_dots<TYPE, 2>(tables, c.xq(), c.xd(), lane, gu, c.area());
+            iq_rows8_coal_dots<TYPE, 2, false>(tables, c.xq(), c.xd(), lane, gu, c.area());
             act = silu_ggml(gu[0]) * gu[1];
             // the next layer's gate/up rows (their registers are free since the rows of this layer lie in LDS; requested
             // behind the dot products, which need every register there is)
@@ -911,7 +913,13 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 
     // (the wave's number as a scalar, the lane's counted where it is needed: no vector register is held for the whole launch)
     const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
     const int r = blockIdx.x;
-    if (__hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {  // an earlier launch failed
+    // (the codebook lookups address the tables by number: this block of LDS has to be the first thing in the workgroup's LDS)
+    const bool lds_at_zero = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t *)lds_res)) == 0u;
+    if (!lds_at_zero && threadIdx.x == 0) {
+        __hip_atomic_store(a.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (a.status_host) __hip_atomic_store(a.status_host, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+    if (!lds_at_zero || __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {  // or an earlier launch failed
         if (threadIdx.x < 4) a.x[4 * r + threadIdx.x] = a.out[4 * r + threadIdx.x] = __builtin_nanf("");
         return;
     }

@@ -64,6 +64,28 @@ struct IqTables {
     uint32_t grid3[512];
     uint64_t grid2[1024];
     uint2 sign[16];
+    WD_DEV uint32_t grid3_at(uint32_t idx) const { return grid3[idx]; }
+    WD_DEV uint32_t grid3_bytes(uint32_t off) const { return *reinterpret_cast<const uint32_t *>(reinterpret_cast<const uint8_t *>(grid3) + off); }  // off = 4 idx
+    WD_DEV uint64_t grid2_at(uint32_t idx) const { return grid2[idx]; }
+    WD_DEV uint2 sign_at(uint32_t nibble) const { return sign[nibble]; }
+};
+// The same tables for a kernel that knows their LDS byte address when it is compiled (BASE: the address of an IqTables
+// in the workgroup's LDS): a lookup's address is then the scaled index alone, the rest goes into the load's offset field.
+template <unsigned BASE>
+struct IqTablesAt {
+    typedef const __attribute__((address_space(3))) uint32_t *Lds32;
+    typedef const __attribute__((address_space(3))) uint64_t *Lds64;
+    WD_DEV uint32_t grid3_at(uint32_t idx) const {
+        return *(Lds32)(uintptr_t)(BASE + static_cast<unsigned>(offsetof(IqTables, grid3)) + 4u * idx);
+    }
+    WD_DEV uint32_t grid3_bytes(uint32_t off) const { return *(Lds32)(uintptr_t)(BASE + static_cast<unsigned>(offsetof(IqTables, grid3)) + off); }
+    WD_DEV uint64_t grid2_at(uint32_t idx) const {
+        return *(Lds64)(uintptr_t)(BASE + static_cast<unsigned>(offsetof(IqTables, grid2)) + 8u * idx);
+    }
+    WD_DEV uint2 sign_at(uint32_t nibble) const {
+        const uint64_t v = *(Lds64)(uintptr_t)(BASE + static_cast<unsigned>(offsetof(IqTables, sign)) + 8u * nibble);
+        return make_uint2(static_cast<uint32_t>(v), static_cast<uint32_t>(v >> 32));
+    }
 };
 
 template <bool NEED3, bool NEED2>
@@ -138,8 +160,8 @@ WD_DEV IqFields iq_load(const uint8_t *blk, int ib) {
     return f;
 }
 
-template <int TYPE>
-WD_DEV void iq_chunks(const IqFields &f, int ib, const IqTables &t, const uint32_t (&a)[8], int (&p)[8]) {
+template <int TYPE, typename Tables>
+WD_DEV void iq_chunks(const IqFields &f, int ib, const Tables &t, const uint32_t (&a)[8], int (&p)[8]) {
     if (TYPE == 21) {
         const int ls = 1 + 2 * static_cast<int>((f.sc >> (4 * (ib & 1))) & 15u);
         // all sixteen lookups first, the arithmetic after: a lane's block then waits for the LDS once, not eight times
@@ -147,11 +169,12 @@ WD_DEV void iq_chunks(const IqFields &f, int ib, const IqTables &t, const uint32
         uint2 sm[8];
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
-            const uint32_t q = ((c < 4 ? f.qs.x : f.qs.y) >> (8 * (c & 3))) & 0xffu;
-            const uint32_t idx = q | ((f.qh << (8 - c)) & 0x100u);
+            // (the entry's byte offset, 4 (q | high bit << 8), put together from parts that are one instruction each)
+            const uint32_t q4 = (((c < 4 ? f.qs.x : f.qs.y) >> (8 * (c & 3))) & 0xffu) << 2;
+            const uint32_t off = q4 | ((f.qh << (10 - c)) & 0x400u);
             const uint32_t sbits = (f.sg >> (4 * c)) & 15u;  // sign byte c>>1, nibble c&1
-            g[c] = t.grid3[idx];
-            sm[c] = t.sign[sbits];
+            g[c] = t.grid3_bytes(off);
+            sm[c] = t.sign_at(sbits);
         }
 #pragma unroll
         for (int c = 0; c < 8; ++c) p[c] = __mul24(ls, sdot4(apply_signs(g[c], sm[c]), a[c], 0));
@@ -161,11 +184,11 @@ WD_DEV void iq_chunks(const IqFields &f, int ib, const IqTables &t, const uint32
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const uint32_t idx = ((f.qs.x >> (8 * g)) & 0xffu) | ((f.qh << (8 - 2 * g)) & 0x300u);
-            const uint64_t mags = t.grid2[idx];
+            const uint64_t mags = t.grid2_at(idx);
             const uint32_t s8 = (f.qs.y >> (8 * g)) & 0xffu;
             const int ls = (g < 2) ? ls_lo : ls_hi;  // chunks 0..3 low nibble, 4..7 high nibble
-            p[2 * g] = __mul24(ls, sdot4(apply_signs(static_cast<uint32_t>(mags), t.sign[s8 & 15u]), a[2 * g], 0));
-            p[2 * g + 1] = __mul24(ls, sdot4(apply_signs(static_cast<uint32_t>(mags >> 32), t.sign[s8 >> 4]), a[2 * g + 1], 0));
+            p[2 * g] = __mul24(ls, sdot4(apply_signs(static_cast<uint32_t>(mags), t.sign_at(s8 & 15u)), a[2 * g], 0));
+            p[2 * g + 1] = __mul24(ls, sdot4(apply_signs(static_cast<uint32_t>(mags >> 32), t.sign_at(s8 >> 4)), a[2 * g + 1], 0));
         }
     }
 }
@@ -371,8 +394,8 @@ WD_DEV float close_chains_pairs(float v) {
     const float c = b + dpp_f<kDppShr1>(0.0f, b);
     return readlane_f(c, 15);
 }
-template <int TYPE, int NR, bool PART = false>
-WD_DEV void iq_rows8_coal_dots(const IqTables &t, const int8_t *act_qs, const float *act_d, int lane, float (&y)[NR],
+template <int TYPE, int NR, bool PART = false, typename Tables = IqTables>
+WD_DEV void iq_rows8_coal_dots(const Tables &t, const int8_t *act_qs, const float *act_d, int lane, float (&y)[NR],
                                const uint8_t *stage, int32_t *partials = nullptr, size_t pstride = 0) {
     constexpr int kBlk = IqRows8Raw<TYPE, NR>::kBlk;
     const int ib = ((lane >> 4) << 1) | (lane & 1), sb = (lane >> 1) & 7;
