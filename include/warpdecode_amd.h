@@ -216,9 +216,12 @@ int wd_moe_scratch_enable_partials(wd_moe_scratch *s, int gate_type, int down_ty
  * Counterpart of the reference's kernel profiler sites, src/qwen38_moe.cuh:296-535. */
 unsigned long long *wd_moe_scratch_trace(wd_moe_scratch *s, int wg);
 /* The same for the one-launch form of wd_moe_stack_f32: uint64 [12][16] = [wave][point] of workgroup `wg` in layer
- * `layer` (waves 0..9 routed rungs, 10 shared expert, 11 router row; points: 0 layer begin, 1 input seen, 2 input in
- * LDS, 3 logits seen / logit stored, 4 id seen, 5 activation stored, 6 activations seen, 7 down rows done, 8/9 begin
- * and end of the combine).  wg == -1: uint64 [512][4][16], waves 0, 9, 10 and 11 of every workgroup. */
+ * `layer` (which wave has which role depends on the SIMDs the waves landed on; as a rule waves 0..9 are routed rungs,
+ * 10 the shared expert, 11 the router row; points: 0 layer begin, 1 input seen, 2 input in LDS, 3 logit stored,
+ * 4 the rung's expert known (and, without a routing trace, its gate/up rows requested), 5 activation stored,
+ * 6 activations seen, 7 down rows done, 8/9 begin and end of the combine, 10 activation record pushed out, 11 gate/up
+ * rows parked and down rows requested, 12 all logits gathered, 13 ids published, 14 weights published - the last three
+ * in workgroup 0's router wave).  wg == -1: uint64 [512][4][16], waves 0, 9, 10 and 11 of every workgroup. */
 unsigned long long *wd_moe_scratch_trace_resident(wd_moe_scratch *s, int wg, int layer);
 
 /* flags for wd_moe_layer_f32 */
@@ -402,7 +405,11 @@ int wd_expert_cache_set_timing(wd_expert_cache *c, int enabled);
 /* One decode step through a stack of layers whose routed experts come from `cache` (layer l of the stack is
  * layer l of the cache; the slot fields of `layers` are ignored and taken from the cache).  x is updated as in
  * wd_moe_stack_f32.  With a routing trace (host and device copies of int32 [n_layers][top_k]) the fills of the
- * next layer overlap the current layer's dispatches; without one each layer's ids go to the host first, as in
+ * next layer overlap the current layer's dispatches - or, with a pool of at least two tokens' experts and a stack of
+ * the geometry wd_moe_stack_f32 runs as one launch, the whole token is acquired ahead and runs as ONE resident launch
+ * that waits, layer by layer, for the fills still on their way (they run beside it on the cache's stream;
+ * WD_MOE_PER_LAYER in `flags` keeps the dispatches per layer; the results are the same bits).  Without a trace each
+ * layer's ids go to the host first, as in
  * the reference's loop (q38_moe_select_experts_f32_x + GpuExpertCache::acquire per selected expert,
  * src/qwen38_moe.cuh:2323-2380, :3650-3779).  Counters: wd_expert_cache_get_stats. */
 int wd_moe_stack_cached_f32(const wd_moe_layer *layers, int n_layers, wd_expert_cache *cache, float *d_x,
