@@ -774,7 +774,8 @@ def bench_hc(args, torch, capi, synth):
 
 def bench_c0(args, torch, capi, synth):
     """The single-layer parity workload at stack depth: the 64-expert top-8 layer with Q8_0 gate/up/down and no shared expert
-    (hidden 2048, ffn 512), `--layers` independent layers chained as in the headline workload, router-selected."""
+    (hidden 2048, ffn 512), `--layers` independent layers chained as in the headline workload, router-selected.  Up to 64
+    layers run as one resident launch (`--path per-layer`: two dispatches per layer)."""
     H, F, k, E, NL = 2048, 512, 8, 64, args.layers
     g = torch.Generator(device="cuda")
     g.manual_seed(synth.BASE_SEED + 5)
@@ -805,9 +806,11 @@ def bench_c0(args, torch, capi, synth):
     d_x = torch.from_numpy(synth.rms_normed(rng, H)).cuda()
     d_out = torch.zeros(H, dtype=torch.float32, device="cuda")
 
+    per_layer = args.path == "per-layer"
+
     def launch(_i):
         capi.call("wd_moe_stack_f32", layers, NL, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()), scratch, None,
-                  RESIDUAL_SCALE, 0, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+                  RESIDUAL_SCALE, 0x200 if per_layer else 0, C.c_void_p(torch.cuda.current_stream().cuda_stream))
 
     us = graph_period_us(torch, launch, 1, 50) / NL
     ok = bool(torch.isfinite(d_x).all().item()) and capi.load().wd_moe_scratch_status(scratch) == 0
@@ -822,7 +825,8 @@ def bench_c0(args, torch, capi, synth):
                    "layers": NL, "bytes_per_layer": nbytes, "tok_s_at_%d_layers" % NL: round(1e6 / (us * NL), 1), "valid": ok},
         "roofline": dict(bound="hbm", achieved=round(nbytes / us / 1e3, 1), peak=HBM_PEAK_GBS, unit="GB/s",
                          frac=round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), traffic=None,
-                         kernel="whole layer (k_layer_ab<Q8_0>, k_layer_c)")}))
+                         kernel="k_stack_resident<Q8_0> (one launch for the %d layers)" % NL if NL <= 64 and not per_layer else
+                                "whole layer (k_layer_ab<Q8_0>, k_layer_c)")}))
     if not ok:
         sys.exit(1)
 

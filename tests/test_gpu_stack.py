@@ -188,8 +188,9 @@ def _run_stack(g, arr, n, x, tr, sc, flags):
 # The last case is the shape the benchmark measures: 512 experts (every workgroup owns a router row, all eight selecting
 # waves of workgroup 0 hold live logits, the poll of the logit records is full), top-10, a shared expert.
 @pytest.mark.parametrize("gate_type,experts,k,shared,nl", [(synth.IQ3_S, 64, 10, True, 5), (synth.IQ2_S, 40, 6, True, 5),
-                                                           (synth.IQ3_S, 128, 9, False, 5), (synth.IQ3_S, 512, 10, True, 3)],
-                         ids=["iq3s-64x10-shared", "iq2s-40x6-shared", "iq3s-128x9", "iq3s-512x10-shared"])
+                                                           (synth.IQ3_S, 128, 9, False, 5), (synth.IQ3_S, 512, 10, True, 3),
+                                                           (synth.Q8_0, 64, 8, False, 4), (synth.Q8_0, 32, 5, True, 3)],
+                         ids=["iq3s-64x10-shared", "iq2s-40x6-shared", "iq3s-128x9", "iq3s-512x10-shared", "q8-64x8", "q8-32x5-shared"])
 def test_one_launch_stack_matches_per_layer_and_oracle(g, oracle, gate_type, experts, k, shared, nl):
     """The resident launch against the per-layer dispatches (every output and every view of the last layer, bit for
     bit) over launches in a row with stacks of different depth, with and without a routing trace; the first token

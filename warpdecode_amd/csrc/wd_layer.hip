@@ -780,7 +780,7 @@ bool resident_shape(const wd_moe_layer *layers, int n_layers, const wd_moe_scrat
     if (flags != 0 || n_layers > kResMaxLayers || s->gup != nullptr) return false;
     const wd_moe_layer &f = layers[0];
     if (f.hidden != kResH || f.expert_ffn != kResF || f.n_experts > 512 || f.n_experts % 8 != 0 || f.top_k > kResMaxK) return false;
-    if (!consumes_q8k(f.gate_type)) return false;
+    if (!consumes_q8k(f.gate_type) && f.gate_type != WD_TYPE_Q8_0) return false;
     for (int l = 0; l < n_layers; ++l) {
         const wd_moe_layer &L = layers[l];
         if (L.hidden != f.hidden || L.expert_ffn != f.expert_ffn || L.n_experts != f.n_experts || L.top_k != f.top_k) return false;
@@ -862,7 +862,11 @@ int stack_resident(const wd_moe_layer *layers, int n_layers, float *d_x, float *
     a.hand = s->res_block, a.status = s->status, a.spin_limit = s->spin_limit;
     a.status_host = reinterpret_cast<unsigned *>(s->h_ids + 16);
     a.trace = s->trace, a.trace_wg = s->trace_wg, a.trace_layer = s->trace_layer;
-    return layers[0].gate_type == WD_TYPE_IQ3_S ? resident_launch<21>(a, s, st) : resident_launch<22>(a, s, st);
+    switch (layers[0].gate_type) {
+        case WD_TYPE_IQ3_S: return resident_launch<21>(a, s, st);
+        case WD_TYPE_IQ2_S: return resident_launch<22>(a, s, st);
+        default: return resident_launch<8>(a, s, st);  // Q8_0 gate/up rows
+    }
 }
 
 }  // namespace

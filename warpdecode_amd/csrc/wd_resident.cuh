@@ -500,7 +500,11 @@ WD_DEV void res_down(const ResidentArgs &a, const ResCtx &c, int l, const Q8Coal
 template <int TYPE, bool STAMPS>
 WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, int lane0, int wave0, int slot0,
                             __amdgpu_buffer_rsrc_t hb, bool &dead) {
-    constexpr int kRow = 8 * ((TYPE == 21) ? 110 : 82);
+    // TYPE 21 / 22: gate/up rows of eight IQ3_S / IQ2_S super-blocks against the Q8_K form of the input; TYPE 8: Q8_0 rows,
+    // one 34-byte block per lane, against its Q8_0 form (the row routine of the shared expert's wave).
+    constexpr bool kQ8 = TYPE == 8;
+    constexpr int kIq = kQ8 ? 21 : TYPE;  // (the type the super-block routines are instantiated with; unused when kQ8)
+    constexpr int kRow = kQ8 ? 64 * 34 : 8 * ((TYPE == 21) ? 110 : 82);
     const bool shared = a.shared != 0;
     const bool traced = a.ids_trace != nullptr;
     auto expert_in_range = [&](uint32_t e) { return e < a.row_limit ? e : 0u; };  // (out of range: a wrong trace, or a wait that ran out)
@@ -512,18 +516,26 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
     };
     // fill_need of layer l, 0 when nothing has to be waited for
     auto fill_needed = [&](int l) { return a.fill_need && l < a.n_layers ? static_cast<uint32_t>(sld_i32(reinterpret_cast<const int32_t *>(a.fill_need) + l)) : 0u; };
+    IqRows8Raw<kIq, 2> raw;
+    raw.u[0] = raw.u[1] = make_uint4(0u, 0u, 0u, 0u);
+    Q8Block gb[2];
+    gb[0].q0 = gb[0].q1 = gb[1].q0 = gb[1].q1 = make_uint4(0u, 0u, 0u, 0u), gb[0].d = gb[1].d = 0;
+    // requests row r of expert e's gate and up matrix (into raw, or into gb)
     auto gate_up_rows = [&](const uint8_t *gate_base, const uint8_t *up_base, uint32_t e, int r, int lane) {
         const uint8_t *const rows[2] = {gate_base + e * a.gate_stride + static_cast<size_t>(r) * kRow,
                                         up_base + e * a.up_stride + static_cast<size_t>(r) * kRow};
-        return iq_rows8_coal_request<TYPE, 2>(rows, lane);
+        if constexpr (kQ8) {
+            gb[0] = q8_load<0>(rows[0] + lane * 34);
+            gb[1] = q8_load<0>(rows[1] + lane * 34);
+        } else {
+            raw = iq_rows8_coal_request<kIq, 2>(rows, lane);
+        }
     };
     // With a routing trace the gate/up rows of a layer are requested while the layer before decodes its own (the
     // registers they arrive in are free from the moment the rows before them lie in LDS), those of the first layer here.
-    IqRows8Raw<TYPE, 2> raw;
-    raw.u[0] = raw.u[1] = make_uint4(0u, 0u, 0u, 0u);
     if (traced && slot0 < a.k) {
         if (const uint32_t need = fill_needed(0)) fill_wait(a, 0, need, dead);
-        raw = gate_up_rows(res_field_s(&a.layers->gate), res_field_s(&a.layers->up), traced_expert(0, slot0), r0, lane0);
+        gate_up_rows(res_field_s(&a.layers->gate), res_field_s(&a.layers->up), traced_expert(0, slot0), r0, lane0);
     }
     bool rows_asked = true;  // with a routing trace: this layer's gate/up rows were requested during the layer before
     for (int l = 0; l < a.n_layers; ++l) {
@@ -566,8 +578,8 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                 float *dst = c.xt() + (4 * (i & 7)) * kResXtRow + (i >> 3);
                 dst[0] = xv.x, dst[kResXtRow] = xv.y, dst[2 * kResXtRow] = xv.z, dst[3 * kResXtRow] = xv.w;
             }
-            wave_quantize_q8_k_regs(xv, c.xq() + 256 * wave, c.xd() + wave, lane);
-            if (shared) {  // Q8_0: a block is eight lanes
+            if constexpr (!kQ8) wave_quantize_q8_k_regs(xv, c.xq() + 256 * wave, c.xd() + wave, lane);
+            if (shared || kQ8) {  // Q8_0: a block is eight lanes
                 float amax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(xv.x), __builtin_fabsf(xv.y)),
                                              __builtin_fmaxf(__builtin_fabsf(xv.z), __builtin_fabsf(xv.w)));
                 amax = quad_max(amax);
@@ -582,11 +594,11 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         if (!traced && on) {  // the id this rung works on, from one of the replicas workgroup 0 publishes
             e = hand_wait4(a, c.hb, kHandIdh + static_cast<unsigned>(((l * kResIdCopies + (r & (kResIdCopies - 1))) * 16 + rung) * 4), true, dead);
             e = expert_in_range(static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(e)));
-            raw = gate_up_rows(gate_base, up_base, e, r, lane);
+            gate_up_rows(gate_base, up_base, e, r, lane);
         }
         if (traced && on && !rows_asked) {  // the layer's slots were still being filled when the layer before asked
             fill_wait(a, l, fill_needed(l), dead);
-            raw = gate_up_rows(res_field_s(&L->gate), res_field_s(&L->up), e, r, lane);
+            gate_up_rows(res_field_s(&L->gate), res_field_s(&L->up), e, r, lane);
         }
         res_mark<STAMPS>(a, c, l, 4);
 
@@ -594,7 +606,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         float act = 0.0f;
         if (on) {
             float gu[2] = {1.0f, 1.0f};
-            iq_rows8_coal_park<TYPE, 2>(raw, lane, c.area());
+            if constexpr (!kQ8) iq_rows8_coal_park<kIq, 2>(raw, lane, c.area());
             // Nothing below may be requested before the gate/up rows are here (the wave's loads return in order, and
             // requested together, the down rows of the waves served first would delay the gate/up rows of the others,
             // which the whole grid waits for): the expert's number passes through a statement the compiler cannot
@@ -602,13 +614,20 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             asm volatile("" : "+s"(e) : : "memory");
             draw = q8_rows4_coal_request<0, 16>(down_base + e * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
             res_mark<STAMPS>(a, c, l, 11);
-            iq_rows8_coal_dots<TYPE, 2, false>(tables, c.xq(), c.xd(), lane, gu, c.area());
+            if constexpr (kQ8) {
+                Q8RowTile &tile = *reinterpret_cast<Q8RowTile *>(c.area());
+                float acc[2] = {0.0f, 0.0f};
+                q8_row_wave_pass<2>(gb, true, lane, c.x0q(), c.x0d(), tile, lane, acc);
+                gu[0] = close_lanes8(acc[0]), gu[1] = close_lanes8(acc[1]);
+            } else {
+                iq_rows8_coal_dots<kIq, 2, false>(tables, c.xq(), c.xd(), lane, gu, c.area());
+            }
             act = silu_ggml(gu[0]) * gu[1];
             // the next layer's gate/up rows (their registers are free since the rows of this layer lie in LDS; requested
             // behind the dot products, which need every register there is)
             if (traced) {
                 rows_asked = need_next == 0u || dead || fill_reached(a, l + 1, need_next);
-                if (rows_asked) raw = gate_up_rows(gate_base, up_base, e_next, r, lane);
+                if (rows_asked) gate_up_rows(gate_base, up_base, e_next, r, lane);
             }
             res_mark<STAMPS>(a, c, l, 5);
         }
