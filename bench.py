@@ -47,7 +47,7 @@ def parse():
     ap.add_argument("--experts", type=int, default=512)
     ap.add_argument("--routing", choices=["zipf", "router"], default="zipf",
                     help="zipf: ids replayed from the Zipf(1.1) trace; router: ids chosen by the router itself")
-    ap.add_argument("--mode", choices=["resident", "lru", "q4-sweep", "q8-sweep", "q6k-head", "hc", "tokens", "c0", "model-layer"], default="resident",
+    ap.add_argument("--mode", choices=["resident", "lru", "q4-sweep", "q8-sweep", "q8-batch", "q6k-head", "hc", "tokens", "c0", "model-layer"], default="resident",
                     help="resident: C3 mode A, every expert in HBM; lru: C3 mode B, experts in pinned host memory "
                          "behind an LRU slot pool of --cache-gib in HBM; q4-sweep: the dense Q4_0 GEMV shapes; "
                          "tokens: the 4-token speculative-verify pass over the same layers; c0: the 64-expert top-8 "
@@ -683,6 +683,72 @@ def bench_q8_sweep(args, torch, capi, synth):
                          kernel="k_gemv_q8_rows8", us_per_launch=head["us_per_gemv"], bytes_per_launch=head["bytes"])}))
 
 
+def bench_q8_batch(args, torch, capi, synth):
+    """The middle sizes of the exact-order Q8_0 GEMV as a block issues them: ten projections of one shape on one activation,
+    as ten launches and as ONE launch (wd_gemv_q8_0_batch_f32).  Every launch of a chain reads another copy of its
+    matrices (>= 1.5 GB of copies), the period is taken over a captured chain."""
+    n_items = 10
+    results = []
+    for rows, cols in [(2048, 2048), (1024, 4096), (512, 8192), (512, 2048)]:
+        nbytes = rows * synth.row_bytes(synth.Q8_0, cols)
+        sets = max(2, -(-int(1.5e9) // (nbytes * n_items)))
+        one = torch.from_numpy(synth.matrix(synth.Q8_0, synth.rng_for(synth.BASE_SEED, 83, rows, cols), rows, cols)).reshape(-1).cuda()
+        w = one.repeat(sets * n_items).reshape(sets, n_items, nbytes)
+        x = torch.from_numpy(synth.rng_for(synth.BASE_SEED, 84, cols).normal(0, 1, cols).astype(np.float32)).cuda()
+        qs = torch.empty(cols, dtype=torch.int8, device="cuda")
+        sc = torch.empty(cols // 32, dtype=torch.int16, device="cuda")
+        y = torch.empty((n_items, rows), dtype=torch.float32, device="cuda")
+        y1 = torch.empty((n_items, rows), dtype=torch.float32, device="cuda")
+        stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        vp = lambda t: C.c_void_p(t.data_ptr())
+        capi.call("wd_q8_0_quantize_f32", vp(x), cols, vp(qs), vp(sc), stream())
+        tables = []
+        for s_ in range(sets):
+            items = (capi.GemvItem * n_items)()
+            for i in range(n_items):
+                items[i].d_w, items[i].rows, items[i].d_act_qs, items[i].d_act_scales, items[i].d_out = (
+                    w[s_, i].data_ptr(), rows, qs.data_ptr(), sc.data_ptr(), y[i].data_ptr())
+            tables.append(items)
+
+        def batched(j):
+            capi.call("wd_gemv_q8_0_batch_f32", synth.Q8_0, tables[j % sets], n_items, cols, stream())
+
+        def single(j):
+            for i in range(n_items):
+                capi.call("wd_gemv_q8_0_f32", synth.Q8_0, C.c_void_p(w[j % sets, i].data_ptr()), rows, cols, vp(qs), vp(sc), vp(y1[i]),
+                          None, stream())
+
+        batched(0)
+        single(0)
+        torch.cuda.synchronize()
+        same = bool(torch.equal(y.view(torch.int32), y1.view(torch.int32)))
+        launches = max(sets, 8)
+        reps = max(3, int(1e11 // (nbytes * n_items * launches)))
+        us_b = graph_period_us(torch, batched, launches, reps)
+        us_s = graph_period_us(torch, single, launches, reps)
+        results.append(dict(rows=rows, cols=cols, items=n_items, bytes_per_item=nbytes, sets=sets, same_bits=same,
+                            us_per_gemv_batched=round(us_b / n_items, 3), us_per_gemv_single=round(us_s / n_items, 3),
+                            gbs_batched=round(nbytes * n_items / us_b / 1e3, 1), gbs_single=round(nbytes * n_items / us_s / 1e3, 1),
+                            frac_batched=round(nbytes * n_items / us_b / 1e3 / HBM_PEAK_GBS, 4),
+                            frac_single=round(nbytes * n_items / us_s / 1e3 / HBM_PEAK_GBS, 4)))
+        note("Q8_0 %dx%d x %d: %.2f us per GEMV in one launch (%.0f GB/s), %.2f us one launch each (%.0f GB/s), same bits %s"
+             % (rows, cols, n_items, us_b / n_items, nbytes * n_items / us_b / 1e3, us_s / n_items, nbytes * n_items / us_s / 1e3, same))
+        del w, one
+        torch.cuda.empty_cache()
+    head = results[0]
+    print(json.dumps({
+        "metric": "ten exact-order Q8_0 GEMVs 2048x2048 in one launch, batch=1: achieved HBM GB/s", "value": head["gbs_batched"],
+        "unit": "GB/s", "n_gpus": 1, "higher_is_better": True, "vs_baseline": None, "dtype": "int8 dot products, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "the middle sizes of the exact-order Q8_0 x Q8_0 GEMV, ten projections per launch against ten launches",
+                   "shapes": results, "valid": all(r["same_bits"] for r in results)},
+        "roofline": dict(bound="hbm", achieved=head["gbs_batched"], peak=HBM_PEAK_GBS, unit="GB/s", frac=head["frac_batched"],
+                         traffic=None, kernel="k_gemv_q8_rows8_split_batch", us_per_launch=round(head["us_per_gemv_batched"] * n_items, 3),
+                         bytes_per_launch=head["bytes_per_item"] * n_items)}))
+    if not all(r["same_bits"] for r in results):
+        sys.exit(1)
+
+
 def bench_q6k_head(args, torch, capi, synth):
     """The output head of the Qwen3 MoE models: Q6_K 151936 x 2048 against the Q8_K image of the F32 activation, once
     per decoded token.  Every launch of a chain reads another copy of the matrix (7 copies, 1.8 GB) so that nothing
@@ -921,6 +987,8 @@ def main():
         return bench_q4_sweep(args, torch, capi, synth)
     if args.mode == "q8-sweep":
         return bench_q8_sweep(args, torch, capi, synth)
+    if args.mode == "q8-batch":
+        return bench_q8_batch(args, torch, capi, synth)
     if args.mode == "c0":
         return bench_c0(args, torch, capi, synth)
     if args.mode == "model-layer":

@@ -218,6 +218,58 @@ def test_q8_0_gemv_misaligned_base(g, oracle):
     assert g.same_bits(g.host(out), want) and g.same_bits(g.host(out_s), want)
 
 
+# cols, then the rows of every item: the projections of a block on one activation (2048 columns), the long rows of a down
+# projection (8192), a list longer than one launch takes (18 items), and lists with items the shared kernel does not
+# take (fewer than 8 rows; 8192 rows and more; a base 2 bytes into an allocation), which are launched by themselves
+@pytest.mark.parametrize("cols,rows_list,shift", [(2048, [2048, 512, 512, 1024, 64, 2048], None), (8192, [512, 256, 2048], None),
+                                                  (4096, [1024] * 18, None), (2048, [96, 5, 8192, 40, 8], None),
+                                                  (1024, [48, 16, 200], None), (2048, [256, 77, 128], 1)],
+                         ids=["2048-projections", "8192-down", "18-items", "odd-ones-out", "1024-general-kernel", "misaligned-item"])
+def test_q8_0_gemv_batch(g, oracle, cols, rows_list, shift):
+    """wd_gemv_q8_0_batch_f32 against the same matrices one call each (the same bits) and against the oracle; two
+    activations shared out over the items."""
+    import torch
+    rng = synth.rng_for(SEED, 29, cols, len(rows_list))
+    acts = []
+    for a in range(2):
+        x = rng.normal(0, 1, cols).astype(np.float32)
+        qs, d = oracle.quantize_q8_0(x)
+        acts.append((qs, d, g.dev(qs), g.dev(d)))
+    items = (capi.GemvItem * len(rows_list))()
+    keep, singles, wants = [], [], []
+    for i, rows in enumerate(rows_list):
+        w = synth.matrix(synth.Q8_0, rng, rows, cols)
+        qs, d, dq, dd = acts[i % 2]
+        if shift == i:
+            buf = torch.zeros(w.size + 16, dtype=torch.uint8, device="cuda")
+            buf[2:2 + w.size] = g.dev(w).reshape(-1)
+            wptr = buf.data_ptr() + 2
+        else:
+            buf = g.dev(w)
+            wptr = buf.data_ptr()
+        out, single = g.empty(rows, np.float32), g.empty(rows, np.float32)
+        keep.append((buf, out))
+        singles.append(single)
+        items[i].d_w, items[i].rows, items[i].d_act_qs, items[i].d_act_scales, items[i].d_out = wptr, rows, dq.data_ptr(), dd.data_ptr(), out.data_ptr()
+        capi.call("wd_gemv_q8_0_f32", synth.Q8_0, wptr, rows, cols, g.ptr(dq), g.ptr(dd), g.ptr(single), None, g.stream())
+        wants.append(oracle.gemv(synth.Q8_0, w, rows, cols, qs, d))
+    capi.call("wd_gemv_q8_0_batch_f32", synth.Q8_0, items, len(rows_list), cols, g.stream())
+    g.sync()
+    for i, rows in enumerate(rows_list):
+        got = g.host(keep[i][1])
+        assert g.same_bits(got, g.host(singles[i])), (i, rows)
+        assert g.same_bits(got, wants[i]), (i, rows)
+
+
+def test_q8_0_gemv_batch_refuses_what_it_cannot_take(g):
+    items = (capi.GemvItem * 1)()
+    lib = capi.load()
+    assert lib.wd_gemv_q8_0_batch_f32(synth.Q4_0, items, 1, 2048, g.stream()) != 0      # exact-order Q8_0 only
+    assert lib.wd_gemv_q8_0_batch_f32(synth.Q8_0, items, 0, 2048, g.stream()) != 0      # no items
+    assert lib.wd_gemv_q8_0_batch_f32(synth.Q8_0, items, 1, 2040, g.stream()) != 0      # not whole blocks
+    assert lib.wd_gemv_q8_0_batch_f32(synth.Q8_0, items, 1, 2048, g.stream()) != 0      # null pointers in the item
+
+
 def test_q4_0_gemv_misaligned_base(g, oracle):
     """A matrix that starts 2 bytes into an allocation (GGUF blocks are only 2-byte aligned) takes the general
     kernel instead of the streaming one; both must give the same block sums."""

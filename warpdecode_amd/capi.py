@@ -25,6 +25,11 @@ class WdError(RuntimeError):
     pass
 
 
+class GemvItem(C.Structure):
+    """wd_gemv_item: one matrix of a batched exact-order Q8_0 GEMV."""
+    _fields_ = [("d_w", vp), ("rows", i32), ("d_act_qs", vp), ("d_act_scales", vp), ("d_out", vp)]
+
+
 class MoeLayer(C.Structure):
     _fields_ = [
         ("hidden", i32), ("expert_ffn", i32), ("n_experts", i32), ("top_k", i32),
@@ -92,6 +97,7 @@ _SIGS = {
     "wd_topk_softmax": (i32, [vp, i32, i32, f32, vp, vp, vp]),
     "wd_gemv_q8_k_f32": (i32, [i32, vp, i32, i32, vp, vp, vp, vp, vp]),
     "wd_gemv_q8_0_f32": (i32, [i32, vp, i32, i32, vp, vp, vp, vp, vp]),
+    "wd_gemv_q8_0_batch_f32": (i32, [i32, vp, i32, i32, vp]),
     "wd_gemv_q8_k_experts_f32": (i32, [i32, vp, i32, i32, i32, vp, vp, vp, vp, vp]),
     "wd_gemv_q8_0_experts_f32": (i32, [i32, vp, i32, i32, i32, vp, vp, vp, vp, vp]),
     "wd_silu_mul_experts_f32": (i32, [vp, vp, i32, i32, vp]),

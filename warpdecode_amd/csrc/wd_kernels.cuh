@@ -586,10 +586,11 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(WAVE
 // their parts of the chains one after the other, handing the 64 accumulators on through LDS: NCH*KB dependent fma per
 // wave, nothing else.  Lane = 8 row + chain as in k_gemv_q8_rows8; nb = KB NCH WAVES blocks per row (KB = 16 or 32).
 // dynamic LDS: cols bytes, cols/32 floats, 256 bytes of accumulators, then one stage of 8 * kQ8sRowStride<KB> per wave.
+// (the body: `group` is the workgroup's group of eight rows)
 template <int KB, int NCH, int WAVES, bool PART>
-__global__ __launch_bounds__(64 * WAVES) void k_gemv_q8_rows8_split(const uint8_t *__restrict__ w, int rows, int nb,
-                                                              const int8_t *__restrict__ act_qs, const uint16_t *__restrict__ act_d,
-                                                              float *__restrict__ out, int32_t *__restrict__ partials) {
+WD_DEV void gemv_q8_rows8_split_body(const uint8_t *__restrict__ w, int rows, int nb, const int8_t *__restrict__ act_qs,
+                                     const uint16_t *__restrict__ act_d, float *__restrict__ out, int32_t *__restrict__ partials,
+                                     int group) {
     constexpr int SEG = NCH * KB;
     using Fetch = Q8sFetch<KB>;
     constexpr int RS = kQ8sRowStride<KB>;
@@ -603,7 +604,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_gemv_q8_rows8_split(const uint8_
     const size_t rb = static_cast<size_t>(nb) * 34;
     const int row = lane >> 3, c = lane & 7;
     // a last group of fewer than eight rows is moved up to end with the matrix (rows >= 8)
-    const int base_row = min(8 * static_cast<int>(blockIdx.x), rows - 8);
+    const int base_row = min(8 * group, rows - 8);
     const uint8_t *src = uniform_ptr(w + static_cast<size_t>(base_row) * rb + static_cast<size_t>(wave) * (34 * SEG));
     uint32_t loff[Fetch::kLoads];
     Fetch f[NCH];
@@ -669,6 +670,34 @@ __global__ __launch_bounds__(64 * WAVES) void k_gemv_q8_rows8_split(const uint8_
         const float y = close_lanes8(acc);
         if (c == 0) out[base_row + row] = y;
     }
+}
+template <int KB, int NCH, int WAVES, bool PART>
+__global__ __launch_bounds__(64 * WAVES) void k_gemv_q8_rows8_split(const uint8_t *__restrict__ w, int rows, int nb,
+                                                              const int8_t *__restrict__ act_qs, const uint16_t *__restrict__ act_d,
+                                                              float *__restrict__ out, int32_t *__restrict__ partials) {
+    gemv_q8_rows8_split_body<KB, NCH, WAVES, PART>(w, rows, nb, act_qs, act_d, out, partials, static_cast<int>(blockIdx.x));
+}
+// Several matrices of the same row length in ONE launch (the projections a block applies to one or a few activations:
+// each of them alone is bound by its launch, not by its bytes).  Workgroup b belongs to the item whose range of row
+// groups holds b; what it computes is what k_gemv_q8_rows8_split computes for that item alone.
+constexpr int kGemvBatchMax = 16;
+struct GemvBatch {
+    const uint8_t *w[kGemvBatchMax];
+    const int8_t *act_qs[kGemvBatchMax];
+    const uint16_t *act_d[kGemvBatchMax];
+    float *out[kGemvBatchMax];
+    int rows[kGemvBatchMax];
+    int first_group[kGemvBatchMax + 1];  // first_group[n]: all groups
+    int n;
+};
+template <int KB, int NCH, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void k_gemv_q8_rows8_split_batch(GemvBatch b, int nb) {
+    int item = 0;
+    for (int i = 1; i < b.n; ++i)
+        if (static_cast<int>(blockIdx.x) >= b.first_group[i]) item = i;
+    item = __builtin_amdgcn_readfirstlane(item);
+    gemv_q8_rows8_split_body<KB, NCH, WAVES, false>(b.w[item], b.rows[item], nb, b.act_qs[item], b.act_d[item], b.out[item], nullptr,
+                                                   static_cast<int>(blockIdx.x) - b.first_group[item]);
 }
 
 // ---- Q6_K x Q8_K GEMV: the waves of the grid take the rows in turn, pass by pass, one pass fetched ahead -------

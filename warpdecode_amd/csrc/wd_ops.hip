@@ -224,6 +224,21 @@ static int launch_gemv_q8k(int type, MatSrc src, int mats, int rows, int cols, c
     return WD_OK;
 }
 
+// The split configuration of the streaming kernel for rows of nb blocks in `groups` groups of eight rows; null when the
+// kernel for that shape is another one.
+struct Q8Split { int nb, kb, nch, waves; };
+static const Q8Split *q8_split_for(int nb, int groups) {
+    static const Q8Split kSplits[] = {{64, 32, 1, 2}, {80, 16, 1, 5}, {128, 32, 1, 4}, {160, 32, 1, 5}, {256, 32, 1, 8},
+                                      {256, 32, 2, 4}, {320, 32, 2, 5}, {512, 32, 2, 8}};
+    for (const Q8Split &sp : kSplits) {
+        if (groups >= 1024 || sp.nb != nb) continue;
+        // 8192 columns: eight waves when a compute unit gets one workgroup, four (two chunks each) when it gets more
+        if (nb == 256 && (sp.waves == 8) != (groups <= 256)) continue;
+        return &sp;
+    }
+    return nullptr;
+}
+
 static int launch_gemv_q8_0(int type, MatSrc src, int mats, int rows, int cols, const int8_t *qs, const uint16_t *d,
                             int act_per_mat, float *out, int32_t *partials, hipStream_t stream) {
     WD_REQUIRE(type == WD_TYPE_Q8_0 || type == WD_TYPE_IQ4_NL || type == WD_TYPE_Q4_0,
@@ -264,13 +279,8 @@ static int launch_gemv_q8_0(int type, MatSrc src, int mats, int rows, int cols, 
         // whole 16-byte words per row chunk and a 16-byte aligned base: the streaming kernel, eight rows per wave
         const int groups = (rows + 7) / 8;
         // few row groups: the waves of a workgroup share a group, the chain runs over prepared pairs
-        struct Split { int nb, kb, nch, waves; };
-        static const Split kSplits[] = {{64, 32, 1, 2}, {80, 16, 1, 5}, {128, 32, 1, 4}, {160, 32, 1, 5}, {256, 32, 1, 8},
-                                        {256, 32, 2, 4}, {320, 32, 2, 5}, {512, 32, 2, 8}};
-        for (const Split &sp : kSplits) {
-            if (groups >= 1024 || sp.nb != nb) continue;
-            // 8192 columns: eight waves when a compute unit gets one workgroup, four (two chunks each) when it gets more
-            if (nb == 256 && (sp.waves == 8) != (groups <= 256)) continue;
+        if (const Q8Split *found = q8_split_for(nb, groups)) {
+            const Q8Split &sp = *found;
             const size_t lds = static_cast<size_t>(cols) + static_cast<size_t>(nb) * 4 + 256 +
                                static_cast<size_t>(sp.waves) * 8 * (sp.kb == 32 ? kQ8sRowStride<32> : kQ8sRowStride<16>);
             auto launch = [&](auto kernel) { kernel<<<groups, 64 * sp.waves, lds, stream>>>(src.single, rows, nb, qs, d, out, partials); };
@@ -370,6 +380,67 @@ int wd_gemv_q8_0_f32(int type, const uint8_t *d_w, int rows, int cols, const int
     MatSrc src{};
     src.single = d_w;
     return launch_gemv_q8_0(type, src, 1, rows, cols, d_act_qs, d_act_scales, 0, d_out, d_partials, as_stream(stream));
+}
+
+int wd_gemv_q8_0_batch_f32(int type, const wd_gemv_item *items, int n_items, int cols, void *stream) {
+    WD_REQUIRE(type == WD_TYPE_Q8_0, "batched GEMV: exact-order Q8_0 matrices only (type %d)", type);
+    WD_REQUIRE(items != nullptr && n_items > 0, "batched GEMV: no items");
+    WD_REQUIRE(cols > 0 && cols % 32 == 0, "batched GEMV: invalid row length %d", cols);
+    for (int i = 0; i < n_items; ++i)
+        WD_REQUIRE(items[i].d_w && items[i].d_act_qs && items[i].d_act_scales && items[i].d_out && items[i].rows > 0,
+                   "batched GEMV: item %d has a null pointer or no rows", i);
+    const int nb = cols / 32;
+    // One launch for as many items in a row as take the same kernel: every item must be a shape the split kernel takes
+    // alone (then its workgroups do here exactly what they do there); anything else is launched by itself.
+    auto splits_alike = [&](const wd_gemv_item &it, const Q8Split *want) {
+        const Q8Split *sp = nb % 16 == 0 && cols <= 16384 && it.rows >= 8 && reinterpret_cast<uintptr_t>(it.d_w) % 16 == 0 &&
+                                    reinterpret_cast<uintptr_t>(it.d_act_qs) % 16 == 0
+                                ? q8_split_for(nb, (it.rows + 7) / 8)
+                                : nullptr;
+        return sp != nullptr && (want == nullptr || sp == want) ? sp : nullptr;
+    };
+    int i = 0;
+    while (i < n_items) {
+        const Q8Split *sp = splits_alike(items[i], nullptr);
+        int j = i + 1;
+        if (sp)
+            while (j < n_items && j - i < kGemvBatchMax && splits_alike(items[j], sp)) ++j;
+        if (!sp || j - i == 1) {
+            if (const int rc = wd_gemv_q8_0_f32(type, items[i].d_w, items[i].rows, cols, items[i].d_act_qs, items[i].d_act_scales,
+                                                items[i].d_out, nullptr, stream))
+                return rc;
+            ++i;
+            continue;
+        }
+        GemvBatch b{};
+        b.n = j - i;
+        int groups = 0;
+        for (int q = 0; q < b.n; ++q) {
+            const wd_gemv_item &it = items[i + q];
+            b.w[q] = it.d_w, b.act_qs[q] = it.d_act_qs, b.act_d[q] = it.d_act_scales, b.out[q] = it.d_out, b.rows[q] = it.rows;
+            b.first_group[q] = groups;
+            groups += (it.rows + 7) / 8;
+        }
+        for (int q = b.n; q <= kGemvBatchMax; ++q) b.first_group[q] = groups;
+        const size_t lds = static_cast<size_t>(cols) + static_cast<size_t>(nb) * 4 + 256 +
+                           static_cast<size_t>(sp->waves) * 8 * (sp->kb == 32 ? kQ8sRowStride<32> : kQ8sRowStride<16>);
+        const hipStream_t st = as_stream(stream);
+#define WD_Q8_BATCH(KB_, NCH_, WAVES_)                                    \
+    if (sp->kb == KB_ && sp->nch == NCH_ && sp->waves == WAVES_)          \
+        k_gemv_q8_rows8_split_batch<KB_, NCH_, WAVES_><<<groups, 64 * WAVES_, lds, st>>>(b, nb);
+        WD_Q8_BATCH(32, 1, 2)
+        WD_Q8_BATCH(16, 1, 5)
+        WD_Q8_BATCH(32, 1, 4)
+        WD_Q8_BATCH(32, 1, 5)
+        WD_Q8_BATCH(32, 1, 8)
+        WD_Q8_BATCH(32, 2, 4)
+        WD_Q8_BATCH(32, 2, 5)
+        WD_Q8_BATCH(32, 2, 8)
+#undef WD_Q8_BATCH
+        WD_LAUNCH_CHECK();
+        i = j;
+    }
+    return WD_OK;
 }
 
 int wd_gemv_q8_k_experts_f32(int type, const uint8_t *const *d_w_experts, int experts, int rows, int cols,

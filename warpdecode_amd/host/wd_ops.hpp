@@ -747,6 +747,11 @@ inline void launch_iq4_nl_gemv_q8_0_f32(const LowBitMatrix &w, const int8_t *act
 inline void q38_hc_launch_exact_q8_0_gemv_f32(const uint8_t *weight, const int8_t *act, const half_bits *act_scales, float *out, int rows, int cols, Stream stream) {
     check(wd_gemv_q8_0_f32(WD_TYPE_Q8_0, weight, rows, cols, act, act_scales, out, nullptr, stream), "Q8_0 GEMV failed");
 }
+// The same for a list of projections of one row length in one launch (no counterpart in the reference, which launches
+// q38_hc_launch_exact_q8_0_gemv_f32 once per projection; the results are the same bits as those calls).
+inline void q38_hc_launch_exact_q8_0_gemv_batch_f32(const wd_gemv_item *items, int n_items, int cols, Stream stream) {
+    check(wd_gemv_q8_0_batch_f32(WD_TYPE_Q8_0, items, n_items, cols, stream), "batched Q8_0 GEMV failed");
+}
 // src/warodecode.cu:1746-1768 (raw Q4_0 blocks; no planar prepack)
 inline void launch_q4_float(const LowBitMatrix &w, const int8_t *act, const half_bits *act_scales, float *out, Stream stream) {
     if (w.type != GgmlType::Q4_0 || w.cols % 32 != 0) throw std::runtime_error("Q4_0 x Q8_0 GEMV geometry mismatch");
