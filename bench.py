@@ -689,10 +689,12 @@ def bench_q8_batch(args, torch, capi, synth):
     matrices (>= 1.5 GB of copies), the period is taken over a captured chain."""
     n_items = 10
     results = []
-    for rows, cols in [(2048, 2048), (1024, 4096), (512, 8192), (512, 2048)]:
-        nbytes = rows * synth.row_bytes(synth.Q8_0, cols)
+    for wtype, rows, cols in [(synth.Q8_0, 2048, 2048), (synth.Q8_0, 1024, 4096), (synth.Q8_0, 512, 8192), (synth.Q8_0, 512, 2048),
+                              (synth.Q4_0, 2048, 2048), (synth.Q4_0, 512, 2048)]:
+        tname = "Q8_0" if wtype == synth.Q8_0 else "Q4_0"
+        nbytes = rows * synth.row_bytes(wtype, cols)
         sets = max(2, -(-int(1.5e9) // (nbytes * n_items)))
-        one = torch.from_numpy(synth.matrix(synth.Q8_0, synth.rng_for(synth.BASE_SEED, 83, rows, cols), rows, cols)).reshape(-1).cuda()
+        one = torch.from_numpy(synth.matrix(wtype, synth.rng_for(synth.BASE_SEED, 83, rows, cols), rows, cols)).reshape(-1).cuda()
         w = one.repeat(sets * n_items).reshape(sets, n_items, nbytes)
         x = torch.from_numpy(synth.rng_for(synth.BASE_SEED, 84, cols).normal(0, 1, cols).astype(np.float32)).cuda()
         qs = torch.empty(cols, dtype=torch.int8, device="cuda")
@@ -711,11 +713,11 @@ def bench_q8_batch(args, torch, capi, synth):
             tables.append(items)
 
         def batched(j):
-            capi.call("wd_gemv_q8_0_batch_f32", synth.Q8_0, tables[j % sets], n_items, cols, stream())
+            capi.call("wd_gemv_q8_0_batch_f32", wtype, tables[j % sets], n_items, cols, stream())
 
         def single(j):
             for i in range(n_items):
-                capi.call("wd_gemv_q8_0_f32", synth.Q8_0, C.c_void_p(w[j % sets, i].data_ptr()), rows, cols, vp(qs), vp(sc), vp(y1[i]),
+                capi.call("wd_gemv_q8_0_f32", wtype, C.c_void_p(w[j % sets, i].data_ptr()), rows, cols, vp(qs), vp(sc), vp(y1[i]),
                           None, stream())
 
         batched(0)
@@ -726,13 +728,13 @@ def bench_q8_batch(args, torch, capi, synth):
         reps = max(3, int(1e11 // (nbytes * n_items * launches)))
         us_b = graph_period_us(torch, batched, launches, reps)
         us_s = graph_period_us(torch, single, launches, reps)
-        results.append(dict(rows=rows, cols=cols, items=n_items, bytes_per_item=nbytes, sets=sets, same_bits=same,
+        results.append(dict(type=tname, rows=rows, cols=cols, items=n_items, bytes_per_item=nbytes, sets=sets, same_bits=same,
                             us_per_gemv_batched=round(us_b / n_items, 3), us_per_gemv_single=round(us_s / n_items, 3),
                             gbs_batched=round(nbytes * n_items / us_b / 1e3, 1), gbs_single=round(nbytes * n_items / us_s / 1e3, 1),
                             frac_batched=round(nbytes * n_items / us_b / 1e3 / HBM_PEAK_GBS, 4),
                             frac_single=round(nbytes * n_items / us_s / 1e3 / HBM_PEAK_GBS, 4)))
-        note("Q8_0 %dx%d x %d: %.2f us per GEMV in one launch (%.0f GB/s), %.2f us one launch each (%.0f GB/s), same bits %s"
-             % (rows, cols, n_items, us_b / n_items, nbytes * n_items / us_b / 1e3, us_s / n_items, nbytes * n_items / us_s / 1e3, same))
+        note("%s %dx%d x %d: %.2f us per GEMV in one launch (%.0f GB/s), %.2f us one launch each (%.0f GB/s), same bits %s"
+             % (tname, rows, cols, n_items, us_b / n_items, nbytes * n_items / us_b / 1e3, us_s / n_items, nbytes * n_items / us_s / 1e3, same))
         del w, one
         torch.cuda.empty_cache()
     head = results[0]
@@ -740,7 +742,8 @@ def bench_q8_batch(args, torch, capi, synth):
         "metric": "ten exact-order Q8_0 GEMVs 2048x2048 in one launch, batch=1: achieved HBM GB/s", "value": head["gbs_batched"],
         "unit": "GB/s", "n_gpus": 1, "higher_is_better": True, "vs_baseline": None, "dtype": "int8 dot products, f32 accumulate",
         "data": "synthetic",
-        "config": {"workload": "the middle sizes of the exact-order Q8_0 x Q8_0 GEMV, ten projections per launch against ten launches",
+        "config": {"workload": "the middle sizes of the dense GEMVs (exact-order Q8_0, Q4_0) against Q8_0 activations, ten projections per "
+                               "launch against ten launches",
                    "shapes": results, "valid": all(r["same_bits"] for r in results)},
         "roofline": dict(bound="hbm", achieved=head["gbs_batched"], peak=HBM_PEAK_GBS, unit="GB/s", frac=head["frac_batched"],
                          traffic=None, kernel="k_gemv_q8_rows8_split_batch", us_per_launch=round(head["us_per_gemv_batched"] * n_items, 3),

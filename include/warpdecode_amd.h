@@ -126,16 +126,18 @@ int wd_gemv_q8_k_f32(int type, const uint8_t *d_w, int rows, int cols, const int
 int wd_gemv_q8_0_f32(int type, const uint8_t *d_w, int rows, int cols, const int8_t *d_act_qs,
                      const uint16_t *d_act_scales, float *d_out, int32_t *d_partials, void *stream);
 
-/* Several exact-order Q8_0 x Q8_0 GEMVs of the same row length in one launch: the projections a block applies to one or
- * a few activations are each bound by their launch, not by their bytes (a 2048 x 2048 matrix alone reaches a seventh of
- * the device's bandwidth).  Item i computes d_out[rows] = W_i (rows x cols) . activation_i exactly as wd_gemv_q8_0_f32
- * does for it alone - the same workgroups do the same arithmetic, the results are the same bits.  `items` is host memory;
- * items whose shape the shared kernel does not take (rows < 8, fewer than 64 or more than 512 blocks per row, 8192 or
- * more rows, pointers not 16-byte aligned) are launched by themselves, in order.  At most 16 items go into one launch;
- * longer lists are cut.
- * reference: the call sites of q38_hc_launch_exact_q8_0_gemv_f32, one launch per projection (src/qwen38_hc.cuh:1020-1049). */
+/* Several dense GEMVs of the same row length against Q8_0 activations in one launch - `type` WD_TYPE_Q8_0 (the exact-order
+ * kernel) or WD_TYPE_Q4_0: the projections a block applies to one or a few activations are each bound by their launch,
+ * not by their bytes (a 2048 x 2048 Q8_0 matrix alone reaches a seventh of the device's bandwidth).  Item i computes
+ * d_out[rows] = W_i (rows x cols) . activation_i exactly as wd_gemv_q8_0_f32 does for it alone - the same workgroups do
+ * the same arithmetic, the results are the same bits.  `items` is host memory; items whose shape the shared kernel does
+ * not take (Q8_0: rows < 8, fewer than 64 or more than 512 blocks per row, 8192 or more rows; Q4_0: rows that are not a
+ * power-of-two number of 8-block groups up to 64; either: pointers not 16-byte aligned) are launched by themselves, in
+ * order.  At most 16 items go into one launch; longer lists are cut.
+ * reference: the call sites of q38_hc_launch_exact_q8_0_gemv_f32, one launch per projection (src/qwen38_hc.cuh:1020-1049),
+ * and of launch_q4_float (src/warodecode.cu:1746-1768). */
 typedef struct wd_gemv_item {
-    const uint8_t *d_w;            /* Q8_0 rows, 34-byte blocks */
+    const uint8_t *d_w;            /* rows of 34-byte (Q8_0) or 18-byte (Q4_0) blocks */
     int rows;
     const int8_t *d_act_qs;        /* the activation's Q8_0 quants [cols] and scales [cols / 32] (wd_q8_0_quantize_f32) */
     const uint16_t *d_act_scales;

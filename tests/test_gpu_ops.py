@@ -261,10 +261,42 @@ def test_q8_0_gemv_batch(g, oracle, cols, rows_list, shift):
         assert g.same_bits(got, wants[i]), (i, rows)
 
 
+# the projections of a Llama-3.2-1B block (q, k, v on one activation; gate and up), a shape the streaming kernel does not
+# take (2560 columns: ten 8-block groups), a list of 17
+@pytest.mark.parametrize("cols,rows_list", [(2048, [2048, 512, 512]), (2048, [8192, 8192]), (2560, [64, 128]), (2048, [256] * 17),
+                                            (8192, [2048, 100])],
+                         ids=["qkv", "gate-up", "general-kernel", "17-items", "down-and-ragged"])
+def test_q4_0_gemv_batch(g, oracle, cols, rows_list):
+    """The same for Q4_0 matrices: the same bits as one call each (the float order of Q4_0 is this library's own, so the
+    oracle is met within 1e-5 as in the single-matrix tests; the int32 block sums are covered there)."""
+    rng = synth.rng_for(SEED, 30, cols, len(rows_list))
+    x = rng.normal(0, 1, cols).astype(np.float32)
+    qs, d = oracle.quantize_q8_0(x)
+    dq, dd = g.dev(qs), g.dev(d)
+    items = (capi.GemvItem * len(rows_list))()
+    keep, singles, wants, mats = [], [], [], []
+    for i, rows in enumerate(rows_list):
+        w = synth.matrix(synth.Q4_0, rng, rows, cols)
+        mats.append(w)
+        dw, out, single = g.dev(w), g.empty(rows, np.float32), g.empty(rows, np.float32)
+        keep.append((dw, out))
+        singles.append(single)
+        items[i].d_w, items[i].rows, items[i].d_act_qs, items[i].d_act_scales, items[i].d_out = dw.data_ptr(), rows, dq.data_ptr(), dd.data_ptr(), out.data_ptr()
+        capi.call("wd_gemv_q8_0_f32", synth.Q4_0, g.ptr(dw), rows, cols, g.ptr(dq), g.ptr(dd), g.ptr(single), None, g.stream())
+        wants.append(oracle.gemv(synth.Q4_0, w, rows, cols, qs, d))
+    capi.call("wd_gemv_q8_0_batch_f32", synth.Q4_0, items, len(rows_list), cols, g.stream())
+    g.sync()
+    for i, rows in enumerate(rows_list):
+        got = g.host(keep[i][1])
+        assert g.same_bits(got, g.host(singles[i])), (i, rows)
+        mag = np.array([np.abs(oracle.dequant_row(synth.Q4_0, mats[i][r], cols)).sum() for r in range(min(rows, 16))]).mean()
+        assert np.allclose(got, wants[i], rtol=1e-5, atol=1e-5 * mag), (i, rows)
+
+
 def test_q8_0_gemv_batch_refuses_what_it_cannot_take(g):
     items = (capi.GemvItem * 1)()
     lib = capi.load()
-    assert lib.wd_gemv_q8_0_batch_f32(synth.Q4_0, items, 1, 2048, g.stream()) != 0      # exact-order Q8_0 only
+    assert lib.wd_gemv_q8_0_batch_f32(synth.IQ4_NL, items, 1, 2048, g.stream()) != 0    # Q8_0 and Q4_0 matrices only
     assert lib.wd_gemv_q8_0_batch_f32(synth.Q8_0, items, 0, 2048, g.stream()) != 0      # no items
     assert lib.wd_gemv_q8_0_batch_f32(synth.Q8_0, items, 1, 2040, g.stream()) != 0      # not whole blocks
     assert lib.wd_gemv_q8_0_batch_f32(synth.Q8_0, items, 1, 2048, g.stream()) != 0      # null pointers in the item

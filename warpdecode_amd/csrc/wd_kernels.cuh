@@ -320,11 +320,11 @@ __global__ __launch_bounds__(256) void k_gemv_q8(MatSrc src, int rows, int cols,
 // A wave takes NP consecutive passes and requests all of them before it touches the first.
 // grid.x * WPB waves * NP passes cover ceil(rows / (64 / lpr)) passes.
 // dynamic LDS: lpr * 272 bytes of quants, then nb floats, then nb ints.
+// (the body: `block` is the workgroup's number among those of its matrix)
 template <bool PART, int NP, int WPB>
-__global__ __launch_bounds__(WPB * 64) void k_gemv_q4_stream(const uint8_t *__restrict__ w, int rows, int nb,
-                                                         const int8_t *__restrict__ act_qs,
-                                                         const uint16_t *__restrict__ act_d, float *__restrict__ out,
-                                                         int32_t *__restrict__ partials) {
+WD_DEV void gemv_q4_stream_body(const uint8_t *__restrict__ w, int rows, int nb, const int8_t *__restrict__ act_qs,
+                                const uint16_t *__restrict__ act_d, float *__restrict__ out, int32_t *__restrict__ partials,
+                                int block) {
     __shared__ uint4 stage[WPB][9 * 64];
     extern __shared__ __align__(16) uint8_t q4_act[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -333,7 +333,7 @@ __global__ __launch_bounds__(WPB * 64) void k_gemv_q4_stream(const uint8_t *__re
     float *ad = reinterpret_cast<float *>(q4_act + lpr * 272);
     int *corr = reinterpret_cast<int *>(ad + nb);
     const size_t rb = static_cast<size_t>(nb) * 18;
-    const long long pass0 = (static_cast<long long>(blockIdx.x) * WPB + wave) * NP;
+    const long long pass0 = (static_cast<long long>(block) * WPB + wave) * NP;
     uint4 v[NP][9];
     auto fetch = [&](long long pass, int slot) {
         const long long row0 = pass * rpp;
@@ -416,6 +416,37 @@ __global__ __launch_bounds__(WPB * 64) void k_gemv_q4_stream(const uint8_t *__re
         for (int mask = lpr >> 1; mask >= 1; mask >>= 1) sumf += lane_xor(sumf, mask);
         if (col == 0 && row < rows) out[row] = sumf;
     }
+}
+template <bool PART, int NP, int WPB>
+__global__ __launch_bounds__(WPB * 64) void k_gemv_q4_stream(const uint8_t *__restrict__ w, int rows, int nb,
+                                                         const int8_t *__restrict__ act_qs,
+                                                         const uint16_t *__restrict__ act_d, float *__restrict__ out,
+                                                         int32_t *__restrict__ partials) {
+    gemv_q4_stream_body<PART, NP, WPB>(w, rows, nb, act_qs, act_d, out, partials, static_cast<int>(blockIdx.x));
+}
+// Several matrices of one row length in one launch (see k_gemv_q8_rows8_split_batch): workgroup b belongs to the item
+// whose range of workgroups holds b and does there what k_gemv_q4_stream does for that item alone.
+constexpr int kGemvBatchMax = 16;
+struct GemvBatch {
+    const uint8_t *w[kGemvBatchMax];
+    const int8_t *act_qs[kGemvBatchMax];
+    const uint16_t *act_d[kGemvBatchMax];
+    float *out[kGemvBatchMax];
+    int rows[kGemvBatchMax];
+    int first_group[kGemvBatchMax + 1];  // the item's first workgroup; first_group[n]: all workgroups
+    int n;
+};
+WD_DEV int gemv_batch_item(const GemvBatch &b) {
+    int item = 0;
+    for (int i = 1; i < b.n; ++i)
+        if (static_cast<int>(blockIdx.x) >= b.first_group[i]) item = i;
+    return __builtin_amdgcn_readfirstlane(item);
+}
+template <int WPB>
+__global__ __launch_bounds__(WPB * 64) void k_gemv_q4_stream_batch(GemvBatch b, int nb) {
+    const int item = gemv_batch_item(b);
+    gemv_q4_stream_body<false, 1, WPB>(b.w[item], b.rows[item], nb, b.act_qs[item], b.act_d[item], b.out[item], nullptr,
+                                       static_cast<int>(blockIdx.x) - b.first_group[item]);
 }
 
 // ---- dense Q8_0 x Q8_0 GEMV, streaming: one lane per (row, chain) ----------------------------------------------
@@ -680,22 +711,9 @@ __global__ __launch_bounds__(64 * WAVES) void k_gemv_q8_rows8_split(const uint8_
 // Several matrices of the same row length in ONE launch (the projections a block applies to one or a few activations:
 // each of them alone is bound by its launch, not by its bytes).  Workgroup b belongs to the item whose range of row
 // groups holds b; what it computes is what k_gemv_q8_rows8_split computes for that item alone.
-constexpr int kGemvBatchMax = 16;
-struct GemvBatch {
-    const uint8_t *w[kGemvBatchMax];
-    const int8_t *act_qs[kGemvBatchMax];
-    const uint16_t *act_d[kGemvBatchMax];
-    float *out[kGemvBatchMax];
-    int rows[kGemvBatchMax];
-    int first_group[kGemvBatchMax + 1];  // first_group[n]: all groups
-    int n;
-};
 template <int KB, int NCH, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void k_gemv_q8_rows8_split_batch(GemvBatch b, int nb) {
-    int item = 0;
-    for (int i = 1; i < b.n; ++i)
-        if (static_cast<int>(blockIdx.x) >= b.first_group[i]) item = i;
-    item = __builtin_amdgcn_readfirstlane(item);
+    const int item = gemv_batch_item(b);
     gemv_q8_rows8_split_body<KB, NCH, WAVES, false>(b.w[item], b.rows[item], nb, b.act_qs[item], b.act_d[item], b.out[item], nullptr,
                                                    static_cast<int>(blockIdx.x) - b.first_group[item]);
 }

@@ -382,13 +382,63 @@ int wd_gemv_q8_0_f32(int type, const uint8_t *d_w, int rows, int cols, const int
     return launch_gemv_q8_0(type, src, 1, rows, cols, d_act_qs, d_act_scales, 0, d_out, d_partials, as_stream(stream));
 }
 
+// Q4_0 matrices: the workgroups per item of the streaming kernel (waves per workgroup in *wpb), 0 when the item takes
+// another kernel alone.
+static int q4_stream_wgs(const wd_gemv_item &it, int nb, int *wpb) {
+    if (!(nb % 8 == 0 && nb / 8 <= 64 && 64 % (nb / 8) == 0 && reinterpret_cast<uintptr_t>(it.d_w) % 16 == 0 &&
+          reinterpret_cast<uintptr_t>(it.d_act_qs) % 16 == 0))
+        return 0;
+    const int rpp = 64 / (nb / 8);
+    const long long passes = (static_cast<long long>(it.rows) + rpp - 1) / rpp;
+    *wpb = passes <= 256 ? 2 : 4;
+    const long long wgs = (passes + *wpb - 1) / *wpb;
+    return wgs <= 4096 ? static_cast<int>(wgs) : 0;  // (large matrices are not bound by their launch)
+}
+static int gemv_q4_0_batch(const wd_gemv_item *items, int n_items, int cols, void *stream) {
+    const int nb = cols / 32;
+    int i = 0;
+    while (i < n_items) {
+        int wpb = 0, other = 0;
+        const int wgs0 = q4_stream_wgs(items[i], nb, &wpb);
+        int j = i + 1;
+        if (wgs0)
+            while (j < n_items && j - i < kGemvBatchMax && q4_stream_wgs(items[j], nb, &other) && other == wpb) ++j;
+        if (!wgs0 || j - i == 1) {
+            if (const int rc = wd_gemv_q8_0_f32(WD_TYPE_Q4_0, items[i].d_w, items[i].rows, cols, items[i].d_act_qs, items[i].d_act_scales,
+                                                items[i].d_out, nullptr, stream))
+                return rc;
+            ++i;
+            continue;
+        }
+        GemvBatch b{};
+        b.n = j - i;
+        int wgs = 0;
+        for (int q = 0; q < b.n; ++q) {
+            const wd_gemv_item &it = items[i + q];
+            b.w[q] = it.d_w, b.act_qs[q] = it.d_act_qs, b.act_d[q] = it.d_act_scales, b.out[q] = it.d_out, b.rows[q] = it.rows;
+            b.first_group[q] = wgs;
+            wgs += q4_stream_wgs(it, nb, &other);
+        }
+        for (int q = b.n; q <= kGemvBatchMax; ++q) b.first_group[q] = wgs;
+        const size_t lds = static_cast<size_t>(nb / 8) * 272 + static_cast<size_t>(nb) * 8;
+        if (wpb == 2)
+            k_gemv_q4_stream_batch<2><<<wgs, 128, lds, as_stream(stream)>>>(b, nb);
+        else
+            k_gemv_q4_stream_batch<4><<<wgs, 256, lds, as_stream(stream)>>>(b, nb);
+        WD_LAUNCH_CHECK();
+        i = j;
+    }
+    return WD_OK;
+}
+
 int wd_gemv_q8_0_batch_f32(int type, const wd_gemv_item *items, int n_items, int cols, void *stream) {
-    WD_REQUIRE(type == WD_TYPE_Q8_0, "batched GEMV: exact-order Q8_0 matrices only (type %d)", type);
+    WD_REQUIRE(type == WD_TYPE_Q8_0 || type == WD_TYPE_Q4_0, "batched GEMV: Q8_0 (exact order) or Q4_0 matrices (type %d)", type);
     WD_REQUIRE(items != nullptr && n_items > 0, "batched GEMV: no items");
     WD_REQUIRE(cols > 0 && cols % 32 == 0, "batched GEMV: invalid row length %d", cols);
     for (int i = 0; i < n_items; ++i)
         WD_REQUIRE(items[i].d_w && items[i].d_act_qs && items[i].d_act_scales && items[i].d_out && items[i].rows > 0,
                    "batched GEMV: item %d has a null pointer or no rows", i);
+    if (type == WD_TYPE_Q4_0) return gemv_q4_0_batch(items, n_items, cols, stream);
     const int nb = cols / 32;
     // One launch for as many items in a row as take the same kernel: every item must be a shape the split kernel takes
     // alone (then its workgroups do here exactly what they do there); anything else is launched by itself.
