@@ -131,10 +131,9 @@ __global__ __launch_bounds__(WD_FILL_THREADS) void k_fill_slots(FillSegments f, 
 // three words in named registers, every store unconditional: no private array).  Beside the stack's six waves a SIMD has
 // 32 vector registers left, and of the scalar registers what the stack kernel's own cap leaves (see k_stack_resident):
 // a kernel that needs more of either is not started before the stack has ended, which the stack, waiting for it, never does.
-#ifndef WD_FILL_BESIDE_WGS
-#define WD_FILL_BESIDE_WGS 54   // as many bytes in flight as WD_FILL_WGS workgroups of the other form have
-#endif
-constexpr int kFillBesideUnroll = 3;
+// 54 workgroups: as many bytes in flight as the 20 of the other form have.  Mode B, tokens per second: 32 workgroups 706,
+// 54 743, 96 656, 160 561 (the more waves sit beside the stack's, the later its slowest workgroup).
+constexpr int kFillBesideWgs = 54, kFillBesideUnroll = 3;
 __global__ __launch_bounds__(WD_FILL_THREADS) void k_fill_slots_beside(FillSegments f, int n_seg, FillMarks m) {
     const uint32_t stride = gridDim.x * WD_FILL_THREADS;
     for (int seg = 0; seg < n_seg; ++seg) {
@@ -1077,7 +1076,7 @@ int launch_fill_segments(wd_expert_cache *c, FillSegments &fills, int &n_fill, u
         // enough workgroups per segment to keep the host link busy, few enough to leave the decode its compute units
         timing_dma_begin(c);
         const bool beside = c->mark_seq != 0u;  // the token goes through a one-launch stack: every fill has to find room beside it
-        const uint32_t round_words = WD_FILL_THREADS * (beside ? kFillBesideUnroll : WD_FILL_UNROLL), most = beside ? WD_FILL_BESIDE_WGS : WD_FILL_WGS;
+        const uint32_t round_words = WD_FILL_THREADS * (beside ? kFillBesideUnroll : WD_FILL_UNROLL), most = beside ? kFillBesideWgs : WD_FILL_WGS;
         const uint32_t per_seg = (max_words + round_words - 1) / round_words;
         const dim3 grid(per_seg < most ? (per_seg ? per_seg : 1) : most);
         if (beside) {

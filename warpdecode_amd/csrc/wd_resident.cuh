@@ -59,18 +59,9 @@ constexpr int kResXtRow = 68;      // floats per row of the transposed input in 
 constexpr int kResGateSlot = 15;   // word of the weights record that holds the shared expert's sigmoid gate
 constexpr int kResSleepPoll = 2;   // s_sleep between two polls of a wait (flat from 1 to 8 in measurements)
 constexpr int kResSleepFold = 24;  // waves that reach a layer while rung 0 still folds the one before wait this long first
-#ifndef WD_RES_SGPRS
-#define WD_RES_SGPRS 96
-#endif
-#ifndef WD_RES_FILL_SLEEPS
-#define WD_RES_FILL_SLEEPS 2
-#endif
-constexpr int kResFillSleeps = WD_RES_FILL_SLEEPS;  // s_sleep 127 (about 4 us each) between two polls of a layer's fills
-#ifndef WD_RES_PRIO_ROUTER
-#define WD_RES_PRIO_ROUTER 3
-#define WD_RES_PRIO_WG0 2
-#endif
-constexpr int kResPrioRouter = WD_RES_PRIO_ROUTER, kResPrioWg0 = WD_RES_PRIO_WG0;  // s_setprio of the router waves / of workgroup 0's other waves (measured: 2-4 % each)
+constexpr int kResSgprs = 96;       // scalar registers per wave (see k_stack_resident)
+constexpr int kResFillSleeps = 2;  // s_sleep 127 (about 4 us each) between two polls of a layer's fills
+constexpr int kResPrioRouter = 3, kResPrioWg0 = 2;  // s_setprio of the router waves / of workgroup 0's other waves (measured: 2-4 % each)
 
 // The bits a value is handed on with: kResEmpty means "not yet written", so that one NaN travels as the default quiet NaN
 // (wd_handword.hpp, checked on the host).
@@ -927,7 +918,7 @@ template <int TYPE, bool STAMPS>
 // The scalar registers are capped below what six waves could share out (102 each): at 96 a SIMD keeps scalar registers
 // free for the waves of another stream's small kernel - the copy kernel that fills expert slots while the stack runs
 // found no room beside waves of 106.  (The cap is only honoured when the upper bound of waves_per_eu is above six.)
-__global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 7), amdgpu_num_sgpr(WD_RES_SGPRS))) void k_stack_resident(ResidentArgs a) {
+__global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 7), amdgpu_num_sgpr(kResSgprs))) void k_stack_resident(ResidentArgs a) {
     extern __shared__ __align__(16) uint8_t lds_res[];
     // (the wave's number as a scalar, the lane's counted where it is needed: no vector register is held for the whole launch)
     const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
