@@ -643,15 +643,22 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         if (rung == 0) {
             res_mark<STAMPS>(a, c, l, 8);
             const float *ybuf = c.ybuf();
+            // (all eleven results requested from LDS at once, then the chain: a loop that reads each term when it needs it
+            // pays the LDS latency eleven times, about half a microsecond between the barrier and the next input's store)
+            float yv[kResMaxK];
+#pragma unroll
+            for (int m = 0; m < kResMaxK; ++m) yv[m] = ybuf[m * 4 + (lane & 3)];
+            float ysh = ybuf[kResSharedSlot * 4 + (lane & 3)];
             float acc = 0.0f;
-            for (int m = 0; m < a.k; ++m) {
-                const float wm = readlane_f(wreg, m);
-                const float prod = ybuf[m * 4 + (lane & 3)] * wm;
-                acc = acc + prod;
+#pragma unroll
+            for (int m = 0; m < kResMaxK; ++m) {
+                const float prod = yv[m] * readlane_f(wreg, m);
+                const float next = acc + prod;
+                acc = m < a.k ? next : acc;
             }
-            float o = acc, ysh = 0.0f;
+            float o = acc;
+            if (!shared) ysh = 0.0f;
             if (shared) {
-                ysh = ybuf[kResSharedSlot * 4 + (lane & 3)];
                 const float prod = ysh * readlane_f(wreg, 16);
                 o = acc + prod;
             }
