@@ -77,7 +77,11 @@ def parse():
     ap.add_argument("--cache-timing", action="store_true",
                     help="lru mode: switch on the cache's device-side timings (the copy stream's waits and fills, in the monitor "
                          "object); the events they need cost about 4 % of the rate")
-    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a captured HIP graph")
+    ap.add_argument("--graph", choices=["auto", "on", "off"], default="auto",
+                    help="replay the step from a captured HIP graph or launch it eagerly; auto: eagerly when the step is one "
+                         "launch (the resident stack: a graph of one kernel costs more than the launch it saves), a graph for "
+                         "the dispatches per layer")
+    ap.add_argument("--no-graph", action="store_true", help="the same as --graph off")
     ap.add_argument("--path", choices=["resident", "per-layer"], default="resident",
                     help="resident mode: the stack as ONE launch of resident workgroups (default), or two dispatches per layer")
     ap.add_argument("--repeats", type=int, default=5, help="further repeats of the timed region, for the spread in the JSON line")
@@ -1038,15 +1042,15 @@ def main():
                   trace_ptr, RESIDUAL_SCALE, stack_flags if flags is None else flags,
                   C.c_void_p(torch.cuda.current_stream().cuda_stream))
 
-    def captured(fn):
-        """fn() warmed on a side stream, then captured into a HIP graph (None with --no-graph)."""
+    def captured(fn, one_launch=False):
+        """fn() warmed on a side stream, then captured into a HIP graph (None when it is to be launched eagerly)."""
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             fn()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
-        if args.no_graph:
+        if args.no_graph or args.graph == "off" or (args.graph == "auto" and one_launch):
             return None
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
@@ -1088,7 +1092,7 @@ def main():
             sys.exit(1)
 
     note("inputs and routing trace ready")
-    graph = captured(launch_stack)
+    graph = captured(launch_stack, one_launch=args.path == "resident")
 
     note("launch mode: %s" % ("eager" if graph is None else "hip-graph replay"))
 
@@ -1188,7 +1192,7 @@ def main():
             def router_stack():
                 capi.call("wd_moe_stack_f32", layers, NL, C.c_void_p(d_x.data_ptr()), C.c_void_p(d_out.data_ptr()), scratch,
                           None, RESIDUAL_SCALE, STACK_FLAGS, C.c_void_p(torch.cuda.current_stream().cuda_stream))
-            g3 = captured(router_stack)
+            g3 = captured(router_stack, one_launch=True)
             run_router = g3.replay if g3 is not None else router_stack
             for j in range(4):
                 bring_in(j)
