@@ -10,7 +10,8 @@ the prescribed scale distributions) and are generated on the device before the t
 
 Prints ONE JSON line (see the keys at the bottom).  `value` is tokens/s with everything resident
 in HBM; `roofline` prices the dominant kernel against the 8 TB/s HBM peak; `cpu_baseline` times the
-reference's CPU MoE path (oracle/_ref when built, else the C port) on a bounded sample.
+reference's CPU MoE path (oracle/_ref when built, else the C port) on a bounded sample; `mode_b` is a
+bounded run of the same stack with its routed experts in pinned host memory behind the slot pool.
 """
 import argparse
 import ctypes as C
