@@ -61,6 +61,7 @@ constexpr int kResSleepPoll = 2;   // s_sleep between two polls of a wait (flat 
 constexpr int kResSleepFold = 24;  // waves that reach a layer while rung 0 still folds the one before wait this long first
 constexpr int kResSgprs = 96;       // scalar registers per wave (see k_stack_resident)
 constexpr int kResFillSleeps = 2;  // s_sleep 127 (about 4 us each) between two polls of a layer's fills
+constexpr int kResPrioFold = 1;     // s_setprio of rung 0 while it folds (the other rungs decode the next layer's rows meanwhile)
 constexpr int kResPrioRouter = 3, kResPrioWg0 = 2;  // s_setprio of the router waves / of workgroup 0's other waves (measured: 2-4 % each)
 
 // The bits a value is handed on with: kResEmpty means "not yet written", so that one NaN travels as the default quiet NaN
@@ -529,6 +530,17 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         gate_up_rows(res_field_s(&a.layers->gate), res_field_s(&a.layers->up), traced_expert(0, slot0), r0, lane0);
     }
     bool rows_asked = true;  // with a routing trace: this layer's gate/up rows were requested during the layer before
+    // With a routing trace the rows of a layer are also DECODED before the layer begins - between the end of the layer
+    // before and the arrival of its output, when the vector units have nothing to do: codebook and sign lookups need no
+    // activation.  What is left for the time after the input has arrived are the dot products, the fold and the chains.
+    IqRows8Decoded<1> dec;
+#pragma unroll
+    for (int i = 0; i < 1; ++i) {
+        dec.d[i] = 0u, dec.ls[i][0] = dec.ls[i][1] = 0;
+#pragma unroll
+        for (int c0 = 0; c0 < 8; ++c0) dec.w[i][c0] = 0u;
+    }
+    bool decoded = false;  // dec holds this layer's rows
     for (int l = 0; l < a.n_layers; ++l) {
         const ResCtx c = res_ctx(lds_base, r0, lane0, wave0, slot0, hb);
         const int r = c.r, lane = c.lane, wave = c.wave, rung = c.slot;
@@ -558,7 +570,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             } else {
                 // (the other waves of the workgroup come here while rung 0 still folds the previous layer: nothing
                 // can have arrived yet)
-                if (rung != 0) __builtin_amdgcn_s_sleep(kResSleepFold);
+                if (rung != 0 && !decoded) __builtin_amdgcn_s_sleep(kResSleepFold);
                 const unsigned off[1] = {xc_off(l, r & (kResCopies - 1)) + kXcStride * i};
                 uint4 v[1];
                 hand_wait16<1>(a, c.hb, off, true, v, dead);
@@ -597,7 +609,12 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         float act = 0.0f;
         if (on) {
             float gu[2] = {1.0f, 1.0f};
-            if constexpr (!kQ8) iq_rows8_coal_park<kIq, 2>(raw, lane, c.area());
+            if constexpr (!kQ8) {
+                if (!decoded) {
+                    iq_rows8_coal_park<kIq, 2>(raw, lane, c.area());
+                    iq_rows8_coal_decode<kIq, 1>(tables, lane, c.area(), dec);
+                }
+            }
             // Nothing below may be requested before the gate/up rows are here (the wave's loads return in order, and
             // requested together, the down rows of the waves served first would delay the gate/up rows of the others,
             // which the whole grid waits for): the expert's number passes through a statement the compiler cannot
@@ -611,7 +628,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                 q8_row_wave_pass<2>(gb, true, lane, c.x0q(), c.x0d(), tile, lane, acc);
                 gu[0] = close_lanes8(acc[0]), gu[1] = close_lanes8(acc[1]);
             } else {
-                iq_rows8_coal_dots<kIq, 2, false>(tables, c.xq(), c.xd(), lane, gu, c.area());
+                iq_rows8_half_decoded_dots<kIq>(dec, tables, c.xq(), c.xd(), lane, gu, c.area());
             }
             act = silu_ggml(gu[0]) * gu[1];
             // the next layer's gate/up rows (their registers are free since the rows of this layer lie in LDS; requested
@@ -641,6 +658,8 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
 
         // ---- ordered weighted sum, shared branch, next input
         if (rung == 0) {
+            // (the other rungs start decoding the next layer's rows now: the fold, which the whole grid waits for, goes first)
+            if (r != 0) __builtin_amdgcn_s_setprio(kResPrioFold);
             res_mark<STAMPS>(a, c, l, 8);
             const float *ybuf = c.ybuf();
             // (all eleven results requested from LDS at once, then the chain: a loop that reads each term when it needs it
@@ -680,6 +699,17 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                 if (lane < kResCopies) hand_store16(c.hb, xc_off(l + 1, lane) + kXcStride * r, piece);
             }
             res_mark<STAMPS>(a, c, l, 9);
+            if (r != 0) __builtin_amdgcn_s_setprio(0);
+        }
+        // The next layer's gate/up rows, requested behind this layer's dot products, have long arrived: they are decoded
+        // now, while the next input is on its way.
+        decoded = false;
+        if constexpr (!kQ8) {
+            if (traced && on && !last && rows_asked) {
+                iq_rows8_coal_park<kIq, 2>(raw, lane, c.area());
+                iq_rows8_coal_decode<kIq, 1>(tables, lane, c.area(), dec);
+                decoded = true;
+            }
         }
     }
 }

@@ -195,27 +195,32 @@ WD_DEV void iq_chunks(const IqFields &f, int ib, const Tables &t, const uint32_t
 
 // The same in two steps, for callers that apply one decoded sub-block to several activations: the 32 signed
 // weights (eight packed dwords) and the odd sub-scale of every chunk first, the chunk sums per activation after.
-template <int TYPE>
-WD_DEV void iq_decode(const IqFields &f, int ib, const IqTables &t, uint32_t (&w)[8], int (&ls)[2]) {
+template <int TYPE, typename Tables>
+WD_DEV void iq_decode(const IqFields &f, int ib, const Tables &t, uint32_t (&w)[8], int (&ls)[2]) {
     if (TYPE == 21) {
         ls[0] = ls[1] = 1 + 2 * static_cast<int>((f.sc >> (4 * (ib & 1))) & 15u);
+        uint32_t g[8];
+        uint2 sm[8];
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
-            const uint32_t q = ((c < 4 ? f.qs.x : f.qs.y) >> (8 * (c & 3))) & 0xffu;
-            const uint32_t idx = q | ((f.qh << (8 - c)) & 0x100u);
+            const uint32_t q4 = (((c < 4 ? f.qs.x : f.qs.y) >> (8 * (c & 3))) & 0xffu) << 2;
+            const uint32_t off = q4 | ((f.qh << (10 - c)) & 0x400u);
             const uint32_t sbits = (f.sg >> (4 * c)) & 15u;
-            w[c] = apply_signs(t.grid3[idx], t.sign[sbits]);
+            g[c] = t.grid3_bytes(off);
+            sm[c] = t.sign_at(sbits);
         }
+#pragma unroll
+        for (int c = 0; c < 8; ++c) w[c] = apply_signs(g[c], sm[c]);
     } else {
         ls[0] = 1 + 2 * static_cast<int>(f.sc & 15u);  // chunks 0..3
         ls[1] = 1 + 2 * static_cast<int>(f.sc >> 4);   // chunks 4..7
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const uint32_t idx = ((f.qs.x >> (8 * g)) & 0xffu) | ((f.qh << (8 - 2 * g)) & 0x300u);
-            const uint64_t mags = t.grid2[idx];
+            const uint64_t mags = t.grid2_at(idx);
             const uint32_t s8 = (f.qs.y >> (8 * g)) & 0xffu;
-            w[2 * g] = apply_signs(static_cast<uint32_t>(mags), t.sign[s8 & 15u]);
-            w[2 * g + 1] = apply_signs(static_cast<uint32_t>(mags >> 32), t.sign[s8 >> 4]);
+            w[2 * g] = apply_signs(static_cast<uint32_t>(mags), t.sign_at(s8 & 15u));
+            w[2 * g + 1] = apply_signs(static_cast<uint32_t>(mags >> 32), t.sign_at(s8 >> 4));
         }
     }
 }
@@ -411,6 +416,80 @@ WD_DEV void iq_rows8_coal_dots(const Tables &t, const int8_t *act_qs, const floa
         const float ds = h2f(f.d) * dx;
         const int P = reduce_scatter_ib_pairs(p, lane);  // lane (c = ib, sb): chunk c of super-block sb
         if (PART) partials[i * pstride + sb * 8 + ib] = P;
+        const float pf = static_cast<float>(P);
+        float v = __builtin_fmaf(ds, pf, 0.0f);
+#pragma unroll
+        for (int s = 1; s < 8; ++s) v = __builtin_fmaf(ds, pf, dpp_f<kDppShr2, 0xf, 0xf, true>(0.0f, v));
+        const float r = close_chains_pairs(v);
+        y[i] = (TYPE == 22) ? 0.125f * r : r;
+    }
+}
+// iq_rows8_coal_dots in two steps, for a caller that has the rows long before it has the activation: the decode (fields
+// from the stage, codebook and sign lookups, signs applied: no activation needed) leaves each lane's 32 signed weights,
+// its sub-scales and the super-block's scale in registers; the dots, the integer fold and the float chains follow when
+// the activation is there.  The same arithmetic in the same order: the same bits.
+template <int NR>
+struct IqRows8Decoded {
+    uint32_t w[NR][8];
+    int ls[NR][2];
+    uint32_t d[NR];  // f16 bits
+};
+template <int TYPE, int NR, typename Tables>
+WD_DEV void iq_rows8_coal_decode(const Tables &t, int lane, const uint8_t *stage, IqRows8Decoded<NR> &dec) {
+    constexpr int kBlk = IqRows8Raw<TYPE, NR>::kBlk;
+    const int ib = ((lane >> 4) << 1) | (lane & 1), sb = (lane >> 1) & 7;
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+        const IqFields f = iq_fields_lds<TYPE>(stage + i * kIqStageBytes + sb * kBlk, ib, sb);
+        iq_decode<TYPE>(f, ib, t, dec.w[i], dec.ls[i]);
+        dec.d[i] = f.d;
+    }
+}
+template <int TYPE, int NR>
+WD_DEV void iq_rows8_decoded_dots(const IqRows8Decoded<NR> &dec, const int8_t *act_qs, const float *act_d, int lane, float (&y)[NR]) {
+    const int ib = ((lane >> 4) << 1) | (lane & 1), sb = (lane >> 1) & 7;
+    const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32);
+    const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32 + 16);
+    const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+    const float dx = act_d[sb];
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+        int p[8];
+        iq_dot_decoded(dec.w[i], dec.ls[i], a, p);
+        const float ds = h2f(static_cast<uint16_t>(dec.d[i])) * dx;
+        const int P = reduce_scatter_ib_pairs(p, lane);
+        const float pf = static_cast<float>(P);
+        float v = __builtin_fmaf(ds, pf, 0.0f);
+#pragma unroll
+        for (int s = 1; s < 8; ++s) v = __builtin_fmaf(ds, pf, dpp_f<kDppShr2, 0xf, 0xf, true>(0.0f, v));
+        const float r = close_chains_pairs(v);
+        y[i] = (TYPE == 22) ? 0.125f * r : r;
+    }
+}
+// Two parked rows of which the first has been decoded ahead (iq_rows8_coal_decode with NR = 1) and the second is decoded
+// here: what a caller does whose idle time before the activation arrives is worth one row's decode, not two.
+template <int TYPE, typename Tables>
+WD_DEV void iq_rows8_half_decoded_dots(const IqRows8Decoded<1> &dec, const Tables &t, const int8_t *act_qs, const float *act_d, int lane,
+                                       float (&y)[2], const uint8_t *stage) {
+    constexpr int kBlk = IqRows8Raw<TYPE, 2>::kBlk;
+    const int ib = ((lane >> 4) << 1) | (lane & 1), sb = (lane >> 1) & 7;
+    const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32);
+    const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32 + 16);
+    const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+    const float dx = act_d[sb];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        int p[8];
+        float ds;
+        if (i == 0) {
+            iq_dot_decoded(dec.w[0], dec.ls[0], a, p);
+            ds = h2f(static_cast<uint16_t>(dec.d[0])) * dx;
+        } else {
+            const IqFields f = iq_fields_lds<TYPE>(stage + kIqStageBytes + sb * kBlk, ib, sb);
+            iq_chunks<TYPE>(f, ib, t, a, p);
+            ds = h2f(f.d) * dx;
+        }
+        const int P = reduce_scatter_ib_pairs(p, lane);
         const float pf = static_cast<float>(P);
         float v = __builtin_fmaf(ds, pf, 0.0f);
 #pragma unroll
