@@ -800,9 +800,12 @@ template <int TYPE>
 int resident_launch(const ResidentArgs &a, wd_moe_scratch *s, hipStream_t st) {
     if (s->res_fits < 0) {  // both variants of the kernel (with and without the time stamps) must fit
         int plain = 0, stamped = 0;
+        // (more dynamic LDS than a kernel may have without asking)
+        const hipError_t a0 = hipFuncSetAttribute(reinterpret_cast<const void *>(k_stack_resident<TYPE, false>), hipFuncAttributeMaxDynamicSharedMemorySize, kResLdsBytes);
+        const hipError_t a1 = hipFuncSetAttribute(reinterpret_cast<const void *>(k_stack_resident<TYPE, true>), hipFuncAttributeMaxDynamicSharedMemorySize, kResLdsBytes);
         const hipError_t e0 = hipOccupancyMaxActiveBlocksPerMultiprocessor(&plain, k_stack_resident<TYPE, false>, kResThreads, kResLdsBytes);
         const hipError_t e1 = hipOccupancyMaxActiveBlocksPerMultiprocessor(&stamped, k_stack_resident<TYPE, true>, kResThreads, kResLdsBytes);
-        s->res_fits = (e0 == hipSuccess && e1 == hipSuccess && std::min(plain, stamped) * s->compute_units >= kResWgs) ? 1 : 0;
+        s->res_fits = (a0 == hipSuccess && a1 == hipSuccess && e0 == hipSuccess && e1 == hipSuccess && std::min(plain, stamped) * s->compute_units >= kResWgs) ? 1 : 0;
     }
     if (!s->res_fits) return kTakePerLayer;  // the workgroups would wait for each other without all being on the device
     SiteScope site(WD_SITE_STACK_RESIDENT, st);

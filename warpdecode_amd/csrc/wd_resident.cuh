@@ -62,6 +62,7 @@ constexpr int kResSleepFold = 24;  // waves that reach a layer while rung 0 stil
 constexpr int kResSgprs = 96;       // scalar registers per wave (see k_stack_resident)
 constexpr int kResFillSleeps = 2;  // s_sleep 127 (about 4 us each) between two polls of a layer's fills
 constexpr int kResPrioFold = 1;     // s_setprio of rung 0 while it folds (the other rungs decode the next layer's rows meanwhile)
+constexpr int kResPrioDots = 1;     // s_setprio of a rung from the input's arrival to its activation, with a routing trace (-1.5 %)
 constexpr int kResPrioRouter = 3, kResPrioWg0 = 2;  // s_setprio of the router waves / of workgroup 0's other waves (measured: 2-4 % each)
 
 // The bits a value is handed on with: kResEmpty means "not yet written", so that one NaN travels as the default quiet NaN
@@ -331,11 +332,12 @@ constexpr int kResLdsY = kResLdsWave + kResActSlots * kResWaveBytes;  // f32 [11
 constexpr int kResLdsSel = kResLdsY + 4 * 4 * kResActSlots;           // selection scratch, then ids [16], weights [16]
 constexpr int kResLdsRoles = kResLdsSel + kTopkLdsBytes1 + 128;       // int [12] SIMD of every wave
 constexpr int kResLdsActv = kResLdsRoles + 64;                        // f32 [12] this workgroup's activations (word 11 zero), u32 [1] arrivals
-constexpr int kResLdsBytes = kResLdsActv + 64;
+constexpr int kResLdsKept = kResLdsActv + 64;                         // per routed rung: 2048 bytes, the next layer's up row decoded ahead
+constexpr int kResLdsBytes = kResLdsKept + kResMaxK * 2048;
 constexpr int kResLdsLand = kResLdsWave;  // f32 [11][512] all activations of the layer, while no slot area is in use
 static_assert(kResLdsXq % 16 == 0 && kResLdsTables % 16 == 0 && kResLdsWave % 16 == 0 && kResWaveBytes % 16 == 0 && kResLdsSel % 16 == 0, "LDS alignment");
 static_assert(sizeof(Q8RowTile) <= sizeof(Q8TileNB<16>) && 2 * kIqStageBytes <= kResTileBytes, "a slot's area serves every stage");
-static_assert(kResLdsBytes <= 65536, "LDS of the resident stack kernel");
+static_assert(kResLdsBytes <= 81920, "LDS of the resident stack kernel: two workgroups per compute unit");
 static_assert(4 * kResActSlots * 512 <= kResActSlots * kResWaveBytes, "the activations land in the slot areas");
 
 // Values the optimiser must take as new in every layer: without them it computes hundreds of per-lane addresses once,
@@ -367,6 +369,7 @@ struct ResCtx {
     // how many waves have handed in their activation of a layer, summed over the layers so far (every wave but the router's: 11 per layer)
     WD_DEV unsigned *arrived() const { return reinterpret_cast<unsigned *>(lds + kResLdsActv + 48); }
     WD_DEV float *land() const { return reinterpret_cast<float *>(lds + kResLdsLand); }
+    WD_DEV uint8_t *kept() const { return lds + kResLdsKept + slot * 2048; }  // (routed rungs only)
 };
 // The context of one layer: the indices made opaque (see fresh_v); `base` is the workgroup's dynamic LDS.
 // The lane number, counted anew from a mask the compiler cannot see through: one number kept from the start of the kernel
@@ -419,10 +422,12 @@ WD_DEV T *res_field_s(T *const *field) {
 // own three barriers; `mine`: this wave's activation, for routed rungs in use and the shared expert).  The workgroup's
 // eleven activations go out as one store of its record; waves 0..7 then wait for the records of all 512 workgroups and
 // lay the values out in LDS by slot; v0, v1 receive values 8 lane .. 8 lane + 7 of this wave's slot.
-// before(): work between handing in the activation and the barrier; meanwhile(): work for a wave that does not gather
-// (waves 8..11) while the others wait for the records.
-template <bool STAMPS, typename Before, typename Meanwhile>
-WD_DEV void res_exchange(const ResidentArgs &a, const ResCtx &c, int l, bool has, float mine, float4 &v0, float4 &v1, bool &dead, Before &&before, Meanwhile &&meanwhile) {
+// before(): work between handing in the activation and the barrier; early(): work of every wave once the workgroup's
+// record is on its way (no record can be complete before the slowest workgroup's has crossed the device); meanwhile():
+// work for a wave that does not gather (waves 8..11) while the others wait for the records.
+template <bool STAMPS, typename Before, typename Early, typename Meanwhile>
+WD_DEV void res_exchange(const ResidentArgs &a, const ResCtx &c, int l, bool has, float mine, float4 &v0, float4 &v1, bool &dead, Before &&before,
+                         Early &&early, Meanwhile &&meanwhile) {
     const int lane = c.lane, wave = c.wave;
     if (lane == 0) {
         if (has) c.actv()[c.slot] = mine;
@@ -436,6 +441,7 @@ WD_DEV void res_exchange(const ResidentArgs &a, const ResCtx &c, int l, bool has
         hand_store16(c.hb, ac_off(l, copy) + kAcRec * c.r + 16u * piece, make_uint4(hand_word(p.x), hand_word(p.y), hand_word(p.z), hand_word(p.w)));
     }
     res_mark<STAMPS>(a, c, l, 10);
+    early();
     if (wave < 8) {  // the group's copy, three 16-byte words per lane: word w is piece w % 3 of workgroup w / 3
         const int i = wave * 64 + lane;
         const unsigned base = ac_off(l, c.r & (kResCopies - 1)) + 16u * i;
@@ -540,7 +546,9 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
 #pragma unroll
         for (int c0 = 0; c0 < 8; ++c0) dec.w[i][c0] = 0u;
     }
-    bool decoded = false;  // dec holds this layer's rows
+    IqRowKept kept;  // (the up row: its weights lie in LDS)
+    kept.ls[0] = kept.ls[1] = 0, kept.d = 0u;
+    bool decoded = false;  // dec, kept and the wave's 2048 bytes of LDS hold this layer's rows
     for (int l = 0; l < a.n_layers; ++l) {
         const ResCtx c = res_ctx(lds_base, r0, lane0, wave0, slot0, hb);
         const int r = c.r, lane = c.lane, wave = c.wave, rung = c.slot;
@@ -607,6 +615,8 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
 
         // ---- routed rung: gate/up row r, then down rows 4r..4r+3
         float act = 0.0f;
+        // (with a routing trace the other workgroup of the compute unit may be decoding rows ahead: what the grid waits for goes first)
+        if (traced && r != 0) __builtin_amdgcn_s_setprio(kResPrioDots);
         if (on) {
             float gu[2] = {1.0f, 1.0f};
             if constexpr (!kQ8) {
@@ -628,7 +638,8 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                 q8_row_wave_pass<2>(gb, true, lane, c.x0q(), c.x0d(), tile, lane, acc);
                 gu[0] = close_lanes8(acc[0]), gu[1] = close_lanes8(acc[1]);
             } else {
-                iq_rows8_half_decoded_dots<kIq>(dec, tables, c.xq(), c.xd(), lane, gu, c.area());
+                if (decoded) iq_rows8_kept_decoded_dots<kIq>(dec, kept, c.kept(), c.xq(), c.xd(), lane, gu);
+                else iq_rows8_half_decoded_dots<kIq>(dec, tables, c.xq(), c.xd(), lane, gu, c.area());
             }
             act = silu_ggml(gu[0]) * gu[1];
             // the next layer's gate/up rows (their registers are free since the rows of this layer lie in LDS; requested
@@ -642,12 +653,19 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         // rung 0 folds the results with the router's weights and the shared expert's gate: published long before this
         // point as a rule, so one request now, answered while the activations are exchanged, replaces a round trip
         // between the down rows and the fold
+        if (traced && r != 0) __builtin_amdgcn_s_setprio(0);
         const bool wlane = rung == 0 && (lane < a.k || (shared && lane == 16));
         const unsigned woff = kHandWh + static_cast<unsigned>((l * 16 + (lane == 16 ? kResGateSlot : lane)) * 4);
         uint32_t wbits = kResEmpty;
         if (wlane && !dead) wbits = hand_load4(c.hb, woff);
         float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
-        res_exchange<STAMPS>(a, c, l, on, act, v0, v1, dead, [] {}, [] {});
+        res_exchange<STAMPS>(a, c, l, on, act, v0, v1, dead, [] {},
+            [&] {  // the next layer's up row, requested behind this layer's dot products: decoded while the records travel
+                if constexpr (!kQ8) {
+                    if (traced && on && !last && rows_asked) iq_row8_coal_decode_kept<kIq>(raw.u[1], tables, lane, c.kept(), kept);
+                }
+            },
+            [] {});
         if (on) res_down<STAMPS>(a, c, l, draw, v0, v1);
         float wreg = 0.0f;
         if (rung == 0) {
@@ -706,7 +724,9 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         decoded = false;
         if constexpr (!kQ8) {
             if (traced && on && !last && rows_asked) {
-                iq_rows8_coal_park<kIq, 2>(raw, lane, c.area());
+                IqRows8Raw<kIq, 1> gate_row;  // (the up row was decoded during the exchange)
+                gate_row.u[0] = raw.u[0];
+                iq_rows8_coal_park<kIq, 1>(gate_row, lane, c.area());
                 iq_rows8_coal_decode<kIq, 1>(tables, lane, c.area(), dec);
                 decoded = true;
             }
@@ -777,6 +797,7 @@ WD_DEV void res_shared_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         float4 v0 = make_float4(0.f, 0.f, 0.f, 0.f), v1 = v0;
         res_exchange<STAMPS>(a, c, l, with_shared, act, v0, v1, dead,
             [&] { if (r == 0 && traced) got = gather_logits(false); },  // the logits ahead of the barrier, if that holds nobody up
+            [] {},
             [&] {
                 if (r == 0 && traced) {
                     if (!got) (void)gather_logits(true);

@@ -498,6 +498,57 @@ WD_DEV void iq_rows8_half_decoded_dots(const IqRows8Decoded<1> &dec, const Table
         y[i] = (TYPE == 22) ? 0.125f * r : r;
     }
 }
+// The second of a caller's two rows decoded long before the first: its sixteen-byte words are parked in `keep` (2048 bytes
+// of LDS that belong to the wave until the dot products), decoded from there, and the 32 signed weights of every lane
+// written back over them - nothing needs the parked words any more once every lane has read its fields (a wave's LDS
+// operations complete in order), and a lane reads back only what it wrote itself.  What stays in registers are the
+// sub-scales and the super-block's scale.
+struct IqRowKept {
+    int ls[2];
+    uint32_t d;  // f16 bits
+};
+template <int TYPE, typename Tables>
+WD_DEV void iq_row8_coal_decode_kept(const uint4 &words, const Tables &t, int lane, uint8_t *keep, IqRowKept &row) {
+    constexpr int kBlk = IqRows8Raw<TYPE, 1>::kBlk;
+    if (lane < IqRows8Raw<TYPE, 1>::kWords) reinterpret_cast<uint4 *>(keep)[lane] = words;
+    wave_lds_fence();
+    const int ib = ((lane >> 4) << 1) | (lane & 1), sb = (lane >> 1) & 7;
+    uint32_t w[8];
+    const IqFields f = iq_fields_lds<TYPE>(keep + sb * kBlk, ib, sb);
+    iq_decode<TYPE>(f, ib, t, w, row.ls);
+    row.d = f.d;
+    asm volatile("" ::: "memory");  // (the stores below stay behind every read above)
+    uint4 *const out = reinterpret_cast<uint4 *>(keep);
+    out[lane] = make_uint4(w[0], w[1], w[2], w[3]);
+    out[64 + lane] = make_uint4(w[4], w[5], w[6], w[7]);
+}
+// The dot products of two rows decoded ahead: the first in registers (iq_rows8_coal_decode with NR = 1), the second kept
+// in LDS (iq_row8_coal_decode_kept).  The arithmetic of iq_rows8_coal_dots in the same order.
+template <int TYPE>
+WD_DEV void iq_rows8_kept_decoded_dots(const IqRows8Decoded<1> &dec, const IqRowKept &row, const uint8_t *keep, const int8_t *act_qs,
+                                       const float *act_d, int lane, float (&y)[2]) {
+    const int ib = ((lane >> 4) << 1) | (lane & 1), sb = (lane >> 1) & 7;
+    const uint4 a0 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32);
+    const uint4 a1 = *reinterpret_cast<const uint4 *>(act_qs + sb * 256 + ib * 32 + 16);
+    const uint32_t a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+    const float dx = act_d[sb];
+    const uint4 w0 = reinterpret_cast<const uint4 *>(keep)[lane], w1 = reinterpret_cast<const uint4 *>(keep)[64 + lane];
+    const uint32_t w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        int p[8];
+        if (i == 0) iq_dot_decoded(dec.w[0], dec.ls[0], a, p);
+        else iq_dot_decoded(w, row.ls, a, p);
+        const float ds = h2f(static_cast<uint16_t>(i == 0 ? dec.d[0] : row.d)) * dx;
+        const int P = reduce_scatter_ib_pairs(p, lane);
+        const float pf = static_cast<float>(P);
+        float v = __builtin_fmaf(ds, pf, 0.0f);
+#pragma unroll
+        for (int s = 1; s < 8; ++s) v = __builtin_fmaf(ds, pf, dpp_f<kDppShr2, 0xf, 0xf, true>(0.0f, v));
+        const float r = close_chains_pairs(v);
+        y[i] = (TYPE == 22) ? 0.125f * r : r;
+    }
+}
 template <int TYPE, int NR, bool PART = false>
 WD_DEV void iq_rows8_coal_finish(const IqRows8Raw<TYPE, NR> &raw, const IqTables &t, const int8_t *act_qs, const float *act_d,
                                  int lane, float (&y)[NR], uint8_t *stage, int32_t *partials = nullptr, size_t pstride = 0) {
