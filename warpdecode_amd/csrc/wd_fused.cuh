@@ -76,9 +76,12 @@ WD_DEV void lds_quantize_q8_0_step(const float4 &v0, const float4 &v1, bool on, 
                         __builtin_fmaxf(__builtin_fabsf(v1.z), __builtin_fabsf(v1.w))));
     amax = quad_max(amax);
     if (on) {
-        uint2 packed;
-        packed.x = q8_0_pack4(v0, amax);
-        packed.y = q8_0_pack4(v1, amax);
+        uint2 packed = make_uint2(0u, 0u);
+        if (amax != 0.0f) {  // (one division for the eight values)
+            const float inv = 127.0f / amax;
+            packed.x = q8_0_pack4_scaled(v0, inv);
+            packed.y = q8_0_pack4_scaled(v1, inv);
+        }
         *reinterpret_cast<uint2 *>(qs + base) = packed;
         if ((tid & 3) == 0) d[base >> 5] = f2h_ref(amax / 127.0f);
     }

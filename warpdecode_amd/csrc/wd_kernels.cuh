@@ -100,6 +100,14 @@ __global__ __launch_bounds__(256) void k_q8_k_quantize(const float *__restrict__
 }
 
 // ---- Q8_0 quantiser: eight lanes per 32-value block, four values per lane -----------------
+// (inv: 127 / amax, for a caller that packs more than four values of a block)
+WD_DEV uint32_t q8_0_pack4_scaled(float4 v, float inv) {
+    const int q0 = max(-128, min(127, static_cast<int>(__builtin_rintf(v.x * inv))));
+    const int q1 = max(-128, min(127, static_cast<int>(__builtin_rintf(v.y * inv))));
+    const int q2 = max(-128, min(127, static_cast<int>(__builtin_rintf(v.z * inv))));
+    const int q3 = max(-128, min(127, static_cast<int>(__builtin_rintf(v.w * inv))));
+    return (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | (static_cast<uint32_t>(q3 & 0xff) << 24);
+}
 WD_DEV uint32_t q8_0_pack4(float4 v, float amax) {
     if (amax == 0.0f) return 0u;
     const float inv = 127.0f / amax;
