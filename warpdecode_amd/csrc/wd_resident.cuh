@@ -479,14 +479,21 @@ WD_DEV void res_exchange(const ResidentArgs &a, const ResCtx &c, int l, bool has
 
 // The down rows 4r..4r+3 of one matrix against the activation values v0, v1 (8 lane .. 8 lane + 7) of slot `c.slot`:
 // quantises them to Q8_0 and runs the four row chains; the result of row 4r + i lands in ybuf[slot * 4 + i].
-template <bool STAMPS>
-WD_DEV void res_down(const ResidentArgs &a, const ResCtx &c, int l, const Q8CoalRaw<0, 16> &draw, const float4 &v0, const float4 &v1) {
+// staged(): called when the rows lie in LDS and their registers are free (it may fill `draw` again).
+template <bool STAMPS, typename Staged>
+WD_DEV void res_down(const ResidentArgs &a, const ResCtx &c, int l, Q8CoalRaw<0, 16> &draw, const float4 &v0, const float4 &v1, Staged &&staged) {
     const int lane = c.lane;
     uint8_t *area = c.area();
     int8_t *aq = reinterpret_cast<int8_t *>(area + kResTileBytes);
     uint16_t *ad = reinterpret_cast<uint16_t *>(area + kResTileBytes + kResF);
+    Q8TileNB<16> &tile = *reinterpret_cast<Q8TileNB<16> *>(area);
+    uint8_t *stage = reinterpret_cast<uint8_t *>(&tile);  // (q8_rows4_coal_finish, with the request of the next rows in between)
+    wave_lds_fence();
+    q8_rows4_coal_stage<0, 16>(draw, stage, lane);
+    staged();
     lds_quantize_q8_0_step(v0, v1, true, lane * 8, aq, ad, lane);
-    const float y = q8_rows4_coal_finish<0, 16>(draw, aq, ad, *reinterpret_cast<Q8TileNB<16> *>(area), lane);
+    wave_lds_fence();
+    const float y = q8_rows4_coal_dots<0, 16>(stage, aq, ad, tile, lane);
     if ((lane & 15) == 0) c.ybuf()[c.slot * 4 + (lane >> 4)] = y;
     res_mark<STAMPS>(a, c, l, 7);
 }
@@ -495,7 +502,9 @@ WD_DEV void res_down(const ResidentArgs &a, const ResCtx &c, int l, const Q8Coal
 // Rungs 0..7 (always waves 0..7) also fetch and quantise the layer's input.
 // Barriers of a layer, the same for every wave of the workgroup: B1 (input in LDS), B2..B4 (exchange of the
 // activations), B5 (down results in LDS).
-template <int TYPE, bool STAMPS>
+// TRACED: the launch has a routing trace (the two forms of the role differ in when they can ask for what: one body for
+// both, chosen at run time, costs the compiler's merging of registers that either form defines in its own place).
+template <int TYPE, bool STAMPS, bool TRACED>
 WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, int lane0, int wave0, int slot0,
                             __amdgpu_buffer_rsrc_t hb, bool &dead) {
     // TYPE 21 / 22: gate/up rows of eight IQ3_S / IQ2_S super-blocks against the Q8_K form of the input; TYPE 8: Q8_0 rows,
@@ -504,7 +513,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
     constexpr int kIq = kQ8 ? 21 : TYPE;  // (the type the super-block routines are instantiated with; unused when kQ8)
     constexpr int kRow = kQ8 ? 64 * 34 : 8 * ((TYPE == 21) ? 110 : 82);
     const bool shared = a.shared != 0;
-    const bool traced = a.ids_trace != nullptr;
+    constexpr bool traced = TRACED;
     auto expert_in_range = [&](uint32_t e) { return e < a.row_limit ? e : 0u; };  // (out of range: a wrong trace, or a wait that ran out)
     // the expert of this rung in layer l according to the routing trace, by the number that addresses the tensors
     // (any layer number: past the end it is the last layer's)
@@ -549,6 +558,17 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
     IqRowKept kept;  // (the up row: its weights lie in LDS)
     kept.ls[0] = kept.ls[1] = 0, kept.d = 0u;
     bool decoded = false;  // dec, kept and the wave's 2048 bytes of LDS hold this layer's rows
+    // With a routing trace the down rows of a layer are requested a layer ahead as well: at the moment the rows of the layer
+    // before have gone from their registers into LDS.  They then arrive while the down rows are worked through, the output
+    // folded and the next input awaited - not while the activations are exchanged, where every poll of a wave comes back
+    // behind the rows the wave has asked for (a wave's loads return in order) and the whole grid waits for the last poll.
+    Q8CoalRaw<0, 16> draw_ahead;
+    draw_ahead.u[0] = draw_ahead.u[1] = draw_ahead.u[2] = make_uint4(0u, 0u, 0u, 0u);
+    bool draw_asked = false;  // draw_ahead holds (or will hold) this layer's down rows
+    if (traced && slot0 < a.k) {
+        draw_ahead = q8_rows4_coal_request<0, 16>(res_field_s(&a.layers->down) + traced_expert(0, slot0) * a.down_stride + static_cast<size_t>(r0) * (4 * 16 * 34), lane0);
+        draw_asked = true;
+    }
     for (int l = 0; l < a.n_layers; ++l) {
         const ResCtx c = res_ctx(lds_base, r0, lane0, wave0, slot0, hb);
         const int r = c.r, lane = c.lane, wave = c.wave, rung = c.slot;
@@ -559,8 +579,9 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
         const bool last = l == a.n_layers - 1;
         const bool on = rung < a.k;
         res_mark<STAMPS>(a, c, l, 0);
-        Q8CoalRaw<0, 16> draw;
-        draw.u[0] = draw.u[1] = draw.u[2] = make_uint4(0u, 0u, 0u, 0u);
+        Q8CoalRaw<0, 16> draw_now;
+        draw_now.u[0] = draw_now.u[1] = draw_now.u[2] = make_uint4(0u, 0u, 0u, 0u);
+        Q8CoalRaw<0, 16> &draw = traced ? draw_ahead : draw_now;
         // what the requests below are made of, asked for now (scalar loads): the tensors of this layer and, with a routing
         // trace, the gate/up tensors and the expert of the next one
         const ResidentLayer *const Ln = a.layers + (last ? l : l + 1);
@@ -630,7 +651,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             // which the whole grid waits for): the expert's number passes through a statement the compiler cannot
             // look into, so that the addresses below do not exist before this point.
             asm volatile("" : "+s"(e) : : "memory");
-            draw = q8_rows4_coal_request<0, 16>(down_base + e * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
+            if (!traced || !draw_asked) draw = q8_rows4_coal_request<0, 16>(down_base + e * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
             res_mark<STAMPS>(a, c, l, 11);
             if constexpr (kQ8) {
                 Q8RowTile &tile = *reinterpret_cast<Q8RowTile *>(c.area());
@@ -666,7 +687,14 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                 }
             },
             [] {});
-        if (on) res_down<STAMPS>(a, c, l, draw, v0, v1);
+        if (on) {
+            res_down<STAMPS>(a, c, l, draw, v0, v1, [&] {
+                if constexpr (traced) {  // the next layer's down rows (its slots filled, if they are slots)
+                    draw_asked = !last && rows_asked;
+                    if (draw_asked) draw = q8_rows4_coal_request<0, 16>(res_field_s(&Ln->down) + e_next * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
+                }
+            });
+        }
         float wreg = 0.0f;
         if (rung == 0) {
             if (__builtin_amdgcn_ballot_w64(wlane && wbits == kResEmpty) != 0ull) wbits = hand_wait4(a, c.hb, woff, wlane, dead);
@@ -804,7 +832,7 @@ WD_DEV void res_shared_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                     denominator();
                 }
             });
-        if (with_shared) res_down<STAMPS>(a, c, l, draw, v0, v1);
+        if (with_shared) res_down<STAMPS>(a, c, l, draw, v0, v1, [] {});
         __syncthreads();  // B5
         // the next layer's rows, asked for on this side of the barrier: the fold of this layer must not wait for a
         // wave that is busy issuing requests
@@ -1039,7 +1067,8 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(6, 
     else if (slot == kResSharedSlot)
         res_shared_role<STAMPS>(a, lds_res, r, fresh_lane(), wave, hb, dead);
     else
-        res_routed_role<TYPE, STAMPS>(a, lds_res, r, fresh_lane(), wave, slot, hb, dead);
+        if (a.ids_trace) res_routed_role<TYPE, STAMPS, true>(a, lds_res, r, fresh_lane(), wave, slot, hb, dead);
+        else res_routed_role<TYPE, STAMPS, false>(a, lds_res, r, fresh_lane(), wave, slot, hb, dead);
 
     // the next launch takes the other set (workgroup 0 can only get here after every workgroup has read the number)
     if (r == 0 && wave == 0 && fresh_lane() == 0 && !dead)

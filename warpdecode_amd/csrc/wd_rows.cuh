@@ -225,8 +225,14 @@ WD_DEV void iq_decode(const IqFields &f, int ib, const Tables &t, uint32_t (&w)[
     }
 }
 WD_DEV void iq_dot_decoded(const uint32_t (&w)[8], const int (&ls)[2], const uint32_t (&a)[8], int (&p)[8]) {
+    // (The sub-scales pass through a statement the compiler cannot look into.  It knows that they are small, drops
+    // __mul24's sign extension of them as redundant and moves what is left out of the caller's loop - and then selects,
+    // for a factor that is just some register, the full 32-bit multiply: a quarter-rate instruction, sixteen times per
+    // pair of rows.  With the extension in place both factors are visibly 24 bits wide and the multiply is v_mul_i32_i24.)
+    int l[2] = {ls[0], ls[1]};
+    asm("" : "+v"(l[0]), "+v"(l[1]));
 #pragma unroll
-    for (int c = 0; c < 8; ++c) p[c] = __mul24(ls[c >> 2], sdot4(w[c], a[c], 0));
+    for (int c = 0; c < 8; ++c) p[c] = __mul24(l[c >> 2], sdot4(w[c], a[c], 0));
 }
 
 // NR rows against one Q8_K activation (act_qs / act_d in global memory or LDS).  y[i] is uniform
