@@ -652,6 +652,15 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             // look into, so that the addresses below do not exist before this point.
             asm volatile("" : "+s"(e) : : "memory");
             if (!traced || !draw_asked) draw = q8_rows4_coal_request<0, 16>(down_base + e * a.down_stride + static_cast<size_t>(r) * (4 * 16 * 34), lane);
+            // With a routing trace the next layer's gate/up rows are requested here, ahead of the dot products: the rows of
+            // this layer are decoded or parked, so their registers are free, and the earlier the rows arrive, the less the
+            // polls for the activations - which come back behind them - have to wait (-0.9 % against a request behind
+            // the dot products).  Q8_0 rows are still in their registers: those are asked for behind the dot products.
+            constexpr bool rows_first = traced && !kQ8;
+            if constexpr (rows_first) {
+                rows_asked = need_next == 0u || dead || fill_reached(a, l + 1, need_next);
+                if (rows_asked) gate_up_rows(gate_base, up_base, e_next, r, lane);
+            }
             res_mark<STAMPS>(a, c, l, 11);
             if constexpr (kQ8) {
                 Q8RowTile &tile = *reinterpret_cast<Q8RowTile *>(c.area());
@@ -663,9 +672,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
                 else iq_rows8_half_decoded_dots<kIq>(dec, tables, c.xq(), c.xd(), lane, gu, c.area());
             }
             act = silu_ggml(gu[0]) * gu[1];
-            // the next layer's gate/up rows (their registers are free since the rows of this layer lie in LDS; requested
-            // behind the dot products, which need every register there is)
-            if (traced) {
+            if constexpr (traced && !rows_first) {
                 rows_asked = need_next == 0u || dead || fill_reached(a, l + 1, need_next);
                 if (rows_asked) gate_up_rows(gate_base, up_base, e_next, r, lane);
             }
