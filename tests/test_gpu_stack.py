@@ -200,6 +200,30 @@ def test_one_launch_stack_matches_per_layer_and_oracle(g, oracle, gate_type, exp
     dls, arr = _descs(g, Ls)
     sc_a, sc_b = g.Scratch(2048, 512, experts, k), g.Scratch(2048, 512, experts, k)
     rng = np.random.default_rng(SEED + 400)
+    # The comparison below says nothing if the first form quietly took the dispatches per layer as well (a device that
+    # does not hold the 512 workgroups at once makes it do so): the site profiler counts the launches of either form.
+    lib = capi.load()
+    site = {lib.wd_profile_site_name(i).decode(): i for i in range(64) if lib.wd_profile_site_name(i) != b"unknown"}
+    site_resident = [i for name, i in site.items() if "resident" in name]
+    assert len(site_resident) == 1, site
+
+    def resident_launches():
+        capi.call("wd_profile_flush_token")
+        st, tokens = capi.ProfileSiteStat(), C.c_ulonglong()
+        capi.call("wd_profile_site", site_resident[0], C.byref(st), C.byref(tokens))
+        return st.calls
+
+    capi.call("wd_profile_enable", 1)
+    capi.call("wd_profile_reset")
+    try:
+        x0 = synth.rms_normed(synth.rng_for(SEED, 83, 0), 2048)
+        _run_stack(g, arr, nl, x0, None, sc_a, 0)
+        assert resident_launches() == 1
+        _run_stack(g, arr, nl, x0, None, sc_b, PER_LAYER)
+        assert resident_launches() == 1
+    finally:
+        capi.call("wd_profile_enable", 0)
+        capi.call("wd_profile_reset")
     for token, depth in enumerate([nl, 2, nl, nl, min(3, nl), nl]):
         x = synth.rms_normed(synth.rng_for(SEED, 84, token), 2048)
         tr = None
