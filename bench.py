@@ -1156,6 +1156,22 @@ def main():
     per_kernel, reps, router_driven = {}, 20, None
     step(0)
     if args.path == "resident":
+        # the figures below are named for k_stack_resident: make sure that it is what the library launches on this device
+        # (it takes the dispatches per layer, silently, where the 512 workgroups cannot all be resident at once)
+        lib = capi.load()
+        sites = [i for i in range(64) if b"resident" in lib.wd_profile_site_name(i)]
+        capi.call("wd_profile_enable", 1)
+        capi.call("wd_profile_reset")
+        bring_in(0)
+        launch_stack()
+        torch.cuda.synchronize()
+        capi.call("wd_profile_flush_token")
+        st, seen = capi.ProfileSiteStat(), C.c_ulonglong()
+        capi.call("wd_profile_site", sites[0], C.byref(st), C.byref(seen))
+        capi.call("wd_profile_enable", 0)
+        capi.call("wd_profile_reset")
+        if len(sites) != 1 or st.calls != 1:
+            raise SystemExit("bench.py: the stack did not run as one resident launch on this device (--path per-layer measures the dispatches per layer)")
         # The dominant kernel is the step itself: one launch of k_stack_resident covers the 48 layers.  Timed live with HIP
         # events on the launch stream over `reps` launches (graph replays) without the input copies of step().
         # (fresh input and routing trace before every launch, as in the timed region; the events bracket the launch alone)
