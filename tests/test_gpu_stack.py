@@ -224,7 +224,7 @@ def test_one_launch_stack_matches_per_layer_and_oracle(g, oracle, gate_type, exp
     finally:
         capi.call("wd_profile_enable", 0)
         capi.call("wd_profile_reset")
-    for token, depth in enumerate([nl, 2, nl, nl, min(3, nl), nl]):
+    for token, depth in enumerate([nl, 2, nl, nl, min(3, nl), nl, 1, 1]):
         x = synth.rms_normed(synth.rng_for(SEED, 84, token), 2048)
         tr = None
         if token % 2 == 1:
