@@ -114,6 +114,10 @@ WD_DEV int sdot4(uint32_t a, uint32_t b, int acc) {
     // (Not the three-operand form with a constant 0 through inline assembly, although it saves the move that zeroes the
     // two-operand form's accumulator: the result of a dot instruction needs wait states before another vector instruction
     // reads it, which the compiler inserts for instructions it knows and not behind assembly text - results were wrong.)
+    // A dot product that starts from zero is asked for with the clamp bit: only the three-operand encoding has one, so the
+    // compiler takes that encoding, with the constant 0 as its third operand, instead of the two-operand form and a
+    // move that zeroes its accumulator first.  (Four products of bytes cannot overflow: the bit changes no result.)
+    if (__builtin_constant_p(acc) && acc == 0) return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), 0, true);
     return __builtin_amdgcn_sdot4(static_cast<int>(a), static_cast<int>(b), acc, false);
 }
 
