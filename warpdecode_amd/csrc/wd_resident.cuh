@@ -20,9 +20,11 @@
 // layer); workgroup 0's router wave gathers the 512 logits, eight per lane, and ranks them in registers (sel_wave_ids,
 // wd_fused.cuh).  Without a routing trace it publishes the ids at once, in sixteen replicas that the rungs of the grid
 // poll, and only then works out the denominator and the weights, which nothing needs before the fold at the end of the
-// layer.  With a routing trace the ids are inputs of the launch: the rungs request the next layer's gate/up rows while
-// they still work on this one, and workgroup 0 ranks between the barriers of its own activation exchange, so that it never
-// holds up its own rungs (the whole grid waits for the slowest workgroup of a layer).  The shared expert's wave of
+// layer.  With a routing trace the ids are inputs of the launch: the rungs request the next layer's gate/up and down rows
+// while they still work on this one - at points chosen so that no request is under way when the grid exchanges values,
+// because a poll comes back behind every row its wave has asked for -, decode the gate/up rows in the stretches in
+// which the vector units would idle (res_routed_role), and workgroup 0 ranks between the barriers of its own
+// activation exchange, so that it never holds up its own rungs (the whole grid waits for the slowest workgroup of a layer).  The shared expert's wave of
 // workgroup 0 computes the softmax denominator meanwhile.  The router waves run at a raised wave priority, as do all
 // waves of workgroup 0: their few instructions are on everybody's critical path.
 // Routed experts in a slot pool (the expert cache's stack, with a routing trace): the pool is addressed as one tensor of
