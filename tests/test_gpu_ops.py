@@ -28,6 +28,7 @@ def _act_cases(n, seed):
     x = rng.normal(0, 1, n); x[n // 2 + 3] = -37.5; xs.append(x)
     xs.append(np.round(rng.normal(0, 20, n)) / 254.0 * 3.0)       # exact .5 products: half-to-even
     xs.append(rng.normal(0, 3e-7, n))                              # fp16 scale below 2^-24 in some blocks
+    x = rng.normal(0, 1, n); x[:256] = np.nan; xs.append(x)        # blocks of nothing but NaN: fmaxf from 0 drops them all
     return [np.asarray(v, np.float32) for v in xs]
 
 

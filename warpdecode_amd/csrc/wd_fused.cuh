@@ -74,7 +74,7 @@ WD_DEV void lds_quantize_q8_0_step(const float4 &v0, const float4 &v1, bool on, 
                         __builtin_fmaxf(__builtin_fabsf(v0.z), __builtin_fabsf(v0.w))),
         __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v1.x), __builtin_fabsf(v1.y)),
                         __builtin_fmaxf(__builtin_fabsf(v1.z), __builtin_fabsf(v1.w))));
-    amax = quad_max(amax);
+    amax = quad_max_nonneg(amax);
     if (on) {
         uint2 packed = make_uint2(0u, 0u);
         if (amax != 0.0f) {  // (one division for the eight values)
@@ -109,7 +109,7 @@ WD_DEV void wave_quantize_q8_k_block(const float *__restrict__ x256, int8_t *qs2
 WD_DEV void wave_quantize_q8_k_regs(const float4 &v, int8_t *qs256, float *d, int lane) {
     float amax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)),
                                  __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
-    amax = wave_max(amax);
+    amax = wave_max_nonneg(amax);
     uint32_t packed = 0;
     float dv = 0.0f;
     if (amax != 0.0f) {

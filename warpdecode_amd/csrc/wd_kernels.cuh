@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void k_q8_k_quantize(const float *__restrict__
     const float4 v = reinterpret_cast<const float4 *>(x + static_cast<size_t>(blk) * 256)[lane];
     float amax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)),
                                  __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
-    amax = wave_max(amax);
+    amax = wave_max_nonneg(amax);
     uint32_t packed = 0;
     int part = 0;
     float d = 0.0f;
@@ -127,8 +127,7 @@ __global__ __launch_bounds__(256) void k_q8_0_quantize(const float *__restrict__
     if (on) v = reinterpret_cast<const float4 *>(x + static_cast<size_t>(blk) * 32)[sub];
     float amax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)),
                                  __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
-    amax = quad_max(amax);
-    amax = __builtin_fmaxf(amax, dpp_f<0x141>(amax, amax));  // row_half_mirror pairs the two quads of a block
+    amax = oct_max_nonneg(amax);
     if (!on) return;
     reinterpret_cast<uint32_t *>(qs + static_cast<size_t>(blk) * 32)[sub] = q8_0_pack4(v, amax);
     if (sub == 0) scales[blk] = f2h_ref(amax / 127.0f);
@@ -146,8 +145,7 @@ WD_DEV uint16_t f2h_rn(float v) {
 WD_DEV float block32_amax(const float4 &v) {
     float amax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)),
                                  __builtin_fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
-    amax = quad_max(amax);
-    return __builtin_fmaxf(amax, dpp_f<0x141>(amax, amax));  // row_half_mirror pairs the two quads of a block
+    return oct_max_nonneg(amax);
 }
 // q8_1_quantize_f32_kernel, src/lowbit.cuh:287-308: d = amax / 127, q = roundf(x / d) (a division; halves away from
 // zero), scale = half(d).  Eight lanes per block, four values per lane.

@@ -616,8 +616,7 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             if (shared || kQ8) {  // Q8_0: a block is eight lanes
                 float amax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(xv.x), __builtin_fabsf(xv.y)),
                                              __builtin_fmaxf(__builtin_fabsf(xv.z), __builtin_fabsf(xv.w)));
-                amax = quad_max(amax);
-                amax = __builtin_fmaxf(amax, dpp_f<0x141>(amax, amax));  // row_half_mirror pairs the two quads of a block
+                amax = oct_max_nonneg(amax);
                 reinterpret_cast<uint32_t *>(c.x0q())[i] = q8_0_pack4(xv, amax);
                 if ((lane & 7) == 0) c.x0d()[i >> 3] = f2h_ref(amax / 127.0f);
             }
