@@ -723,11 +723,22 @@ WD_DEV void res_routed_role(const ResidentArgs &a, uint8_t *lds_base, int r0, in
             for (int m = 0; m < kResMaxK; ++m) yv[m] = ybuf[m * 4 + (lane & 3)];
             float ysh = ybuf[kResSharedSlot * 4 + (lane & 3)];
             float acc = 0.0f;
+            if (traced && fresh_s(a.k) == kResMaxK) {  // (with a routing trace only: the other form of the role came out slower with it)
+                // (every term in use, the usual case: no select between two additions of the one chain the whole grid waits
+                // for - the compiler keeps the selects' ten lane masks parked in lanes of a vector register and fetches one
+                // back, two instructions and their wait states, per term)
 #pragma unroll
-            for (int m = 0; m < kResMaxK; ++m) {
-                const float prod = yv[m] * readlane_f(wreg, m);
-                const float next = acc + prod;
-                acc = m < a.k ? next : acc;
+                for (int m = 0; m < kResMaxK; ++m) {
+                    const float prod = yv[m] * readlane_f(wreg, m);
+                    acc = acc + prod;
+                }
+            } else {
+#pragma unroll
+                for (int m = 0; m < kResMaxK; ++m) {
+                    const float prod = yv[m] * readlane_f(wreg, m);
+                    const float next = acc + prod;
+                    acc = m < a.k ? next : acc;
+                }
             }
             float o = acc;
             if (!shared) ysh = 0.0f;
