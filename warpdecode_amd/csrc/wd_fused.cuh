@@ -560,10 +560,11 @@ struct SelWaveState {
 };
 
 WD_DEV uint32_t wave_max_u32(uint32_t v) {  // the result is uniform
-    v = max(v, static_cast<uint32_t>(dpp_i<kDppXor1>(static_cast<int>(v), static_cast<int>(v))));
-    v = max(v, static_cast<uint32_t>(dpp_i<kDppXor2>(static_cast<int>(v), static_cast<int>(v))));
-    v = max(v, static_cast<uint32_t>(dpp_i<kDppRor4>(static_cast<int>(v), static_cast<int>(v))));
-    v = max(v, static_cast<uint32_t>(dpp_i<kDppRor8>(static_cast<int>(v), static_cast<int>(v))));  // every lane: its row's largest
+    // (umax_step: written so that the shuffle and the maximum become one instruction)
+    v = umax_step<kDppXor1>(v);
+    v = umax_step<kDppXor2>(v);
+    v = umax_step<kDppRor4>(v);
+    v = umax_step<kDppRor8>(v);  // every lane: its row's largest
     const wd_uint2v t = __builtin_amdgcn_permlane32_swap(v, v, false, false);
     v = max(t.x, t.y);                                                                            // rows 0|2 and 1|3
     return max(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), 0)),
